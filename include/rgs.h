@@ -1,0 +1,182 @@
+/*
+ * rgs.h -- C ABI of librgs_gfx950.so, the MI355X (gfx950) half-Gaussian rasterizer.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream (as void*;
+ * NULL = the default stream).  The library never allocates or frees device memory:
+ * the caller sizes the three workspaces with the rgs_*_bytes() functions and owns
+ * them.  All float data is fp32, contiguous, on the device the stream belongs to.
+ * Matrices are 16 floats in the reference's layout (row-vector convention, i.e.
+ * element [4*c + r] is row r, column c of the usual column-vector matrix).
+ *
+ * Functions return 0 on success; on failure they return non-zero and
+ * rgs_last_error() gives the reason for the calling thread.
+ *
+ * Citations name the interface of the reference that each entry point replaces,
+ * with K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian.
+ */
+#ifndef RGS_H_INCLUDED
+#define RGS_H_INCLUDED
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Library version (major*10000 + minor*100 + patch). */
+int rgs_version(void);
+
+/* Message for the last failure on the calling thread ("" if none).
+ * Replaces the exceptions thrown through CHECK_CUDA (K/cuda_rasterizer_hgs/auxiliary.h:182-189)
+ * and AT_ERROR (K/rasterize_points.cu:60-62). */
+const char* rgs_last_error(void);
+
+/* The reference's sort-key width helper: number of bits needed for n tile ids
+ * (getHigherMsb, K/cuda_rasterizer_hgs/rasterizer_impl.cu:35-50). */
+uint32_t rgs_get_higher_msb(uint32_t n);
+
+/* ---- workspace sizing -------------------------------------------------------------
+ * Replace required<GeometryState>/<BinningState>/<ImageState>
+ * (K/cuda_rasterizer_hgs/rasterizer_impl.h:65-72, rasterizer_impl.cu:155-194). */
+size_t rgs_geom_bytes(int P);
+size_t rgs_binning_bytes(int R);
+size_t rgs_image_bytes(int width, int height);
+
+/* Byte offsets of the arrays inside the workspaces, for tests and tools that want to
+ * look at intermediate results.  The workspaces are otherwise opaque. */
+enum {
+	RGS_GEOM_DEPTHS = 0,        /* float[P]   view-space z */
+	RGS_GEOM_XY,                /* float2[P]  pixel centre */
+	RGS_GEOM_CLIP_W,            /* float[P]   clip-space w */
+	RGS_GEOM_COV3D,             /* float[6P] */
+	RGS_GEOM_CONIC_OPACITY,     /* float4[P] */
+	RGS_GEOM_RGB,               /* float[3P] */
+	RGS_GEOM_TILES_TOUCHED,     /* uint32[P] */
+	RGS_GEOM_POINT_OFFSETS,     /* uint32[P]  inclusive prefix sum of tiles_touched */
+	RGS_GEOM_CLAMPED,           /* uint8[P]   bit c set: colour channel c was clamped at 0 */
+	RGS_GEOM_BLOCK_SUMS,        /* uint32[ceil(P/256)+1] */
+	RGS_GEOM_TOTAL,             /* uint32     number of (Gaussian, tile) instances */
+	RGS_GEOM_FIELDS
+};
+enum {
+	RGS_BIN_KEYS_UNSORTED = 0,  /* uint64[R]  (tile << 32) | depth bits, emission order */
+	RGS_BIN_KEYS_SORTED,        /* uint64[R] */
+	RGS_BIN_VALUES_UNSORTED,    /* uint32[R]  Gaussian index */
+	RGS_BIN_VALUES_SORTED,      /* uint32[R]  the per-tile Gaussian lists, tile after tile */
+	RGS_BIN_SORT_TEMP,          /* uint32[..] */
+	RGS_BIN_FIELDS
+};
+enum {
+	RGS_IMG_RANGES = 0,         /* uint2[tiles]  [start, end) of each tile in the sorted list */
+	RGS_IMG_N_CONTRIB,          /* uint32[H*W]   list position of the last blended Gaussian */
+	RGS_IMG_FIELDS
+};
+int rgs_geom_layout(int P, size_t offsets[RGS_GEOM_FIELDS]);
+/* After rgs_forward_raster the *_UNSORTED arrays have been used as sort scratch.  Which
+ * physical buffer ends up holding the sorted data depends on the number of radix
+ * passes, so the layout is reported for a given image size. */
+int rgs_binning_layout(int R, int width, int height, size_t offsets[RGS_BIN_FIELDS]);
+int rgs_image_layout(int width, int height, size_t offsets[RGS_IMG_FIELDS]);
+
+/* ---- rasterizer ---------------------------------------------------------------------- */
+
+/* Frustum mask: present[i] = (view-space z of means3D[i] > 0.2).
+ * Replaces Rasterizer::markVisible (K/cuda_rasterizer_hgs/rasterizer.h:22-27,
+ * rasterizer_impl.cu:141-153) behind _C.mark_visible (K/ext.cpp:18). */
+int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const float* projmatrix,
+                     uint8_t* present, void* stream);
+
+/* First half of Rasterizer::forward (K/cuda_rasterizer_hgs/rasterizer.h:29-58,
+ * rasterizer_impl.cu:198-287): per-Gaussian preprocess and the prefix sum of the tile
+ * counts.  Writes radii[P], fills the geometry workspace and stores the number of
+ * (Gaussian, tile) instances R to *num_rendered_host (host memory, preferably
+ * pinned); the stream has been synchronised when the call returns, exactly where the
+ * reference blocks on its device-to-host copy (rasterizer_impl.cu:287).
+ * Exactly one of shs / colors_precomp and one of (scales, rotations) / cov3D_precomp
+ * is non-NULL.  D = active SH degree (0..3), M = SH coefficients per Gaussian. */
+int rgs_forward_geom(int P, int D, int M, int width, int height,
+                     const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
+                     const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                     const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                     float tan_fovx, float tan_fovy, int prefiltered,
+                     int* radii, void* geom_ws, size_t geom_bytes,
+                     uint32_t* num_rendered_host, void* stream, int debug);
+
+/* Second half of Rasterizer::forward (rasterizer_impl.cu:289-351): key duplication,
+ * stable sort of the (tile | depth) keys, tile ranges and the per-tile blend with the
+ * per-pixel submodel-box test.  R is the value rgs_forward_geom reported.
+ * Writes out_color (3,H,W), out_depth (1,H,W), out_alpha (1,H,W). */
+int rgs_forward_raster(int P, int R, int width, int height,
+                       const float* background, float tan_fovx, float tan_fovy,
+                       const float* projmatrix_inv, const float* range_low, const float* range_up,
+                       const float* colors_precomp, const int* radii,
+                       void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                       void* image_ws, size_t image_bytes,
+                       float* out_color, float* out_depth, float* out_alpha, void* stream, int debug);
+
+/* Layout of grad_accum (12*P floats), the per-Gaussian sums the backward blend
+ * accumulates atomically; offsets are in units of P floats. */
+enum {
+	RGS_ACC_MEAN2D = 0,   /* (P,3): d/dx, d/dy of the pixel centre, third column stays 0 */
+	RGS_ACC_CONIC = 3,    /* (P,4): xx, xy, unused, yy */
+	RGS_ACC_OPACITY = 7,  /* (P)   */
+	RGS_ACC_COLOR = 8,    /* (P,3) */
+	RGS_ACC_DEPTH = 11,   /* (P)   */
+	RGS_ACC_FLOATS = 12
+};
+
+/* Rasterizer::backward (K/cuda_rasterizer_hgs/rasterizer.h:60-96, rasterizer_impl.cu:355-466)
+ * together with the zero-initialisation done by its torch shim
+ * (K/rasterize_points.cu:165-174).  grad_accum need not be cleared by the caller.
+ * dL_dmean3D (P,3), dL_dcov3D (P,6), dL_dsh (P,M,3), dL_dscale (P,3), dL_drot (P,4) are
+ * written for every Gaussian (zeros where it was not rendered); dL_dsh / dL_dscale /
+ * dL_drot may be NULL when shs / scales are NULL. */
+int rgs_backward(int P, int D, int M, int R, int width, int height,
+                 const float* background, const float* means3D, const float* shs, const float* colors_precomp,
+                 const float* alphas, const float* scales, float scale_modifier, const float* rotations,
+                 const float* cov3D_precomp, const float* viewmatrix, const float* projmatrix,
+                 const float* projmatrix_inv, const float* range_low, const float* range_up, const float* cam_pos,
+                 float tan_fovx, float tan_fovy, const int* radii,
+                 const void* geom_ws, const void* binning_ws, const void* image_ws,
+                 const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
+                 float* grad_accum, float* dL_dmean3D, float* dL_dcov3D, float* dL_dsh, float* dL_dscale,
+                 float* dL_drot, void* stream, int debug);
+
+/* ---- stand-alone binning primitives ---------------------------------------------------- */
+
+/* Inclusive uint32 prefix sum; replaces the cub::DeviceScan::InclusiveSum call at
+ * K/cuda_rasterizer_hgs/rasterizer_impl.cu:283.  temp: rgs_scan_temp_bytes(n) bytes. */
+size_t rgs_scan_temp_bytes(size_t n);
+int rgs_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, void* temp, void* stream);
+
+/* Stable sort of (uint64 key, uint32 value) pairs on key bits [0, end_bit); replaces the
+ * cub::DeviceRadixSort::SortPairs call at K/cuda_rasterizer_hgs/rasterizer_impl.cu:312-317.
+ * keys_in / vals_in are overwritten (used as scratch).  temp: rgs_sort_temp_bytes(n) bytes. */
+size_t rgs_sort_temp_bytes(size_t n);
+int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                   int end_bit, void* temp, void* stream);
+
+/* ---- partial-image compositor ------------------------------------------------------------
+ * Replaces the tensor expression in blender_render_result
+ * (parallel_utils/basic_parallel_trainer/result_aggregator.py:244-259) and its autograd
+ * backward.  images[k] (3,H,W), depths[k] (1,H,W), alphas[k] (1,H,W) are HOST arrays of
+ * K device pointers, already in front-to-back order; K <= RGS_MAX_COMPOSITE.
+ * background: 3 floats on the device, or NULL for black. */
+#define RGS_MAX_COMPOSITE 64
+int rgs_composite_forward(int K, int height, int width,
+                          const float* const* images, const float* const* depths, const float* const* alphas,
+                          const float* background, float* out_image, float* out_depth, float* out_alpha,
+                          void* stream);
+/* g_depth / g_alpha may be NULL (treated as zero).  d_images[k], d_depths[k], d_alphas[k]
+ * receive the gradients and are fully written. */
+int rgs_composite_backward(int K, int height, int width,
+                           const float* const* images, const float* const* depths, const float* const* alphas,
+                           const float* background, const float* g_image, const float* g_depth,
+                           const float* g_alpha, float* const* d_images, float* const* d_depths,
+                           float* const* d_alphas, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RGS_H_INCLUDED */

@@ -1,0 +1,106 @@
+"""ctypes binding of librgs_gfx950.so (declarations: include/rgs.h).
+
+The library is the only implementation: if it is missing, importing this module
+fails with instructions to build it; nothing falls back to another code path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librgs_gfx950.so")
+
+GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles_touched", "point_offsets",
+               "clamped", "block_sums", "total")
+BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
+IMG_FIELDS = ("ranges", "n_contrib")
+ACC_MEAN2D, ACC_CONIC, ACC_OPACITY, ACC_COLOR, ACC_DEPTH, ACC_FLOATS = 0, 3, 7, 8, 11, 12
+MAX_COMPOSITE = 64
+
+
+class RgsError(RuntimeError):
+    pass
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m retinags_amd.build` "
+            "(hipcc, gfx950). There is no fallback implementation.")
+    lib = C.CDLL(LIB_PATH)
+    vp, f, i, sz = C.c_void_p, C.c_float, C.c_int, C.c_size_t
+    lib.rgs_version.restype = i
+    lib.rgs_last_error.restype = C.c_char_p
+    lib.rgs_get_higher_msb.restype = C.c_uint32
+    lib.rgs_get_higher_msb.argtypes = [C.c_uint32]
+    for name, args in (("rgs_geom_bytes", [i]), ("rgs_binning_bytes", [i]), ("rgs_image_bytes", [i, i]),
+                       ("rgs_scan_temp_bytes", [sz]), ("rgs_sort_temp_bytes", [sz])):
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = sz, args
+    lib.rgs_geom_layout.argtypes = [i, C.POINTER(sz)]
+    lib.rgs_binning_layout.argtypes = [i, i, i, C.POINTER(sz)]
+    lib.rgs_image_layout.argtypes = [i, i, C.POINTER(sz)]
+    lib.rgs_mark_visible.argtypes = [i, vp, vp, vp, vp, vp]
+    lib.rgs_forward_geom.argtypes = [i, i, i, i, i, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, f, f, i,
+                                     vp, vp, sz, vp, vp, i]
+    lib.rgs_forward_raster.argtypes = [i, i, i, i, vp, f, f, vp, vp, vp, vp, vp, vp, sz, vp, sz, vp, sz,
+                                       vp, vp, vp, vp, i]
+    lib.rgs_backward.argtypes = [i, i, i, i, i, i, vp, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, vp, vp, vp,
+                                 f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i]
+    lib.rgs_inclusive_sum.argtypes = [vp, vp, sz, vp, vp]
+    lib.rgs_sort_pairs.argtypes = [vp, vp, vp, vp, sz, i, vp, vp]
+    pp = C.POINTER(vp)
+    lib.rgs_composite_forward.argtypes = [i, i, i, pp, pp, pp, vp, vp, vp, vp, vp]
+    lib.rgs_composite_backward.argtypes = [i, i, i, pp, pp, pp, vp, vp, vp, vp, pp, pp, pp, vp]
+    for name in ("rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
+                 "rgs_forward_geom", "rgs_forward_raster", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
+                 "rgs_composite_forward", "rgs_composite_backward"):
+        getattr(lib, name).restype = i
+    return lib
+
+
+lib = _load()
+
+EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_bytes", "rgs_binning_bytes",
+           "rgs_image_bytes", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
+           "rgs_forward_geom", "rgs_forward_raster", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
+           "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward")
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise RgsError(lib.rgs_last_error().decode("utf-8", "replace"))
+
+
+def geom_layout(P: int) -> dict:
+    off = (C.c_size_t * len(GEOM_FIELDS))()
+    check(lib.rgs_geom_layout(P, off))
+    return dict(zip(GEOM_FIELDS, off))
+
+
+def binning_layout(R: int, width: int, height: int) -> dict:
+    off = (C.c_size_t * len(BIN_FIELDS))()
+    check(lib.rgs_binning_layout(R, width, height, off))
+    return dict(zip(BIN_FIELDS, off))
+
+
+def image_layout(width: int, height: int) -> dict:
+    off = (C.c_size_t * len(IMG_FIELDS))()
+    check(lib.rgs_image_layout(width, height, off))
+    return dict(zip(IMG_FIELDS, off))
+
+
+def ptr(t) -> C.c_void_p:
+    """Device (or pinned host) address of a tensor; None and empty tensors map to NULL,
+    which is how the reference passes absent inputs (torch.Tensor([]) -> nullptr)."""
+    if t is None or t.numel() == 0:
+        return C.c_void_p(0)
+    return C.c_void_p(t.data_ptr())
+
+
+def ptr_table(tensors):
+    arr = (C.c_void_p * len(tensors))()
+    for k, t in enumerate(tensors):
+        arr[k] = t.data_ptr()
+    return arr

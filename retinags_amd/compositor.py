@@ -1,0 +1,114 @@
+"""Front-to-back compositing of per-submodel partial images, forward and backward, as
+one fused HIP pass each.  Host-side mirror of blender_render_result
+(parallel_utils/basic_parallel_trainer/result_aggregator.py:193-260): the same ordering
+rule (ascending value of the relation vector, negative = not related), the same three
+outputs (render, depth, alpha) and the same gradients torch autograd produces for the
+reference's cat / cumprod / sum expression.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from . import _capi
+from ._capi import lib, check, ptr, ptr_table
+
+
+def _prep(t: torch.Tensor, device, shape) -> torch.Tensor:
+    if t.device != device or t.dtype != torch.float32:
+        t = t.to(device=device, dtype=torch.float32)
+    if tuple(t.shape) != tuple(shape):
+        raise RuntimeError(f"partial image plane has shape {tuple(t.shape)}, expected {tuple(shape)}")
+    return t.contiguous()
+
+
+class _CompositePartialImages(torch.autograd.Function):
+    """apply(background_or_None, K, image_0.., depth_0.., alpha_0..) -> (image, depth, alpha)."""
+
+    @staticmethod
+    def forward(ctx, background, K, *planes):
+        images, depths, alphas = planes[:K], planes[K:2 * K], planes[2 * K:3 * K]
+        device = images[0].device
+        if not images[0].is_cuda:
+            raise RuntimeError("the compositor needs its inputs on a GPU (device memory)")
+        H, W = int(images[0].shape[-2]), int(images[0].shape[-1])
+        images = [_prep(t, device, (3, H, W)) for t in images]
+        depths = [_prep(t, device, (1, H, W)) for t in depths]
+        alphas = [_prep(t, device, (1, H, W)) for t in alphas]
+        bg = None if background is None else _prep(background.reshape(-1), device, (3,))
+        out_image = torch.empty((3, H, W), dtype=torch.float32, device=device)
+        out_depth = torch.empty((1, H, W), dtype=torch.float32, device=device)
+        out_alpha = torch.empty((1, H, W), dtype=torch.float32, device=device)
+        with torch.cuda.device(device):
+            check(lib.rgs_composite_forward(
+                K, H, W, ptr_table(images), ptr_table(depths), ptr_table(alphas), ptr(bg), ptr(out_image),
+                ptr(out_depth), ptr(out_alpha), C.c_void_p(torch.cuda.current_stream(device).cuda_stream)))
+        ctx.K, ctx.hw = K, (H, W)
+        ctx.has_bg = bg is not None
+        ctx.save_for_backward(*(images + depths + alphas + ([bg] if bg is not None else [])))
+        return out_image, out_depth, out_alpha
+
+    @staticmethod
+    def backward(ctx, g_image, g_depth, g_alpha):
+        K, (H, W) = ctx.K, ctx.hw
+        saved = ctx.saved_tensors
+        images, depths, alphas = list(saved[:K]), list(saved[K:2 * K]), list(saved[2 * K:3 * K])
+        bg = saved[3 * K] if ctx.has_bg else None
+        device = images[0].device
+        f32 = dict(dtype=torch.float32, device=device)
+        g_image = torch.zeros((3, H, W), **f32) if g_image is None else _prep(g_image, device, (3, H, W))
+        g_depth = None if g_depth is None else _prep(g_depth, device, (1, H, W))
+        g_alpha = None if g_alpha is None else _prep(g_alpha, device, (1, H, W))
+        d_images = [torch.empty((3, H, W), **f32) for _ in range(K)]
+        d_depths = [torch.empty((1, H, W), **f32) for _ in range(K)]
+        d_alphas = [torch.empty((1, H, W), **f32) for _ in range(K)]
+        with torch.cuda.device(device):
+            check(lib.rgs_composite_backward(
+                K, H, W, ptr_table(images), ptr_table(depths), ptr_table(alphas), ptr(bg), ptr(g_image), ptr(g_depth),
+                ptr(g_alpha), ptr_table(d_images), ptr_table(d_depths), ptr_table(d_alphas),
+                C.c_void_p(torch.cuda.current_stream(device).cuda_stream)))
+        # The reference's background is a constant (or a fresh random tensor); it gets no gradient.
+        return (None, None, *d_images, *d_depths, *d_alphas)
+
+
+def composite_partial_images(images: Sequence[torch.Tensor], depths: Sequence[torch.Tensor],
+                             alphas: Sequence[torch.Tensor], background: Optional[torch.Tensor] = None):
+    """Composite K partial images that are already in front-to-back order.
+    images[k]: (3,H,W); depths[k], alphas[k]: (1,H,W).  Returns (image, depth, alpha).
+    More than MAX_COMPOSITE inputs are folded in groups: compositing is associative in
+    (image, depth, alpha) when the inner groups use a black background."""
+    K = len(images)
+    if K == 0 or len(depths) != K or len(alphas) != K:
+        raise RuntimeError("composite_partial_images needs K >= 1 images, depths and alphas")
+    images, depths, alphas = list(images), list(depths), list(alphas)
+    while len(images) > _capi.MAX_COMPOSITE:
+        n = _capi.MAX_COMPOSITE
+        img, dep, alp = _CompositePartialImages.apply(None, n, *images[:n], *depths[:n], *alphas[:n])
+        images, depths, alphas = [img] + images[n:], [dep] + depths[n:], [alp] + alphas[n:]
+    K = len(images)
+    return _CompositePartialImages.apply(background, K, *images, *depths, *alphas)
+
+
+def blender_render_result(render_results: Dict[int, dict], relation_vector, background: Optional[torch.Tensor]):
+    """Same contract as the reference function of this name
+    (parallel_utils/basic_parallel_trainer/result_aggregator.py:193-260) for one camera on
+    one GPU: `render_results` maps submodel id -> {"render","depth","alpha"} (what
+    render4renderinfo returns), `relation_vector[model_id]` is the compositing rank of that
+    submodel or a negative value when it is not related to the camera.  Returns a dict with
+    "render", "depth", "alpha".  A missing background draws a random colour, like the
+    reference (:256)."""
+    if isinstance(relation_vector, torch.Tensor):
+        relation_vector = relation_vector.cpu().numpy()
+    related = [(int(relation_vector[m]), m) for m in render_results if relation_vector[m] >= 0]
+    num_related = int(sum(1 for v in relation_vector if v >= 0))
+    if len(related) != num_related:
+        raise RuntimeError("NUM_RELATED mis-match")
+    related.sort(key=lambda x: x[0])
+    pk = [render_results[m] for _, m in related]
+    device = pk[0]["render"].device
+    bkg = background if background is not None else torch.rand((3,), device=device)
+    image, depth, alpha = composite_partial_images([p["render"] for p in pk], [p["depth"] for p in pk],
+                                                   [p["alpha"] for p in pk], bkg)
+    return {"render": image, "depth": depth, "alpha": alpha}

@@ -1,0 +1,533 @@
+// extern "C" surface of librgs_gfx950.so: argument checks, workspace carving, stage
+// sequencing and error reporting.  The declarations and the reference interfaces they
+// replace are in include/rgs.h.
+#include "../../include/rgs.h"
+#include "rgs_kernels.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(const char* fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_error, sizeof(g_error), fmt, ap);
+	va_end(ap);
+	return 1;
+}
+
+#define RGS_REQUIRE(cond, ...)          \
+	do {                                \
+		if (!(cond))                    \
+			return fail(__VA_ARGS__);   \
+	} while (0)
+
+// Launch errors are cheap to poll; in debug mode every stage is also synchronised, which
+// is where the reference's CHECK_CUDA does its cudaDeviceSynchronize.
+int check_stage(const char* stage, hipStream_t s, int debug)
+{
+	hipError_t e = hipGetLastError();
+	if (e == hipSuccess && debug)
+		e = hipStreamSynchronize(s);
+	if (e != hipSuccess)
+		return fail("%s: %s", stage, hipGetErrorString(e));
+	return 0;
+}
+
+#define RGS_STAGE(name)                               \
+	do {                                              \
+		if (int rc_ = check_stage(name, s, debug))    \
+			return rc_;                               \
+	} while (0)
+
+constexpr size_t kAlign = 256;
+
+size_t align_up(size_t v)
+{
+	return (v + kAlign - 1) & ~(kAlign - 1);
+}
+
+struct Carver {
+	size_t cursor = 0;
+	size_t take(size_t bytes)
+	{
+		const size_t at = cursor;
+		cursor = align_up(cursor + bytes);
+		return at;
+	}
+};
+
+size_t geom_layout(size_t P, size_t* off)
+{
+	Carver c;
+	off[RGS_GEOM_DEPTHS] = c.take(4 * P);
+	off[RGS_GEOM_XY] = c.take(8 * P);
+	off[RGS_GEOM_CLIP_W] = c.take(4 * P);
+	off[RGS_GEOM_COV3D] = c.take(24 * P);
+	off[RGS_GEOM_CONIC_OPACITY] = c.take(16 * P);
+	off[RGS_GEOM_RGB] = c.take(12 * P);
+	off[RGS_GEOM_TILES_TOUCHED] = c.take(4 * P);
+	off[RGS_GEOM_POINT_OFFSETS] = c.take(4 * P);
+	off[RGS_GEOM_CLAMPED] = c.take(P);
+	off[RGS_GEOM_BLOCK_SUMS] = c.take(4 * ((P + 255) / 256 + 1));
+	off[RGS_GEOM_TOTAL] = c.take(4);
+	return c.cursor;
+}
+
+int sort_end_bit(int width, int height)
+{
+	const uint32_t tiles = (uint32_t)((width + rgs::kTile - 1) / rgs::kTile) * (uint32_t)((height + rgs::kTile - 1) / rgs::kTile);
+	return 32 + (int)rgs_get_higher_msb(tiles);
+}
+
+// Physical buffers: A receives the duplicated keys, B is its ping-pong partner.
+struct BinningPhysical {
+	size_t keys_a, keys_b, vals_a, vals_b, temp, total;
+};
+
+BinningPhysical binning_physical(size_t R)
+{
+	Carver c;
+	BinningPhysical b;
+	b.keys_a = c.take(8 * R);
+	b.keys_b = c.take(8 * R);
+	b.vals_a = c.take(4 * R);
+	b.vals_b = c.take(4 * R);
+	b.temp = c.take(4 * rgs::sort_temp_words(R));
+	b.total = c.cursor;
+	return b;
+}
+
+size_t image_layout(int width, int height, size_t* off)
+{
+	const size_t tiles = (size_t)((width + rgs::kTile - 1) / rgs::kTile) * (size_t)((height + rgs::kTile - 1) / rgs::kTile);
+	Carver c;
+	off[RGS_IMG_RANGES] = c.take(8 * tiles);
+	off[RGS_IMG_N_CONTRIB] = c.take(4 * (size_t)width * height);
+	return c.cursor;
+}
+
+template <typename T>
+T* at(void* base, size_t off)
+{
+	return reinterpret_cast<T*>(static_cast<char*>(base) + off);
+}
+template <typename T>
+const T* at(const void* base, size_t off)
+{
+	return reinterpret_cast<const T*>(static_cast<const char*>(base) + off);
+}
+
+}  // namespace
+
+extern "C" {
+
+int rgs_version(void)
+{
+	return 100;
+}
+
+const char* rgs_last_error(void)
+{
+	return g_error;
+}
+
+uint32_t rgs_get_higher_msb(uint32_t n)
+{
+	// Smallest b with (n >> b) == 0, found by the reference's halving search
+	// (K/cuda_rasterizer_hgs/rasterizer_impl.cu:35-50); both agree for every n.
+	uint32_t msb = 16, step = 16;
+	while (step > 1) {
+		step >>= 1;
+		msb = (n >> msb) ? msb + step : msb - step;
+	}
+	return (n >> msb) ? msb + 1 : msb;
+}
+
+size_t rgs_geom_bytes(int P)
+{
+	size_t off[RGS_GEOM_FIELDS];
+	return geom_layout(P > 0 ? (size_t)P : 0, off) + kAlign;
+}
+
+size_t rgs_binning_bytes(int R)
+{
+	return binning_physical(R > 0 ? (size_t)R : 0).total + kAlign;
+}
+
+size_t rgs_image_bytes(int width, int height)
+{
+	size_t off[RGS_IMG_FIELDS];
+	return image_layout(width, height, off) + kAlign;
+}
+
+int rgs_geom_layout(int P, size_t offsets[RGS_GEOM_FIELDS])
+{
+	RGS_REQUIRE(P >= 0 && offsets, "rgs_geom_layout: bad arguments");
+	geom_layout((size_t)P, offsets);
+	return 0;
+}
+
+int rgs_binning_layout(int R, int width, int height, size_t offsets[RGS_BIN_FIELDS])
+{
+	RGS_REQUIRE(R >= 0 && width > 0 && height > 0 && offsets, "rgs_binning_layout: bad arguments");
+	const BinningPhysical b = binning_physical((size_t)R);
+	const bool sorted_in_a = (((sort_end_bit(width, height) + 7) / 8) % 2) == 0;
+	offsets[RGS_BIN_KEYS_UNSORTED] = sorted_in_a ? b.keys_b : b.keys_a;
+	offsets[RGS_BIN_KEYS_SORTED] = sorted_in_a ? b.keys_a : b.keys_b;
+	offsets[RGS_BIN_VALUES_UNSORTED] = sorted_in_a ? b.vals_b : b.vals_a;
+	offsets[RGS_BIN_VALUES_SORTED] = sorted_in_a ? b.vals_a : b.vals_b;
+	offsets[RGS_BIN_SORT_TEMP] = b.temp;
+	return 0;
+}
+
+int rgs_image_layout(int width, int height, size_t offsets[RGS_IMG_FIELDS])
+{
+	RGS_REQUIRE(width > 0 && height > 0 && offsets, "rgs_image_layout: bad arguments");
+	image_layout(width, height, offsets);
+	return 0;
+}
+
+int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const float* projmatrix,
+                     uint8_t* present, void* stream)
+{
+	(void)projmatrix;
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const int debug = 0;
+	RGS_REQUIRE(P >= 0, "rgs_mark_visible: negative P");
+	if (P == 0)
+		return 0;
+	RGS_REQUIRE(means3D && viewmatrix && present, "rgs_mark_visible: null pointer");
+	rgs::launch_mark_visible(P, means3D, viewmatrix, present, s);
+	RGS_STAGE("mark_visible");
+	return 0;
+}
+
+int rgs_forward_geom(int P, int D, int M, int width, int height,
+                     const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
+                     const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                     const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                     float tan_fovx, float tan_fovy, int prefiltered,
+                     int* radii, void* geom_ws, size_t geom_bytes,
+                     uint32_t* num_rendered_host, void* stream, int debug)
+{
+	// `prefiltered` promises that no Gaussian is culled; the reference traps the device when
+	// the promise is broken (K/cuda_rasterizer_hgs/auxiliary.h:172-176).  Here a culled
+	// Gaussian is simply skipped.
+	(void)prefiltered;
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	RGS_REQUIRE(P > 0, "rgs_forward_geom: P must be positive (the caller short-circuits P == 0)");
+	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_geom: bad image size %dx%d", width, height);
+	RGS_REQUIRE(means3D && opacities && viewmatrix && projmatrix && cam_pos && radii && geom_ws && num_rendered_host,
+	            "rgs_forward_geom: null pointer");
+	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr),
+	            "rgs_forward_geom: provide exactly one of SHs or precomputed colours");
+	RGS_REQUIRE(((scales != nullptr) && (rotations != nullptr)) != (cov3D_precomp != nullptr) &&
+	                ((scales != nullptr) == (rotations != nullptr)),
+	            "rgs_forward_geom: provide exactly one of scale/rotation or precomputed 3D covariance");
+	RGS_REQUIRE(D >= 0 && D <= 3, "rgs_forward_geom: SH degree %d out of range", D);
+	RGS_REQUIRE(!shs || M >= (D + 1) * (D + 1), "rgs_forward_geom: %d SH coefficients cannot hold degree %d", M, D);
+	RGS_REQUIRE(geom_bytes >= rgs_geom_bytes(P), "rgs_forward_geom: geometry workspace too small");
+	RGS_REQUIRE((reinterpret_cast<uintptr_t>(geom_ws) & 15) == 0, "rgs_forward_geom: workspace must be 16-byte aligned");
+
+	size_t off[RGS_GEOM_FIELDS];
+	geom_layout((size_t)P, off);
+
+	rgs::PreprocessArgs a;
+	a.P = P; a.D = D; a.M = M;
+	a.means = means3D; a.scales = scales; a.scale_modifier = scale_modifier; a.rotations = rotations;
+	a.opacities = opacities; a.shs = shs; a.cov3D_precomp = cov3D_precomp; a.colors_precomp = colors_precomp;
+	a.view = viewmatrix; a.proj = projmatrix; a.campos = cam_pos;
+	a.W = width; a.H = height;
+	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
+	// K/cuda_rasterizer_hgs/rasterizer_impl.cu:227-228
+	a.focal_y = height / (2.0f * tan_fovy);
+	a.focal_x = width / (2.0f * tan_fovx);
+	a.grid_x = (width + rgs::kTile - 1) / rgs::kTile;
+	a.grid_y = (height + rgs::kTile - 1) / rgs::kTile;
+	a.radii = radii;
+	a.xy = at<float2>(geom_ws, off[RGS_GEOM_XY]);
+	a.clip_w = at<float>(geom_ws, off[RGS_GEOM_CLIP_W]);
+	a.depths = at<float>(geom_ws, off[RGS_GEOM_DEPTHS]);
+	a.cov3D = at<float>(geom_ws, off[RGS_GEOM_COV3D]);
+	a.rgb = at<float>(geom_ws, off[RGS_GEOM_RGB]);
+	a.conic_opacity = at<float4>(geom_ws, off[RGS_GEOM_CONIC_OPACITY]);
+	a.tiles_touched = at<uint32_t>(geom_ws, off[RGS_GEOM_TILES_TOUCHED]);
+	a.clamped = at<uint8_t>(geom_ws, off[RGS_GEOM_CLAMPED]);
+	a.block_sums = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_SUMS]);
+
+	rgs::launch_preprocess_forward(a, s);
+	RGS_STAGE("preprocess");
+	rgs::launch_offsets_from_block_sums(a.tiles_touched, a.block_sums, at<uint32_t>(geom_ws, off[RGS_GEOM_POINT_OFFSETS]),
+	                                    P, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), s);
+	RGS_STAGE("offset scan");
+
+	hipError_t e = hipMemcpyAsync(num_rendered_host, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), sizeof(uint32_t),
+	                              hipMemcpyDeviceToHost, s);
+	if (e == hipSuccess)
+		e = hipStreamSynchronize(s);
+	if (e != hipSuccess)
+		return fail("rgs_forward_geom: reading the instance count failed: %s", hipGetErrorString(e));
+	RGS_REQUIRE(*num_rendered_host < 0x80000000u,
+	            "rgs_forward_geom: %u (Gaussian, tile) instances exceed the 2^31 limit of the sort", *num_rendered_host);
+	return 0;
+}
+
+int rgs_forward_raster(int P, int R, int width, int height,
+                       const float* background, float tan_fovx, float tan_fovy,
+                       const float* projmatrix_inv, const float* range_low, const float* range_up,
+                       const float* colors_precomp, const int* radii,
+                       void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                       void* image_ws, size_t image_bytes,
+                       float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	RGS_REQUIRE(P > 0 && R >= 0, "rgs_forward_raster: bad sizes P=%d R=%d", P, R);
+	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_raster: bad image size %dx%d", width, height);
+	RGS_REQUIRE(background && projmatrix_inv && range_low && range_up && radii && geom_ws && image_ws && out_color &&
+	                out_depth && out_alpha,
+	            "rgs_forward_raster: null pointer");
+	RGS_REQUIRE(R == 0 || binning_ws, "rgs_forward_raster: null binning workspace");
+	RGS_REQUIRE(geom_bytes >= rgs_geom_bytes(P), "rgs_forward_raster: geometry workspace too small");
+	RGS_REQUIRE(R == 0 || binning_bytes >= rgs_binning_bytes(R), "rgs_forward_raster: binning workspace too small");
+	RGS_REQUIRE(image_bytes >= rgs_image_bytes(width, height), "rgs_forward_raster: image workspace too small");
+
+	size_t goff[RGS_GEOM_FIELDS], ioff[RGS_IMG_FIELDS];
+	geom_layout((size_t)P, goff);
+	image_layout(width, height, ioff);
+	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
+	uint2* ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
+	const uint32_t* point_list = nullptr;
+
+	if (R > 0) {
+		const BinningPhysical b = binning_physical((size_t)R);
+		uint64_t* keys_a = at<uint64_t>(binning_ws, b.keys_a);
+		uint64_t* keys_b = at<uint64_t>(binning_ws, b.keys_b);
+		uint32_t* vals_a = at<uint32_t>(binning_ws, b.vals_a);
+		uint32_t* vals_b = at<uint32_t>(binning_ws, b.vals_b);
+		rgs::launch_duplicate_with_keys(P, at<float2>(geom_ws, goff[RGS_GEOM_XY]), at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]),
+		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_POINT_OFFSETS]), radii, gx, gy, keys_a, vals_a, s);
+		RGS_STAGE("duplicate_with_keys");
+		const int end_bit = sort_end_bit(width, height);
+		rgs::launch_sort_pairs(keys_a, keys_b, vals_a, vals_b, (size_t)R, end_bit, at<uint32_t>(binning_ws, b.temp), s);
+		RGS_STAGE("sort_pairs");
+		const bool sorted_in_a = (((end_bit + 7) / 8) % 2) == 0;
+		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, ranges, gx * gy, s);
+		RGS_STAGE("tile_ranges");
+		point_list = sorted_in_a ? vals_a : vals_b;
+	} else {
+		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, s);
+		RGS_STAGE("tile_ranges");
+	}
+
+	rgs::BlendArgs a;
+	memset(&a, 0, sizeof(a));
+	a.ranges = ranges;
+	a.point_list = point_list;
+	a.W = width; a.H = height; a.grid_x = gx; a.grid_y = gy;
+	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
+	a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up; a.bg = background;
+	a.xy = at<float2>(geom_ws, goff[RGS_GEOM_XY]);
+	a.clip_w = at<float>(geom_ws, goff[RGS_GEOM_CLIP_W]);
+	a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
+	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
+	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
+	a.out_color = out_color; a.out_depth = out_depth; a.out_alpha = out_alpha;
+	a.n_contrib = at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]);
+	rgs::launch_blend_forward(a, s);
+	RGS_STAGE("blend_forward");
+	return 0;
+}
+
+int rgs_backward(int P, int D, int M, int R, int width, int height,
+                 const float* background, const float* means3D, const float* shs, const float* colors_precomp,
+                 const float* alphas, const float* scales, float scale_modifier, const float* rotations,
+                 const float* cov3D_precomp, const float* viewmatrix, const float* projmatrix,
+                 const float* projmatrix_inv, const float* range_low, const float* range_up, const float* cam_pos,
+                 float tan_fovx, float tan_fovy, const int* radii,
+                 const void* geom_ws, const void* binning_ws, const void* image_ws,
+                 const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
+                 float* grad_accum, float* dL_dmean3D, float* dL_dcov3D, float* dL_dsh, float* dL_dscale,
+                 float* dL_drot, void* stream, int debug)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	RGS_REQUIRE(P > 0 && R >= 0, "rgs_backward: bad sizes P=%d R=%d", P, R);
+	RGS_REQUIRE(width > 0 && height > 0, "rgs_backward: bad image size %dx%d", width, height);
+	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
+	                cam_pos && radii && geom_ws && image_ws && dL_dpix && dL_dpix_depth && dL_dalphas && grad_accum &&
+	                dL_dmean3D && dL_dcov3D,
+	            "rgs_backward: null pointer");
+	RGS_REQUIRE(R == 0 || binning_ws, "rgs_backward: null binning workspace");
+	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr), "rgs_backward: provide exactly one of SHs or colours");
+	RGS_REQUIRE(!shs || dL_dsh, "rgs_backward: dL_dsh is required with SHs");
+	RGS_REQUIRE(!scales || (rotations && dL_dscale && dL_drot), "rgs_backward: scale/rotation outputs missing");
+	RGS_REQUIRE(scales || cov3D_precomp, "rgs_backward: neither scales nor precomputed covariance");
+
+	size_t goff[RGS_GEOM_FIELDS], ioff[RGS_IMG_FIELDS];
+	geom_layout((size_t)P, goff);
+	image_layout(width, height, ioff);
+	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
+	const size_t n = (size_t)P;
+
+	rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, RGS_ACC_FLOATS * n, s);
+	RGS_STAGE("clear gradient sums");
+
+	const float* colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
+	if (R > 0) {
+		const BinningPhysical b = binning_physical((size_t)R);
+		const bool sorted_in_a = (((sort_end_bit(width, height) + 7) / 8) % 2) == 0;
+		rgs::BlendArgs a;
+		memset(&a, 0, sizeof(a));
+		a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
+		a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
+		a.W = width; a.H = height; a.grid_x = gx; a.grid_y = gy;
+		a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
+		a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up; a.bg = background;
+		a.xy = at<float2>(geom_ws, goff[RGS_GEOM_XY]);
+		a.clip_w = at<float>(geom_ws, goff[RGS_GEOM_CLIP_W]);
+		a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
+		a.colors = colors;
+		a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
+		a.out_alpha = const_cast<float*>(alphas);
+		a.n_contrib = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]));
+		a.dL_dpix = dL_dpix; a.dL_dpix_depth = dL_dpix_depth; a.dL_dalpha = dL_dalphas;
+		a.dL_dmean2D = grad_accum + RGS_ACC_MEAN2D * n;
+		a.dL_dconic = grad_accum + RGS_ACC_CONIC * n;
+		a.dL_dopacity = grad_accum + RGS_ACC_OPACITY * n;
+		a.dL_dcolors = grad_accum + RGS_ACC_COLOR * n;
+		a.dL_ddepths = grad_accum + RGS_ACC_DEPTH * n;
+		rgs::launch_blend_backward(a, s);
+		RGS_STAGE("blend_backward");
+	}
+
+	rgs::PreprocessBackwardArgs p;
+	memset(&p, 0, sizeof(p));
+	p.P = P; p.D = D; p.M = M;
+	p.means = means3D; p.radii = radii; p.shs = shs;
+	p.clamped = at<uint8_t>(geom_ws, goff[RGS_GEOM_CLAMPED]);
+	p.scales = scales; p.rotations = rotations; p.scale_modifier = scale_modifier;
+	p.cov3D = cov3D_precomp ? cov3D_precomp : at<float>(geom_ws, goff[RGS_GEOM_COV3D]);
+	p.view = viewmatrix; p.proj = projmatrix; p.campos = cam_pos;
+	p.focal_y = height / (2.0f * tan_fovy);
+	p.focal_x = width / (2.0f * tan_fovx);
+	p.tanfovx = tan_fovx; p.tanfovy = tan_fovy;
+	p.dL_dmean2D = grad_accum + RGS_ACC_MEAN2D * n;
+	p.dL_dconic = grad_accum + RGS_ACC_CONIC * n;
+	p.dL_dcolor = grad_accum + RGS_ACC_COLOR * n;
+	p.dL_ddepth = grad_accum + RGS_ACC_DEPTH * n;
+	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
+	rgs::launch_preprocess_backward(p, s);
+	RGS_STAGE("preprocess_backward");
+	return 0;
+}
+
+size_t rgs_scan_temp_bytes(size_t n)
+{
+	return 4 * rgs::scan_temp_words(n);
+}
+
+int rgs_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, void* temp, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const int debug = 0;
+	if (n == 0)
+		return 0;
+	RGS_REQUIRE(in && out && temp, "rgs_inclusive_sum: null pointer");
+	RGS_REQUIRE(n < ((size_t)1 << 38), "rgs_inclusive_sum: n too large");
+	rgs::launch_inclusive_sum(in, out, n, static_cast<uint32_t*>(temp), s);
+	RGS_STAGE("inclusive_sum");
+	return 0;
+}
+
+size_t rgs_sort_temp_bytes(size_t n)
+{
+	return 4 * rgs::sort_temp_words(n);
+}
+
+int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                   int end_bit, void* temp, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const int debug = 0;
+	RGS_REQUIRE(end_bit >= 1 && end_bit <= 64, "rgs_sort_pairs: end_bit %d out of range", end_bit);
+	if (n == 0)
+		return 0;
+	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out && temp, "rgs_sort_pairs: null pointer");
+	RGS_REQUIRE(n < 0x80000000ull, "rgs_sort_pairs: more than 2^31 pairs");
+	rgs::launch_sort_pairs(keys_in, keys_out, vals_in, vals_out, n, end_bit, static_cast<uint32_t*>(temp), s);
+	RGS_STAGE("sort_pairs");
+	if ((((end_bit + 7) / 8) % 2) == 0) {
+		// An even number of passes leaves the result in the input buffers; hand it over.
+		hipError_t e = hipMemcpyAsync(keys_out, keys_in, n * sizeof(uint64_t), hipMemcpyDeviceToDevice, s);
+		if (e == hipSuccess)
+			e = hipMemcpyAsync(vals_out, vals_in, n * sizeof(uint32_t), hipMemcpyDeviceToDevice, s);
+		if (e != hipSuccess)
+			return fail("rgs_sort_pairs: copy failed: %s", hipGetErrorString(e));
+	}
+	return 0;
+}
+
+static int fill_composite(rgs::CompositeArgs& a, int K, int height, int width, const float* const* images,
+                          const float* const* depths, const float* const* alphas, const float* background)
+{
+	RGS_REQUIRE(K >= 1 && K <= RGS_MAX_COMPOSITE, "composite: K=%d outside 1..%d", K, RGS_MAX_COMPOSITE);
+	RGS_REQUIRE(height > 0 && width > 0, "composite: bad image size %dx%d", width, height);
+	RGS_REQUIRE(images && depths && alphas, "composite: null pointer table");
+	memset(&a, 0, sizeof(a));
+	a.K = K; a.H = height; a.W = width; a.bg = background;
+	for (int k = 0; k < K; k++) {
+		RGS_REQUIRE(images[k] && depths[k] && alphas[k], "composite: null input plane at k=%d", k);
+		a.images[k] = images[k];
+		a.depths[k] = depths[k];
+		a.alphas[k] = alphas[k];
+	}
+	return 0;
+}
+
+int rgs_composite_forward(int K, int height, int width,
+                          const float* const* images, const float* const* depths, const float* const* alphas,
+                          const float* background, float* out_image, float* out_depth, float* out_alpha,
+                          void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const int debug = 0;
+	rgs::CompositeArgs a;
+	if (int rc = fill_composite(a, K, height, width, images, depths, alphas, background))
+		return rc;
+	RGS_REQUIRE(out_image && out_depth && out_alpha, "rgs_composite_forward: null output");
+	a.out_image = out_image; a.out_depth = out_depth; a.out_alpha = out_alpha;
+	rgs::launch_composite_forward(a, s);
+	RGS_STAGE("composite_forward");
+	return 0;
+}
+
+int rgs_composite_backward(int K, int height, int width,
+                           const float* const* images, const float* const* depths, const float* const* alphas,
+                           const float* background, const float* g_image, const float* g_depth,
+                           const float* g_alpha, float* const* d_images, float* const* d_depths,
+                           float* const* d_alphas, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const int debug = 0;
+	rgs::CompositeArgs a;
+	if (int rc = fill_composite(a, K, height, width, images, depths, alphas, background))
+		return rc;
+	RGS_REQUIRE(g_image && d_images && d_depths && d_alphas, "rgs_composite_backward: null pointer");
+	a.g_image = g_image; a.g_depth = g_depth; a.g_alpha = g_alpha;
+	for (int k = 0; k < K; k++) {
+		RGS_REQUIRE(d_images[k] && d_depths[k] && d_alphas[k], "rgs_composite_backward: null output plane at k=%d", k);
+		a.d_images[k] = d_images[k];
+		a.d_depths[k] = d_depths[k];
+		a.d_alphas[k] = d_alphas[k];
+	}
+	rgs::launch_composite_backward(a, s);
+	RGS_STAGE("composite_backward");
+	return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,344 @@
+// Binning stages: offset scan, (tile | depth) key duplication, stable 64-bit radix
+// sort and per-tile range extraction.  All integer work; results are bit-exact
+// by construction.  K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian.
+#include "rgs_kernels.h"
+
+namespace rgs {
+
+// ---- prefix sums ---------------------------------------------------------------------------
+// Replaces cub::DeviceScan::InclusiveSum at K/cuda_rasterizer_hgs/rasterizer_impl.cu:283
+// with three small kernels: per-256 block totals, one single-block scan of those totals,
+// and a per-block scan that adds the block's base.  The forward preprocess kernel already
+// emits the block totals, so the rasterizer path only runs the last two.
+
+__global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __restrict__ in, size_t n,
+                                                            uint32_t* __restrict__ totals)
+{
+	__shared__ uint32_t lds[8];
+	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+	const uint32_t v = i < n ? in[i] : 0u;
+	uint32_t total;
+	(void)block256_exclusive_scan_u32(v, lds, total);
+	if (threadIdx.x == 0)
+		totals[blockIdx.x] = total;
+}
+
+// In-place exclusive scan of `data[0..n)` by one block of 1024 threads; the grand total goes
+// to *total_out (if non-null).
+__global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(uint32_t* __restrict__ data, size_t n,
+                                                                            uint32_t* __restrict__ total_out)
+{
+	__shared__ uint32_t wave_tot[16];
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const size_t chunk = (n + 1023) / 1024;
+	const size_t lo = (size_t)tid * chunk;
+	const size_t hi = lo + chunk < n ? lo + chunk : n;
+	uint32_t sum = 0;
+	for (size_t i = lo; i < hi; i++)
+		sum += data[i];
+	const uint32_t inc = wave_inclusive_scan_u32(sum);
+	if (lane == 63)
+		wave_tot[wave] = inc;
+	__syncthreads();
+	uint32_t base = 0, total = 0;
+#pragma unroll
+	for (int w = 0; w < 16; w++) {
+		const uint32_t s = wave_tot[w];
+		if (w < wave)
+			base += s;
+		total += s;
+	}
+	uint32_t run = base + inc - sum;
+	for (size_t i = lo; i < hi; i++) {
+		const uint32_t v = data[i];
+		data[i] = run;
+		run += v;
+	}
+	if (tid == 0 && total_out)
+		*total_out = total;
+}
+
+__global__ __launch_bounds__(256) void block_inclusive_scan_kernel(const uint32_t* __restrict__ in,
+                                                                    const uint32_t* __restrict__ block_base, size_t n,
+                                                                    uint32_t* __restrict__ out)
+{
+	__shared__ uint32_t lds[8];
+	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+	const uint32_t v = i < n ? in[i] : 0u;
+	uint32_t total;
+	const uint32_t ex = block256_exclusive_scan_u32(v, lds, total);
+	if (i < n)
+		out[i] = block_base[blockIdx.x] + ex + v;
+}
+
+size_t scan_temp_words(size_t n)
+{
+	return (n + 255) / 256 + 1;
+}
+
+void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, hipStream_t s)
+{
+	if (n == 0)
+		return;
+	const size_t nb = (n + 255) / 256;
+	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, temp);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, nb, (uint32_t*)nullptr);
+	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, temp, n, out);
+}
+
+void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* block_sums, uint32_t* offsets, int P,
+                                    uint32_t* total_out, hipStream_t s)
+{
+	const size_t nb = ((size_t)P + 255) / 256;
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb, total_out);
+	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, tiles_touched, block_sums,
+	                   (size_t)P, offsets);
+}
+
+// ---- key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) ----------------------
+
+__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(int P, const float2* __restrict__ xy,
+                                                                   const float* __restrict__ depths,
+                                                                   const uint32_t* __restrict__ offsets,
+                                                                   const int* __restrict__ radii, int gx, int gy,
+                                                                   uint64_t* __restrict__ keys,
+                                                                   uint32_t* __restrict__ values)
+{
+	const int idx = blockIdx.x * 256 + threadIdx.x;
+	if (idx >= P)
+		return;
+	const int radius = radii[idx];
+	if (!(radius > 0))
+		return;
+	uint32_t off = (idx == 0) ? 0u : offsets[idx - 1];
+	const float2 p = xy[idx];
+	const TileRect rc = tile_rect(p.x, p.y, radius, gx, gy);
+	const uint64_t dbits = (uint64_t)__float_as_uint(depths[idx]);
+	for (uint32_t y = rc.y0; y < rc.y1; y++) {
+		for (uint32_t x = rc.x0; x < rc.x1; x++) {
+			const uint64_t key = ((uint64_t)(y * (uint32_t)gx + x) << 32) | dbits;
+			keys[off] = key;
+			values[off] = (uint32_t)idx;
+			off++;
+		}
+	}
+}
+
+void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, const uint32_t* offsets,
+                                const int* radii, int grid_x, int grid_y, uint64_t* keys, uint32_t* values,
+                                hipStream_t s)
+{
+	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, P, xy, depths, offsets,
+	                   radii, grid_x, grid_y, keys, values);
+}
+
+// ---- radix sort -------------------------------------------------------------------------------
+// Replaces cub::DeviceRadixSort::SortPairs at K/cuda_rasterizer_hgs/rasterizer_impl.cu:312-317:
+// a stable least-significant-digit sort of (u64 key, u32 value) on key bits [0, end_bit),
+// 8 bits per pass.  Each pass: per-block digit histogram -> one scan of the
+// (digit-major) block x digit table -> rank-and-scatter.  A sort block owns kSortBlock
+// consecutive pairs; element order inside the block is (wave, round, lane), and ranking
+// preserves it, which makes every pass stable.
+
+__device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t mask)
+{
+	return (uint32_t)(key >> shift) & mask;
+}
+
+__global__ __launch_bounds__(256) void sort_histogram_kernel(const uint64_t* __restrict__ keys, size_t n, int shift,
+                                                              uint32_t mask, uint32_t* __restrict__ table,
+                                                              uint32_t nblocks)
+{
+	__shared__ uint32_t hist[256];
+	hist[threadIdx.x] = 0;
+	__syncthreads();
+	const size_t base = (size_t)blockIdx.x * kSortBlock;
+#pragma unroll 4
+	for (int i = 0; i < kSortItems; i++) {
+		const size_t k = base + (size_t)i * 256 + threadIdx.x;
+		if (k < n)
+			atomicAdd(&hist[digit_of(keys[k], shift, mask)], 1u);
+	}
+	__syncthreads();
+	table[(size_t)threadIdx.x * nblocks + blockIdx.x] = hist[threadIdx.x];
+}
+
+__global__ __launch_bounds__(256) void sort_scatter_kernel(const uint64_t* __restrict__ keys_in,
+                                                            const uint32_t* __restrict__ vals_in,
+                                                            uint64_t* __restrict__ keys_out,
+                                                            uint32_t* __restrict__ vals_out, size_t n, int shift,
+                                                            uint32_t mask, const uint32_t* __restrict__ table,
+                                                            uint32_t nblocks)
+{
+	__shared__ uint64_t s_keys[kSortBlock];
+	__shared__ uint32_t s_vals[kSortBlock];
+	__shared__ uint32_t s_wave_hist[4][256];  // per-wave digit counts, then exclusive prefix over waves
+	__shared__ uint32_t s_digit_base[256];    // exclusive prefix over digits within the block
+	__shared__ uint32_t s_global_base[256];   // where this block's run of each digit starts globally
+	__shared__ uint32_t s_scan[8];
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const size_t block_base = (size_t)blockIdx.x * kSortBlock;
+	const size_t wave_base = block_base + (size_t)wave * (kSortItems * 64);
+
+#pragma unroll
+	for (int w = 0; w < 4; w++)
+		s_wave_hist[w][tid] = 0;
+	s_global_base[tid] = table[(size_t)tid * nblocks + blockIdx.x];
+	__syncthreads();
+
+	uint64_t key[kSortItems];
+	uint32_t val[kSortItems];
+	uint32_t rank[kSortItems];
+#pragma unroll
+	for (int i = 0; i < kSortItems; i++) {
+		const size_t k = wave_base + (size_t)i * 64 + lane;
+		const bool ok = k < n;
+		key[i] = ok ? keys_in[k] : ~0ull;
+		val[i] = ok ? vals_in[k] : 0u;
+	}
+
+	const uint64_t lanes_below = (1ull << lane) - 1ull;
+#pragma unroll
+	for (int i = 0; i < kSortItems; i++) {
+		const size_t k = wave_base + (size_t)i * 64 + lane;
+		// Padding elements rank as digit 255 after every real element, so they never disturb one.
+		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : 255u;
+		uint64_t same = ~0ull;
+#pragma unroll
+		for (int b = 0; b < 8; b++) {
+			const bool bit = (d >> b) & 1u;
+			const uint64_t vote = __ballot(bit);
+			same &= bit ? vote : ~vote;
+		}
+		const uint32_t below = (uint32_t)__popcll(same & lanes_below);
+		const uint32_t count = (uint32_t)__popcll(same);
+		const int leader = __ffsll((unsigned long long)same) - 1;
+		uint32_t prior = 0;
+		if (lane == leader) {
+			prior = s_wave_hist[wave][d];
+			s_wave_hist[wave][d] = prior + count;
+		}
+		prior = __shfl(prior, leader);
+		rank[i] = prior + below;
+		__builtin_amdgcn_wave_barrier();
+	}
+	__syncthreads();
+
+	// Per digit: exclusive prefix over the 4 waves, block total, then exclusive prefix over digits.
+	{
+		const uint32_t c0 = s_wave_hist[0][tid], c1 = s_wave_hist[1][tid], c2 = s_wave_hist[2][tid],
+		               c3 = s_wave_hist[3][tid];
+		s_wave_hist[0][tid] = 0;
+		s_wave_hist[1][tid] = c0;
+		s_wave_hist[2][tid] = c0 + c1;
+		s_wave_hist[3][tid] = c0 + c1 + c2;
+		uint32_t total;
+		const uint32_t ex = block256_exclusive_scan_u32(c0 + c1 + c2 + c3, s_scan, total);
+		s_digit_base[tid] = ex;
+	}
+	__syncthreads();
+
+#pragma unroll
+	for (int i = 0; i < kSortItems; i++) {
+		const size_t k = wave_base + (size_t)i * 64 + lane;
+		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : 255u;
+		const uint32_t pos = s_digit_base[d] + s_wave_hist[wave][d] + rank[i];
+		s_keys[pos] = key[i];
+		s_vals[pos] = val[i];
+	}
+	__syncthreads();
+
+	const size_t remaining = n - block_base;
+	const uint32_t valid = remaining < (size_t)kSortBlock ? (uint32_t)remaining : (uint32_t)kSortBlock;
+#pragma unroll 4
+	for (int i = 0; i < kSortItems; i++) {
+		const uint32_t p = (uint32_t)i * 256 + tid;
+		if (p < valid) {
+			const uint64_t kk = s_keys[p];
+			const uint32_t d = digit_of(kk, shift, mask);
+			const size_t dst = (size_t)s_global_base[d] + (p - s_digit_base[d]);
+			keys_out[dst] = kk;
+			vals_out[dst] = s_vals[p];
+		}
+	}
+}
+
+size_t sort_temp_words(size_t n)
+{
+	const size_t nblocks = (n + kSortBlock - 1) / kSortBlock;
+	return 256 * (nblocks > 0 ? nblocks : 1) + 64;
+}
+
+// Returns 0 when the sorted pairs end in keys_out/vals_out, 1 when they end in keys_in/vals_in.
+int sort_pairs_passes(int end_bit)
+{
+	return (end_bit + 7) / 8;
+}
+
+void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                       int end_bit, uint32_t* temp, hipStream_t s)
+{
+	if (n == 0)
+		return;
+	const uint32_t nblocks = (uint32_t)((n + kSortBlock - 1) / kSortBlock);
+	uint64_t *ksrc = keys_in, *kdst = keys_out;
+	uint32_t *vsrc = vals_in, *vdst = vals_out;
+	for (int shift = 0; shift < end_bit; shift += 8) {
+		const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+		const uint32_t mask = (1u << bits) - 1u;
+		hipLaunchKernelGGL(sort_histogram_kernel, dim3(nblocks), dim3(256), 0, s, ksrc, n, shift, mask, temp, nblocks);
+		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, (size_t)256 * nblocks,
+		                   (uint32_t*)nullptr);
+		hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, shift, mask,
+		                   temp, nblocks);
+		uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
+		uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
+	}
+}
+
+// ---- tile ranges (K/cuda_rasterizer_hgs/rasterizer_impl.cu:116-138 and the memset at :319) ----
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t v, size_t n)
+{
+	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (i < n)
+		p[i] = v;
+}
+
+void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
+{
+	if (n == 0)
+		return;
+	hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, v, n);
+}
+
+__global__ __launch_bounds__(256) void tile_ranges_kernel(const uint64_t* __restrict__ keys, size_t n,
+                                                           uint2* __restrict__ ranges)
+{
+	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= n)
+		return;
+	const uint32_t cur = (uint32_t)(keys[idx] >> 32);
+	if (idx == 0) {
+		ranges[cur].x = 0;
+	} else {
+		const uint32_t prev = (uint32_t)(keys[idx - 1] >> 32);
+		if (cur != prev) {
+			ranges[prev].y = (uint32_t)idx;
+			ranges[cur].x = (uint32_t)idx;
+		}
+	}
+	if (idx == n - 1)
+		ranges[cur].y = (uint32_t)n;
+}
+
+void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, hipStream_t s)
+{
+	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2, s);
+	if (n == 0)
+		return;
+	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges);
+}
+
+}  // namespace rgs

@@ -1,0 +1,144 @@
+// Argument blocks and launcher prototypes shared between the kernel files and the
+// C-ABI layer.  All pointers are device pointers unless a comment says otherwise.
+#pragma once
+#include "rgs_device.h"
+
+namespace rgs {
+
+constexpr int kMaxComposite = 64;  // most partial images one composite call can take
+
+struct PreprocessArgs {
+	int P, D, M;
+	const float* means;
+	const float* scales;
+	float scale_modifier;
+	const float* rotations;
+	const float* opacities;
+	const float* shs;
+	const float* cov3D_precomp;   // may be null
+	const float* colors_precomp;  // may be null
+	const float* view;
+	const float* proj;
+	const float* campos;
+	int W, H;
+	float tanfovx, tanfovy, focal_x, focal_y;
+	int grid_x, grid_y;
+	// outputs
+	int* radii;
+	float2* xy;
+	float* clip_w;
+	float* depths;
+	float* cov3D;
+	float* rgb;
+	float4* conic_opacity;
+	uint32_t* tiles_touched;
+	uint8_t* clamped;
+	uint32_t* block_sums;  // one per 256 Gaussians
+};
+
+struct PreprocessBackwardArgs {
+	int P, D, M;
+	const float* means;
+	const int* radii;
+	const float* shs;      // may be null
+	const uint8_t* clamped;
+	const float* scales;   // may be null
+	const float* rotations;
+	float scale_modifier;
+	const float* cov3D;
+	const float* view;
+	const float* proj;
+	const float* campos;
+	float focal_x, focal_y, tanfovx, tanfovy;
+	const float* dL_dmean2D;  // (P,3)
+	const float* dL_dconic;   // (P,4)
+	const float* dL_dcolor;   // (P,3)
+	const float* dL_ddepth;   // (P)
+	// outputs, fully written
+	float* dL_dmeans;   // (P,3)
+	float* dL_dcov3D;   // (P,6)
+	float* dL_dsh;      // (P,M,3)
+	float* dL_dscale;   // (P,3)
+	float* dL_drot;     // (P,4)
+};
+
+struct BlendArgs {
+	const uint2* ranges;
+	const uint32_t* point_list;
+	int W, H, grid_x, grid_y;
+	float tanfovx, tanfovy;
+	const float* projinv;
+	const float* range_low;
+	const float* range_up;
+	const float* bg;
+	const float2* xy;
+	const float* clip_w;
+	const float4* conic_opacity;
+	const float* colors;  // (P,3)
+	const float* depths;
+	// forward outputs / backward inputs
+	float* out_color;
+	float* out_depth;
+	float* out_alpha;
+	uint32_t* n_contrib;
+	// backward
+	const float* dL_dpix;
+	const float* dL_dpix_depth;
+	const float* dL_dalpha;
+	float* dL_dmean2D;   // (P,3)
+	float* dL_dconic;    // (P,4)
+	float* dL_dopacity;  // (P)
+	float* dL_dcolors;   // (P,3)
+	float* dL_ddepths;   // (P)
+};
+
+struct CompositeArgs {
+	int K, H, W;
+	const float* bg;  // may be null (black)
+	const float* images[kMaxComposite];
+	const float* depths[kMaxComposite];
+	const float* alphas[kMaxComposite];
+	float* out_image;
+	float* out_depth;
+	float* out_alpha;
+	// backward
+	const float* g_image;
+	const float* g_depth;  // may be null
+	const float* g_alpha;  // may be null
+	float* d_images[kMaxComposite];
+	float* d_depths[kMaxComposite];
+	float* d_alphas[kMaxComposite];
+};
+
+// preprocess.hip
+void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s);
+void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s);
+void launch_preprocess_backward(const PreprocessBackwardArgs& a, hipStream_t s);
+
+// binning.hip
+constexpr int kSortItems = 16;                    // keys per thread in one sort block
+constexpr int kSortBlock = 256 * kSortItems;      // keys per sort block
+size_t scan_temp_words(size_t n);                 // u32 words of scratch for launch_inclusive_sum
+void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, hipStream_t s);
+void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* block_sums, uint32_t* offsets, int P,
+                                    uint32_t* total_out, hipStream_t s);
+void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, const uint32_t* offsets,
+                                const int* radii, int grid_x, int grid_y, uint64_t* keys, uint32_t* values,
+                                hipStream_t s);
+size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs
+// Stable LSD radix sort on key bits [0, end_bit).  Result lands in keys_out/vals_out;
+// keys_in/vals_in are overwritten (they serve as the ping-pong partner).
+void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                       int end_bit, uint32_t* temp, hipStream_t s);
+void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, hipStream_t s);
+
+// blend.hip
+void launch_blend_forward(const BlendArgs& a, hipStream_t s);
+void launch_blend_backward(const BlendArgs& a, hipStream_t s);
+
+// composite.hip
+void launch_composite_forward(const CompositeArgs& a, hipStream_t s);
+void launch_composite_backward(const CompositeArgs& a, hipStream_t s);
+void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s);
+
+}  // namespace rgs

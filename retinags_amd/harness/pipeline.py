@@ -1,0 +1,99 @@
+"""One-GPU render -> composite -> backward loop over the submodels of a partitioned scene:
+what the reference does per camera in gather_RenderResult_pool
+(parallel_utils/basic_parallel_trainer/result_aggregator.py:22-38), forward_blender_local
+(parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:417-434) and the backward
+through both, with every submodel resident on the same GPU and rendered one after another.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+from ..rasterizer import GaussianRasterizationSettings, GaussianRasterizer
+from ..compositor import blender_render_result
+from .partition import Partition, partition_scene, relation_vector
+from .scenes import Camera
+
+
+@dataclass
+class Submodel:
+    """The tensors render4renderinfo takes from a BoundedGaussianModel and its shared
+    Gaussians (gaussian_renderer/render_half_gs.py:103-110): activated values, box."""
+    means3D: torch.Tensor
+    opacity: torch.Tensor
+    scales: torch.Tensor
+    rotations: torch.Tensor
+    shs: torch.Tensor
+    range_low: torch.Tensor
+    range_up: torch.Tensor
+    active_sh_degree: int = 3
+
+    def parameters(self) -> List[torch.Tensor]:
+        return [self.means3D, self.opacity, self.scales, self.rotations, self.shs]
+
+    def requires_grad_(self, flag: bool = True) -> "Submodel":
+        for t in self.parameters():
+            t.requires_grad_(flag)
+        return self
+
+
+def submodels_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device) -> List[Submodel]:
+    subs = []
+    for k, ids in enumerate(part.members):
+        idx = torch.from_numpy(ids)
+        pick = lambda t: t[idx].to(device).contiguous()
+        subs.append(Submodel(pick(scene["xyz"]), pick(scene["opacity"]), pick(scene["scales"]),
+                             pick(scene["rotations"]), pick(scene["shs"]),
+                             torch.from_numpy(part.box_low[k]).to(device), torch.from_numpy(part.box_up[k]).to(device)))
+    return subs
+
+
+def whole_scene_submodel(scene: Dict[str, torch.Tensor], device, margin: float = 1.0) -> Submodel:
+    """A single submodel whose box encloses every Gaussian (bvh_depth = 0)."""
+    xyz = scene["xyz"]
+    pad = 3.0 * float(scene["scales"].max()) + margin
+    low = (xyz.min(dim=0).values - pad).to(device)
+    up = (xyz.max(dim=0).values + pad).to(device)
+    mv = lambda t: t.to(device).contiguous()
+    return Submodel(mv(xyz), mv(scene["opacity"]), mv(scene["scales"]), mv(scene["rotations"]), mv(scene["shs"]), low, up)
+
+
+def raster_settings(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0,
+                    debug: bool = False) -> GaussianRasterizationSettings:
+    return GaussianRasterizationSettings(
+        image_height=int(cam.image_height), image_width=int(cam.image_width),
+        tanfovx=math.tan(cam.FoVx * 0.5), tanfovy=math.tan(cam.FoVy * 0.5),
+        bg=bg, scale_modifier=scaling_modifier, viewmatrix=cam.world_view_transform,
+        projmatrix=cam.full_proj_transform, projmatrix_inv=cam.projection_matrix_inv,
+        range_low=sub.range_low, range_up=sub.range_up, sh_degree=sub.active_sh_degree,
+        campos=cam.camera_center, prefiltered=False, debug=debug)
+
+
+def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0,
+                    debug: bool = False) -> dict:
+    """Same call sequence and return dict as render4renderinfo
+    (gaussian_renderer/render_half_gs.py:112-182)."""
+    rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug))
+    means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
+    color, radii, depth, alpha = rasterizer(
+        means3D=sub.means3D, means2D=means2D, shs=sub.shs, colors_precomp=None, opacities=sub.opacity,
+        scales=sub.scales, rotations=sub.rotations, cov3D_precomp=None)
+    return {"render": color, "viewspace_points": means2D, "visibility_filter": radii > 0, "radii": radii,
+            "depth": depth, "alpha": alpha, "num_rendered": -1}
+
+
+def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
+                 submodel_bg: Optional[torch.Tensor] = None) -> dict:
+    """Render every related submodel (black background, as the trainer does:
+    trainer4tree_partition.py:397) and composite the partial images in BVH order."""
+    device = subs[0].means3D.device
+    if submodel_bg is None:
+        submodel_bg = torch.zeros(3, device=device)
+    partial = {m: render_submodel(cam, subs[m], submodel_bg) for m in range(len(subs)) if relation[m] >= 0}
+    out = blender_render_result(partial, relation, background)
+    out["partial"] = partial
+    return out

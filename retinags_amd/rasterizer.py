@@ -1,0 +1,338 @@
+"""Host-side mirror of the reference's rasterizer module
+(K/diff_gaussian_rasterization_half_gaussian/__init__.py with
+K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian): the same
+names, argument order, return values and error behaviour, driving PyTorch-ROCm
+tensors through the C ABI of librgs_gfx950.so instead of a pybind extension.
+
+PyTorch only provides device memory and the current stream here; every stage of
+the rasterizer runs in the HIP library.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import NamedTuple
+
+import torch
+import torch.nn as nn
+
+from . import _capi
+from ._capi import lib, check, ptr
+
+
+def cpu_deep_copy_tuple(input_tuple):
+    copied_tensors = [item.cpu().clone() if isinstance(item, torch.Tensor) else item for item in input_tuple]
+    return tuple(copied_tensors)
+
+
+class GaussianRasterizationSettings(NamedTuple):
+    """K/diff_gaussian_rasterization_half_gaussian/__init__.py:166-181, field for field."""
+    image_height: int
+    image_width: int
+    tanfovx: float
+    tanfovy: float
+    bg: torch.Tensor
+    scale_modifier: float
+    viewmatrix: torch.Tensor
+    projmatrix: torch.Tensor
+    projmatrix_inv: torch.Tensor
+    range_low: torch.Tensor
+    range_up: torch.Tensor
+    sh_degree: int
+    campos: torch.Tensor
+    prefiltered: bool
+    debug: bool
+
+
+_pinned_words = {}
+
+
+def _pinned_word(device: torch.device) -> torch.Tensor:
+    """One pinned uint32 per device: the landing spot of the instance count."""
+    key = (device.type, device.index)
+    t = _pinned_words.get(key)
+    if t is None:
+        t = torch.zeros(1, dtype=torch.int32).pin_memory()
+        _pinned_words[key] = t
+    return t
+
+
+def _dev_f32(t: torch.Tensor, device, name: str) -> torch.Tensor:
+    """Contiguous fp32 tensor on `device`; the reference calls .contiguous() on every
+    argument (K/rasterize_points.cu:99-121)."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if t.numel() == 0:
+        return t
+    if t.device != device or t.dtype != torch.float32:
+        t = t.to(device=device, dtype=torch.float32)
+    return t.contiguous()
+
+
+def _stream_ptr(device) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _rasterize_forward(bg, means3D, colors_precomp, opacities, scales, rotations, scale_modifier, cov3Ds_precomp,
+                       viewmatrix, projmatrix, projmatrix_inv, range_low, range_up, tanfovx, tanfovy, image_height,
+                       image_width, sh, sh_degree, campos, prefiltered, debug):
+    """Counterpart of RasterizeGaussiansCUDA_hgs (K/rasterize_points.cu:35-125): allocates the
+    outputs and the three workspaces, runs the forward, returns the same 8-tuple."""
+    if means3D.ndim != 2 or means3D.shape[1] != 3:
+        raise RuntimeError("means3D must have dimensions (num_points, 3)")
+    if not means3D.is_cuda:
+        raise RuntimeError("the rasterizer needs its inputs on a GPU (device memory)")
+    device = means3D.device
+    P, H, W = int(means3D.shape[0]), int(image_height), int(image_width)
+    f32 = dict(dtype=torch.float32, device=device)
+    byte = dict(dtype=torch.uint8, device=device)
+
+    out_color = torch.empty((3, H, W), **f32)
+    out_depth = torch.empty((1, H, W), **f32)
+    out_alpha = torch.empty((1, H, W), **f32)
+    radii = torch.empty((P,), dtype=torch.int32, device=device)
+    if P == 0:
+        out_color.zero_(); out_depth.zero_(); out_alpha.zero_()
+        empty = torch.empty(0, **byte)
+        return 0, out_color, out_depth, out_alpha, radii, empty, empty, empty
+
+    means3D = _dev_f32(means3D, device, "means3D")
+    colors_precomp = _dev_f32(colors_precomp, device, "colors_precomp")
+    opacities = _dev_f32(opacities, device, "opacities")
+    scales = _dev_f32(scales, device, "scales")
+    rotations = _dev_f32(rotations, device, "rotations")
+    cov3Ds_precomp = _dev_f32(cov3Ds_precomp, device, "cov3Ds_precomp")
+    sh = _dev_f32(sh, device, "sh")
+    bg = _dev_f32(bg, device, "bg")
+    viewmatrix = _dev_f32(viewmatrix, device, "viewmatrix")
+    projmatrix = _dev_f32(projmatrix, device, "projmatrix")
+    projmatrix_inv = _dev_f32(projmatrix_inv, device, "projmatrix_inv")
+    range_low = _dev_f32(range_low, device, "range_low")
+    range_up = _dev_f32(range_up, device, "range_up")
+    campos = _dev_f32(campos, device, "campos")
+    M = int(sh.shape[1]) if sh.numel() != 0 else 0
+
+    with torch.cuda.device(device):
+        stream = _stream_ptr(device)
+        geom_bytes = lib.rgs_geom_bytes(P)
+        image_bytes = lib.rgs_image_bytes(W, H)
+        geomBuffer = torch.empty(geom_bytes, **byte)
+        imgBuffer = torch.empty(image_bytes, **byte)
+        count = _pinned_word(device)
+        check(lib.rgs_forward_geom(
+            P, int(sh_degree), M, W, H, ptr(means3D), ptr(sh), ptr(colors_precomp), ptr(opacities), ptr(scales),
+            float(scale_modifier), ptr(rotations), ptr(cov3Ds_precomp), ptr(viewmatrix), ptr(projmatrix), ptr(campos),
+            float(tanfovx), float(tanfovy), int(bool(prefiltered)), ptr(radii), ptr(geomBuffer), geom_bytes,
+            C.c_void_p(count.data_ptr()), stream, int(bool(debug))))
+        rendered = int(count.item())
+        binning_bytes = lib.rgs_binning_bytes(rendered) if rendered > 0 else 0
+        binningBuffer = torch.empty(binning_bytes, **byte)
+        check(lib.rgs_forward_raster(
+            P, rendered, W, H, ptr(bg), float(tanfovx), float(tanfovy), ptr(projmatrix_inv), ptr(range_low),
+            ptr(range_up), ptr(colors_precomp), ptr(radii), ptr(geomBuffer), geom_bytes, ptr(binningBuffer),
+            binning_bytes, ptr(imgBuffer), image_bytes, ptr(out_color), ptr(out_depth), ptr(out_alpha), stream,
+            int(bool(debug))))
+    return rendered, out_color, out_depth, out_alpha, radii, geomBuffer, binningBuffer, imgBuffer
+
+
+def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, scale_modifier, cov3Ds_precomp,
+                        viewmatrix, projmatrix, projmatrix_inv, range_low, range_up, tanfovx, tanfovy, grad_color,
+                        grad_depth, grad_alpha, sh, sh_degree, campos, geomBuffer, num_rendered, binningBuffer,
+                        imgBuffer, alpha, debug):
+    """Counterpart of RasterizeGaussiansBackwardCUDA_hgs (K/rasterize_points.cu:127-220);
+    returns the same 8 tensors in the same order."""
+    device = means3D.device
+    P = int(means3D.shape[0])
+    H, W = int(grad_color.shape[1]), int(grad_color.shape[2])
+    M = int(sh.shape[1]) if sh.numel() != 0 else 0
+    f32 = dict(dtype=torch.float32, device=device)
+
+    if P == 0:
+        z = lambda *s: torch.zeros(s, **f32)
+        return z(0, 3), z(0, 3), z(0, 1), z(0, 3), z(0, 6), z(0, M, 3), z(0, 3), z(0, 4)
+
+    means3D = _dev_f32(means3D, device, "means3D")
+    colors_precomp = _dev_f32(colors_precomp, device, "colors_precomp")
+    scales = _dev_f32(scales, device, "scales")
+    rotations = _dev_f32(rotations, device, "rotations")
+    cov3Ds_precomp = _dev_f32(cov3Ds_precomp, device, "cov3Ds_precomp")
+    sh = _dev_f32(sh, device, "sh")
+    grad_color = _dev_f32(grad_color, device, "grad_color")
+    grad_depth = _dev_f32(grad_depth, device, "grad_depth")
+    grad_alpha = _dev_f32(grad_alpha, device, "grad_alpha")
+    alpha = _dev_f32(alpha, device, "alpha")
+    bg = _dev_f32(bg, device, "bg")
+    viewmatrix = _dev_f32(viewmatrix, device, "viewmatrix")
+    projmatrix = _dev_f32(projmatrix, device, "projmatrix")
+    projmatrix_inv = _dev_f32(projmatrix_inv, device, "projmatrix_inv")
+    range_low = _dev_f32(range_low, device, "range_low")
+    range_up = _dev_f32(range_up, device, "range_up")
+    campos = _dev_f32(campos, device, "campos")
+
+    # The five sums the blend accumulates atomically live in one buffer that the library clears.
+    acc = torch.empty((_capi.ACC_FLOATS * P,), **f32)
+    dL_dmeans3D = torch.empty((P, 3), **f32)
+    dL_dcov3D = torch.empty((P, 6), **f32)
+    dL_dsh = torch.empty((P, M, 3), **f32)
+    has_scales = scales.numel() != 0
+    dL_dscales = torch.empty((P, 3), **f32) if has_scales else torch.zeros((P, 3), **f32)
+    dL_drotations = torch.empty((P, 4), **f32) if has_scales else torch.zeros((P, 4), **f32)
+
+    with torch.cuda.device(device):
+        check(lib.rgs_backward(
+            P, int(sh_degree), M, int(num_rendered), W, H, ptr(bg), ptr(means3D), ptr(sh), ptr(colors_precomp),
+            ptr(alpha), ptr(scales), float(scale_modifier), ptr(rotations), ptr(cov3Ds_precomp), ptr(viewmatrix),
+            ptr(projmatrix), ptr(projmatrix_inv), ptr(range_low), ptr(range_up), ptr(campos), float(tanfovx),
+            float(tanfovy), ptr(radii), ptr(geomBuffer), ptr(binningBuffer), ptr(imgBuffer), ptr(grad_color),
+            ptr(grad_depth), ptr(grad_alpha), ptr(acc), ptr(dL_dmeans3D), ptr(dL_dcov3D), ptr(dL_dsh),
+            ptr(dL_dscales) if has_scales else C.c_void_p(0), ptr(dL_drotations) if has_scales else C.c_void_p(0),
+            _stream_ptr(device), int(bool(debug))))
+
+    dL_dmeans2D = acc[_capi.ACC_MEAN2D * P:(_capi.ACC_MEAN2D + 3) * P].view(P, 3)
+    dL_dopacity = acc[_capi.ACC_OPACITY * P:(_capi.ACC_OPACITY + 1) * P].view(P, 1)
+    dL_dcolors = acc[_capi.ACC_COLOR * P:(_capi.ACC_COLOR + 3) * P].view(P, 3)
+    return dL_dmeans2D, dL_dcolors, dL_dopacity, dL_dmeans3D, dL_dcov3D, dL_dsh, dL_dscales, dL_drotations
+
+
+def _mark_visible(means3D, viewmatrix, projmatrix):
+    """Counterpart of markVisible_hgs (K/rasterize_points.cu:222-241)."""
+    device = means3D.device
+    if not means3D.is_cuda:
+        raise RuntimeError("the rasterizer needs its inputs on a GPU (device memory)")
+    P = int(means3D.shape[0])
+    present = torch.zeros((P,), dtype=torch.bool, device=device)
+    if P != 0:
+        means3D = _dev_f32(means3D, device, "means3D")
+        viewmatrix = _dev_f32(viewmatrix, device, "viewmatrix")
+        projmatrix = _dev_f32(projmatrix, device, "projmatrix")
+        with torch.cuda.device(device):
+            check(lib.rgs_mark_visible(P, ptr(means3D), ptr(viewmatrix), ptr(projmatrix), ptr(present),
+                                       _stream_ptr(device)))
+    return present
+
+
+def rasterize_gaussians(means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp,
+                        raster_settings):
+    return _RasterizeGaussians.apply(means3D, means2D, sh, colors_precomp, opacities, scales, rotations,
+                                     cov3Ds_precomp, raster_settings)
+
+
+class _RasterizeGaussians(torch.autograd.Function):
+    """K/diff_gaussian_rasterization_half_gaussian/__init__.py:44-164."""
+
+    @staticmethod
+    def forward(ctx, means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp,
+                raster_settings):
+        args = (
+            raster_settings.bg, means3D, colors_precomp, opacities, scales, rotations, raster_settings.scale_modifier,
+            cov3Ds_precomp, raster_settings.viewmatrix, raster_settings.projmatrix, raster_settings.projmatrix_inv,
+            raster_settings.range_low, raster_settings.range_up, raster_settings.tanfovx, raster_settings.tanfovy,
+            raster_settings.image_height, raster_settings.image_width, sh, raster_settings.sh_degree,
+            raster_settings.campos, raster_settings.prefiltered, raster_settings.debug,
+        )
+        if raster_settings.debug:
+            cpu_args = cpu_deep_copy_tuple(args)  # copy them before they can be corrupted
+            try:
+                outs = _rasterize_forward(*args)
+            except Exception as ex:
+                torch.save(cpu_args, "snapshot_fw.dump")
+                print("\nAn error occured in forward. Please forward snapshot_fw.dump for debugging.")
+                raise ex
+        else:
+            outs = _rasterize_forward(*args)
+        num_rendered, color, depth, alpha, radii, geomBuffer, binningBuffer, imgBuffer = outs
+
+        ctx.raster_settings = raster_settings
+        ctx.num_rendered = num_rendered
+        ctx.save_for_backward(colors_precomp, means3D, scales, rotations, cov3Ds_precomp, radii, sh, geomBuffer,
+                              binningBuffer, imgBuffer, alpha)
+        ctx.mark_non_differentiable(radii)
+        return color, radii, depth, alpha
+
+    @staticmethod
+    def backward(ctx, grad_color, grad_radii, grad_depth, grad_alpha):
+        num_rendered = ctx.num_rendered
+        raster_settings = ctx.raster_settings
+        (colors_precomp, means3D, scales, rotations, cov3Ds_precomp, radii, sh, geomBuffer, binningBuffer, imgBuffer,
+         alpha) = ctx.saved_tensors
+
+        # Outputs that did not take part in the loss arrive as None; the reference's C++ side
+        # always receives dense tensors, so they become zeros.
+        if grad_color is None:
+            grad_color = torch.zeros((3,) + tuple(alpha.shape[1:]), dtype=alpha.dtype, device=alpha.device)
+        if grad_depth is None:
+            grad_depth = torch.zeros_like(alpha)
+        if grad_alpha is None:
+            grad_alpha = torch.zeros_like(alpha)
+
+        args = (raster_settings.bg, means3D, radii, colors_precomp, scales, rotations,
+                raster_settings.scale_modifier, cov3Ds_precomp, raster_settings.viewmatrix,
+                raster_settings.projmatrix, raster_settings.projmatrix_inv, raster_settings.range_low,
+                raster_settings.range_up, raster_settings.tanfovx, raster_settings.tanfovy, grad_color, grad_depth,
+                grad_alpha, sh, raster_settings.sh_degree, raster_settings.campos, geomBuffer, num_rendered,
+                binningBuffer, imgBuffer, alpha, raster_settings.debug)
+
+        if raster_settings.debug:
+            cpu_args = cpu_deep_copy_tuple(args)
+            try:
+                outs = _rasterize_backward(*args)
+            except Exception as ex:
+                torch.save(cpu_args, "snapshot_bw.dump")
+                print("\nAn error occured in backward. Writing snapshot_bw.dump for debugging.\n")
+                raise ex
+        else:
+            outs = _rasterize_backward(*args)
+        (grad_means2D, grad_colors_precomp, grad_opacities, grad_means3D, grad_cov3Ds_precomp, grad_sh, grad_scales,
+         grad_rotations) = outs
+
+        grads = (
+            grad_means3D,
+            grad_means2D,
+            grad_sh if sh.numel() else None,
+            grad_colors_precomp if colors_precomp.numel() else None,
+            grad_opacities,
+            grad_scales if scales.numel() else None,
+            grad_rotations if rotations.numel() else None,
+            grad_cov3Ds_precomp if cov3Ds_precomp.numel() else None,
+            None,
+        )
+        return grads
+
+
+class GaussianRasterizer(nn.Module):
+    """K/diff_gaussian_rasterization_half_gaussian/__init__.py:183-232."""
+
+    def __init__(self, raster_settings):
+        super().__init__()
+        self.raster_settings = raster_settings
+
+    def markVisible(self, positions):
+        # Mark visible points (based on frustum culling for camera) with a boolean
+        with torch.no_grad():
+            raster_settings = self.raster_settings
+            visible = _mark_visible(positions, raster_settings.viewmatrix, raster_settings.projmatrix)
+        return visible
+
+    def forward(self, means3D, means2D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
+                cov3D_precomp=None):
+        raster_settings = self.raster_settings
+
+        if (shs is None and colors_precomp is None) or (shs is not None and colors_precomp is not None):
+            raise Exception('Please provide excatly one of either SHs or precomputed colors!')
+
+        if ((scales is None or rotations is None) and cov3D_precomp is None) or \
+                ((scales is not None or rotations is not None) and cov3D_precomp is not None):
+            raise Exception('Please provide exactly one of either scale/rotation pair or precomputed 3D covariance!')
+
+        if shs is None:
+            shs = torch.Tensor([])
+        if colors_precomp is None:
+            colors_precomp = torch.Tensor([])
+        if scales is None:
+            scales = torch.Tensor([])
+        if rotations is None:
+            rotations = torch.Tensor([])
+        if cov3D_precomp is None:
+            cov3D_precomp = torch.Tensor([])
+
+        return rasterize_gaussians(means3D, means2D, shs, colors_precomp, opacities, scales, rotations, cov3D_precomp,
+                                   raster_settings)

@@ -1,0 +1,172 @@
+"""HIP rasterizer vs the CPU checker on identical seeded inputs, stage by stage.
+
+Bit-exact: radii, tile counts, pixel centres, depth bits, clip-w, offsets, duplicated
+keys/values, sorted keys, per-tile Gaussian lists, tile ranges.  Within 1e-4 max-abs:
+rendered colour, depth and alpha planes.  Within 1e-3 relative L2: every gradient.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import (DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, MAX_BORDERLINE_FRACTION, np32, oracle_settings, orc,
+                     rel_l2, scenes, view_ws)
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_gpu_forward(sub, cam, bg, dev, sh_degree=3, scale_modifier=1.0, debug=False):
+    from retinags_amd import rasterizer as R
+    e = torch.Tensor([])
+    return R._rasterize_forward(
+        bg.to(dev), sub["xyz"].to(dev), e, sub["opacity"].to(dev), sub["scales"].to(dev), sub["rotations"].to(dev),
+        scale_modifier, e, cam.world_view_transform.to(dev), cam.full_proj_transform.to(dev),
+        cam.projection_matrix_inv.to(dev), sub["low"].to(dev), sub["up"].to(dev), cam.tanfovx, cam.tanfovy,
+        cam.image_height, cam.image_width, sub["shs"].to(dev), sh_degree, cam.camera_center.to(dev), False, debug)
+
+
+def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
+    from retinags_amd import _capi
+    dev = torch.device("cuda:0")
+    s = oracle_settings(cam, sub["low"], sub["up"], bg, sh_degree, scale_modifier)
+    st = orc.forward(s, np32(sub["xyz"]), np32(sub["opacity"]), shs=np32(sub["shs"]), scales=np32(sub["scales"]),
+                     rotations=np32(sub["rotations"]), want_margin=True)
+    R, color, depth, alpha, radii, geom, binning, img = _run_gpu_forward(sub, cam, bg, dev, sh_degree, scale_modifier)
+    torch.cuda.synchronize()
+    P, W, H = st.P, cam.image_width, cam.image_height
+    T = s.grid[0] * s.grid[1]
+
+    # ---- per-Gaussian geometry: bit-exact
+    assert R == st.R
+    radii = radii.cpu().numpy()
+    assert np.array_equal(radii, st.radii)
+    vis = st.radii > 0
+    g = _capi.geom_layout(P)
+    assert np.array_equal(view_ws(geom, g["tiles_touched"], P, np.uint32), st.tiles_touched)
+    assert np.array_equal(view_ws(geom, g["point_offsets"], P, np.uint32), st.point_offsets)
+    xy = view_ws(geom, g["xy"], 2 * P, np.float32).reshape(P, 2)
+    assert np.array_equal(xy[vis].view(np.uint32), st.xy[vis].view(np.uint32))
+    assert np.array_equal(view_ws(geom, g["depths"], P, np.uint32)[vis], st.depths.view(np.uint32)[vis])
+    assert np.array_equal(view_ws(geom, g["clip_w"], P, np.uint32)[vis], st.zw[:, 1].copy().view(np.uint32)[vis])
+    co = view_ws(geom, g["conic_opacity"], 4 * P, np.float32).reshape(P, 4)
+    assert np.array_equal(co[vis].view(np.uint32), st.conic_opacity[vis].view(np.uint32))
+    cov = view_ws(geom, g["cov3D"], 6 * P, np.float32).reshape(P, 6)
+    assert np.array_equal(cov[vis].view(np.uint32), st.cov3D[vis].view(np.uint32))
+    rgb = view_ws(geom, g["rgb"], 3 * P, np.float32).reshape(P, 3)
+    assert np.array_equal(rgb[vis].view(np.uint32), st.rgb[vis].view(np.uint32))
+    clamped = view_ws(geom, g["clamped"], P, np.uint8)
+    packed = st.clamped[:, 0] | (st.clamped[:, 1] << 1) | (st.clamped[:, 2] << 2)
+    assert np.array_equal(clamped[vis], packed[vis])
+
+    # ---- binning: bit-exact
+    if R > 0:
+        b = _capi.binning_layout(R, W, H)
+        assert np.array_equal(view_ws(binning, b["keys_sorted"], R, np.uint64), st.keys)
+        assert np.array_equal(view_ws(binning, b["values_sorted"], R, np.uint32), st.point_list)
+    im = _capi.image_layout(W, H)
+    assert np.array_equal(view_ws(img, im["ranges"], 2 * T, np.uint32).reshape(T, 2), st.ranges)
+
+    # ---- blend: tolerance, away from decision thresholds
+    n_contrib = view_ws(img, im["n_contrib"], H * W, np.uint32)
+    safe = (st.margin > DECISION_MARGIN).reshape(H, W)
+    assert (~safe).mean() <= MAX_BORDERLINE_FRACTION
+    for got, want in ((color, st.color), (depth, st.depth), (alpha, st.alpha)):
+        diff = np.abs(got.cpu().numpy() - want)
+        assert diff[:, safe].max() <= IMAGE_TOL
+        # a borderline pixel may gain or lose one blended Gaussian, nothing more
+        assert diff.max() <= 2e-2
+    assert np.array_equal(n_contrib.reshape(H, W)[safe], st.n_contrib.reshape(H, W)[safe])
+    # accumulated alpha and remaining transmittance are complementary
+    assert float(alpha.min()) >= 0.0 and float(alpha.max()) <= 1.0 + 1e-5
+    return st
+
+
+def _scene_sub(scene, low=None, up=None):
+    xyz = scene["xyz"]
+    pad = 3.0 * float(scene["scales"].max()) + 1.0
+    low = xyz.min(dim=0).values - pad if low is None else low
+    up = xyz.max(dim=0).values + pad if up is None else up
+    return dict(xyz=xyz, opacity=scene["opacity"], scales=scene["scales"], rotations=scene["rotations"],
+                shs=scene["shs"], low=low.float(), up=up.float())
+
+
+def test_cube_forward_stages():
+    scene, cam, _ = scenes.make_config("C0", shrink=5, resolution_scale=0.5)
+    _check_forward_stages(_scene_sub(scene), cam, torch.tensor([0.1, 0.2, 0.3]))
+
+
+def test_cube_forward_lower_sh_degrees_and_scale_modifier():
+    scene, cam, _ = scenes.make_config("C0", shrink=50, resolution_scale=0.25)
+    for deg, mod in ((0, 1.0), (1, 0.7), (2, 1.5)):
+        _check_forward_stages(_scene_sub(scene), cam, torch.zeros(3), sh_degree=deg, scale_modifier=mod)
+
+
+def test_cube_half_box_clips():
+    """A box that ends in the middle of the cube: the per-pixel test must clip exactly like the checker."""
+    scene, cam, _ = scenes.make_config("C0", shrink=20, resolution_scale=0.5)
+    sub = _scene_sub(scene, up=torch.tensor([0.13, 0.4, 4.2]))
+    st = _check_forward_stages(sub, cam, torch.zeros(3))
+    assert st.counters[3] < st.counters[2]  # some samples were clipped by the box
+
+
+def test_garden_odd_resolution():
+    """Garden-like scene at a resolution that is not a multiple of the tile size."""
+    scene, cam, _ = scenes.make_config("C1", shrink=200, resolution_scale=0.2)
+    assert cam.image_width % 16 != 0 or cam.image_height % 16 != 0
+    _check_forward_stages(_scene_sub(scene), cam, torch.tensor([1.0, 1.0, 1.0]))
+
+
+def _check_backward(sub, cam, bg, seed, with_depth_alpha):
+    from retinags_amd import GaussianRasterizationSettings, GaussianRasterizer
+    dev = torch.device("cuda:0")
+    H, W = cam.image_height, cam.image_width
+    gen = torch.Generator().manual_seed(seed)
+    g_color = torch.randn(3, H, W, generator=gen) * 1e-2
+    g_depth = torch.randn(1, H, W, generator=gen) * 1e-2 if with_depth_alpha else None
+    g_alpha = torch.randn(1, H, W, generator=gen) * 1e-2 if with_depth_alpha else None
+
+    s = oracle_settings(cam, sub["low"], sub["up"], bg)
+    st = orc.forward(s, np32(sub["xyz"]), np32(sub["opacity"]), shs=np32(sub["shs"]), scales=np32(sub["scales"]),
+                     rotations=np32(sub["rotations"]))
+    want = orc.backward(s, st, np32(g_color), None if g_depth is None else np32(g_depth),
+                        None if g_alpha is None else np32(g_alpha))
+
+    leaf = {k: sub[k].to(dev).clone().requires_grad_(True) for k in ("xyz", "opacity", "scales", "rotations", "shs")}
+    means2D = torch.zeros_like(leaf["xyz"], requires_grad=True)
+    settings = GaussianRasterizationSettings(
+        image_height=H, image_width=W, tanfovx=cam.tanfovx, tanfovy=cam.tanfovy, bg=bg.to(dev), scale_modifier=1.0,
+        viewmatrix=cam.world_view_transform.to(dev), projmatrix=cam.full_proj_transform.to(dev),
+        projmatrix_inv=cam.projection_matrix_inv.to(dev), range_low=sub["low"].to(dev), range_up=sub["up"].to(dev),
+        sh_degree=3, campos=cam.camera_center.to(dev), prefiltered=False, debug=False)
+    color, radii, depth, alpha = GaussianRasterizer(settings)(
+        means3D=leaf["xyz"], means2D=means2D, opacities=leaf["opacity"], shs=leaf["shs"], scales=leaf["scales"],
+        rotations=leaf["rotations"])
+    loss = (color * g_color.to(dev)).sum()
+    if with_depth_alpha:
+        loss = loss + (depth * g_depth.to(dev)).sum() + (alpha * g_alpha.to(dev)).sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    got = dict(means3D=leaf["xyz"].grad, means2D=means2D.grad, sh=leaf["shs"].grad, opacity=leaf["opacity"].grad,
+               scales=leaf["scales"].grad, rotations=leaf["rotations"].grad)
+    for k, v in got.items():
+        err = rel_l2(v.cpu().numpy(), want[k])
+        assert err <= GRAD_TOL, f"gradient {k}: relative L2 {err:.3e}"
+    # Gaussians that were not rendered get exactly zero
+    dead = torch.from_numpy(st.radii <= 0).to(dev)
+    for k in ("means3D", "sh", "scales", "rotations", "opacity", "means2D"):
+        assert float(got[k][dead].abs().sum()) == 0.0
+
+
+def test_cube_backward_colour_only():
+    scene, cam, _ = scenes.make_config("C0", shrink=10, resolution_scale=0.5)
+    _check_backward(_scene_sub(scene), cam, torch.zeros(3), seed=7, with_depth_alpha=False)
+
+
+def test_cube_backward_all_outputs_with_background_and_box():
+    scene, cam, _ = scenes.make_config("C0", shrink=20, resolution_scale=0.5)
+    sub = _scene_sub(scene, up=torch.tensor([0.3, 2.0, 4.5]))
+    _check_backward(sub, cam, torch.tensor([0.3, 0.6, 0.9]), seed=8, with_depth_alpha=True)
+
+
+def test_garden_backward():
+    scene, cam, _ = scenes.make_config("C1", shrink=400, resolution_scale=0.2)
+    _check_backward(_scene_sub(scene), cam, torch.zeros(3), seed=9, with_depth_alpha=True)
