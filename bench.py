@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the half-Gaussian rasterizer + compositor on one MI355X.
+
+A step is one forward + backward pass of the whole hot path over one synthetic frame:
+every related submodel is rendered in turn (preprocess, key duplication, sort, tile ranges,
+blend), the partial images are composited front to back, a random upstream gradient is sent
+back through the compositor and through every submodel's rasterizer backward.  Inputs
+(Gaussian parameters, camera, upstream gradient) are resident in HBM before the timed region.
+
+Prints one JSON line: metric/value per the driver contract, plus `roofline` for the
+dominant kernel (HIP-event timing taken live on the stream the kernels run on), `stages`
+(every stage's time and achieved rate) and `cpu_baseline` (the CPU checker timed on this
+host's cores for the same workload).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="C1", choices=["C0", "C1", "C2", "C3", "C4"])
+    ap.add_argument("--shrink", type=float, default=1.0, help="divide the Gaussian count (debugging only)")
+    ap.add_argument("--resolution-scale", type=float, default=1.0, help="scale the image size (debugging only)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-threads", type=int, default=0)
+    return ap.parse_args()
+
+
+def ensure_built():
+    lib = os.path.join(ROOT, "retinags_amd", "librgs_gfx950.so")
+    if not os.path.exists(lib):
+        from retinags_amd import build as b
+        b.build(verbose=False)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: the submodels of a frame are rendered one after another on a single "
+              f"MI355X and composited there; --gpus {args.gpus} is not supported.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP library is the only implementation).", file=sys.stderr)
+        sys.exit(2)
+    ensure_built()
+    from retinags_amd import _capi, rasterizer as R
+    from retinags_amd.harness import scenes, partition, pipeline
+
+    dev = torch.device("cuda:0")
+    t0 = time.time()
+    scene, cam, cfg = scenes.make_config(args.config, "cpu", args.shrink, args.resolution_scale)
+    depth = cfg["bvh_depth"]
+    if depth > 0:
+        part = partition.partition_scene(scene["xyz"], scene["scales"], depth)
+        rel = partition.relation_vector(part, cam)
+        subs = pipeline.submodels_from_partition(scene, part, dev)
+        members = part.members
+    else:
+        part = None
+        rel = np.zeros(1, dtype=np.int64)
+        subs = [pipeline.whole_scene_submodel(scene, dev)]
+        members = [np.arange(scene["xyz"].shape[0])]
+    cam_d = cam.to(dev)
+    H, W = cam.image_height, cam.image_width
+    do_backward = bool(cfg["backward"])
+    if do_backward:
+        for s in subs:
+            s.requires_grad_(True)
+    bg = torch.zeros(3, device=dev)
+    gen = torch.Generator().manual_seed(cfg["seed"] + 77)
+    upstream = (torch.randn(3, H, W, generator=gen) * 1e-2).to(dev)
+    related = [m for m in range(len(subs)) if rel[m] >= 0]
+    setup_s = time.time() - t0
+
+    def step():
+        for s in subs:
+            for p in s.parameters():
+                p.grad = None
+        out = pipeline.render_frame(cam_d, subs, rel, bg)
+        if do_backward:
+            torch.autograd.backward([out["render"]], [upstream])
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t1
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # ---- per-stage time: HIP events recorded by the library on the stream it launches on
+    prof_steps = max(1, min(args.steps, 5))
+    _capi.stage_timing(True)
+    for _ in range(prof_steps):
+        step()
+    stage_ms = _capi.stage_timing_read()
+    _capi.stage_timing(False)
+
+    # ---- work sizes for the algorithmic byte / flop counts
+    P_tot = P_vis = R_tot = 0
+    counters = np.zeros(_capi.WORK_COUNTERS, dtype=np.uint64)
+    e = torch.Tensor([])
+    with torch.no_grad():
+        for m in related:
+            s = subs[m]
+            outs = R._rasterize_forward(bg, s.means3D.detach(), e, s.opacity.detach(), s.scales.detach(),
+                                        s.rotations.detach(), 1.0, e, cam_d.world_view_transform,
+                                        cam_d.full_proj_transform, cam_d.projection_matrix_inv, s.range_low,
+                                        s.range_up, cam.tanfovx, cam.tanfovy, H, W, s.shs.detach(), 3,
+                                        cam_d.camera_center, False, False)
+            Rm, _, _, _, radii, geom, binning, img = outs
+            Pm = int(s.means3D.shape[0])
+            P_tot += Pm
+            P_vis += int((radii > 0).sum())
+            R_tot += Rm
+            cnt = torch.zeros(_capi.WORK_COUNTERS, dtype=torch.int64, device=dev)
+            _capi.check(_capi.lib.rgs_blend_work_counters(
+                Pm, Rm, W, H, cam.tanfovx, cam.tanfovy, _capi.ptr(cam_d.projection_matrix_inv),
+                _capi.ptr(s.range_low), _capi.ptr(s.range_up), C.c_void_p(0), _capi.ptr(geom), _capi.ptr(binning),
+                _capi.ptr(img), _capi.ptr(cnt), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+            counters += cnt.cpu().numpy().astype(np.uint64)
+            del outs, geom, binning, img
+    nA, nB, nC, nD, nE, nBl, nCl = (float(v) for v in counters)
+    K = len(related)
+    T = ((W + 15) // 16) * ((H + 15) // 16)
+    N = W * H
+    passes = (32 + int(_capi.lib.rgs_get_higher_msb(T)) + 7) // 8
+    # Per-pixel entries the backward revisits: everything up to the last blended entry.
+    # It is not counted separately; the forward visit count bounds it from above.
+    flops_fwd = 12 * nA + 3 * nB + 27 * nC + 3 * nD + 14 * nE
+    flops_bwd = 12 * nA + 3 * nBl + 27 * nCl + 80 * nE
+    # Algorithmic bytes per frame of every HBM-bound stage (one launch per submodel; the sort
+    # kernels run `passes` times per submodel).
+    alg_bytes = {
+        "preprocess_forward": 20.0 * P_tot + 299.0 * P_vis,
+        "offset_scan": 8.0 * P_tot,
+        "duplicate_with_keys": 4.0 * P_tot + 16.0 * P_vis + 12.0 * R_tot,
+        "sort_histogram": 8.0 * R_tot * passes,
+        "sort_scatter": 24.0 * R_tot * passes,
+        "tile_ranges": 8.0 * R_tot + 16.0 * T * K,
+        "preprocess_backward": 4.0 * P_tot + 559.0 * P_vis,
+        "composite_forward": (20.0 * K + 20.0) * N,
+        "composite_backward": (40.0 * K + 20.0) * N,
+    }
+    alg_flops = {"blend_forward": flops_fwd, "blend_backward": flops_bwd}
+
+    stages = {}
+    for name, (ms, launches) in stage_ms.items():
+        per_step = ms / prof_steps
+        entry = {"ms_per_step": round(per_step, 4), "launches_per_step": launches / prof_steps,
+                 "avg_launch_ms": round(ms / max(launches, 1), 5)}
+        if name in alg_bytes and per_step > 0:
+            entry["bound"] = "hbm"
+            entry["achieved_GBps"] = round(alg_bytes[name] / (per_step * 1e-3) / 1e9, 2)
+            entry["frac"] = round(entry["achieved_GBps"] / HBM_PEAK_GBS, 4)
+        if name in alg_flops and per_step > 0:
+            entry["bound"] = "valu"
+            entry["achieved_TFLOPs"] = round(alg_flops[name] / (per_step * 1e-3) / 1e12, 3)
+            entry["frac"] = round(entry["achieved_TFLOPs"] / FP32_PEAK_TFLOPS, 4)
+        stages[name] = entry
+    dominant = max(stages, key=lambda n: stages[n]["ms_per_step"]) if stages else None
+    roofline = None
+    if dominant is not None:
+        d = stages[dominant]
+        if d.get("bound") == "hbm":
+            roofline = {"kernel": dominant, "bound": "hbm", "achieved": d["achieved_GBps"], "peak": HBM_PEAK_GBS,
+                        "unit": "GB/s", "frac": d["frac"], "traffic": None}
+        elif d.get("bound") == "valu":
+            roofline = {"kernel": dominant, "bound": "valu", "achieved": d["achieved_TFLOPs"],
+                        "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": d["frac"], "traffic": None}
+        if roofline is not None:
+            roofline["avg_launch_ms"] = d["avg_launch_ms"]
+            roofline["launches_per_step"] = d["launches_per_step"]
+
+    gpu_stage_ms = sum(v["ms_per_step"] for v in stages.values())
+    evals = {
+        "visits_per_frame": nA, "exp_per_frame": nB, "blended_per_frame": nE,
+        "fwd_visits_per_s": round(nA / (stages["blend_forward"]["ms_per_step"] * 1e-3), 1)
+        if "blend_forward" in stages and stages["blend_forward"]["ms_per_step"] > 0 else None,
+    }
+
+    # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(scene, members, part, cam, rel, related, upstream.cpu().numpy(), do_backward, args)
+
+    line = {
+        "metric": "fwd+bwd iterations/s, 5.6M Gaussians, 1600x1036, 4 composited submodels" if args.config == "C1"
+        else f"fwd{'+bwd' if do_backward else ''} iterations/s, config {args.config}",
+        "value": round(args.steps / elapsed, 4), "unit": "it/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.config}: {cfg['n']} Gaussians, {W}x{H}, bvh_depth={depth} "
+                               f"({K} of {len(subs)} submodels related), SH degree 3, "
+                               f"{'fwd+bwd' if do_backward else 'fwd only'}",
+                   "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
+                   "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1)},
+        "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
+        "blend_work": evals,
+    }
+    print(json.dumps(line))
+
+
+def cpu_baseline(scene, members, part, cam, rel, related, upstream, do_backward, args):
+    """One full forward(+backward) of the same frame on the CPU checker, OpenMP over this
+    host's cores.  Test infrastructure used as a measuring stick, never as the product path."""
+    from oracle import rgs_oracle as orc
+    oracle_settings = orc.settings_from_camera
+    np32 = lambda t: np.ascontiguousarray(t.detach().cpu().numpy().astype(np.float32))
+    threads = args.cpu_threads or min(16, orc.max_threads(), os.cpu_count() or 1)
+    orc.set_threads(threads)
+    order = sorted(related, key=lambda m: rel[m])
+    bg = torch.zeros(3)
+    xyz, opa, sc, rot, shs = (np32(scene[k]) for k in ("xyz", "opacity", "scales", "rotations", "shs"))
+    if part is not None:
+        lows, ups = part.box_low, part.box_up
+    else:
+        pad = 3.0 * float(scene["scales"].max()) + 1.0
+        lows = [np32(scene["xyz"].min(dim=0).values - pad)]
+        ups = [np32(scene["xyz"].max(dim=0).values + pad)]
+    t0 = time.perf_counter()
+    states, sets = [], []
+    for m in order:
+        ids = members[m]
+        s = oracle_settings(cam, torch.from_numpy(np.asarray(lows[m])), torch.from_numpy(np.asarray(ups[m])), bg)
+        st = orc.forward(s, xyz[ids], opa[ids], shs=shs[ids], scales=sc[ids], rotations=rot[ids])
+        states.append(st)
+        sets.append(s)
+    imgs = [st.color for st in states]
+    deps = [st.depth for st in states]
+    alps = [st.alpha for st in states]
+    orc.composite_forward(imgs, deps, alps, np.zeros(3, np.float32))
+    if do_backward:
+        d_img, d_dep, d_alp = orc.composite_backward(imgs, deps, alps, np.zeros(3, np.float32), upstream)
+        for k, st in enumerate(states):
+            orc.backward(sets[k], st, d_img[k], d_dep[k], d_alp[k])
+    dt = time.perf_counter() - t0
+    orc.set_threads(1)
+    return {"value": round(1.0 / dt, 5), "unit": "it/s", "cores": threads, "kind": "port",
+            "sample": f"1 full iteration of the same frame ({dt:.1f} s wall), C checker with OpenMP",
+            "host_cpus": os.cpu_count()}
+
+
+if __name__ == "__main__":
+    main()

@@ -143,6 +143,28 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  float* grad_accum, float* dL_dmean3D, float* dL_dcov3D, float* dL_dsh, float* dL_dscale,
                  float* dL_drot, void* stream, int debug);
 
+/* ---- measurement aids (no counterpart in the reference, which times whole iterations
+ * with CUDA events: parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:590-643) -- */
+
+/* Per-stage timing with HIP events on the caller's stream.  rgs_stage_timing(1) clears and
+ * starts recording, rgs_stage_timing(0) stops.  rgs_stage_timing_read waits for the recorded
+ * work, fills up to max_stages (name, total milliseconds, launches) triples, clears the record
+ * and returns the number of stages (negative on error).  The names are static strings.
+ * Recording is process-wide and not thread-safe; leave it off outside measurements. */
+int rgs_stage_timing(int enable);
+int rgs_stage_timing_read(int max_stages, const char** names, float* total_ms, int* launches);
+
+/* Work accounting of the blend for the frame held in the workspaces after rgs_forward_raster:
+ * re-walks every tile exactly like the forward blend and writes RGS_WORK_COUNTERS uint64 sums
+ * to `counters` (device memory): [0] list entries visited by a live pixel, [1] of those with
+ * power <= 0, [2] with alpha >= 1/255, [3] inside the submodel box, [4] blended; [5], [6] are
+ * [1], [2] restricted to entries up to each pixel's last blended one (the backward's share). */
+#define RGS_WORK_COUNTERS 7
+int rgs_blend_work_counters(int P, int R, int width, int height, float tan_fovx, float tan_fovy,
+                            const float* projmatrix_inv, const float* range_low, const float* range_up,
+                            const float* colors_precomp, const void* geom_ws, const void* binning_ws,
+                            const void* image_ws, uint64_t* counters, void* stream);
+
 /* ---- stand-alone binning primitives ---------------------------------------------------- */
 
 /* Inclusive uint32 prefix sum; replaces the cub::DeviceScan::InclusiveSum call at

@@ -99,6 +99,21 @@ class Settings:
         return ((self.image_width + 15) // 16, (self.image_height + 15) // 16)
 
 
+def settings_from_camera(cam, range_low, range_up, bg, sh_degree=3, scale_modifier=1.0) -> Settings:
+    """Settings for a harness camera (retinags_amd.harness.scenes.Camera, torch CPU tensors)
+    and a submodel box, exactly the fields render4renderinfo fills
+    (gaussian_renderer/render_half_gs.py:121-137)."""
+    import math
+    a = lambda t: np.ascontiguousarray(np.asarray(t.detach().cpu().numpy() if hasattr(t, "detach") else t,
+                                                  dtype=np.float32))
+    return Settings(
+        image_height=int(cam.image_height), image_width=int(cam.image_width), tanfovx=math.tan(cam.FoVx * 0.5),
+        tanfovy=math.tan(cam.FoVy * 0.5), bg=a(bg), scale_modifier=scale_modifier,
+        viewmatrix=a(cam.world_view_transform), projmatrix=a(cam.full_proj_transform),
+        projmatrix_inv=a(cam.projection_matrix_inv), range_low=a(range_low), range_up=a(range_up),
+        sh_degree=sh_degree, campos=a(cam.camera_center))
+
+
 @dataclass
 class ForwardState:
     """Everything the forward produced (the reference keeps the same data in

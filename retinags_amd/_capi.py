@@ -53,7 +53,10 @@ def _load():
     pp = C.POINTER(vp)
     lib.rgs_composite_forward.argtypes = [i, i, i, pp, pp, pp, vp, vp, vp, vp, vp]
     lib.rgs_composite_backward.argtypes = [i, i, i, pp, pp, pp, vp, vp, vp, vp, pp, pp, pp, vp]
-    for name in ("rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
+    lib.rgs_stage_timing.argtypes = [i]
+    lib.rgs_stage_timing_read.argtypes = [i, C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.POINTER(C.c_int)]
+    lib.rgs_blend_work_counters.argtypes = [i, i, i, i, f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
                  "rgs_forward_geom", "rgs_forward_raster", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
                  "rgs_composite_forward", "rgs_composite_backward"):
         getattr(lib, name).restype = i
@@ -65,7 +68,9 @@ lib = _load()
 EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_bytes", "rgs_binning_bytes",
            "rgs_image_bytes", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
            "rgs_forward_geom", "rgs_forward_raster", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
-           "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward")
+           "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward",
+           "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters")
+WORK_COUNTERS = 7
 
 
 def check(rc: int) -> None:
@@ -89,6 +94,21 @@ def image_layout(width: int, height: int) -> dict:
     off = (C.c_size_t * len(IMG_FIELDS))()
     check(lib.rgs_image_layout(width, height, off))
     return dict(zip(IMG_FIELDS, off))
+
+
+def stage_timing(enable: bool) -> None:
+    check(lib.rgs_stage_timing(1 if enable else 0))
+
+
+def stage_timing_read(max_stages: int = 64) -> dict:
+    """{stage: (total_ms, launches)} recorded since the last read; waits for the work."""
+    names = (C.c_char_p * max_stages)()
+    ms = (C.c_float * max_stages)()
+    cnt = (C.c_int * max_stages)()
+    n = lib.rgs_stage_timing_read(max_stages, names, ms, cnt)
+    if n < 0:
+        raise RgsError(lib.rgs_last_error().decode("utf-8", "replace"))
+    return {names[k].decode(): (float(ms[k]), int(cnt[k])) for k in range(n)}
 
 
 def ptr(t) -> C.c_void_p:

@@ -7,6 +7,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <string>
+#include <vector>
 
 namespace {
 
@@ -44,6 +46,41 @@ int check_stage(const char* stage, hipStream_t s, int debug)
 		if (int rc_ = check_stage(name, s, debug))    \
 			return rc_;                               \
 	} while (0)
+
+// ---- optional stage timing -------------------------------------------------------------
+// While enabled, every launcher records a HIP event on the caller's stream before its kernel
+// (rgs::stage_mark) and every entry point records one when it has queued its last kernel.
+// The time between two consecutive events is charged to the earlier event's stage.
+struct StageTimer {
+	bool on = false;
+	std::vector<hipEvent_t> pool;
+	std::vector<const char*> tags;  // tag of event i; nullptr closes an entry point
+	size_t used = 0;
+};
+StageTimer g_timer;
+constexpr size_t kMaxTimerEvents = 1 << 16;
+
+void timer_record(const char* tag, hipStream_t s)
+{
+	if (!g_timer.on || g_timer.used >= kMaxTimerEvents)
+		return;
+	if (g_timer.used == g_timer.pool.size()) {
+		hipEvent_t e;
+		if (hipEventCreate(&e) != hipSuccess)
+			return;
+		g_timer.pool.push_back(e);
+		g_timer.tags.push_back(nullptr);
+	}
+	g_timer.tags[g_timer.used] = tag;
+	if (hipEventRecord(g_timer.pool[g_timer.used], s) == hipSuccess)
+		g_timer.used++;
+}
+
+struct EntryScope {
+	hipStream_t s;
+	explicit EntryScope(hipStream_t stream) : s(stream) {}
+	~EntryScope() { timer_record(nullptr, s); }
+};
 
 constexpr size_t kAlign = 256;
 
@@ -125,7 +162,55 @@ const T* at(const void* base, size_t off)
 
 }  // namespace
 
+namespace rgs {
+void stage_mark(const char* name, hipStream_t s)
+{
+	timer_record(name, s);
+}
+}  // namespace rgs
+
 extern "C" {
+
+int rgs_stage_timing(int enable)
+{
+	g_timer.on = enable != 0;
+	g_timer.used = 0;
+	return 0;
+}
+
+int rgs_stage_timing_read(int max_stages, const char** names, float* total_ms, int* launches)
+{
+	RGS_REQUIRE(max_stages >= 0 && (max_stages == 0 || (names && total_ms && launches)), "rgs_stage_timing_read: bad arguments");
+	int n = 0;
+	if (g_timer.used > 0) {
+		hipError_t e = hipEventSynchronize(g_timer.pool[g_timer.used - 1]);
+		if (e != hipSuccess)
+			return -fail("rgs_stage_timing_read: %s", hipGetErrorString(e));
+	}
+	for (size_t i = 0; i + 1 < g_timer.used; i++) {
+		const char* tag = g_timer.tags[i];
+		if (!tag)
+			continue;
+		float ms = 0.f;
+		if (hipEventElapsedTime(&ms, g_timer.pool[i], g_timer.pool[i + 1]) != hipSuccess)
+			continue;
+		int k = 0;
+		while (k < n && strcmp(names[k], tag) != 0)
+			k++;
+		if (k == n) {
+			if (n == max_stages)
+				continue;
+			names[n] = tag;
+			total_ms[n] = 0.f;
+			launches[n] = 0;
+			n++;
+		}
+		total_ms[k] += ms;
+		launches[k] += 1;
+	}
+	g_timer.used = 0;
+	return n;
+}
 
 int rgs_version(void)
 {
@@ -198,6 +283,7 @@ int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const
 {
 	(void)projmatrix;
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	const int debug = 0;
 	RGS_REQUIRE(P >= 0, "rgs_mark_visible: negative P");
 	if (P == 0)
@@ -221,6 +307,7 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
 	// Gaussian is simply skipped.
 	(void)prefiltered;
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	RGS_REQUIRE(P > 0, "rgs_forward_geom: P must be positive (the caller short-circuits P == 0)");
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_geom: bad image size %dx%d", width, height);
 	RGS_REQUIRE(means3D && opacities && viewmatrix && projmatrix && cam_pos && radii && geom_ws && num_rendered_host,
@@ -287,6 +374,7 @@ int rgs_forward_raster(int P, int R, int width, int height,
                        float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	RGS_REQUIRE(P > 0 && R >= 0, "rgs_forward_raster: bad sizes P=%d R=%d", P, R);
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_raster: bad image size %dx%d", width, height);
 	RGS_REQUIRE(background && projmatrix_inv && range_low && range_up && radii && geom_ws && image_ws && out_color &&
@@ -356,6 +444,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  float* dL_drot, void* stream, int debug)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	RGS_REQUIRE(P > 0 && R >= 0, "rgs_backward: bad sizes P=%d R=%d", P, R);
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_backward: bad image size %dx%d", width, height);
 	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
@@ -426,6 +515,46 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	return 0;
 }
 
+int rgs_blend_work_counters(int P, int R, int width, int height, float tan_fovx, float tan_fovy,
+                            const float* projmatrix_inv, const float* range_low, const float* range_up,
+                            const float* colors_precomp, const void* geom_ws, const void* binning_ws,
+                            const void* image_ws, uint64_t* counters, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(P > 0 && R >= 0 && width > 0 && height > 0, "rgs_blend_work_counters: bad sizes");
+	RGS_REQUIRE(projmatrix_inv && range_low && range_up && geom_ws && image_ws && counters && (R == 0 || binning_ws),
+	            "rgs_blend_work_counters: null pointer");
+	size_t goff[RGS_GEOM_FIELDS], ioff[RGS_IMG_FIELDS];
+	geom_layout((size_t)P, goff);
+	image_layout(width, height, ioff);
+	rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(counters), 0u, 2 * RGS_WORK_COUNTERS, s);
+	if (R == 0)
+		return 0;
+	const BinningPhysical b = binning_physical((size_t)R);
+	const bool sorted_in_a = (((sort_end_bit(width, height) + 7) / 8) % 2) == 0;
+	rgs::BlendArgs a;
+	memset(&a, 0, sizeof(a));
+	a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
+	a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
+	a.W = width; a.H = height;
+	a.grid_x = (width + rgs::kTile - 1) / rgs::kTile;
+	a.grid_y = (height + rgs::kTile - 1) / rgs::kTile;
+	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
+	a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up;
+	a.bg = range_low;  // unused by the counting kernel
+	a.xy = at<float2>(geom_ws, goff[RGS_GEOM_XY]);
+	a.clip_w = at<float>(geom_ws, goff[RGS_GEOM_CLIP_W]);
+	a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
+	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
+	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
+	a.counters = counters;
+	rgs::launch_blend_forward(a, s);
+	RGS_STAGE("blend_count");
+	return 0;
+}
+
 size_t rgs_scan_temp_bytes(size_t n)
 {
 	return 4 * rgs::scan_temp_words(n);
@@ -434,6 +563,7 @@ size_t rgs_scan_temp_bytes(size_t n)
 int rgs_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, void* temp, void* stream)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	const int debug = 0;
 	if (n == 0)
 		return 0;
@@ -453,6 +583,7 @@ int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uin
                    int end_bit, void* temp, void* stream)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	const int debug = 0;
 	RGS_REQUIRE(end_bit >= 1 && end_bit <= 64, "rgs_sort_pairs: end_bit %d out of range", end_bit);
 	if (n == 0)
@@ -495,6 +626,7 @@ int rgs_composite_forward(int K, int height, int width,
                           void* stream)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	const int debug = 0;
 	rgs::CompositeArgs a;
 	if (int rc = fill_composite(a, K, height, width, images, depths, alphas, background))
@@ -513,6 +645,7 @@ int rgs_composite_backward(int K, int height, int width,
                            float* const* d_alphas, void* stream)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
 	const int debug = 0;
 	rgs::CompositeArgs a;
 	if (int rc = fill_composite(a, K, height, width, images, depths, alphas, background))

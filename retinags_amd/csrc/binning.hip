@@ -81,6 +81,7 @@ void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t*
 	if (n == 0)
 		return;
 	const size_t nb = (n + 255) / 256;
+	stage_mark("inclusive_sum", s);
 	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, temp);
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, nb, (uint32_t*)nullptr);
 	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, temp, n, out);
@@ -90,6 +91,7 @@ void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* blo
                                     uint32_t* total_out, hipStream_t s)
 {
 	const size_t nb = ((size_t)P + 255) / 256;
+	stage_mark("offset_scan", s);
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb, total_out);
 	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, tiles_touched, block_sums,
 	                   (size_t)P, offsets);
@@ -128,6 +130,7 @@ void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, co
                                 const int* radii, int grid_x, int grid_y, uint64_t* keys, uint32_t* values,
                                 hipStream_t s)
 {
+	stage_mark("duplicate_with_keys", s);
 	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, P, xy, depths, offsets,
 	                   radii, grid_x, grid_y, keys, values);
 }
@@ -287,9 +290,12 @@ void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in,
 	for (int shift = 0; shift < end_bit; shift += 8) {
 		const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
 		const uint32_t mask = (1u << bits) - 1u;
+		stage_mark("sort_histogram", s);
 		hipLaunchKernelGGL(sort_histogram_kernel, dim3(nblocks), dim3(256), 0, s, ksrc, n, shift, mask, temp, nblocks);
+		stage_mark("sort_scan", s);
 		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, (size_t)256 * nblocks,
 		                   (uint32_t*)nullptr);
+		stage_mark("sort_scatter", s);
 		hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, shift, mask,
 		                   temp, nblocks);
 		uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
@@ -335,6 +341,7 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint64_t* __rest
 
 void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, hipStream_t s)
 {
+	stage_mark("tile_ranges", s);
 	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2, s);
 	if (n == 0)
 		return;

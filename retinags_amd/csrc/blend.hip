@@ -29,6 +29,12 @@ __device__ __forceinline__ bool clipped_by_box(const PixelRay& ray, float w, flo
 
 // ---- forward (K/cuda_rasterizer_hgs/forward.cu:263-405) ---------------------------------------
 
+// kCount = true is the instrumented twin used for work accounting: it writes no image and
+// instead adds, over all pixels, the number of list entries visited by a live pixel (A), those
+// with power <= 0 (B), those with alpha >= 1/255 (C), those inside the box (D), those blended
+// (E), and the B and C counts restricted to entries up to each pixel's last blended one (B', C'),
+// which is what the backward pass re-evaluates.
+template <bool kCount>
 __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 {
 	__shared__ float2 s_xy[256];
@@ -56,6 +62,7 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	float T = 1.0f;
 	uint32_t last_contributor = 0;
 	float C0 = 0.f, C1 = 0.f, C2 = 0.f, weight = 0.f, D = 0.f;
+	uint32_t nA = 0, nB = 0, nC = 0, nD = 0, nE = 0, nB_last = 0, nC_last = 0;
 
 	for (int i = 0; i < rounds; i++, todo -= 256) {
 		const int alive = __ballot(!done) != 0ull;
@@ -80,17 +87,26 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 			const float2 d = {xy.x - pixf.x, xy.y - pixf.y};
 			const float4 co = s_co[j];
 			const float power = -0.5f * (co.x * d.x * d.x + co.z * d.y * d.y) - co.y * d.x * d.y;
+			if (kCount) nA++;
 			if (power > 0.0f)
 				continue;
+			if (kCount) nB++;
 			const float alpha = fminf(0.99f, co.w * expf(power));
 			if (alpha < 1.0f / 255.0f)
 				continue;
+			if (kCount) nC++;
 			if (clipped_by_box(ray, s_w[j], a.tanfovx, a.tanfovy, a.projinv, lo, hi))
 				continue;
+			if (kCount) nD++;
 			const float test_T = T * (1 - alpha);
 			if (test_T < 0.0001f) {
 				done = true;
 				continue;
+			}
+			if (kCount) {
+				nE++;
+				nB_last = nB;
+				nC_last = nC;
 			}
 			const float4 cd = s_cd[j];
 			C0 += cd.x * alpha * T;
@@ -104,6 +120,16 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 		__syncthreads();
 	}
 
+	if (kCount) {
+		const uint32_t c[7] = {nA, nB, nC, nD, nE, nB_last, nC_last};
+#pragma unroll
+		for (int q = 0; q < 7; q++) {
+			const uint32_t tot = wave_inclusive_scan_u32(c[q]);
+			if (lane == 63)
+				atomicAdd(reinterpret_cast<unsigned long long*>(a.counters) + q, (unsigned long long)tot);
+		}
+		return;
+	}
 	if (inside) {
 		const size_t plane = (size_t)a.H * a.W;
 		a.n_contrib[pix_id] = last_contributor;
@@ -295,11 +321,16 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 
 void launch_blend_forward(const BlendArgs& a, hipStream_t s)
 {
-	hipLaunchKernelGGL(blend_forward_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+	stage_mark(a.counters ? "blend_count" : "blend_forward", s);
+	if (a.counters)
+		hipLaunchKernelGGL(blend_forward_kernel<true>, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+	else
+		hipLaunchKernelGGL(blend_forward_kernel<false>, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
 }
 
 void launch_blend_backward(const BlendArgs& a, hipStream_t s)
 {
+	stage_mark("blend_backward", s);
 	hipLaunchKernelGGL(blend_backward_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
 }
 

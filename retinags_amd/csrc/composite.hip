@@ -74,12 +74,14 @@ __global__ __launch_bounds__(256) void composite_backward_kernel(CompositeArgs a
 void launch_composite_forward(const CompositeArgs& a, hipStream_t s)
 {
 	const size_t n = (size_t)a.H * a.W;
+	stage_mark("composite_forward", s);
 	hipLaunchKernelGGL(composite_forward_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a);
 }
 
 void launch_composite_backward(const CompositeArgs& a, hipStream_t s)
 {
 	const size_t n = (size_t)a.H * a.W;
+	stage_mark("composite_backward", s);
 	hipLaunchKernelGGL(composite_backward_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a);
 }
 

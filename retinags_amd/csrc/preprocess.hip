@@ -464,16 +464,19 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBack
 
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s)
 {
+	stage_mark("mark_visible", s);
 	hipLaunchKernelGGL(mark_visible_kernel, dim3((P + 255) / 256), dim3(256), 0, s, P, means, view, present);
 }
 
 void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s)
 {
+	stage_mark("preprocess_forward", s);
 	hipLaunchKernelGGL(preprocess_forward_kernel, dim3((a.P + 255) / 256), dim3(256), 0, s, a);
 }
 
 void launch_preprocess_backward(const PreprocessBackwardArgs& a, hipStream_t s)
 {
+	stage_mark("preprocess_backward", s);
 	hipLaunchKernelGGL(preprocess_backward_kernel, dim3((a.P + 255) / 256), dim3(256), 0, s, a);
 }
 

@@ -81,6 +81,7 @@ struct BlendArgs {
 	float* out_depth;
 	float* out_alpha;
 	uint32_t* n_contrib;
+	uint64_t* counters;  // non-null selects the work-accounting twin of the forward blend (7 sums)
 	// backward
 	const float* dL_dpix;
 	const float* dL_dpix_depth;
@@ -126,8 +127,9 @@ void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, co
                                 const int* radii, int grid_x, int grid_y, uint64_t* keys, uint32_t* values,
                                 hipStream_t s);
 size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs
-// Stable LSD radix sort on key bits [0, end_bit).  Result lands in keys_out/vals_out;
-// keys_in/vals_in are overwritten (they serve as the ping-pong partner).
+// Stable LSD radix sort on key bits [0, end_bit), ceil(end_bit/8) passes that ping-pong between
+// the two buffer pairs starting in -> out: an odd pass count leaves the result in
+// keys_out/vals_out, an even one in keys_in/vals_in.
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s);
 void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, hipStream_t s);
@@ -140,5 +142,8 @@ void launch_blend_backward(const BlendArgs& a, hipStream_t s);
 void launch_composite_forward(const CompositeArgs& a, hipStream_t s);
 void launch_composite_backward(const CompositeArgs& a, hipStream_t s);
 void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s);
+
+// api.hip: optional stage timing.  A mark names the work launched after it.
+void stage_mark(const char* name, hipStream_t s);
 
 }  // namespace rgs

@@ -29,12 +29,7 @@ def np32(t):
 
 
 def oracle_settings(cam, range_low, range_up, bg, sh_degree=3, scale_modifier=1.0):
-    return orc.Settings(
-        image_height=cam.image_height, image_width=cam.image_width, tanfovx=math.tan(cam.FoVx * 0.5),
-        tanfovy=math.tan(cam.FoVy * 0.5), bg=np32(bg), scale_modifier=scale_modifier,
-        viewmatrix=np32(cam.world_view_transform), projmatrix=np32(cam.full_proj_transform),
-        projmatrix_inv=np32(cam.projection_matrix_inv), range_low=np32(range_low), range_up=np32(range_up),
-        sh_degree=sh_degree, campos=np32(cam.camera_center))
+    return orc.settings_from_camera(cam, range_low, range_up, bg, sh_degree, scale_modifier)
 
 
 def rel_l2(a, b):
