@@ -35,7 +35,11 @@ def covariance3d(scales, quats, mod=1.0):
 def real_sh_basis(dirs, degree=3):
     """(n, (degree+1)^2) real spherical harmonics in the sign convention of 3D Gaussian
     splatting: index l*l + l + m, equal to (-1)^m times the usual real harmonics."""
-    from scipy.special import sph_harm
+    try:  # scipy >= 1.15: sph_harm_y(l, m, polar, azimuth)
+        from scipy.special import sph_harm_y
+        sph_harm = lambda m, l, azimuth, polar: sph_harm_y(l, m, polar, azimuth)
+    except ImportError:
+        from scipy.special import sph_harm
     d = np.asarray(dirs, dtype=np.float64)
     d = d / np.linalg.norm(d, axis=1, keepdims=True)
     theta = np.arctan2(d[:, 1], d[:, 0])          # azimuth
@@ -115,11 +119,12 @@ def render_reference(params, cam, W, H, low, up, bg, sh_degree=3, mod=1.0):
     cov2d = ewa_cov2d(xyz, cov3d, view_t, W, H, tanx, tany)
     conic = torch.linalg.inv(cov2d)
     with torch.no_grad():
-        lam = torch.linalg.eigvalsh(cov2d)[:, 1]
-        mid = 0.5 * (cov2d[:, 0, 0] + cov2d[:, 1, 1])
-        det = torch.linalg.det(cov2d)
-        lam_ref = mid + torch.sqrt(torch.clamp(mid * mid - det, min=0.1))
-        radius = torch.ceil(3 * torch.sqrt(torch.maximum(lam_ref, lam * 0 + lam_ref)))
+        # extent: 3 sigma of the larger eigenvalue, where the half-gap between the two
+        # eigenvalues is floored at sqrt(0.1) (the forward's definition of the radius)
+        lam = torch.linalg.eigvalsh(cov2d)
+        mid = 0.5 * (lam[:, 0] + lam[:, 1])
+        half_gap = 0.5 * (lam[:, 1] - lam[:, 0])
+        radius = torch.ceil(3 * torch.sqrt(mid + torch.sqrt(torch.clamp(half_gap ** 2, min=0.1))))
         visible = depth > 0.2
         rects = []
         for i in range(n):
@@ -162,7 +167,9 @@ def render_reference(params, cam, W, H, low, up, bg, sh_degree=3, mod=1.0):
             cn = conic[idt]
             power = -0.5 * (cn[:, 0, 0] * d[:, 0] ** 2 + cn[:, 1, 1] * d[:, 1] ** 2) - cn[:, 0, 1] * d[:, 0] * d[:, 1]
             G = torch.exp(power)
-            alpha = torch.clamp(opac[idt, 0] * G, max=0.99)
+            # 0.99 clamp with a straight-through gradient
+            raw = opac[idt, 0] * G
+            alpha = raw + (torch.clamp(raw, max=0.99) - raw).detach()
             # ray point at each Gaussian's clip-w, in world space
             ndcx = (2.0 * px + 1.0) / W - 1.0
             ndcy = (2.0 * py + 1.0) / H - 1.0

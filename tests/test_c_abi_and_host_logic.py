@@ -1,0 +1,153 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol that include/rgs.h
+declares, size/layout queries behave (they launch nothing), and the Python mirror of the
+reference module validates arguments like the reference
+(K/diff_gaussian_rasterization_half_gaussian/__init__.py:199-207,
+ K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian).  No kernel runs here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ROOT, orc
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rgs.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rgs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from retinags_amd import _capi
+    names = _declared_symbols()
+    assert len(names) >= 20
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/rgs.h but not exported"
+    assert set(_capi.EXPORTS) == set(names)
+    assert _capi.lib.rgs_version() >= 100
+    assert _capi.lib.rgs_last_error() is not None
+
+
+def test_higher_msb_matches_checker():
+    from retinags_amd import _capi
+    for n in list(range(1, 3000)) + [6500, 8160, 68250, 2 ** 20 - 1, 2 ** 20, 2 ** 31 - 1]:
+        assert _capi.lib.rgs_get_higher_msb(n) == orc.get_higher_msb(n) == n.bit_length()
+
+
+def test_workspace_sizes_and_layouts_are_consistent():
+    from retinags_amd import _capi
+    for P in (1, 255, 256, 257, 100_000):
+        lay = _capi.geom_layout(P)
+        total = _capi.lib.rgs_geom_bytes(P)
+        sizes = dict(depths=4 * P, xy=8 * P, clip_w=4 * P, cov3D=24 * P, conic_opacity=16 * P, rgb=12 * P,
+                     tiles_touched=4 * P, point_offsets=4 * P, clamped=P, block_sums=4 * ((P + 255) // 256 + 1), total=4)
+        spans = sorted((lay[k], lay[k] + sizes[k]) for k in sizes)
+        assert all(a % 256 == 0 for a, _ in spans)
+        assert all(spans[i][1] <= spans[i + 1][0] for i in range(len(spans) - 1))
+        assert spans[-1][1] <= total
+    for R, (W, H) in ((1, (512, 512)), (4097, (1600, 1036)), (10 ** 6, (5185, 3359))):
+        lay = _capi.binning_layout(R, W, H)
+        total = _capi.lib.rgs_binning_bytes(R)
+        sizes = dict(keys_unsorted=8 * R, keys_sorted=8 * R, values_unsorted=4 * R, values_sorted=4 * R,
+                     sort_temp=_capi.lib.rgs_sort_temp_bytes(R))
+        spans = sorted((lay[k], lay[k] + sizes[k]) for k in sizes)
+        assert all(spans[i][1] <= spans[i + 1][0] for i in range(len(spans) - 1))
+        assert spans[-1][1] <= total
+    lay = _capi.image_layout(1600, 1036)
+    assert lay["n_contrib"] >= 8 * 6500 and lay["n_contrib"] + 4 * 1600 * 1036 <= _capi.lib.rgs_image_bytes(1600, 1036)
+
+
+def test_entry_points_reject_bad_arguments_without_launching():
+    from retinags_amd import _capi
+    lib = _capi.lib
+    null = ctypes.c_void_p(0)
+    assert lib.rgs_mark_visible(-1, null, null, null, null, null) != 0
+    assert b"negative" in lib.rgs_last_error()
+    assert lib.rgs_mark_visible(0, null, null, null, null, null) == 0
+    assert lib.rgs_sort_pairs(null, null, null, null, 10, 0, null, null) != 0
+    assert lib.rgs_sort_pairs(null, null, null, null, 0, 40, null, null) == 0
+    assert lib.rgs_inclusive_sum(null, null, 0, null, null) == 0
+    tbl = (ctypes.c_void_p * 1)()
+    assert lib.rgs_composite_forward(0, 4, 4, tbl, tbl, tbl, null, null, null, null, null) != 0
+    assert lib.rgs_composite_forward(65, 4, 4, tbl, tbl, tbl, null, null, null, null, null) != 0
+    assert b"outside" in lib.rgs_last_error()
+    rc = lib.rgs_forward_geom(0, 3, 16, 64, 64, null, null, null, null, null, 1.0, null, null, null, null, null,
+                              1.0, 1.0, 0, null, null, 0, null, null, 0)
+    assert rc != 0 and b"P must be positive" in lib.rgs_last_error()
+
+
+def test_rasterizer_argument_validation_matches_reference():
+    from diff_gaussian_rasterization_half_gaussian import GaussianRasterizationSettings, GaussianRasterizer
+    z = torch.zeros
+    settings = GaussianRasterizationSettings(
+        image_height=32, image_width=32, tanfovx=0.5, tanfovy=0.5, bg=z(3), scale_modifier=1.0, viewmatrix=torch.eye(4),
+        projmatrix=torch.eye(4), projmatrix_inv=torch.eye(4), range_low=-torch.ones(3), range_up=torch.ones(3),
+        sh_degree=3, campos=z(3), prefiltered=False, debug=False)
+    assert settings._fields == ("image_height", "image_width", "tanfovx", "tanfovy", "bg", "scale_modifier",
+                                "viewmatrix", "projmatrix", "projmatrix_inv", "range_low", "range_up", "sh_degree",
+                                "campos", "prefiltered", "debug")
+    r = GaussianRasterizer(settings)
+    m = z(5, 3)
+    with pytest.raises(Exception, match="SHs or precomputed colors"):
+        r(means3D=m, means2D=m, opacities=z(5, 1), scales=z(5, 3), rotations=z(5, 4))
+    with pytest.raises(Exception, match="SHs or precomputed colors"):
+        r(means3D=m, means2D=m, opacities=z(5, 1), shs=z(5, 16, 3), colors_precomp=z(5, 3), scales=z(5, 3), rotations=z(5, 4))
+    with pytest.raises(Exception, match="scale/rotation pair or precomputed 3D covariance"):
+        r(means3D=m, means2D=m, opacities=z(5, 1), shs=z(5, 16, 3))
+    with pytest.raises(Exception, match="scale/rotation pair or precomputed 3D covariance"):
+        r(means3D=m, means2D=m, opacities=z(5, 1), shs=z(5, 16, 3), scales=z(5, 3), rotations=z(5, 4), cov3D_precomp=z(5, 6))
+    # wrong rank of means3D is an error (K/rasterize_points.cu:60-62); host tensors cannot be rasterized
+    with pytest.raises(RuntimeError, match="num_points, 3"):
+        r(means3D=z(5), means2D=m, opacities=z(5, 1), shs=z(5, 16, 3), scales=z(5, 3), rotations=z(5, 4))
+    with pytest.raises(RuntimeError, match="GPU"):
+        r(means3D=m, means2D=m, opacities=z(5, 1), shs=z(5, 16, 3), scales=z(5, 3), rotations=z(5, 4))
+
+
+def test_no_shipped_module_touches_the_checker():
+    """The product path must not import, load or call anything under oracle/."""
+    for base, _, files in os.walk(os.path.join(ROOT, "retinags_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text and "rgs_oracle" not in text, os.path.join(base, f)
+    text = open(os.path.join(ROOT, "diff_gaussian_rasterization_half_gaussian", "__init__.py")).read()
+    assert "oracle" not in text
+
+
+def test_partition_and_order_invariants():
+    from retinags_amd.harness import scenes, partition
+    scene, cam, _ = scenes.make_config("C1", shrink=200)
+    n = scene["xyz"].shape[0]
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    assert len(part.leaves) == 4 and [l.path for l in part.leaves] == ["00", "01", "10", "11"]
+    # leaves tile the grid without overlap
+    cells = np.zeros(part.grid.size, dtype=np.int32)
+    for l in part.leaves:
+        cells[l.low[0]:l.up[0], l.low[1]:l.up[1], l.low[2]:l.up[2]] += 1
+    assert (cells == 1).all()
+    # balanced by load within a few percent at this size
+    own_counts = np.bincount(part.owner, minlength=4)
+    assert own_counts.sum() == n and own_counts.min() > 0.2 * n
+    xyz = scene["xyz"].numpy()
+    for k in range(4):
+        ids = part.members[k]
+        own = ids[: own_counts[k]]
+        assert (part.owner[own] == k).all() and (np.diff(own) > 0).all()
+        assert ((xyz[own] >= part.box_low[k]) & (xyz[own] <= part.box_up[k])).all()
+        shared = ids[own_counts[k]:]
+        assert (part.owner[shared] != k).all()
+        src = part.owner[shared]
+        assert (np.diff(src) >= 0).all()  # ascending source submodel
+        r = 3.0 * scene["scales"].numpy()[shared].max(axis=1)
+        assert ((xyz[shared] + r[:, None] >= part.box_low[k]) & (xyz[shared] - r[:, None] <= part.box_up[k])).all()
+    rel = partition.relation_vector(part, cam)
+    seen = sorted(v for v in rel if v >= 0)
+    assert len(set(seen)) == len(seen)
+    # the submodel that contains the camera's (x, y) is composited first
+    c = cam.camera_center.numpy()
+    inside = [k for k in range(4) if (c[:2] >= part.box_low[k][:2]).all() and (c[:2] <= part.box_up[k][:2]).all()]
+    assert inside and rel[inside[0]] == min(seen)

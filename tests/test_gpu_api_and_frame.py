@@ -1,0 +1,177 @@
+"""The public API of the HIP rasterizer on the GPU: golden vectors, input modes of the
+reference interface (precomputed colours / covariance, empty input, markVisible, debug),
+and a whole partitioned frame (4 submodels rendered in turn, composited, differentiated)
+against the CPU checker."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import (DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, ROOT, np32, oracle_settings, orc, rel_l2, scenes)
+from test_golden_cpu import load_cases, settings_of
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _settings(c_or_s, debug=False):
+    from retinags_amd import GaussianRasterizationSettings
+    s = c_or_s
+    t = lambda a: torch.from_numpy(np.asarray(a, np.float32)).to(DEV)
+    return GaussianRasterizationSettings(
+        image_height=s.image_height, image_width=s.image_width, tanfovx=s.tanfovx, tanfovy=s.tanfovy, bg=t(s.bg),
+        scale_modifier=s.scale_modifier, viewmatrix=t(s.viewmatrix).view(4, 4), projmatrix=t(s.projmatrix).view(4, 4),
+        projmatrix_inv=t(s.projmatrix_inv).view(4, 4), range_low=t(s.range_low), range_up=t(s.range_up),
+        sh_degree=s.sh_degree, campos=t(s.campos), prefiltered=False, debug=debug)
+
+
+def test_golden_vectors_forward_and_backward():
+    from retinags_amd import GaussianRasterizer
+    for name, c in load_cases().items():
+        s = settings_of(c)
+        t = lambda k: torch.from_numpy(c[k]).to(DEV).requires_grad_(True)
+        xyz, opa, sc, rot, shs = t("xyz"), t("opacity"), t("scales"), t("rotations"), t("shs")
+        m2d = torch.zeros_like(xyz, requires_grad=True)
+        color, radii, depth, alpha = GaussianRasterizer(_settings(s))(
+            means3D=xyz, means2D=m2d, opacities=opa, shs=shs, scales=sc, rotations=rot)
+        assert np.array_equal(radii.cpu().numpy(), c["radii"]), name
+        H, W = s.image_height, s.image_width
+        safe = (c["margin"] > DECISION_MARGIN).reshape(H, W)
+        for got, key in ((color, "color"), (depth, "depth"), (alpha, "alpha")):
+            assert np.abs(got.detach().cpu().numpy() - c[key])[:, safe].max() <= IMAGE_TOL, (name, key)
+        d = lambda k: torch.from_numpy(c[k]).to(DEV)
+        torch.autograd.backward([color, depth, alpha], [d("g_color"), d("g_depth"), d("g_alpha")])
+        for got, key in ((xyz.grad, "means3D"), (m2d.grad, "means2D"), (opa.grad, "opacity"), (sc.grad, "scales"),
+                         (rot.grad, "rotations"), (shs.grad, "sh")):
+            assert rel_l2(got.cpu().numpy(), c["grad_" + key]) <= GRAD_TOL, (name, key)
+
+
+def _small_inputs(n=3000, seed=3):
+    scene, cam, _ = scenes.make_config("C0", shrink=100_000 / n, resolution_scale=0.25)
+    pad = 3.0 * float(scene["scales"].max()) + 1.0
+    low, up = scene["xyz"].min(0).values - pad, scene["xyz"].max(0).values + pad
+    return scene, cam, low, up
+
+
+def test_precomputed_colours_and_covariance_modes():
+    """colors_precomp / cov3D_precomp inputs (K/.../__init__.py:209-218) give the same image as
+    SHs / scale+rotation when fed the values the preprocess would compute, and their
+    gradients match the checker's."""
+    from retinags_amd import GaussianRasterizer
+    scene, cam, low, up = _small_inputs()
+    bg = torch.tensor([0.2, 0.1, 0.4])
+    s = oracle_settings(cam, low, up, bg)
+    st = orc.forward(s, np32(scene["xyz"]), np32(scene["opacity"]), shs=np32(scene["shs"]),
+                     scales=np32(scene["scales"]), rotations=np32(scene["rotations"]))
+    rgb, cov = st.rgb.copy(), st.cov3D.copy()
+    st2 = orc.forward(s, np32(scene["xyz"]), np32(scene["opacity"]), colors_precomp=rgb, cov3D_precomp=cov)
+    assert np.array_equal(st2.color, st.color)
+    H, W = cam.image_height, cam.image_width
+    g_color = np32(torch.randn(3, H, W, generator=torch.Generator().manual_seed(1)) * 1e-2)
+    want = orc.backward(s, st2, g_color)
+    xyz = scene["xyz"].to(DEV).requires_grad_(True)
+    opa = scene["opacity"].to(DEV).requires_grad_(True)
+    col = torch.from_numpy(rgb).to(DEV).requires_grad_(True)
+    c3d = torch.from_numpy(cov).to(DEV).requires_grad_(True)
+    color, radii, depth, alpha = GaussianRasterizer(_settings(s))(
+        means3D=xyz, means2D=torch.zeros_like(xyz), opacities=opa, colors_precomp=col, cov3D_precomp=c3d)
+    assert np.array_equal(radii.cpu().numpy(), st.radii)
+    assert np.abs(color.detach().cpu().numpy() - st.color).max() <= 2e-2
+    assert np.median(np.abs(color.detach().cpu().numpy() - st.color)) <= 1e-6
+    torch.autograd.backward([color], [torch.from_numpy(g_color).to(DEV)])
+    assert rel_l2(col.grad.cpu().numpy(), want["colors"]) <= GRAD_TOL
+    assert rel_l2(c3d.grad.cpu().numpy(), want["cov3D"]) <= GRAD_TOL
+    assert rel_l2(xyz.grad.cpu().numpy(), want["means3D"]) <= GRAD_TOL
+    assert rel_l2(opa.grad.cpu().numpy(), want["opacity"]) <= GRAD_TOL
+
+
+def test_empty_input_and_nothing_visible():
+    from retinags_amd import GaussianRasterizer
+    scene, cam, low, up = _small_inputs(64)
+    s = oracle_settings(cam, low, up, torch.tensor([0.3, 0.6, 0.9]))
+    r = GaussianRasterizer(_settings(s))
+    z = lambda *shape: torch.zeros(*shape, device=DEV)
+    color, radii, depth, alpha = r(means3D=z(0, 3), means2D=z(0, 3), opacities=z(0, 1), shs=z(0, 16, 3),
+                                   scales=z(0, 3), rotations=z(0, 4))
+    assert radii.numel() == 0 and float(color.abs().sum()) == 0.0 and float(alpha.abs().sum()) == 0.0
+    # every Gaussian behind the camera: no instance is generated, the image is the background
+    xyz = scene["xyz"].clone()
+    xyz[:, 2] = -xyz[:, 2]
+    xyz = xyz.to(DEV).requires_grad_(True)
+    color, radii, depth, alpha = r(means3D=xyz, means2D=torch.zeros_like(xyz), opacities=scene["opacity"].to(DEV),
+                                   shs=scene["shs"].to(DEV), scales=scene["scales"].to(DEV),
+                                   rotations=scene["rotations"].to(DEV))
+    assert int(radii.abs().sum()) == 0 and float(alpha.abs().sum()) == 0.0
+    assert torch.allclose(color, torch.tensor([0.3, 0.6, 0.9], device=DEV).view(3, 1, 1).expand_as(color))
+    color.sum().backward()
+    assert float(xyz.grad.abs().sum()) == 0.0
+
+
+def test_mark_visible_and_debug_mode():
+    from retinags_amd import GaussianRasterizer
+    scene, cam, low, up = _small_inputs(5000)
+    scene["xyz"][::3, 2] -= 6.0
+    s = oracle_settings(cam, low, up, torch.zeros(3))
+    r = GaussianRasterizer(_settings(s, debug=True))
+    vis = r.markVisible(scene["xyz"].to(DEV))
+    assert vis.dtype == torch.bool
+    assert np.array_equal(vis.cpu().numpy(), orc.mark_visible(s, np32(scene["xyz"])))
+    st = orc.forward(s, np32(scene["xyz"]), np32(scene["opacity"]), shs=np32(scene["shs"]),
+                     scales=np32(scene["scales"]), rotations=np32(scene["rotations"]))
+    xyz = scene["xyz"].to(DEV).requires_grad_(True)
+    color, radii, _, _ = r(means3D=xyz, means2D=torch.zeros_like(xyz), opacities=scene["opacity"].to(DEV),
+                           shs=scene["shs"].to(DEV), scales=scene["scales"].to(DEV), rotations=scene["rotations"].to(DEV))
+    assert np.array_equal(radii.cpu().numpy(), st.radii)
+    color.sum().backward()  # every stage synchronised and checked in debug mode
+    assert torch.isfinite(xyz.grad).all()
+
+
+def test_partitioned_frame_against_checker():
+    """4 submodels with shared boundary Gaussians, rendered one after another, composited in
+    BVH order, differentiated: images and every submodel's gradients vs the CPU checker."""
+    from retinags_amd.harness import partition, pipeline
+    scene, cam, _ = scenes.make_config("C1", shrink=150, resolution_scale=0.25)
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    rel = partition.relation_vector(part, cam)
+    subs = [s.requires_grad_(True) for s in pipeline.submodels_from_partition(scene, part, DEV)]
+    H, W = cam.image_height, cam.image_width
+    up = torch.randn(3, H, W, generator=torch.Generator().manual_seed(2)) * 1e-2
+    bg = torch.tensor([0.5, 0.5, 0.5])
+    out = pipeline.render_frame(cam.to(DEV), subs, rel, bg.to(DEV))
+    torch.autograd.backward([out["render"]], [up.to(DEV)])
+    torch.cuda.synchronize()
+
+    order = sorted((m for m in range(4) if rel[m] >= 0), key=lambda m: rel[m])
+    assert len(order) >= 2
+    states, sets = [], []
+    margin = np.full(H * W, np.inf, np.float32)
+    for m in order:
+        ids = part.members[m]
+        s = oracle_settings(cam, torch.from_numpy(part.box_low[m]), torch.from_numpy(part.box_up[m]), torch.zeros(3))
+        st = orc.forward(s, np32(scene["xyz"])[ids], np32(scene["opacity"])[ids], shs=np32(scene["shs"])[ids],
+                         scales=np32(scene["scales"])[ids], rotations=np32(scene["rotations"])[ids], want_margin=True)
+        margin = np.minimum(margin, st.margin)
+        states.append(st)
+        sets.append(s)
+        got = out["partial"][m]
+        assert np.array_equal(got["radii"].cpu().numpy(), st.radii)
+    safe = (margin > DECISION_MARGIN).reshape(H, W)
+    imgs, deps, alps = [st.color for st in states], [st.depth for st in states], [st.alpha for st in states]
+    w_img, w_dep, w_alp = orc.composite_forward(imgs, deps, alps, np32(bg))
+    assert np.abs(out["render"].detach().cpu().numpy() - w_img)[:, safe].max() <= IMAGE_TOL
+    assert np.abs(out["alpha"].detach().cpu().numpy() - w_alp)[:, safe].max() <= IMAGE_TOL
+    assert np.abs(out["depth"].detach().cpu().numpy() - w_dep)[:, safe].max() <= IMAGE_TOL * 10  # depths are O(10)
+    d_img, d_dep, d_alp = orc.composite_backward(imgs, deps, alps, np32(bg), np32(up))
+    for k, m in enumerate(order):
+        g = orc.backward(sets[k], states[k], d_img[k], d_dep[k], d_alp[k])
+        for key, t in (("means3D", subs[m].means3D), ("sh", subs[m].shs), ("opacity", subs[m].opacity),
+                       ("scales", subs[m].scales), ("rotations", subs[m].rotations)):
+            assert rel_l2(t.grad.cpu().numpy(), g[key]) <= GRAD_TOL, (m, key)
+    # the partition is exact where it matters: compositing the clipped partial renders agrees
+    # with one unclipped render of the whole scene up to the early-termination thresholds
+    pad = 3.0 * float(scene["scales"].max()) + 1.0
+    s_all = oracle_settings(cam, scene["xyz"].min(0).values - pad, scene["xyz"].max(0).values + pad, bg)
+    whole = orc.forward(s_all, np32(scene["xyz"]), np32(scene["opacity"]), shs=np32(scene["shs"]),
+                        scales=np32(scene["scales"]), rotations=np32(scene["rotations"]))
+    assert np.abs(w_img - whole.color).mean() < 2e-3
