@@ -102,8 +102,8 @@ def test_empty_input_and_nothing_visible():
     color, radii, depth, alpha = r(means3D=xyz, means2D=torch.zeros_like(xyz), opacities=scene["opacity"].to(DEV),
                                    shs=scene["shs"].to(DEV), scales=scene["scales"].to(DEV),
                                    rotations=scene["rotations"].to(DEV))
-    assert int(radii.abs().sum()) == 0 and float(alpha.abs().sum()) == 0.0
-    assert torch.allclose(color, torch.tensor([0.3, 0.6, 0.9], device=DEV).view(3, 1, 1).expand_as(color))
+    assert int(radii.abs().sum()) == 0 and float(alpha.detach().abs().sum()) == 0.0
+    assert torch.allclose(color.detach(), torch.tensor([0.3, 0.6, 0.9], device=DEV).view(3, 1, 1).expand_as(color))
     color.sum().backward()
     assert float(xyz.grad.abs().sum()) == 0.0
 
