@@ -360,8 +360,8 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
 		e = hipStreamSynchronize(s);
 	if (e != hipSuccess)
 		return fail("rgs_forward_geom: reading the instance count failed: %s", hipGetErrorString(e));
-	RGS_REQUIRE(*num_rendered_host < 0x80000000u,
-	            "rgs_forward_geom: %u (Gaussian, tile) instances exceed the 2^31 limit of the sort", *num_rendered_host);
+	RGS_REQUIRE(*num_rendered_host < 0x40000000u,
+	            "rgs_forward_geom: %u (Gaussian, tile) instances exceed the 2^30 limit of the sort", *num_rendered_host);
 	return 0;
 }
 
@@ -405,11 +405,19 @@ int rgs_forward_raster(int P, int R, int width, int height,
 		rgs::launch_sort_pairs(keys_a, keys_b, vals_a, vals_b, (size_t)R, end_bit, at<uint32_t>(binning_ws, b.temp), s);
 		RGS_STAGE("sort_pairs");
 		const bool sorted_in_a = (((end_bit + 7) / 8) % 2) == 0;
-		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, ranges, gx * gy, s);
+		if (debug) {
+			uint32_t status = 0;
+			hipError_t e = hipMemcpy(&status, rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), sizeof(status),
+			                         hipMemcpyDeviceToHost);
+			if (e != hipSuccess || status != 0)
+				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
+		}
+		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, ranges, gx * gy,
+		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), s);
 		RGS_STAGE("tile_ranges");
 		point_list = sorted_in_a ? vals_a : vals_b;
 	} else {
-		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, s);
+		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, nullptr, s);
 		RGS_STAGE("tile_ranges");
 	}
 
@@ -589,7 +597,7 @@ int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uin
 	if (n == 0)
 		return 0;
 	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out && temp, "rgs_sort_pairs: null pointer");
-	RGS_REQUIRE(n < 0x80000000ull, "rgs_sort_pairs: more than 2^31 pairs");
+	RGS_REQUIRE(n < 0x40000000ull, "rgs_sort_pairs: 2^30 pairs or more");
 	rgs::launch_sort_pairs(keys_in, keys_out, vals_in, vals_out, n, end_bit, static_cast<uint32_t*>(temp), s);
 	RGS_STAGE("sort_pairs");
 	if ((((end_bit + 7) / 8) % 2) == 0) {

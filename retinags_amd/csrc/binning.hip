@@ -138,57 +138,98 @@ void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, co
 // ---- radix sort -------------------------------------------------------------------------------
 // Replaces cub::DeviceRadixSort::SortPairs at K/cuda_rasterizer_hgs/rasterizer_impl.cu:312-317:
 // a stable least-significant-digit sort of (u64 key, u32 value) on key bits [0, end_bit),
-// 8 bits per pass.  Each pass: per-block digit histogram -> one scan of the
-// (digit-major) block x digit table -> rank-and-scatter.  A sort block owns kSortBlock
-// consecutive pairs; element order inside the block is (wave, round, lane), and ranking
-// preserves it, which makes every pass stable.
+// 8 bits per pass, in the one-sweep form: one kernel reads the keys once and builds the digit
+// histogram of every pass, then each pass is a single kernel whose blocks take tiles of
+// kSortBlock pairs in arrival order, rank them in LDS, obtain their global digit offsets from
+// the blocks before them through a chained look-back over per-tile status words, and scatter.
+// Element order inside a tile is (wave, round, lane); ranking preserves it, and tiles are
+// ordered by their id, so every pass is stable.
+//
+// Scratch layout (u32 words):
+//   [0, 2048)      digit histograms of up to 8 passes, turned into exclusive digit starts
+//   [2048, 2056)   tile counter of each pass
+//   [2056]         status: non-zero if a look-back ever gave up waiting (never expected)
+//   [kSortHeader + pass * 256 * tiles + tile * 256 + digit]  look-back words
+
+constexpr int kSortMaxPasses = 8;
+constexpr uint32_t kSortCounters = 2048;
+constexpr uint32_t kSortStatus = 2056;
+constexpr uint32_t kSortHeader = 2112;
+constexpr uint32_t kFlagAggregate = 1u << 30;  // word holds this tile's own digit count
+constexpr uint32_t kFlagInclusive = 2u << 30;  // word holds the count of this and all earlier tiles
+constexpr uint32_t kValueMask = (1u << 30) - 1u;
+constexpr int kLookbackSpinLimit = 1 << 18;
 
 __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t mask)
 {
 	return (uint32_t)(key >> shift) & mask;
 }
 
-__global__ __launch_bounds__(256) void sort_histogram_kernel(const uint64_t* __restrict__ keys, size_t n, int shift,
-                                                              uint32_t mask, uint32_t* __restrict__ table,
-                                                              uint32_t nblocks)
+__global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const uint64_t* __restrict__ keys, size_t n,
+                                                                    int passes, int end_bit,
+                                                                    uint32_t* __restrict__ hist)
 {
-	__shared__ uint32_t hist[256];
-	hist[threadIdx.x] = 0;
+	__shared__ uint32_t s_hist[kSortMaxPasses][256];
+#pragma unroll
+	for (int p = 0; p < kSortMaxPasses; p++)
+		s_hist[p][threadIdx.x] = 0;
 	__syncthreads();
-	const size_t base = (size_t)blockIdx.x * kSortBlock;
-#pragma unroll 4
-	for (int i = 0; i < kSortItems; i++) {
-		const size_t k = base + (size_t)i * 256 + threadIdx.x;
-		if (k < n)
-			atomicAdd(&hist[digit_of(keys[k], shift, mask)], 1u);
+	for (size_t k = (size_t)blockIdx.x * 256 + threadIdx.x; k < n; k += (size_t)gridDim.x * 256) {
+		const uint64_t key = keys[k];
+		for (int p = 0; p < passes; p++) {
+			const int shift = 8 * p;
+			const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+			atomicAdd(&s_hist[p][digit_of(key, shift, (1u << bits) - 1u)], 1u);
+		}
 	}
 	__syncthreads();
-	table[(size_t)threadIdx.x * nblocks + blockIdx.x] = hist[threadIdx.x];
+	for (int p = 0; p < passes; p++) {
+		const uint32_t c = s_hist[p][threadIdx.x];
+		if (c)
+			atomicAdd(&hist[p * 256 + threadIdx.x], c);
+	}
 }
 
-__global__ __launch_bounds__(256) void sort_scatter_kernel(const uint64_t* __restrict__ keys_in,
-                                                            const uint32_t* __restrict__ vals_in,
-                                                            uint64_t* __restrict__ keys_out,
-                                                            uint32_t* __restrict__ vals_out, size_t n, int shift,
-                                                            uint32_t mask, const uint32_t* __restrict__ table,
-                                                            uint32_t nblocks)
+__global__ __launch_bounds__(256) void sort_digit_starts_kernel(uint32_t* __restrict__ hist, int passes)
+{
+	__shared__ uint32_t lds[8];
+	for (int p = 0; p < passes; p++) {
+		uint32_t total;
+		const uint32_t c = hist[p * 256 + threadIdx.x];
+		const uint32_t ex = block256_exclusive_scan_u32(c, lds, total);
+		hist[p * 256 + threadIdx.x] = ex;
+	}
+}
+
+__global__ __launch_bounds__(256) void sort_onesweep_kernel(const uint64_t* __restrict__ keys_in,
+                                                             const uint32_t* __restrict__ vals_in,
+                                                             uint64_t* __restrict__ keys_out,
+                                                             uint32_t* __restrict__ vals_out, size_t n, int shift,
+                                                             uint32_t mask, const uint32_t* __restrict__ digit_start,
+                                                             uint32_t* __restrict__ lookback,
+                                                             uint32_t* __restrict__ tile_counter,
+                                                             uint32_t* __restrict__ status)
 {
 	__shared__ uint64_t s_keys[kSortBlock];
 	__shared__ uint32_t s_vals[kSortBlock];
 	__shared__ uint32_t s_wave_hist[4][256];  // per-wave digit counts, then exclusive prefix over waves
-	__shared__ uint32_t s_digit_base[256];    // exclusive prefix over digits within the block
-	__shared__ uint32_t s_global_base[256];   // where this block's run of each digit starts globally
+	__shared__ uint32_t s_digit_base[256];    // exclusive prefix over digits within the tile
+	__shared__ uint32_t s_global_base[256];   // where this tile's run of each digit starts globally
 	__shared__ uint32_t s_scan[8];
+	__shared__ uint32_t s_tile;
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const size_t block_base = (size_t)blockIdx.x * kSortBlock;
-	const size_t wave_base = block_base + (size_t)wave * (kSortItems * 64);
-
+	// Tiles are handed out in arrival order, so every tile a block waits for below belongs to
+	// a block that is already running.
+	if (tid == 0)
+		s_tile = atomicAdd(tile_counter, 1u);
 #pragma unroll
 	for (int w = 0; w < 4; w++)
 		s_wave_hist[w][tid] = 0;
-	s_global_base[tid] = table[(size_t)tid * nblocks + blockIdx.x];
 	__syncthreads();
+	const uint32_t tile = s_tile;
+	const size_t block_base = (size_t)tile * kSortBlock;
+	const size_t wave_base = block_base + (size_t)wave * (kSortItems * 64);
 
 	uint64_t key[kSortItems];
 	uint32_t val[kSortItems];
@@ -228,17 +269,60 @@ __global__ __launch_bounds__(256) void sort_scatter_kernel(const uint64_t* __res
 	}
 	__syncthreads();
 
-	// Per digit: exclusive prefix over the 4 waves, block total, then exclusive prefix over digits.
+	// Thread d owns digit d: prefix over the 4 waves, publish the tile's count, look back.
 	{
+		const size_t remaining = n - block_base;
+		const uint32_t valid = remaining < (size_t)kSortBlock ? (uint32_t)remaining : (uint32_t)kSortBlock;
 		const uint32_t c0 = s_wave_hist[0][tid], c1 = s_wave_hist[1][tid], c2 = s_wave_hist[2][tid],
 		               c3 = s_wave_hist[3][tid];
 		s_wave_hist[0][tid] = 0;
 		s_wave_hist[1][tid] = c0;
 		s_wave_hist[2][tid] = c0 + c1;
 		s_wave_hist[3][tid] = c0 + c1 + c2;
+		uint32_t count = c0 + c1 + c2 + c3;
 		uint32_t total;
-		const uint32_t ex = block256_exclusive_scan_u32(c0 + c1 + c2 + c3, s_scan, total);
+		const uint32_t ex = block256_exclusive_scan_u32(count, s_scan, total);
 		s_digit_base[tid] = ex;
+		if (tid == 255)
+			count -= (uint32_t)kSortBlock - valid;  // padding is not published
+
+		uint32_t* my_word = lookback + (size_t)tile * 256 + tid;
+		uint32_t exclusive = 0;
+		if (tile == 0) {
+			__hip_atomic_store(my_word, count | kFlagInclusive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		} else {
+			__hip_atomic_store(my_word, count | kFlagAggregate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			uint32_t t = tile;
+			bool gave_up = false;
+			while (true) {
+				t--;
+				const uint32_t* word = lookback + (size_t)t * 256 + tid;
+				uint32_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				for (int spins = 0; (v >> 30) == 0u; spins++) {
+					// give up after a bounded wait, or as soon as any other look-back has
+					if (spins >= kLookbackSpinLimit ||
+					    ((spins & 255) == 255 &&
+					     __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+						gave_up = true;
+						break;
+					}
+					__builtin_amdgcn_s_sleep(1);
+					v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				}
+				if (gave_up)
+					break;
+				exclusive += v & kValueMask;
+				if ((v & kFlagInclusive) || t == 0)
+					break;
+			}
+			if (gave_up)
+				atomicOr(status, 1u);
+			// On the (never expected) give-up path `exclusive` is too small, which keeps every
+			// scatter address inside the array; the status word tells the consumer to discard it.
+			__hip_atomic_store(my_word, ((exclusive + count) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
+			                   __HIP_MEMORY_SCOPE_AGENT);
+		}
+		s_global_base[tid] = digit_start[tid] + exclusive;
 	}
 	__syncthreads();
 
@@ -261,22 +345,23 @@ __global__ __launch_bounds__(256) void sort_scatter_kernel(const uint64_t* __res
 			const uint64_t kk = s_keys[p];
 			const uint32_t d = digit_of(kk, shift, mask);
 			const size_t dst = (size_t)s_global_base[d] + (p - s_digit_base[d]);
-			keys_out[dst] = kk;
-			vals_out[dst] = s_vals[p];
+			if (dst < n) {
+				keys_out[dst] = kk;
+				vals_out[dst] = s_vals[p];
+			}
 		}
 	}
 }
 
 size_t sort_temp_words(size_t n)
 {
-	const size_t nblocks = (n + kSortBlock - 1) / kSortBlock;
-	return 256 * (nblocks > 0 ? nblocks : 1) + 64;
+	const size_t tiles = (n + kSortBlock - 1) / kSortBlock;
+	return kSortHeader + (size_t)kSortMaxPasses * 256 * (tiles > 0 ? tiles : 1);
 }
 
-// Returns 0 when the sorted pairs end in keys_out/vals_out, 1 when they end in keys_in/vals_in.
-int sort_pairs_passes(int end_bit)
+const uint32_t* sort_status_word(const uint32_t* temp)
 {
-	return (end_bit + 7) / 8;
+	return temp + kSortStatus;
 }
 
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
@@ -284,20 +369,23 @@ void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in,
 {
 	if (n == 0)
 		return;
-	const uint32_t nblocks = (uint32_t)((n + kSortBlock - 1) / kSortBlock);
+	const uint32_t tiles = (uint32_t)((n + kSortBlock - 1) / kSortBlock);
+	const int passes = (end_bit + 7) / 8;
+	stage_mark("sort_setup", s);
+	launch_fill_u32(temp, 0u, kSortHeader + (size_t)passes * 256 * tiles, s);
+	const uint32_t hist_blocks = tiles < 2048u ? tiles : 2048u;
+	hipLaunchKernelGGL(sort_digit_histogram_kernel, dim3(hist_blocks), dim3(256), 0, s, keys_in, n, passes, end_bit, temp);
+	hipLaunchKernelGGL(sort_digit_starts_kernel, dim3(1), dim3(256), 0, s, temp, passes);
 	uint64_t *ksrc = keys_in, *kdst = keys_out;
 	uint32_t *vsrc = vals_in, *vdst = vals_out;
-	for (int shift = 0; shift < end_bit; shift += 8) {
+	for (int p = 0; p < passes; p++) {
+		const int shift = 8 * p;
 		const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
 		const uint32_t mask = (1u << bits) - 1u;
-		stage_mark("sort_histogram", s);
-		hipLaunchKernelGGL(sort_histogram_kernel, dim3(nblocks), dim3(256), 0, s, ksrc, n, shift, mask, temp, nblocks);
-		stage_mark("sort_scan", s);
-		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, (size_t)256 * nblocks,
-		                   (uint32_t*)nullptr);
-		stage_mark("sort_scatter", s);
-		hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, shift, mask,
-		                   temp, nblocks);
+		stage_mark("sort_onesweep", s);
+		hipLaunchKernelGGL(sort_onesweep_kernel, dim3(tiles), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, shift, mask,
+		                   temp + p * 256, temp + kSortHeader + (size_t)p * 256 * tiles, temp + kSortCounters + p,
+		                   temp + kSortStatus);
 		uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
 		uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
 	}
@@ -319,11 +407,16 @@ void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 	hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, v, n);
 }
 
+// `sort_status` (may be null) is the sort's status word: if the sort reported a failure the
+// ranges stay empty, so no later stage walks an unsorted list.
 __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint64_t* __restrict__ keys, size_t n,
-                                                           uint2* __restrict__ ranges)
+                                                           uint2* __restrict__ ranges,
+                                                           const uint32_t* __restrict__ sort_status)
 {
 	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
 	if (idx >= n)
+		return;
+	if (sort_status && *sort_status != 0u)
 		return;
 	const uint32_t cur = (uint32_t)(keys[idx] >> 32);
 	if (idx == 0) {
@@ -339,13 +432,15 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint64_t* __rest
 		ranges[cur].y = (uint32_t)n;
 }
 
-void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, hipStream_t s)
+void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
+                        hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
 	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2, s);
 	if (n == 0)
 		return;
-	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges);
+	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges,
+	                   sort_status);
 }
 
 }  // namespace rgs

@@ -132,7 +132,9 @@ size_t sort_temp_words(size_t n);                 // u32 words of scratch for la
 // keys_out/vals_out, an even one in keys_in/vals_in.
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s);
-void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, hipStream_t s);
+const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
+void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
+                        hipStream_t s);
 
 // blend.hip
 void launch_blend_forward(const BlendArgs& a, hipStream_t s);
