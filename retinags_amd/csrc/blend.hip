@@ -1,12 +1,23 @@
 // Per-tile alpha blending, forward and backward.  One 16x16 tile per 256-thread block:
-// 4 wavefronts of 64 lanes, wavefront w owns pixel rows 4w..4w+3 of the tile, one pixel
-// per lane.  Tile lists are staged through LDS in batches of 256 entries.
+// 4 wavefronts of 64 lanes, wavefront w owns the strip of pixel rows 4w..4w+3 of the tile,
+// one pixel per lane.  Tile lists are staged through LDS in batches of 256 entries.
 //
 // Compiled with -ffp-contract=off: every per-pixel decision (power > 0, alpha < 1/255,
 // the half-Gaussian box test, T(1-alpha) < 1e-4) is evaluated with the unfused
 // single-precision expressions of K/cuda_rasterizer_hgs/forward.cu:338-392
 // (K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian), so a pixel
 // can only differ from that evaluation through the last-bit behaviour of exp().
+//
+// Most (pixel, Gaussian) visits of the reference loop end at "alpha < 1/255".  Two
+// conservative filters remove such visits without changing any result:
+//  * alpha >= 1/255 needs power >= -ln(255 * opacity).  The staging thread stores that floor
+//    (minus a margin) with the Gaussian, and a wavefront skips an entry with one ballot when
+//    no live lane reaches it, before exp() is evaluated.
+//  * power >= floor describes an ellipse around the Gaussian's centre.  The staging thread
+//    intersects the ellipse's bounding box with the four 16x4 strips of the tile and files the
+//    entry only in the lists of the strips it can reach; each wavefront walks its own list,
+//    four entries at a time so that the LDS reads and the four exponent evaluations overlap.
+// Both filters only drop visits that the exact evaluation would have skipped too.
 #include "rgs_kernels.h"
 
 namespace rgs {
@@ -27,20 +38,118 @@ __device__ __forceinline__ bool clipped_by_box(const PixelRay& ray, float w, flo
 	return (wx <= lo.x) || (wx > hi.x) || (wy <= lo.y) || (wy > hi.y) || (wz <= lo.z) || (wz > hi.z);
 }
 
+// Lower bound on `power` below which alpha = min(0.99, opacity * exp(power)) is certainly
+// under 1/255.  A NaN opacity makes alpha 0.99 in the exact evaluation (fminf drops the NaN),
+// so it must never be culled; a non-positive one can never reach 1/255.
+__device__ __forceinline__ float exponent_floor(float opacity)
+{
+	if (opacity != opacity)
+		return -INFINITY;
+	if (!(opacity > 0.f))
+		return INFINITY;
+	return -logf(255.0f * opacity) - 1e-3f;
+}
+
+// Bit w set: some pixel of strip w (rows 4w..4w+3 of the tile whose first pixel is
+// (x0, y0)) may reach power >= floor.  The region power >= floor is the ellipse
+// d^T Q d <= -2 floor with Q the conic; its bounding box has half-widths
+// sqrt(-2 floor * Q^-1_xx) and sqrt(-2 floor * Q^-1_yy), inflated here against rounding.
+// Every comparison is written so that NaN or a non-positive-definite conic keeps the entry.
+__device__ __forceinline__ uint32_t reachable_strips(float gx, float gy, const float4 conic, float floor, float x0,
+                                                     float y0)
+{
+	if (floor > 0.f)
+		return 0u;  // even power = 0 gives alpha < 1/255
+	const float det = conic.x * conic.z - conic.y * conic.y;
+	if (!(det > 0.f))
+		return 0xFu;
+	const float c = -2.f * floor;
+	const float hx = sqrtf(c * conic.z / det) * 1.0001f + 1e-2f;
+	const float hy = sqrtf(c * conic.x / det) * 1.0001f + 1e-2f;
+	if ((gx + hx < x0) || (gx - hx > x0 + 15.f))
+		return 0u;
+	uint32_t mask = 0u;
+#pragma unroll
+	for (int w = 0; w < 4; w++) {
+		const float ya = y0 + 4.f * w;
+		if (!((gy + hy < ya) || (gy - hy > ya + 3.f)))
+			mask |= 1u << w;
+	}
+	return mask;
+}
+
+constexpr int kPadSlot = 256;  // staged slot that never passes the floor test; pads lists to a multiple of 4
+
+// Files the staging thread's entry (slot `tid`, reachable strips `strips`) in the per-strip
+// lists.  Each staging wavefront owns a 64-entry segment of every strip's list and fills it in
+// slot order, so walking segments 0..3 visits a strip's entries in list order.
+__device__ __forceinline__ void file_in_strip_lists(uint32_t strips, int tid, uint16_t (*s_list)[256],
+                                                    uint32_t (*s_count)[4])
+{
+	const int lane = tid & 63, wave = tid >> 6;
+	const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll
+	for (int w = 0; w < 4; w++) {
+		const bool mine = (strips >> w) & 1u;
+		const uint64_t m = __ballot(mine);
+		const uint32_t n = (uint32_t)__popcll(m);
+		if (mine)
+			s_list[w][wave * 64 + __popcll(m & below)] = (uint16_t)tid;
+		if ((uint32_t)lane < ((4u - (n & 3u)) & 3u))
+			s_list[w][wave * 64 + n + lane] = (uint16_t)kPadSlot;
+		if (lane == 0)
+			s_count[wave][w] = n;
+	}
+}
+
+__device__ __forceinline__ float exponent_of(const float4 g, const float4 co, const float2 pixf, float2& d)
+{
+	d = float2{g.x - pixf.x, g.y - pixf.y};
+	return -0.5f * (co.x * d.x * d.x + co.z * d.y * d.y) - co.y * d.x * d.y;
+}
+
 // ---- forward (K/cuda_rasterizer_hgs/forward.cu:263-405) ---------------------------------------
 
-// kCount = true is the instrumented twin used for work accounting: it writes no image and
-// instead adds, over all pixels, the number of list entries visited by a live pixel (A), those
-// with power <= 0 (B), those with alpha >= 1/255 (C), those inside the box (D), those blended
-// (E), and the B and C counts restricted to entries up to each pixel's last blended one (B', C'),
-// which is what the backward pass re-evaluates.
-template <bool kCount>
+struct ForwardPixel {
+	bool done;
+	float T, C0, C1, C2, weight, D;
+	uint32_t last_contributor;
+};
+
+__device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, float power, const float4 g,
+                                              const float4 co, const float4* s_cd, int slot, uint32_t position,
+                                              const PixelRay& ray, const BlendArgs& a, const float3 lo, const float3 hi)
+{
+	candidate = candidate && !p.done;
+	if (__ballot(candidate) == 0ull)
+		return;
+	if (candidate) {
+		const float alpha = fminf(0.99f, co.w * expf(power));
+		if (!(alpha < 1.0f / 255.0f) && !clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi)) {
+			const float test_T = p.T * (1 - alpha);
+			if (test_T < 0.0001f) {
+				p.done = true;
+			} else {
+				const float4 cd = s_cd[slot];
+				p.C0 += cd.x * alpha * p.T;
+				p.C1 += cd.y * alpha * p.T;
+				p.C2 += cd.z * alpha * p.T;
+				p.weight += alpha * p.T;
+				p.D += cd.w * alpha * p.T;
+				p.T = test_T;
+				p.last_contributor = position;
+			}
+		}
+	}
+}
+
 __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 {
-	__shared__ float2 s_xy[256];
-	__shared__ float4 s_co[256];
-	__shared__ float4 s_cd[256];  // r, g, b, view depth
-	__shared__ float s_w[256];
+	__shared__ float4 s_geom[257];   // pixel x, pixel y, exponent floor, clip w
+	__shared__ float4 s_conic[257];  // conic xx, xy, yy, opacity
+	__shared__ float4 s_cd[256];     // r, g, b, view depth
+	__shared__ __attribute__((aligned(8))) uint16_t s_list[4][256];
+	__shared__ uint32_t s_count[4][4];  // [staging wave][strip]
 	__shared__ int s_alive[2][4];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -53,91 +162,145 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
 	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
 	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
+	const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
 
+	const uint2 range = a.ranges[tile];
+	const int rounds = (int)((range.y - range.x + 255) / 256);
+
+	ForwardPixel p = {!inside, 1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u};
+	if (tid == 0) {
+		s_geom[kPadSlot] = float4{0.f, 0.f, INFINITY, 0.f};
+		s_conic[kPadSlot] = float4{0.f, 0.f, 0.f, 0.f};
+	}
+
+	for (int i = 0; i < rounds; i++) {
+		uint64_t live = __ballot(!p.done);
+		if (lane == 0)
+			s_alive[i & 1][wave] = live != 0ull;
+		const uint32_t src = range.x + (uint32_t)i * 256 + tid;
+		uint32_t strips = 0u;
+		if (src < range.y) {
+			const uint32_t id = a.point_list[src];
+			const float2 xy = a.xy[id];
+			const float4 co = a.conic_opacity[id];
+			const float floor = exponent_floor(co.w);
+			strips = reachable_strips(xy.x, xy.y, co, floor, tile_x0, tile_y0);
+			s_geom[tid] = float4{xy.x, xy.y, floor, a.clip_w[id]};
+			s_conic[tid] = co;
+			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
+			                   a.depths[id]};
+		}
+		file_in_strip_lists(strips, tid, s_list, s_count);
+		__syncthreads();
+		if (!(s_alive[i & 1][0] | s_alive[i & 1][1] | s_alive[i & 1][2] | s_alive[i & 1][3]))
+			break;
+
+		for (int seg = 0; seg < 4 && live != 0ull; seg++) {
+			const int n = (int)s_count[seg][wave];
+			for (int k = 0; k < n && live != 0ull; k += 4) {
+				const uint2 packed = *reinterpret_cast<const uint2*>(&s_list[wave][seg * 64 + k]);
+				const int j0 = packed.x & 0xFFFFu, j1 = packed.x >> 16, j2 = packed.y & 0xFFFFu, j3 = packed.y >> 16;
+				const float4 g0 = s_geom[j0], g1 = s_geom[j1], g2 = s_geom[j2], g3 = s_geom[j3];
+				const float4 c0 = s_conic[j0], c1 = s_conic[j1], c2 = s_conic[j2], c3 = s_conic[j3];
+				float2 d;
+				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
+				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
+				// written with negations so that a NaN exponent is kept, as in the exact loop
+				const bool q0 = !(w0 > 0.0f) && !(w0 < g0.z), q1 = !(w1 > 0.0f) && !(w1 < g1.z),
+				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
+				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
+					continue;
+				const uint32_t base = (uint32_t)i * 256 + 1;
+				forward_visit(p, q0, w0, g0, c0, s_cd, j0, base + j0, ray, a, lo, hi);
+				forward_visit(p, q1, w1, g1, c1, s_cd, j1, base + j1, ray, a, lo, hi);
+				forward_visit(p, q2, w2, g2, c2, s_cd, j2, base + j2, ray, a, lo, hi);
+				forward_visit(p, q3, w3, g3, c3, s_cd, j3, base + j3, ray, a, lo, hi);
+				live = __ballot(!p.done);
+			}
+		}
+		__syncthreads();
+	}
+
+	if (inside) {
+		const size_t plane = (size_t)a.H * a.W;
+		a.n_contrib[pix_id] = p.last_contributor;
+		a.out_color[pix_id] = p.C0 + p.T * a.bg[0];
+		a.out_color[plane + pix_id] = p.C1 + p.T * a.bg[1];
+		a.out_color[2 * plane + pix_id] = p.C2 + p.T * a.bg[2];
+		a.out_alpha[pix_id] = p.weight;
+		a.out_depth[pix_id] = p.D;
+	}
+}
+
+// Work accounting: the reference loop taken literally, one list entry at a time with no
+// filter, counting over all pixels the entries visited by a live pixel (A), those with
+// power <= 0 (B), with alpha >= 1/255 (C), inside the box (D), blended (E), and B and C
+// restricted to entries up to each pixel's last blended one (the backward's share).
+__global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
+{
+	__shared__ float4 s_geom[256];
+	__shared__ float4 s_conic[256];
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int tile = blockIdx.x;
+	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
+	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
+	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
+	const float2 pixf = {(float)px, (float)py};
+	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
+	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
+	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
 	const uint2 range = a.ranges[tile];
 	const int rounds = (int)((range.y - range.x + 255) / 256);
 	int todo = (int)(range.y - range.x);
 
 	bool done = !inside;
 	float T = 1.0f;
-	uint32_t last_contributor = 0;
-	float C0 = 0.f, C1 = 0.f, C2 = 0.f, weight = 0.f, D = 0.f;
 	uint32_t nA = 0, nB = 0, nC = 0, nD = 0, nE = 0, nB_last = 0, nC_last = 0;
-
 	for (int i = 0; i < rounds; i++, todo -= 256) {
-		const int alive = __ballot(!done) != 0ull;
-		if (lane == 0)
-			s_alive[i & 1][wave] = alive;
+		__syncthreads();
 		const uint32_t src = range.x + (uint32_t)i * 256 + tid;
 		if (src < range.y) {
 			const uint32_t id = a.point_list[src];
-			s_xy[tid] = a.xy[id];
-			s_co[tid] = a.conic_opacity[id];
-			s_w[tid] = a.clip_w[id];
-			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
-			                   a.depths[id]};
+			const float2 xy = a.xy[id];
+			s_geom[tid] = float4{xy.x, xy.y, 0.f, a.clip_w[id]};
+			s_conic[tid] = a.conic_opacity[id];
 		}
 		__syncthreads();
-		if (!(s_alive[i & 1][0] | s_alive[i & 1][1] | s_alive[i & 1][2] | s_alive[i & 1][3]))
-			break;
-
 		const int count = todo < 256 ? todo : 256;
 		for (int j = 0; !done && j < count; j++) {
-			const float2 xy = s_xy[j];
-			const float2 d = {xy.x - pixf.x, xy.y - pixf.y};
-			const float4 co = s_co[j];
-			const float power = -0.5f * (co.x * d.x * d.x + co.z * d.y * d.y) - co.y * d.x * d.y;
-			if (kCount) nA++;
+			const float4 g = s_geom[j];
+			const float4 co = s_conic[j];
+			float2 d;
+			const float power = exponent_of(g, co, pixf, d);
+			nA++;
 			if (power > 0.0f)
 				continue;
-			if (kCount) nB++;
+			nB++;
 			const float alpha = fminf(0.99f, co.w * expf(power));
 			if (alpha < 1.0f / 255.0f)
 				continue;
-			if (kCount) nC++;
-			if (clipped_by_box(ray, s_w[j], a.tanfovx, a.tanfovy, a.projinv, lo, hi))
+			nC++;
+			if (clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))
 				continue;
-			if (kCount) nD++;
+			nD++;
 			const float test_T = T * (1 - alpha);
 			if (test_T < 0.0001f) {
 				done = true;
 				continue;
 			}
-			if (kCount) {
-				nE++;
-				nB_last = nB;
-				nC_last = nC;
-			}
-			const float4 cd = s_cd[j];
-			C0 += cd.x * alpha * T;
-			C1 += cd.y * alpha * T;
-			C2 += cd.z * alpha * T;
-			weight += alpha * T;
-			D += cd.w * alpha * T;
+			nE++;
+			nB_last = nB;
+			nC_last = nC;
 			T = test_T;
-			last_contributor = (uint32_t)(i * 256 + j + 1);
 		}
-		__syncthreads();
 	}
-
-	if (kCount) {
-		const uint32_t c[7] = {nA, nB, nC, nD, nE, nB_last, nC_last};
+	const uint32_t c[7] = {nA, nB, nC, nD, nE, nB_last, nC_last};
 #pragma unroll
-		for (int q = 0; q < 7; q++) {
-			const uint32_t tot = wave_inclusive_scan_u32(c[q]);
-			if (lane == 63)
-				atomicAdd(reinterpret_cast<unsigned long long*>(a.counters) + q, (unsigned long long)tot);
-		}
-		return;
-	}
-	if (inside) {
-		const size_t plane = (size_t)a.H * a.W;
-		a.n_contrib[pix_id] = last_contributor;
-		a.out_color[pix_id] = C0 + T * a.bg[0];
-		a.out_color[plane + pix_id] = C1 + T * a.bg[1];
-		a.out_color[2 * plane + pix_id] = C2 + T * a.bg[2];
-		a.out_alpha[pix_id] = weight;
-		a.out_depth[pix_id] = D;
+	for (int q = 0; q < 7; q++) {
+		const uint32_t tot = wave_inclusive_scan_u32(c[q]);
+		if (lane == 63)
+			atomicAdd(reinterpret_cast<unsigned long long*>(a.counters) + q, (unsigned long long)tot);
 	}
 }
 
@@ -149,14 +312,92 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 
 constexpr int kGradSlots = 10;  // mean2D x,y | conic xx,xy,yy | opacity | colour r,g,b | depth
 
+struct BackwardPixel {
+	float T, T_final;
+	float accum_r, accum_g, accum_b, accum_depth, accum_alpha;
+	float last_alpha, last_r, last_g, last_b, last_depth;
+	float g_r, g_g, g_b, g_depth, g_alpha;
+	float bg_dot_dpixel, ddelx_dx, ddely_dy;
+};
+
+__device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
+                                               const float4 co, const float2 pixf, const float4* s_cd,
+                                               float (*s_acc)[256], int slot, const PixelRay& ray, const BlendArgs& a,
+                                               const float3 lo, const float3 hi, int lane)
+{
+	if (__ballot(candidate) == 0ull)
+		return;
+	float v[kGradSlots];
+#pragma unroll
+	for (int q = 0; q < kGradSlots; q++)
+		v[q] = 0.f;
+	bool valid = false;
+	if (candidate) {
+		const float2 d = {g.x - pixf.x, g.y - pixf.y};
+		const float G = expf(power);
+		const float alpha = fminf(0.99f, co.w * G);
+		if (!(alpha < 1.0f / 255.0f) && !clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi)) {
+			valid = true;
+			p.T = p.T / (1.f - alpha);
+			const float aT = alpha * p.T;
+			const float4 cd = s_cd[slot];
+			float dL_dopa = 0.0f;
+			p.accum_r = p.last_alpha * p.last_r + (1.f - p.last_alpha) * p.accum_r;
+			p.last_r = cd.x;
+			dL_dopa += (cd.x - p.accum_r) * p.g_r;
+			p.accum_g = p.last_alpha * p.last_g + (1.f - p.last_alpha) * p.accum_g;
+			p.last_g = cd.y;
+			dL_dopa += (cd.y - p.accum_g) * p.g_g;
+			p.accum_b = p.last_alpha * p.last_b + (1.f - p.last_alpha) * p.accum_b;
+			p.last_b = cd.z;
+			dL_dopa += (cd.z - p.accum_b) * p.g_b;
+			p.accum_depth = p.last_alpha * p.last_depth + (1.f - p.last_alpha) * p.accum_depth;
+			p.last_depth = cd.w;
+			dL_dopa += (cd.w - p.accum_depth) * p.g_depth;
+			p.accum_alpha = p.last_alpha + (1.f - p.last_alpha) * p.accum_alpha;
+			dL_dopa += (1 - p.accum_alpha) * p.g_alpha;
+			dL_dopa *= p.T;
+			p.last_alpha = alpha;
+			dL_dopa += (-p.T_final / (1.f - alpha)) * p.bg_dot_dpixel;
+
+			const float dL_dG = co.w * dL_dopa;
+			const float gdx = G * d.x;
+			const float gdy = G * d.y;
+			const float dG_ddelx = -gdx * co.x - gdy * co.y;
+			const float dG_ddely = -gdy * co.z - gdx * co.y;
+			v[0] = dL_dG * dG_ddelx * p.ddelx_dx;
+			v[1] = dL_dG * dG_ddely * p.ddely_dy;
+			v[2] = -0.5f * gdx * d.x * dL_dG;
+			v[3] = -0.5f * gdx * d.y * dL_dG;
+			v[4] = -0.5f * gdy * d.y * dL_dG;
+			v[5] = G * dL_dopa;
+			v[6] = aT * p.g_r;
+			v[7] = aT * p.g_g;
+			v[8] = aT * p.g_b;
+			v[9] = aT * p.g_depth;
+		}
+	}
+	if (__ballot(valid) == 0ull)
+		return;
+#pragma unroll
+	for (int q = 0; q < kGradSlots; q++)
+		v[q] = wave_sum_to_lane63(v[q]);
+	if (lane == 63) {
+#pragma unroll
+		for (int q = 0; q < kGradSlots; q++)
+			atomicAdd(&s_acc[q][slot], v[q]);
+	}
+}
+
 __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 {
-	__shared__ float2 s_xy[256];
-	__shared__ float4 s_co[256];
+	__shared__ float4 s_geom[257];
+	__shared__ float4 s_conic[257];
 	__shared__ float4 s_cd[256];
-	__shared__ float s_w[256];
 	__shared__ uint32_t s_id[256];
 	__shared__ float s_acc[kGradSlots][256];
+	__shared__ __attribute__((aligned(8))) uint16_t s_list[4][256];
+	__shared__ uint32_t s_count[4][4];
 	__shared__ uint32_t s_max[4];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -170,133 +411,101 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
 	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
 	const size_t plane = (size_t)a.H * a.W;
+	const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
 
 	const uint2 range = a.ranges[tile];
 	const uint32_t last_contributor = inside ? a.n_contrib[pix_id] : 0u;
 
 	// Entries at or beyond the largest last_contributor of the tile are skipped by every
-	// pixel, so the walk starts there instead of at the end of the list.
-	uint32_t wmax = last_contributor;
+	// pixel, so the walk starts there instead of at the end of the list; likewise a strip's
+	// list only takes entries below the largest last_contributor of that strip's 64 pixels.
+	uint32_t wave_span = last_contributor;
 #pragma unroll
 	for (int off = 32; off > 0; off >>= 1)
-		wmax = max(wmax, (uint32_t)__shfl_xor((int)wmax, off));
+		wave_span = max(wave_span, (uint32_t)__shfl_xor((int)wave_span, off));
 	if (lane == 0)
-		s_max[wave] = wmax;
+		s_max[wave] = wave_span;
 #pragma unroll
 	for (int q = 0; q < kGradSlots; q++)
 		s_acc[q][tid] = 0.f;
+	if (tid == 0) {
+		s_geom[kPadSlot] = float4{0.f, 0.f, INFINITY, 0.f};
+		s_conic[kPadSlot] = float4{0.f, 0.f, 0.f, 0.f};
+	}
 	__syncthreads();
-	const uint32_t span = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3]));
+	const uint32_t span0 = s_max[0], span1 = s_max[1], span2 = s_max[2], span3 = s_max[3];
+	const uint32_t span = max(max(span0, span1), max(span2, span3));
 	if (span == 0)
 		return;
 	const uint32_t back = range.x + span;  // one past the last entry any pixel uses
 	const int rounds = (int)((span + 255) / 256);
 	int todo = (int)span;
 
-	const float T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
-	float T = T_final;
-	float accum_r = 0.f, accum_g = 0.f, accum_b = 0.f, accum_depth = 0.f, accum_alpha = 0.f;
-	float g_r = 0.f, g_g = 0.f, g_b = 0.f, g_depth = 0.f, g_alpha = 0.f;
+	BackwardPixel p;
+	p.T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
+	p.T = p.T_final;
+	p.accum_r = p.accum_g = p.accum_b = p.accum_depth = p.accum_alpha = 0.f;
+	p.last_alpha = p.last_r = p.last_g = p.last_b = p.last_depth = 0.f;
+	p.g_r = p.g_g = p.g_b = p.g_depth = p.g_alpha = 0.f;
 	if (inside) {
-		g_r = a.dL_dpix[pix_id];
-		g_g = a.dL_dpix[plane + pix_id];
-		g_b = a.dL_dpix[2 * plane + pix_id];
-		g_depth = a.dL_dpix_depth[pix_id];
-		g_alpha = a.dL_dalpha[pix_id];
+		p.g_r = a.dL_dpix[pix_id];
+		p.g_g = a.dL_dpix[plane + pix_id];
+		p.g_b = a.dL_dpix[2 * plane + pix_id];
+		p.g_depth = a.dL_dpix_depth[pix_id];
+		p.g_alpha = a.dL_dalpha[pix_id];
 	}
-	float last_alpha = 0.f, last_r = 0.f, last_g = 0.f, last_b = 0.f, last_depth = 0.f;
-	const float ddelx_dx = 0.5 * a.W;
-	const float ddely_dy = 0.5 * a.H;
-	const float bg_dot_dpixel = (0.f + a.bg[0] * g_r + a.bg[1] * g_g) + a.bg[2] * g_b;
+	p.ddelx_dx = 0.5 * a.W;
+	p.ddely_dy = 0.5 * a.H;
+	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
 
 	for (int i = 0; i < rounds; i++, todo -= 256) {
 		const uint32_t progress = (uint32_t)i * 256 + tid;
+		uint32_t strips = 0u;
 		if (progress < span) {
+			const uint32_t entry = span - 1 - progress;  // 0-based position in the tile list
 			const uint32_t id = a.point_list[back - progress - 1];
+			const float2 xy = a.xy[id];
+			const float4 co = a.conic_opacity[id];
+			const float floor = exponent_floor(co.w);
+			strips = reachable_strips(xy.x, xy.y, co, floor, tile_x0, tile_y0);
+			strips &= (entry < span0 ? 1u : 0u) | (entry < span1 ? 2u : 0u) | (entry < span2 ? 4u : 0u) |
+			          (entry < span3 ? 8u : 0u);
 			s_id[tid] = id;
-			s_xy[tid] = a.xy[id];
-			s_co[tid] = a.conic_opacity[id];
-			s_w[tid] = a.clip_w[id];
+			s_geom[tid] = float4{xy.x, xy.y, floor, a.clip_w[id]};
+			s_conic[tid] = co;
 			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
 			                   a.depths[id]};
+		}
+		file_in_strip_lists(strips, tid, s_list, s_count);
+		__syncthreads();
+
+		for (int seg = 0; seg < 4; seg++) {
+			const int n = (int)s_count[seg][wave];
+			for (int k = 0; k < n; k += 4) {
+				const uint2 packed = *reinterpret_cast<const uint2*>(&s_list[wave][seg * 64 + k]);
+				const int j0 = packed.x & 0xFFFFu, j1 = packed.x >> 16, j2 = packed.y & 0xFFFFu, j3 = packed.y >> 16;
+				const float4 g0 = s_geom[j0], g1 = s_geom[j1], g2 = s_geom[j2], g3 = s_geom[j3];
+				const float4 c0 = s_conic[j0], c1 = s_conic[j1], c2 = s_conic[j2], c3 = s_conic[j3];
+				float2 d;
+				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
+				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
+				// position of slot j in the tile list: span - 1 - (i * 256 + j)
+				const uint32_t top = span - 1 - (uint32_t)i * 256;
+				const bool q0 = (top - j0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z),
+				           q1 = (top - j1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z),
+				           q2 = (top - j2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z),
+				           q3 = (top - j3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
+				if (__ballot(q0 | q1 | q2 | q3) == 0ull)
+					continue;
+				backward_visit(p, q0, w0, g0, c0, pixf, s_cd, s_acc, j0, ray, a, lo, hi, lane);
+				backward_visit(p, q1, w1, g1, c1, pixf, s_cd, s_acc, j1, ray, a, lo, hi, lane);
+				backward_visit(p, q2, w2, g2, c2, pixf, s_cd, s_acc, j2, ray, a, lo, hi, lane);
+				backward_visit(p, q3, w3, g3, c3, pixf, s_cd, s_acc, j3, ray, a, lo, hi, lane);
+			}
 		}
 		__syncthreads();
 
 		const int count = todo < 256 ? todo : 256;
-		for (int j = 0; j < count; j++) {
-			// 0-based position of this entry in the tile list
-			const uint32_t entry = span - 1 - ((uint32_t)i * 256 + j);
-			float v[kGradSlots];
-			bool valid = false;
-			if (inside && entry < last_contributor) {
-				const float2 xy = s_xy[j];
-				const float2 d = {xy.x - pixf.x, xy.y - pixf.y};
-				const float4 co = s_co[j];
-				const float power = -0.5f * (co.x * d.x * d.x + co.z * d.y * d.y) - co.y * d.x * d.y;
-				if (!(power > 0.0f)) {
-					const float G = expf(power);
-					const float alpha = fminf(0.99f, co.w * G);
-					if (!(alpha < 1.0f / 255.0f) &&
-					    !clipped_by_box(ray, s_w[j], a.tanfovx, a.tanfovy, a.projinv, lo, hi)) {
-						valid = true;
-						T = T / (1.f - alpha);
-						const float aT = alpha * T;
-						const float4 cd = s_cd[j];
-						float dL_dopa = 0.0f;
-						accum_r = last_alpha * last_r + (1.f - last_alpha) * accum_r;
-						last_r = cd.x;
-						dL_dopa += (cd.x - accum_r) * g_r;
-						accum_g = last_alpha * last_g + (1.f - last_alpha) * accum_g;
-						last_g = cd.y;
-						dL_dopa += (cd.y - accum_g) * g_g;
-						accum_b = last_alpha * last_b + (1.f - last_alpha) * accum_b;
-						last_b = cd.z;
-						dL_dopa += (cd.z - accum_b) * g_b;
-						accum_depth = last_alpha * last_depth + (1.f - last_alpha) * accum_depth;
-						last_depth = cd.w;
-						dL_dopa += (cd.w - accum_depth) * g_depth;
-						accum_alpha = last_alpha + (1.f - last_alpha) * accum_alpha;
-						dL_dopa += (1 - accum_alpha) * g_alpha;
-						dL_dopa *= T;
-						last_alpha = alpha;
-						dL_dopa += (-T_final / (1.f - alpha)) * bg_dot_dpixel;
-
-						const float dL_dG = co.w * dL_dopa;
-						const float gdx = G * d.x;
-						const float gdy = G * d.y;
-						const float dG_ddelx = -gdx * co.x - gdy * co.y;
-						const float dG_ddely = -gdy * co.z - gdx * co.y;
-						v[0] = dL_dG * dG_ddelx * ddelx_dx;
-						v[1] = dL_dG * dG_ddely * ddely_dy;
-						v[2] = -0.5f * gdx * d.x * dL_dG;
-						v[3] = -0.5f * gdx * d.y * dL_dG;
-						v[4] = -0.5f * gdy * d.y * dL_dG;
-						v[5] = G * dL_dopa;
-						v[6] = aT * g_r;
-						v[7] = aT * g_g;
-						v[8] = aT * g_b;
-						v[9] = aT * g_depth;
-					}
-				}
-			}
-			if (__ballot(valid) == 0ull)
-				continue;
-			if (!valid) {
-#pragma unroll
-				for (int q = 0; q < kGradSlots; q++)
-					v[q] = 0.f;
-			}
-#pragma unroll
-			for (int q = 0; q < kGradSlots; q++)
-				v[q] = wave_sum_to_lane63(v[q]);
-			if (lane == 63) {
-#pragma unroll
-				for (int q = 0; q < kGradSlots; q++)
-					atomicAdd(&s_acc[q][j], v[q]);
-			}
-		}
-		__syncthreads();
-
 		if (tid < count) {
 			const size_t id = s_id[tid];
 			float r[kGradSlots];
@@ -323,9 +532,9 @@ void launch_blend_forward(const BlendArgs& a, hipStream_t s)
 {
 	stage_mark(a.counters ? "blend_count" : "blend_forward", s);
 	if (a.counters)
-		hipLaunchKernelGGL(blend_forward_kernel<true>, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+		hipLaunchKernelGGL(blend_count_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
 	else
-		hipLaunchKernelGGL(blend_forward_kernel<false>, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+		hipLaunchKernelGGL(blend_forward_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
 }
 
 void launch_blend_backward(const BlendArgs& a, hipStream_t s)
