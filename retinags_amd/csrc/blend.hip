@@ -38,6 +38,20 @@ __device__ __forceinline__ bool clipped_by_box(const PixelRay& ray, float w, flo
 	return (wx <= lo.x) || (wx > hi.x) || (wy <= lo.y) || (wy > hi.y) || (wz <= lo.z) || (wz > hi.z);
 }
 
+// exp(x) for the exponents of the blend (x <= 0, modest magnitude): 2^(x log2 e) on the
+// hardware exp2 unit, with the rounding error of the product x * log2(e) folded back in, which
+// keeps the relative error at about one unit in the last place.  Forward and backward use
+// the same function, so they take the same per-pixel decisions.
+__device__ __forceinline__ float exp_of_exponent(float x)
+{
+	const float kLog2eHi = 1.44269502e+0f, kLog2eLo = 1.92596303e-8f;
+	const float t = x * kLog2eHi;
+	float r = __builtin_fmaf(x, kLog2eHi, -t);
+	r = __builtin_fmaf(x, kLog2eLo, r);
+	const float e = __builtin_amdgcn_exp2f(t);
+	return __builtin_fmaf(e, r * 0.693147182f, e);
+}
+
 // Lower bound on `power` below which alpha = min(0.99, opacity * exp(power)) is certainly
 // under 1/255.  A NaN opacity makes alpha 0.99 in the exact evaluation (fminf drops the NaN),
 // so it must never be culled; a non-positive one can never reach 1/255.
@@ -76,6 +90,43 @@ __device__ __forceinline__ uint32_t reachable_strips(float gx, float gy, const f
 			mask |= 1u << w;
 	}
 	return mask;
+}
+
+// Where the rays of a whole tile, sampled at clip-w `w`, fall relative to the submodel box.
+// The world-space sample is affine in the pixel's NDC coordinates, so its extremes over the
+// tile are attained at the tile's corner pixels.  With a tolerance far above the rounding error
+// of that affine map: kBoxInside = every pixel's exact test passes, kBoxOutside = every
+// pixel's exact test fails, kBoxMixed = decide per pixel.
+enum { kBoxMixed = 0, kBoxInside = 1, kBoxOutside = 2 };
+
+__device__ __forceinline__ int classify_tile_against_box(float w, float tile_x0, float tile_y0, const BlendArgs& a,
+                                                         const float3 lo, const float3 hi)
+{
+	const float* __restrict__ m = a.projinv;
+	float pmin[3] = {INFINITY, INFINITY, INFINITY}, pmax[3] = {-INFINITY, -INFINITY, -INFINITY};
+#pragma unroll
+	for (int c = 0; c < 4; c++) {
+		const float nx = pix_to_ndc(tile_x0 + ((c & 1) ? 15.f : 0.f), a.W);
+		const float ny = pix_to_ndc(tile_y0 + ((c & 2) ? 15.f : 0.f), a.H);
+		const float3 ph = {nx * (w + 0.0000001f) * a.tanfovx, ny * (w + 0.0000001f) * a.tanfovy, w};
+		const float q[3] = {m[0] * ph.x + m[4] * ph.y + m[8] * ph.z + m[12], m[1] * ph.x + m[5] * ph.y + m[9] * ph.z + m[13],
+		                    m[2] * ph.x + m[6] * ph.y + m[10] * ph.z + m[14]};
+#pragma unroll
+		for (int k = 0; k < 3; k++) {
+			pmin[k] = fminf(pmin[k], q[k]);
+			pmax[k] = fmaxf(pmax[k], q[k]);
+		}
+	}
+	const float lov[3] = {lo.x, lo.y, lo.z}, hiv[3] = {hi.x, hi.y, hi.z};
+	bool inside = true, outside = false;
+#pragma unroll
+	for (int k = 0; k < 3; k++) {
+		const float tol = 1e-4f * fmaxf(fmaxf(fabsf(pmin[k]), fabsf(pmax[k])), 1.f);
+		inside = inside && (pmin[k] > lov[k] + tol) && (pmax[k] < hiv[k] - tol);
+		outside = outside || (pmax[k] < lov[k] - tol) || (pmin[k] > hiv[k] + tol);
+	}
+	// NaN anywhere leaves both flags false except `outside`, which a NaN cannot set
+	return outside ? kBoxOutside : (inside ? kBoxInside : kBoxMixed);
 }
 
 constexpr int kPadSlot = 256;  // staged slot that never passes the floor test; pads lists to a multiple of 4
@@ -124,8 +175,10 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 	if (__ballot(candidate) == 0ull)
 		return;
 	if (candidate) {
-		const float alpha = fminf(0.99f, co.w * expf(power));
-		if (!(alpha < 1.0f / 255.0f) && !clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi)) {
+		const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
+		// a NaN clip-w marks an entry whose whole tile footprint lies inside the box
+		if (!(alpha < 1.0f / 255.0f) &&
+		    !((g.w == g.w) && clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))) {
 			const float test_T = p.T * (1 - alpha);
 			if (test_T < 0.0001f) {
 				p.done = true;
@@ -185,7 +238,15 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 			const float4 co = a.conic_opacity[id];
 			const float floor = exponent_floor(co.w);
 			strips = reachable_strips(xy.x, xy.y, co, floor, tile_x0, tile_y0);
-			s_geom[tid] = float4{xy.x, xy.y, floor, a.clip_w[id]};
+			float w = a.clip_w[id];
+			if (strips) {
+				const int where = classify_tile_against_box(w, tile_x0, tile_y0, a, lo, hi);
+				if (where == kBoxOutside)
+					strips = 0u;
+				if (where == kBoxInside)
+					w = __int_as_float(0x7FC00000);
+			}
+			s_geom[tid] = float4{xy.x, xy.y, floor, w};
 			s_conic[tid] = co;
 			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
 			                   a.depths[id]};
@@ -334,9 +395,10 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	bool valid = false;
 	if (candidate) {
 		const float2 d = {g.x - pixf.x, g.y - pixf.y};
-		const float G = expf(power);
+		const float G = exp_of_exponent(power);
 		const float alpha = fminf(0.99f, co.w * G);
-		if (!(alpha < 1.0f / 255.0f) && !clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi)) {
+		if (!(alpha < 1.0f / 255.0f) &&
+		    !((g.w == g.w) && clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))) {
 			valid = true;
 			p.T = p.T / (1.f - alpha);
 			const float aT = alpha * p.T;
@@ -470,8 +532,16 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			strips = reachable_strips(xy.x, xy.y, co, floor, tile_x0, tile_y0);
 			strips &= (entry < span0 ? 1u : 0u) | (entry < span1 ? 2u : 0u) | (entry < span2 ? 4u : 0u) |
 			          (entry < span3 ? 8u : 0u);
+			float w = a.clip_w[id];
+			if (strips) {
+				const int where = classify_tile_against_box(w, tile_x0, tile_y0, a, lo, hi);
+				if (where == kBoxOutside)
+					strips = 0u;
+				if (where == kBoxInside)
+					w = __int_as_float(0x7FC00000);
+			}
 			s_id[tid] = id;
-			s_geom[tid] = float4{xy.x, xy.y, floor, a.clip_w[id]};
+			s_geom[tid] = float4{xy.x, xy.y, floor, w};
 			s_conic[tid] = co;
 			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
 			                   a.depths[id]};
