@@ -268,32 +268,51 @@ __device__ __forceinline__ void sh_backward_channel(int deg, float x, float y, f
 	ddz += dRGBdz * g;
 }
 
-__global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBackwardArgs a)
+// One wavefront per block.  Every lane builds its Gaussian's 16 + 3M gradient floats in an
+// LDS row (stride 65 words: conflict-free for per-lane rows), then the wavefront writes
+// the five output arrays with fully coalesced stores; rows of Gaussians that were not
+// rendered stay zero.
+constexpr int kBwdRow = 65;
+constexpr int kBwdMeans = 0, kBwdCov = 3, kBwdScale = 9, kBwdRot = 12, kBwdSh = 16, kBwdShMax = 48;
+
+__device__ __forceinline__ void store_rows(float* __restrict__ dst, const float* s_out, int field, int width, int rows,
+                                           int lane)
 {
-	const int idx = blockIdx.x * 256 + threadIdx.x;
-	if (idx >= a.P)
-		return;
+	const int n = rows * width;
+	int r = 0, c = lane;
+	while (c >= width) {
+		c -= width;
+		r++;
+	}
+	for (int t = lane; t < n; t += 64) {
+		dst[t] = s_out[r * kBwdRow + field + c];
+		c += 64;
+		while (c >= width) {
+			c -= width;
+			r++;
+		}
+	}
+}
+
+__global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackwardArgs a)
+{
+	__shared__ float s_out[64 * kBwdRow];
+	const int lane = threadIdx.x;
+	const int first = blockIdx.x * 64;
+	const int idx = first + lane;
 	const size_t i = (size_t)idx;
 	const int n_sh = a.shs ? a.M * 3 : 0;
-
-	if (!(a.radii[idx] > 0)) {
-		a.dL_dmeans[3 * i + 0] = 0.f;
-		a.dL_dmeans[3 * i + 1] = 0.f;
-		a.dL_dmeans[3 * i + 2] = 0.f;
+	const bool sh_in_lds = n_sh <= kBwdShMax;
+	float* row = s_out + lane * kBwdRow;
 #pragma unroll
-		for (int k = 0; k < 6; k++)
-			a.dL_dcov3D[6 * i + k] = 0.f;
+	for (int k = 0; k < 64; k++)
+		row[k] = 0.f;
+	const bool visible = idx < a.P && a.radii[idx > a.P - 1 ? a.P - 1 : idx] > 0;
+	if (!sh_in_lds && idx < a.P && !visible)
 		for (int k = 0; k < n_sh; k++)
 			a.dL_dsh[i * n_sh + k] = 0.f;
-		if (a.scales) {
-			a.dL_dscale[3 * i + 0] = 0.f;
-			a.dL_dscale[3 * i + 1] = 0.f;
-			a.dL_dscale[3 * i + 2] = 0.f;
-			reinterpret_cast<float4*>(a.dL_drot)[i] = float4{0.f, 0.f, 0.f, 0.f};
-		}
-		return;
-	}
 
+	if (visible) {
 	const float* __restrict__ view = a.view;
 	const float* __restrict__ proj = a.proj;
 	const float3 mean = {a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
@@ -335,7 +354,7 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBack
 	}
 #pragma unroll
 	for (int k = 0; k < 6; k++)
-		a.dL_dcov3D[6 * i + k] = dcov[k];
+		row[kBwdCov + k] = dcov[k];
 
 	const float dL_dT00 = 2 * (TM(0, 0) * VM(0, 0) + TM(0, 1) * VM(0, 1) + TM(0, 2) * VM(0, 2)) * dL_da +
 	                      (TM(1, 0) * VM(0, 0) + TM(1, 1) * VM(0, 1) + TM(1, 2) * VM(0, 2)) * dL_db;
@@ -393,12 +412,14 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBack
 		const float x = d0.x / len, y = d0.y / len, z = d0.z / len;
 		const uint32_t cl = a.clamped[i];
 		const float* sh = a.shs + i * n_sh;
-		float* dsh = a.dL_dsh + i * n_sh;
 		float ddx = 0.f, ddy = 0.f, ddz = 0.f;
 #pragma unroll
 		for (int ch = 0; ch < 3; ch++) {
 			const float g = a.dL_dcolor[3 * i + ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-			sh_backward_channel(a.D, x, y, z, sh + ch, g, dsh + ch, ddx, ddy, ddz);
+			if (sh_in_lds)  // the usual case: rows go out through LDS, coalesced
+				sh_backward_channel(a.D, x, y, z, sh + ch, g, row + kBwdSh + ch, ddx, ddy, ddz);
+			else
+				sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
 		}
 		// normalisation Jacobian (auxiliary.h:123-133)
 		const float sum2 = d0.x * d0.x + d0.y * d0.y + d0.z * d0.z;
@@ -407,9 +428,9 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBack
 		dmean.y += (-d0.x * d0.y * ddx + (sum2 - d0.y * d0.y) * ddy - d0.z * d0.y * ddz) * invsum32;
 		dmean.z += (-d0.x * d0.z * ddx - d0.y * d0.z * ddy + (sum2 - d0.z * d0.z) * ddz) * invsum32;
 	}
-	a.dL_dmeans[3 * i + 0] = dmean.x;
-	a.dL_dmeans[3 * i + 1] = dmean.y;
-	a.dL_dmeans[3 * i + 2] = dmean.z;
+	row[kBwdMeans + 0] = dmean.x;
+	row[kBwdMeans + 1] = dmean.y;
+	row[kBwdMeans + 2] = dmean.z;
 
 	// -- 3D covariance -> scale and raw quaternion (backward.cu:278-341)
 	if (a.scales) {
@@ -438,9 +459,9 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBack
 #pragma unroll
 		for (int k = 0; k < 3; k++)
 			ds[k] = Rt.c[k][0] * dMt.c[k][0] + Rt.c[k][1] * dMt.c[k][1] + Rt.c[k][2] * dMt.c[k][2];
-		a.dL_dscale[3 * i + 0] = ds[0];
-		a.dL_dscale[3 * i + 1] = ds[1];
-		a.dL_dscale[3 * i + 2] = ds[2];
+		row[kBwdScale + 0] = ds[0];
+		row[kBwdScale + 1] = ds[1];
+		row[kBwdScale + 2] = ds[2];
 #pragma unroll
 		for (int k = 0; k < 3; k++)
 #pragma unroll
@@ -456,8 +477,23 @@ __global__ __launch_bounds__(256) void preprocess_backward_kernel(PreprocessBack
 		dq.w = 2 * r * (DM(0, 1) - DM(1, 0)) + 2 * x * (DM(2, 0) + DM(0, 2)) + 2 * y * (DM(1, 2) + DM(2, 1)) -
 		       4 * z * (DM(1, 1) + DM(0, 0));
 #undef DM
-		reinterpret_cast<float4*>(a.dL_drot)[i] = dq;
+		row[kBwdRot + 0] = dq.x;
+		row[kBwdRot + 1] = dq.y;
+		row[kBwdRot + 2] = dq.z;
+		row[kBwdRot + 3] = dq.w;
 	}
+	}  // visible
+
+	__syncthreads();
+	const int rows = a.P - first < 64 ? a.P - first : 64;
+	store_rows(a.dL_dmeans + 3 * (size_t)first, s_out, kBwdMeans, 3, rows, lane);
+	store_rows(a.dL_dcov3D + 6 * (size_t)first, s_out, kBwdCov, 6, rows, lane);
+	if (a.scales) {
+		store_rows(a.dL_dscale + 3 * (size_t)first, s_out, kBwdScale, 3, rows, lane);
+		store_rows(a.dL_drot + 4 * (size_t)first, s_out, kBwdRot, 4, rows, lane);
+	}
+	if (n_sh > 0 && sh_in_lds)
+		store_rows(a.dL_dsh + (size_t)n_sh * first, s_out, kBwdSh, n_sh, rows, lane);
 }
 
 // ---- launchers -----------------------------------------------------------------------------
@@ -477,7 +513,7 @@ void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s)
 void launch_preprocess_backward(const PreprocessBackwardArgs& a, hipStream_t s)
 {
 	stage_mark("preprocess_backward", s);
-	hipLaunchKernelGGL(preprocess_backward_kernel, dim3((a.P + 255) / 256), dim3(256), 0, s, a);
+	hipLaunchKernelGGL(preprocess_backward_kernel, dim3((a.P + 63) / 64), dim3(64), 0, s, a);
 }
 
 }  // namespace rgs
