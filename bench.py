@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--resolution-scale", type=float, default=1.0, help="scale the image size (debugging only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-threads", type=int, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 1 GiB device-to-device copy, the known-size reference for HBM traffic counters")
     return ap.parse_args()
 
 
@@ -109,6 +111,14 @@ def main():
     elapsed = time.perf_counter() - t1
     ms_per_step = elapsed * 1e3 / args.steps
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- per-stage time: HIP events recorded by the library on the stream it launches on
     prof_steps = max(1, min(args.steps, 5))
     _capi.stage_timing(True)
@@ -156,8 +166,8 @@ def main():
         "preprocess_forward": 20.0 * P_tot + 299.0 * P_vis,
         "offset_scan": 8.0 * P_tot,
         "duplicate_with_keys": 4.0 * P_tot + 16.0 * P_vis + 12.0 * R_tot,
-        "sort_histogram": 8.0 * R_tot * passes,
-        "sort_scatter": 24.0 * R_tot * passes,
+        "sort_setup": 8.0 * R_tot,
+        "sort_onesweep": 24.0 * R_tot * passes,
         "tile_ranges": 8.0 * R_tot + 16.0 * T * K,
         "preprocess_backward": 4.0 * P_tot + 559.0 * P_vis,
         "composite_forward": (20.0 * K + 20.0) * N,

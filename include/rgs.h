@@ -57,6 +57,9 @@ enum {
 	RGS_GEOM_CLAMPED,           /* uint8[P]   bit c set: colour channel c was clamped at 0 */
 	RGS_GEOM_BLOCK_SUMS,        /* uint32[ceil(P/256)+1] */
 	RGS_GEOM_TOTAL,             /* uint32     number of (Gaussian, tile) instances */
+	RGS_GEOM_BLEND_RECORD,      /* float[16P] one 64-byte record per Gaussian with everything the blend reads:
+	                               x, y, exponent floor, clip w | conic xx, xy, yy, opacity | r, g, b, depth |
+	                               half-width, half-height of the alpha >= 1/255 ellipse's bounding box, 0, 0 */
 	RGS_GEOM_FIELDS
 };
 enum {

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RGS_LIBRARY") or os.path.join(_HERE, "librgs_gfx950.so")
 
 GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles_touched", "point_offsets",
-               "clamped", "block_sums", "total")
+               "clamped", "block_sums", "total", "blend_record")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
 IMG_FIELDS = ("ranges", "n_contrib")
 ACC_MEAN2D, ACC_CONIC, ACC_OPACITY, ACC_COLOR, ACC_DEPTH, ACC_FLOATS = 0, 3, 7, 8, 11, 12

@@ -113,6 +113,7 @@ size_t geom_layout(size_t P, size_t* off)
 	off[RGS_GEOM_CLAMPED] = c.take(P);
 	off[RGS_GEOM_BLOCK_SUMS] = c.take(4 * ((P + 255) / 256 + 1));
 	off[RGS_GEOM_TOTAL] = c.take(4);
+	off[RGS_GEOM_BLEND_RECORD] = c.take(64 * P);
 	return c.cursor;
 }
 
@@ -347,6 +348,7 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
 	a.tiles_touched = at<uint32_t>(geom_ws, off[RGS_GEOM_TILES_TOUCHED]);
 	a.clamped = at<uint8_t>(geom_ws, off[RGS_GEOM_CLAMPED]);
 	a.block_sums = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_SUMS]);
+	a.blend_record = at<float4>(geom_ws, off[RGS_GEOM_BLEND_RECORD]);
 
 	rgs::launch_preprocess_forward(a, s);
 	RGS_STAGE("preprocess");
@@ -433,6 +435,7 @@ int rgs_forward_raster(int P, int R, int width, int height,
 	a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
 	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
 	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
+	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 	a.out_color = out_color; a.out_depth = out_depth; a.out_alpha = out_alpha;
 	a.n_contrib = at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]);
 	rgs::launch_blend_forward(a, s);
@@ -490,6 +493,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 		a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
 		a.colors = colors;
 		a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
+		a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 		a.out_alpha = const_cast<float*>(alphas);
 		a.n_contrib = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]));
 		a.dL_dpix = dL_dpix; a.dL_dpix_depth = dL_dpix_depth; a.dL_dalpha = dL_dalphas;
@@ -557,6 +561,7 @@ int rgs_blend_work_counters(int P, int R, int width, int height, float tan_fovx,
 	a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
 	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
 	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
+	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 	a.counters = counters;
 	rgs::launch_blend_forward(a, s);
 	RGS_STAGE("blend_count");

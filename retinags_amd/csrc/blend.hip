@@ -52,34 +52,14 @@ __device__ __forceinline__ float exp_of_exponent(float x)
 	return __builtin_fmaf(e, r * 0.693147182f, e);
 }
 
-// Lower bound on `power` below which alpha = min(0.99, opacity * exp(power)) is certainly
-// under 1/255.  A NaN opacity makes alpha 0.99 in the exact evaluation (fminf drops the NaN),
-// so it must never be culled; a non-positive one can never reach 1/255.
-__device__ __forceinline__ float exponent_floor(float opacity)
-{
-	if (opacity != opacity)
-		return -INFINITY;
-	if (!(opacity > 0.f))
-		return INFINITY;
-	return -logf(255.0f * opacity) - 1e-3f;
-}
-
 // Bit w set: some pixel of strip w (rows 4w..4w+3 of the tile whose first pixel is
-// (x0, y0)) may reach power >= floor.  The region power >= floor is the ellipse
-// d^T Q d <= -2 floor with Q the conic; its bounding box has half-widths
-// sqrt(-2 floor * Q^-1_xx) and sqrt(-2 floor * Q^-1_yy), inflated here against rounding.
-// Every comparison is written so that NaN or a non-positive-definite conic keeps the entry.
-__device__ __forceinline__ uint32_t reachable_strips(float gx, float gy, const float4 conic, float floor, float x0,
+// (x0, y0)) may reach power >= floor, judged by the bounding box (half-widths hx, hy) of the
+// ellipse power >= floor.  Every comparison is written so that NaN keeps the entry.
+__device__ __forceinline__ uint32_t reachable_strips(float gx, float gy, float hx, float hy, float floor, float x0,
                                                      float y0)
 {
 	if (floor > 0.f)
 		return 0u;  // even power = 0 gives alpha < 1/255
-	const float det = conic.x * conic.z - conic.y * conic.y;
-	if (!(det > 0.f))
-		return 0xFu;
-	const float c = -2.f * floor;
-	const float hx = sqrtf(c * conic.z / det) * 1.0001f + 1e-2f;
-	const float hy = sqrtf(c * conic.x / det) * 1.0001f + 1e-2f;
 	if ((gx + hx < x0) || (gx - hx > x0 + 15.f))
 		return 0u;
 	uint32_t mask = 0u;
@@ -234,11 +214,10 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 		uint32_t strips = 0u;
 		if (src < range.y) {
 			const uint32_t id = a.point_list[src];
-			const float2 xy = a.xy[id];
-			const float4 co = a.conic_opacity[id];
-			const float floor = exponent_floor(co.w);
-			strips = reachable_strips(xy.x, xy.y, co, floor, tile_x0, tile_y0);
-			float w = a.clip_w[id];
+			const float4* rec = a.record + 4 * (size_t)id;
+			const float4 geom = rec[0], co = rec[1], cd = rec[2], half = rec[3];
+			strips = reachable_strips(geom.x, geom.y, half.x, half.y, geom.z, tile_x0, tile_y0);
+			float w = geom.w;
 			if (strips) {
 				const int where = classify_tile_against_box(w, tile_x0, tile_y0, a, lo, hi);
 				if (where == kBoxOutside)
@@ -246,10 +225,9 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				if (where == kBoxInside)
 					w = __int_as_float(0x7FC00000);
 			}
-			s_geom[tid] = float4{xy.x, xy.y, floor, w};
+			s_geom[tid] = float4{geom.x, geom.y, geom.z, w};
 			s_conic[tid] = co;
-			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
-			                   a.depths[id]};
+			s_cd[tid] = cd;
 		}
 		file_in_strip_lists(strips, tid, s_list, s_count);
 		__syncthreads();
@@ -526,13 +504,12 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 		if (progress < span) {
 			const uint32_t entry = span - 1 - progress;  // 0-based position in the tile list
 			const uint32_t id = a.point_list[back - progress - 1];
-			const float2 xy = a.xy[id];
-			const float4 co = a.conic_opacity[id];
-			const float floor = exponent_floor(co.w);
-			strips = reachable_strips(xy.x, xy.y, co, floor, tile_x0, tile_y0);
+			const float4* rec = a.record + 4 * (size_t)id;
+			const float4 geom = rec[0], co = rec[1], cd = rec[2], half = rec[3];
+			strips = reachable_strips(geom.x, geom.y, half.x, half.y, geom.z, tile_x0, tile_y0);
 			strips &= (entry < span0 ? 1u : 0u) | (entry < span1 ? 2u : 0u) | (entry < span2 ? 4u : 0u) |
 			          (entry < span3 ? 8u : 0u);
-			float w = a.clip_w[id];
+			float w = geom.w;
 			if (strips) {
 				const int where = classify_tile_against_box(w, tile_x0, tile_y0, a, lo, hi);
 				if (where == kBoxOutside)
@@ -541,10 +518,9 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 					w = __int_as_float(0x7FC00000);
 			}
 			s_id[tid] = id;
-			s_geom[tid] = float4{xy.x, xy.y, floor, w};
+			s_geom[tid] = float4{geom.x, geom.y, geom.z, w};
 			s_conic[tid] = co;
-			s_cd[tid] = float4{a.colors[3 * (size_t)id], a.colors[3 * (size_t)id + 1], a.colors[3 * (size_t)id + 2],
-			                   a.depths[id]};
+			s_cd[tid] = cd;
 		}
 		file_in_strip_lists(strips, tid, s_list, s_count);
 		__syncthreads();

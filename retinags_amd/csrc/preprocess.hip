@@ -192,6 +192,23 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs 
 			a.xy[idx] = pix;
 			a.clip_w[idx] = p_hom.w;
 			a.conic_opacity[idx] = conic_o;
+			{
+				// Packed copy for the blend kernels, which gather per-Gaussian data in depth order:
+				// one 64-byte record instead of one cache line from each of five arrays.
+				float3 col;
+				if (a.colors_precomp)
+					col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
+					             a.colors_precomp[3 * (size_t)idx + 2]};
+				else
+					col = float3{a.rgb[3 * (size_t)idx], a.rgb[3 * (size_t)idx + 1], a.rgb[3 * (size_t)idx + 2]};
+				const float floor = exponent_floor(conic_o.w);
+				const float2 half = alpha_ellipse_half_extent(conic_o, floor);
+				float4* rec = a.blend_record + 4 * (size_t)idx;
+				rec[0] = float4{pix.x, pix.y, floor, p_hom.w};
+				rec[1] = conic_o;
+				rec[2] = float4{col.x, col.y, col.z, p_view.z};
+				rec[3] = float4{half.x, half.y, 0.f, 0.f};
+			}
 			radius_out = (int)my_radius;
 			touched = ntiles;
 		} while (false);

@@ -97,6 +97,34 @@ __device__ __forceinline__ TileRect tile_rect(float px, float py, int radius, in
 	return r;
 }
 
+// ---- conservative bounds used to skip blend work without changing any result ---------------
+
+// Lower bound on the exponent `power` below which alpha = min(0.99, opacity * exp(power)) is
+// certainly under 1/255: alpha >= 1/255 needs power >= -ln(255 * opacity).  A NaN opacity
+// makes alpha 0.99 in the exact evaluation (fminf drops the NaN), so it is never culled; a
+// non-positive one can never reach 1/255.
+__device__ __forceinline__ float exponent_floor(float opacity)
+{
+	if (opacity != opacity)
+		return -INFINITY;
+	if (!(opacity > 0.f))
+		return INFINITY;
+	return -logf(255.0f * opacity) - 1e-3f;
+}
+
+// power >= floor is the ellipse d^T Q d <= -2 floor around the Gaussian's centre (Q = conic).
+// Half-widths of its bounding box, sqrt(-2 floor * Q^-1_xx) and sqrt(-2 floor * Q^-1_yy),
+// inflated against rounding.  Infinite when the conic is not positive definite or the floor is
+// -inf, so that nothing is culled; unused when floor > 0 (then no pixel can reach 1/255).
+__device__ __forceinline__ float2 alpha_ellipse_half_extent(const float4 conic, float floor)
+{
+	const float det = conic.x * conic.z - conic.y * conic.y;
+	if (!(det > 0.f) || !(floor <= 0.f))
+		return float2{INFINITY, INFINITY};
+	const float c = -2.f * floor;
+	return float2{sqrtf(c * conic.z / det) * 1.0001f + 1e-2f, sqrtf(c * conic.x / det) * 1.0001f + 1e-2f};
+}
+
 // ---- wave64 cross-lane primitives (DPP) -----------------------------------------------
 
 template <int Ctrl, int RowMask, int BankMask>

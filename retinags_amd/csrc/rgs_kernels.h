@@ -34,6 +34,7 @@ struct PreprocessArgs {
 	uint32_t* tiles_touched;
 	uint8_t* clamped;
 	uint32_t* block_sums;  // one per 256 Gaussians
+	float4* blend_record;  // 4 float4 per Gaussian, see blend.hip
 };
 
 struct PreprocessBackwardArgs {
@@ -76,6 +77,7 @@ struct BlendArgs {
 	const float4* conic_opacity;
 	const float* colors;  // (P,3)
 	const float* depths;
+	const float4* record;  // 4 float4 per Gaussian: the packed copy of the arrays above that the blend gathers
 	// forward outputs / backward inputs
 	float* out_color;
 	float* out_depth;
