@@ -8,16 +8,24 @@
 // (K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian), so a pixel
 // can only differ from that evaluation through the last-bit behaviour of exp().
 //
-// Most (pixel, Gaussian) visits of the reference loop end at "alpha < 1/255".  Two
-// conservative filters remove such visits without changing any result:
-//  * alpha >= 1/255 needs power >= -ln(255 * opacity).  The staging thread stores that floor
-//    (minus a margin) with the Gaussian, and a wavefront skips an entry with one ballot when
-//    no live lane reaches it, before exp() is evaluated.
-//  * power >= floor describes an ellipse around the Gaussian's centre.  The staging thread
-//    intersects the ellipse's bounding box with the four 16x4 strips of the tile and files the
-//    entry only in the lists of the strips it can reach; each wavefront walks its own list,
-//    four entries at a time so that the LDS reads and the four exponent evaluations overlap.
-// Both filters only drop visits that the exact evaluation would have skipped too.
+// The four wavefronts of a block never synchronise with each other: measured per wave, more
+// than half of a heavy tile's time used to go into waiting for the slowest strip at the
+// end-of-batch barrier.  Each wavefront instead streams the tile's list by itself in chunks
+// of 64 entries (lane l takes entry l of the chunk; the next chunk's records and the ids of
+// the one after are already in flight while the current chunk is processed), keeps the
+// entries that can matter to its strip in a wave-private LDS list, and walks that list.
+//
+// Most (pixel, Gaussian) visits of the reference loop end at "alpha < 1/255" or at the box
+// test.  Three conservative filters remove such visits without changing any result:
+//  * alpha >= 1/255 needs power >= -ln(255 * opacity); that floor (minus a margin) is stored
+//    with the Gaussian, and a group of entries is skipped with one ballot when no live lane
+//    reaches it, before exp() is evaluated.
+//  * power >= floor is an ellipse around the Gaussian's centre; an entry whose ellipse's
+//    bounding box misses the strip is not filed at all.
+//  * the world-space ray sample is affine in the pixel, so its extremes over the strip are at
+//    the strip's corner pixels: an entry whose corners are all outside the submodel box is not
+//    filed, one whose corners are all inside skips the per-pixel box test.
+// All three only drop work that the exact evaluation would have skipped too.
 #include "rgs_kernels.h"
 
 namespace rgs {
@@ -52,42 +60,34 @@ __device__ __forceinline__ float exp_of_exponent(float x)
 	return __builtin_fmaf(e, r * 0.693147182f, e);
 }
 
-// Bit w set: some pixel of strip w (rows 4w..4w+3 of the tile whose first pixel is
-// (x0, y0)) may reach power >= floor, judged by the bounding box (half-widths hx, hy) of the
-// ellipse power >= floor.  Every comparison is written so that NaN keeps the entry.
-__device__ __forceinline__ uint32_t reachable_strips(float gx, float gy, float hx, float hy, float floor, float x0,
-                                                     float y0)
+// True if some pixel of the strip whose first pixel is (x0, ya) (16 wide, 4 high) may reach
+// power >= floor, judged by the bounding box (half-widths hx, hy) of that ellipse.  Written so
+// that NaN keeps the entry.
+__device__ __forceinline__ bool reaches_strip(float gx, float gy, float hx, float hy, float floor, float x0, float ya)
 {
 	if (floor > 0.f)
-		return 0u;  // even power = 0 gives alpha < 1/255
-	if ((gx + hx < x0) || (gx - hx > x0 + 15.f))
-		return 0u;
-	uint32_t mask = 0u;
-#pragma unroll
-	for (int w = 0; w < 4; w++) {
-		const float ya = y0 + 4.f * w;
-		if (!((gy + hy < ya) || (gy - hy > ya + 3.f)))
-			mask |= 1u << w;
-	}
-	return mask;
+		return false;  // even power = 0 gives alpha < 1/255
+	return !((gx + hx < x0) || (gx - hx > x0 + 15.f) || (gy + hy < ya) || (gy - hy > ya + 3.f));
 }
 
-// Where the rays of a whole tile, sampled at clip-w `w`, fall relative to the submodel box.
-// The world-space sample is affine in the pixel's NDC coordinates, so its extremes over the
-// tile are attained at the tile's corner pixels.  With a tolerance far above the rounding error
-// of that affine map: kBoxInside = every pixel's exact test passes, kBoxOutside = every
-// pixel's exact test fails, kBoxMixed = decide per pixel.
+// Where the rays of a whole strip, sampled at clip-w `w`, fall relative to the submodel box.
+// With a tolerance far above the rounding error of the affine map: kBoxInside = every pixel's
+// exact test passes, kBoxOutside = every pixel's exact test fails, kBoxMixed = decide per pixel.
 enum { kBoxMixed = 0, kBoxInside = 1, kBoxOutside = 2 };
 
-__device__ __forceinline__ int classify_tile_against_box(float w, float tile_x0, float tile_y0, const BlendArgs& a,
-                                                         const float3 lo, const float3 hi)
+struct StripCorners {
+	float nx0, nx1, ny0, ny1;  // NDC of the strip's first/last pixel column and row
+};
+
+__device__ __forceinline__ int classify_strip_against_box(float w, const StripCorners& sc, const BlendArgs& a,
+                                                          const float3 lo, const float3 hi)
 {
 	const float* __restrict__ m = a.projinv;
 	float pmin[3] = {INFINITY, INFINITY, INFINITY}, pmax[3] = {-INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
 	for (int c = 0; c < 4; c++) {
-		const float nx = pix_to_ndc(tile_x0 + ((c & 1) ? 15.f : 0.f), a.W);
-		const float ny = pix_to_ndc(tile_y0 + ((c & 2) ? 15.f : 0.f), a.H);
+		const float nx = (c & 1) ? sc.nx1 : sc.nx0;
+		const float ny = (c & 2) ? sc.ny1 : sc.ny0;
 		const float3 ph = {nx * (w + 0.0000001f) * a.tanfovx, ny * (w + 0.0000001f) * a.tanfovy, w};
 		const float q[3] = {m[0] * ph.x + m[4] * ph.y + m[8] * ph.z + m[12], m[1] * ph.x + m[5] * ph.y + m[9] * ph.z + m[13],
 		                    m[2] * ph.x + m[6] * ph.y + m[10] * ph.z + m[14]};
@@ -105,32 +105,50 @@ __device__ __forceinline__ int classify_tile_against_box(float w, float tile_x0,
 		inside = inside && (pmin[k] > lov[k] + tol) && (pmax[k] < hiv[k] - tol);
 		outside = outside || (pmax[k] < lov[k] - tol) || (pmin[k] > hiv[k] + tol);
 	}
-	// NaN anywhere leaves both flags false except `outside`, which a NaN cannot set
+	// a NaN can set neither flag, which leaves the decision to the per-pixel test
 	return outside ? kBoxOutside : (inside ? kBoxInside : kBoxMixed);
 }
 
-constexpr int kPadSlot = 256;  // staged slot that never passes the floor test; pads lists to a multiple of 4
+constexpr int kChunk = 64;  // list entries a wavefront takes per step, one per lane
 
-// Files the staging thread's entry (slot `tid`, reachable strips `strips`) in the per-strip
-// lists.  Each staging wavefront owns a 64-entry segment of every strip's list and fills it in
-// slot order, so walking segments 0..3 visits a strip's entries in list order.
-__device__ __forceinline__ void file_in_strip_lists(uint32_t strips, int tid, uint16_t (*s_list)[256],
-                                                    uint32_t (*s_count)[4])
+// One entry of the tile list as a lane holds it between the load and the filter.
+struct LoadedEntry {
+	float4 geom, conic, cd, half;
+	uint32_t id;
+};
+
+__device__ __forceinline__ LoadedEntry load_entry(const BlendArgs& a, uint32_t id, bool in_range)
 {
-	const int lane = tid & 63, wave = tid >> 6;
-	const uint64_t below = (1ull << lane) - 1ull;
-#pragma unroll
-	for (int w = 0; w < 4; w++) {
-		const bool mine = (strips >> w) & 1u;
-		const uint64_t m = __ballot(mine);
-		const uint32_t n = (uint32_t)__popcll(m);
-		if (mine)
-			s_list[w][wave * 64 + __popcll(m & below)] = (uint16_t)tid;
-		if ((uint32_t)lane < ((4u - (n & 3u)) & 3u))
-			s_list[w][wave * 64 + n + lane] = (uint16_t)kPadSlot;
-		if (lane == 0)
-			s_count[wave][w] = n;
+	LoadedEntry e;
+	e.id = id;
+	if (in_range) {
+		const float4* rec = a.record + 4 * (size_t)id;
+		e.geom = rec[0];
+		e.conic = rec[1];
+		e.cd = rec[2];
+		e.half = rec[3];
+	} else {
+		e.geom = float4{0.f, 0.f, INFINITY, 0.f};  // floor = +inf: never filed
+		e.conic = float4{0.f, 0.f, 0.f, 0.f};
+		e.cd = float4{0.f, 0.f, 0.f, 0.f};
+		e.half = float4{0.f, 0.f, 0.f, 0.f};
 	}
+	return e;
+}
+
+// Decides whether the lane's entry is filed for this strip; a filed entry whose strip lies
+// entirely inside the box gets a NaN clip-w, which tells the walk to skip the per-pixel test.
+__device__ __forceinline__ bool file_entry(LoadedEntry& e, float x0, float ya, const StripCorners& sc, const BlendArgs& a,
+                                           const float3 lo, const float3 hi)
+{
+	if (!reaches_strip(e.geom.x, e.geom.y, e.half.x, e.half.y, e.geom.z, x0, ya))
+		return false;
+	const int where = classify_strip_against_box(e.geom.w, sc, a, lo, hi);
+	if (where == kBoxOutside)
+		return false;
+	if (where == kBoxInside)
+		e.geom.w = __int_as_float(0x7FC00000);
+	return true;
 }
 
 __device__ __forceinline__ float exponent_of(const float4 g, const float4 co, const float2 pixf, float2& d)
@@ -147,30 +165,36 @@ struct ForwardPixel {
 	uint32_t last_contributor;
 };
 
+struct ForwardStage {  // wave-private
+	float4 geom[kChunk + 4];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
+	float4 conic[kChunk + 4];  // conic xx, xy, yy, opacity
+	float4 cd[kChunk];         // r, g, b, view depth
+	uint32_t position[kChunk]; // 1-based position in the tile list
+};
+
 __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, float power, const float4 g,
-                                              const float4 co, const float4* s_cd, int slot, uint32_t position,
-                                              const PixelRay& ray, const BlendArgs& a, const float3 lo, const float3 hi)
+                                              const float4 co, const ForwardStage& st, int slot, const PixelRay& ray,
+                                              const BlendArgs& a, const float3 lo, const float3 hi)
 {
 	candidate = candidate && !p.done;
 	if (__ballot(candidate) == 0ull)
 		return;
 	if (candidate) {
 		const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
-		// a NaN clip-w marks an entry whose whole tile footprint lies inside the box
 		if (!(alpha < 1.0f / 255.0f) &&
 		    !((g.w == g.w) && clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))) {
 			const float test_T = p.T * (1 - alpha);
 			if (test_T < 0.0001f) {
 				p.done = true;
 			} else {
-				const float4 cd = s_cd[slot];
+				const float4 cd = st.cd[slot];
 				p.C0 += cd.x * alpha * p.T;
 				p.C1 += cd.y * alpha * p.T;
 				p.C2 += cd.z * alpha * p.T;
 				p.weight += alpha * p.T;
 				p.D += cd.w * alpha * p.T;
 				p.T = test_T;
-				p.last_contributor = position;
+				p.last_contributor = st.position[slot];
 			}
 		}
 	}
@@ -178,15 +202,12 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 
 __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 {
-	__shared__ float4 s_geom[257];   // pixel x, pixel y, exponent floor, clip w
-	__shared__ float4 s_conic[257];  // conic xx, xy, yy, opacity
-	__shared__ float4 s_cd[256];     // r, g, b, view depth
-	__shared__ __attribute__((aligned(8))) uint16_t s_list[4][256];
-	__shared__ uint32_t s_count[4][4];  // [staging wave][strip]
-	__shared__ int s_alive[2][4];
+	__shared__ ForwardStage s_stage[4];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int tile = blockIdx.x;
+	const uint2 range = a.ranges[tile];
+	const uint32_t n = range.y - range.x;
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
 	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
@@ -195,52 +216,45 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
 	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
 	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
-	const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
-
-	const uint2 range = a.ranges[tile];
-	const int rounds = (int)((range.y - range.x + 255) / 256);
+	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
+	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
+	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
+	ForwardStage& st = s_stage[wave];
+	const uint64_t below = (1ull << lane) - 1ull;
 
 	ForwardPixel p = {!inside, 1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u};
-	if (tid == 0) {
-		s_geom[kPadSlot] = float4{0.f, 0.f, INFINITY, 0.f};
-		s_conic[kPadSlot] = float4{0.f, 0.f, 0.f, 0.f};
-	}
+	uint64_t live = __ballot(!p.done);
 
-	for (int i = 0; i < rounds; i++) {
-		uint64_t live = __ballot(!p.done);
-		if (lane == 0)
-			s_alive[i & 1][wave] = live != 0ull;
-		const uint32_t src = range.x + (uint32_t)i * 256 + tid;
-		uint32_t strips = 0u;
-		if (src < range.y) {
-			const uint32_t id = a.point_list[src];
-			const float4* rec = a.record + 4 * (size_t)id;
-			const float4 geom = rec[0], co = rec[1], cd = rec[2], half = rec[3];
-			strips = reachable_strips(geom.x, geom.y, half.x, half.y, geom.z, tile_x0, tile_y0);
-			float w = geom.w;
-			if (strips) {
-				const int where = classify_tile_against_box(w, tile_x0, tile_y0, a, lo, hi);
-				if (where == kBoxOutside)
-					strips = 0u;
-				if (where == kBoxInside)
-					w = __int_as_float(0x7FC00000);
+	if (n != 0u && live != 0ull) {
+		const uint32_t* list = a.point_list + range.x;
+		// two chunks of ids and one chunk of records are always in flight ahead of the walk
+		LoadedEntry cur = load_entry(a, (uint32_t)lane < n ? list[lane] : 0u, (uint32_t)lane < n);
+		uint32_t id_next = (uint32_t)(kChunk + lane) < n ? list[kChunk + lane] : 0u;
+
+		for (uint32_t first = 0; first < n && live != 0ull; first += kChunk) {
+			const uint32_t e1 = first + kChunk + lane, e2 = first + 2 * kChunk + lane;
+			LoadedEntry nxt = load_entry(a, id_next, e1 < n);
+			id_next = e2 < n ? list[e2] : 0u;
+
+			const bool filed = file_entry(cur, strip_x0, strip_y0, sc, a, lo, hi);
+			const uint64_t m = __ballot(filed);
+			const int count = __popcll(m);
+			if (filed) {
+				const int slot = __popcll(m & below);
+				st.geom[slot] = cur.geom;
+				st.conic[slot] = cur.conic;
+				st.cd[slot] = cur.cd;
+				st.position[slot] = first + lane + 1;
 			}
-			s_geom[tid] = float4{geom.x, geom.y, geom.z, w};
-			s_conic[tid] = co;
-			s_cd[tid] = cd;
-		}
-		file_in_strip_lists(strips, tid, s_list, s_count);
-		__syncthreads();
-		if (!(s_alive[i & 1][0] | s_alive[i & 1][1] | s_alive[i & 1][2] | s_alive[i & 1][3]))
-			break;
+			if (lane < 4) {  // pad to a multiple of four with entries that never pass the floor test
+				st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
+				st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
+			}
+			__builtin_amdgcn_wave_barrier();
 
-		for (int seg = 0; seg < 4 && live != 0ull; seg++) {
-			const int n = (int)s_count[seg][wave];
-			for (int k = 0; k < n && live != 0ull; k += 4) {
-				const uint2 packed = *reinterpret_cast<const uint2*>(&s_list[wave][seg * 64 + k]);
-				const int j0 = packed.x & 0xFFFFu, j1 = packed.x >> 16, j2 = packed.y & 0xFFFFu, j3 = packed.y >> 16;
-				const float4 g0 = s_geom[j0], g1 = s_geom[j1], g2 = s_geom[j2], g3 = s_geom[j3];
-				const float4 c0 = s_conic[j0], c1 = s_conic[j1], c2 = s_conic[j2], c3 = s_conic[j3];
+			for (int k = 0; k < count && live != 0ull; k += 4) {
+				const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
+				const float4 c0 = st.conic[k], c1 = st.conic[k + 1], c2 = st.conic[k + 2], c3 = st.conic[k + 3];
 				float2 d;
 				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
 				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
@@ -249,15 +263,15 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
 				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
 					continue;
-				const uint32_t base = (uint32_t)i * 256 + 1;
-				forward_visit(p, q0, w0, g0, c0, s_cd, j0, base + j0, ray, a, lo, hi);
-				forward_visit(p, q1, w1, g1, c1, s_cd, j1, base + j1, ray, a, lo, hi);
-				forward_visit(p, q2, w2, g2, c2, s_cd, j2, base + j2, ray, a, lo, hi);
-				forward_visit(p, q3, w3, g3, c3, s_cd, j3, base + j3, ray, a, lo, hi);
+				forward_visit(p, q0, w0, g0, c0, st, k, ray, a, lo, hi);
+				forward_visit(p, q1, w1, g1, c1, st, k + 1, ray, a, lo, hi);
+				forward_visit(p, q2, w2, g2, c2, st, k + 2, ray, a, lo, hi);
+				forward_visit(p, q3, w3, g3, c3, st, k + 3, ray, a, lo, hi);
 				live = __ballot(!p.done);
 			}
+			__builtin_amdgcn_wave_barrier();
+			cur = nxt;
 		}
-		__syncthreads();
 	}
 
 	if (inside) {
@@ -344,10 +358,11 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 }
 
 // ---- backward (K/cuda_rasterizer_hgs/backward.cu:415-622) ---------------------------------------
-// The tile list is walked back to front.  Each lane forms its pixel's ten partial
-// derivatives for the staged Gaussian; they are summed over the wavefront with DPP,
-// lane 63 adds the wave total to a per-batch LDS accumulator, and after the batch every
-// thread flushes one Gaussian's ten sums with one global atomic each.
+// Each wavefront walks the tile list back to front, starting at the largest last_contributor
+// of its own 64 pixels.  A lane forms its pixel's ten partial derivatives for an entry; they
+// are summed over the wavefront with DPP and lane 63 parks the sums in a wave-private LDS row
+// for that entry.  After the chunk, every lane flushes one entry's ten sums with one global
+// atomic each (one per (strip, Gaussian) and quantity).
 
 constexpr int kGradSlots = 10;  // mean2D x,y | conic xx,xy,yy | opacity | colour r,g,b | depth
 
@@ -359,13 +374,23 @@ struct BackwardPixel {
 	float bg_dot_dpixel, ddelx_dx, ddely_dy;
 };
 
-__device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
-                                               const float4 co, const float2 pixf, const float4* s_cd,
-                                               float (*s_acc)[256], int slot, const PixelRay& ray, const BlendArgs& a,
-                                               const float3 lo, const float3 hi, int lane)
+struct BackwardStage {  // wave-private
+	float4 geom[kChunk + 4];
+	float4 conic[kChunk + 4];
+	float4 cd[kChunk];
+	uint32_t entry[kChunk + 4];  // 0-based position in the tile list
+	uint32_t id[kChunk];
+	float sums[kGradSlots][kChunk];
+};
+
+// Returns true (wave-uniform) when the entry received sums.
+__device__ __forceinline__ bool backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
+                                               const float4 co, const float2 pixf, BackwardStage& st, int slot,
+                                               const PixelRay& ray, const BlendArgs& a, const float3 lo, const float3 hi,
+                                               int lane)
 {
 	if (__ballot(candidate) == 0ull)
-		return;
+		return false;
 	float v[kGradSlots];
 #pragma unroll
 	for (int q = 0; q < kGradSlots; q++)
@@ -380,7 +405,7 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 			valid = true;
 			p.T = p.T / (1.f - alpha);
 			const float aT = alpha * p.T;
-			const float4 cd = s_cd[slot];
+			const float4 cd = st.cd[slot];
 			float dL_dopa = 0.0f;
 			p.accum_r = p.last_alpha * p.last_r + (1.f - p.last_alpha) * p.accum_r;
 			p.last_r = cd.x;
@@ -418,30 +443,25 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 		}
 	}
 	if (__ballot(valid) == 0ull)
-		return;
+		return false;
 #pragma unroll
 	for (int q = 0; q < kGradSlots; q++)
 		v[q] = wave_sum_to_lane63(v[q]);
 	if (lane == 63) {
 #pragma unroll
 		for (int q = 0; q < kGradSlots; q++)
-			atomicAdd(&s_acc[q][slot], v[q]);
+			st.sums[q][slot] = v[q];
 	}
+	return true;
 }
 
 __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 {
-	__shared__ float4 s_geom[257];
-	__shared__ float4 s_conic[257];
-	__shared__ float4 s_cd[256];
-	__shared__ uint32_t s_id[256];
-	__shared__ float s_acc[kGradSlots][256];
-	__shared__ __attribute__((aligned(8))) uint16_t s_list[4][256];
-	__shared__ uint32_t s_count[4][4];
-	__shared__ uint32_t s_max[4];
+	__shared__ BackwardStage s_stage[4];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int tile = blockIdx.x;
+	const uint2 range = a.ranges[tile];
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
 	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
@@ -451,35 +471,22 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
 	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
 	const size_t plane = (size_t)a.H * a.W;
-	const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
+	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
+	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
+	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
+	BackwardStage& st = s_stage[wave];
+	const uint64_t below = (1ull << lane) - 1ull;
 
-	const uint2 range = a.ranges[tile];
+	if (range.y == range.x)
+		return;
 	const uint32_t last_contributor = inside ? a.n_contrib[pix_id] : 0u;
-
-	// Entries at or beyond the largest last_contributor of the tile are skipped by every
-	// pixel, so the walk starts there instead of at the end of the list; likewise a strip's
-	// list only takes entries below the largest last_contributor of that strip's 64 pixels.
-	uint32_t wave_span = last_contributor;
+	// entries at or beyond the largest last_contributor of the strip are skipped by all its pixels
+	uint32_t span = last_contributor;
 #pragma unroll
 	for (int off = 32; off > 0; off >>= 1)
-		wave_span = max(wave_span, (uint32_t)__shfl_xor((int)wave_span, off));
-	if (lane == 0)
-		s_max[wave] = wave_span;
-#pragma unroll
-	for (int q = 0; q < kGradSlots; q++)
-		s_acc[q][tid] = 0.f;
-	if (tid == 0) {
-		s_geom[kPadSlot] = float4{0.f, 0.f, INFINITY, 0.f};
-		s_conic[kPadSlot] = float4{0.f, 0.f, 0.f, 0.f};
-	}
-	__syncthreads();
-	const uint32_t span0 = s_max[0], span1 = s_max[1], span2 = s_max[2], span3 = s_max[3];
-	const uint32_t span = max(max(span0, span1), max(span2, span3));
-	if (span == 0)
+		span = max(span, (uint32_t)__shfl_xor((int)span, off));
+	if (span == 0u)
 		return;
-	const uint32_t back = range.x + span;  // one past the last entry any pixel uses
-	const int rounds = (int)((span + 255) / 256);
-	int todo = (int)span;
 
 	BackwardPixel p;
 	p.T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
@@ -498,68 +505,61 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	p.ddely_dy = 0.5 * a.H;
 	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
 
-	for (int i = 0; i < rounds; i++, todo -= 256) {
-		const uint32_t progress = (uint32_t)i * 256 + tid;
-		uint32_t strips = 0u;
-		if (progress < span) {
-			const uint32_t entry = span - 1 - progress;  // 0-based position in the tile list
-			const uint32_t id = a.point_list[back - progress - 1];
-			const float4* rec = a.record + 4 * (size_t)id;
-			const float4 geom = rec[0], co = rec[1], cd = rec[2], half = rec[3];
-			strips = reachable_strips(geom.x, geom.y, half.x, half.y, geom.z, tile_x0, tile_y0);
-			strips &= (entry < span0 ? 1u : 0u) | (entry < span1 ? 2u : 0u) | (entry < span2 ? 4u : 0u) |
-			          (entry < span3 ? 8u : 0u);
-			float w = geom.w;
-			if (strips) {
-				const int where = classify_tile_against_box(w, tile_x0, tile_y0, a, lo, hi);
-				if (where == kBoxOutside)
-					strips = 0u;
-				if (where == kBoxInside)
-					w = __int_as_float(0x7FC00000);
-			}
-			s_id[tid] = id;
-			s_geom[tid] = float4{geom.x, geom.y, geom.z, w};
-			s_conic[tid] = co;
-			s_cd[tid] = cd;
-		}
-		file_in_strip_lists(strips, tid, s_list, s_count);
-		__syncthreads();
+	// lane l of the chunk starting `first` entries from the back takes list position span-1-first-l
+	const uint32_t* list = a.point_list + range.x;
+	LoadedEntry cur = load_entry(a, (uint32_t)lane < span ? list[span - 1 - lane] : 0u, (uint32_t)lane < span);
+	uint32_t id_next = (uint32_t)(kChunk + lane) < span ? list[span - 1 - (kChunk + lane)] : 0u;
 
-		for (int seg = 0; seg < 4; seg++) {
-			const int n = (int)s_count[seg][wave];
-			for (int k = 0; k < n; k += 4) {
-				const uint2 packed = *reinterpret_cast<const uint2*>(&s_list[wave][seg * 64 + k]);
-				const int j0 = packed.x & 0xFFFFu, j1 = packed.x >> 16, j2 = packed.y & 0xFFFFu, j3 = packed.y >> 16;
-				const float4 g0 = s_geom[j0], g1 = s_geom[j1], g2 = s_geom[j2], g3 = s_geom[j3];
-				const float4 c0 = s_conic[j0], c1 = s_conic[j1], c2 = s_conic[j2], c3 = s_conic[j3];
-				float2 d;
-				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
-				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
-				// position of slot j in the tile list: span - 1 - (i * 256 + j)
-				const uint32_t top = span - 1 - (uint32_t)i * 256;
-				const bool q0 = (top - j0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z),
-				           q1 = (top - j1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z),
-				           q2 = (top - j2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z),
-				           q3 = (top - j3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
-				if (__ballot(q0 | q1 | q2 | q3) == 0ull)
-					continue;
-				backward_visit(p, q0, w0, g0, c0, pixf, s_cd, s_acc, j0, ray, a, lo, hi, lane);
-				backward_visit(p, q1, w1, g1, c1, pixf, s_cd, s_acc, j1, ray, a, lo, hi, lane);
-				backward_visit(p, q2, w2, g2, c2, pixf, s_cd, s_acc, j2, ray, a, lo, hi, lane);
-				backward_visit(p, q3, w3, g3, c3, pixf, s_cd, s_acc, j3, ray, a, lo, hi, lane);
-			}
-		}
-		__syncthreads();
+	for (uint32_t first = 0; first < span; first += kChunk) {
+		const uint32_t e1 = first + kChunk + lane, e2 = first + 2 * kChunk + lane;
+		LoadedEntry nxt = load_entry(a, id_next, e1 < span);
+		id_next = e2 < span ? list[span - 1 - e2] : 0u;
 
-		const int count = todo < 256 ? todo : 256;
-		if (tid < count) {
-			const size_t id = s_id[tid];
+		const bool filed = file_entry(cur, strip_x0, strip_y0, sc, a, lo, hi);
+		const uint64_t m = __ballot(filed);
+		const int count = __popcll(m);
+		if (filed) {
+			const int slot = __popcll(m & below);
+			st.geom[slot] = cur.geom;
+			st.conic[slot] = cur.conic;
+			st.cd[slot] = cur.cd;
+			st.entry[slot] = span - 1 - (first + lane);
+			st.id[slot] = cur.id;
+		}
+		if (lane < 4) {
+			st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
+			st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
+			st.entry[count + lane] = 0xFFFFFFFFu;
+		}
+		__builtin_amdgcn_wave_barrier();
+
+		uint64_t touched = 0ull;  // entries of this chunk that received sums (wave-uniform)
+		for (int k = 0; k < count; k += 4) {
+			const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
+			const float4 c0 = st.conic[k], c1 = st.conic[k + 1], c2 = st.conic[k + 2], c3 = st.conic[k + 3];
+			const uint32_t p0 = st.entry[k], p1 = st.entry[k + 1], p2 = st.entry[k + 2], p3 = st.entry[k + 3];
+			float2 d;
+			const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
+			            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
+			const bool q0 = (p0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z),
+			           q1 = (p1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z),
+			           q2 = (p2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z),
+			           q3 = (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
+			if (__ballot(q0 | q1 | q2 | q3) == 0ull)
+				continue;
+			if (backward_visit(p, q0, w0, g0, c0, pixf, st, k, ray, a, lo, hi, lane)) touched |= 1ull << k;
+			if (backward_visit(p, q1, w1, g1, c1, pixf, st, k + 1, ray, a, lo, hi, lane)) touched |= 1ull << (k + 1);
+			if (backward_visit(p, q2, w2, g2, c2, pixf, st, k + 2, ray, a, lo, hi, lane)) touched |= 1ull << (k + 2);
+			if (backward_visit(p, q3, w3, g3, c3, pixf, st, k + 3, ray, a, lo, hi, lane)) touched |= 1ull << (k + 3);
+		}
+		__builtin_amdgcn_wave_barrier();
+
+		if ((touched >> lane) & 1ull) {
+			const size_t id = st.id[lane];
 			float r[kGradSlots];
 #pragma unroll
-			for (int q = 0; q < kGradSlots; q++) {
-				r[q] = s_acc[q][tid];
-				s_acc[q][tid] = 0.f;
-			}
+			for (int q = 0; q < kGradSlots; q++)
+				r[q] = st.sums[q][lane];
 			if (r[0] != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 0], r[0]);
 			if (r[1] != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 1], r[1]);
 			if (r[2] != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 0], r[2]);
@@ -571,6 +571,8 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			if (r[8] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 2], r[8]);
 			if (r[9] != 0.f) unsafeAtomicAdd(&a.dL_ddepths[id], r[9]);
 		}
+		__builtin_amdgcn_wave_barrier();
+		cur = nxt;
 	}
 }
 
