@@ -402,8 +402,12 @@ __device__ __forceinline__ bool backward_visit(BackwardPixel& p, bool candidate,
 		const float alpha = fminf(0.99f, co.w * G);
 		if (!(alpha < 1.0f / 255.0f) &&
 		    !((g.w == g.w) && clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))) {
+			// From here on nothing feeds a decision: gradients are compared by tolerance, so the
+			// compiler may contract multiply-adds and the divisions use the hardware reciprocal.
+#pragma clang fp contract(fast)
 			valid = true;
-			p.T = p.T / (1.f - alpha);
+			const float inv_one_minus_alpha = __builtin_amdgcn_rcpf(1.f - alpha);
+			p.T = p.T * inv_one_minus_alpha;
 			const float aT = alpha * p.T;
 			const float4 cd = st.cd[slot];
 			float dL_dopa = 0.0f;
@@ -423,7 +427,7 @@ __device__ __forceinline__ bool backward_visit(BackwardPixel& p, bool candidate,
 			dL_dopa += (1 - p.accum_alpha) * p.g_alpha;
 			dL_dopa *= p.T;
 			p.last_alpha = alpha;
-			dL_dopa += (-p.T_final / (1.f - alpha)) * p.bg_dot_dpixel;
+			dL_dopa += (-p.T_final * inv_one_minus_alpha) * p.bg_dot_dpixel;
 
 			const float dL_dG = co.w * dL_dopa;
 			const float gdx = G * d.x;
