@@ -359,19 +359,28 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 
 // ---- backward (K/cuda_rasterizer_hgs/backward.cu:415-622) ---------------------------------------
 // Each wavefront walks the tile list back to front, starting at the largest last_contributor
-// of its own 64 pixels.  A lane forms its pixel's ten partial derivatives for an entry; they
-// are summed over the wavefront with DPP and lane 63 parks the sums in a wave-private LDS row
-// for that entry.  After the chunk, every lane flushes one entry's ten sums with one global
-// atomic each (one per (strip, Gaussian) and quantity).
+// of its own 64 pixels.  The pass is split in two so that no cross-lane reduction is needed
+// per entry:
+//  * pixel-parallel part (lane = pixel, as in the forward): the per-pixel recurrences of the
+//    reference loop give, for an entry, two numbers per pixel: u = G dL/dalpha-term and
+//    aT = alpha T.  They are parked in one LDS row per entry.
+//  * entry-parallel part, run whenever 16 rows are full (lane = (entry, strip row)): each lane
+//    sweeps the 16 pixels of its strip row and accumulates sum u, sum u dx, sum u dx^2 and
+//    sum aT g_{r,g,b,depth}; dy is constant along a strip row, so the y moments follow from
+//    those; two cross-row exchanges finish the sums and 16 lanes issue the ten global atomics
+//    of their entry (one per (strip, Gaussian) and quantity).
+// All ten sums of the reference (mean2D x/y, conic xx/xy/yy, opacity, colour r/g/b, depth)
+// are linear in u and aT, which is what makes the split possible.
 
-constexpr int kGradSlots = 10;  // mean2D x,y | conic xx,xy,yy | opacity | colour r,g,b | depth
+constexpr int kRows = 16;     // entries gathered before the entry-parallel part runs
+constexpr int kRowStride = 65;
 
 struct BackwardPixel {
 	float T, T_final;
 	float accum_r, accum_g, accum_b, accum_depth, accum_alpha;
 	float last_alpha, last_r, last_g, last_b, last_depth;
 	float g_r, g_g, g_b, g_depth, g_alpha;
-	float bg_dot_dpixel, ddelx_dx, ddely_dy;
+	float bg_dot_dpixel;
 };
 
 struct BackwardStage {  // wave-private
@@ -380,24 +389,84 @@ struct BackwardStage {  // wave-private
 	float4 cd[kChunk];
 	uint32_t entry[kChunk + 4];  // 0-based position in the tile list
 	uint32_t id[kChunk];
-	float sums[kGradSlots][kChunk];
+	float u[kRows * kRowStride];   // [row][pixel]
+	float at[kRows * kRowStride];  // [row][pixel]
+	float4 row_conic[kRows];
+	float2 row_xy[kRows];
+	uint32_t row_id[kRows];
+	float upstream[4][kChunk];     // dL/dpixel r, g, b, depth of the strip's 64 pixels
 };
 
-// Returns true (wave-uniform) when the entry received sums.
-__device__ __forceinline__ bool backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
-                                               const float4 co, const float2 pixf, BackwardStage& st, int slot,
-                                               const PixelRay& ray, const BlendArgs& a, const float3 lo, const float3 hi,
-                                               int lane)
+struct StripFrame {
+	float x0, y0;            // first pixel of the strip
+	float ddelx_dx, ddely_dy;
+};
+
+// Entry-parallel part for the first `rows` rows.  Lane (e = lane & 15, h = lane >> 4) sums row e
+// over the 16 pixels of strip row h.
+__device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, const StripFrame& f, const BlendArgs& a,
+                                           int lane)
+{
+#pragma clang fp contract(fast)
+	__builtin_amdgcn_wave_barrier();
+	const int e = lane & 15, h = lane >> 4;
+	const float2 xy = st.row_xy[e];
+	const float dy = xy.y - (f.y0 + (float)h);
+	float s0 = 0.f, sx = 0.f, sxx = 0.f, cr = 0.f, cg = 0.f, cb = 0.f, cdp = 0.f;
+	const float* urow = st.u + e * kRowStride + h * 16;
+	const float* arow = st.at + e * kRowStride + h * 16;
+#pragma unroll
+	for (int step = 0; step < 16; step++) {
+		const float uu = urow[step], tt = arow[step];
+		const float dx = xy.x - (f.x0 + (float)step);
+		const float t = uu * dx;
+		s0 += uu;
+		sx += t;
+		sxx += t * dx;
+		const int pix = h * 16 + step;
+		cr += tt * st.upstream[0][pix];
+		cg += tt * st.upstream[1][pix];
+		cb += tt * st.upstream[2][pix];
+		cdp += tt * st.upstream[3][pix];
+	}
+	float v[10] = {s0, sx, dy * s0, sxx, dy * sx, dy * dy * s0, cr, cg, cb, cdp};
+#pragma unroll
+	for (int q = 0; q < 10; q++) {
+		v[q] += __shfl_xor(v[q], 16);
+		v[q] += __shfl_xor(v[q], 32);
+	}
+	if (h == 0 && e < rows) {
+		const float4 co = st.row_conic[e];
+		const size_t id = st.row_id[e];
+		const float S0 = v[0], Sx = v[1], Sy = v[2], Sxx = v[3], Sxy = v[4], Syy = v[5];
+		const float m0 = -co.w * f.ddelx_dx * (co.x * Sx + co.y * Sy);
+		const float m1 = -co.w * f.ddely_dy * (co.z * Sy + co.y * Sx);
+		const float k0 = -0.5f * co.w * Sxx, k1 = -0.5f * co.w * Sxy, k3 = -0.5f * co.w * Syy;
+		if (m0 != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 0], m0);
+		if (m1 != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 1], m1);
+		if (k0 != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 0], k0);
+		if (k1 != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 1], k1);
+		if (k3 != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 3], k3);
+		if (S0 != 0.f) unsafeAtomicAdd(&a.dL_dopacity[id], S0);
+		if (v[6] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 0], v[6]);
+		if (v[7] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 1], v[7]);
+		if (v[8] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 2], v[8]);
+		if (v[9] != 0.f) unsafeAtomicAdd(&a.dL_ddepths[id], v[9]);
+	}
+	__builtin_amdgcn_wave_barrier();
+}
+
+// Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
+__device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
+                                               const float4 co, BackwardStage& st, int slot, int& rows,
+                                               const StripFrame& f, const PixelRay& ray, const BlendArgs& a,
+                                               const float3 lo, const float3 hi, int lane)
 {
 	if (__ballot(candidate) == 0ull)
-		return false;
-	float v[kGradSlots];
-#pragma unroll
-	for (int q = 0; q < kGradSlots; q++)
-		v[q] = 0.f;
+		return;
+	float u = 0.f, aT = 0.f;
 	bool valid = false;
 	if (candidate) {
-		const float2 d = {g.x - pixf.x, g.y - pixf.y};
 		const float G = exp_of_exponent(power);
 		const float alpha = fminf(0.99f, co.w * G);
 		if (!(alpha < 1.0f / 255.0f) &&
@@ -408,55 +477,44 @@ __device__ __forceinline__ bool backward_visit(BackwardPixel& p, bool candidate,
 			valid = true;
 			const float inv_one_minus_alpha = __builtin_amdgcn_rcpf(1.f - alpha);
 			p.T = p.T * inv_one_minus_alpha;
-			const float aT = alpha * p.T;
+			aT = alpha * p.T;
 			const float4 cd = st.cd[slot];
+			const float keep = 1.f - p.last_alpha;
 			float dL_dopa = 0.0f;
-			p.accum_r = p.last_alpha * p.last_r + (1.f - p.last_alpha) * p.accum_r;
+			p.accum_r = p.last_alpha * p.last_r + keep * p.accum_r;
 			p.last_r = cd.x;
 			dL_dopa += (cd.x - p.accum_r) * p.g_r;
-			p.accum_g = p.last_alpha * p.last_g + (1.f - p.last_alpha) * p.accum_g;
+			p.accum_g = p.last_alpha * p.last_g + keep * p.accum_g;
 			p.last_g = cd.y;
 			dL_dopa += (cd.y - p.accum_g) * p.g_g;
-			p.accum_b = p.last_alpha * p.last_b + (1.f - p.last_alpha) * p.accum_b;
+			p.accum_b = p.last_alpha * p.last_b + keep * p.accum_b;
 			p.last_b = cd.z;
 			dL_dopa += (cd.z - p.accum_b) * p.g_b;
-			p.accum_depth = p.last_alpha * p.last_depth + (1.f - p.last_alpha) * p.accum_depth;
+			p.accum_depth = p.last_alpha * p.last_depth + keep * p.accum_depth;
 			p.last_depth = cd.w;
 			dL_dopa += (cd.w - p.accum_depth) * p.g_depth;
-			p.accum_alpha = p.last_alpha + (1.f - p.last_alpha) * p.accum_alpha;
+			p.accum_alpha = p.last_alpha + keep * p.accum_alpha;
 			dL_dopa += (1 - p.accum_alpha) * p.g_alpha;
 			dL_dopa *= p.T;
 			p.last_alpha = alpha;
 			dL_dopa += (-p.T_final * inv_one_minus_alpha) * p.bg_dot_dpixel;
-
-			const float dL_dG = co.w * dL_dopa;
-			const float gdx = G * d.x;
-			const float gdy = G * d.y;
-			const float dG_ddelx = -gdx * co.x - gdy * co.y;
-			const float dG_ddely = -gdy * co.z - gdx * co.y;
-			v[0] = dL_dG * dG_ddelx * p.ddelx_dx;
-			v[1] = dL_dG * dG_ddely * p.ddely_dy;
-			v[2] = -0.5f * gdx * d.x * dL_dG;
-			v[3] = -0.5f * gdx * d.y * dL_dG;
-			v[4] = -0.5f * gdy * d.y * dL_dG;
-			v[5] = G * dL_dopa;
-			v[6] = aT * p.g_r;
-			v[7] = aT * p.g_g;
-			v[8] = aT * p.g_b;
-			v[9] = aT * p.g_depth;
+			u = G * dL_dopa;
 		}
 	}
 	if (__ballot(valid) == 0ull)
-		return false;
-#pragma unroll
-	for (int q = 0; q < kGradSlots; q++)
-		v[q] = wave_sum_to_lane63(v[q]);
-	if (lane == 63) {
-#pragma unroll
-		for (int q = 0; q < kGradSlots; q++)
-			st.sums[q][slot] = v[q];
+		return;
+	st.u[rows * kRowStride + lane] = u;
+	st.at[rows * kRowStride + lane] = aT;
+	if (lane == 0) {
+		st.row_conic[rows] = co;
+		st.row_xy[rows] = float2{g.x, g.y};
+		st.row_id[rows] = st.id[slot];
 	}
-	return true;
+	rows++;
+	if (rows == kRows) {
+		flush_rows(st, kRows, f, a, lane);
+		rows = 0;
+	}
 }
 
 __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
@@ -478,6 +536,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
 	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
 	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
+	const StripFrame frame = {strip_x0, strip_y0, (float)(0.5 * a.W), (float)(0.5 * a.H)};
 	BackwardStage& st = s_stage[wave];
 	const uint64_t below = (1ull << lane) - 1ull;
 
@@ -505,9 +564,12 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 		p.g_depth = a.dL_dpix_depth[pix_id];
 		p.g_alpha = a.dL_dalpha[pix_id];
 	}
-	p.ddelx_dx = 0.5 * a.W;
-	p.ddely_dy = 0.5 * a.H;
 	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
+	st.upstream[0][lane] = p.g_r;
+	st.upstream[1][lane] = p.g_g;
+	st.upstream[2][lane] = p.g_b;
+	st.upstream[3][lane] = p.g_depth;
+	int rows = 0;
 
 	// lane l of the chunk starting `first` entries from the back takes list position span-1-first-l
 	const uint32_t* list = a.point_list + range.x;
@@ -537,7 +599,6 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 		}
 		__builtin_amdgcn_wave_barrier();
 
-		uint64_t touched = 0ull;  // entries of this chunk that received sums (wave-uniform)
 		for (int k = 0; k < count; k += 4) {
 			const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
 			const float4 c0 = st.conic[k], c1 = st.conic[k + 1], c2 = st.conic[k + 2], c3 = st.conic[k + 3];
@@ -551,33 +612,16 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			           q3 = (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
 			if (__ballot(q0 | q1 | q2 | q3) == 0ull)
 				continue;
-			if (backward_visit(p, q0, w0, g0, c0, pixf, st, k, ray, a, lo, hi, lane)) touched |= 1ull << k;
-			if (backward_visit(p, q1, w1, g1, c1, pixf, st, k + 1, ray, a, lo, hi, lane)) touched |= 1ull << (k + 1);
-			if (backward_visit(p, q2, w2, g2, c2, pixf, st, k + 2, ray, a, lo, hi, lane)) touched |= 1ull << (k + 2);
-			if (backward_visit(p, q3, w3, g3, c3, pixf, st, k + 3, ray, a, lo, hi, lane)) touched |= 1ull << (k + 3);
-		}
-		__builtin_amdgcn_wave_barrier();
-
-		if ((touched >> lane) & 1ull) {
-			const size_t id = st.id[lane];
-			float r[kGradSlots];
-#pragma unroll
-			for (int q = 0; q < kGradSlots; q++)
-				r[q] = st.sums[q][lane];
-			if (r[0] != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 0], r[0]);
-			if (r[1] != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 1], r[1]);
-			if (r[2] != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 0], r[2]);
-			if (r[3] != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 1], r[3]);
-			if (r[4] != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 3], r[4]);
-			if (r[5] != 0.f) unsafeAtomicAdd(&a.dL_dopacity[id], r[5]);
-			if (r[6] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 0], r[6]);
-			if (r[7] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 1], r[7]);
-			if (r[8] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 2], r[8]);
-			if (r[9] != 0.f) unsafeAtomicAdd(&a.dL_ddepths[id], r[9]);
+			backward_visit(p, q0, w0, g0, c0, st, k, rows, frame, ray, a, lo, hi, lane);
+			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, frame, ray, a, lo, hi, lane);
+			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, frame, ray, a, lo, hi, lane);
+			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, lo, hi, lane);
 		}
 		__builtin_amdgcn_wave_barrier();
 		cur = nxt;
 	}
+	if (rows > 0)
+		flush_rows(st, rows, frame, a, lane);
 }
 
 void launch_blend_forward(const BlendArgs& a, hipStream_t s)
