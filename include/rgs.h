@@ -118,20 +118,17 @@ int rgs_forward_raster(int P, int R, int width, int height,
                        void* image_ws, size_t image_bytes,
                        float* out_color, float* out_depth, float* out_alpha, void* stream, int debug);
 
-/* Layout of grad_accum (12*P floats), the per-Gaussian sums the backward blend
- * accumulates atomically; offsets are in units of P floats. */
-enum {
-	RGS_ACC_MEAN2D = 0,   /* (P,3): d/dx, d/dy of the pixel centre, third column stays 0 */
-	RGS_ACC_CONIC = 3,    /* (P,4): xx, xy, unused, yy */
-	RGS_ACC_OPACITY = 7,  /* (P)   */
-	RGS_ACC_COLOR = 8,    /* (P,3) */
-	RGS_ACC_DEPTH = 11,   /* (P)   */
-	RGS_ACC_FLOATS = 12
-};
+/* grad_accum is scratch for the backward pass: RGS_ACC_FLOATS floats per Gaussian in which
+ * the backward blend accumulates its per-Gaussian sums atomically (one 48-byte row per
+ * Gaussian, so that the adds a wavefront issues for one Gaussian share a cache line).  The
+ * library clears it and the fused preprocess backward consumes it; its contents are not
+ * part of the interface. */
+enum { RGS_ACC_FLOATS = 12 };
 
 /* Rasterizer::backward (K/cuda_rasterizer_hgs/rasterizer.h:60-96, rasterizer_impl.cu:355-466)
  * together with the zero-initialisation done by its torch shim
- * (K/rasterize_points.cu:165-174).  grad_accum need not be cleared by the caller.
+ * (K/rasterize_points.cu:165-174).  grad_accum (RGS_ACC_FLOATS*P floats) need not be cleared
+ * by the caller.  dL_dmean2D (P,3; third column 0), dL_dopacity (P), dL_dcolor (P,3),
  * dL_dmean3D (P,3), dL_dcov3D (P,6), dL_dsh (P,M,3), dL_dscale (P,3), dL_drot (P,4) are
  * written for every Gaussian (zeros where it was not rendered); dL_dsh / dL_dscale /
  * dL_drot may be NULL when shs / scales are NULL. */
@@ -143,8 +140,8 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  float tan_fovx, float tan_fovy, const int* radii,
                  const void* geom_ws, const void* binning_ws, const void* image_ws,
                  const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
-                 float* grad_accum, float* dL_dmean3D, float* dL_dcov3D, float* dL_dsh, float* dL_dscale,
-                 float* dL_drot, void* stream, int debug);
+                 float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
+                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, void* stream, int debug);
 
 /* ---- measurement aids (no counterpart in the reference, which times whole iterations
  * with CUDA events: parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:590-643) -- */

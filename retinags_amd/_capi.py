@@ -16,7 +16,7 @@ GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles
                "clamped", "block_sums", "total", "blend_record")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
 IMG_FIELDS = ("ranges", "n_contrib")
-ACC_MEAN2D, ACC_CONIC, ACC_OPACITY, ACC_COLOR, ACC_DEPTH, ACC_FLOATS = 0, 3, 7, 8, 11, 12
+ACC_FLOATS = 12
 MAX_COMPOSITE = 64
 
 
@@ -48,7 +48,7 @@ def _load():
     lib.rgs_forward_raster.argtypes = [i, i, i, i, vp, f, f, vp, vp, vp, vp, vp, vp, sz, vp, sz, vp, sz,
                                        vp, vp, vp, vp, i]
     lib.rgs_backward.argtypes = [i, i, i, i, i, i, vp, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, vp, vp, vp,
-                                 f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i]
+                                 f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i]
     lib.rgs_inclusive_sum.argtypes = [vp, vp, sz, vp, vp]
     lib.rgs_sort_pairs.argtypes = [vp, vp, vp, vp, sz, i, vp, vp]
     pp = C.POINTER(vp)

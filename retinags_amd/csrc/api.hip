@@ -451,8 +451,8 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  float tan_fovx, float tan_fovy, const int* radii,
                  const void* geom_ws, const void* binning_ws, const void* image_ws,
                  const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
-                 float* grad_accum, float* dL_dmean3D, float* dL_dcov3D, float* dL_dsh, float* dL_dscale,
-                 float* dL_drot, void* stream, int debug)
+                 float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
+                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, void* stream, int debug)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
@@ -460,7 +460,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_backward: bad image size %dx%d", width, height);
 	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
 	                cam_pos && radii && geom_ws && image_ws && dL_dpix && dL_dpix_depth && dL_dalphas && grad_accum &&
-	                dL_dmean3D && dL_dcov3D,
+	                dL_dmean2D && dL_dopacity && dL_dcolor && dL_dmean3D && dL_dcov3D,
 	            "rgs_backward: null pointer");
 	RGS_REQUIRE(R == 0 || binning_ws, "rgs_backward: null binning workspace");
 	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr), "rgs_backward: provide exactly one of SHs or colours");
@@ -474,7 +474,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
 	const size_t n = (size_t)P;
 
-	rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, RGS_ACC_FLOATS * n, s);
+	rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, (size_t)RGS_ACC_FLOATS * n, s);
 	RGS_STAGE("clear gradient sums");
 
 	const float* colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
@@ -497,11 +497,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 		a.out_alpha = const_cast<float*>(alphas);
 		a.n_contrib = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]));
 		a.dL_dpix = dL_dpix; a.dL_dpix_depth = dL_dpix_depth; a.dL_dalpha = dL_dalphas;
-		a.dL_dmean2D = grad_accum + RGS_ACC_MEAN2D * n;
-		a.dL_dconic = grad_accum + RGS_ACC_CONIC * n;
-		a.dL_dopacity = grad_accum + RGS_ACC_OPACITY * n;
-		a.dL_dcolors = grad_accum + RGS_ACC_COLOR * n;
-		a.dL_ddepths = grad_accum + RGS_ACC_DEPTH * n;
+		a.sums = grad_accum;
 		rgs::launch_blend_backward(a, s);
 		RGS_STAGE("blend_backward");
 	}
@@ -517,10 +513,8 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	p.focal_y = height / (2.0f * tan_fovy);
 	p.focal_x = width / (2.0f * tan_fovx);
 	p.tanfovx = tan_fovx; p.tanfovy = tan_fovy;
-	p.dL_dmean2D = grad_accum + RGS_ACC_MEAN2D * n;
-	p.dL_dconic = grad_accum + RGS_ACC_CONIC * n;
-	p.dL_dcolor = grad_accum + RGS_ACC_COLOR * n;
-	p.dL_ddepth = grad_accum + RGS_ACC_DEPTH * n;
+	p.sums = grad_accum;
+	p.dL_dmean2D = dL_dmean2D; p.dL_dopacity = dL_dopacity; p.dL_dcolor = dL_dcolor;
 	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
 	rgs::launch_preprocess_backward(p, s);
 	RGS_STAGE("preprocess_backward");

@@ -373,7 +373,11 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 // are linear in u and aT, which is what makes the split possible.
 
 constexpr int kRows = 16;     // entries gathered before the entry-parallel part runs
-constexpr int kRowStride = 65;
+// Pixel p of the strip sits in column p + (p >> 5) of a row of kRowStride words: with these two
+// numbers neither the per-pixel writes nor the per-(entry, strip row) reads below hit an LDS
+// bank twice within a half wavefront.
+constexpr int kRowStride = 66;
+__device__ __forceinline__ int row_column(int pixel) { return pixel + (pixel >> 5); }
 
 struct BackwardPixel {
 	float T, T_final;
@@ -389,12 +393,12 @@ struct BackwardStage {  // wave-private
 	float4 cd[kChunk];
 	uint32_t entry[kChunk + 4];  // 0-based position in the tile list
 	uint32_t id[kChunk];
-	float u[kRows * kRowStride];   // [row][pixel]
-	float at[kRows * kRowStride];  // [row][pixel]
+	float u[kRows * kRowStride];   // [row][row_column(pixel)]
+	float at[kRows * kRowStride];  // [row][row_column(pixel)]
 	float4 row_conic[kRows];
 	float2 row_xy[kRows];
 	uint32_t row_id[kRows];
-	float upstream[4][kChunk];     // dL/dpixel r, g, b, depth of the strip's 64 pixels
+	float upstream[4][kRowStride];  // dL/dpixel r, g, b, depth of the strip's 64 pixels, by row_column
 };
 
 struct StripFrame {
@@ -402,19 +406,28 @@ struct StripFrame {
 	float ddelx_dx, ddely_dy;
 };
 
-// Entry-parallel part for the first `rows` rows.  Lane (e = lane & 15, h = lane >> 4) sums row e
-// over the 16 pixels of strip row h.
+template <int QuadPerm>
+__device__ __forceinline__ float quad_exchange_add(float v)
+{
+	const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), QuadPerm, 0xF, 0xF, true);
+	return v + __builtin_bit_cast(float, moved);
+}
+
+// Entry-parallel part for the first `rows` rows.  Lane (e = lane >> 2, h = lane & 3) sums row e
+// over the 16 pixels of strip row h; the four lanes of a quad then hold one entry and add the
+// entry's ten sums into the Gaussian's row of `sums`, four neighbouring columns per instruction.
 __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, const StripFrame& f, const BlendArgs& a,
                                            int lane)
 {
 #pragma clang fp contract(fast)
 	__builtin_amdgcn_wave_barrier();
-	const int e = lane & 15, h = lane >> 4;
+	const int e = lane >> 2, h = lane & 3;
 	const float2 xy = st.row_xy[e];
 	const float dy = xy.y - (f.y0 + (float)h);
 	float s0 = 0.f, sx = 0.f, sxx = 0.f, cr = 0.f, cg = 0.f, cb = 0.f, cdp = 0.f;
-	const float* urow = st.u + e * kRowStride + h * 16;
-	const float* arow = st.at + e * kRowStride + h * 16;
+	const int col0 = row_column(h * 16);
+	const float* urow = st.u + e * kRowStride + col0;
+	const float* arow = st.at + e * kRowStride + col0;
 #pragma unroll
 	for (int step = 0; step < 16; step++) {
 		const float uu = urow[step], tt = arow[step];
@@ -423,35 +436,31 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 		s0 += uu;
 		sx += t;
 		sxx += t * dx;
-		const int pix = h * 16 + step;
-		cr += tt * st.upstream[0][pix];
-		cg += tt * st.upstream[1][pix];
-		cb += tt * st.upstream[2][pix];
-		cdp += tt * st.upstream[3][pix];
+		cr += tt * st.upstream[0][col0 + step];
+		cg += tt * st.upstream[1][col0 + step];
+		cb += tt * st.upstream[2][col0 + step];
+		cdp += tt * st.upstream[3][col0 + step];
 	}
 	float v[10] = {s0, sx, dy * s0, sxx, dy * sx, dy * dy * s0, cr, cg, cb, cdp};
 #pragma unroll
 	for (int q = 0; q < 10; q++) {
-		v[q] += __shfl_xor(v[q], 16);
-		v[q] += __shfl_xor(v[q], 32);
+		v[q] = quad_exchange_add<0xB1>(v[q]);  // quad_perm:[1,0,3,2]
+		v[q] = quad_exchange_add<0x4E>(v[q]);  // quad_perm:[2,3,0,1]
 	}
-	if (h == 0 && e < rows) {
+	if (e < rows) {
 		const float4 co = st.row_conic[e];
-		const size_t id = st.row_id[e];
 		const float S0 = v[0], Sx = v[1], Sy = v[2], Sxx = v[3], Sxy = v[4], Syy = v[5];
 		const float m0 = -co.w * f.ddelx_dx * (co.x * Sx + co.y * Sy);
 		const float m1 = -co.w * f.ddely_dy * (co.z * Sy + co.y * Sx);
 		const float k0 = -0.5f * co.w * Sxx, k1 = -0.5f * co.w * Sxy, k3 = -0.5f * co.w * Syy;
-		if (m0 != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 0], m0);
-		if (m1 != 0.f) unsafeAtomicAdd(&a.dL_dmean2D[3 * id + 1], m1);
-		if (k0 != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 0], k0);
-		if (k1 != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 1], k1);
-		if (k3 != 0.f) unsafeAtomicAdd(&a.dL_dconic[4 * id + 3], k3);
-		if (S0 != 0.f) unsafeAtomicAdd(&a.dL_dopacity[id], S0);
-		if (v[6] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 0], v[6]);
-		if (v[7] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 1], v[7]);
-		if (v[8] != 0.f) unsafeAtomicAdd(&a.dL_dcolors[3 * id + 2], v[8]);
-		if (v[9] != 0.f) unsafeAtomicAdd(&a.dL_ddepths[id], v[9]);
+		// column 4 j + h of the row: see SumCol
+		const float w0 = h == 0 ? m0 : h == 1 ? m1 : h == 2 ? k0 : k1;
+		const float w1 = h == 0 ? k3 : h == 1 ? S0 : h == 2 ? v[6] : v[7];
+		const float w2 = h == 0 ? v[8] : h == 1 ? v[9] : 0.f;
+		float* row = a.sums + (size_t)kSumCols * st.row_id[e] + h;
+		if (w0 != 0.f) unsafeAtomicAdd(row, w0);
+		if (w1 != 0.f) unsafeAtomicAdd(row + 4, w1);
+		if (w2 != 0.f) unsafeAtomicAdd(row + 8, w2);
 	}
 	__builtin_amdgcn_wave_barrier();
 }
@@ -503,8 +512,8 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	}
 	if (__ballot(valid) == 0ull)
 		return;
-	st.u[rows * kRowStride + lane] = u;
-	st.at[rows * kRowStride + lane] = aT;
+	st.u[rows * kRowStride + row_column(lane)] = u;
+	st.at[rows * kRowStride + row_column(lane)] = aT;
 	if (lane == 0) {
 		st.row_conic[rows] = co;
 		st.row_xy[rows] = float2{g.x, g.y};
@@ -565,10 +574,10 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 		p.g_alpha = a.dL_dalpha[pix_id];
 	}
 	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
-	st.upstream[0][lane] = p.g_r;
-	st.upstream[1][lane] = p.g_g;
-	st.upstream[2][lane] = p.g_b;
-	st.upstream[3][lane] = p.g_depth;
+	st.upstream[0][row_column(lane)] = p.g_r;
+	st.upstream[1][row_column(lane)] = p.g_g;
+	st.upstream[2][row_column(lane)] = p.g_b;
+	st.upstream[3][row_column(lane)] = p.g_depth;
 	int rows = 0;
 
 	// lane l of the chunk starting `first` entries from the back takes list position span-1-first-l

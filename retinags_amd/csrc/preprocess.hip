@@ -325,6 +325,7 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 	for (int k = 0; k < 64; k++)
 		row[k] = 0.f;
 	const bool visible = idx < a.P && a.radii[idx > a.P - 1 ? a.P - 1 : idx] > 0;
+	float mean2d_x = 0.f, mean2d_y = 0.f, opacity_sum = 0.f, color_sum[3] = {0.f, 0.f, 0.f};
 	if (!sh_in_lds && idx < a.P && !visible)
 		for (int k = 0; k < n_sh; k++)
 			a.dL_dsh[i * n_sh + k] = 0.f;
@@ -334,7 +335,16 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 	const float* __restrict__ proj = a.proj;
 	const float3 mean = {a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
 	const float* cov6 = a.cov3D + 6 * i;
-	const float3 dLc = {a.dL_dconic[4 * i], a.dL_dconic[4 * i + 1], a.dL_dconic[4 * i + 3]};
+	const float4* sums = reinterpret_cast<const float4*>(a.sums + kSumCols * i);
+	const float4 sum0 = sums[0], sum1 = sums[1], sum2v = sums[2];
+	const float3 dLc = {sum0.z, sum0.w, sum1.x};  // kSumConicXX, kSumConicXY, kSumConicYY
+	const float sum_color[3] = {sum1.z, sum1.w, sum2v.x};
+	mean2d_x = sum0.x;
+	mean2d_y = sum0.y;
+	opacity_sum = sum1.y;
+	color_sum[0] = sum_color[0];
+	color_sum[1] = sum_color[1];
+	color_sum[2] = sum_color[2];
 
 	// -- conic -> cov2D -> cov3D and mean (backward.cu:144-274)
 	float cov6r[6];
@@ -407,7 +417,7 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 	// -- screen-space mean through the perspective divide (backward.cu:369-389)
 	const float4 m_hom = xform_point_4x4(mean, proj);
 	const float m_w = 1.0f / (m_hom.w + 0.0000001f);
-	const float g2x = a.dL_dmean2D[3 * i], g2y = a.dL_dmean2D[3 * i + 1];
+	const float g2x = mean2d_x, g2y = mean2d_y;
 	const float mul1 = (proj[0] * mean.x + proj[4] * mean.y + proj[8] * mean.z + proj[12]) * m_w * m_w;
 	const float mul2 = (proj[1] * mean.x + proj[5] * mean.y + proj[9] * mean.z + proj[13]) * m_w * m_w;
 	dmean.x += (proj[0] * m_w - proj[3] * mul1) * g2x + (proj[1] * m_w - proj[3] * mul2) * g2y;
@@ -415,7 +425,7 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 	dmean.z += (proj[8] * m_w - proj[11] * mul1) * g2x + (proj[9] * m_w - proj[11] * mul2) * g2y;
 
 	// -- per-Gaussian depth (backward.cu:391-403)
-	const float gd = a.dL_ddepth[i];
+	const float gd = sum2v.y;  // kSumDepth
 	const float mul3 = view[2] * mean.x + view[6] * mean.y + view[10] * mean.z + view[14];
 	dmean.x += (view[2] - view[3] * mul3) * gd;
 	dmean.y += (view[6] - view[7] * mul3) * gd;
@@ -432,7 +442,7 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 		float ddx = 0.f, ddy = 0.f, ddz = 0.f;
 #pragma unroll
 		for (int ch = 0; ch < 3; ch++) {
-			const float g = a.dL_dcolor[3 * i + ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
+			const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
 			if (sh_in_lds)  // the usual case: rows go out through LDS, coalesced
 				sh_backward_channel(a.D, x, y, z, sh + ch, g, row + kBwdSh + ch, ddx, ddy, ddz);
 			else
@@ -511,6 +521,20 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 	}
 	if (n_sh > 0 && sh_in_lds)
 		store_rows(a.dL_dsh + (size_t)n_sh * first, s_out, kBwdSh, n_sh, rows, lane);
+
+	// the sums that are gradients as they stand leave through the same rows
+	__syncthreads();
+	row[0] = mean2d_x;
+	row[1] = mean2d_y;
+	row[2] = 0.f;
+	row[3] = opacity_sum;
+	row[4] = color_sum[0];
+	row[5] = color_sum[1];
+	row[6] = color_sum[2];
+	__syncthreads();
+	store_rows(a.dL_dmean2D + 3 * (size_t)first, s_out, 0, 3, rows, lane);
+	store_rows(a.dL_dopacity + (size_t)first, s_out, 3, 1, rows, lane);
+	store_rows(a.dL_dcolor + 3 * (size_t)first, s_out, 4, 3, rows, lane);
 }
 
 // ---- launchers -----------------------------------------------------------------------------

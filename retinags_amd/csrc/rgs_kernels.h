@@ -51,11 +51,11 @@ struct PreprocessBackwardArgs {
 	const float* proj;
 	const float* campos;
 	float focal_x, focal_y, tanfovx, tanfovy;
-	const float* dL_dmean2D;  // (P,3)
-	const float* dL_dconic;   // (P,4)
-	const float* dL_dcolor;   // (P,3)
-	const float* dL_ddepth;   // (P)
+	const float* sums;  // (P, kSumCols): what the backward blend accumulated, see SumCol
 	// outputs, fully written
+	float* dL_dmean2D;  // (P,3), third column 0
+	float* dL_dopacity; // (P)
+	float* dL_dcolor;   // (P,3)
 	float* dL_dmeans;   // (P,3)
 	float* dL_dcov3D;   // (P,6)
 	float* dL_dsh;      // (P,M,3)
@@ -88,11 +88,15 @@ struct BlendArgs {
 	const float* dL_dpix;
 	const float* dL_dpix_depth;
 	const float* dL_dalpha;
-	float* dL_dmean2D;   // (P,3)
-	float* dL_dconic;    // (P,4)
-	float* dL_dopacity;  // (P)
-	float* dL_dcolors;   // (P,3)
-	float* dL_ddepths;   // (P)
+	float* sums;  // (P, kSumCols), cleared by the caller; the blend adds into it atomically
+};
+
+// Columns of a Gaussian's row of gradient sums.  One row is 48 bytes, so the (up to) ten atomic
+// adds that a wavefront issues for a Gaussian fall into one or two cache lines.
+enum SumCol {
+	kSumMeanX = 0, kSumMeanY = 1, kSumConicXX = 2, kSumConicXY = 3,
+	kSumConicYY = 4, kSumOpacity = 5, kSumR = 6, kSumG = 7,
+	kSumB = 8, kSumDepth = 9, kSumCols = 12
 };
 
 struct CompositeArgs {

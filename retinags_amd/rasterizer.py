@@ -168,8 +168,11 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
     range_up = _dev_f32(range_up, device, "range_up")
     campos = _dev_f32(campos, device, "campos")
 
-    # The five sums the blend accumulates atomically live in one buffer that the library clears.
+    # Scratch rows in which the blend accumulates its per-Gaussian sums; the library clears them.
     acc = torch.empty((_capi.ACC_FLOATS * P,), **f32)
+    dL_dmeans2D = torch.empty((P, 3), **f32)
+    dL_dopacity = torch.empty((P, 1), **f32)
+    dL_dcolors = torch.empty((P, 3), **f32)
     dL_dmeans3D = torch.empty((P, 3), **f32)
     dL_dcov3D = torch.empty((P, 6), **f32)
     dL_dsh = torch.empty((P, M, 3), **f32)
@@ -183,13 +186,11 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
             ptr(alpha), ptr(scales), float(scale_modifier), ptr(rotations), ptr(cov3Ds_precomp), ptr(viewmatrix),
             ptr(projmatrix), ptr(projmatrix_inv), ptr(range_low), ptr(range_up), ptr(campos), float(tanfovx),
             float(tanfovy), ptr(radii), ptr(geomBuffer), ptr(binningBuffer), ptr(imgBuffer), ptr(grad_color),
-            ptr(grad_depth), ptr(grad_alpha), ptr(acc), ptr(dL_dmeans3D), ptr(dL_dcov3D), ptr(dL_dsh),
+            ptr(grad_depth), ptr(grad_alpha), ptr(acc), ptr(dL_dmeans2D), ptr(dL_dopacity), ptr(dL_dcolors),
+            ptr(dL_dmeans3D), ptr(dL_dcov3D), ptr(dL_dsh),
             ptr(dL_dscales) if has_scales else C.c_void_p(0), ptr(dL_drotations) if has_scales else C.c_void_p(0),
             _stream_ptr(device), int(bool(debug))))
 
-    dL_dmeans2D = acc[_capi.ACC_MEAN2D * P:(_capi.ACC_MEAN2D + 3) * P].view(P, 3)
-    dL_dopacity = acc[_capi.ACC_OPACITY * P:(_capi.ACC_OPACITY + 1) * P].view(P, 1)
-    dL_dcolors = acc[_capi.ACC_COLOR * P:(_capi.ACC_COLOR + 3) * P].view(P, 3)
     return dL_dmeans2D, dL_dcolors, dL_dopacity, dL_dmeans3D, dL_dcov3D, dL_dsh, dL_dscales, dL_drotations
 
 
