@@ -34,16 +34,44 @@ struct PixelRay {
 	float ndc_x, ndc_y;  // pixel centre in NDC
 };
 
+__device__ __forceinline__ float wave_uniform(float v)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
+// What the half-Gaussian test needs besides the pixel: rows 0..2 of the inverse projection
+// (column-major 4x4, m[c][r] = element (r, c)) and the submodel box.  Read once per wavefront
+// into scalar registers; the test itself runs for every blended sample.
+struct BoxFrame {
+	float m[4][3];
+	float3 lo, hi;
+	float tanx, tany;
+};
+
+__device__ __forceinline__ BoxFrame load_box_frame(const BlendArgs& a)
+{
+	BoxFrame b;
+#pragma unroll
+	for (int c = 0; c < 4; c++)
+#pragma unroll
+		for (int r = 0; r < 3; r++)
+			b.m[c][r] = wave_uniform(a.projinv[4 * c + r]);
+	b.lo = float3{wave_uniform(a.range_low[0]), wave_uniform(a.range_low[1]), wave_uniform(a.range_low[2])};
+	b.hi = float3{wave_uniform(a.range_up[0]), wave_uniform(a.range_up[1]), wave_uniform(a.range_up[2])};
+	b.tanx = a.tanfovx;
+	b.tany = a.tanfovy;
+	return b;
+}
+
 // World-space point of the pixel's ray at clip-w `w`, tested against the submodel box
 // (low, up] (K/cuda_rasterizer_hgs/forward.cu:360-372).  True when the sample is clipped.
-__device__ __forceinline__ bool clipped_by_box(const PixelRay& ray, float w, float tanx, float tany,
-                                               const float* __restrict__ m, const float3 lo, const float3 hi)
+__device__ __forceinline__ bool clipped_by_box(const PixelRay& ray, float w, const BoxFrame& b)
 {
-	const float3 ph = {ray.ndc_x * (w + 0.0000001f) * tanx, ray.ndc_y * (w + 0.0000001f) * tany, w};
-	const float wx = m[0] * ph.x + m[4] * ph.y + m[8] * ph.z + m[12];
-	const float wy = m[1] * ph.x + m[5] * ph.y + m[9] * ph.z + m[13];
-	const float wz = m[2] * ph.x + m[6] * ph.y + m[10] * ph.z + m[14];
-	return (wx <= lo.x) || (wx > hi.x) || (wy <= lo.y) || (wy > hi.y) || (wz <= lo.z) || (wz > hi.z);
+	const float3 ph = {ray.ndc_x * (w + 0.0000001f) * b.tanx, ray.ndc_y * (w + 0.0000001f) * b.tany, w};
+	const float wx = b.m[0][0] * ph.x + b.m[1][0] * ph.y + b.m[2][0] * ph.z + b.m[3][0];
+	const float wy = b.m[0][1] * ph.x + b.m[1][1] * ph.y + b.m[2][1] * ph.z + b.m[3][1];
+	const float wz = b.m[0][2] * ph.x + b.m[1][2] * ph.y + b.m[2][2] * ph.z + b.m[3][2];
+	return (wx <= b.lo.x) || (wx > b.hi.x) || (wy <= b.lo.y) || (wy > b.hi.y) || (wz <= b.lo.z) || (wz > b.hi.z);
 }
 
 // exp(x) for the exponents of the blend (x <= 0, modest magnitude): 2^(x log2 e) on the
@@ -79,25 +107,24 @@ struct StripCorners {
 	float nx0, nx1, ny0, ny1;  // NDC of the strip's first/last pixel column and row
 };
 
-__device__ __forceinline__ int classify_strip_against_box(float w, const StripCorners& sc, const BlendArgs& a,
-                                                          const float3 lo, const float3 hi)
+__device__ __forceinline__ int classify_strip_against_box(float w, const StripCorners& sc, const BoxFrame& b)
 {
-	const float* __restrict__ m = a.projinv;
 	float pmin[3] = {INFINITY, INFINITY, INFINITY}, pmax[3] = {-INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
 	for (int c = 0; c < 4; c++) {
 		const float nx = (c & 1) ? sc.nx1 : sc.nx0;
 		const float ny = (c & 2) ? sc.ny1 : sc.ny0;
-		const float3 ph = {nx * (w + 0.0000001f) * a.tanfovx, ny * (w + 0.0000001f) * a.tanfovy, w};
-		const float q[3] = {m[0] * ph.x + m[4] * ph.y + m[8] * ph.z + m[12], m[1] * ph.x + m[5] * ph.y + m[9] * ph.z + m[13],
-		                    m[2] * ph.x + m[6] * ph.y + m[10] * ph.z + m[14]};
+		const float3 ph = {nx * (w + 0.0000001f) * b.tanx, ny * (w + 0.0000001f) * b.tany, w};
+		const float q[3] = {b.m[0][0] * ph.x + b.m[1][0] * ph.y + b.m[2][0] * ph.z + b.m[3][0],
+		                    b.m[0][1] * ph.x + b.m[1][1] * ph.y + b.m[2][1] * ph.z + b.m[3][1],
+		                    b.m[0][2] * ph.x + b.m[1][2] * ph.y + b.m[2][2] * ph.z + b.m[3][2]};
 #pragma unroll
 		for (int k = 0; k < 3; k++) {
 			pmin[k] = fminf(pmin[k], q[k]);
 			pmax[k] = fmaxf(pmax[k], q[k]);
 		}
 	}
-	const float lov[3] = {lo.x, lo.y, lo.z}, hiv[3] = {hi.x, hi.y, hi.z};
+	const float lov[3] = {b.lo.x, b.lo.y, b.lo.z}, hiv[3] = {b.hi.x, b.hi.y, b.hi.z};
 	bool inside = true, outside = false;
 #pragma unroll
 	for (int k = 0; k < 3; k++) {
@@ -138,12 +165,11 @@ __device__ __forceinline__ LoadedEntry load_entry(const BlendArgs& a, uint32_t i
 
 // Decides whether the lane's entry is filed for this strip; a filed entry whose strip lies
 // entirely inside the box gets a NaN clip-w, which tells the walk to skip the per-pixel test.
-__device__ __forceinline__ bool file_entry(LoadedEntry& e, float x0, float ya, const StripCorners& sc, const BlendArgs& a,
-                                           const float3 lo, const float3 hi)
+__device__ __forceinline__ bool file_entry(LoadedEntry& e, float x0, float ya, const StripCorners& sc, const BoxFrame& box)
 {
 	if (!reaches_strip(e.geom.x, e.geom.y, e.half.x, e.half.y, e.geom.z, x0, ya))
 		return false;
-	const int where = classify_strip_against_box(e.geom.w, sc, a, lo, hi);
+	const int where = classify_strip_against_box(e.geom.w, sc, box);
 	if (where == kBoxOutside)
 		return false;
 	if (where == kBoxInside)
@@ -174,15 +200,15 @@ struct ForwardStage {  // wave-private
 
 __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, float power, const float4 g,
                                               const float4 co, const ForwardStage& st, int slot, const PixelRay& ray,
-                                              const BlendArgs& a, const float3 lo, const float3 hi)
+                                              const BoxFrame& box)
 {
 	candidate = candidate && !p.done;
 	if (__ballot(candidate) == 0ull)
 		return;
+	const float clip_w = wave_uniform(g.w);  // NaN: the whole strip is inside the box
 	if (candidate) {
 		const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
-		if (!(alpha < 1.0f / 255.0f) &&
-		    !((g.w == g.w) && clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))) {
+		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, box))) {
 			const float test_T = p.T * (1 - alpha);
 			if (test_T < 0.0001f) {
 				p.done = true;
@@ -214,8 +240,7 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	const uint32_t pix_id = (uint32_t)a.W * py + px;
 	const float2 pixf = {(float)px, (float)py};
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
-	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
-	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
+	const BoxFrame box = load_box_frame(a);
 	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
 	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
 	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
@@ -236,7 +261,7 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 			LoadedEntry nxt = load_entry(a, id_next, e1 < n);
 			id_next = e2 < n ? list[e2] : 0u;
 
-			const bool filed = file_entry(cur, strip_x0, strip_y0, sc, a, lo, hi);
+			const bool filed = file_entry(cur, strip_x0, strip_y0, sc, box);
 			const uint64_t m = __ballot(filed);
 			const int count = __popcll(m);
 			if (filed) {
@@ -263,10 +288,10 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
 				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
 					continue;
-				forward_visit(p, q0, w0, g0, c0, st, k, ray, a, lo, hi);
-				forward_visit(p, q1, w1, g1, c1, st, k + 1, ray, a, lo, hi);
-				forward_visit(p, q2, w2, g2, c2, st, k + 2, ray, a, lo, hi);
-				forward_visit(p, q3, w3, g3, c3, st, k + 3, ray, a, lo, hi);
+				forward_visit(p, q0, w0, g0, c0, st, k, ray, box);
+				forward_visit(p, q1, w1, g1, c1, st, k + 1, ray, box);
+				forward_visit(p, q2, w2, g2, c2, st, k + 2, ray, box);
+				forward_visit(p, q3, w3, g3, c3, st, k + 3, ray, box);
 				live = __ballot(!p.done);
 			}
 			__builtin_amdgcn_wave_barrier();
@@ -301,8 +326,7 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
 	const float2 pixf = {(float)px, (float)py};
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
-	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
-	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
+	const BoxFrame box = load_box_frame(a);
 	const uint2 range = a.ranges[tile];
 	const int rounds = (int)((range.y - range.x + 255) / 256);
 	int todo = (int)(range.y - range.x);
@@ -334,7 +358,7 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 			if (alpha < 1.0f / 255.0f)
 				continue;
 			nC++;
-			if (clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))
+			if (clipped_by_box(ray, g.w, box))
 				continue;
 			nD++;
 			const float test_T = T * (1 - alpha);
@@ -469,17 +493,17 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
                                                const float4 co, BackwardStage& st, int slot, int& rows,
                                                const StripFrame& f, const PixelRay& ray, const BlendArgs& a,
-                                               const float3 lo, const float3 hi, int lane)
+                                               const BoxFrame& box, int lane)
 {
 	if (__ballot(candidate) == 0ull)
 		return;
 	float u = 0.f, aT = 0.f;
 	bool valid = false;
+	const float clip_w = wave_uniform(g.w);  // NaN: the whole strip is inside the box
 	if (candidate) {
 		const float G = exp_of_exponent(power);
 		const float alpha = fminf(0.99f, co.w * G);
-		if (!(alpha < 1.0f / 255.0f) &&
-		    !((g.w == g.w) && clipped_by_box(ray, g.w, a.tanfovx, a.tanfovy, a.projinv, lo, hi))) {
+		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, box))) {
 			// From here on nothing feeds a decision: gradients are compared by tolerance, so the
 			// compiler may contract multiply-adds and the divisions use the hardware reciprocal.
 #pragma clang fp contract(fast)
@@ -539,8 +563,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	const uint32_t pix_id = (uint32_t)a.W * py + px;
 	const float2 pixf = {(float)px, (float)py};
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
-	const float3 lo = {a.range_low[0], a.range_low[1], a.range_low[2]};
-	const float3 hi = {a.range_up[0], a.range_up[1], a.range_up[2]};
+	const BoxFrame box = load_box_frame(a);
 	const size_t plane = (size_t)a.H * a.W;
 	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
 	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
@@ -590,7 +613,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 		LoadedEntry nxt = load_entry(a, id_next, e1 < span);
 		id_next = e2 < span ? list[span - 1 - e2] : 0u;
 
-		const bool filed = file_entry(cur, strip_x0, strip_y0, sc, a, lo, hi);
+		const bool filed = file_entry(cur, strip_x0, strip_y0, sc, box);
 		const uint64_t m = __ballot(filed);
 		const int count = __popcll(m);
 		if (filed) {
@@ -621,10 +644,10 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			           q3 = (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
 			if (__ballot(q0 | q1 | q2 | q3) == 0ull)
 				continue;
-			backward_visit(p, q0, w0, g0, c0, st, k, rows, frame, ray, a, lo, hi, lane);
-			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, frame, ray, a, lo, hi, lane);
-			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, frame, ray, a, lo, hi, lane);
-			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, lo, hi, lane);
+			backward_visit(p, q0, w0, g0, c0, st, k, rows, frame, ray, a, box, lane);
+			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, frame, ray, a, box, lane);
+			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, frame, ray, a, box, lane);
+			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, box, lane);
 		}
 		__builtin_amdgcn_wave_barrier();
 		cur = nxt;
