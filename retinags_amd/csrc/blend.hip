@@ -27,6 +27,7 @@
 //    filed, one whose corners are all inside skips the per-pixel box test.
 // All three only drop work that the exact evaluation would have skipped too.
 #include "rgs_kernels.h"
+#include "tile_order.h"
 
 namespace rgs {
 
@@ -163,6 +164,15 @@ __device__ __forceinline__ LoadedEntry load_entry(const BlendArgs& a, uint32_t i
 	return e;
 }
 
+// The last two words of a record are padding.  Registers that a load in flight will write
+// cannot be reused, but the compiler would hand these two to the walk as temporaries, and the
+// walk would then wait for the very prefetch it is meant to overlap; naming them as used after
+// the walk keeps them reserved.
+__device__ __forceinline__ void keep_padding_registers(const LoadedEntry& e)
+{
+	asm volatile("" ::"v"(e.half.z), "v"(e.half.w));
+}
+
 // Decides whether the lane's entry is filed for this strip; a filed entry whose strip lies
 // entirely inside the box gets a NaN clip-w, which tells the walk to skip the per-pixel test.
 __device__ __forceinline__ bool file_entry(LoadedEntry& e, float x0, float ya, const StripCorners& sc, const BoxFrame& box)
@@ -231,7 +241,9 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	__shared__ ForwardStage s_stage[4];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const int tile = blockIdx.x;
+	const int tile = tile_of_block((int)blockIdx.x, a.grid_x, a.grid_y);
+	if (tile < 0)
+		return;
 	const uint2 range = a.ranges[tile];
 	const uint32_t n = range.y - range.x;
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
@@ -295,7 +307,8 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				live = __ballot(!p.done);
 			}
 			__builtin_amdgcn_wave_barrier();
-			cur = nxt;
+			keep_padding_registers(nxt);
+		cur = nxt;
 		}
 	}
 
@@ -320,7 +333,9 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 	__shared__ float4 s_conic[256];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const int tile = blockIdx.x;
+	const int tile = tile_of_block((int)blockIdx.x, a.grid_x, a.grid_y);
+	if (tile < 0)
+		return;
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
 	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
@@ -555,7 +570,9 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	__shared__ BackwardStage s_stage[4];
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const int tile = blockIdx.x;
+	const int tile = tile_of_block((int)blockIdx.x, a.grid_x, a.grid_y);
+	if (tile < 0)
+		return;
 	const uint2 range = a.ranges[tile];
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
@@ -650,6 +667,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, box, lane);
 		}
 		__builtin_amdgcn_wave_barrier();
+		keep_padding_registers(nxt);
 		cur = nxt;
 	}
 	if (rows > 0)
@@ -660,15 +678,15 @@ void launch_blend_forward(const BlendArgs& a, hipStream_t s)
 {
 	stage_mark(a.counters ? "blend_count" : "blend_forward", s);
 	if (a.counters)
-		hipLaunchKernelGGL(blend_count_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+		hipLaunchKernelGGL(blend_count_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
 	else
-		hipLaunchKernelGGL(blend_forward_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+		hipLaunchKernelGGL(blend_forward_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
 }
 
 void launch_blend_backward(const BlendArgs& a, hipStream_t s)
 {
 	stage_mark("blend_backward", s);
-	hipLaunchKernelGGL(blend_backward_kernel, dim3(a.grid_x * a.grid_y), dim3(256), 0, s, a);
+	hipLaunchKernelGGL(blend_backward_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
 }
 
 }  // namespace rgs

@@ -151,3 +151,14 @@ def test_partition_and_order_invariants():
     c = cam.camera_center.numpy()
     inside = [k for k in range(4) if (c[:2] >= part.box_low[k][:2]).all() and (c[:2] <= part.box_up[k][:2]).all()]
     assert inside and rel[inside[0]] == min(seen)
+
+
+def test_banded_tile_order_is_a_bijection(tmp_path):
+    """The blend kernels take tiles in an XCD-banded order; every tile must be taken exactly once."""
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = str(tmp_path / "tile_order_check")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-I", os.path.join(here, "..", "retinags_amd", "csrc"),
+                    os.path.join(here, "tile_order_check.cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    assert out.strip() == "ok"
