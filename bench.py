@@ -30,6 +30,17 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
 
+# HBM bytes per launch of each stage's kernels on the default workload (C1 at full size), from
+# rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this script scaled by what the same counters read
+# for a 1 GiB copy (x2.000 and x1.000 to KiB); mean over the launches of a step.  Counters
+# cannot be read from inside the process, so the figures are carried here; other workloads
+# report null.
+C1_TRAFFIC_MB_PER_LAUNCH = {
+    "preprocess_forward": 292.14, "duplicate_with_keys": 59.83, "sort_onesweep": 76.69, "tile_ranges": 24.89,
+    "blend_forward": 225.09, "composite_forward": 165.79, "composite_backward": 371.97, "blend_backward": 276.28,
+    "preprocess_backward": 598.19,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -41,6 +52,8 @@ def parse():
     ap.add_argument("--resolution-scale", type=float, default=1.0, help="scale the image size (debugging only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-threads", type=int, default=0)
+    ap.add_argument("--streams", type=int, default=4,
+                    help="render the submodels of a frame on this many HIP streams (0: all on the current stream)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device-to-device copy, the known-size reference for HBM traffic counters")
     return ap.parse_args()
@@ -92,11 +105,13 @@ def main():
     related = [m for m in range(len(subs)) if rel[m] >= 0]
     setup_s = time.time() - t0
 
-    def step():
+    streams = [torch.cuda.Stream(device=dev) for _ in range(args.streams)] if args.streams > 0 else None
+
+    def step(streams=streams):
         for s in subs:
             for p in s.parameters():
                 p.grad = None
-        out = pipeline.render_frame(cam_d, subs, rel, bg)
+        out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams)
         if do_backward:
             torch.autograd.backward([out["render"]], [upstream])
         return out
@@ -123,7 +138,7 @@ def main():
     prof_steps = max(1, min(args.steps, 5))
     _capi.stage_timing(True)
     for _ in range(prof_steps):
-        step()
+        step(streams=None)  # one stream, so that consecutive events bracket one stage each
     stage_ms = _capi.stage_timing_read()
     _capi.stage_timing(False)
 
@@ -200,6 +215,10 @@ def main():
             roofline = {"kernel": dominant, "bound": "valu", "achieved": d["achieved_TFLOPs"],
                         "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": d["frac"], "traffic": None}
         if roofline is not None:
+            full_c1 = args.config == "C1" and args.shrink == 1.0 and args.resolution_scale == 1.0
+            if full_c1 and dominant in C1_TRAFFIC_MB_PER_LAUNCH:
+                roofline["traffic"] = C1_TRAFFIC_MB_PER_LAUNCH[dominant] * 1e6  # bytes per launch
+            roofline["timing"] = "HIP events on the launching stream, all submodels on one stream"
             roofline["avg_launch_ms"] = d["avg_launch_ms"]
             roofline["launches_per_step"] = d["launches_per_step"]
 

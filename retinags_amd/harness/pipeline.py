@@ -87,13 +87,37 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
 
 
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
-                 submodel_bg: Optional[torch.Tensor] = None) -> dict:
+                 submodel_bg: Optional[torch.Tensor] = None,
+                 streams: Optional[List["torch.cuda.Stream"]] = None) -> dict:
     """Render every related submodel (black background, as the trainer does:
-    trainer4tree_partition.py:397) and composite the partial images in BVH order."""
+    trainer4tree_partition.py:397) and composite the partial images in BVH order.
+
+    The reference renders the submodels on different GPUs at the same time.  On one GPU the
+    same independence is offered to the hardware through `streams`: submodel k is rendered on
+    streams[k % len(streams)] (default priority), so one submodel's short kernels and the tail
+    of its blend run beside another's; autograd replays each submodel's backward on the stream
+    its forward used.  The compositor runs on the caller's stream after all of them.
+    """
     device = subs[0].means3D.device
     if submodel_bg is None:
         submodel_bg = torch.zeros(3, device=device)
-    partial = {m: render_submodel(cam, subs[m], submodel_bg) for m in range(len(subs)) if relation[m] >= 0}
+    related = [m for m in range(len(subs)) if relation[m] >= 0]
+    if not streams:
+        partial = {m: render_submodel(cam, subs[m], submodel_bg) for m in related}
+    else:
+        main = torch.cuda.current_stream(device)
+        partial = {}
+        for k, m in enumerate(related):
+            side = streams[k % len(streams)]
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                partial[m] = render_submodel(cam, subs[m], submodel_bg)
+        for side in streams[:len(related)]:
+            main.wait_stream(side)
+        for res in partial.values():
+            for t in res.values():
+                if torch.is_tensor(t) and t.is_cuda:
+                    t.record_stream(main)
     out = blender_render_result(partial, relation, background)
     out["partial"] = partial
     return out

@@ -175,3 +175,39 @@ def test_partitioned_frame_against_checker():
     whole = orc.forward(s_all, np32(scene["xyz"]), np32(scene["opacity"]), shs=np32(scene["shs"]),
                         scales=np32(scene["scales"]), rotations=np32(scene["rotations"]))
     assert np.abs(w_img - whole.color).mean() < 2e-3
+
+
+def test_frame_on_several_streams_matches_one_stream():
+    """Submodels rendered on separate HIP streams (forward and, through autograd, backward)
+    give the images of the one-stream frame bit for bit and the same gradients up to the
+    order of the atomic adds; repeated, to catch a missing dependency between streams."""
+    from retinags_amd.harness import partition, pipeline
+    scene, cam, _ = scenes.make_config("C1", shrink=40, resolution_scale=0.5)
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    rel = partition.relation_vector(part, cam)
+    subs = [s.requires_grad_(True) for s in pipeline.submodels_from_partition(scene, part, DEV)]
+    H, W = cam.image_height, cam.image_width
+    up = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(5)) * 1e-2).to(DEV)
+    bg = torch.tensor([0.2, 0.3, 0.4], device=DEV)
+    cam_d = cam.to(DEV)
+
+    def frame(streams):
+        for s in subs:
+            for p in s.parameters():
+                p.grad = None
+        out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams)
+        torch.autograd.backward([out["render"]], [up])
+        torch.cuda.synchronize()
+        grads = [[p.grad.clone() for p in s.parameters()] for s in subs]
+        return out["render"].detach().clone(), out["depth"].detach().clone(), out["alpha"].detach().clone(), grads
+
+    ref = frame(None)
+    for n_streams in (2, 4, 4):
+        streams = [torch.cuda.Stream(device=DEV) for _ in range(n_streams)]
+        got = frame(streams)
+        for a, b in zip(ref[:3], got[:3]):
+            assert torch.equal(a, b)
+        for ga, gb in zip(ref[3], got[3]):
+            for a, b in zip(ga, gb):
+                # float atomics commute only up to rounding; two one-stream runs differ as much
+                assert rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-4
