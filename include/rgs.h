@@ -106,6 +106,20 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
                      int* radii, void* geom_ws, size_t geom_bytes,
                      uint32_t* num_rendered_host, void* stream, int debug);
 
+/* rgs_forward_geom without the wait: enqueues the same work and the copy of R to
+ * *num_rendered_pinned, which must be pinned host memory, and returns.  The caller reads R
+ * after the stream (or an event recorded behind this call) has completed.  The reference
+ * has no counterpart (it always blocks, rasterizer_impl.cu:287); this is for a caller that
+ * renders several submodels of a frame on separate streams and wants every geometry stage
+ * in flight before it waits for the first count. */
+int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
+                     const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
+                     const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                     const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                     float tan_fovx, float tan_fovy, int prefiltered,
+                     int* radii, void* geom_ws, size_t geom_bytes,
+                     uint32_t* num_rendered_pinned, void* stream, int debug);
+
 /* Second half of Rasterizer::forward (rasterizer_impl.cu:289-351): key duplication,
  * stable sort of the (tile | depth) keys, tile ranges and the per-tile blend with the
  * per-pixel submodel-box test.  R is the value rgs_forward_geom reported.

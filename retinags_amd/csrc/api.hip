@@ -295,13 +295,13 @@ int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const
 	return 0;
 }
 
-int rgs_forward_geom(int P, int D, int M, int width, int height,
-                     const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
-                     const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
-                     const float* viewmatrix, const float* projmatrix, const float* cam_pos,
-                     float tan_fovx, float tan_fovy, int prefiltered,
-                     int* radii, void* geom_ws, size_t geom_bytes,
-                     uint32_t* num_rendered_host, void* stream, int debug)
+static int forward_geom(bool wait_for_count, const char* who, int P, int D, int M, int width, int height,
+                        const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
+                        const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                        const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                        float tan_fovx, float tan_fovy, int prefiltered,
+                        int* radii, void* geom_ws, size_t geom_bytes,
+                        uint32_t* num_rendered_host, void* stream, int debug)
 {
 	// `prefiltered` promises that no Gaussian is culled; the reference traps the device when
 	// the promise is broken (K/cuda_rasterizer_hgs/auxiliary.h:172-176).  Here a culled
@@ -309,19 +309,19 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
 	(void)prefiltered;
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
-	RGS_REQUIRE(P > 0, "rgs_forward_geom: P must be positive (the caller short-circuits P == 0)");
-	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_geom: bad image size %dx%d", width, height);
+	RGS_REQUIRE(P > 0, "%s: P must be positive (the caller short-circuits P == 0)", who);
+	RGS_REQUIRE(width > 0 && height > 0, "%s: bad image size %dx%d", who, width, height);
 	RGS_REQUIRE(means3D && opacities && viewmatrix && projmatrix && cam_pos && radii && geom_ws && num_rendered_host,
-	            "rgs_forward_geom: null pointer");
+	            "%s: null pointer", who);
 	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr),
-	            "rgs_forward_geom: provide exactly one of SHs or precomputed colours");
+	            "%s: provide exactly one of SHs or precomputed colours", who);
 	RGS_REQUIRE(((scales != nullptr) && (rotations != nullptr)) != (cov3D_precomp != nullptr) &&
 	                ((scales != nullptr) == (rotations != nullptr)),
-	            "rgs_forward_geom: provide exactly one of scale/rotation or precomputed 3D covariance");
-	RGS_REQUIRE(D >= 0 && D <= 3, "rgs_forward_geom: SH degree %d out of range", D);
-	RGS_REQUIRE(!shs || M >= (D + 1) * (D + 1), "rgs_forward_geom: %d SH coefficients cannot hold degree %d", M, D);
-	RGS_REQUIRE(geom_bytes >= rgs_geom_bytes(P), "rgs_forward_geom: geometry workspace too small");
-	RGS_REQUIRE((reinterpret_cast<uintptr_t>(geom_ws) & 15) == 0, "rgs_forward_geom: workspace must be 16-byte aligned");
+	            "%s: provide exactly one of scale/rotation or precomputed 3D covariance", who);
+	RGS_REQUIRE(D >= 0 && D <= 3, "%s: SH degree %d out of range", who, D);
+	RGS_REQUIRE(!shs || M >= (D + 1) * (D + 1), "%s: %d SH coefficients cannot hold degree %d", who, M, D);
+	RGS_REQUIRE(geom_bytes >= rgs_geom_bytes(P), "%s: geometry workspace too small", who);
+	RGS_REQUIRE((reinterpret_cast<uintptr_t>(geom_ws) & 15) == 0, "%s: workspace must be 16-byte aligned", who);
 
 	size_t off[RGS_GEOM_FIELDS];
 	geom_layout((size_t)P, off);
@@ -358,14 +358,42 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
 
 	hipError_t e = hipMemcpyAsync(num_rendered_host, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), sizeof(uint32_t),
 	                              hipMemcpyDeviceToHost, s);
-	if (e == hipSuccess)
+	if (e == hipSuccess && wait_for_count)
 		e = hipStreamSynchronize(s);
 	if (e != hipSuccess)
-		return fail("rgs_forward_geom: reading the instance count failed: %s", hipGetErrorString(e));
-	RGS_REQUIRE(*num_rendered_host < 0x40000000u,
-	            "rgs_forward_geom: %u (Gaussian, tile) instances exceed the 2^30 limit of the sort", *num_rendered_host);
+		return fail("%s: reading the instance count failed: %s", who, hipGetErrorString(e));
+	if (wait_for_count)
+		RGS_REQUIRE(*num_rendered_host < 0x40000000u,
+		            "%s: %u (Gaussian, tile) instances exceed the 2^30 limit of the sort", who, *num_rendered_host);
 	return 0;
 }
+
+int rgs_forward_geom(int P, int D, int M, int width, int height,
+                     const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
+                     const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                     const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                     float tan_fovx, float tan_fovy, int prefiltered,
+                     int* radii, void* geom_ws, size_t geom_bytes,
+                     uint32_t* num_rendered_host, void* stream, int debug)
+{
+	return forward_geom(true, "rgs_forward_geom", P, D, M, width, height, means3D, shs, colors_precomp, opacities, scales,
+	                    scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, cam_pos, tan_fovx, tan_fovy,
+	                    prefiltered, radii, geom_ws, geom_bytes, num_rendered_host, stream, debug);
+}
+
+int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
+                             const float* means3D, const float* shs, const float* colors_precomp,
+                             const float* opacities, const float* scales, float scale_modifier, const float* rotations,
+                             const float* cov3D_precomp, const float* viewmatrix, const float* projmatrix,
+                             const float* cam_pos, float tan_fovx, float tan_fovy, int prefiltered,
+                             int* radii, void* geom_ws, size_t geom_bytes,
+                             uint32_t* num_rendered_pinned, void* stream, int debug)
+{
+	return forward_geom(false, "rgs_forward_geom_enqueue", P, D, M, width, height, means3D, shs, colors_precomp, opacities,
+	                    scales, scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, cam_pos, tan_fovx,
+	                    tan_fovy, prefiltered, radii, geom_ws, geom_bytes, num_rendered_pinned, stream, debug);
+}
+
 
 int rgs_forward_raster(int P, int R, int width, int height,
                        const float* background, float tan_fovx, float tan_fovy,
@@ -378,6 +406,7 @@ int rgs_forward_raster(int P, int R, int width, int height,
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
 	RGS_REQUIRE(P > 0 && R >= 0, "rgs_forward_raster: bad sizes P=%d R=%d", P, R);
+	RGS_REQUIRE(R < 0x40000000, "rgs_forward_raster: %d (Gaussian, tile) instances exceed the 2^30 limit of the sort", R);
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_raster: bad image size %dx%d", width, height);
 	RGS_REQUIRE(background && projmatrix_inv && range_low && range_up && radii && geom_ws && image_ws && out_color &&
 	                out_depth && out_alpha,

@@ -74,16 +74,29 @@ def raster_settings(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
 
 
 def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0,
-                    debug: bool = False) -> dict:
+                    debug: bool = False, started=None) -> dict:
     """Same call sequence and return dict as render4renderinfo
-    (gaussian_renderer/render_half_gs.py:112-182)."""
-    rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug))
+    (gaussian_renderer/render_half_gs.py:112-182).  `started` is what start_submodel returned
+    for the same submodel, if its geometry stage is already in flight."""
+    if started is None:
+        rasterizer, geometry = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug)), None
+    else:
+        rasterizer, geometry = started
     means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
     color, radii, depth, alpha = rasterizer(
         means3D=sub.means3D, means2D=means2D, shs=sub.shs, colors_precomp=None, opacities=sub.opacity,
-        scales=sub.scales, rotations=sub.rotations, cov3D_precomp=None)
+        scales=sub.scales, rotations=sub.rotations, cov3D_precomp=None, geometry=geometry)
     return {"render": color, "viewspace_points": means2D, "visibility_filter": radii > 0, "radii": radii,
             "depth": depth, "alpha": alpha, "num_rendered": -1}
+
+
+def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0, debug: bool = False):
+    """Enqueues the geometry stage of a submodel's forward on the current stream without waiting
+    for its instance count; hand the result to render_submodel(..., started=...)."""
+    rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug))
+    geometry = rasterizer.enqueue_geometry(means3D=sub.means3D, opacities=sub.opacity, shs=sub.shs,
+                                           scales=sub.scales, rotations=sub.rotations)
+    return rasterizer, geometry
 
 
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
@@ -96,7 +109,9 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     same independence is offered to the hardware through `streams`: submodel k is rendered on
     streams[k % len(streams)] (default priority), so one submodel's short kernels and the tail
     of its blend run beside another's; autograd replays each submodel's backward on the stream
-    its forward used.  The compositor runs on the caller's stream after all of them.
+    its forward used.  The compositor runs on the caller's stream after all of them.  The
+    forward is issued in two rounds (all geometry stages, then all sort-and-blend stages): the
+    host has to read each submodel's instance count in between, and this way it waits once.
     """
     device = subs[0].means3D.device
     if submodel_bg is None:
@@ -105,13 +120,17 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     if not streams:
         partial = {m: render_submodel(cam, subs[m], submodel_bg) for m in related}
     else:
+        # every geometry stage is enqueued before the host waits for the first instance count
         main = torch.cuda.current_stream(device)
-        partial = {}
+        partial, started = {}, {}
         for k, m in enumerate(related):
             side = streams[k % len(streams)]
             side.wait_stream(main)
             with torch.cuda.stream(side):
-                partial[m] = render_submodel(cam, subs[m], submodel_bg)
+                started[m] = start_submodel(cam, subs[m], submodel_bg)
+        for k, m in enumerate(related):
+            with torch.cuda.stream(streams[k % len(streams)]):
+                partial[m] = render_submodel(cam, subs[m], submodel_bg, started=started[m])
         for side in streams[:len(related)]:
             main.wait_stream(side)
         for res in partial.values():

@@ -72,66 +72,120 @@ def _stream_ptr(device) -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def _rasterize_forward(bg, means3D, colors_precomp, opacities, scales, rotations, scale_modifier, cov3Ds_precomp,
-                       viewmatrix, projmatrix, projmatrix_inv, range_low, range_up, tanfovx, tanfovy, image_height,
-                       image_width, sh, sh_degree, campos, prefiltered, debug):
-    """Counterpart of RasterizeGaussiansCUDA_hgs (K/rasterize_points.cu:35-125): allocates the
-    outputs and the three workspaces, runs the forward, returns the same 8-tuple."""
+class GeometryStage:
+    """What the first half of a forward call leaves behind: the geometry workspace, the
+    radii and the place where the instance count lands.  Produced by
+    GaussianRasterizer.enqueue_geometry, consumed once by GaussianRasterizer.forward."""
+
+    __slots__ = ("device", "stream", "P", "H", "W", "tensors", "settings", "radii", "geomBuffer", "geom_bytes",
+                 "count", "event", "source", "used")
+
+    def matches(self, means3D, raster_settings) -> bool:
+        return (self.source == (means3D.data_ptr(), int(means3D.shape[0])) and self.settings is raster_settings
+                and not self.used)
+
+
+_free_pinned_words = []
+
+
+def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations, scale_modifier, cov3Ds_precomp,
+                      viewmatrix, projmatrix, projmatrix_inv, range_low, range_up, tanfovx, tanfovy, image_height,
+                      image_width, sh, sh_degree, campos, prefiltered, debug, wait=True):
+    """First half of RasterizeGaussiansCUDA_hgs (K/rasterize_points.cu:35-125): argument checks,
+    the geometry workspace, per-Gaussian preprocess and the instance count.  With wait=False the
+    count is still on its way when this returns."""
     if means3D.ndim != 2 or means3D.shape[1] != 3:
         raise RuntimeError("means3D must have dimensions (num_points, 3)")
     if not means3D.is_cuda:
         raise RuntimeError("the rasterizer needs its inputs on a GPU (device memory)")
     device = means3D.device
-    P, H, W = int(means3D.shape[0]), int(image_height), int(image_width)
+    st = GeometryStage()
+    st.device = device
+    st.source = (means3D.data_ptr(), int(means3D.shape[0]))
+    st.used = False
+    st.P, st.H, st.W = int(means3D.shape[0]), int(image_height), int(image_width)
+    st.stream = torch.cuda.current_stream(device).cuda_stream
+    st.settings = None
+    st.event = None
+    st.count = None
+    byte = dict(dtype=torch.uint8, device=device)
+    st.radii = torch.empty((st.P,), dtype=torch.int32, device=device)
+    names = ("means3D", "colors_precomp", "opacities", "scales", "rotations", "cov3Ds_precomp", "sh", "bg",
+             "viewmatrix", "projmatrix", "projmatrix_inv", "range_low", "range_up", "campos")
+    values = (means3D, colors_precomp, opacities, scales, rotations, cov3Ds_precomp, sh, bg, viewmatrix, projmatrix,
+              projmatrix_inv, range_low, range_up, campos)
+    st.tensors = {n: _dev_f32(v, device, n) for n, v in zip(names, values)}
+    st.tensors.update(tanfovx=float(tanfovx), tanfovy=float(tanfovy), debug=int(bool(debug)))
+    if st.P == 0:
+        st.geomBuffer, st.geom_bytes = torch.empty(0, **byte), 0
+        return st
+    t = st.tensors
+    M = int(t["sh"].shape[1]) if t["sh"].numel() != 0 else 0
+    with torch.cuda.device(device):
+        st.geom_bytes = lib.rgs_geom_bytes(st.P)
+        st.geomBuffer = torch.empty(st.geom_bytes, **byte)
+        if wait:
+            st.count = _pinned_word(device)
+            entry = lib.rgs_forward_geom
+        else:
+            st.count = _free_pinned_words.pop() if _free_pinned_words else torch.zeros(1, dtype=torch.int32).pin_memory()
+            entry = lib.rgs_forward_geom_enqueue
+        check(entry(
+            st.P, int(sh_degree), M, st.W, st.H, ptr(t["means3D"]), ptr(t["sh"]), ptr(t["colors_precomp"]),
+            ptr(t["opacities"]), ptr(t["scales"]), float(scale_modifier), ptr(t["rotations"]),
+            ptr(t["cov3Ds_precomp"]), ptr(t["viewmatrix"]), ptr(t["projmatrix"]), ptr(t["campos"]), float(tanfovx),
+            float(tanfovy), int(bool(prefiltered)), ptr(st.radii), ptr(st.geomBuffer), st.geom_bytes,
+            C.c_void_p(st.count.data_ptr()), C.c_void_p(st.stream), int(bool(debug))))
+        if not wait:
+            st.event = torch.cuda.Event()
+            st.event.record(torch.cuda.current_stream(device))
+    return st
+
+
+def _forward_blend(st: GeometryStage):
+    """Second half: waits for the instance count if it is still on its way, sizes the binning
+    workspace with it, sorts and blends.  Returns the 8-tuple of K/rasterize_points.cu:124."""
+    device, P, H, W = st.device, st.P, st.H, st.W
+    if st.used:
+        raise RuntimeError("this geometry stage has already been consumed")
+    st.used = True
     f32 = dict(dtype=torch.float32, device=device)
     byte = dict(dtype=torch.uint8, device=device)
-
+    if torch.cuda.current_stream(device).cuda_stream != st.stream:
+        raise RuntimeError("the geometry stage was enqueued on another stream than the one current now")
     out_color = torch.empty((3, H, W), **f32)
     out_depth = torch.empty((1, H, W), **f32)
     out_alpha = torch.empty((1, H, W), **f32)
-    radii = torch.empty((P,), dtype=torch.int32, device=device)
     if P == 0:
         out_color.zero_(); out_depth.zero_(); out_alpha.zero_()
         empty = torch.empty(0, **byte)
-        return 0, out_color, out_depth, out_alpha, radii, empty, empty, empty
-
-    means3D = _dev_f32(means3D, device, "means3D")
-    colors_precomp = _dev_f32(colors_precomp, device, "colors_precomp")
-    opacities = _dev_f32(opacities, device, "opacities")
-    scales = _dev_f32(scales, device, "scales")
-    rotations = _dev_f32(rotations, device, "rotations")
-    cov3Ds_precomp = _dev_f32(cov3Ds_precomp, device, "cov3Ds_precomp")
-    sh = _dev_f32(sh, device, "sh")
-    bg = _dev_f32(bg, device, "bg")
-    viewmatrix = _dev_f32(viewmatrix, device, "viewmatrix")
-    projmatrix = _dev_f32(projmatrix, device, "projmatrix")
-    projmatrix_inv = _dev_f32(projmatrix_inv, device, "projmatrix_inv")
-    range_low = _dev_f32(range_low, device, "range_low")
-    range_up = _dev_f32(range_up, device, "range_up")
-    campos = _dev_f32(campos, device, "campos")
-    M = int(sh.shape[1]) if sh.numel() != 0 else 0
-
+        return 0, out_color, out_depth, out_alpha, st.radii, empty, empty, empty
+    t = st.tensors
     with torch.cuda.device(device):
-        stream = _stream_ptr(device)
-        geom_bytes = lib.rgs_geom_bytes(P)
+        if st.event is not None:
+            st.event.synchronize()
+            rendered = int(st.count.item())
+            _free_pinned_words.append(st.count)
+            st.event = None
+        else:
+            rendered = int(st.count.item())
+        st.count = None
         image_bytes = lib.rgs_image_bytes(W, H)
-        geomBuffer = torch.empty(geom_bytes, **byte)
         imgBuffer = torch.empty(image_bytes, **byte)
-        count = _pinned_word(device)
-        check(lib.rgs_forward_geom(
-            P, int(sh_degree), M, W, H, ptr(means3D), ptr(sh), ptr(colors_precomp), ptr(opacities), ptr(scales),
-            float(scale_modifier), ptr(rotations), ptr(cov3Ds_precomp), ptr(viewmatrix), ptr(projmatrix), ptr(campos),
-            float(tanfovx), float(tanfovy), int(bool(prefiltered)), ptr(radii), ptr(geomBuffer), geom_bytes,
-            C.c_void_p(count.data_ptr()), stream, int(bool(debug))))
-        rendered = int(count.item())
         binning_bytes = lib.rgs_binning_bytes(rendered) if rendered > 0 else 0
         binningBuffer = torch.empty(binning_bytes, **byte)
         check(lib.rgs_forward_raster(
-            P, rendered, W, H, ptr(bg), float(tanfovx), float(tanfovy), ptr(projmatrix_inv), ptr(range_low),
-            ptr(range_up), ptr(colors_precomp), ptr(radii), ptr(geomBuffer), geom_bytes, ptr(binningBuffer),
-            binning_bytes, ptr(imgBuffer), image_bytes, ptr(out_color), ptr(out_depth), ptr(out_alpha), stream,
-            int(bool(debug))))
-    return rendered, out_color, out_depth, out_alpha, radii, geomBuffer, binningBuffer, imgBuffer
+            P, rendered, W, H, ptr(t["bg"]), t["tanfovx"], t["tanfovy"], ptr(t["projmatrix_inv"]),
+            ptr(t["range_low"]), ptr(t["range_up"]), ptr(t["colors_precomp"]), ptr(st.radii), ptr(st.geomBuffer),
+            st.geom_bytes, ptr(binningBuffer), binning_bytes, ptr(imgBuffer), image_bytes, ptr(out_color),
+            ptr(out_depth), ptr(out_alpha), C.c_void_p(st.stream), t["debug"]))
+    return rendered, out_color, out_depth, out_alpha, st.radii, st.geomBuffer, binningBuffer, imgBuffer
+
+
+def _rasterize_forward(*args):
+    """Counterpart of RasterizeGaussiansCUDA_hgs (K/rasterize_points.cu:35-125): allocates the
+    outputs and the three workspaces, runs the forward, returns the same 8-tuple."""
+    return _forward_blend(_forward_geometry(*args, wait=True))
 
 
 def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, scale_modifier, cov3Ds_precomp,
@@ -212,9 +266,9 @@ def _mark_visible(means3D, viewmatrix, projmatrix):
 
 
 def rasterize_gaussians(means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp,
-                        raster_settings):
+                        raster_settings, geometry=None):
     return _RasterizeGaussians.apply(means3D, means2D, sh, colors_precomp, opacities, scales, rotations,
-                                     cov3Ds_precomp, raster_settings)
+                                     cov3Ds_precomp, raster_settings, geometry)
 
 
 class _RasterizeGaussians(torch.autograd.Function):
@@ -222,7 +276,13 @@ class _RasterizeGaussians(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp,
-                raster_settings):
+                raster_settings, geometry=None):
+        if geometry is not None:
+            if not geometry.matches(means3D, raster_settings):
+                raise RuntimeError("the geometry stage was enqueued for other inputs or settings, or already used")
+            outs = _forward_blend(geometry)
+            return _RasterizeGaussians._finish_forward(ctx, outs, raster_settings, colors_precomp, means3D, scales,
+                                                       rotations, cov3Ds_precomp, sh)
         args = (
             raster_settings.bg, means3D, colors_precomp, opacities, scales, rotations, raster_settings.scale_modifier,
             cov3Ds_precomp, raster_settings.viewmatrix, raster_settings.projmatrix, raster_settings.projmatrix_inv,
@@ -240,6 +300,11 @@ class _RasterizeGaussians(torch.autograd.Function):
                 raise ex
         else:
             outs = _rasterize_forward(*args)
+        return _RasterizeGaussians._finish_forward(ctx, outs, raster_settings, colors_precomp, means3D, scales,
+                                                   rotations, cov3Ds_precomp, sh)
+
+    @staticmethod
+    def _finish_forward(ctx, outs, raster_settings, colors_precomp, means3D, scales, rotations, cov3Ds_precomp, sh):
         num_rendered, color, depth, alpha, radii, geomBuffer, binningBuffer, imgBuffer = outs
 
         ctx.raster_settings = raster_settings
@@ -295,6 +360,7 @@ class _RasterizeGaussians(torch.autograd.Function):
             grad_rotations if rotations.numel() else None,
             grad_cov3Ds_precomp if cov3Ds_precomp.numel() else None,
             None,
+            None,
         )
         return grads
 
@@ -313,10 +379,8 @@ class GaussianRasterizer(nn.Module):
             visible = _mark_visible(positions, raster_settings.viewmatrix, raster_settings.projmatrix)
         return visible
 
-    def forward(self, means3D, means2D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
-                cov3D_precomp=None):
-        raster_settings = self.raster_settings
-
+    @staticmethod
+    def _check_and_fill(shs, colors_precomp, scales, rotations, cov3D_precomp):
         if (shs is None and colors_precomp is None) or (shs is not None and colors_precomp is not None):
             raise Exception('Please provide excatly one of either SHs or precomputed colors!')
 
@@ -334,6 +398,33 @@ class GaussianRasterizer(nn.Module):
             rotations = torch.Tensor([])
         if cov3D_precomp is None:
             cov3D_precomp = torch.Tensor([])
+        return shs, colors_precomp, scales, rotations, cov3D_precomp
 
+    def forward(self, means3D, means2D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
+                cov3D_precomp=None, geometry=None):
+        """As the reference's forward.  `geometry`, if given, is what enqueue_geometry returned for
+        these same inputs: the call then only waits for that stage and goes on from there."""
+        raster_settings = self.raster_settings
+        shs, colors_precomp, scales, rotations, cov3D_precomp = self._check_and_fill(
+            shs, colors_precomp, scales, rotations, cov3D_precomp)
         return rasterize_gaussians(means3D, means2D, shs, colors_precomp, opacities, scales, rotations, cov3D_precomp,
-                                   raster_settings)
+                                   raster_settings, geometry)
+
+    def enqueue_geometry(self, means3D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
+                         cov3D_precomp=None) -> GeometryStage:
+        """Starts the first half of a forward call (preprocess and instance count) on the current
+        stream and returns without waiting for it.  No counterpart in the reference, whose forward
+        always blocks on the count (K/cuda_rasterizer_hgs/rasterizer_impl.cu:287): a caller that
+        renders several submodels on separate streams enqueues every geometry stage first and
+        then calls forward(..., geometry=stage) for each, on the stream the stage was enqueued
+        on, so that the host's wait for one count no longer holds back the other submodels."""
+        rs = self.raster_settings
+        shs, colors_precomp, scales, rotations, cov3D_precomp = self._check_and_fill(
+            shs, colors_precomp, scales, rotations, cov3D_precomp)
+        with torch.no_grad():
+            stage = _forward_geometry(
+                rs.bg, means3D, colors_precomp, opacities, scales, rotations, rs.scale_modifier, cov3D_precomp,
+                rs.viewmatrix, rs.projmatrix, rs.projmatrix_inv, rs.range_low, rs.range_up, rs.tanfovx, rs.tanfovy,
+                rs.image_height, rs.image_width, shs, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, wait=False)
+        stage.settings = rs
+        return stage

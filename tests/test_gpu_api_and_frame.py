@@ -211,3 +211,28 @@ def test_frame_on_several_streams_matches_one_stream():
             for a, b in zip(ga, gb):
                 # float atomics commute only up to rounding; two one-stream runs differ as much
                 assert rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-4
+
+
+def test_enqueued_geometry_stage_gives_the_same_forward_and_is_checked():
+    """forward(..., geometry=stage) continues a stage started by enqueue_geometry: same outputs
+    as the one-call forward, bit for bit; a stage cannot be used twice or for other inputs."""
+    from retinags_amd import GaussianRasterizer
+    scene, cam, low, up = _small_inputs(n=4000, seed=11)
+    r = GaussianRasterizer(_settings(oracle_settings(cam, low, up, torch.tensor([0.1, 0.2, 0.3]))))
+    kw = dict(means3D=scene["xyz"].to(DEV), opacities=scene["opacity"].to(DEV), shs=scene["shs"].to(DEV),
+              scales=scene["scales"].to(DEV), rotations=scene["rotations"].to(DEV))
+    m2d = torch.zeros_like(kw["means3D"])
+    ref = r(means2D=m2d, **kw)
+    stage = r.enqueue_geometry(**kw)
+    got = r(means2D=m2d, geometry=stage, **kw)
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError):
+        r(means2D=m2d, geometry=stage, **kw)  # already consumed
+    stage2 = r.enqueue_geometry(**kw)
+    other = dict(kw, means3D=kw["means3D"].clone())
+    with pytest.raises(RuntimeError):
+        r(means2D=m2d, geometry=stage2, **other)  # enqueued for another tensor
+    got2 = r(means2D=m2d, geometry=stage2, **kw)  # the refused call did not consume it
+    assert torch.equal(ref[0], got2[0])
+    torch.cuda.synchronize()
