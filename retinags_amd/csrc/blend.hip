@@ -427,10 +427,10 @@ struct BackwardPixel {
 };
 
 struct BackwardStage {  // wave-private
-	float4 geom[kChunk + 4];
-	float4 conic[kChunk + 4];
+	float4 geom[kChunk + 3];  // + padding up to a multiple of four entries
+	float4 conic[kChunk + 3];
 	float4 cd[kChunk];
-	uint32_t entry[kChunk + 4];  // 0-based position in the tile list
+	uint32_t entry[kChunk + 3];  // 0-based position in the tile list
 	uint32_t id[kChunk];
 	float u[kRows * kRowStride];   // [row][row_column(pixel)]
 	float at[kRows * kRowStride];  // [row][row_column(pixel)]
@@ -626,10 +626,6 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	uint32_t id_next = (uint32_t)(kChunk + lane) < span ? list[span - 1 - (kChunk + lane)] : 0u;
 
 	for (uint32_t first = 0; first < span; first += kChunk) {
-		const uint32_t e1 = first + kChunk + lane, e2 = first + 2 * kChunk + lane;
-		LoadedEntry nxt = load_entry(a, id_next, e1 < span);
-		id_next = e2 < span ? list[span - 1 - e2] : 0u;
-
 		const bool filed = file_entry(cur, strip_x0, strip_y0, sc, box);
 		const uint64_t m = __ballot(filed);
 		const int count = __popcll(m);
@@ -641,12 +637,16 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			st.entry[slot] = span - 1 - (first + lane);
 			st.id[slot] = cur.id;
 		}
-		if (lane < 4) {
+		if (lane < 3) {
 			st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
 			st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
 			st.entry[count + lane] = 0xFFFFFFFFu;
 		}
 		__builtin_amdgcn_wave_barrier();
+		// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
+		const uint32_t e1 = first + kChunk + lane, e2 = first + 2 * kChunk + lane;
+		cur = load_entry(a, id_next, e1 < span);
+		id_next = e2 < span ? list[span - 1 - e2] : 0u;
 
 		for (int k = 0; k < count; k += 4) {
 			const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
@@ -667,8 +667,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, box, lane);
 		}
 		__builtin_amdgcn_wave_barrier();
-		keep_padding_registers(nxt);
-		cur = nxt;
+		keep_padding_registers(cur);
 	}
 	if (rows > 0)
 		flush_rows(st, rows, frame, a, lane);
