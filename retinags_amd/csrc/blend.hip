@@ -565,12 +565,13 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	}
 }
 
-__global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
+__global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 {
-	__shared__ BackwardStage s_stage[4];
+	__shared__ BackwardStage s_stage;
 
-	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const int tile = tile_of_block((int)blockIdx.x, a.grid_x, a.grid_y);
+	const int lane = threadIdx.x;
+	int wave;  // which strip of the tile
+	const int tile = tile_of_strip_block((int)blockIdx.x, a.grid_x, a.grid_y, wave);
 	if (tile < 0)
 		return;
 	const uint2 range = a.ranges[tile];
@@ -586,7 +587,7 @@ __global__ __launch_bounds__(256) void blend_backward_kernel(BlendArgs a)
 	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
 	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
 	const StripFrame frame = {strip_x0, strip_y0, (float)(0.5 * a.W), (float)(0.5 * a.H)};
-	BackwardStage& st = s_stage[wave];
+	BackwardStage& st = s_stage;
 	const uint64_t below = (1ull << lane) - 1ull;
 
 	if (range.y == range.x)
@@ -685,7 +686,7 @@ void launch_blend_forward(const BlendArgs& a, hipStream_t s)
 void launch_blend_backward(const BlendArgs& a, hipStream_t s)
 {
 	stage_mark("blend_backward", s);
-	hipLaunchKernelGGL(blend_backward_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
+	hipLaunchKernelGGL(blend_backward_kernel, dim3(strip_order_blocks(a.grid_x, a.grid_y)), dim3(64), 0, s, a);
 }
 
 }  // namespace rgs
