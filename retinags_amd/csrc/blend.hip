@@ -137,7 +137,8 @@ __device__ __forceinline__ int classify_strip_against_box(float w, const StripCo
 	return outside ? kBoxOutside : (inside ? kBoxInside : kBoxMixed);
 }
 
-constexpr int kChunk = 64;  // list entries a wavefront takes per step, one per lane
+constexpr int kPerLane = 1;             // list entries per lane and step (2 was measured slower)
+constexpr int kChunk = 64 * kPerLane;   // list entries a wavefront takes per step
 
 // One entry of the tile list as a lane holds it between the load and the filter.
 struct LoadedEntry {
@@ -202,8 +203,8 @@ struct ForwardPixel {
 };
 
 struct ForwardStage {  // wave-private
-	float4 geom[kChunk + 4];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
-	float4 conic[kChunk + 4];  // conic xx, xy, yy, opacity
+	float4 geom[kChunk + 3];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
+	float4 conic[kChunk + 3];  // conic xx, xy, yy, opacity
 	float4 cd[kChunk];         // r, g, b, view depth
 	uint32_t position[kChunk]; // 1-based position in the tile list
 };
@@ -264,30 +265,44 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 
 	if (n != 0u && live != 0ull) {
 		const uint32_t* list = a.point_list + range.x;
-		// two chunks of ids and one chunk of records are always in flight ahead of the walk
-		LoadedEntry cur = load_entry(a, (uint32_t)lane < n ? list[lane] : 0u, (uint32_t)lane < n);
-		uint32_t id_next = (uint32_t)(kChunk + lane) < n ? list[kChunk + lane] : 0u;
+		// lane l holds entries first + 64 e + l (e < kPerLane) of the chunk; the next chunk's records
+		// and the ids of the chunk after it are in flight while the current one is walked
+		LoadedEntry cur[kPerLane];
+		uint32_t id_next[kPerLane];
+#pragma unroll
+		for (int e = 0; e < kPerLane; e++) {
+			const uint32_t i0 = 64 * e + lane, i1 = kChunk + i0;
+			cur[e] = load_entry(a, i0 < n ? list[i0] : 0u, i0 < n);
+			id_next[e] = i1 < n ? list[i1] : 0u;
+		}
 
 		for (uint32_t first = 0; first < n && live != 0ull; first += kChunk) {
-			const uint32_t e1 = first + kChunk + lane, e2 = first + 2 * kChunk + lane;
-			LoadedEntry nxt = load_entry(a, id_next, e1 < n);
-			id_next = e2 < n ? list[e2] : 0u;
-
-			const bool filed = file_entry(cur, strip_x0, strip_y0, sc, box);
-			const uint64_t m = __ballot(filed);
-			const int count = __popcll(m);
-			if (filed) {
-				const int slot = __popcll(m & below);
-				st.geom[slot] = cur.geom;
-				st.conic[slot] = cur.conic;
-				st.cd[slot] = cur.cd;
-				st.position[slot] = first + lane + 1;
+			int count = 0;
+#pragma unroll
+			for (int e = 0; e < kPerLane; e++) {
+				const bool filed = file_entry(cur[e], strip_x0, strip_y0, sc, box);
+				const uint64_t m = __ballot(filed);
+				if (filed) {
+					const int slot = count + __popcll(m & below);
+					st.geom[slot] = cur[e].geom;
+					st.conic[slot] = cur[e].conic;
+					st.cd[slot] = cur[e].cd;
+					st.position[slot] = first + 64 * e + lane + 1;
+				}
+				count += __popcll(m);
 			}
-			if (lane < 4) {  // pad to a multiple of four with entries that never pass the floor test
+			if (lane < 3) {  // pad to a multiple of four with entries that never pass the floor test
 				st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
 				st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
 			}
 			__builtin_amdgcn_wave_barrier();
+			// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
+#pragma unroll
+			for (int e = 0; e < kPerLane; e++) {
+				const uint32_t i1 = first + kChunk + 64 * e + lane, i2 = i1 + kChunk;
+				cur[e] = load_entry(a, id_next[e], i1 < n);
+				id_next[e] = i2 < n ? list[i2] : 0u;
+			}
 
 			for (int k = 0; k < count && live != 0ull; k += 4) {
 				const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
@@ -307,8 +322,9 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				live = __ballot(!p.done);
 			}
 			__builtin_amdgcn_wave_barrier();
-			keep_padding_registers(nxt);
-		cur = nxt;
+#pragma unroll
+			for (int e = 0; e < kPerLane; e++)
+				keep_padding_registers(cur[e]);
 		}
 	}
 
@@ -621,22 +637,32 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 	st.upstream[3][row_column(lane)] = p.g_depth;
 	int rows = 0;
 
-	// lane l of the chunk starting `first` entries from the back takes list position span-1-first-l
+	// lane l holds the entries first + 64 e + l from the back (list position span-1-that), e < kPerLane
 	const uint32_t* list = a.point_list + range.x;
-	LoadedEntry cur = load_entry(a, (uint32_t)lane < span ? list[span - 1 - lane] : 0u, (uint32_t)lane < span);
-	uint32_t id_next = (uint32_t)(kChunk + lane) < span ? list[span - 1 - (kChunk + lane)] : 0u;
+	LoadedEntry cur[kPerLane];
+	uint32_t id_next[kPerLane];
+#pragma unroll
+	for (int e = 0; e < kPerLane; e++) {
+		const uint32_t i0 = 64 * e + lane, i1 = kChunk + i0;
+		cur[e] = load_entry(a, i0 < span ? list[span - 1 - i0] : 0u, i0 < span);
+		id_next[e] = i1 < span ? list[span - 1 - i1] : 0u;
+	}
 
 	for (uint32_t first = 0; first < span; first += kChunk) {
-		const bool filed = file_entry(cur, strip_x0, strip_y0, sc, box);
-		const uint64_t m = __ballot(filed);
-		const int count = __popcll(m);
-		if (filed) {
-			const int slot = __popcll(m & below);
-			st.geom[slot] = cur.geom;
-			st.conic[slot] = cur.conic;
-			st.cd[slot] = cur.cd;
-			st.entry[slot] = span - 1 - (first + lane);
-			st.id[slot] = cur.id;
+		int count = 0;
+#pragma unroll
+		for (int e = 0; e < kPerLane; e++) {
+			const bool filed = file_entry(cur[e], strip_x0, strip_y0, sc, box);
+			const uint64_t m = __ballot(filed);
+			if (filed) {
+				const int slot = count + __popcll(m & below);
+				st.geom[slot] = cur[e].geom;
+				st.conic[slot] = cur[e].conic;
+				st.cd[slot] = cur[e].cd;
+				st.entry[slot] = span - 1 - (first + 64 * e + lane);
+				st.id[slot] = cur[e].id;
+			}
+			count += __popcll(m);
 		}
 		if (lane < 3) {
 			st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
@@ -645,9 +671,12 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 		}
 		__builtin_amdgcn_wave_barrier();
 		// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
-		const uint32_t e1 = first + kChunk + lane, e2 = first + 2 * kChunk + lane;
-		cur = load_entry(a, id_next, e1 < span);
-		id_next = e2 < span ? list[span - 1 - e2] : 0u;
+#pragma unroll
+		for (int e = 0; e < kPerLane; e++) {
+			const uint32_t i1 = first + kChunk + 64 * e + lane, i2 = i1 + kChunk;
+			cur[e] = load_entry(a, id_next[e], i1 < span);
+			id_next[e] = i2 < span ? list[span - 1 - i2] : 0u;
+		}
 
 		for (int k = 0; k < count; k += 4) {
 			const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
@@ -668,7 +697,9 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, box, lane);
 		}
 		__builtin_amdgcn_wave_barrier();
-		keep_padding_registers(cur);
+#pragma unroll
+		for (int e = 0; e < kPerLane; e++)
+			keep_padding_registers(cur[e]);
 	}
 	if (rows > 0)
 		flush_rows(st, rows, frame, a, lane);
