@@ -105,7 +105,10 @@ def main():
     related = [m for m in range(len(subs)) if rel[m] >= 0]
     setup_s = time.time() - t0
 
-    streams = [torch.cuda.Stream(device=dev) for _ in range(args.streams)] if args.streams > 0 else None
+    # the current stream counts as one of them: a process has 4 hardware queues here, and a fifth
+    # stream would share a queue with another, which serialises the two
+    streams = ([torch.cuda.current_stream(dev)] + [torch.cuda.Stream(device=dev) for _ in range(args.streams - 1)]
+               if args.streams > 0 else None)
 
     def step(streams=streams):
         for s in subs:
