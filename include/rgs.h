@@ -53,18 +53,24 @@ enum {
 	RGS_GEOM_CONIC_OPACITY,     /* float4[P] */
 	RGS_GEOM_RGB,               /* float[3P] */
 	RGS_GEOM_TILES_TOUCHED,     /* uint32[P] */
-	RGS_GEOM_POINT_OFFSETS,     /* uint32[P]  inclusive prefix sum of tiles_touched */
+	RGS_GEOM_POINT_OFFSETS,     /* uint32[P]  inclusive prefix sum of the tile counts of the Gaussians in
+	                               RGS_GEOM_DEPTH_ORDER (as many entries as that has) */
 	RGS_GEOM_CLAMPED,           /* uint8[P]   bit c set: colour channel c was clamped at 0 */
 	RGS_GEOM_BLOCK_SUMS,        /* uint32[ceil(P/256)+1] */
 	RGS_GEOM_TOTAL,             /* uint32     number of (Gaussian, tile) instances */
 	RGS_GEOM_BLEND_RECORD,      /* float[16P] one 64-byte record per Gaussian with everything the blend reads:
 	                               x, y, exponent floor, clip w | conic xx, xy, yy, opacity | r, g, b, depth |
 	                               half-width, half-height of the alpha >= 1/255 ellipse's bounding box, 0, 0 */
+	RGS_GEOM_DEPTH_ORDER,       /* uint32[P]  the Gaussians that touch a tile by increasing depth, ties by index;
+	                               entries from RGS_GEOM_VISIBLE_COUNT on are unused */
+	RGS_GEOM_BLOCK_VISIBLE,     /* uint32[ceil(P/256)+1] */
+	RGS_GEOM_VISIBLE_COUNT,     /* uint32     number of Gaussians that touch a tile */
+	RGS_GEOM_ORDER_SCRATCH,     /* scratch of the depth sort */
 	RGS_GEOM_FIELDS
 };
 enum {
-	RGS_BIN_KEYS_UNSORTED = 0,  /* uint64[R]  (tile << 32) | depth bits, emission order */
-	RGS_BIN_KEYS_SORTED,        /* uint64[R] */
+	RGS_BIN_KEYS_UNSORTED = 0,  /* uint32[R]  tile of each instance, emitted Gaussian after Gaussian in depth order */
+	RGS_BIN_KEYS_SORTED,        /* uint32[R]  the same after the stable sort by tile */
 	RGS_BIN_VALUES_UNSORTED,    /* uint32[R]  Gaussian index */
 	RGS_BIN_VALUES_SORTED,      /* uint32[R]  the per-tile Gaussian lists, tile after tile */
 	RGS_BIN_SORT_TEMP,          /* uint32[..] */

@@ -13,7 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RGS_LIBRARY") or os.path.join(_HERE, "librgs_gfx950.so")
 
 GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles_touched", "point_offsets",
-               "clamped", "block_sums", "total", "blend_record")
+               "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
+               "order_scratch")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
 IMG_FIELDS = ("ranges", "n_contrib")
 ACC_FLOATS = 12

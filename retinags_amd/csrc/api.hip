@@ -99,6 +99,25 @@ struct Carver {
 	}
 };
 
+// Scratch of the depth sort of the Gaussians, inside the geometry workspace.
+struct OrderScratch {
+	size_t keys_a, keys_b, vals_b, tiles_in_order, sort_temp, scan_temp, total;
+};
+
+OrderScratch order_scratch(size_t P)
+{
+	Carver c;
+	OrderScratch o;
+	o.keys_a = c.take(4 * P);
+	o.keys_b = c.take(4 * P);
+	o.vals_b = c.take(4 * P);
+	o.tiles_in_order = c.take(4 * P);
+	o.sort_temp = c.take(4 * rgs::sort_temp_words(P));
+	o.scan_temp = c.take(4 * rgs::scan_temp_words(P));
+	o.total = c.cursor;
+	return o;
+}
+
 size_t geom_layout(size_t P, size_t* off)
 {
 	Carver c;
@@ -114,13 +133,18 @@ size_t geom_layout(size_t P, size_t* off)
 	off[RGS_GEOM_BLOCK_SUMS] = c.take(4 * ((P + 255) / 256 + 1));
 	off[RGS_GEOM_TOTAL] = c.take(4);
 	off[RGS_GEOM_BLEND_RECORD] = c.take(64 * P);
+	off[RGS_GEOM_DEPTH_ORDER] = c.take(4 * P);
+	off[RGS_GEOM_BLOCK_VISIBLE] = c.take(4 * ((P + 255) / 256 + 1));
+	off[RGS_GEOM_VISIBLE_COUNT] = c.take(4);
+	off[RGS_GEOM_ORDER_SCRATCH] = c.take(order_scratch(P).total);
 	return c.cursor;
 }
 
-int sort_end_bit(int width, int height)
+// Bits of the tile key that the instance sort looks at.
+int tile_key_bits(int width, int height)
 {
 	const uint32_t tiles = (uint32_t)((width + rgs::kTile - 1) / rgs::kTile) * (uint32_t)((height + rgs::kTile - 1) / rgs::kTile);
-	return 32 + (int)rgs_get_higher_msb(tiles);
+	return (int)rgs_get_higher_msb(tiles);
 }
 
 // Physical buffers: A receives the duplicated keys, B is its ping-pong partner.
@@ -132,8 +156,8 @@ BinningPhysical binning_physical(size_t R)
 {
 	Carver c;
 	BinningPhysical b;
-	b.keys_a = c.take(8 * R);
-	b.keys_b = c.take(8 * R);
+	b.keys_a = c.take(4 * R);
+	b.keys_b = c.take(4 * R);
 	b.vals_a = c.take(4 * R);
 	b.vals_b = c.take(4 * R);
 	b.temp = c.take(4 * rgs::sort_temp_words(R));
@@ -263,7 +287,7 @@ int rgs_binning_layout(int R, int width, int height, size_t offsets[RGS_BIN_FIEL
 {
 	RGS_REQUIRE(R >= 0 && width > 0 && height > 0 && offsets, "rgs_binning_layout: bad arguments");
 	const BinningPhysical b = binning_physical((size_t)R);
-	const bool sorted_in_a = (((sort_end_bit(width, height) + 7) / 8) % 2) == 0;
+	const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
 	offsets[RGS_BIN_KEYS_UNSORTED] = sorted_in_a ? b.keys_b : b.keys_a;
 	offsets[RGS_BIN_KEYS_SORTED] = sorted_in_a ? b.keys_a : b.keys_b;
 	offsets[RGS_BIN_VALUES_UNSORTED] = sorted_in_a ? b.vals_b : b.vals_a;
@@ -349,15 +373,26 @@ static int forward_geom(bool wait_for_count, const char* who, int P, int D, int 
 	a.clamped = at<uint8_t>(geom_ws, off[RGS_GEOM_CLAMPED]);
 	a.block_sums = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_SUMS]);
 	a.blend_record = at<float4>(geom_ws, off[RGS_GEOM_BLEND_RECORD]);
+	a.block_visible = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_VISIBLE]);
 
 	rgs::launch_preprocess_forward(a, s);
 	RGS_STAGE("preprocess");
-	rgs::launch_offsets_from_block_sums(a.tiles_touched, a.block_sums, at<uint32_t>(geom_ws, off[RGS_GEOM_POINT_OFFSETS]),
-	                                    P, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), s);
-	RGS_STAGE("offset scan");
-
+	rgs::launch_total_from_block_sums(a.block_sums, P, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), s);
+	RGS_STAGE("instance count");
 	hipError_t e = hipMemcpyAsync(num_rendered_host, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), sizeof(uint32_t),
 	                              hipMemcpyDeviceToHost, s);
+	{
+		// depth order of the Gaussians and the offsets of their instances in that order: needs
+		// nothing from the host, so it is queued behind the count's copy
+		const OrderScratch o = order_scratch((size_t)P);
+		char* scratch = at<char>(geom_ws, off[RGS_GEOM_ORDER_SCRATCH]);
+		rgs::launch_depth_order(P, a.depths, a.tiles_touched, a.block_visible, at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_COUNT]),
+		                        at<uint32_t>(scratch, o.keys_a), at<uint32_t>(scratch, o.keys_b),
+		                        at<uint32_t>(geom_ws, off[RGS_GEOM_DEPTH_ORDER]), at<uint32_t>(scratch, o.vals_b),
+		                        at<uint32_t>(scratch, o.tiles_in_order), at<uint32_t>(geom_ws, off[RGS_GEOM_POINT_OFFSETS]),
+		                        at<uint32_t>(scratch, o.sort_temp), at<uint32_t>(scratch, o.scan_temp), s);
+		RGS_STAGE("depth order");
+	}
 	if (e == hipSuccess && wait_for_count)
 		e = hipStreamSynchronize(s);
 	if (e != hipSuccess)
@@ -425,30 +460,38 @@ int rgs_forward_raster(int P, int R, int width, int height,
 
 	if (R > 0) {
 		const BinningPhysical b = binning_physical((size_t)R);
-		uint64_t* keys_a = at<uint64_t>(binning_ws, b.keys_a);
-		uint64_t* keys_b = at<uint64_t>(binning_ws, b.keys_b);
+		uint32_t* keys_a = at<uint32_t>(binning_ws, b.keys_a);
+		uint32_t* keys_b = at<uint32_t>(binning_ws, b.keys_b);
 		uint32_t* vals_a = at<uint32_t>(binning_ws, b.vals_a);
 		uint32_t* vals_b = at<uint32_t>(binning_ws, b.vals_b);
-		rgs::launch_duplicate_with_keys(P, at<float2>(geom_ws, goff[RGS_GEOM_XY]), at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]),
-		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_POINT_OFFSETS]), radii, gx, gy, keys_a, vals_a, s);
+		const uint32_t* order_status =
+		    rgs::sort_status_word(at<uint32_t>(at<char>(geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).sort_temp));
+		rgs::launch_duplicate_with_keys(P, at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]),
+		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_DEPTH_ORDER]),
+		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_POINT_OFFSETS]), at<float2>(geom_ws, goff[RGS_GEOM_XY]),
+		                                radii, gx, gy, keys_a, vals_a, s);
 		RGS_STAGE("duplicate_with_keys");
-		const int end_bit = sort_end_bit(width, height);
-		rgs::launch_sort_pairs(keys_a, keys_b, vals_a, vals_b, (size_t)R, end_bit, at<uint32_t>(binning_ws, b.temp), s);
+		const int end_bit = tile_key_bits(width, height);
+		rgs::launch_sort_pairs_u32(keys_a, keys_b, vals_a, vals_b, (size_t)R, nullptr, end_bit, at<uint32_t>(binning_ws, b.temp),
+		                           "sort", s);
 		RGS_STAGE("sort_pairs");
 		const bool sorted_in_a = (((end_bit + 7) / 8) % 2) == 0;
 		if (debug) {
-			uint32_t status = 0;
+			uint32_t status = 0, status2 = 0;
 			hipError_t e = hipMemcpy(&status, rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), sizeof(status),
 			                         hipMemcpyDeviceToHost);
+			if (e == hipSuccess)
+				e = hipMemcpy(&status2, order_status, sizeof(status2), hipMemcpyDeviceToHost);
+			status |= status2;
 			if (e != hipSuccess || status != 0)
 				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
 		}
 		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, ranges, gx * gy,
-		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), s);
+		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, s);
 		RGS_STAGE("tile_ranges");
 		point_list = sorted_in_a ? vals_a : vals_b;
 	} else {
-		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, nullptr, s);
+		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, nullptr, nullptr, s);
 		RGS_STAGE("tile_ranges");
 	}
 
@@ -509,7 +552,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	const float* colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
 	if (R > 0) {
 		const BinningPhysical b = binning_physical((size_t)R);
-		const bool sorted_in_a = (((sort_end_bit(width, height) + 7) / 8) % 2) == 0;
+		const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
 		rgs::BlendArgs a;
 		memset(&a, 0, sizeof(a));
 		a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
@@ -568,7 +611,7 @@ int rgs_blend_work_counters(int P, int R, int width, int height, float tan_fovx,
 	if (R == 0)
 		return 0;
 	const BinningPhysical b = binning_physical((size_t)R);
-	const bool sorted_in_a = (((sort_end_bit(width, height) + 7) / 8) % 2) == 0;
+	const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
 	rgs::BlendArgs a;
 	memset(&a, 0, sizeof(a));
 	a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
@@ -605,7 +648,7 @@ int rgs_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, void* temp, v
 		return 0;
 	RGS_REQUIRE(in && out && temp, "rgs_inclusive_sum: null pointer");
 	RGS_REQUIRE(n < ((size_t)1 << 38), "rgs_inclusive_sum: n too large");
-	rgs::launch_inclusive_sum(in, out, n, static_cast<uint32_t*>(temp), s);
+	rgs::launch_inclusive_sum(in, out, n, static_cast<uint32_t*>(temp), "inclusive_sum", s);
 	RGS_STAGE("inclusive_sum");
 	return 0;
 }

@@ -1,6 +1,18 @@
-// Binning stages: offset scan, (tile | depth) key duplication, stable 64-bit radix
-// sort and per-tile range extraction.  All integer work; results are bit-exact
-// by construction.  K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian.
+// Binning stages: offset scans, depth order of the Gaussians, tile-key duplication, stable
+// radix sorts and per-tile range extraction.  All integer work; results are bit-exact by
+// construction.  K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian.
+//
+// The reference sorts R (Gaussian, tile) instances by the 64-bit key (tile << 32) | depth bits
+// with a stable sort (K/cuda_rasterizer_hgs/rasterizer_impl.cu:300-317): 6 passes over 12-byte
+// pairs at 6 500 tiles.  The same permutation is produced here in two cheaper steps:
+//   1. the P Gaussians are sorted by their depth bits (stable, so equal depths stay in index
+//      order), 4 passes over P 8-byte pairs;
+//   2. instances are emitted in that order with the tile as a 32-bit key and sorted by it
+//      (stable, so every tile keeps depth order, ties in index order), ceil(log2(tiles)/8)
+//      passes over R 8-byte pairs.
+// A stable sort by (tile, depth) of instances emitted in index order and a stable sort by tile
+// of instances emitted in (depth, index) order give the same list: within a tile both order by
+// depth and break ties by Gaussian index (a Gaussian touches a tile at most once).
 #include "rgs_kernels.h"
 
 namespace rgs {
@@ -11,10 +23,14 @@ namespace rgs {
 // and a per-block scan that adds the block's base.  The forward preprocess kernel already
 // emits the block totals, so the rasterizer path only runs the last two.
 
+// In all three kernels a non-null n_device overrides n (the launch is then sized for an upper bound).
 __global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __restrict__ in, size_t n,
+                                                            const uint32_t* __restrict__ n_device,
                                                             uint32_t* __restrict__ totals)
 {
 	__shared__ uint32_t lds[8];
+	if (n_device)
+		n = *n_device;
 	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
 	const uint32_t v = i < n ? in[i] : 0u;
 	uint32_t total;
@@ -26,9 +42,12 @@ __global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __res
 // In-place exclusive scan of `data[0..n)` by one block of 1024 threads; the grand total goes
 // to *total_out (if non-null).
 __global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(uint32_t* __restrict__ data, size_t n,
+                                                                            const uint32_t* __restrict__ n_device,
                                                                             uint32_t* __restrict__ total_out)
 {
 	__shared__ uint32_t wave_tot[16];
+	if (n_device)
+		n = ((size_t)*n_device + 255) / 256;  // one entry per 256 elements
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const size_t chunk = (n + 1023) / 1024;
 	const size_t lo = (size_t)tid * chunk;
@@ -60,9 +79,12 @@ __global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(uint3
 
 __global__ __launch_bounds__(256) void block_inclusive_scan_kernel(const uint32_t* __restrict__ in,
                                                                     const uint32_t* __restrict__ block_base, size_t n,
+                                                                    const uint32_t* __restrict__ n_device,
                                                                     uint32_t* __restrict__ out)
 {
 	__shared__ uint32_t lds[8];
+	if (n_device)
+		n = *n_device;
 	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
 	const uint32_t v = i < n ? in[i] : 0u;
 	uint32_t total;
@@ -76,15 +98,32 @@ size_t scan_temp_words(size_t n)
 	return (n + 255) / 256 + 1;
 }
 
-void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, hipStream_t s)
+static void inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, const uint32_t* n_device, uint32_t* temp,
+                          hipStream_t s)
+{
+	const size_t nb = (n + 255) / 256;
+	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, n_device, temp);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, nb, n_device,
+	                   (uint32_t*)nullptr);
+	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, temp, n, n_device, out);
+}
+
+void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, const char* stage,
+                          hipStream_t s)
 {
 	if (n == 0)
 		return;
-	const size_t nb = (n + 255) / 256;
-	stage_mark("inclusive_sum", s);
-	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, temp);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, nb, (uint32_t*)nullptr);
-	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, temp, n, out);
+	if (stage)
+		stage_mark(stage, s);
+	inclusive_sum(in, out, n, nullptr, temp, s);
+}
+
+void launch_total_from_block_sums(uint32_t* block_sums, int P, uint32_t* total_out, hipStream_t s)
+{
+	const size_t nb = ((size_t)P + 255) / 256;
+	stage_mark("offset_scan", s);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb,
+	                   (const uint32_t*)nullptr, total_out);
 }
 
 void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* block_sums, uint32_t* offsets, int P,
@@ -92,47 +131,95 @@ void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* blo
 {
 	const size_t nb = ((size_t)P + 255) / 256;
 	stage_mark("offset_scan", s);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb, total_out);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb,
+	                   (const uint32_t*)nullptr, total_out);
 	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, tiles_touched, block_sums,
-	                   (size_t)P, offsets);
+	                   (size_t)P, (const uint32_t*)nullptr, offsets);
 }
 
-// ---- key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) ----------------------
+// ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------
 
-__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(int P, const float2* __restrict__ xy,
-                                                                   const float* __restrict__ depths,
+// (depth bits, index) pairs of the Gaussians that touch a tile, compacted in index order:
+// block b of 256 Gaussians writes from visible_base[b] on.  Depths of rendered Gaussians are
+// positive floats (> 0.2), whose bit patterns order like the values.
+__global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __restrict__ depths,
+                                                           const uint32_t* __restrict__ tiles_touched,
+                                                           const uint32_t* __restrict__ visible_base,
+                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ values)
+{
+	__shared__ uint32_t lds[8];
+	const int idx = blockIdx.x * 256 + threadIdx.x;
+	const bool visible = idx < P && tiles_touched[idx] != 0u;
+	uint32_t total;
+	const uint32_t rank = block256_exclusive_scan_u32(visible ? 1u : 0u, lds, total);
+	if (visible) {
+		const uint32_t at = visible_base[blockIdx.x] + rank;
+		keys[at] = __float_as_uint(depths[idx]);
+		values[at] = (uint32_t)idx;
+	}
+}
+
+__global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ n_device,
+                                                          const uint32_t* __restrict__ index,
+                                                          const uint32_t* __restrict__ in, uint32_t* __restrict__ out)
+{
+	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+	if (k < *n_device)
+		out[k] = in[index[k]];
+}
+
+// Thread k takes the k-th Gaussian in depth order and writes its instances, tiles row by row
+// like the reference, at the offsets of the scan taken in that same order.
+__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t* __restrict__ visible_count,
+                                                                   const uint32_t* __restrict__ order,
                                                                    const uint32_t* __restrict__ offsets,
+                                                                   const float2* __restrict__ xy,
                                                                    const int* __restrict__ radii, int gx, int gy,
-                                                                   uint64_t* __restrict__ keys,
+                                                                   uint32_t* __restrict__ keys,
                                                                    uint32_t* __restrict__ values)
 {
-	const int idx = blockIdx.x * 256 + threadIdx.x;
-	if (idx >= P)
+	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+	if (k >= *visible_count)
 		return;
+	const uint32_t idx = order[k];
 	const int radius = radii[idx];
-	if (!(radius > 0))
-		return;
-	uint32_t off = (idx == 0) ? 0u : offsets[idx - 1];
+	uint32_t off = (k == 0) ? 0u : offsets[k - 1];
 	const float2 p = xy[idx];
 	const TileRect rc = tile_rect(p.x, p.y, radius, gx, gy);
-	const uint64_t dbits = (uint64_t)__float_as_uint(depths[idx]);
 	for (uint32_t y = rc.y0; y < rc.y1; y++) {
 		for (uint32_t x = rc.x0; x < rc.x1; x++) {
-			const uint64_t key = ((uint64_t)(y * (uint32_t)gx + x) << 32) | dbits;
-			keys[off] = key;
-			values[off] = (uint32_t)idx;
+			keys[off] = y * (uint32_t)gx + x;
+			values[off] = idx;
 			off++;
 		}
 	}
 }
 
-void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, const uint32_t* offsets,
-                                const int* radii, int grid_x, int grid_y, uint64_t* keys, uint32_t* values,
-                                hipStream_t s)
+void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touched, uint32_t* block_visible,
+                        uint32_t* visible_count, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
+                        uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
+                        hipStream_t s)
+{
+	const unsigned nb = (unsigned)((P + 255) / 256);
+	stage_mark("depth_order", s);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_visible, (size_t)nb,
+	                   (const uint32_t*)nullptr, visible_count);
+	hipLaunchKernelGGL(depth_pairs_kernel, dim3(nb), dim3(256), 0, s, P, depths, tiles_touched, block_visible, keys_a,
+	                   order);
+	// 4 passes: the sorted pairs end up in the first buffer pair again
+	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, nullptr, s);
+	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched,
+	                   tiles_in_order);
+	inclusive_sum(tiles_in_order, offsets_in_order, (size_t)P, visible_count, scan_temp, s);
+}
+
+void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
+                                const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
+                                int grid_y, uint32_t* keys, uint32_t* values, hipStream_t s)
 {
 	stage_mark("duplicate_with_keys", s);
-	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, P, xy, depths, offsets,
-	                   radii, grid_x, grid_y, keys, values);
+	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, visible_count, order,
+	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values);
 }
 
 // ---- radix sort -------------------------------------------------------------------------------
@@ -160,22 +247,27 @@ constexpr uint32_t kFlagInclusive = 2u << 30;  // word holds the count of this a
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
 constexpr int kLookbackSpinLimit = 1 << 18;
 
-__device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t mask)
+template <typename KeyT>
+__device__ __forceinline__ uint32_t digit_of(KeyT key, int shift, uint32_t mask)
 {
 	return (uint32_t)(key >> shift) & mask;
 }
 
-__global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const uint64_t* __restrict__ keys, size_t n,
+template <typename KeyT>
+__global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const KeyT* __restrict__ keys, size_t n,
+                                                                    const uint32_t* __restrict__ n_device,
                                                                     int passes, int end_bit,
                                                                     uint32_t* __restrict__ hist)
 {
 	__shared__ uint32_t s_hist[kSortMaxPasses][256];
+	if (n_device)
+		n = *n_device;
 #pragma unroll
 	for (int p = 0; p < kSortMaxPasses; p++)
 		s_hist[p][threadIdx.x] = 0;
 	__syncthreads();
 	for (size_t k = (size_t)blockIdx.x * 256 + threadIdx.x; k < n; k += (size_t)gridDim.x * 256) {
-		const uint64_t key = keys[k];
+		const KeyT key = keys[k];
 		for (int p = 0; p < passes; p++) {
 			const int shift = 8 * p;
 			const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
@@ -201,16 +293,18 @@ __global__ __launch_bounds__(256) void sort_digit_starts_kernel(uint32_t* __rest
 	}
 }
 
-__global__ __launch_bounds__(256) void sort_onesweep_kernel(const uint64_t* __restrict__ keys_in,
+template <typename KeyT>
+__global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restrict__ keys_in,
                                                              const uint32_t* __restrict__ vals_in,
-                                                             uint64_t* __restrict__ keys_out,
-                                                             uint32_t* __restrict__ vals_out, size_t n, int shift,
+                                                             KeyT* __restrict__ keys_out,
+                                                             uint32_t* __restrict__ vals_out, size_t n,
+                                                             const uint32_t* __restrict__ n_device, int shift,
                                                              uint32_t mask, const uint32_t* __restrict__ digit_start,
                                                              uint32_t* __restrict__ lookback,
                                                              uint32_t* __restrict__ tile_counter,
                                                              uint32_t* __restrict__ status)
 {
-	__shared__ uint64_t s_keys[kSortBlock];
+	__shared__ KeyT s_keys[kSortBlock];
 	__shared__ uint32_t s_vals[kSortBlock];
 	__shared__ uint32_t s_wave_hist[4][256];  // per-wave digit counts, then exclusive prefix over waves
 	__shared__ uint32_t s_digit_base[256];    // exclusive prefix over digits within the tile
@@ -229,16 +323,21 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const uint64_t* __re
 	__syncthreads();
 	const uint32_t tile = s_tile;
 	const size_t block_base = (size_t)tile * kSortBlock;
+	if (n_device)
+		n = *n_device;
+	// launched for an upper bound of n: tiles beyond the data leave, and no tile waits for them
+	if (block_base >= n)
+		return;
 	const size_t wave_base = block_base + (size_t)wave * (kSortItems * 64);
 
-	uint64_t key[kSortItems];
+	KeyT key[kSortItems];
 	uint32_t val[kSortItems];
 	uint32_t rank[kSortItems];
 #pragma unroll
 	for (int i = 0; i < kSortItems; i++) {
 		const size_t k = wave_base + (size_t)i * 64 + lane;
 		const bool ok = k < n;
-		key[i] = ok ? keys_in[k] : ~0ull;
+		key[i] = ok ? keys_in[k] : (KeyT)~(KeyT)0;
 		val[i] = ok ? vals_in[k] : 0u;
 	}
 
@@ -342,7 +441,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const uint64_t* __re
 	for (int i = 0; i < kSortItems; i++) {
 		const uint32_t p = (uint32_t)i * 256 + tid;
 		if (p < valid) {
-			const uint64_t kk = s_keys[p];
+			const KeyT kk = s_keys[p];
 			const uint32_t d = digit_of(kk, shift, mask);
 			const size_t dst = (size_t)s_global_base[d] + (p - s_digit_base[d]);
 			if (dst < n) {
@@ -364,31 +463,48 @@ const uint32_t* sort_status_word(const uint32_t* temp)
 	return temp + kSortStatus;
 }
 
-void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                       int end_bit, uint32_t* temp, hipStream_t s)
+template <typename KeyT>
+static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                       const uint32_t* n_device, int end_bit, uint32_t* temp, bool mark_stages, hipStream_t s)
 {
 	if (n == 0)
 		return;
 	const uint32_t tiles = (uint32_t)((n + kSortBlock - 1) / kSortBlock);
 	const int passes = (end_bit + 7) / 8;
-	stage_mark("sort_setup", s);
+	if (mark_stages)
+		stage_mark("sort_setup", s);
 	launch_fill_u32(temp, 0u, kSortHeader + (size_t)passes * 256 * tiles, s);
 	const uint32_t hist_blocks = tiles < 2048u ? tiles : 2048u;
-	hipLaunchKernelGGL(sort_digit_histogram_kernel, dim3(hist_blocks), dim3(256), 0, s, keys_in, n, passes, end_bit, temp);
+	hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks), dim3(256), 0, s, keys_in, n, n_device, passes,
+	                   end_bit, temp);
 	hipLaunchKernelGGL(sort_digit_starts_kernel, dim3(1), dim3(256), 0, s, temp, passes);
-	uint64_t *ksrc = keys_in, *kdst = keys_out;
+	KeyT *ksrc = keys_in, *kdst = keys_out;
 	uint32_t *vsrc = vals_in, *vdst = vals_out;
 	for (int p = 0; p < passes; p++) {
 		const int shift = 8 * p;
 		const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
 		const uint32_t mask = (1u << bits) - 1u;
-		stage_mark("sort_onesweep", s);
-		hipLaunchKernelGGL(sort_onesweep_kernel, dim3(tiles), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, shift, mask,
+		if (mark_stages)
+			stage_mark("sort_onesweep", s);
+		hipLaunchKernelGGL(sort_onesweep_kernel<KeyT>, dim3(tiles), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, n_device, shift,
+		                   mask,
 		                   temp + p * 256, temp + kSortHeader + (size_t)p * 256 * tiles, temp + kSortCounters + p,
 		                   temp + kSortStatus);
-		uint64_t* tk = ksrc; ksrc = kdst; kdst = tk;
+		KeyT* tk = ksrc; ksrc = kdst; kdst = tk;
 		uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
 	}
+}
+
+void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                       int end_bit, uint32_t* temp, hipStream_t s)
+{
+	sort_pairs<uint64_t>(keys_in, keys_out, vals_in, vals_out, n, nullptr, end_bit, temp, true, s);
+}
+
+void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                           const uint32_t* n_device, int end_bit, uint32_t* temp, const char* stage, hipStream_t s)
+{
+	sort_pairs<uint32_t>(keys_in, keys_out, vals_in, vals_out, n, n_device, end_bit, temp, stage != nullptr, s);
 }
 
 // ---- tile ranges (K/cuda_rasterizer_hgs/rasterizer_impl.cu:116-138 and the memset at :319) ----
@@ -407,22 +523,23 @@ void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 	hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, v, n);
 }
 
-// `sort_status` (may be null) is the sort's status word: if the sort reported a failure the
+// The status words (may be null) are those of the two sorts: if either reported a failure the
 // ranges stay empty, so no later stage walks an unsorted list.
-__global__ __launch_bounds__(256) void tile_ranges_kernel(const uint64_t* __restrict__ keys, size_t n,
+__global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __restrict__ keys, size_t n,
                                                            uint2* __restrict__ ranges,
-                                                           const uint32_t* __restrict__ sort_status)
+                                                           const uint32_t* __restrict__ sort_status,
+                                                           const uint32_t* __restrict__ order_status)
 {
 	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
 	if (idx >= n)
 		return;
-	if (sort_status && *sort_status != 0u)
+	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u))
 		return;
-	const uint32_t cur = (uint32_t)(keys[idx] >> 32);
+	const uint32_t cur = keys[idx];
 	if (idx == 0) {
 		ranges[cur].x = 0;
 	} else {
-		const uint32_t prev = (uint32_t)(keys[idx - 1] >> 32);
+		const uint32_t prev = keys[idx - 1];
 		if (cur != prev) {
 			ranges[prev].y = (uint32_t)idx;
 			ranges[cur].x = (uint32_t)idx;
@@ -432,15 +549,15 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint64_t* __rest
 		ranges[cur].y = (uint32_t)n;
 }
 
-void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
-                        hipStream_t s)
+void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
+                        const uint32_t* order_status, hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
 	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2, s);
 	if (n == 0)
 		return;
 	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges,
-	                   sort_status);
+	                   sort_status, order_status);
 }
 
 }  // namespace rgs

@@ -221,6 +221,11 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs 
 	(void)block256_exclusive_scan_u32(touched, s_scan, total);
 	if (threadIdx.x == 0)
 		a.block_sums[blockIdx.x] = total;
+	// ... and of the Gaussians that touch any tile: first level of the scan that compacts them
+	__syncthreads();
+	(void)block256_exclusive_scan_u32(touched != 0u ? 1u : 0u, s_scan, total);
+	if (threadIdx.x == 0)
+		a.block_visible[blockIdx.x] = total;
 }
 
 // ---- backward preprocess -------------------------------------------------------------------

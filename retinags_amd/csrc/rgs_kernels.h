@@ -34,6 +34,7 @@ struct PreprocessArgs {
 	uint32_t* tiles_touched;
 	uint8_t* clamped;
 	uint32_t* block_sums;  // one per 256 Gaussians
+	uint32_t* block_visible;  // one per 256 Gaussians: how many of them touch a tile
 	float4* blend_record;  // 4 float4 per Gaussian, see blend.hip
 };
 
@@ -126,21 +127,40 @@ void launch_preprocess_backward(const PreprocessBackwardArgs& a, hipStream_t s);
 constexpr int kSortItems = 16;                    // keys per thread in one sort block
 constexpr int kSortBlock = 256 * kSortItems;      // keys per sort block
 size_t scan_temp_words(size_t n);                 // u32 words of scratch for launch_inclusive_sum
-void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, hipStream_t s);
+// `stage` (may be null) names the stage for the timing aid.
+void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, const char* stage,
+                          hipStream_t s);
+// Scans the per-256 block sums of the tile counts in place; *total_out = number of instances.
+void launch_total_from_block_sums(uint32_t* block_sums, int P, uint32_t* total_out, hipStream_t s);
 void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* block_sums, uint32_t* offsets, int P,
                                     uint32_t* total_out, hipStream_t s);
-void launch_duplicate_with_keys(int P, const float2* xy, const float* depths, const uint32_t* offsets,
-                                const int* radii, int grid_x, int grid_y, uint64_t* keys, uint32_t* values,
-                                hipStream_t s);
-size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs
+// Depth order of the Gaussians that touch a tile.  block_visible holds their count per 256
+// Gaussians (scanned in place; the total goes to *visible_count).  On return order[0..count)
+// lists them by increasing depth, ties by index, and offsets_in_order is the inclusive scan of
+// their tile counts in that order.  The count stays on the device: every kernel is launched
+// for P elements and reads it.
+void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touched, uint32_t* block_visible,
+                        uint32_t* visible_count, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
+                        uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
+                        hipStream_t s);
+void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
+                                const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
+                                int grid_y, uint32_t* keys, uint32_t* values, hipStream_t s);
+size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs*
 // Stable LSD radix sort on key bits [0, end_bit), ceil(end_bit/8) passes that ping-pong between
 // the two buffer pairs starting in -> out: an odd pass count leaves the result in
 // keys_out/vals_out, an even one in keys_in/vals_in.
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s);
+// The same for 32-bit keys; with a null `stage` its kernels are not marked for the timing aid.
+// With a non-null n_device the number of pairs is read from there by the kernels and `n` is only
+// its upper bound (grids and scratch are sized for it).
+void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                           const uint32_t* n_device, int end_bit, uint32_t* temp, const char* stage, hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
-void launch_tile_ranges(const uint64_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
-                        hipStream_t s);
+// Either status word (may be null) being non-zero leaves every range empty.
+void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
+                        const uint32_t* order_status, hipStream_t s);
 
 // blend.hip
 void launch_blend_forward(const BlendArgs& a, hipStream_t s);

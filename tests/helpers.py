@@ -46,3 +46,28 @@ def view_ws(buf, offset, count, dtype):
     nbytes = count * np.dtype(dtype).itemsize
     raw = buf[offset:offset + nbytes].cpu().numpy()
     return raw.view(dtype)
+
+
+def check_binning_against(st, geom, binning, P, R, W, H):
+    """The library's binning state against the checker's, bit for bit.  The library sorts the
+    Gaussians by depth first and the (Gaussian, tile) instances by tile afterwards; the checker
+    follows the reference (one stable sort of instances on (tile << 32) | depth bits).  Both must
+    give the same lists, and the 64-bit keys of the reference are rebuilt from the parts."""
+    from retinags_amd import _capi
+    g = _capi.geom_layout(P)
+    touched = view_ws(geom, g["tiles_touched"], P, np.uint32)
+    depth_bits = view_ws(geom, g["depths"], P, np.uint32)
+    visible = np.flatnonzero(touched != 0).astype(np.uint32)
+    n_vis = int(view_ws(geom, g["visible_count"], 1, np.uint32)[0])
+    assert n_vis == len(visible)
+    order = view_ws(geom, g["depth_order"], P, np.uint32)[:n_vis]
+    assert np.array_equal(order, visible[np.argsort(depth_bits[visible], kind="stable")])
+    in_order = view_ws(geom, g["point_offsets"], P, np.uint32)[:n_vis]
+    assert np.array_equal(in_order, np.cumsum(touched[order].astype(np.uint64)).astype(np.uint32))
+    if R == 0:
+        return
+    b = _capi.binning_layout(R, W, H)
+    tiles = view_ws(binning, b["keys_sorted"], R, np.uint32)
+    vals = view_ws(binning, b["values_sorted"], R, np.uint32)
+    assert np.array_equal(vals, st.point_list)
+    assert np.array_equal((tiles.astype(np.uint64) << np.uint64(32)) | depth_bits[vals].astype(np.uint64), st.keys)

@@ -44,7 +44,9 @@ def test_workspace_sizes_and_layouts_are_consistent():
         lay = _capi.geom_layout(P)
         total = _capi.lib.rgs_geom_bytes(P)
         sizes = dict(depths=4 * P, xy=8 * P, clip_w=4 * P, cov3D=24 * P, conic_opacity=16 * P, rgb=12 * P,
-                     tiles_touched=4 * P, point_offsets=4 * P, clamped=P, block_sums=4 * ((P + 255) // 256 + 1), total=4)
+                     tiles_touched=4 * P, point_offsets=4 * P, clamped=P, block_sums=4 * ((P + 255) // 256 + 1), total=4,
+                     blend_record=64 * P, depth_order=4 * P, block_visible=4 * ((P + 255) // 256 + 1),
+                     visible_count=4, order_scratch=16 * P)
         spans = sorted((lay[k], lay[k] + sizes[k]) for k in sizes)
         assert all(a % 256 == 0 for a, _ in spans)
         assert all(spans[i][1] <= spans[i + 1][0] for i in range(len(spans) - 1))
@@ -52,7 +54,7 @@ def test_workspace_sizes_and_layouts_are_consistent():
     for R, (W, H) in ((1, (512, 512)), (4097, (1600, 1036)), (10 ** 6, (5185, 3359))):
         lay = _capi.binning_layout(R, W, H)
         total = _capi.lib.rgs_binning_bytes(R)
-        sizes = dict(keys_unsorted=8 * R, keys_sorted=8 * R, values_unsorted=4 * R, values_sorted=4 * R,
+        sizes = dict(keys_unsorted=4 * R, keys_sorted=4 * R, values_unsorted=4 * R, values_sorted=4 * R,
                      sort_temp=_capi.lib.rgs_sort_temp_bytes(R))
         spans = sorted((lay[k], lay[k] + sizes[k]) for k in sizes)
         assert all(spans[i][1] <= spans[i + 1][0] for i in range(len(spans) - 1))

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import scenes, view_ws
+from helpers import check_binning_against, scenes, view_ws
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -31,15 +31,22 @@ def _check_binning_structure(outs, P, W, H):
     g = _capi.geom_layout(P)
     radii = radii.cpu().numpy()
     touched = view_ws(geom, g["tiles_touched"], P, np.uint32)
-    offsets = view_ws(geom, g["point_offsets"], P, np.uint32)
+    n_vis = int(view_ws(geom, g["visible_count"], 1, np.uint32)[0])
+    offsets = view_ws(geom, g["point_offsets"], P, np.uint32)[:n_vis]
+    order = view_ws(geom, g["depth_order"], P, np.uint32)[:n_vis]
+    depth_bits = view_ws(geom, g["depths"], P, np.uint32)
     assert int(touched.astype(np.int64).sum()) == Rn
-    assert np.array_equal(offsets, np.cumsum(touched.astype(np.uint64)).astype(np.uint32))
+    assert np.array_equal(np.sort(order), np.flatnonzero(touched != 0).astype(np.uint32))   # the visible ones, once each
+    assert (np.diff(depth_bits[order].astype(np.int64)) >= 0).all()                         # by depth
+    assert np.array_equal(offsets, np.cumsum(touched[order].astype(np.uint64)).astype(np.uint32))
     assert np.array_equal(radii > 0, touched > 0)
     if Rn == 0:
         return
     b = _capi.binning_layout(Rn, W, H)
-    keys = view_ws(binning, b["keys_sorted"], Rn, np.uint64)
     vals = view_ws(binning, b["values_sorted"], Rn, np.uint32)
+    # the reference's 64-bit keys, rebuilt: the tile the sort used and the Gaussian's depth bits
+    keys = (view_ws(binning, b["keys_sorted"], Rn, np.uint32).astype(np.uint64) << np.uint64(32)) | \
+        depth_bits[vals].astype(np.uint64)
     assert (np.diff(keys.astype(np.uint64).view(np.int64)) >= 0).all()          # sorted (keys < 2^63)
     same = keys[1:] == keys[:-1]
     assert (vals[1:][same] > vals[:-1][same]).all()                             # ties keep emission order
@@ -172,9 +179,7 @@ def test_garden_full_size_against_checker():
             sub = subs[m].requires_grad_(True)
             raw = _forward_raw(sub, cam.to(DEV), cam, torch.zeros(3, device=DEV))
             assert raw[0] == st.R
-            b = _capi.binning_layout(st.R, W, H)
-            assert np.array_equal(view_ws(raw[6], b["keys_sorted"], st.R, np.uint64), st.keys)
-            assert np.array_equal(view_ws(raw[6], b["values_sorted"], st.R, np.uint32), st.point_list)
+            check_binning_against(st, raw[5], raw[6], st.P, st.R, W, H)
             assert np.array_equal(view_ws(raw[7], _capi.image_layout(W, H)["ranges"], 2 * len(st.ranges), np.uint32),
                                   st.ranges.ravel())
             del raw

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import (DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, MAX_BORDERLINE_FRACTION, np32, oracle_settings, orc,
+from helpers import (check_binning_against, DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, MAX_BORDERLINE_FRACTION, np32, oracle_settings, orc,
                      rel_l2, scenes, view_ws)
 
 pytestmark = pytest.mark.gpu
@@ -42,7 +42,6 @@ def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
     vis = st.radii > 0
     g = _capi.geom_layout(P)
     assert np.array_equal(view_ws(geom, g["tiles_touched"], P, np.uint32), st.tiles_touched)
-    assert np.array_equal(view_ws(geom, g["point_offsets"], P, np.uint32), st.point_offsets)
     xy = view_ws(geom, g["xy"], 2 * P, np.float32).reshape(P, 2)
     assert np.array_equal(xy[vis].view(np.uint32), st.xy[vis].view(np.uint32))
     assert np.array_equal(view_ws(geom, g["depths"], P, np.uint32)[vis], st.depths.view(np.uint32)[vis])
@@ -58,10 +57,7 @@ def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
     assert np.array_equal(clamped[vis], packed[vis])
 
     # ---- binning: bit-exact
-    if R > 0:
-        b = _capi.binning_layout(R, W, H)
-        assert np.array_equal(view_ws(binning, b["keys_sorted"], R, np.uint64), st.keys)
-        assert np.array_equal(view_ws(binning, b["values_sorted"], R, np.uint32), st.point_list)
+    check_binning_against(st, geom, binning, P, R, W, H)
     im = _capi.image_layout(W, H)
     assert np.array_equal(view_ws(img, im["ranges"], 2 * T, np.uint32).reshape(T, 2), st.ranges)
 
