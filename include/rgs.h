@@ -65,6 +65,7 @@ enum {
 	                               entries from RGS_GEOM_VISIBLE_COUNT on are unused */
 	RGS_GEOM_BLOCK_VISIBLE,     /* uint32[ceil(P/256)+1] */
 	RGS_GEOM_VISIBLE_COUNT,     /* uint32     number of Gaussians that touch a tile */
+	RGS_GEOM_VISIBLE_LIST,      /* uint32[P]  their indices in increasing order (as many entries as the count) */
 	RGS_GEOM_ORDER_SCRATCH,     /* scratch of the depth sort */
 	RGS_GEOM_FIELDS
 };
@@ -150,8 +151,11 @@ enum { RGS_ACC_FLOATS = 12 };
  * (K/rasterize_points.cu:165-174).  grad_accum (RGS_ACC_FLOATS*P floats) need not be cleared
  * by the caller.  dL_dmean2D (P,3; third column 0), dL_dopacity (P), dL_dcolor (P,3),
  * dL_dmean3D (P,3), dL_dcov3D (P,6), dL_dsh (P,M,3), dL_dscale (P,3), dL_drot (P,4) are
- * written for every Gaussian (zeros where it was not rendered); dL_dsh / dL_dscale /
- * dL_drot may be NULL when shs / scales are NULL. */
+ * complete when the call has run: rows of rendered Gaussians are computed, all others are
+ * zero.  With outputs_zeroed = 0 the library clears the eight arrays itself, like the
+ * reference's shim; a caller that hands over arrays it has already cleared (say, while the
+ * forward pass was still running) passes 1 and saves that pass over them.  dL_dsh /
+ * dL_dscale / dL_drot may be NULL when shs / scales are NULL. */
 int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const float* background, const float* means3D, const float* shs, const float* colors_precomp,
                  const float* alphas, const float* scales, float scale_modifier, const float* rotations,
@@ -161,7 +165,8 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const void* geom_ws, const void* binning_ws, const void* image_ws,
                  const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
                  float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
-                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, void* stream, int debug);
+                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int outputs_zeroed, void* stream,
+                 int debug);
 
 /* ---- measurement aids (no counterpart in the reference, which times whole iterations
  * with CUDA events: parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:590-643) -- */

@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("RGS_LIBRARY") or os.path.join(_HERE, "librgs_gfx950.s
 
 GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles_touched", "point_offsets",
                "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
-               "order_scratch")
+               "visible_list", "order_scratch")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
 IMG_FIELDS = ("ranges", "n_contrib")
 ACC_FLOATS = 12
@@ -50,7 +50,7 @@ def _load():
     lib.rgs_forward_raster.argtypes = [i, i, i, i, vp, f, f, vp, vp, vp, vp, vp, vp, sz, vp, sz, vp, sz,
                                        vp, vp, vp, vp, i]
     lib.rgs_backward.argtypes = [i, i, i, i, i, i, vp, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, vp, vp, vp,
-                                 f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i]
+                                 f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, i]
     lib.rgs_inclusive_sum.argtypes = [vp, vp, sz, vp, vp]
     lib.rgs_sort_pairs.argtypes = [vp, vp, vp, vp, sz, i, vp, vp]
     pp = C.POINTER(vp)

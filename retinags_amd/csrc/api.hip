@@ -136,6 +136,7 @@ size_t geom_layout(size_t P, size_t* off)
 	off[RGS_GEOM_DEPTH_ORDER] = c.take(4 * P);
 	off[RGS_GEOM_BLOCK_VISIBLE] = c.take(4 * ((P + 255) / 256 + 1));
 	off[RGS_GEOM_VISIBLE_COUNT] = c.take(4);
+	off[RGS_GEOM_VISIBLE_LIST] = c.take(4 * P);
 	off[RGS_GEOM_ORDER_SCRATCH] = c.take(order_scratch(P).total);
 	return c.cursor;
 }
@@ -387,6 +388,7 @@ static int forward_geom(bool wait_for_count, const char* who, int P, int D, int 
 		const OrderScratch o = order_scratch((size_t)P);
 		char* scratch = at<char>(geom_ws, off[RGS_GEOM_ORDER_SCRATCH]);
 		rgs::launch_depth_order(P, a.depths, a.tiles_touched, a.block_visible, at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_COUNT]),
+		                        at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_LIST]),
 		                        at<uint32_t>(scratch, o.keys_a), at<uint32_t>(scratch, o.keys_b),
 		                        at<uint32_t>(geom_ws, off[RGS_GEOM_DEPTH_ORDER]), at<uint32_t>(scratch, o.vals_b),
 		                        at<uint32_t>(scratch, o.tiles_in_order), at<uint32_t>(geom_ws, off[RGS_GEOM_POINT_OFFSETS]),
@@ -524,7 +526,8 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const void* geom_ws, const void* binning_ws, const void* image_ws,
                  const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
                  float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
-                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, void* stream, int debug)
+                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int outputs_zeroed, void* stream,
+                 int debug)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
@@ -588,7 +591,9 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	p.sums = grad_accum;
 	p.dL_dmean2D = dL_dmean2D; p.dL_dopacity = dL_dopacity; p.dL_dcolor = dL_dcolor;
 	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
-	rgs::launch_preprocess_backward(p, s);
+	p.visible_list = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_LIST]);
+	p.visible_count = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
+	rgs::launch_preprocess_backward(p, outputs_zeroed != 0, s);
 	RGS_STAGE("preprocess_backward");
 	return 0;
 }

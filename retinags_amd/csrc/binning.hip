@@ -145,7 +145,8 @@ void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* blo
 __global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __restrict__ depths,
                                                            const uint32_t* __restrict__ tiles_touched,
                                                            const uint32_t* __restrict__ visible_base,
-                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ values)
+                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                           uint32_t* __restrict__ visible_list)
 {
 	__shared__ uint32_t lds[8];
 	const int idx = blockIdx.x * 256 + threadIdx.x;
@@ -156,6 +157,7 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __
 		const uint32_t at = visible_base[blockIdx.x] + rank;
 		keys[at] = __float_as_uint(depths[idx]);
 		values[at] = (uint32_t)idx;
+		visible_list[at] = (uint32_t)idx;  // the sort reorders `values`; this copy stays in index order
 	}
 }
 
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t
 }
 
 void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touched, uint32_t* block_visible,
-                        uint32_t* visible_count, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
+                        uint32_t* visible_count, uint32_t* visible_list, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
                         uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
                         hipStream_t s)
 {
@@ -205,7 +207,7 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_visible, (size_t)nb,
 	                   (const uint32_t*)nullptr, visible_count);
 	hipLaunchKernelGGL(depth_pairs_kernel, dim3(nb), dim3(256), 0, s, P, depths, tiles_touched, block_visible, keys_a,
-	                   order);
+	                   order, visible_list);
 	// 4 passes: the sorted pairs end up in the first buffer pair again
 	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, nullptr, s);
 	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched,

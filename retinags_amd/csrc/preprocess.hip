@@ -230,8 +230,10 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs 
 
 // ---- backward preprocess -------------------------------------------------------------------
 // Fuses K/cuda_rasterizer_hgs/backward.cu:144-274 (conic -> 3D covariance and mean)
-// with :346-412 (projection, depth, SH, scale/rotation).  Gaussians that were not
-// rendered get zero gradients written here, so the caller allocates without clearing.
+// with :346-412 (projection, depth, SH, scale/rotation).  Only Gaussians that were rendered
+// have non-zero gradients; the kernel runs over the compacted list of those (in index order,
+// every lane busy) and writes their rows.  The rows of all others must be zero beforehand:
+// the caller says whether they already are, otherwise the launcher clears the arrays first.
 
 __device__ __forceinline__ void sh_backward_channel(int deg, float x, float y, float z, const float* __restrict__ sh,
                                                     float g, float* __restrict__ dsh, float& ddx, float& ddy,
@@ -290,52 +292,23 @@ __device__ __forceinline__ void sh_backward_channel(int deg, float x, float y, f
 	ddz += dRGBdz * g;
 }
 
-// One wavefront per block.  Every lane builds its Gaussian's 16 + 3M gradient floats in an
-// LDS row (stride 65 words: conflict-free for per-lane rows), then the wavefront writes
-// the five output arrays with fully coalesced stores; rows of Gaussians that were not
-// rendered stay zero.
-constexpr int kBwdRow = 65;
-constexpr int kBwdMeans = 0, kBwdCov = 3, kBwdScale = 9, kBwdRot = 12, kBwdSh = 16, kBwdShMax = 48;
+constexpr int kBwdShMax = 48;  // SH gradient floats kept in registers until they are stored
 
-__device__ __forceinline__ void store_rows(float* __restrict__ dst, const float* s_out, int field, int width, int rows,
-                                           int lane)
+__global__ __launch_bounds__(128) void preprocess_backward_kernel(PreprocessBackwardArgs a)
 {
-	const int n = rows * width;
-	int r = 0, c = lane;
-	while (c >= width) {
-		c -= width;
-		r++;
-	}
-	for (int t = lane; t < n; t += 64) {
-		dst[t] = s_out[r * kBwdRow + field + c];
-		c += 64;
-		while (c >= width) {
-			c -= width;
-			r++;
-		}
-	}
-}
-
-__global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackwardArgs a)
-{
-	__shared__ float s_out[64 * kBwdRow];
-	const int lane = threadIdx.x;
-	const int first = blockIdx.x * 64;
-	const int idx = first + lane;
-	const size_t i = (size_t)idx;
+	const uint32_t k_vis = blockIdx.x * 128 + threadIdx.x;
+	if (k_vis >= *a.visible_count)
+		return;
+	const size_t i = (size_t)a.visible_list[k_vis];
 	const int n_sh = a.shs ? a.M * 3 : 0;
-	const bool sh_in_lds = n_sh <= kBwdShMax;
-	float* row = s_out + lane * kBwdRow;
+	const bool sh_in_regs = n_sh <= kBwdShMax;
+	float shg[kBwdShMax];
 #pragma unroll
-	for (int k = 0; k < 64; k++)
-		row[k] = 0.f;
-	const bool visible = idx < a.P && a.radii[idx > a.P - 1 ? a.P - 1 : idx] > 0;
+	for (int k = 0; k < kBwdShMax; k++)
+		shg[k] = 0.f;
 	float mean2d_x = 0.f, mean2d_y = 0.f, opacity_sum = 0.f, color_sum[3] = {0.f, 0.f, 0.f};
-	if (!sh_in_lds && idx < a.P && !visible)
-		for (int k = 0; k < n_sh; k++)
-			a.dL_dsh[i * n_sh + k] = 0.f;
 
-	if (visible) {
+	{
 	const float* __restrict__ view = a.view;
 	const float* __restrict__ proj = a.proj;
 	const float3 mean = {a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
@@ -386,7 +359,7 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 	}
 #pragma unroll
 	for (int k = 0; k < 6; k++)
-		row[kBwdCov + k] = dcov[k];
+		a.dL_dcov3D[6 * i + k] = dcov[k];
 
 	const float dL_dT00 = 2 * (TM(0, 0) * VM(0, 0) + TM(0, 1) * VM(0, 1) + TM(0, 2) * VM(0, 2)) * dL_da +
 	                      (TM(1, 0) * VM(0, 0) + TM(1, 1) * VM(0, 1) + TM(1, 2) * VM(0, 2)) * dL_db;
@@ -448,8 +421,8 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 #pragma unroll
 		for (int ch = 0; ch < 3; ch++) {
 			const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-			if (sh_in_lds)  // the usual case: rows go out through LDS, coalesced
-				sh_backward_channel(a.D, x, y, z, sh + ch, g, row + kBwdSh + ch, ddx, ddy, ddz);
+			if (sh_in_regs)  // the usual case: the row is stored 16 bytes at a time below
+				sh_backward_channel(a.D, x, y, z, sh + ch, g, shg + ch, ddx, ddy, ddz);
 			else
 				sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
 		}
@@ -460,9 +433,9 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 		dmean.y += (-d0.x * d0.y * ddx + (sum2 - d0.y * d0.y) * ddy - d0.z * d0.y * ddz) * invsum32;
 		dmean.z += (-d0.x * d0.z * ddx - d0.y * d0.z * ddy + (sum2 - d0.z * d0.z) * ddz) * invsum32;
 	}
-	row[kBwdMeans + 0] = dmean.x;
-	row[kBwdMeans + 1] = dmean.y;
-	row[kBwdMeans + 2] = dmean.z;
+	a.dL_dmeans[3 * i + 0] = dmean.x;
+	a.dL_dmeans[3 * i + 1] = dmean.y;
+	a.dL_dmeans[3 * i + 2] = dmean.z;
 
 	// -- 3D covariance -> scale and raw quaternion (backward.cu:278-341)
 	if (a.scales) {
@@ -491,9 +464,9 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 #pragma unroll
 		for (int k = 0; k < 3; k++)
 			ds[k] = Rt.c[k][0] * dMt.c[k][0] + Rt.c[k][1] * dMt.c[k][1] + Rt.c[k][2] * dMt.c[k][2];
-		row[kBwdScale + 0] = ds[0];
-		row[kBwdScale + 1] = ds[1];
-		row[kBwdScale + 2] = ds[2];
+		a.dL_dscale[3 * i + 0] = ds[0];
+		a.dL_dscale[3 * i + 1] = ds[1];
+		a.dL_dscale[3 * i + 2] = ds[2];
 #pragma unroll
 		for (int k = 0; k < 3; k++)
 #pragma unroll
@@ -509,37 +482,31 @@ __global__ __launch_bounds__(64) void preprocess_backward_kernel(PreprocessBackw
 		dq.w = 2 * r * (DM(0, 1) - DM(1, 0)) + 2 * x * (DM(2, 0) + DM(0, 2)) + 2 * y * (DM(1, 2) + DM(2, 1)) -
 		       4 * z * (DM(1, 1) + DM(0, 0));
 #undef DM
-		row[kBwdRot + 0] = dq.x;
-		row[kBwdRot + 1] = dq.y;
-		row[kBwdRot + 2] = dq.z;
-		row[kBwdRot + 3] = dq.w;
+		reinterpret_cast<float4*>(a.dL_drot)[i] = dq;
 	}
-	}  // visible
-
-	__syncthreads();
-	const int rows = a.P - first < 64 ? a.P - first : 64;
-	store_rows(a.dL_dmeans + 3 * (size_t)first, s_out, kBwdMeans, 3, rows, lane);
-	store_rows(a.dL_dcov3D + 6 * (size_t)first, s_out, kBwdCov, 6, rows, lane);
-	if (a.scales) {
-		store_rows(a.dL_dscale + 3 * (size_t)first, s_out, kBwdScale, 3, rows, lane);
-		store_rows(a.dL_drot + 4 * (size_t)first, s_out, kBwdRot, 4, rows, lane);
 	}
-	if (n_sh > 0 && sh_in_lds)
-		store_rows(a.dL_dsh + (size_t)n_sh * first, s_out, kBwdSh, n_sh, rows, lane);
 
-	// the sums that are gradients as they stand leave through the same rows
-	__syncthreads();
-	row[0] = mean2d_x;
-	row[1] = mean2d_y;
-	row[2] = 0.f;
-	row[3] = opacity_sum;
-	row[4] = color_sum[0];
-	row[5] = color_sum[1];
-	row[6] = color_sum[2];
-	__syncthreads();
-	store_rows(a.dL_dmean2D + 3 * (size_t)first, s_out, 0, 3, rows, lane);
-	store_rows(a.dL_dopacity + (size_t)first, s_out, 3, 1, rows, lane);
-	store_rows(a.dL_dcolor + 3 * (size_t)first, s_out, 4, 3, rows, lane);
+	if (n_sh > 0 && sh_in_regs) {
+		float* dst = a.dL_dsh + i * n_sh;
+		if ((n_sh & 3) == 0) {
+#pragma unroll
+			for (int k = 0; k < kBwdShMax; k += 4)
+				if (k < n_sh)
+					*reinterpret_cast<float4*>(dst + k) = float4{shg[k], shg[k + 1], shg[k + 2], shg[k + 3]};
+		} else {
+#pragma unroll
+			for (int k = 0; k < kBwdShMax; k++)
+				if (k < n_sh)
+					dst[k] = shg[k];
+		}
+	}
+	// the sums that are gradients as they stand
+	a.dL_dmean2D[3 * i + 0] = mean2d_x;
+	a.dL_dmean2D[3 * i + 1] = mean2d_y;
+	a.dL_dopacity[i] = opacity_sum;
+	a.dL_dcolor[3 * i + 0] = color_sum[0];
+	a.dL_dcolor[3 * i + 1] = color_sum[1];
+	a.dL_dcolor[3 * i + 2] = color_sum[2];
 }
 
 // ---- launchers -----------------------------------------------------------------------------
@@ -556,10 +523,25 @@ void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s)
 	hipLaunchKernelGGL(preprocess_forward_kernel, dim3((a.P + 255) / 256), dim3(256), 0, s, a);
 }
 
-void launch_preprocess_backward(const PreprocessBackwardArgs& a, hipStream_t s)
+void launch_preprocess_backward(const PreprocessBackwardArgs& a, bool outputs_zeroed, hipStream_t s)
 {
+	if (!outputs_zeroed) {
+		stage_mark("clear_gradients", s);
+		const size_t n = (size_t)a.P;
+		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmean2D), 0u, 3 * n, s);
+		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dopacity), 0u, n, s);
+		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcolor), 0u, 3 * n, s);
+		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmeans), 0u, 3 * n, s);
+		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcov3D), 0u, 6 * n, s);
+		if (a.shs)
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dsh), 0u, (size_t)a.M * 3 * n, s);
+		if (a.scales) {
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dscale), 0u, 3 * n, s);
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_drot), 0u, 4 * n, s);
+		}
+	}
 	stage_mark("preprocess_backward", s);
-	hipLaunchKernelGGL(preprocess_backward_kernel, dim3((a.P + 63) / 64), dim3(64), 0, s, a);
+	hipLaunchKernelGGL(preprocess_backward_kernel, dim3((a.P + 127) / 128), dim3(128), 0, s, a);
 }
 
 }  // namespace rgs

@@ -53,7 +53,9 @@ struct PreprocessBackwardArgs {
 	const float* campos;
 	float focal_x, focal_y, tanfovx, tanfovy;
 	const float* sums;  // (P, kSumCols): what the backward blend accumulated, see SumCol
-	// outputs, fully written
+	const uint32_t* visible_list;   // the Gaussians that touch a tile, in index order
+	const uint32_t* visible_count;  // how many (on the device)
+	// outputs: rows of the listed Gaussians are written, all other rows must be zero already
 	float* dL_dmean2D;  // (P,3), third column 0
 	float* dL_dopacity; // (P)
 	float* dL_dcolor;   // (P,3)
@@ -121,7 +123,8 @@ struct CompositeArgs {
 // preprocess.hip
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s);
 void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s);
-void launch_preprocess_backward(const PreprocessBackwardArgs& a, hipStream_t s);
+// With outputs_zeroed false the eight output arrays are cleared first.
+void launch_preprocess_backward(const PreprocessBackwardArgs& a, bool outputs_zeroed, hipStream_t s);
 
 // binning.hip
 constexpr int kSortItems = 16;                    // keys per thread in one sort block
@@ -137,10 +140,10 @@ void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* blo
 // Depth order of the Gaussians that touch a tile.  block_visible holds their count per 256
 // Gaussians (scanned in place; the total goes to *visible_count).  On return order[0..count)
 // lists them by increasing depth, ties by index, and offsets_in_order is the inclusive scan of
-// their tile counts in that order.  The count stays on the device: every kernel is launched
+// their tile counts in that order; visible_list keeps them in index order.  The count stays on the device: every kernel is launched
 // for P elements and reads it.
 void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touched, uint32_t* block_visible,
-                        uint32_t* visible_count, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
+                        uint32_t* visible_count, uint32_t* visible_list, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
                         uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
                         hipStream_t s);
 void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,

@@ -99,9 +99,19 @@ def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifie
     return rasterizer, geometry
 
 
+_pools = {}
+
+
+def _host_pool(n: int):
+    from concurrent.futures import ThreadPoolExecutor
+    if n not in _pools:
+        _pools[n] = ThreadPoolExecutor(max_workers=n, thread_name_prefix="rgs-stream")
+    return _pools[n]
+
+
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
                  submodel_bg: Optional[torch.Tensor] = None,
-                 streams: Optional[List["torch.cuda.Stream"]] = None) -> dict:
+                 streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = True) -> dict:
     """Render every related submodel (black background, as the trainer does:
     trainer4tree_partition.py:397) and composite the partial images in BVH order.
 
@@ -110,6 +120,8 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     streams[k % len(streams)] (default priority), so one submodel's short kernels and the tail
     of its blend run beside another's; autograd replays each submodel's backward on the stream
     its forward used.  The compositor runs on the caller's stream after all of them.  The
+    With host_threads each stream's forward calls are issued by a host thread of their own (the
+    library releases no lock but ctypes releases the interpreter's while inside it); without, the
     forward is issued in two rounds (all geometry stages, then all sort-and-blend stages): the
     host has to read each submodel's instance count in between, and this way it waits once.
     """
@@ -120,17 +132,30 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     if not streams:
         partial = {m: render_submodel(cam, subs[m], submodel_bg) for m in related}
     else:
-        # every geometry stage is enqueued before the host waits for the first instance count
         main = torch.cuda.current_stream(device)
-        partial, started = {}, {}
-        for k, m in enumerate(related):
-            side = streams[k % len(streams)]
+        for side in streams[:len(related)]:
             side.wait_stream(main)
-            with torch.cuda.stream(side):
-                started[m] = start_submodel(cam, subs[m], submodel_bg)
-        for k, m in enumerate(related):
-            with torch.cuda.stream(streams[k % len(streams)]):
-                partial[m] = render_submodel(cam, subs[m], submodel_bg, started=started[m])
+        partial = {}
+        if host_threads:
+            # one host thread per stream: a forward call is some thirty kernel launches, and issued
+            # from one thread the four submodels' launches would queue up behind each other
+            def forward_on(j):
+                with torch.cuda.device(device), torch.cuda.stream(streams[j]):
+                    return [(m, render_submodel(cam, subs[m], submodel_bg,
+                                                started=start_submodel(cam, subs[m], submodel_bg)))
+                            for k, m in enumerate(related) if k % len(streams) == j]
+            for done in _host_pool(len(streams)).map(forward_on, range(min(len(streams), len(related)))):
+                partial.update(done)
+            partial = {m: partial[m] for m in related}
+        else:
+            # every geometry stage is enqueued before the host waits for the first instance count
+            started = {}
+            for k, m in enumerate(related):
+                with torch.cuda.stream(streams[k % len(streams)]):
+                    started[m] = start_submodel(cam, subs[m], submodel_bg)
+            for k, m in enumerate(related):
+                with torch.cuda.stream(streams[k % len(streams)]):
+                    partial[m] = render_submodel(cam, subs[m], submodel_bg, started=started[m])
         for side in streams[:len(related)]:
             main.wait_stream(side)
         for res in partial.values():

@@ -188,12 +188,23 @@ def _rasterize_forward(*args):
     return _forward_blend(_forward_geometry(*args, wait=True))
 
 
+def _gradient_outputs(P, M, has_scales, device, make):
+    """The eight dense gradient tensors of K/rasterize_points.cu:165-174, made with `make`
+    (torch.empty or torch.zeros); without scales the scale / rotation gradients are zeros."""
+    f32 = dict(dtype=torch.float32, device=device)
+    return {"means2D": make((P, 3), **f32), "opacity": make((P, 1), **f32), "colors": make((P, 3), **f32),
+            "means3D": make((P, 3), **f32), "cov3D": make((P, 6), **f32), "sh": make((P, M, 3), **f32),
+            "scales": (make if has_scales else torch.zeros)((P, 3), **f32),
+            "rotations": (make if has_scales else torch.zeros)((P, 4), **f32)}
+
+
 def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, scale_modifier, cov3Ds_precomp,
                         viewmatrix, projmatrix, projmatrix_inv, range_low, range_up, tanfovx, tanfovy, grad_color,
                         grad_depth, grad_alpha, sh, sh_degree, campos, geomBuffer, num_rendered, binningBuffer,
-                        imgBuffer, alpha, debug):
+                        imgBuffer, alpha, debug, cleared=None):
     """Counterpart of RasterizeGaussiansBackwardCUDA_hgs (K/rasterize_points.cu:127-220);
-    returns the same 8 tensors in the same order."""
+    returns the same 8 tensors in the same order.  `cleared`, if given, is the dict of output
+    tensors that the forward made with _gradient_outputs(..., torch.zeros)."""
     device = means3D.device
     P = int(means3D.shape[0])
     H, W = int(grad_color.shape[1]), int(grad_color.shape[2])
@@ -224,15 +235,12 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
 
     # Scratch rows in which the blend accumulates its per-Gaussian sums; the library clears them.
     acc = torch.empty((_capi.ACC_FLOATS * P,), **f32)
-    dL_dmeans2D = torch.empty((P, 3), **f32)
-    dL_dopacity = torch.empty((P, 1), **f32)
-    dL_dcolors = torch.empty((P, 3), **f32)
-    dL_dmeans3D = torch.empty((P, 3), **f32)
-    dL_dcov3D = torch.empty((P, 6), **f32)
-    dL_dsh = torch.empty((P, M, 3), **f32)
     has_scales = scales.numel() != 0
-    dL_dscales = torch.empty((P, 3), **f32) if has_scales else torch.zeros((P, 3), **f32)
-    dL_drotations = torch.empty((P, 4), **f32) if has_scales else torch.zeros((P, 4), **f32)
+    outputs_zeroed = cleared is not None
+    out = cleared if outputs_zeroed else _gradient_outputs(P, M, has_scales, device, torch.empty)
+    dL_dmeans2D, dL_dopacity, dL_dcolors = out["means2D"], out["opacity"], out["colors"]
+    dL_dmeans3D, dL_dcov3D, dL_dsh = out["means3D"], out["cov3D"], out["sh"]
+    dL_dscales, dL_drotations = out["scales"], out["rotations"]
 
     with torch.cuda.device(device):
         check(lib.rgs_backward(
@@ -243,7 +251,7 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
             ptr(grad_depth), ptr(grad_alpha), ptr(acc), ptr(dL_dmeans2D), ptr(dL_dopacity), ptr(dL_dcolors),
             ptr(dL_dmeans3D), ptr(dL_dcov3D), ptr(dL_dsh),
             ptr(dL_dscales) if has_scales else C.c_void_p(0), ptr(dL_drotations) if has_scales else C.c_void_p(0),
-            _stream_ptr(device), int(bool(debug))))
+            int(outputs_zeroed), _stream_ptr(device), int(bool(debug))))
 
     return dL_dmeans2D, dL_dcolors, dL_dopacity, dL_dmeans3D, dL_dcov3D, dL_dsh, dL_dscales, dL_drotations
 
@@ -309,6 +317,15 @@ class _RasterizeGaussians(torch.autograd.Function):
 
         ctx.raster_settings = raster_settings
         ctx.num_rendered = num_rendered
+        # Only rendered Gaussians get non-zero gradients and the library writes just those rows;
+        # the rest of the gradient tensors is cleared here, behind the forward blend on this
+        # stream, where the clearing (pure memory traffic) overlaps other streams' blend kernels
+        # instead of lengthening the backward pass.
+        ctx.cleared = None
+        P = int(means3D.shape[0])
+        if P > 0 and any(ctx.needs_input_grad):
+            M = int(sh.shape[1]) if sh.numel() != 0 else 0
+            ctx.cleared = _gradient_outputs(P, M, scales.numel() != 0, means3D.device, torch.zeros)
         ctx.save_for_backward(colors_precomp, means3D, scales, rotations, cov3Ds_precomp, radii, sh, geomBuffer,
                               binningBuffer, imgBuffer, alpha)
         ctx.mark_non_differentiable(radii)
@@ -340,13 +357,14 @@ class _RasterizeGaussians(torch.autograd.Function):
         if raster_settings.debug:
             cpu_args = cpu_deep_copy_tuple(args)
             try:
-                outs = _rasterize_backward(*args)
+                outs = _rasterize_backward(*args, cleared=ctx.cleared)
             except Exception as ex:
                 torch.save(cpu_args, "snapshot_bw.dump")
                 print("\nAn error occured in backward. Writing snapshot_bw.dump for debugging.\n")
                 raise ex
         else:
-            outs = _rasterize_backward(*args)
+            outs = _rasterize_backward(*args, cleared=ctx.cleared)
+        ctx.cleared = None  # the tensors now belong to the caller
         (grad_means2D, grad_colors_precomp, grad_opacities, grad_means3D, grad_cov3Ds_precomp, grad_sh, grad_scales,
          grad_rotations) = outs
 

@@ -238,3 +238,27 @@ def test_enqueued_geometry_stage_gives_the_same_forward_and_is_checked():
     got2 = r(means2D=m2d, geometry=stage2, **kw)  # the refused call did not consume it
     assert torch.equal(ref[0], got2[0])
     torch.cuda.synchronize()
+
+
+def test_backward_clears_the_gradients_itself_when_the_caller_has_not():
+    """The first backward of a forward call uses gradient tensors cleared during the forward;
+    a second one over the retained graph has none and lets the library clear them.  Both give
+    the same gradients (up to the order of the float atomics)."""
+    from retinags_amd import GaussianRasterizer
+    scene, cam, low, up = _small_inputs(n=5000, seed=4)
+    scene = dict(scene)
+    scene["xyz"] = scene["xyz"].clone()
+    scene["xyz"][::3] = 2.0 * cam.camera_center - scene["xyz"][::3]  # every third one behind the camera
+    r = GaussianRasterizer(_settings(oracle_settings(cam, low, up, torch.tensor([0.3, 0.2, 0.1]))))
+    leaves = {k: scene[k].to(DEV).requires_grad_(True) for k in ("xyz", "opacity", "shs", "scales", "rotations")}
+    m2d = torch.zeros_like(leaves["xyz"], requires_grad=True)
+    color, radii, depth, alpha = r(means3D=leaves["xyz"], means2D=m2d, opacities=leaves["opacity"], shs=leaves["shs"],
+                                   scales=leaves["scales"], rotations=leaves["rotations"])
+    g = torch.randn(color.shape, generator=torch.Generator().manual_seed(9)).to(DEV) * 1e-2
+    tensors = [m2d] + list(leaves.values())
+    first = torch.autograd.grad([color], tensors, [g], retain_graph=True)
+    second = torch.autograd.grad([color], tensors, [g])
+    assert (radii > 0).any() and not (radii > 0).all()
+    for a, b in zip(first, second):
+        assert rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-4
+        assert torch.equal((a == 0).all(dim=tuple(range(1, a.ndim))), (b == 0).all(dim=tuple(range(1, b.ndim))))
