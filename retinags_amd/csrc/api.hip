@@ -320,6 +320,14 @@ int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const
 	return 0;
 }
 
+// Whether SH rows can be moved 16 bytes at a time: aligned base, row length a multiple of four
+// floats, at most 48 of them, and enough of them for the degree's rounded-up count.
+static bool sh_rows_by_16_bytes(const float* shs, int M, int D)
+{
+	const int n = 3 * M, needed = (3 * (D + 1) * (D + 1) + 3) & ~3;
+	return shs && (reinterpret_cast<uintptr_t>(shs) & 15) == 0 && (n & 3) == 0 && n <= 48 && needed <= n;
+}
+
 static int forward_geom(bool wait_for_count, const char* who, int P, int D, int M, int width, int height,
                         const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
                         const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
@@ -375,6 +383,7 @@ static int forward_geom(bool wait_for_count, const char* who, int P, int D, int 
 	a.block_sums = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_SUMS]);
 	a.blend_record = at<float4>(geom_ws, off[RGS_GEOM_BLEND_RECORD]);
 	a.block_visible = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_VISIBLE]);
+	a.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D);
 
 	rgs::launch_preprocess_forward(a, s);
 	RGS_STAGE("preprocess");
@@ -592,6 +601,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	p.dL_dmean2D = dL_dmean2D; p.dL_dopacity = dL_dopacity; p.dL_dcolor = dL_dcolor;
 	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
 	p.visible_list = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_LIST]);
+	p.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D) && (reinterpret_cast<uintptr_t>(dL_dsh) & 15) == 0;
 	p.visible_count = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
 	rgs::launch_preprocess_backward(p, outputs_zeroed != 0, s);
 	RGS_STAGE("preprocess_backward");

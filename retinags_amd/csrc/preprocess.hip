@@ -116,6 +116,27 @@ __device__ __forceinline__ float sh_channel(int deg, float x, float y, float z, 
 	return result + 0.5f;
 }
 
+// An SH row of up to 48 floats, read 16 bytes at a time into registers.  The evaluation reads
+// coefficient k of channel c at float 3 k + c; done with one 4-byte load each, a wavefront's 48
+// loads all touch 64 different cache lines and the address unit, not memory, sets the pace.
+// Only the floats the active degree needs are read (3 (deg + 1)^2, rounded up to four).
+constexpr int kShRegs = 48;
+
+__device__ __forceinline__ void load_sh_row(const float* __restrict__ row, int deg, float (&out)[kShRegs])
+{
+	const int needed = 3 * (deg + 1) * (deg + 1);
+#pragma unroll
+	for (int k = 0; k < kShRegs; k += 4) {
+		float4 v = {0.f, 0.f, 0.f, 0.f};
+		if (k < needed)
+			v = *reinterpret_cast<const float4*>(row + k);
+		out[k] = v.x;
+		out[k + 1] = v.y;
+		out[k + 2] = v.z;
+		out[k + 3] = v.w;
+	}
+}
+
 // ---- forward preprocess (K/cuda_rasterizer_hgs/forward.cu:155-258) -------------------------
 
 __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs a)
@@ -171,10 +192,21 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs 
 				const float dx = dir.x / len, dy = dir.y / len, dz = dir.z / len;
 				const float* sh = a.shs + (size_t)idx * a.M * 3;
 				uint32_t clamp_bits = 0;
-				float rgb[3];
+				float rgb[3], raw[3];
+				if (a.sh_rows_by_16_bytes) {
+					float row[kShRegs];
+					load_sh_row(sh, a.D, row);
+#pragma unroll
+					for (int ch = 0; ch < 3; ch++)
+						raw[ch] = sh_channel(a.D, dx, dy, dz, row + ch);
+				} else {
+#pragma unroll
+					for (int ch = 0; ch < 3; ch++)
+						raw[ch] = sh_channel(a.D, dx, dy, dz, sh + ch);
+				}
 #pragma unroll
 				for (int ch = 0; ch < 3; ch++) {
-					const float v = sh_channel(a.D, dx, dy, dz, sh + ch);
+					const float v = raw[ch];
 					clamp_bits |= (v < 0) ? (1u << ch) : 0u;
 					rgb[ch] = fmaxf(v, 0.0f);
 				}
@@ -418,13 +450,23 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(PreprocessBack
 		const uint32_t cl = a.clamped[i];
 		const float* sh = a.shs + i * n_sh;
 		float ddx = 0.f, ddy = 0.f, ddz = 0.f;
+		if (a.sh_rows_by_16_bytes) {  // the usual case: rows are read and written 16 bytes at a time
+			float row[kShRegs];
+			load_sh_row(sh, a.D, row);
 #pragma unroll
-		for (int ch = 0; ch < 3; ch++) {
-			const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-			if (sh_in_regs)  // the usual case: the row is stored 16 bytes at a time below
-				sh_backward_channel(a.D, x, y, z, sh + ch, g, shg + ch, ddx, ddy, ddz);
-			else
-				sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
+			for (int ch = 0; ch < 3; ch++) {
+				const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
+				sh_backward_channel(a.D, x, y, z, row + ch, g, shg + ch, ddx, ddy, ddz);
+			}
+		} else {
+#pragma unroll
+			for (int ch = 0; ch < 3; ch++) {
+				const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
+				if (sh_in_regs)
+					sh_backward_channel(a.D, x, y, z, sh + ch, g, shg + ch, ddx, ddy, ddz);
+				else
+					sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
+			}
 		}
 		// normalisation Jacobian (auxiliary.h:123-133)
 		const float sum2 = d0.x * d0.x + d0.y * d0.y + d0.z * d0.z;

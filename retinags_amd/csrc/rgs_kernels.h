@@ -35,6 +35,7 @@ struct PreprocessArgs {
 	uint8_t* clamped;
 	uint32_t* block_sums;  // one per 256 Gaussians
 	uint32_t* block_visible;  // one per 256 Gaussians: how many of them touch a tile
+	bool sh_rows_by_16_bytes; // SH rows are 16-byte aligned, a multiple of 16 bytes long and at most 48 floats
 	float4* blend_record;  // 4 float4 per Gaussian, see blend.hip
 };
 
@@ -55,6 +56,7 @@ struct PreprocessBackwardArgs {
 	const float* sums;  // (P, kSumCols): what the backward blend accumulated, see SumCol
 	const uint32_t* visible_list;   // the Gaussians that touch a tile, in index order
 	const uint32_t* visible_count;  // how many (on the device)
+	bool sh_rows_by_16_bytes;       // SH rows are 16-byte aligned, a multiple of 16 bytes long and at most 48 floats
 	// outputs: rows of the listed Gaussians are written, all other rows must be zero already
 	float* dL_dmean2D;  // (P,3), third column 0
 	float* dL_dopacity; // (P)
