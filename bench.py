@@ -173,7 +173,7 @@ def main():
     K = len(related)
     T = ((W + 15) // 16) * ((H + 15) // 16)
     N = W * H
-    passes = (32 + int(_capi.lib.rgs_get_higher_msb(T)) + 7) // 8
+    passes = (int(_capi.lib.rgs_get_higher_msb(T)) + 7) // 8   # of the instance sort, on the tile key
     # Per-pixel entries the backward revisits: everything up to the last blended entry.
     # It is not counted separately; the forward visit count bounds it from above.
     flops_fwd = 12 * nA + 3 * nB + 27 * nC + 3 * nD + 14 * nE
@@ -182,12 +182,16 @@ def main():
     # kernels run `passes` times per submodel).
     alg_bytes = {
         "preprocess_forward": 20.0 * P_tot + 299.0 * P_vis,
-        "offset_scan": 8.0 * P_tot,
-        "duplicate_with_keys": 4.0 * P_tot + 16.0 * P_vis + 12.0 * R_tot,
-        "sort_setup": 8.0 * R_tot,
-        "sort_onesweep": 24.0 * R_tot * passes,
-        "tile_ranges": 8.0 * R_tot + 16.0 * T * K,
-        "preprocess_backward": 4.0 * P_tot + 559.0 * P_vis,
+        # tile counts and depths of all, then 4 passes over the (depth, index) pairs of the visible
+        # ones, the gathered tile counts and their scan
+        "depth_order": 8.0 * P_tot + (12.0 + 4 * 16.0 + 16.0) * P_vis,
+        "duplicate_with_keys": 20.0 * P_vis + 8.0 * R_tot,
+        "sort_setup": 4.0 * R_tot,
+        "sort_onesweep": 16.0 * R_tot * passes,
+        "tile_ranges": 4.0 * R_tot + 16.0 * T * K,
+        # rows of the rendered Gaussians only: sums, mean, covariance, SH, scale, rotation in;
+        # the eight gradient rows out
+        "preprocess_backward": (309.0 + 284.0) * P_vis,
         "composite_forward": (20.0 * K + 20.0) * N,
         "composite_backward": (40.0 * K + 20.0) * N,
     }
