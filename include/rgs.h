@@ -101,8 +101,9 @@ int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const
  * rasterizer_impl.cu:198-287): per-Gaussian preprocess and the prefix sum of the tile
  * counts.  Writes radii[P], fills the geometry workspace and stores the number of
  * (Gaussian, tile) instances R to *num_rendered_host (host memory, preferably
- * pinned); the stream has been synchronised when the call returns, exactly where the
- * reference blocks on its device-to-host copy (rasterizer_impl.cu:287).
+ * pinned); the call returns when that copy has completed, which is where the reference
+ * blocks too (rasterizer_impl.cu:287); kernels that prepare the sort may still be running
+ * on the stream.
  * Exactly one of shs / colors_precomp and one of (scales, rotations) / cov3D_precomp
  * is non-NULL.  D = active SH degree (0..3), M = SH coefficients per Gaussian. */
 int rgs_forward_geom(int P, int D, int M, int width, int height,
@@ -114,18 +115,19 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
                      uint32_t* num_rendered_host, void* stream, int debug);
 
 /* rgs_forward_geom without the wait: enqueues the same work and the copy of R to
- * *num_rendered_pinned, which must be pinned host memory, and returns.  The caller reads R
- * after the stream (or an event recorded behind this call) has completed.  The reference
- * has no counterpart (it always blocks, rasterizer_impl.cu:287); this is for a caller that
- * renders several submodels of a frame on separate streams and wants every geometry stage
- * in flight before it waits for the first count. */
+ * *num_rendered_pinned, which must be pinned host memory, and returns.  count_ready_event
+ * (a hipEvent_t, or NULL) is recorded right behind that copy, ahead of the kernels that
+ * do not concern the host; the caller reads R once that event (or the whole stream) has
+ * completed.  The reference has no counterpart (it always blocks, rasterizer_impl.cu:287);
+ * this is for a caller that renders several submodels of a frame on separate streams and
+ * wants every geometry stage in flight before it waits for the first count. */
 int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
                      const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
                      const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
                      const float* viewmatrix, const float* projmatrix, const float* cam_pos,
                      float tan_fovx, float tan_fovy, int prefiltered,
                      int* radii, void* geom_ws, size_t geom_bytes,
-                     uint32_t* num_rendered_pinned, void* stream, int debug);
+                     uint32_t* num_rendered_pinned, void* count_ready_event, void* stream, int debug);
 
 /* Second half of Rasterizer::forward (rasterizer_impl.cu:289-351): key duplication,
  * stable sort of the (tile | depth) keys, tile ranges and the per-tile blend with the

@@ -46,7 +46,7 @@ def _load():
     lib.rgs_mark_visible.argtypes = [i, vp, vp, vp, vp, vp]
     lib.rgs_forward_geom.argtypes = [i, i, i, i, i, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, f, f, i,
                                      vp, vp, sz, vp, vp, i]
-    lib.rgs_forward_geom_enqueue.argtypes = lib.rgs_forward_geom.argtypes
+    lib.rgs_forward_geom_enqueue.argtypes = lib.rgs_forward_geom.argtypes[:-2] + [vp, vp, i]
     lib.rgs_forward_raster.argtypes = [i, i, i, i, vp, f, f, vp, vp, vp, vp, vp, vp, sz, vp, sz, vp, sz,
                                        vp, vp, vp, vp, i]
     lib.rgs_backward.argtypes = [i, i, i, i, i, i, vp, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, vp, vp, vp,

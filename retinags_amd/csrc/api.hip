@@ -328,7 +328,20 @@ static bool sh_rows_by_16_bytes(const float* shs, int M, int D)
 	return shs && (reinterpret_cast<uintptr_t>(shs) & 15) == 0 && (n & 3) == 0 && n <= 48 && needed <= n;
 }
 
-static int forward_geom(bool wait_for_count, const char* who, int P, int D, int M, int width, int height,
+// One event per host thread and device, for waiting on the copy of the instance count alone.
+static hipEvent_t count_event_of_this_thread()
+{
+	constexpr int kMaxDevices = 64;
+	static thread_local hipEvent_t events[kMaxDevices] = {};
+	int dev = 0;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+		return nullptr;
+	if (!events[dev] && hipEventCreateWithFlags(&events[dev], hipEventDisableTiming) != hipSuccess)
+		events[dev] = nullptr;
+	return events[dev];
+}
+
+static int forward_geom(bool wait_for_count, void* count_ready_event, const char* who, int P, int D, int M, int width, int height,
                         const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
                         const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
                         const float* viewmatrix, const float* projmatrix, const float* cam_pos,
@@ -391,6 +404,10 @@ static int forward_geom(bool wait_for_count, const char* who, int P, int D, int 
 	RGS_STAGE("instance count");
 	hipError_t e = hipMemcpyAsync(num_rendered_host, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), sizeof(uint32_t),
 	                              hipMemcpyDeviceToHost, s);
+	// the host only needs the count: it waits for this event, not for the kernels queued below
+	hipEvent_t ready = wait_for_count ? count_event_of_this_thread() : static_cast<hipEvent_t>(count_ready_event);
+	if (e == hipSuccess && ready)
+		e = hipEventRecord(ready, s);
 	{
 		// depth order of the Gaussians and the offsets of their instances in that order: needs
 		// nothing from the host, so it is queued behind the count's copy
@@ -405,7 +422,7 @@ static int forward_geom(bool wait_for_count, const char* who, int P, int D, int 
 		RGS_STAGE("depth order");
 	}
 	if (e == hipSuccess && wait_for_count)
-		e = hipStreamSynchronize(s);
+		e = ready ? hipEventSynchronize(ready) : hipStreamSynchronize(s);
 	if (e != hipSuccess)
 		return fail("%s: reading the instance count failed: %s", who, hipGetErrorString(e));
 	if (wait_for_count)
@@ -422,7 +439,7 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
                      int* radii, void* geom_ws, size_t geom_bytes,
                      uint32_t* num_rendered_host, void* stream, int debug)
 {
-	return forward_geom(true, "rgs_forward_geom", P, D, M, width, height, means3D, shs, colors_precomp, opacities, scales,
+	return forward_geom(true, nullptr, "rgs_forward_geom", P, D, M, width, height, means3D, shs, colors_precomp, opacities, scales,
 	                    scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, cam_pos, tan_fovx, tan_fovy,
 	                    prefiltered, radii, geom_ws, geom_bytes, num_rendered_host, stream, debug);
 }
@@ -433,9 +450,9 @@ int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
                              const float* cov3D_precomp, const float* viewmatrix, const float* projmatrix,
                              const float* cam_pos, float tan_fovx, float tan_fovy, int prefiltered,
                              int* radii, void* geom_ws, size_t geom_bytes,
-                             uint32_t* num_rendered_pinned, void* stream, int debug)
+                             uint32_t* num_rendered_pinned, void* count_ready_event, void* stream, int debug)
 {
-	return forward_geom(false, "rgs_forward_geom_enqueue", P, D, M, width, height, means3D, shs, colors_precomp, opacities,
+	return forward_geom(false, count_ready_event, "rgs_forward_geom_enqueue", P, D, M, width, height, means3D, shs, colors_precomp, opacities,
 	                    scales, scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, cam_pos, tan_fovx,
 	                    tan_fovy, prefiltered, radii, geom_ws, geom_bytes, num_rendered_pinned, stream, debug);
 }

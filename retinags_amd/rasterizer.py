@@ -85,7 +85,15 @@ class GeometryStage:
                 and not self.used)
 
 
-_free_pinned_words = []
+_free_count_slots = {}   # per device: (pinned word, event) pairs of finished calls, for reuse
+
+
+def _new_count_slot(device):
+    """A pinned word for an instance count and the event that says it has arrived."""
+    event = torch.cuda.Event()
+    event.record(torch.cuda.current_stream(device))  # the first record creates the hipEvent_t
+    return torch.zeros(1, dtype=torch.int32).pin_memory(), event
+
 
 
 def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations, scale_modifier, cov3Ds_precomp,
@@ -124,21 +132,21 @@ def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations,
     with torch.cuda.device(device):
         st.geom_bytes = lib.rgs_geom_bytes(st.P)
         st.geomBuffer = torch.empty(st.geom_bytes, **byte)
+        args = (st.P, int(sh_degree), M, st.W, st.H, ptr(t["means3D"]), ptr(t["sh"]), ptr(t["colors_precomp"]),
+                ptr(t["opacities"]), ptr(t["scales"]), float(scale_modifier), ptr(t["rotations"]),
+                ptr(t["cov3Ds_precomp"]), ptr(t["viewmatrix"]), ptr(t["projmatrix"]), ptr(t["campos"]),
+                float(tanfovx), float(tanfovy), int(bool(prefiltered)), ptr(st.radii), ptr(st.geomBuffer),
+                st.geom_bytes)
         if wait:
             st.count = _pinned_word(device)
-            entry = lib.rgs_forward_geom
+            check(lib.rgs_forward_geom(*args, C.c_void_p(st.count.data_ptr()), C.c_void_p(st.stream),
+                                       int(bool(debug))))
         else:
-            st.count = _free_pinned_words.pop() if _free_pinned_words else torch.zeros(1, dtype=torch.int32).pin_memory()
-            entry = lib.rgs_forward_geom_enqueue
-        check(entry(
-            st.P, int(sh_degree), M, st.W, st.H, ptr(t["means3D"]), ptr(t["sh"]), ptr(t["colors_precomp"]),
-            ptr(t["opacities"]), ptr(t["scales"]), float(scale_modifier), ptr(t["rotations"]),
-            ptr(t["cov3Ds_precomp"]), ptr(t["viewmatrix"]), ptr(t["projmatrix"]), ptr(t["campos"]), float(tanfovx),
-            float(tanfovy), int(bool(prefiltered)), ptr(st.radii), ptr(st.geomBuffer), st.geom_bytes,
-            C.c_void_p(st.count.data_ptr()), C.c_void_p(st.stream), int(bool(debug))))
-        if not wait:
-            st.event = torch.cuda.Event()
-            st.event.record(torch.cuda.current_stream(device))
+            free = _free_count_slots.setdefault((device.type, device.index), [])
+            st.count, st.event = free.pop() if free else _new_count_slot(device)
+            check(lib.rgs_forward_geom_enqueue(*args, C.c_void_p(st.count.data_ptr()),
+                                               C.c_void_p(st.event.cuda_event), C.c_void_p(st.stream),
+                                               int(bool(debug))))
     return st
 
 
@@ -162,16 +170,18 @@ def _forward_blend(st: GeometryStage):
         return 0, out_color, out_depth, out_alpha, st.radii, empty, empty, empty
     t = st.tensors
     with torch.cuda.device(device):
+        image_bytes = lib.rgs_image_bytes(W, H)
+        imgBuffer = torch.empty(image_bytes, **byte)
         if st.event is not None:
             st.event.synchronize()
             rendered = int(st.count.item())
-            _free_pinned_words.append(st.count)
+            _free_count_slots[(device.type, device.index)].append((st.count, st.event))
             st.event = None
         else:
             rendered = int(st.count.item())
         st.count = None
-        image_bytes = lib.rgs_image_bytes(W, H)
-        imgBuffer = torch.empty(image_bytes, **byte)
+        if rendered >= 1 << 30:
+            raise _capi.RgsError(f"{rendered} (Gaussian, tile) instances exceed the 2^30 limit of the sort")
         binning_bytes = lib.rgs_binning_bytes(rendered) if rendered > 0 else 0
         binningBuffer = torch.empty(binning_bytes, **byte)
         check(lib.rgs_forward_raster(
