@@ -10,6 +10,7 @@ the rasterizer runs in the HIP library.
 from __future__ import annotations
 
 import ctypes as C
+import math
 from typing import NamedTuple
 
 import torch
@@ -199,13 +200,21 @@ def _rasterize_forward(*args):
 
 
 def _gradient_outputs(P, M, has_scales, device, make):
-    """The eight dense gradient tensors of K/rasterize_points.cu:165-174, made with `make`
-    (torch.empty or torch.zeros); without scales the scale / rotation gradients are zeros."""
-    f32 = dict(dtype=torch.float32, device=device)
-    return {"means2D": make((P, 3), **f32), "opacity": make((P, 1), **f32), "colors": make((P, 3), **f32),
-            "means3D": make((P, 3), **f32), "cov3D": make((P, 6), **f32), "sh": make((P, M, 3), **f32),
-            "scales": (make if has_scales else torch.zeros)((P, 3), **f32),
-            "rotations": (make if has_scales else torch.zeros)((P, 4), **f32)}
+    """The eight dense gradient tensors of K/rasterize_points.cu:165-174, carved out of one
+    allocation made with `make` (torch.empty or torch.zeros: one fill instead of eight);
+    without scales the scale / rotation gradients are zeros in either case."""
+    shapes = {"means2D": (P, 3), "opacity": (P, 1), "colors": (P, 3), "means3D": (P, 3), "cov3D": (P, 6),
+              "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4)}
+    sizes = {k: (math.prod(v) + 63) // 64 * 64 for k, v in shapes.items()}  # 256-byte aligned parts
+    flat = make((sum(sizes.values()),), dtype=torch.float32, device=device)
+    out, at = {}, 0
+    for k, shape in shapes.items():
+        out[k] = flat[at:at + math.prod(shape)].view(shape)
+        at += sizes[k]
+    if not has_scales and make is not torch.zeros:
+        out["scales"].zero_()
+        out["rotations"].zero_()
+    return out
 
 
 def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, scale_modifier, cov3Ds_precomp,
