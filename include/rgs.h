@@ -80,6 +80,8 @@ enum {
 enum {
 	RGS_IMG_RANGES = 0,         /* uint2[tiles]  [start, end) of each tile in the sorted list */
 	RGS_IMG_N_CONTRIB,          /* uint32[H*W]   list position of the last blended Gaussian */
+	RGS_IMG_STRIP_SPAN,         /* uint32[4*tiles] largest n_contrib of each 16x4 strip (tile * 4 + strip) */
+	RGS_IMG_STRIP_ORDER,        /* uint32[4*tiles] the strips by decreasing span: the order the backward blend takes them in */
 	RGS_IMG_FIELDS
 };
 int rgs_geom_layout(int P, size_t offsets[RGS_GEOM_FIELDS]);

@@ -16,7 +16,7 @@ GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles
                "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
                "visible_list", "order_scratch")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
-IMG_FIELDS = ("ranges", "n_contrib")
+IMG_FIELDS = ("ranges", "n_contrib", "strip_span", "strip_order")
 ACC_FLOATS = 12
 MAX_COMPOSITE = 64
 

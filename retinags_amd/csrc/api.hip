@@ -170,8 +170,10 @@ size_t image_layout(int width, int height, size_t* off)
 {
 	const size_t tiles = (size_t)((width + rgs::kTile - 1) / rgs::kTile) * (size_t)((height + rgs::kTile - 1) / rgs::kTile);
 	Carver c;
-	off[RGS_IMG_RANGES] = c.take(8 * tiles);
+	off[RGS_IMG_RANGES] = c.take(8 * tiles + 4 * rgs::kRangeTailWords);  // + the strip class counters, cleared with it
 	off[RGS_IMG_N_CONTRIB] = c.take(4 * (size_t)width * height);
+	off[RGS_IMG_STRIP_SPAN] = c.take(4 * 4 * tiles);
+	off[RGS_IMG_STRIP_ORDER] = c.take(4 * 4 * tiles);
 	return c.cursor;
 }
 
@@ -538,6 +540,9 @@ int rgs_forward_raster(int P, int R, int width, int height,
 	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 	a.out_color = out_color; a.out_depth = out_depth; a.out_alpha = out_alpha;
 	a.n_contrib = at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]);
+	a.strip_span = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_SPAN]);
+	a.strip_order = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_ORDER]);
+	a.strip_classes = reinterpret_cast<uint32_t*>(ranges) + 2 * (size_t)gx * gy;
 	rgs::launch_blend_forward(a, s);
 	RGS_STAGE("blend_forward");
 	return 0;
@@ -597,6 +602,8 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 		a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 		a.out_alpha = const_cast<float*>(alphas);
 		a.n_contrib = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]));
+		a.strip_span = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_SPAN]));
+		a.strip_order = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_ORDER]));
 		a.dL_dpix = dL_dpix; a.dL_dpix_depth = dL_dpix_depth; a.dL_dalpha = dL_dalphas;
 		a.sums = grad_accum;
 		rgs::launch_blend_backward(a, s);

@@ -555,7 +555,7 @@ void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles
                         const uint32_t* order_status, hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
-	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2, s);
+	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2 + kRangeTailWords, s);
 	if (n == 0)
 		return;
 	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges,

@@ -137,6 +137,10 @@ __device__ __forceinline__ int classify_strip_against_box(float w, const StripCo
 	return outside ? kBoxOutside : (inside ? kBoxInside : kBoxMixed);
 }
 
+// Launch-order classes of the backward's strips, by the length of list they have to walk.
+constexpr int kStripClasses = 256;
+__device__ __forceinline__ uint32_t strip_class(uint32_t span) { return 255u - min(span >> 4, 255u); }
+
 constexpr int kPerLane = 1;             // list entries per lane and step (2 was measured slower)
 constexpr int kChunk = 64 * kPerLane;   // list entries a wavefront takes per step
 
@@ -328,6 +332,14 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 		}
 	}
 
+	{
+		uint32_t span = inside ? p.last_contributor : 0u;
+#pragma unroll
+		for (int off = 32; off > 0; off >>= 1)
+			span = max(span, (uint32_t)__shfl_xor((int)span, off));
+		if (lane == 0)
+			a.strip_span[4 * tile + wave] = span;
+	}
 	if (inside) {
 		const size_t plane = (size_t)a.H * a.W;
 		a.n_contrib[pix_id] = p.last_contributor;
@@ -586,10 +598,9 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 	__shared__ BackwardStage s_stage;
 
 	const int lane = threadIdx.x;
-	int wave;  // which strip of the tile
-	const int tile = tile_of_strip_block((int)blockIdx.x, a.grid_x, a.grid_y, wave);
-	if (tile < 0)
-		return;
+	// longest strips first: a long strip that starts late is what the whole launch waits for
+	const uint32_t strip_id = a.strip_order[blockIdx.x];
+	const int tile = (int)(strip_id >> 2), wave = (int)(strip_id & 3u);  // wave: which strip of the tile
 	const uint2 range = a.ranges[tile];
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
@@ -705,19 +716,73 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 		flush_rows(st, rows, frame, a, lane);
 }
 
+// Strips by decreasing span, in kStripClasses classes of 16 list entries (longer ones share
+// the first class); the order inside a class is whatever the atomics give, which is all a
+// launch order needs.  Two small kernels: count the strips of every class, then place them.
+// Both aggregate in LDS first: most strips fall into one class (nothing to walk), and
+// thousands of global atomics on one word would take longer than the blend itself.
+__global__ __launch_bounds__(256) void strip_count_kernel(const uint32_t* __restrict__ span, uint32_t n,
+                                                           uint32_t* __restrict__ class_count)
+{
+	__shared__ uint32_t s_count[kStripClasses];
+	s_count[threadIdx.x] = 0;
+	__syncthreads();
+	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+	if (k < n)
+		atomicAdd(&s_count[strip_class(span[k])], 1u);
+	__syncthreads();
+	if (s_count[threadIdx.x] != 0u)
+		atomicAdd(&class_count[threadIdx.x], s_count[threadIdx.x]);
+}
+
+__global__ __launch_bounds__(256) void strip_place_kernel(const uint32_t* __restrict__ span, uint32_t n,
+                                                           const uint32_t* __restrict__ class_count,
+                                                           uint32_t* __restrict__ class_cursor,
+                                                           uint32_t* __restrict__ order)
+{
+	__shared__ uint32_t s_count[kStripClasses];  // strips of this block per class, then where they go
+	__shared__ uint32_t s_scan[8];
+	s_count[threadIdx.x] = 0;
+	__syncthreads();
+	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+	uint32_t c = 0, rank = 0;
+	if (k < n) {
+		c = strip_class(span[k]);
+		rank = atomicAdd(&s_count[c], 1u);
+	}
+	__syncthreads();
+	uint32_t total;
+	const uint32_t start = block256_exclusive_scan_u32(class_count[threadIdx.x], s_scan, total);
+	const uint32_t mine = s_count[threadIdx.x];
+	__syncthreads();
+	s_count[threadIdx.x] = start + (mine != 0u ? atomicAdd(&class_cursor[threadIdx.x], mine) : 0u);
+	__syncthreads();
+	if (k < n)
+		order[s_count[c] + rank] = k;
+}
+
 void launch_blend_forward(const BlendArgs& a, hipStream_t s)
 {
 	stage_mark(a.counters ? "blend_count" : "blend_forward", s);
 	if (a.counters)
 		hipLaunchKernelGGL(blend_count_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
 	else
+	{
 		hipLaunchKernelGGL(blend_forward_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
+		// the order in which the backward will take the strips (longest first was measured no
+		// faster for the forward's tiles, whose length is only known as the list length)
+		const uint32_t strips = (uint32_t)(4 * a.grid_x * a.grid_y);
+		hipLaunchKernelGGL(strip_count_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_span, strips,
+		                   a.strip_classes);
+		hipLaunchKernelGGL(strip_place_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_span, strips,
+		                   a.strip_classes, a.strip_classes + kStripClasses, a.strip_order);
+	}
 }
 
 void launch_blend_backward(const BlendArgs& a, hipStream_t s)
 {
 	stage_mark("blend_backward", s);
-	hipLaunchKernelGGL(blend_backward_kernel, dim3(strip_order_blocks(a.grid_x, a.grid_y)), dim3(64), 0, s, a);
+	hipLaunchKernelGGL(blend_backward_kernel, dim3(4 * a.grid_x * a.grid_y), dim3(64), 0, s, a);
 }
 
 }  // namespace rgs

@@ -88,6 +88,9 @@ struct BlendArgs {
 	float* out_depth;
 	float* out_alpha;
 	uint32_t* n_contrib;
+	uint32_t* strip_span;   // per 16x4 strip (tile * 4 + strip): the largest n_contrib of its pixels
+	uint32_t* strip_order;  // strips by decreasing span, written behind the forward blend
+	uint32_t* strip_classes;  // 2 x 256 words, zero before the forward blend: strips per span class, placement cursors
 	uint64_t* counters;  // non-null selects the work-accounting twin of the forward blend (7 sums)
 	// backward
 	const float* dL_dpix;
@@ -163,7 +166,9 @@ void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in,
 void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                            const uint32_t* n_device, int end_bit, uint32_t* temp, const char* stage, hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
-// Either status word (may be null) being non-zero leaves every range empty.
+// Either status word (may be null) being non-zero leaves every range empty.  Clears `ranges` and
+// the kRangeTailWords words behind it (the strip class counters of the blend).
+constexpr int kRangeTailWords = 512;
 void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
                         const uint32_t* order_status, hipStream_t s);
 

@@ -49,23 +49,4 @@ RGS_HOST_DEVICE inline int tile_of_block(int b, int grid_x, int grid_y)
 	return row * grid_x + col;
 }
 
-// The blend kernels run one wavefront per workgroup, a workgroup per strip (4 strips of
-// 16x4 pixels make a tile): strips end at very different times, and a slot freed by a short
-// strip should go to the next strip at once instead of idling until its tile's longest strip
-// is done.  The four strips of a tile take four consecutive turns of the same XCD.
-constexpr int kStripsPerTile = 4;
-
-RGS_HOST_DEVICE inline int strip_order_blocks(int grid_x, int grid_y)
-{
-	return kStripsPerTile * tile_order_blocks(grid_x, grid_y);
-}
-
-// Tile of strip-workgroup `b` (-1: none) and, in `strip`, which quarter of the tile it takes.
-RGS_HOST_DEVICE inline int tile_of_strip_block(int b, int grid_x, int grid_y, int& strip)
-{
-	const int xcd = b % kXcds, turn = b / kXcds;
-	strip = turn % kStripsPerTile;
-	return tile_of_block((turn / kStripsPerTile) * kXcds + xcd, grid_x, grid_y);
-}
-
 }  // namespace rgs

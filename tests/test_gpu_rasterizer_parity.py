@@ -61,6 +61,16 @@ def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
     im = _capi.image_layout(W, H)
     assert np.array_equal(view_ws(img, im["ranges"], 2 * T, np.uint32).reshape(T, 2), st.ranges)
 
+    # ---- the order in which the backward blend takes the 16x4 strips: longest span first
+    spans = view_ws(img, im["strip_span"], 4 * T, np.uint32)
+    order = view_ws(img, im["strip_order"], 4 * T, np.uint32)
+    assert np.array_equal(np.sort(order), np.arange(4 * T, dtype=np.uint32))
+    assert (np.diff(np.minimum(spans[order] >> 4, 255).astype(np.int64)) <= 0).all()
+    nc = np.zeros((s.grid[1] * 16, s.grid[0] * 16), np.uint32)
+    nc[:H, :W] = view_ws(img, im["n_contrib"], H * W, np.uint32).reshape(H, W)
+    per_strip = nc.reshape(s.grid[1], 4, 4, s.grid[0], 16).max(axis=(2, 4)).transpose(0, 2, 1).reshape(-1)
+    assert np.array_equal(spans, per_strip)
+
     # ---- blend: tolerance, away from decision thresholds
     n_contrib = view_ws(img, im["n_contrib"], H * W, np.uint32)
     safe = (st.margin > DECISION_MARGIN).reshape(H, W)

@@ -31,34 +31,6 @@ int main()
 					return 1;
 				}
 		}
-	// strip workgroups: every (tile, strip) exactly once, the strips of a tile on one XCD
-	for (int gx = 1; gx <= 30; gx += 7)
-		for (int gy = 1; gy <= 40; gy += 3) {
-			const int n = gx * gy;
-			std::vector<int> seen(n * rgs::kStripsPerTile, 0), home(n, -1);
-			const int blocks = rgs::strip_order_blocks(gx, gy);
-			for (int b = 0; b < blocks; b++) {
-				int strip = -1;
-				const int t = rgs::tile_of_strip_block(b, gx, gy, strip);
-				if (t < 0)
-					continue;
-				if (t >= n || strip < 0 || strip >= rgs::kStripsPerTile) {
-					std::printf("strip block %d of %dx%d out of range\n", b, gx, gy);
-					return 1;
-				}
-				seen[t * rgs::kStripsPerTile + strip]++;
-				if (home[t] >= 0 && home[t] != b % rgs::kXcds) {
-					std::printf("%dx%d: tile %d split over XCDs\n", gx, gy, t);
-					return 1;
-				}
-				home[t] = b % rgs::kXcds;
-			}
-			for (int v : seen)
-				if (v != 1) {
-					std::printf("%dx%d: a strip taken %d times\n", gx, gy, v);
-					return 1;
-				}
-		}
 	// most neighbours along a row share an XCD: in a 100x65 grid, tiles (r, c) and (r, c+1)
 	const int gx = 100, gy = 65, blocks = rgs::tile_order_blocks(gx, gy);
 	std::vector<int> xcd(gx * gy, -1);
