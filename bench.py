@@ -54,6 +54,8 @@ def parse():
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--streams", type=int, default=4,
                     help="render the submodels of a frame on this many HIP streams (0: all on the current stream)")
+    ap.add_argument("--host-threads", action="store_true",
+                    help="issue each stream's forward calls from a host thread of its own")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device-to-device copy, the known-size reference for HBM traffic counters")
     return ap.parse_args()
@@ -114,7 +116,7 @@ def main():
         for s in subs:
             for p in s.parameters():
                 p.grad = None
-        out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams)
+        out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=args.host_threads)
         if do_backward:
             torch.autograd.backward([out["render"]], [upstream])
         return out

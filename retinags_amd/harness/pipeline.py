@@ -111,7 +111,7 @@ def _host_pool(n: int):
 
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
                  submodel_bg: Optional[torch.Tensor] = None,
-                 streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = True) -> dict:
+                 streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = False) -> dict:
     """Render every related submodel (black background, as the trainer does:
     trainer4tree_partition.py:397) and composite the partial images in BVH order.
 
@@ -120,10 +120,11 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     streams[k % len(streams)] (default priority), so one submodel's short kernels and the tail
     of its blend run beside another's; autograd replays each submodel's backward on the stream
     its forward used.  The compositor runs on the caller's stream after all of them.  The
-    With host_threads each stream's forward calls are issued by a host thread of their own (the
-    library releases no lock but ctypes releases the interpreter's while inside it); without, the
-    forward is issued in two rounds (all geometry stages, then all sort-and-blend stages): the
+    The forward is issued in two rounds (all geometry stages, then all sort-and-blend stages): the
     host has to read each submodel's instance count in between, and this way it waits once.
+    With host_threads each stream's forward calls are instead issued by a host thread of their
+    own (ctypes releases the interpreter lock inside the library); measured no faster, and less
+    steady, than the two rounds: the threads contend for the interpreter between the calls.
     """
     device = subs[0].means3D.device
     if submodel_bg is None:
