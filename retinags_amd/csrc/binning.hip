@@ -235,7 +235,7 @@ void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint
 // ordered by their id, so every pass is stable.
 //
 // Scratch layout (u32 words):
-//   [0, 2048)      digit histograms of up to 8 passes, turned into exclusive digit starts
+//   [0, 2048)      digit histograms of up to 8 passes (every block of a pass scans its 256 counts itself)
 //   [2048, 2056)   tile counter of each pass
 //   [2056]         status: non-zero if a look-back ever gave up waiting (never expected)
 //   [kSortHeader + pass * 256 * tiles + tile * 256 + digit]  look-back words
@@ -284,24 +284,13 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const KeyT* _
 	}
 }
 
-__global__ __launch_bounds__(256) void sort_digit_starts_kernel(uint32_t* __restrict__ hist, int passes)
-{
-	__shared__ uint32_t lds[8];
-	for (int p = 0; p < passes; p++) {
-		uint32_t total;
-		const uint32_t c = hist[p * 256 + threadIdx.x];
-		const uint32_t ex = block256_exclusive_scan_u32(c, lds, total);
-		hist[p * 256 + threadIdx.x] = ex;
-	}
-}
-
 template <typename KeyT>
 __global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restrict__ keys_in,
                                                              const uint32_t* __restrict__ vals_in,
                                                              KeyT* __restrict__ keys_out,
                                                              uint32_t* __restrict__ vals_out, size_t n,
                                                              const uint32_t* __restrict__ n_device, int shift,
-                                                             uint32_t mask, const uint32_t* __restrict__ digit_start,
+                                                             uint32_t mask, const uint32_t* __restrict__ digit_count,
                                                              uint32_t* __restrict__ lookback,
                                                              uint32_t* __restrict__ tile_counter,
                                                              uint32_t* __restrict__ status)
@@ -423,7 +412,10 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restri
 			__hip_atomic_store(my_word, ((exclusive + count) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
 			                   __HIP_MEMORY_SCOPE_AGENT);
 		}
-		s_global_base[tid] = digit_start[tid] + exclusive;
+		// where the digit's run starts in the whole array: the exclusive scan of the digit counts
+		uint32_t all;
+		const uint32_t digit_start = block256_exclusive_scan_u32(digit_count[tid], s_scan, all);
+		s_global_base[tid] = digit_start + exclusive;
 	}
 	__syncthreads();
 
@@ -479,7 +471,6 @@ static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_
 	const uint32_t hist_blocks = tiles < 2048u ? tiles : 2048u;
 	hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks), dim3(256), 0, s, keys_in, n, n_device, passes,
 	                   end_bit, temp);
-	hipLaunchKernelGGL(sort_digit_starts_kernel, dim3(1), dim3(256), 0, s, temp, passes);
 	KeyT *ksrc = keys_in, *kdst = keys_out;
 	uint32_t *vsrc = vals_in, *vdst = vals_out;
 	for (int p = 0; p < passes; p++) {
