@@ -161,13 +161,24 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __
 	}
 }
 
+// out[k] = in[index[k]] for k below the count on the device, and the sum of every 256 of them
+// (the first level of the scan that follows).
 __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ n_device,
                                                           const uint32_t* __restrict__ index,
-                                                          const uint32_t* __restrict__ in, uint32_t* __restrict__ out)
+                                                          const uint32_t* __restrict__ in, uint32_t* __restrict__ out,
+                                                          uint32_t* __restrict__ block_totals)
 {
+	__shared__ uint32_t lds[8];
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
-	if (k < *n_device)
-		out[k] = in[index[k]];
+	uint32_t v = 0;
+	if (k < *n_device) {
+		v = in[index[k]];
+		out[k] = v;
+	}
+	uint32_t total;
+	(void)block256_exclusive_scan_u32(v, lds, total);
+	if (threadIdx.x == 0)
+		block_totals[blockIdx.x] = total;
 }
 
 // Thread k takes the k-th Gaussian in depth order and writes its instances, tiles row by row
@@ -211,8 +222,11 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
 	// 4 passes: the sorted pairs end up in the first buffer pair again
 	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, nullptr, s);
 	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched,
-	                   tiles_in_order);
-	inclusive_sum(tiles_in_order, offsets_in_order, (size_t)P, visible_count, scan_temp, s);
+	                   tiles_in_order, scan_temp);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan_temp, (size_t)nb,
+	                   visible_count, (uint32_t*)nullptr);
+	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3(nb), dim3(256), 0, s, tiles_in_order, scan_temp, (size_t)P,
+	                   visible_count, offsets_in_order);
 }
 
 void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
