@@ -20,8 +20,9 @@ namespace rgs {
 // ---- prefix sums ---------------------------------------------------------------------------
 // Replaces cub::DeviceScan::InclusiveSum at K/cuda_rasterizer_hgs/rasterizer_impl.cu:283
 // with three small kernels: per-256 block totals, one single-block scan of those totals,
-// and a per-block scan that adds the block's base.  The forward preprocess kernel already
-// emits the block totals, so the rasterizer path only runs the last two.
+// and a per-block scan that adds the block's base.  On the rasterizer path the block totals
+// come from the kernel that produces the values (the forward preprocess, the gather of the
+// depth order), so only the last two run there.
 
 // In all three kernels a non-null n_device overrides n (the launch is then sized for an upper bound).
 __global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __restrict__ in, size_t n,
@@ -124,17 +125,6 @@ void launch_total_from_block_sums(uint32_t* block_sums, int P, uint32_t* total_o
 	stage_mark("offset_scan", s);
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb,
 	                   (const uint32_t*)nullptr, total_out);
-}
-
-void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* block_sums, uint32_t* offsets, int P,
-                                    uint32_t* total_out, hipStream_t s)
-{
-	const size_t nb = ((size_t)P + 255) / 256;
-	stage_mark("offset_scan", s);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb,
-	                   (const uint32_t*)nullptr, total_out);
-	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, tiles_touched, block_sums,
-	                   (size_t)P, (const uint32_t*)nullptr, offsets);
 }
 
 // ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------

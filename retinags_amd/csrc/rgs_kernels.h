@@ -140,8 +140,6 @@ void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t*
                           hipStream_t s);
 // Scans the per-256 block sums of the tile counts in place; *total_out = number of instances.
 void launch_total_from_block_sums(uint32_t* block_sums, int P, uint32_t* total_out, hipStream_t s);
-void launch_offsets_from_block_sums(const uint32_t* tiles_touched, uint32_t* block_sums, uint32_t* offsets, int P,
-                                    uint32_t* total_out, hipStream_t s);
 // Depth order of the Gaussians that touch a tile.  block_visible holds their count per 256
 // Gaussians (scanned in place; the total goes to *visible_count).  On return order[0..count)
 // lists them by increasing depth, ties by index, and offsets_in_order is the inclusive scan of
