@@ -400,9 +400,13 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 	a.block_visible = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_VISIBLE]);
 	a.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D);
 
+	const OrderScratch order = order_scratch((size_t)P);
+	a.clear = at<uint32_t>(at<char>(geom_ws, off[RGS_GEOM_ORDER_SCRATCH]), order.sort_temp);
+	a.clear_words = rgs::sort_clear_words((size_t)P, 32);
 	rgs::launch_preprocess_forward(a, s);
 	RGS_STAGE("preprocess");
-	rgs::launch_total_from_block_sums(a.block_sums, P, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), s);
+	rgs::launch_totals_from_block_sums(a.block_sums, a.block_visible, P, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]),
+	                                   at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_COUNT]), s);
 	RGS_STAGE("instance count");
 	hipError_t e = hipMemcpyAsync(num_rendered_host, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), sizeof(uint32_t),
 	                              hipMemcpyDeviceToHost, s);
@@ -413,7 +417,7 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 	{
 		// depth order of the Gaussians and the offsets of their instances in that order: needs
 		// nothing from the host, so it is queued behind the count's copy
-		const OrderScratch o = order_scratch((size_t)P);
+		const OrderScratch& o = order;
 		char* scratch = at<char>(geom_ws, off[RGS_GEOM_ORDER_SCRATCH]);
 		rgs::launch_depth_order(P, a.depths, a.tiles_touched, a.block_visible, at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_COUNT]),
 		                        at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_LIST]),
@@ -499,10 +503,13 @@ int rgs_forward_raster(int P, int R, int width, int height,
 		rgs::launch_duplicate_with_keys(P, at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]),
 		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_DEPTH_ORDER]),
 		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_POINT_OFFSETS]), at<float2>(geom_ws, goff[RGS_GEOM_XY]),
-		                                radii, gx, gy, keys_a, vals_a, s);
+		                                radii, gx, gy, keys_a, vals_a, at<uint32_t>(binning_ws, b.temp),
+		                                rgs::sort_clear_words((size_t)R, tile_key_bits(width, height)), s);
 		RGS_STAGE("duplicate_with_keys");
 		const int end_bit = tile_key_bits(width, height);
+		// the first kernel of the sort also clears the tile ranges (and the counters behind them)
 		rgs::launch_sort_pairs_u32(keys_a, keys_b, vals_a, vals_b, (size_t)R, nullptr, end_bit, at<uint32_t>(binning_ws, b.temp),
+		                           true, reinterpret_cast<uint32_t*>(ranges), (size_t)gx * gy * 2 + rgs::kRangeTailWords,
 		                           "sort", s);
 		RGS_STAGE("sort_pairs");
 		const bool sorted_in_a = (((end_bit + 7) / 8) % 2) == 0;
@@ -517,11 +524,11 @@ int rgs_forward_raster(int P, int R, int width, int height,
 				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
 		}
 		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, ranges, gx * gy,
-		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, s);
+		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, true, s);
 		RGS_STAGE("tile_ranges");
 		point_list = sorted_in_a ? vals_a : vals_b;
 	} else {
-		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, nullptr, nullptr, s);
+		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, nullptr, nullptr, false, s);
 		RGS_STAGE("tile_ranges");
 	}
 

@@ -42,11 +42,18 @@ __global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __res
 
 // In-place exclusive scan of `data[0..n)` by one block of 1024 threads; the grand total goes
 // to *total_out (if non-null).
+// Block 1, if launched, does the same for a second array of the same length.
 __global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(uint32_t* __restrict__ data, size_t n,
                                                                             const uint32_t* __restrict__ n_device,
-                                                                            uint32_t* __restrict__ total_out)
+                                                                            uint32_t* __restrict__ total_out,
+                                                                            uint32_t* __restrict__ data_b,
+                                                                            uint32_t* __restrict__ total_out_b)
 {
 	__shared__ uint32_t wave_tot[16];
+	if (blockIdx.x == 1) {
+		data = data_b;
+		total_out = total_out_b;
+	}
 	if (n_device)
 		n = ((size_t)*n_device + 255) / 256;  // one entry per 256 elements
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -105,7 +112,7 @@ static void inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, const uin
 	const size_t nb = (n + 255) / 256;
 	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, n_device, temp);
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, nb, n_device,
-	                   (uint32_t*)nullptr);
+	                   (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr);
 	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, temp, n, n_device, out);
 }
 
@@ -119,12 +126,13 @@ void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t*
 	inclusive_sum(in, out, n, nullptr, temp, s);
 }
 
-void launch_total_from_block_sums(uint32_t* block_sums, int P, uint32_t* total_out, hipStream_t s)
+void launch_totals_from_block_sums(uint32_t* block_sums, uint32_t* block_visible, int P, uint32_t* total_out,
+                                   uint32_t* visible_count, hipStream_t s)
 {
 	const size_t nb = ((size_t)P + 255) / 256;
 	stage_mark("offset_scan", s);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_sums, nb,
-	                   (const uint32_t*)nullptr, total_out);
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(2), dim3(1024), 0, s, block_sums, nb,
+	                   (const uint32_t*)nullptr, total_out, block_visible, visible_count);
 }
 
 // ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------
@@ -179,9 +187,13 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t
                                                                    const float2* __restrict__ xy,
                                                                    const int* __restrict__ radii, int gx, int gy,
                                                                    uint32_t* __restrict__ keys,
-                                                                   uint32_t* __restrict__ values)
+                                                                   uint32_t* __restrict__ values,
+                                                                   uint32_t* __restrict__ clear, size_t clear_words)
 {
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+	// the scratch of the sort that follows is cleared here, which saves a launch
+	for (size_t w = k; w < clear_words; w += (size_t)gridDim.x * 256)
+		clear[w] = 0u;
 	if (k >= *visible_count)
 		return;
 	const uint32_t idx = order[k];
@@ -205,27 +217,27 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
 {
 	const unsigned nb = (unsigned)((P + 255) / 256);
 	stage_mark("depth_order", s);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, block_visible, (size_t)nb,
-	                   (const uint32_t*)nullptr, visible_count);
 	hipLaunchKernelGGL(depth_pairs_kernel, dim3(nb), dim3(256), 0, s, P, depths, tiles_touched, block_visible, keys_a,
 	                   order, visible_list);
 	// 4 passes: the sorted pairs end up in the first buffer pair again
-	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, nullptr, s);
+	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, true, nullptr, 0, nullptr,
+	                      s);
 	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched,
 	                   tiles_in_order, scan_temp);
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan_temp, (size_t)nb,
-	                   visible_count, (uint32_t*)nullptr);
+	                   visible_count, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr);
 	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3(nb), dim3(256), 0, s, tiles_in_order, scan_temp, (size_t)P,
 	                   visible_count, offsets_in_order);
 }
 
 void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
                                 const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
-                                int grid_y, uint32_t* keys, uint32_t* values, hipStream_t s)
+                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t* clear, size_t clear_words,
+                                hipStream_t s)
 {
 	stage_mark("duplicate_with_keys", s);
 	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, visible_count, order,
-	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values);
+	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values, clear, clear_words);
 }
 
 // ---- radix sort -------------------------------------------------------------------------------
@@ -263,9 +275,12 @@ template <typename KeyT>
 __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const KeyT* __restrict__ keys, size_t n,
                                                                     const uint32_t* __restrict__ n_device,
                                                                     int passes, int end_bit,
-                                                                    uint32_t* __restrict__ hist)
+                                                                    uint32_t* __restrict__ hist,
+                                                                    uint32_t* __restrict__ clear, size_t clear_words)
 {
 	__shared__ uint32_t s_hist[kSortMaxPasses][256];
+	for (size_t w = (size_t)blockIdx.x * 256 + threadIdx.x; w < clear_words; w += (size_t)gridDim.x * 256)
+		clear[w] = 0u;  // an array that a later kernel of the same stream wants cleared
 	if (n_device)
 		n = *n_device;
 #pragma unroll
@@ -461,9 +476,16 @@ const uint32_t* sort_status_word(const uint32_t* temp)
 	return temp + kSortStatus;
 }
 
+size_t sort_clear_words(size_t n, int end_bit)
+{
+	const size_t tiles = (n + kSortBlock - 1) / kSortBlock;
+	return kSortHeader + (size_t)((end_bit + 7) / 8) * 256 * tiles;
+}
+
 template <typename KeyT>
 static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                       const uint32_t* n_device, int end_bit, uint32_t* temp, bool mark_stages, hipStream_t s)
+                       const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, bool mark_stages,
+                       uint32_t* also_clear, size_t also_clear_words, hipStream_t s)
 {
 	if (n == 0)
 		return;
@@ -471,10 +493,11 @@ static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_
 	const int passes = (end_bit + 7) / 8;
 	if (mark_stages)
 		stage_mark("sort_setup", s);
-	launch_fill_u32(temp, 0u, kSortHeader + (size_t)passes * 256 * tiles, s);
+	if (!temp_cleared)
+		launch_fill_u32(temp, 0u, sort_clear_words(n, end_bit), s);
 	const uint32_t hist_blocks = tiles < 2048u ? tiles : 2048u;
 	hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks), dim3(256), 0, s, keys_in, n, n_device, passes,
-	                   end_bit, temp);
+	                   end_bit, temp, also_clear, also_clear_words);
 	KeyT *ksrc = keys_in, *kdst = keys_out;
 	uint32_t *vsrc = vals_in, *vdst = vals_out;
 	for (int p = 0; p < passes; p++) {
@@ -495,13 +518,15 @@ static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s)
 {
-	sort_pairs<uint64_t>(keys_in, keys_out, vals_in, vals_out, n, nullptr, end_bit, temp, true, s);
+	sort_pairs<uint64_t>(keys_in, keys_out, vals_in, vals_out, n, nullptr, end_bit, temp, false, true, nullptr, 0, s);
 }
 
 void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                           const uint32_t* n_device, int end_bit, uint32_t* temp, const char* stage, hipStream_t s)
+                           const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, uint32_t* also_clear,
+                           size_t also_clear_words, const char* stage, hipStream_t s)
 {
-	sort_pairs<uint32_t>(keys_in, keys_out, vals_in, vals_out, n, n_device, end_bit, temp, stage != nullptr, s);
+	sort_pairs<uint32_t>(keys_in, keys_out, vals_in, vals_out, n, n_device, end_bit, temp, temp_cleared, stage != nullptr,
+	                     also_clear, also_clear_words, s);
 }
 
 // ---- tile ranges (K/cuda_rasterizer_hgs/rasterizer_impl.cu:116-138 and the memset at :319) ----
@@ -547,10 +572,11 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __rest
 }
 
 void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
-                        const uint32_t* order_status, hipStream_t s)
+                        const uint32_t* order_status, bool ranges_cleared, hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
-	launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2 + kRangeTailWords, s);
+	if (!ranges_cleared)
+		launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2 + kRangeTailWords, s);
 	if (n == 0)
 		return;
 	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges,

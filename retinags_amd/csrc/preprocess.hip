@@ -143,6 +143,9 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs 
 {
 	__shared__ uint32_t s_scan[8];
 	const int idx = blockIdx.x * 256 + threadIdx.x;
+	// the scratch of the depth sort that follows is cleared here, which saves a launch
+	for (size_t w = (size_t)idx; w < a.clear_words; w += (size_t)gridDim.x * 256)
+		a.clear[w] = 0u;
 	uint32_t touched = 0;
 
 	if (idx < a.P) {

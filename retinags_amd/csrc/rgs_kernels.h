@@ -36,6 +36,8 @@ struct PreprocessArgs {
 	uint32_t* block_sums;  // one per 256 Gaussians
 	uint32_t* block_visible;  // one per 256 Gaussians: how many of them touch a tile
 	bool sh_rows_by_16_bytes; // SH rows are 16-byte aligned, a multiple of 16 bytes long and at most 48 floats
+	uint32_t* clear;          // clear_words words that the kernel sets to zero for a later stage
+	size_t clear_words;
 	float4* blend_record;  // 4 float4 per Gaussian, see blend.hip
 };
 
@@ -138,10 +140,13 @@ size_t scan_temp_words(size_t n);                 // u32 words of scratch for la
 // `stage` (may be null) names the stage for the timing aid.
 void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, const char* stage,
                           hipStream_t s);
-// Scans the per-256 block sums of the tile counts in place; *total_out = number of instances.
-void launch_total_from_block_sums(uint32_t* block_sums, int P, uint32_t* total_out, hipStream_t s);
-// Depth order of the Gaussians that touch a tile.  block_visible holds their count per 256
-// Gaussians (scanned in place; the total goes to *visible_count).  On return order[0..count)
+// Scans the per-256 block sums of the tile counts and of the visible flags in place;
+// *total_out = number of instances, *visible_count = number of Gaussians that touch a tile.
+void launch_totals_from_block_sums(uint32_t* block_sums, uint32_t* block_visible, int P, uint32_t* total_out,
+                                   uint32_t* visible_count, hipStream_t s);
+// Depth order of the Gaussians that touch a tile.  block_visible holds the exclusive scan of
+// their count per 256 Gaussians and *visible_count the total; sort_temp has been cleared
+// (sort_clear_words(P, 32) words).  On return order[0..count)
 // lists them by increasing depth, ties by index, and offsets_in_order is the inclusive scan of
 // their tile counts in that order; visible_list keeps them in index order.  The count stays on the device: every kernel is launched
 // for P elements and reads it.
@@ -149,9 +154,12 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
                         uint32_t* visible_count, uint32_t* visible_list, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
                         uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
                         hipStream_t s);
+// Also sets clear[0..clear_words) to zero (the scratch of the sort that follows).
 void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
                                 const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
-                                int grid_y, uint32_t* keys, uint32_t* values, hipStream_t s);
+                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t* clear, size_t clear_words,
+                                hipStream_t s);
+size_t sort_clear_words(size_t n, int end_bit);    // words of the sort scratch that must be zero before a sort
 size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs*
 // Stable LSD radix sort on key bits [0, end_bit), ceil(end_bit/8) passes that ping-pong between
 // the two buffer pairs starting in -> out: an odd pass count leaves the result in
@@ -161,14 +169,18 @@ void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in,
 // The same for 32-bit keys; with a null `stage` its kernels are not marked for the timing aid.
 // With a non-null n_device the number of pairs is read from there by the kernels and `n` is only
 // its upper bound (grids and scratch are sized for it).
+// temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of temp already.
+// also_clear: an array the first kernel sets to zero on the way (for a later stage), or null.
 void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                           const uint32_t* n_device, int end_bit, uint32_t* temp, const char* stage, hipStream_t s);
+                           const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, uint32_t* also_clear,
+                           size_t also_clear_words, const char* stage, hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
 // Either status word (may be null) being non-zero leaves every range empty.  Clears `ranges` and
 // the kRangeTailWords words behind it (the strip class counters of the blend).
 constexpr int kRangeTailWords = 512;
+// ranges_cleared: an earlier kernel has done that clearing.
 void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
-                        const uint32_t* order_status, hipStream_t s);
+                        const uint32_t* order_status, bool ranges_cleared, hipStream_t s);
 
 // blend.hip
 void launch_blend_forward(const BlendArgs& a, hipStream_t s);
