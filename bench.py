@@ -36,9 +36,9 @@ FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
 # cannot be read from inside the process, so the figures are carried here; other workloads
 # report null.
 C1_TRAFFIC_MB_PER_LAUNCH = {
-    "preprocess_forward": 252.01, "duplicate_with_keys": 112.63, "sort_onesweep": 23.06, "tile_ranges": 13.22,
-    "blend_forward": 224.22, "composite_forward": 165.79, "composite_backward": 372.01, "blend_backward": 303.62,
-    "preprocess_backward": 370.06,
+    "preprocess_forward": 253.53, "duplicate_with_keys": 114.82, "sort_onesweep": 23.17, "tile_ranges": 13.22,
+    "blend_forward": 223.79, "composite_forward": 165.79, "composite_backward": 372.01, "blend_backward": 542.45,
+    "preprocess_backward": 370.05,
 }
 
 
