@@ -572,7 +572,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	RGS_REQUIRE(P > 0 && R >= 0, "rgs_backward: bad sizes P=%d R=%d", P, R);
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_backward: bad image size %dx%d", width, height);
 	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
-	                cam_pos && radii && geom_ws && image_ws && dL_dpix && dL_dpix_depth && dL_dalphas && grad_accum &&
+	                cam_pos && radii && geom_ws && image_ws && dL_dpix && grad_accum &&
 	                dL_dmean2D && dL_dopacity && dL_dcolor && dL_dmean3D && dL_dcov3D,
 	            "rgs_backward: null pointer");
 	RGS_REQUIRE(R == 0 || binning_ws, "rgs_backward: null binning workspace");

@@ -638,8 +638,8 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 		p.g_r = a.dL_dpix[pix_id];
 		p.g_g = a.dL_dpix[plane + pix_id];
 		p.g_b = a.dL_dpix[2 * plane + pix_id];
-		p.g_depth = a.dL_dpix_depth[pix_id];
-		p.g_alpha = a.dL_dalpha[pix_id];
+		p.g_depth = a.dL_dpix_depth ? a.dL_dpix_depth[pix_id] : 0.f;  // absent: no gradient came in
+		p.g_alpha = a.dL_dalpha ? a.dL_dalpha[pix_id] : 0.f;
 	}
 	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
 	st.upstream[0][row_column(lane)] = p.g_r;

@@ -86,6 +86,8 @@ class GeometryStage:
                 and not self.used)
 
 
+_EMPTY = torch.Tensor([])  # stands for an absent input, as in the reference (it becomes a null pointer)
+
 _free_count_slots = {}   # per device: (pinned word, event) pairs of finished calls, for reuse
 
 
@@ -357,14 +359,15 @@ class _RasterizeGaussians(torch.autograd.Function):
         (colors_precomp, means3D, scales, rotations, cov3Ds_precomp, radii, sh, geomBuffer, binningBuffer, imgBuffer,
          alpha) = ctx.saved_tensors
 
-        # Outputs that did not take part in the loss arrive as None; the reference's C++ side
-        # always receives dense tensors, so they become zeros.
+        # Outputs that did not take part in the loss arrive as None.  The reference's C++ side
+        # always receives dense tensors; here an absent depth / alpha gradient goes down as a
+        # null pointer, which the library takes as zero.
         if grad_color is None:
             grad_color = torch.zeros((3,) + tuple(alpha.shape[1:]), dtype=alpha.dtype, device=alpha.device)
         if grad_depth is None:
-            grad_depth = torch.zeros_like(alpha)
+            grad_depth = _EMPTY
         if grad_alpha is None:
-            grad_alpha = torch.zeros_like(alpha)
+            grad_alpha = _EMPTY
 
         args = (raster_settings.bg, means3D, radii, colors_precomp, scales, rotations,
                 raster_settings.scale_modifier, cov3Ds_precomp, raster_settings.viewmatrix,
@@ -426,15 +429,15 @@ class GaussianRasterizer(nn.Module):
             raise Exception('Please provide exactly one of either scale/rotation pair or precomputed 3D covariance!')
 
         if shs is None:
-            shs = torch.Tensor([])
+            shs = _EMPTY
         if colors_precomp is None:
-            colors_precomp = torch.Tensor([])
+            colors_precomp = _EMPTY
         if scales is None:
-            scales = torch.Tensor([])
+            scales = _EMPTY
         if rotations is None:
-            rotations = torch.Tensor([])
+            rotations = _EMPTY
         if cov3D_precomp is None:
-            cov3D_precomp = torch.Tensor([])
+            cov3D_precomp = _EMPTY
         return shs, colors_precomp, scales, rotations, cov3D_precomp
 
     def forward(self, means3D, means2D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
