@@ -75,13 +75,15 @@ enum {
 	RGS_BIN_VALUES_UNSORTED,    /* uint32[R]  Gaussian index */
 	RGS_BIN_VALUES_SORTED,      /* uint32[R]  the per-tile Gaussian lists, tile after tile */
 	RGS_BIN_SORT_TEMP,          /* uint32[..] */
+	RGS_BIN_STRIP_LISTS,        /* uint32[4R] written by the forward blend: for strip s of a tile with list [x, x+n), from
+	                               4x + s*n on, the list positions that can matter to the strip (bit 31: strip inside the box) */
 	RGS_BIN_FIELDS
 };
 enum {
 	RGS_IMG_RANGES = 0,         /* uint2[tiles]  [start, end) of each tile in the sorted list */
 	RGS_IMG_N_CONTRIB,          /* uint32[H*W]   list position of the last blended Gaussian */
-	RGS_IMG_STRIP_SPAN,         /* uint32[4*tiles] largest n_contrib of each 16x4 strip (tile * 4 + strip) */
-	RGS_IMG_STRIP_ORDER,        /* uint32[4*tiles] the strips by decreasing span: the order the backward blend takes them in */
+	RGS_IMG_STRIP_FILED,        /* uint32[4*tiles] per 16x4 strip (tile * 4 + strip): entries of RGS_BIN_STRIP_LISTS the backward walks */
+	RGS_IMG_STRIP_ORDER,        /* uint32[4*tiles] the strips by decreasing RGS_IMG_STRIP_FILED: the order the backward blend takes them in */
 	RGS_IMG_FIELDS
 };
 int rgs_geom_layout(int P, size_t offsets[RGS_GEOM_FIELDS]);

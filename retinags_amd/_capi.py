@@ -15,8 +15,8 @@ LIB_PATH = os.environ.get("RGS_LIBRARY") or os.path.join(_HERE, "librgs_gfx950.s
 GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles_touched", "point_offsets",
                "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
                "visible_list", "order_scratch")
-BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp")
-IMG_FIELDS = ("ranges", "n_contrib", "strip_span", "strip_order")
+BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp", "strip_lists")
+IMG_FIELDS = ("ranges", "n_contrib", "strip_filed", "strip_order")
 ACC_FLOATS = 12
 MAX_COMPOSITE = 64
 

@@ -150,7 +150,7 @@ int tile_key_bits(int width, int height)
 
 // Physical buffers: A receives the duplicated keys, B is its ping-pong partner.
 struct BinningPhysical {
-	size_t keys_a, keys_b, vals_a, vals_b, temp, total;
+	size_t keys_a, keys_b, vals_a, vals_b, temp, strip_lists, total;
 };
 
 BinningPhysical binning_physical(size_t R)
@@ -162,6 +162,7 @@ BinningPhysical binning_physical(size_t R)
 	b.vals_a = c.take(4 * R);
 	b.vals_b = c.take(4 * R);
 	b.temp = c.take(4 * rgs::sort_temp_words(R));
+	b.strip_lists = c.take(16 * R);
 	b.total = c.cursor;
 	return b;
 }
@@ -172,7 +173,7 @@ size_t image_layout(int width, int height, size_t* off)
 	Carver c;
 	off[RGS_IMG_RANGES] = c.take(8 * tiles + 4 * rgs::kRangeTailWords);  // + the strip class counters, cleared with it
 	off[RGS_IMG_N_CONTRIB] = c.take(4 * (size_t)width * height);
-	off[RGS_IMG_STRIP_SPAN] = c.take(4 * 4 * tiles);
+	off[RGS_IMG_STRIP_FILED] = c.take(4 * 4 * tiles);
 	off[RGS_IMG_STRIP_ORDER] = c.take(4 * 4 * tiles);
 	return c.cursor;
 }
@@ -296,6 +297,7 @@ int rgs_binning_layout(int R, int width, int height, size_t offsets[RGS_BIN_FIEL
 	offsets[RGS_BIN_VALUES_UNSORTED] = sorted_in_a ? b.vals_b : b.vals_a;
 	offsets[RGS_BIN_VALUES_SORTED] = sorted_in_a ? b.vals_a : b.vals_b;
 	offsets[RGS_BIN_SORT_TEMP] = b.temp;
+	offsets[RGS_BIN_STRIP_LISTS] = b.strip_lists;
 	return 0;
 }
 
@@ -547,8 +549,9 @@ int rgs_forward_raster(int P, int R, int width, int height,
 	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 	a.out_color = out_color; a.out_depth = out_depth; a.out_alpha = out_alpha;
 	a.n_contrib = at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]);
-	a.strip_span = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_SPAN]);
+	a.strip_filed = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_FILED]);
 	a.strip_order = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_ORDER]);
+	a.strip_lists = R > 0 ? at<uint32_t>(binning_ws, binning_physical((size_t)R).strip_lists) : nullptr;
 	a.strip_classes = reinterpret_cast<uint32_t*>(ranges) + 2 * (size_t)gx * gy;
 	rgs::launch_blend_forward(a, s);
 	RGS_STAGE("blend_forward");
@@ -609,8 +612,9 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 		a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 		a.out_alpha = const_cast<float*>(alphas);
 		a.n_contrib = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]));
-		a.strip_span = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_SPAN]));
+		a.strip_filed = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_FILED]));
 		a.strip_order = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_ORDER]));
+		a.strip_lists = const_cast<uint32_t*>(at<uint32_t>(binning_ws, b.strip_lists));
 		a.dL_dpix = dL_dpix; a.dL_dpix_depth = dL_dpix_depth; a.dL_dalpha = dL_dalphas;
 		a.sums = grad_accum;
 		rgs::launch_blend_backward(a, s);

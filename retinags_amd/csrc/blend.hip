@@ -137,9 +137,9 @@ __device__ __forceinline__ int classify_strip_against_box(float w, const StripCo
 	return outside ? kBoxOutside : (inside ? kBoxInside : kBoxMixed);
 }
 
-// Launch-order classes of the backward's strips, by the length of list they have to walk.
+// Launch-order classes of the backward's strips, by the number of entries they have to walk.
 constexpr int kStripClasses = 256;
-__device__ __forceinline__ uint32_t strip_class(uint32_t span) { return 255u - min(span >> 4, 255u); }
+__device__ __forceinline__ uint32_t strip_class(uint32_t filed) { return 255u - min(filed >> 3, 255u); }
 
 constexpr int kPerLane = 1;             // list entries per lane and step (2 was measured slower)
 constexpr int kChunk = 64 * kPerLane;   // list entries a wavefront takes per step
@@ -165,6 +165,29 @@ __device__ __forceinline__ LoadedEntry load_entry(const BlendArgs& a, uint32_t i
 		e.conic = float4{0.f, 0.f, 0.f, 0.f};
 		e.cd = float4{0.f, 0.f, 0.f, 0.f};
 		e.half = float4{0.f, 0.f, 0.f, 0.f};
+	}
+	return e;
+}
+
+// What the backward reads of a record: it takes the forward's word for which entries matter.
+struct LoadedRecord {
+	float4 geom, conic, cd;
+	uint32_t id;
+};
+
+__device__ __forceinline__ LoadedRecord load_record(const BlendArgs& a, uint32_t id, bool in_range)
+{
+	LoadedRecord e;
+	e.id = id;
+	if (in_range) {
+		const float4* rec = a.record + 4 * (size_t)id;
+		e.geom = rec[0];
+		e.conic = rec[1];
+		e.cd = rec[2];
+	} else {
+		e.geom = float4{0.f, 0.f, INFINITY, 0.f};
+		e.conic = float4{0.f, 0.f, 0.f, 0.f};
+		e.cd = float4{0.f, 0.f, 0.f, 0.f};
 	}
 	return e;
 }
@@ -204,6 +227,7 @@ struct ForwardPixel {
 	bool done;
 	float T, C0, C1, C2, weight, D;
 	uint32_t last_contributor;
+	uint32_t last_filed;  // like last_contributor, but counted in entries filed for the strip
 };
 
 struct ForwardStage {  // wave-private
@@ -213,9 +237,10 @@ struct ForwardStage {  // wave-private
 	uint32_t position[kChunk]; // 1-based position in the tile list
 };
 
+// `filed_index` is the entry's 1-based number among those filed for the strip.
 __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, float power, const float4 g,
-                                              const float4 co, const ForwardStage& st, int slot, const PixelRay& ray,
-                                              const BoxFrame& box)
+                                              const float4 co, const ForwardStage& st, int slot, uint32_t filed_index,
+                                              const PixelRay& ray, const BoxFrame& box)
 {
 	candidate = candidate && !p.done;
 	if (__ballot(candidate) == 0ull)
@@ -236,6 +261,7 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 				p.D += cd.w * alpha * p.T;
 				p.T = test_T;
 				p.last_contributor = st.position[slot];
+				p.last_filed = filed_index;
 			}
 		}
 	}
@@ -264,8 +290,13 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	ForwardStage& st = s_stage[wave];
 	const uint64_t below = (1ull << lane) - 1ull;
 
-	ForwardPixel p = {!inside, 1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u};
+	ForwardPixel p = {!inside, 1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u, 0u};
 	uint64_t live = __ballot(!p.done);
+	// The entries filed for this strip are also written out, for the backward pass: their list
+	// positions in order, bit 31 set where the strip lies inside the box.  The backward needs
+	// them up to the last one that some pixel blended (the largest last_filed of the strip).
+	uint32_t* filed_list = a.strip_lists + 4 * (size_t)range.x + (size_t)wave * n;
+	uint32_t filed_total = 0;
 
 	if (n != 0u && live != 0ull) {
 		const uint32_t* list = a.point_list + range.x;
@@ -292,9 +323,13 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 					st.conic[slot] = cur[e].conic;
 					st.cd[slot] = cur[e].cd;
 					st.position[slot] = first + 64 * e + lane + 1;
+					const bool strip_inside_box = cur[e].geom.w != cur[e].geom.w;
+					filed_list[filed_total + slot] = (first + 64 * e + lane) | (strip_inside_box ? 0x80000000u : 0u);
 				}
 				count += __popcll(m);
 			}
+			const uint32_t chunk_base = filed_total;
+			filed_total += (uint32_t)count;
 			if (lane < 3) {  // pad to a multiple of four with entries that never pass the floor test
 				st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
 				st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
@@ -319,10 +354,11 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
 				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
 					continue;
-				forward_visit(p, q0, w0, g0, c0, st, k, ray, box);
-				forward_visit(p, q1, w1, g1, c1, st, k + 1, ray, box);
-				forward_visit(p, q2, w2, g2, c2, st, k + 2, ray, box);
-				forward_visit(p, q3, w3, g3, c3, st, k + 3, ray, box);
+				const uint32_t f = chunk_base + (uint32_t)k;
+				forward_visit(p, q0, w0, g0, c0, st, k, f + 1, ray, box);
+				forward_visit(p, q1, w1, g1, c1, st, k + 1, f + 2, ray, box);
+				forward_visit(p, q2, w2, g2, c2, st, k + 2, f + 3, ray, box);
+				forward_visit(p, q3, w3, g3, c3, st, k + 3, f + 4, ray, box);
 				live = __ballot(!p.done);
 			}
 			__builtin_amdgcn_wave_barrier();
@@ -333,12 +369,12 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	}
 
 	{
-		uint32_t span = inside ? p.last_contributor : 0u;
+		uint32_t upto = inside ? p.last_filed : 0u;
 #pragma unroll
 		for (int off = 32; off > 0; off >>= 1)
-			span = max(span, (uint32_t)__shfl_xor((int)span, off));
+			upto = max(upto, (uint32_t)__shfl_xor((int)upto, off));
 		if (lane == 0)
-			a.strip_span[4 * tile + wave] = span;
+			a.strip_filed[4 * tile + wave] = upto;
 	}
 	if (inside) {
 		const size_t plane = (size_t)a.H * a.W;
@@ -598,7 +634,7 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 	__shared__ BackwardStage s_stage;
 
 	const int lane = threadIdx.x;
-	// longest strips first: a long strip that starts late is what the whole launch waits for
+	// strips with the most entries first: a long strip that starts late is what the whole launch waits for
 	const uint32_t strip_id = a.strip_order[blockIdx.x];
 	const int tile = (int)(strip_id >> 2), wave = (int)(strip_id & 3u);  // wave: which strip of the tile
 	const uint2 range = a.ranges[tile];
@@ -611,22 +647,16 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 	const BoxFrame box = load_box_frame(a);
 	const size_t plane = (size_t)a.H * a.W;
 	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
-	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
-	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
 	const StripFrame frame = {strip_x0, strip_y0, (float)(0.5 * a.W), (float)(0.5 * a.H)};
 	BackwardStage& st = s_stage;
-	const uint64_t below = (1ull << lane) - 1ull;
 
-	if (range.y == range.x)
+	// The forward blend has written down which entries of the tile's list matter to this strip
+	// (its conservative filters, not repeated here), up to the last one that any pixel blended.
+	const uint32_t filed = a.strip_filed[strip_id];
+	if (filed == 0u)
 		return;
+	const uint32_t n = range.y - range.x;
 	const uint32_t last_contributor = inside ? a.n_contrib[pix_id] : 0u;
-	// entries at or beyond the largest last_contributor of the strip are skipped by all its pixels
-	uint32_t span = last_contributor;
-#pragma unroll
-	for (int off = 32; off > 0; off >>= 1)
-		span = max(span, (uint32_t)__shfl_xor((int)span, off));
-	if (span == 0u)
-		return;
 
 	BackwardPixel p;
 	p.T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
@@ -648,46 +678,44 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 	st.upstream[3][row_column(lane)] = p.g_depth;
 	int rows = 0;
 
-	// lane l holds the entries first + 64 e + l from the back (list position span-1-that), e < kPerLane
+	// Lane l of the chunk that starts `first` entries from the back takes filed entry
+	// filed-1-first-l: its list position (and box flag), through that the Gaussian's index,
+	// through that its record.  Three chunks are in flight: the records of the next one, the
+	// indices of the one after, the positions of the one after that.
 	const uint32_t* list = a.point_list + range.x;
-	LoadedEntry cur[kPerLane];
-	uint32_t id_next[kPerLane];
-#pragma unroll
-	for (int e = 0; e < kPerLane; e++) {
-		const uint32_t i0 = 64 * e + lane, i1 = kChunk + i0;
-		cur[e] = load_entry(a, i0 < span ? list[span - 1 - i0] : 0u, i0 < span);
-		id_next[e] = i1 < span ? list[span - 1 - i1] : 0u;
-	}
+	const uint32_t* filed_list = a.strip_lists + 4 * (size_t)range.x + (size_t)wave * n;
+	constexpr uint32_t kNone = 0xFFFFFFFFu, kPosition = 0x7FFFFFFFu;
+	uint32_t pos_cur = (uint32_t)lane < filed ? filed_list[filed - 1 - lane] : kNone;
+	uint32_t pos_next = (uint32_t)(64 + lane) < filed ? filed_list[filed - 1 - (64 + lane)] : kNone;
+	uint32_t pos_after = (uint32_t)(128 + lane) < filed ? filed_list[filed - 1 - (128 + lane)] : kNone;
+	LoadedRecord cur = load_record(a, pos_cur != kNone ? list[pos_cur & kPosition] : 0u, pos_cur != kNone);
+	uint32_t id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
 
-	for (uint32_t first = 0; first < span; first += kChunk) {
-		int count = 0;
-#pragma unroll
-		for (int e = 0; e < kPerLane; e++) {
-			const bool filed = file_entry(cur[e], strip_x0, strip_y0, sc, box);
-			const uint64_t m = __ballot(filed);
-			if (filed) {
-				const int slot = count + __popcll(m & below);
-				st.geom[slot] = cur[e].geom;
-				st.conic[slot] = cur[e].conic;
-				st.cd[slot] = cur[e].cd;
-				st.entry[slot] = span - 1 - (first + 64 * e + lane);
-				st.id[slot] = cur[e].id;
-			}
-			count += __popcll(m);
+	for (uint32_t first = 0; first < filed; first += 64) {
+		const int count = (int)min(filed - first, 64u);
+		if (lane < count) {
+			float4 g = cur.geom;
+			if (pos_cur & 0x80000000u)
+				g.w = __int_as_float(0x7FC00000);  // the strip lies inside the box: no per-pixel test
+			st.geom[lane] = g;
+			st.conic[lane] = cur.conic;
+			st.cd[lane] = cur.cd;
+			st.entry[lane] = pos_cur & kPosition;
+			st.id[lane] = cur.id;
 		}
-		if (lane < 3) {
+		if (lane < 3) {  // pad to a multiple of four with entries that never pass the floor test
 			st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
 			st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
 			st.entry[count + lane] = 0xFFFFFFFFu;
 		}
 		__builtin_amdgcn_wave_barrier();
 		// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
-#pragma unroll
-		for (int e = 0; e < kPerLane; e++) {
-			const uint32_t i1 = first + kChunk + 64 * e + lane, i2 = i1 + kChunk;
-			cur[e] = load_entry(a, id_next[e], i1 < span);
-			id_next[e] = i2 < span ? list[span - 1 - i2] : 0u;
-		}
+		cur = load_record(a, id_next, pos_next != kNone);
+		pos_cur = pos_next;
+		pos_next = pos_after;
+		id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
+		const uint32_t e3 = first + 192 + (uint32_t)lane;
+		pos_after = e3 < filed ? filed_list[filed - 1 - e3] : kNone;
 
 		for (int k = 0; k < count; k += 4) {
 			const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
@@ -708,20 +736,17 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, box, lane);
 		}
 		__builtin_amdgcn_wave_barrier();
-#pragma unroll
-		for (int e = 0; e < kPerLane; e++)
-			keep_padding_registers(cur[e]);
 	}
 	if (rows > 0)
 		flush_rows(st, rows, frame, a, lane);
 }
 
-// Strips by decreasing span, in kStripClasses classes of 16 list entries (longer ones share
+// Strips by decreasing number of filed entries, in kStripClasses classes of 8 (longer ones share
 // the first class); the order inside a class is whatever the atomics give, which is all a
 // launch order needs.  Two small kernels: count the strips of every class, then place them.
 // Both aggregate in LDS first: most strips fall into one class (nothing to walk), and
 // thousands of global atomics on one word would take longer than the blend itself.
-__global__ __launch_bounds__(256) void strip_count_kernel(const uint32_t* __restrict__ span, uint32_t n,
+__global__ __launch_bounds__(256) void strip_count_kernel(const uint32_t* __restrict__ filed, uint32_t n,
                                                            uint32_t* __restrict__ class_count)
 {
 	__shared__ uint32_t s_count[kStripClasses];
@@ -729,13 +754,13 @@ __global__ __launch_bounds__(256) void strip_count_kernel(const uint32_t* __rest
 	__syncthreads();
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
 	if (k < n)
-		atomicAdd(&s_count[strip_class(span[k])], 1u);
+		atomicAdd(&s_count[strip_class(filed[k])], 1u);
 	__syncthreads();
 	if (s_count[threadIdx.x] != 0u)
 		atomicAdd(&class_count[threadIdx.x], s_count[threadIdx.x]);
 }
 
-__global__ __launch_bounds__(256) void strip_place_kernel(const uint32_t* __restrict__ span, uint32_t n,
+__global__ __launch_bounds__(256) void strip_place_kernel(const uint32_t* __restrict__ filed, uint32_t n,
                                                            const uint32_t* __restrict__ class_count,
                                                            uint32_t* __restrict__ class_cursor,
                                                            uint32_t* __restrict__ order)
@@ -747,7 +772,7 @@ __global__ __launch_bounds__(256) void strip_place_kernel(const uint32_t* __rest
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
 	uint32_t c = 0, rank = 0;
 	if (k < n) {
-		c = strip_class(span[k]);
+		c = strip_class(filed[k]);
 		rank = atomicAdd(&s_count[c], 1u);
 	}
 	__syncthreads();
@@ -772,9 +797,9 @@ void launch_blend_forward(const BlendArgs& a, hipStream_t s)
 		// the order in which the backward will take the strips (longest first was measured no
 		// faster for the forward's tiles, whose length is only known as the list length)
 		const uint32_t strips = (uint32_t)(4 * a.grid_x * a.grid_y);
-		hipLaunchKernelGGL(strip_count_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_span, strips,
+		hipLaunchKernelGGL(strip_count_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_filed, strips,
 		                   a.strip_classes);
-		hipLaunchKernelGGL(strip_place_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_span, strips,
+		hipLaunchKernelGGL(strip_place_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_filed, strips,
 		                   a.strip_classes, a.strip_classes + kStripClasses, a.strip_order);
 	}
 }

@@ -90,9 +90,11 @@ struct BlendArgs {
 	float* out_depth;
 	float* out_alpha;
 	uint32_t* n_contrib;
-	uint32_t* strip_span;   // per 16x4 strip (tile * 4 + strip): the largest n_contrib of its pixels
-	uint32_t* strip_order;  // strips by decreasing span, written behind the forward blend
-	uint32_t* strip_classes;  // 2 x 256 words, zero before the forward blend: strips per span class, placement cursors
+	uint32_t* strip_lists;  // 4 R words: for strip s of a tile whose list is [x, x + n), the entries the forward
+	                        // filed for it, at 4 x + s n: list position, bit 31 = strip inside the box
+	uint32_t* strip_filed;  // per 16x4 strip (tile * 4 + strip): how many of them, up to the last one blended
+	uint32_t* strip_order;  // strips by decreasing strip_filed, written behind the forward blend
+	uint32_t* strip_classes;  // 2 x 256 words, zero before the forward blend: strips per class of strip_filed, placement cursors
 	uint64_t* counters;  // non-null selects the work-accounting twin of the forward blend (7 sums)
 	// backward
 	const float* dL_dpix;

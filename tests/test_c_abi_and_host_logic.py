@@ -55,7 +55,7 @@ def test_workspace_sizes_and_layouts_are_consistent():
         lay = _capi.binning_layout(R, W, H)
         total = _capi.lib.rgs_binning_bytes(R)
         sizes = dict(keys_unsorted=4 * R, keys_sorted=4 * R, values_unsorted=4 * R, values_sorted=4 * R,
-                     sort_temp=_capi.lib.rgs_sort_temp_bytes(R))
+                     sort_temp=_capi.lib.rgs_sort_temp_bytes(R), strip_lists=16 * R)
         spans = sorted((lay[k], lay[k] + sizes[k]) for k in sizes)
         assert all(spans[i][1] <= spans[i + 1][0] for i in range(len(spans) - 1))
         assert spans[-1][1] <= total

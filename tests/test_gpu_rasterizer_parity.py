@@ -61,15 +61,24 @@ def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
     im = _capi.image_layout(W, H)
     assert np.array_equal(view_ws(img, im["ranges"], 2 * T, np.uint32).reshape(T, 2), st.ranges)
 
-    # ---- the order in which the backward blend takes the 16x4 strips: longest span first
-    spans = view_ws(img, im["strip_span"], 4 * T, np.uint32)
+    # ---- what the forward blend leaves for the backward: per 16x4 strip the entries it filed, up
+    # to the last one blended, and the strips ordered by how many those are
+    filed = view_ws(img, im["strip_filed"], 4 * T, np.uint32)
     order = view_ws(img, im["strip_order"], 4 * T, np.uint32)
     assert np.array_equal(np.sort(order), np.arange(4 * T, dtype=np.uint32))
-    assert (np.diff(np.minimum(spans[order] >> 4, 255).astype(np.int64)) <= 0).all()
+    assert (np.diff(np.minimum(filed[order] >> 3, 255).astype(np.int64)) <= 0).all()
     nc = np.zeros((s.grid[1] * 16, s.grid[0] * 16), np.uint32)
     nc[:H, :W] = view_ws(img, im["n_contrib"], H * W, np.uint32).reshape(H, W)
-    per_strip = nc.reshape(s.grid[1], 4, 4, s.grid[0], 16).max(axis=(2, 4)).transpose(0, 2, 1).reshape(-1)
-    assert np.array_equal(spans, per_strip)
+    span = nc.reshape(s.grid[1], 4, 4, s.grid[0], 16).max(axis=(2, 4)).transpose(0, 2, 1).reshape(-1)
+    assert np.array_equal(filed == 0, span == 0)
+    if R > 0:
+        lists = view_ws(binning, _capi.binning_layout(R, W, H)["strip_lists"], 4 * R, np.uint32)
+        ranges = st.ranges.astype(np.int64)
+        for sid in np.flatnonzero(filed)[:: max(1, int((filed > 0).sum()) // 200)]:   # a sample of strips
+            t, w = sid >> 2, sid & 3
+            x, n = ranges[t, 0], ranges[t, 1] - ranges[t, 0]
+            mine = lists[4 * x + w * n: 4 * x + w * n + filed[sid]] & 0x7FFFFFFF
+            assert (np.diff(mine.astype(np.int64)) > 0).all() and mine[-1] == span[sid] - 1 and mine[-1] < n
 
     # ---- blend: tolerance, away from decision thresholds
     n_contrib = view_ws(img, im["n_contrib"], H * W, np.uint32)
