@@ -179,8 +179,13 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restr
 		block_totals[blockIdx.x] = total;
 }
 
-// Thread k takes the k-th Gaussian in depth order and writes its instances, tiles row by row
-// like the reference, at the offsets of the scan taken in that same order.
+// Instances of the Gaussians in depth order, tiles row by row like the reference, at the offsets
+// of the scan taken in that same order.  A wavefront takes 64 Gaussians; their instances form one
+// contiguous run of the output, which the wavefront writes 64 consecutive entries at a time:
+// each lane finds the Gaussian its output position belongs to by a binary search over the 64
+// inclusive offsets, then the tile from the position inside that Gaussian's rectangle.  (With
+// one thread per Gaussian every store touched 64 different cache lines, and a Gaussian that
+// covers hundreds of tiles kept its wavefront busy alone.)
 __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t* __restrict__ visible_count,
                                                                    const uint32_t* __restrict__ order,
                                                                    const uint32_t* __restrict__ offsets,
@@ -190,22 +195,51 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t
                                                                    uint32_t* __restrict__ values,
                                                                    uint32_t* __restrict__ clear, size_t clear_words)
 {
+	__shared__ uint32_t s_end[4][64];     // inclusive offset of each of the wavefront's Gaussians
+	__shared__ uint32_t s_origin[4][64];  // first tile of its rectangle
+	__shared__ uint32_t s_width[4][64];   // tiles per row of its rectangle
+	__shared__ uint32_t s_index[4][64];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
 	// the scratch of the sort that follows is cleared here, which saves a launch
 	for (size_t w = k; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;
-	if (k >= *visible_count)
+	const uint32_t n = *visible_count;
+	const uint32_t k0 = k - (uint32_t)lane;  // the wavefront's first Gaussian
+	if (k0 >= n)
 		return;
-	const uint32_t idx = order[k];
-	const int radius = radii[idx];
-	uint32_t off = (k == 0) ? 0u : offsets[k - 1];
-	const float2 p = xy[idx];
-	const TileRect rc = tile_rect(p.x, p.y, radius, gx, gy);
-	for (uint32_t y = rc.y0; y < rc.y1; y++) {
-		for (uint32_t x = rc.x0; x < rc.x1; x++) {
-			keys[off] = y * (uint32_t)gx + x;
-			values[off] = idx;
-			off++;
+	const uint32_t run_begin = k0 == 0u ? 0u : offsets[k0 - 1];
+	uint32_t end = 0, origin = 0, width = 1, idx = 0;
+	if (k < n) {
+		idx = order[k];
+		end = offsets[k];
+		const float2 p = xy[idx];
+		const TileRect rc = tile_rect(p.x, p.y, radii[idx], gx, gy);
+		origin = rc.y0 * (uint32_t)gx + rc.x0;
+		width = rc.x1 - rc.x0;
+	} else {
+		end = offsets[n - 1];  // no instances of its own
+	}
+	s_end[wave][lane] = end;
+	s_origin[wave][lane] = origin;
+	s_width[wave][lane] = width;
+	s_index[wave][lane] = idx;
+	__builtin_amdgcn_wave_barrier();
+	const uint32_t run_end = s_end[wave][63];
+	for (uint32_t base = run_begin; base < run_end; base += 64) {
+		const uint32_t pos = base + (uint32_t)lane;
+		if (pos < run_end) {
+			// the first Gaussian whose inclusive offset exceeds pos
+			int lo = 0;
+#pragma unroll
+			for (int step = 32; step > 0; step >>= 1)
+				if (s_end[wave][lo + step - 1] <= pos)
+					lo += step;
+			const uint32_t first = lo == 0 ? run_begin : s_end[wave][lo - 1];
+			const uint32_t t = pos - first, w = s_width[wave][lo];
+			const uint32_t row = t / w;
+			keys[pos] = s_origin[wave][lo] + row * (uint32_t)gx + (t - row * w);
+			values[pos] = s_index[wave][lo];
 		}
 	}
 }
