@@ -36,9 +36,9 @@ FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
 # cannot be read from inside the process, so the figures are carried here; other workloads
 # report null.
 C1_TRAFFIC_MB_PER_LAUNCH = {
-    "preprocess_forward": 253.53, "duplicate_with_keys": 114.82, "sort_onesweep": 23.17, "tile_ranges": 13.22,
-    "blend_forward": 223.79, "composite_forward": 165.79, "composite_backward": 372.01, "blend_backward": 542.45,
-    "preprocess_backward": 370.05,
+    "preprocess_forward": 253.68, "duplicate_with_keys": 108.30, "sort_onesweep": 23.08, "tile_ranges": 13.22,
+    "blend_forward": 237.65, "composite_forward": 165.79, "composite_backward": 372.11, "blend_backward": 308.29,
+    "preprocess_backward": 370.17,
 }
 
 
