@@ -20,8 +20,8 @@
 //  * alpha >= 1/255 needs power >= -ln(255 * opacity); that floor (minus a margin) is stored
 //    with the Gaussian, and a group of entries is skipped with one ballot when no live lane
 //    reaches it, before exp() is evaluated.
-//  * power >= floor is an ellipse around the Gaussian's centre; an entry whose ellipse's
-//    bounding box misses the strip is not filed at all.
+//  * power >= floor is an ellipse around the Gaussian's centre; an entry whose ellipse (first
+//    its bounding box, then the ellipse itself) misses the strip's rectangle is not filed at all.
 //  * the world-space ray sample is affine in the pixel, so its extremes over the strip are at
 //    the strip's corner pixels: an entry whose corners are all outside the submodel box is not
 //    filed, one whose corners are all inside skips the per-pixel box test.
@@ -97,6 +97,38 @@ __device__ __forceinline__ bool reaches_strip(float gx, float gy, float hx, floa
 	if (floor > 0.f)
 		return false;  // even power = 0 gives alpha < 1/255
 	return !((gx + hx < x0) || (gx - hx > x0 + 15.f) || (gy + hy < ya) || (gy - hy > ya + 3.f));
+}
+
+// The same question answered with the ellipse itself: the smallest value over the strip's
+// rectangle of q(d) = a dx^2 + 2 b dx dy + c dy^2 (d = centre - pixel, conic = (a, b, c)), against
+// the -2 floor that power = -q / 2 >= floor allows.  With the centre outside the rectangle the
+// minimum of the convex q lies on one of the four edges, where it is a clamped parabola vertex.
+// Conservative: the rectangle contains the pixels, and the comparison leaves room for the
+// rounding of q (relative to its largest terms).  Anything that is not an ellipse, or NaN, is kept.
+__device__ __forceinline__ bool ellipse_reaches_strip(float gx, float gy, const float4 co, float floor, float x0, float ya)
+{
+	const float a = co.x, b = co.y, c = co.z;
+	if (!(a > 0.f) || !(c > 0.f) || !(a * c - b * b > 0.f))
+		return true;
+	const float dxl = gx - (x0 + 15.f), dxh = gx - x0, dyl = gy - (ya + 3.f), dyh = gy - ya;
+	if (!(dxl > 0.f) && !(dxh < 0.f) && !(dyl > 0.f) && !(dyh < 0.f))
+		return true;  // the centre lies within the strip
+	float qmin = INFINITY;
+#pragma unroll
+	for (int edge = 0; edge < 2; edge++) {
+		const float dy = edge ? dyh : dyl;
+		const float dx = fminf(dxh, fmaxf(dxl, -b * dy / a));
+		qmin = fminf(qmin, (a * dx + 2.f * b * dy) * dx + c * dy * dy);
+	}
+#pragma unroll
+	for (int edge = 0; edge < 2; edge++) {
+		const float dx = edge ? dxh : dxl;
+		const float dy = fminf(dyh, fmaxf(dyl, -b * dx / c));
+		qmin = fminf(qmin, (c * dy + 2.f * b * dx) * dy + a * dx * dx);
+	}
+	const float largest = a * fmaxf(dxl * dxl, dxh * dxh) + c * fmaxf(dyl * dyl, dyh * dyh);
+	const float limit = -2.f * floor;
+	return !(qmin > limit + (1e-3f + 1e-4f * limit + 1e-5f * largest));
 }
 
 // Where the rays of a whole strip, sampled at clip-w `w`, fall relative to the submodel box.
@@ -206,6 +238,8 @@ __device__ __forceinline__ void keep_padding_registers(const LoadedEntry& e)
 __device__ __forceinline__ bool file_entry(LoadedEntry& e, float x0, float ya, const StripCorners& sc, const BoxFrame& box)
 {
 	if (!reaches_strip(e.geom.x, e.geom.y, e.half.x, e.half.y, e.geom.z, x0, ya))
+		return false;
+	if (!ellipse_reaches_strip(e.geom.x, e.geom.y, e.conic, e.geom.z, x0, ya))
 		return false;
 	const int where = classify_strip_against_box(e.geom.w, sc, box);
 	if (where == kBoxOutside)
