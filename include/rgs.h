@@ -154,13 +154,12 @@ enum { RGS_ACC_FLOATS = 12 };
 
 /* Rasterizer::backward (K/cuda_rasterizer_hgs/rasterizer.h:60-96, rasterizer_impl.cu:355-466)
  * together with the zero-initialisation done by its torch shim
- * (K/rasterize_points.cu:165-174).  grad_accum (RGS_ACC_FLOATS*P floats) need not be cleared
- * by the caller.  dL_dmean2D (P,3; third column 0), dL_dopacity (P), dL_dcolor (P,3),
+ * (K/rasterize_points.cu:165-174).  grad_accum is RGS_ACC_FLOATS*P floats.  dL_dmean2D (P,3; third column 0), dL_dopacity (P), dL_dcolor (P,3),
  * dL_dmean3D (P,3), dL_dcov3D (P,6), dL_dsh (P,M,3), dL_dscale (P,3), dL_drot (P,4) are
  * complete when the call has run: rows of rendered Gaussians are computed, all others are
- * zero.  With outputs_zeroed = 0 the library clears the eight arrays itself, like the
- * reference's shim; a caller that hands over arrays it has already cleared (say, while the
- * forward pass was still running) passes 1 and saves that pass over them.  dL_dsh /
+ * zero.  With outputs_zeroed = 0 the library clears the eight arrays and grad_accum itself,
+ * like the reference's shim; a caller that hands over all nine already cleared (say, while
+ * the forward pass was still running) passes 1 and saves that pass over them.  dL_dsh /
  * dL_dscale / dL_drot may be NULL when shs / scales are NULL; dL_dpix_depth / dL_dalphas
  * may be NULL when no gradient arrived for the depth / alpha image (taken as zero). */
 int rgs_backward(int P, int D, int M, int R, int width, int height,

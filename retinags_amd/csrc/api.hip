@@ -590,8 +590,10 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
 	const size_t n = (size_t)P;
 
-	rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, (size_t)RGS_ACC_FLOATS * n, s);
-	RGS_STAGE("clear gradient sums");
+	if (!outputs_zeroed) {
+		rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, (size_t)RGS_ACC_FLOATS * n, s);
+		RGS_STAGE("clear gradient sums");
+	}
 
 	const float* colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
 	if (R > 0) {

@@ -202,11 +202,12 @@ def _rasterize_forward(*args):
 
 
 def _gradient_outputs(P, M, has_scales, device, make):
-    """The eight dense gradient tensors of K/rasterize_points.cu:165-174, carved out of one
-    allocation made with `make` (torch.empty or torch.zeros: one fill instead of eight);
+    """The eight dense gradient tensors of K/rasterize_points.cu:165-174 and the backward's
+    scratch for the per-Gaussian sums, carved out of one allocation made with `make`
+    (torch.empty or torch.zeros: one fill instead of nine);
     without scales the scale / rotation gradients are zeros in either case."""
     shapes = {"means2D": (P, 3), "opacity": (P, 1), "colors": (P, 3), "means3D": (P, 3), "cov3D": (P, 6),
-              "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4)}
+              "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4), "sums": (P, _capi.ACC_FLOATS)}
     sizes = {k: (math.prod(v) + 63) // 64 * 64 for k, v in shapes.items()}  # 256-byte aligned parts
     flat = make((sum(sizes.values()),), dtype=torch.float32, device=device)
     out, at = {}, 0
@@ -254,11 +255,10 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
     range_up = _dev_f32(range_up, device, "range_up")
     campos = _dev_f32(campos, device, "campos")
 
-    # Scratch rows in which the blend accumulates its per-Gaussian sums; the library clears them.
-    acc = torch.empty((_capi.ACC_FLOATS * P,), **f32)
     has_scales = scales.numel() != 0
     outputs_zeroed = cleared is not None
     out = cleared if outputs_zeroed else _gradient_outputs(P, M, has_scales, device, torch.empty)
+    acc = out["sums"]  # scratch rows in which the blend accumulates its per-Gaussian sums
     dL_dmeans2D, dL_dopacity, dL_dcolors = out["means2D"], out["opacity"], out["colors"]
     dL_dmeans3D, dL_dcov3D, dL_dsh = out["means3D"], out["cov3D"], out["sh"]
     dL_dscales, dL_drotations = out["scales"], out["rotations"]
