@@ -71,8 +71,8 @@ def ensure_built():
 def main():
     args = parse()
     if args.gpus != 1:
-        print(f"bench.py measures one GPU: the submodels of a frame are rendered one after another on a single "
-              f"MI355X and composited there; --gpus {args.gpus} is not supported.", file=sys.stderr)
+        print(f"bench.py measures one GPU: all submodels of a frame are rendered on a single MI355X (on its HIP "
+              f"streams) and composited there; --gpus {args.gpus} is not supported.", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the HIP library is the only implementation).", file=sys.stderr)
