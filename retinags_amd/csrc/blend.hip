@@ -1,6 +1,8 @@
-// Per-tile alpha blending, forward and backward.  One 16x16 tile per 256-thread block:
-// 4 wavefronts of 64 lanes, wavefront w owns the strip of pixel rows 4w..4w+3 of the tile,
-// one pixel per lane.  Tile lists are staged through LDS in batches of 256 entries.
+// Per-tile alpha blending, forward and backward.  A 16x16 tile is four strips of 16x4 pixels;
+// a wavefront owns one strip, one pixel per lane.  The forward runs a tile's four wavefronts
+// in one 256-thread block, the backward launches every strip as a block of its own (strips
+// end at very different times there, and a wave slot should not idle until its tile's longest
+// strip is done), longest strips first.
 //
 // Compiled with -ffp-contract=off: every per-pixel decision (power > 0, alpha < 1/255,
 // the half-Gaussian box test, T(1-alpha) < 1e-4) is evaluated with the unfused
@@ -14,6 +16,8 @@
 // of 64 entries (lane l takes entry l of the chunk; the next chunk's records and the ids of
 // the one after are already in flight while the current chunk is processed), keeps the
 // entries that can matter to its strip in a wave-private LDS list, and walks that list.
+// The forward also writes those entries' list positions out, strip by strip; the backward
+// walks exactly them (up to the last one any pixel blended) and repeats none of the filtering.
 //
 // Most (pixel, Gaussian) visits of the reference loop end at "alpha < 1/255" or at the box
 // test.  Three conservative filters remove such visits without changing any result:
@@ -495,17 +499,18 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 }
 
 // ---- backward (K/cuda_rasterizer_hgs/backward.cu:415-622) ---------------------------------------
-// Each wavefront walks the tile list back to front, starting at the largest last_contributor
-// of its own 64 pixels.  The pass is split in two so that no cross-lane reduction is needed
-// per entry:
+// Each wavefront walks, back to front, the entries the forward filed for its strip, starting at
+// the last one that any of its 64 pixels blended.  The pass is split in two so that no
+// cross-lane reduction is needed per entry:
 //  * pixel-parallel part (lane = pixel, as in the forward): the per-pixel recurrences of the
 //    reference loop give, for an entry, two numbers per pixel: u = G dL/dalpha-term and
 //    aT = alpha T.  They are parked in one LDS row per entry.
 //  * entry-parallel part, run whenever 16 rows are full (lane = (entry, strip row)): each lane
 //    sweeps the 16 pixels of its strip row and accumulates sum u, sum u dx, sum u dx^2 and
 //    sum aT g_{r,g,b,depth}; dy is constant along a strip row, so the y moments follow from
-//    those; two cross-row exchanges finish the sums and 16 lanes issue the ten global atomics
-//    of their entry (one per (strip, Gaussian) and quantity).
+//    those; two exchanges inside each quad of lanes finish the sums, and the quad adds its
+//    entry's ten sums into the Gaussian's row of `sums`, four neighbouring columns per atomic
+//    instruction.
 // All ten sums of the reference (mean2D x/y, conic xx/xy/yy, opacity, colour r/g/b, depth)
 // are linear in u and aT, which is what makes the split possible.
 
