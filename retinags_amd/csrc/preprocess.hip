@@ -1,6 +1,6 @@
 // Per-Gaussian stages: visibility marking, forward preprocess (projection, EWA
 // covariance, conic, radius, tile rectangle, SH colour) and the fused backward
-// preprocess.  One thread per Gaussian, 256 threads per block.
+// preprocess.  One thread per Gaussian (in the backward: per rendered Gaussian).
 //
 // This file is compiled with -ffp-contract=off: radii, tile counts, pixel
 // centres and depth bits feed the integer stages and must equal the unfused

@@ -1,7 +1,8 @@
 """HIP rasterizer vs the CPU checker on identical seeded inputs, stage by stage.
 
-Bit-exact: radii, tile counts, pixel centres, depth bits, clip-w, offsets, duplicated
-keys/values, sorted keys, per-tile Gaussian lists, tile ranges.  Within 1e-4 max-abs:
+Bit-exact: radii, tile counts, pixel centres, depth bits, clip-w, the depth order of the
+Gaussians and their offsets, the sorted (tile, depth) keys (rebuilt from the library's tile
+keys and depth bits), per-tile Gaussian lists, tile ranges.  Within 1e-4 max-abs:
 rendered colour, depth and alpha planes.  Within 1e-3 relative L2: every gradient.
 """
 import numpy as np
