@@ -11,6 +11,8 @@ loop needs.  Restates, in numpy:
 """
 from __future__ import annotations
 
+import math
+
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Tuple
 
@@ -144,27 +146,60 @@ def partition_scene(xyz: torch.Tensor, scales_activated: torch.Tensor, depth: in
     return Partition(grid, nodes, leaves, box_low, box_up, owner, members)
 
 
-def _box_may_be_seen(low, up, cam) -> bool:
-    """Conservative frustum test: a box is dropped only when all eight corners lie behind
-    the near plane or beyond one side plane.  (The reference intersects the exact hulls,
-    parallel_utils/grid_utils/utils.py:115-137; a box kept here that it would drop
-    renders an empty partial image, which composites as a no-op.)"""
-    corners = np.array([[x, y, z, 1.0] for x in (low[0], up[0]) for y in (low[1], up[1]) for z in (low[2], up[2])])
-    v = corners @ cam.world_view_transform.cpu().numpy().astype(np.float64)
-    z = v[:, 2]
-    if np.all(z < 0.01):
-        return False
-    tx, ty = cam.tanfovx, cam.tanfovy
-    for a, t in ((v[:, 0], tx), (v[:, 1], ty)):
-        if np.all(a > t * np.maximum(z, 0.0) + 1e-6) and np.all(z > 0):
-            return False
-        if np.all(a < -t * np.maximum(z, 0.0) - 1e-6) and np.all(z > 0):
-            return False
-    return True
+_BOX_CORNERS = np.array([[x, y, z] for x in (0, 1) for y in (0, 1) for z in (0, 1)], dtype=np.float32)
 
 
-def relation_vector(part: Partition, cam) -> np.ndarray:
-    """Compositing rank of every submodel for this camera, -1 when it cannot be seen."""
+def view_frustum_vertices(cam, z_near: Optional[float] = None, z_far: Optional[float] = None) -> np.ndarray:
+    """The eight corners, in camera space, of the frustum between z_near and z_far
+    (parallel_utils/grid_utils/utils.py:80-112: z_near is at least 0.01, z_far at most 1e6)."""
+    near = max(0.01, 0.01 if z_near is None else z_near)
+    far = min(1e6, 1e6 if z_far is None else z_far)
+    tx, ty = math.tan(cam.FoVx / 2), math.tan(cam.FoVy / 2)
+    unit = np.array([(tx, ty, 1), (tx, -ty, 1), (-tx, ty, 1), (-tx, -ty, 1)], dtype=np.float32)
+    return np.concatenate((unit * np.float32(near), unit * np.float32(far)), axis=0)
+
+
+def boxes_overlap_view(low: np.ndarray, up: np.ndarray, cam, z_near: float = 0.01, z_far: float = 1e6) -> np.ndarray:
+    """For K world-space boxes (low, up: (K,3)): does the box meet the camera's frustum?
+
+    Same predicate as is_overlapping_SpaceBox_View (parallel_utils/grid_utils/utils.py:115-137),
+    which asks whether the origin lies in the convex hull of the Minkowski difference of the two
+    vertex sets, i.e. whether the two convex bodies share a point (touching counts).  Decided
+    here without a hull: two convex polyhedra are disjoint exactly when one of the face normals
+    of either, or one of the cross products of an edge of one with an edge of the other,
+    separates their vertex sets.  A box in camera space has 3 face normals and 3 edge directions,
+    the frustum 5 face normals and 6 edge directions: 26 candidate axes, all K boxes at once.
+    """
+    low = np.asarray(low, dtype=np.float32).reshape(-1, 3)
+    up = np.asarray(up, dtype=np.float32).reshape(-1, 3)
+    corners = np.where(_BOX_CORNERS[None] > 0, up[:, None, :], low[:, None, :])
+    w2c_t = cam.world_view_transform.detach().cpu().numpy().astype(np.float32)
+    homogeneous = np.concatenate((corners, np.ones(corners.shape[:2] + (1,), dtype=np.float32)), axis=2)
+    box = np.dot(homogeneous, w2c_t)[..., :3].astype(np.float64)               # (K,8,3) camera space
+    frustum = view_frustum_vertices(cam, z_near, z_far).astype(np.float64)     # (8,3)
+    tx, ty = frustum[0, 0] / frustum[0, 2], frustum[0, 1] / frustum[0, 2]
+
+    # edge directions of the box in camera space (images of the world axes)
+    box_edges = np.stack((box[:, 4] - box[:, 0], box[:, 2] - box[:, 0], box[:, 1] - box[:, 0]), axis=1)   # (K,3,3)
+    box_normals = np.stack((np.cross(box_edges[:, 1], box_edges[:, 2]), np.cross(box_edges[:, 2], box_edges[:, 0]),
+                            np.cross(box_edges[:, 0], box_edges[:, 1])), axis=1)
+    frustum_normals = np.array([(0, 0, 1), (1, 0, -tx), (-1, 0, -tx), (0, 1, -ty), (0, -1, -ty)], dtype=np.float64)
+    frustum_edges = np.array([(1, 0, 0), (0, 1, 0), (tx, ty, 1), (tx, -ty, 1), (-tx, ty, 1), (-tx, -ty, 1)], dtype=np.float64)
+    crossed = np.cross(box_edges[:, :, None, :], frustum_edges[None, None, :, :]).reshape(len(box), 18, 3)
+    axes = np.concatenate((box_normals, np.broadcast_to(frustum_normals, (len(box), 5, 3)), crossed), axis=1)  # (K,26,3)
+    length = np.linalg.norm(axes, axis=2, keepdims=True)
+    axes = np.where(length > 1e-12, axes / np.maximum(length, 1e-300), 0.0)    # a vanishing cross product separates nothing
+
+    on_box = np.einsum("kad,kvd->kav", axes, box)
+    on_frustum = np.einsum("kad,vd->kav", axes, frustum)
+    apart = (on_box.max(axis=2) < on_frustum.min(axis=2)) | (on_frustum.max(axis=2) < on_box.min(axis=2))
+    return ~apart.any(axis=1)
+
+
+def relation_vector(part: Partition, cam, z_near: float = 0.01, z_far: float = 1000.0) -> np.ndarray:
+    """Compositing rank of every submodel for this camera, -1 when its box misses the frustum
+    between z_near and z_far (defaults: main.py:94-95).  A camera that sees no box at all gets
+    rank 0 everywhere (scene_utils.py:313-315)."""
     center = cam.camera_center.cpu().numpy().astype(np.float64)
     depth_bit = {"": 0}
     for path, node in part.nodes.items():
@@ -180,8 +215,9 @@ def relation_vector(part: Partition, cam) -> np.ndarray:
         keyed.append((tuple(depth_bit[leaf.path[:i + 1]] for i in range(len(leaf.path))), mid))
     keyed.sort(key=lambda t: t[0])
     rel = np.full(len(part.leaves), -1, dtype=np.int64)
+    seen = boxes_overlap_view(part.box_low, part.box_up, cam, z_near, z_far)
     for order, (_, mid) in enumerate(keyed):
-        if _box_may_be_seen(part.box_low[mid], part.box_up[mid], cam):
+        if seen[mid]:
             rel[mid] = order
     if (rel < 0).all():
         rel[:] = 0
