@@ -229,6 +229,66 @@ int rgs_composite_backward(int K, int height, int width,
                            const float* g_alpha, float* const* d_images, float* const* d_depths,
                            float* const* d_alphas, void* stream);
 
+/* ---- boundary straddlers: what a submodel lends to its neighbours ---------------------------
+ * The reference picks, per source submodel, the Gaussians whose 3-sigma cube reaches a face of
+ * the source's box, then per destination those whose cube meets the destination's box, with
+ * boolean-mask indexing of six tensors each time (gather_SharedGSInfo_with_boxes,
+ * parallel_utils/basic_parallel_trainer/result_aggregator.py:55-121), and concatenates a
+ * destination's own rows with what every other submodel lends it (merge_SharedGSInfo,
+ * result_aggregator.py:263-288).  Here the selection yields row lists and the merge reads the
+ * sources through them, once.
+ *
+ * rgs_straddler_select: means3D (n,3), scales (n,3; activated) on the device.  src_low/src_up
+ * (3 floats) and boxes_low/boxes_up (n_boxes x 3) are HOST arrays in world units;
+ * n_boxes <= RGS_MAX_SHARE_BOXES.  Box `skip` (the source itself; -1 for none) is lent nothing.
+ * counts[b] (device) receives the number of rows lent to box b and rows[b*capacity + j] their
+ * row numbers in ascending order; a count above `capacity` means the list was truncated and
+ * the call must be repeated with more room.  scratch: rgs_straddler_scratch_bytes(n, n_boxes). */
+#define RGS_MAX_SHARE_BOXES 64
+size_t rgs_straddler_scratch_bytes(int n, int n_boxes);
+int rgs_straddler_select(int n, const float* means3D, const float* scales,
+                         const float* src_low, const float* src_up,
+                         int n_boxes, const float* boxes_low, const float* boxes_up, int skip,
+                         uint32_t* counts, uint32_t* rows, uint32_t capacity, void* scratch, void* stream);
+
+/* One source's share of a destination: the five forward fields of the reference's SharedGSInfo
+ * (parallel_utils/basic_parallel_trainer/task_utils.py:230-247; its means2D is all zero in the
+ * forward direction, render_half_gs.py:7-14), device arrays of widths 3, 1, 3, 4, sh_floats,
+ * and the rows to take (device; NULL takes rows 0..count-1, which is how a destination's own
+ * rows are passed). */
+typedef struct rgs_shared_rows {
+	const float* means3D;
+	const float* opacity;
+	const float* scales;
+	const float* rotations;
+	const float* shs;
+	const uint32_t* rows;
+	uint32_t count;
+} rgs_shared_rows;
+/* Writes the segments one behind the other into the destination's arrays from row dst_row0 on
+ * (torch.cat of the picked rows, result_aggregator.py:279-286).  `segments` is a HOST array. */
+int rgs_merge_rows(int n_segments, const rgs_shared_rows* segments, uint32_t dst_row0, int sh_floats,
+                   float* means3D, float* opacity, float* scales, float* rotations, float* shs, void* stream);
+
+/* The adjoint (what autograd does for indexing followed by torch.cat): the gradient rows
+ * dst_row0.. of the merged arrays are ADDED to the rows they were read from.  A segment names
+ * the source's six gradient arrays (means2D included: its gradient is what densification reads,
+ * render_half_gs.py:16-18) and the same row list as in the forward, which must not be NULL.
+ * Any array pointer may be NULL on either side (that field is skipped). */
+typedef struct rgs_shared_grads {
+	float* means3D;
+	float* means2D;
+	float* opacity;
+	float* scales;
+	float* rotations;
+	float* shs;
+	const uint32_t* rows;
+	uint32_t count;
+} rgs_shared_grads;
+int rgs_merge_rows_backward(int n_segments, const rgs_shared_grads* segments, uint32_t dst_row0, int sh_floats,
+                            const float* g_means3D, const float* g_means2D, const float* g_opacity,
+                            const float* g_scales, const float* g_rotations, const float* g_shs, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -19,6 +19,19 @@ BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted"
 IMG_FIELDS = ("ranges", "n_contrib", "strip_filed", "strip_order")
 ACC_FLOATS = 12
 MAX_COMPOSITE = 64
+MAX_SHARE_BOXES = 64
+
+
+class SharedRows(C.Structure):
+    """rgs_shared_rows of include/rgs.h."""
+    _fields_ = [("means3D", C.c_void_p), ("opacity", C.c_void_p), ("scales", C.c_void_p), ("rotations", C.c_void_p),
+                ("shs", C.c_void_p), ("rows", C.c_void_p), ("count", C.c_uint32)]
+
+
+class SharedGrads(C.Structure):
+    """rgs_shared_grads of include/rgs.h."""
+    _fields_ = [("means3D", C.c_void_p), ("means2D", C.c_void_p), ("opacity", C.c_void_p), ("scales", C.c_void_p),
+                ("rotations", C.c_void_p), ("shs", C.c_void_p), ("rows", C.c_void_p), ("count", C.c_uint32)]
 
 
 class RgsError(RuntimeError):
@@ -56,12 +69,18 @@ def _load():
     pp = C.POINTER(vp)
     lib.rgs_composite_forward.argtypes = [i, i, i, pp, pp, pp, vp, vp, vp, vp, vp]
     lib.rgs_composite_backward.argtypes = [i, i, i, pp, pp, pp, vp, vp, vp, vp, pp, pp, pp, vp]
+    lib.rgs_straddler_scratch_bytes.restype, lib.rgs_straddler_scratch_bytes.argtypes = sz, [i, i]
+    fp = C.POINTER(C.c_float)
+    lib.rgs_straddler_select.argtypes = [i, vp, vp, fp, fp, i, fp, fp, i, vp, vp, C.c_uint32, vp, vp]
+    lib.rgs_merge_rows.argtypes = [i, C.POINTER(SharedRows), C.c_uint32, i, vp, vp, vp, vp, vp, vp]
+    lib.rgs_merge_rows_backward.argtypes = [i, C.POINTER(SharedGrads), C.c_uint32, i, vp, vp, vp, vp, vp, vp, vp]
     lib.rgs_stage_timing.argtypes = [i]
     lib.rgs_stage_timing_read.argtypes = [i, C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.POINTER(C.c_int)]
     lib.rgs_blend_work_counters.argtypes = [i, i, i, i, f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
                  "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
-                 "rgs_composite_forward", "rgs_composite_backward"):
+                 "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
+                 "rgs_merge_rows_backward"):
         getattr(lib, name).restype = i
     return lib
 
@@ -72,7 +91,8 @@ EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_byte
            "rgs_image_bytes", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
            "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
            "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward",
-           "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters")
+           "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",
+           "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward")
 WORK_COUNTERS = 7
 
 

@@ -30,6 +30,7 @@ SOURCES = {
     "binning.hip": [],
     "blend.hip": ["-ffp-contract=off"],
     "composite.hip": [],
+    "sharing.hip": ["-ffp-contract=off"],
 }
 
 HEADERS = ["rgs_device.h", "rgs_kernels.h", os.path.join("..", "..", "include", "rgs.h")]

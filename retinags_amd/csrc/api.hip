@@ -794,4 +794,148 @@ int rgs_composite_backward(int K, int height, int width,
 	return 0;
 }
 
+size_t rgs_straddler_scratch_bytes(int n, int n_boxes)
+{
+	if (n < 0 || n_boxes < 0)
+		return 0;
+	return sizeof(uint32_t) * (size_t)n_boxes * (rgs::straddler_select_blocks(n) + 1);
+}
+
+int rgs_straddler_select(int n, const float* means3D, const float* scales, const float* src_low, const float* src_up,
+                         int n_boxes, const float* boxes_low, const float* boxes_up, int skip, uint32_t* counts,
+                         uint32_t* rows, uint32_t capacity, void* scratch, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(n >= 0, "rgs_straddler_select: negative n");
+	RGS_REQUIRE(n_boxes >= 1 && n_boxes <= rgs::kMaxShareBoxes, "rgs_straddler_select: n_boxes = %d, must be 1..%d", n_boxes,
+	            rgs::kMaxShareBoxes);
+	RGS_REQUIRE(skip >= -1 && skip < n_boxes, "rgs_straddler_select: skip = %d is not a box", skip);
+	RGS_REQUIRE(src_low && src_up && boxes_low && boxes_up, "rgs_straddler_select: null box");
+	RGS_REQUIRE(counts && scratch, "rgs_straddler_select: null counts or scratch");
+	RGS_REQUIRE(n == 0 || (means3D && scales), "rgs_straddler_select: null input");
+	RGS_REQUIRE(capacity == 0 || rows, "rgs_straddler_select: null rows");
+	rgs::StraddlerSelectArgs a;
+	a.n = n;
+	a.means3D = means3D;
+	a.scales = scales;
+	for (int c = 0; c < 3; c++) {
+		a.src_low[c] = src_low[c];
+		a.src_up[c] = src_up[c];
+	}
+	a.boxes.count = n_boxes;
+	for (int b = 0; b < n_boxes; b++)
+		for (int c = 0; c < 3; c++) {
+			a.boxes.low[b][c] = boxes_low[3 * b + c];
+			a.boxes.up[b][c] = boxes_up[3 * b + c];
+		}
+	a.skip = skip;
+	a.block_counts = static_cast<uint32_t*>(scratch);
+	a.counts = counts;
+	a.rows = rows;
+	a.capacity = capacity;
+	rgs::launch_straddler_select(a, s);
+	RGS_STAGE("straddler_select");
+	return 0;
+}
+
+namespace {
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+}
+
+int rgs_merge_rows(int n_segments, const rgs_shared_rows* segments, uint32_t dst_row0, int sh_floats, float* means3D,
+                   float* opacity, float* scales, float* rotations, float* shs, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(n_segments >= 0 && (n_segments == 0 || segments), "rgs_merge_rows: bad segment list");
+	RGS_REQUIRE(sh_floats >= 0, "rgs_merge_rows: negative sh_floats");
+	uint64_t total = dst_row0;
+	for (int i = 0; i < n_segments; i++) {
+		const rgs_shared_rows& g = segments[i];
+		RGS_REQUIRE(g.count == 0 || (g.means3D && g.opacity && g.scales && g.rotations && (g.shs || sh_floats == 0)),
+		            "rgs_merge_rows: null field in segment %d", i);
+		total += g.count;
+	}
+	RGS_REQUIRE(total <= 0xffffffffull, "rgs_merge_rows: more than 2^32 rows");
+	if (total == dst_row0)
+		return 0;
+	RGS_REQUIRE(means3D && opacity && scales && rotations && (shs || sh_floats == 0), "rgs_merge_rows: null destination");
+	uint32_t row0 = dst_row0;
+	int i = 0;
+	while (i < n_segments) {
+		rgs::MergeArgs a;
+		a.segments = 0;
+		a.sh_floats = sh_floats;
+		a.means3D = means3D; a.opacity = opacity; a.scales = scales; a.rotations = rotations; a.shs = shs;
+		bool wide = sh_floats % 4 == 0 && aligned16(shs) && aligned16(rotations);
+		uint32_t blocks = 0;
+		for (; i < n_segments && a.segments < rgs::kMaxMergeSegments; i++) {
+			const rgs_shared_rows& g = segments[i];
+			if (g.count == 0)
+				continue;
+			rgs::MergeSegment& m = a.seg[a.segments++];
+			m.means3D = g.means3D; m.opacity = g.opacity; m.scales = g.scales; m.rotations = g.rotations; m.shs = g.shs;
+			m.rows = g.rows;
+			m.count = g.count;
+			m.dst_row0 = row0;
+			m.block0 = blocks;
+			wide = wide && aligned16(g.shs) && aligned16(g.rotations);
+			row0 += g.count;
+			blocks += rgs::merge_blocks_for(g.count);
+		}
+		rgs::launch_merge_rows(a, blocks, wide, s);
+		RGS_STAGE("merge_rows");
+	}
+	return 0;
+}
+
+int rgs_merge_rows_backward(int n_segments, const rgs_shared_grads* segments, uint32_t dst_row0, int sh_floats,
+                            const float* g_means3D, const float* g_means2D, const float* g_opacity, const float* g_scales,
+                            const float* g_rotations, const float* g_shs, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(n_segments >= 0 && (n_segments == 0 || segments), "rgs_merge_rows_backward: bad segment list");
+	RGS_REQUIRE(sh_floats >= 0, "rgs_merge_rows_backward: negative sh_floats");
+	uint64_t total = dst_row0;
+	for (int i = 0; i < n_segments; i++) {
+		RGS_REQUIRE(segments[i].count == 0 || segments[i].rows, "rgs_merge_rows_backward: segment %d has no row list", i);
+		total += segments[i].count;
+	}
+	RGS_REQUIRE(total <= 0xffffffffull, "rgs_merge_rows_backward: more than 2^32 rows");
+	uint32_t row0 = dst_row0;
+	int i = 0;
+	while (i < n_segments) {
+		rgs::MergeBackwardArgs a;
+		a.segments = 0;
+		a.sh_floats = sh_floats;
+		a.means3D = g_means3D; a.means2D = g_means2D; a.opacity = g_opacity; a.scales = g_scales;
+		a.rotations = g_rotations; a.shs = g_shs;
+		bool wide = sh_floats % 4 == 0 && aligned16(g_shs) && aligned16(g_rotations);
+		uint32_t blocks = 0;
+		for (; i < n_segments && a.segments < rgs::kMaxMergeSegments; i++) {
+			const rgs_shared_grads& g = segments[i];
+			if (g.count == 0)
+				continue;
+			rgs::MergeBackwardSegment& m = a.seg[a.segments++];
+			m.means3D = g.means3D; m.means2D = g.means2D; m.opacity = g.opacity; m.scales = g.scales;
+			m.rotations = g.rotations; m.shs = g.shs;
+			m.rows = g.rows;
+			m.count = g.count;
+			m.dst_row0 = row0;
+			m.block0 = blocks;
+			wide = wide && aligned16(g.shs) && aligned16(g.rotations);
+			row0 += g.count;
+			blocks += rgs::merge_blocks_for(g.count);
+		}
+		rgs::launch_merge_rows_backward(a, blocks, wide, s);
+		RGS_STAGE("merge_rows_backward");
+	}
+	return 0;
+}
+
 }  // extern "C"

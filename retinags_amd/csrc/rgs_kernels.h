@@ -129,6 +129,67 @@ struct CompositeArgs {
 	float* d_alphas[kMaxComposite];
 };
 
+// Boundary straddlers (sharing.hip).  Boxes are passed by value: at most kMaxShareBoxes per launch.
+constexpr int kMaxShareBoxes = 64;
+struct ShareBoxes {
+	float low[kMaxShareBoxes][3];
+	float up[kMaxShareBoxes][3];
+	int count;
+};
+struct StraddlerSelectArgs {
+	int n;
+	const float* means3D;   // (n,3)
+	const float* scales;    // (n,3) activated
+	float src_low[3], src_up[3];
+	ShareBoxes boxes;       // destinations
+	int skip;               // index of a destination that is never lent to (the source itself), or -1
+	uint32_t* block_counts; // boxes.count x straddler_select_blocks(n) words of scratch
+	uint32_t* counts;       // boxes.count
+	uint32_t* rows;         // boxes.count x capacity; rows beyond capacity are counted, not stored
+	uint32_t capacity;
+};
+constexpr int kMaxMergeSegments = 32;
+struct MergeSegment {
+	const float* means3D;
+	const float* opacity;
+	const float* scales;
+	const float* rotations;
+	const float* shs;
+	const uint32_t* rows;   // null: rows 0..count-1 of the source
+	uint32_t count, dst_row0, block0;
+};
+struct MergeArgs {
+	MergeSegment seg[kMaxMergeSegments];
+	int segments;
+	int sh_floats;
+	float* means3D;
+	float* opacity;
+	float* scales;
+	float* rotations;
+	float* shs;
+};
+struct MergeBackwardSegment {
+	float* means3D;
+	float* means2D;
+	float* opacity;
+	float* scales;
+	float* rotations;
+	float* shs;
+	const uint32_t* rows;
+	uint32_t count, dst_row0, block0;
+};
+struct MergeBackwardArgs {
+	MergeBackwardSegment seg[kMaxMergeSegments];
+	int segments;
+	int sh_floats;
+	const float* means3D;   // gradients of the merged arrays; any may be null
+	const float* means2D;
+	const float* opacity;
+	const float* scales;
+	const float* rotations;
+	const float* shs;
+};
+
 // preprocess.hip
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s);
 void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s);
@@ -192,6 +253,13 @@ void launch_blend_backward(const BlendArgs& a, hipStream_t s);
 void launch_composite_forward(const CompositeArgs& a, hipStream_t s);
 void launch_composite_backward(const CompositeArgs& a, hipStream_t s);
 void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s);
+
+// sharing.hip
+uint32_t straddler_select_blocks(int n);
+void launch_straddler_select(const StraddlerSelectArgs& a, hipStream_t s);
+uint32_t merge_blocks_for(uint32_t rows);   // workgroups one segment of that many rows takes
+void launch_merge_rows(const MergeArgs& a, uint32_t blocks, bool by_16_bytes, hipStream_t s);
+void launch_merge_rows_backward(const MergeBackwardArgs& a, uint32_t blocks, bool by_16_bytes, hipStream_t s);
 
 // api.hip: optional stage timing.  A mark names the work launched after it.
 void stage_mark(const char* name, hipStream_t s);

@@ -31,6 +31,7 @@ class Submodel:
     range_low: torch.Tensor
     range_up: torch.Tensor
     active_sh_degree: int = 3
+    means2D: Optional[torch.Tensor] = None   # screen-space placeholder whose gradient densification reads
 
     def parameters(self) -> List[torch.Tensor]:
         return [self.means3D, self.opacity, self.scales, self.rotations, self.shs]
@@ -50,6 +51,25 @@ def submodels_from_partition(scene: Dict[str, torch.Tensor], part: Partition, de
                              pick(scene["rotations"]), pick(scene["shs"]),
                              torch.from_numpy(part.box_low[k]).to(device), torch.from_numpy(part.box_up[k]).to(device)))
     return subs
+
+
+def owned_models_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device) -> List["SharedGSInfo"]:
+    """Every submodel's OWN Gaussians (no lent rows) as the six tensors it shows its neighbours."""
+    from ..sharing import SharedGSInfo
+    out = []
+    for k in range(len(part.leaves)):
+        idx = torch.from_numpy(np.nonzero(part.owner == k)[0])
+        pick = lambda t: t[idx].to(device).contiguous()
+        xyz = pick(scene["xyz"])
+        out.append(SharedGSInfo(xyz, torch.zeros_like(xyz), pick(scene["opacity"]), pick(scene["scales"]),
+                                pick(scene["rotations"]), pick(scene["shs"])))
+    return out
+
+
+def submodels_from_shared(merged: List["SharedGSInfo"], part: Partition, device) -> List[Submodel]:
+    """Renderer inputs from merged (own + lent) tensors, e.g. those of sharing.merge_shared."""
+    return [Submodel(m.means3D, m.opacity, m.scales, m.rotations, m.shs, torch.from_numpy(part.box_low[k]).to(device),
+                     torch.from_numpy(part.box_up[k]).to(device), means2D=m.means2D) for k, m in enumerate(merged)]
 
 
 def whole_scene_submodel(scene: Dict[str, torch.Tensor], device, margin: float = 1.0) -> Submodel:
@@ -82,7 +102,9 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
         rasterizer, geometry = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug)), None
     else:
         rasterizer, geometry = started
-    means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
+    means2D = sub.means2D
+    if means2D is None:
+        means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
     color, radii, depth, alpha = rasterizer(
         means3D=sub.means3D, means2D=means2D, shs=sub.shs, colors_precomp=None, opacities=sub.opacity,
         scales=sub.scales, rotations=sub.rotations, cov3D_precomp=None, geometry=geometry)
