@@ -238,6 +238,10 @@ def main():
         if "blend_forward" in stages and stages["blend_forward"]["ms_per_step"] > 0 else None,
     }
 
+    # ---- the step before the path: who lends which Gaussians to whom, and the merged inputs
+    sharing = ({"appending": sharing_stages(scene, part, dev, prof_steps, True),
+                "copying": sharing_stages(scene, part, dev, prof_steps, False)} if part is not None else None)
+
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
     cpu = None
     if not args.no_cpu_baseline:
@@ -255,9 +259,63 @@ def main():
                    "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
                    "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1)},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
-        "blend_work": evals,
+        "blend_work": evals, "sharing": sharing,
     }
     print(json.dumps(line))
+
+
+def sharing_stages(scene, part, dev, repeats, append):
+    """Times the selection of boundary straddlers, the merge of every submodel's input and the
+    backward of the merge (not part of a step: the step starts from merged inputs).  HIP events
+    recorded by the library on the launching stream; algorithmic bytes: one read of means and
+    scales per Gaussian and 4 per lent row for the selection, one read and one write of every
+    merged row (59 floats) for the merge, one read of a lent row's gradient (62 floats) and a
+    read-modify-write of the lender's row for the backward.  append: a submodel's own rows stay in
+    place and only the lent rows move; otherwise the merge copies the own rows too, as the
+    reference's torch.cat does."""
+    from retinags_amd import _capi, sharing
+    from retinags_amd.harness import pipeline
+    models = pipeline.owned_models_from_partition(scene, part, dev, spare_fraction=0.1 if append else 0.0)
+    for m in models:
+        for t in m.fields():
+            t.requires_grad_(True)
+    K = len(models)
+
+    def once():
+        table = sharing.select_straddlers(models, part.box_low, part.box_up)
+        merged = sharing.merge_shared(models, table, reuse_gradients=True, append=append)
+        outs = [t for m in merged for t in m.fields()]
+        torch.autograd.backward(outs, [torch.ones_like(t) for t in outs])
+        for m in models:
+            for t in m.fields():
+                t.grad = None
+        return table
+
+    table = once()
+    torch.cuda.synchronize()
+    _capi.stage_timing(True)
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        once()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / repeats
+    ms = _capi.stage_timing_read()
+    _capi.stage_timing(False)
+    owned = float(sum(table.own))
+    lent = float(table.counts.sum())
+    merged_rows = owned + lent
+    alg = {"straddler_select": 24.0 * owned + 4.0 * lent,
+           "merge_rows": 2 * 236.0 * (lent if append else merged_rows) + 4.0 * lent,
+           "merge_rows_backward": (248.0 + 2 * 248.0 + 4.0) * lent}
+    out = {"owned_gaussians": int(owned), "lent_rows": int(lent), "submodels": K, "wall_ms_per_pass": round(wall_ms, 3),
+           "own_rows": "in place, lent rows appended behind them" if append else "copied into the merged arrays"}
+    for name, (total, launches) in ms.items():
+        per = total / repeats
+        out[name] = {"ms_per_pass": round(per, 4), "launches_per_pass": launches / repeats,
+                     "achieved_GBps": round(alg[name] / (per * 1e-3) / 1e9, 1) if name in alg and per > 0 else None}
+        if out[name]["achieved_GBps"] is not None:
+            out[name]["frac"] = round(out[name]["achieved_GBps"] / HBM_PEAK_GBS, 4)
+    return out
 
 
 def cpu_baseline(scene, members, part, cam, rel, related, upstream, do_backward, args):

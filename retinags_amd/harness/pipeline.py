@@ -53,15 +53,19 @@ def submodels_from_partition(scene: Dict[str, torch.Tensor], part: Partition, de
     return subs
 
 
-def owned_models_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device) -> List["SharedGSInfo"]:
-    """Every submodel's OWN Gaussians (no lent rows) as the six tensors it shows its neighbours."""
-    from ..sharing import SharedGSInfo
+def owned_models_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device,
+                                spare_fraction: float = 0.0) -> List["SharedGSInfo"]:
+    """Every submodel's OWN Gaussians (no lent rows) as the six tensors it shows its neighbours.
+    With spare_fraction every tensor has room for that share of its rows (+4096) behind them,
+    which is what sharing.merge_shared(append=True) writes the lent rows into."""
+    from ..sharing import SharedGSInfo, with_spare_rows
     out = []
     for k in range(len(part.leaves)):
         idx = torch.from_numpy(np.nonzero(part.owner == k)[0])
-        pick = lambda t: t[idx].to(device).contiguous()
+        spare = int(len(idx) * spare_fraction) + 4096 if spare_fraction > 0 else 0
+        pick = lambda t: with_spare_rows(t[idx].to(device).contiguous(), spare)
         xyz = pick(scene["xyz"])
-        out.append(SharedGSInfo(xyz, torch.zeros_like(xyz), pick(scene["opacity"]), pick(scene["scales"]),
+        out.append(SharedGSInfo(xyz, with_spare_rows(torch.zeros_like(xyz), spare), pick(scene["opacity"]), pick(scene["scales"]),
                                 pick(scene["rotations"]), pick(scene["shs"])))
     return out
 

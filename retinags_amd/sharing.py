@@ -116,12 +116,25 @@ def _segments_for(dst: int, table: StraddlerTable) -> List[Tuple[int, Optional[t
     return out
 
 
+def _room_behind(t: torch.Tensor, rows: int) -> bool:
+    """Does the allocation t lives in continue for `rows` rows of t's width past t's first row?"""
+    width = int(np.prod(t.shape[1:])) if t.dim() > 1 else 1
+    return (t.storage_offset() + rows * width) * t.element_size() <= t.untyped_storage().nbytes()
+
+
+def _grown(t: torch.Tensor, rows: int) -> torch.Tensor:
+    """A tensor over the same memory as t with `rows` rows: t's own rows and the room behind them."""
+    width = tuple(t.shape[1:])
+    stride = tuple(t.stride())
+    return torch.empty(0, dtype=t.dtype, device=t.device).set_(t.untyped_storage(), t.storage_offset(), (rows,) + width, stride)
+
+
 class _MergeShared(torch.autograd.Function):
     """All destinations at once, so that a lender's gradient is written in one place: its own
     rows' gradient plus what every borrower adds."""
 
     @staticmethod
-    def forward(ctx, table: StraddlerTable, reuse_gradients: bool, *flat):
+    def forward(ctx, table: StraddlerTable, reuse_gradients: bool, append: bool, *flat):
         K = len(table.own)
         models = [flat[6 * m:6 * m + 6] for m in range(K)]
         device = flat[0].device
@@ -131,16 +144,28 @@ class _MergeShared(torch.autograd.Function):
         outs = []
         for dst in range(K):
             P = table.merged_size(dst)
-            merged = [torch.empty((P, 3), device=device), torch.zeros((P, 3), device=device), torch.empty((P, 1), device=device),
-                      torch.empty((P, 3), device=device), torch.empty((P, 4), device=device),
-                      torch.empty((P,) + sh_shape, device=device)]
-            segs = _segments_for(dst, table)
+            if append:
+                # the lent rows go behind the destination's own rows, which stay where they are
+                for f, t in enumerate(models[dst]):
+                    if not _room_behind(t, P):
+                        raise RuntimeError(f"submodel {dst}: no room for {P - table.own[dst]} lent rows behind its "
+                                           f"{FIELDS[f]}; allocate the field with spare rows or merge with append=False")
+                merged = [_grown(t, P) for t in models[dst]]
+                merged[1][table.own[dst]:].zero_()
+                segs = _segments_for(dst, table)[1:]
+                first = table.own[dst]
+            else:
+                merged = [torch.empty((P, 3), device=device), torch.zeros((P, 3), device=device),
+                          torch.empty((P, 1), device=device), torch.empty((P, 3), device=device),
+                          torch.empty((P, 4), device=device), torch.empty((P,) + sh_shape, device=device)]
+                segs = _segments_for(dst, table)
+                first = 0
             arr = (_capi.SharedRows * len(segs))()
             for k, (src, rows, count) in enumerate(segs):
                 m3, _, op, sc, ro, sh = models[src]
                 arr[k] = _capi.SharedRows(m3.data_ptr(), op.data_ptr(), sc.data_ptr(), ro.data_ptr(), sh.data_ptr(),
                                           rows.data_ptr() if rows is not None else None, count)
-            check(lib.rgs_merge_rows(len(segs), arr, 0, sh_floats, ptr(merged[0]), ptr(merged[2]), ptr(merged[3]),
+            check(lib.rgs_merge_rows(len(segs), arr, first, sh_floats, ptr(merged[0]), ptr(merged[2]), ptr(merged[3]),
                                      ptr(merged[4]), ptr(merged[5]), stream))
             outs.extend(merged)
         ctx.table = table
@@ -174,12 +199,19 @@ class _MergeShared(torch.autograd.Function):
             g = [grads[6 * dst + f] for f in range(6)]
             g = [None if t is None else t.contiguous() for t in g]
             check(lib.rgs_merge_rows_backward(len(segs), arr, table.own[dst], ctx.sh_floats, *[ptr(t) for t in g], stream))
-        return (None, None) + tuple(out)
+        return (None, None, None) + tuple(out)
 
 
-def merge_shared(models: Sequence[SharedGSInfo], table: StraddlerTable, reuse_gradients: bool = False) -> List[SharedGSInfo]:
+def merge_shared(models: Sequence[SharedGSInfo], table: StraddlerTable, reuse_gradients: bool = False,
+                 append: bool = False) -> List[SharedGSInfo]:
     """Every submodel's merged input (merge_SharedGSInfo, result_aggregator.py:263-288, for all
     destinations), differentiable with respect to every field of every submodel.
+
+    append: instead of copying a submodel's own rows into new arrays, write the lent rows into
+    the memory right behind them and return tensors over both.  Every field of every submodel
+    must then sit in an allocation with that much room behind its rows (with_spare_rows makes
+    such tensors); the merged tensors alias the submodel's own, and the room behind is
+    overwritten by every merge.
 
     reuse_gradients: the backward returns the incoming gradient buffers of the merged arrays,
     with the borrowers' rows added in place, instead of copies.  Only for callers that do not
@@ -189,5 +221,12 @@ def merge_shared(models: Sequence[SharedGSInfo], table: StraddlerTable, reuse_gr
             _require_device_rows(getattr(m, name), width, name)
         _require_device_rows(m.shs, tuple(models[0].shs.shape[1:]), "shs")
     flat = [t for m in models for t in m.fields()]
-    outs = _MergeShared.apply(table, reuse_gradients, *flat)
+    outs = _MergeShared.apply(table, reuse_gradients, append, *flat)
     return [SharedGSInfo(*outs[6 * m:6 * m + 6]) for m in range(len(models))]
+
+
+def with_spare_rows(t: torch.Tensor, spare: int) -> torch.Tensor:
+    """A copy of t (N rows) at the start of an allocation of N + spare rows, for merge_shared(append=True)."""
+    room = torch.empty((t.shape[0] + spare,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+    room[:t.shape[0]].copy_(t)
+    return room[:t.shape[0]]

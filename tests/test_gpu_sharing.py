@@ -13,13 +13,13 @@ DEV = "cuda:0"
 NAMES = ("means3D", "means2D", "opacity", "scales", "rotations", "shs")
 
 
-def _setup(shrink, depth, scale_shift=0.0):
+def _setup(shrink, depth, scale_shift=0.0, spare_fraction=0.0):
     from retinags_amd.harness import partition, pipeline
     scene, cam, _ = scenes.make_config("C1", shrink=shrink)
     if scale_shift:
         scene["scales"] = scene["scales"] * float(np.exp(scale_shift))
     part = partition.partition_scene(scene["xyz"], scene["scales"], depth)
-    models = pipeline.owned_models_from_partition(scene, part, DEV)
+    models = pipeline.owned_models_from_partition(scene, part, DEV, spare_fraction)
     return scene, cam, part, models
 
 
@@ -123,6 +123,38 @@ def test_in_place_gradients_match_copies():
         results.append([t.grad.clone() for m in models for t in m.fields()])
     for a, b in zip(*results):
         assert torch.equal(a, b)
+
+
+def test_lent_rows_appended_in_place_match_the_copying_merge():
+    """append=True leaves a submodel's own rows where they are and writes the lent rows behind
+    them; merged values and every gradient are those of the copying merge."""
+    from retinags_amd import sharing
+    scene, cam, part, models = _setup(100, 2, 1.0, spare_fraction=0.2)
+    K = len(models)
+    for m in models:
+        for t in m.fields():
+            t.requires_grad_(True)
+    table = sharing.select_straddlers(models, part.box_low, part.box_up)
+    values, grads = [], []
+    for append in (False, True):
+        for m in models:
+            for t in m.fields():
+                t.grad = None
+        merged = sharing.merge_shared(models, table, reuse_gradients=append, append=append)
+        if append:
+            assert all(a.data_ptr() == b.data_ptr() for m, g in zip(models, merged) for a, b in zip(m.fields(), g.fields()))
+        values.append([t.detach().clone() for g in merged for t in g.fields()])
+        gen = torch.Generator().manual_seed(12)
+        outs = [t for g in merged for t in g.fields()]
+        torch.autograd.backward(outs, [torch.randn(o.shape, generator=gen).to(DEV) for o in outs])
+        torch.cuda.synchronize()
+        grads.append([t.grad.clone() for m in models for t in m.fields()])
+    assert all(torch.equal(a, b) for a, b in zip(*values))
+    assert all(torch.equal(a, b) for a, b in zip(*grads))
+    # without room behind the rows the request is refused
+    tight = [sharing.SharedGSInfo(*[t.detach().clone() for t in m.fields()]) for m in models]
+    with pytest.raises(RuntimeError, match="no room"):
+        sharing.merge_shared(tight, table, append=True)
 
 
 def test_frame_through_shared_rows_matches_frame_from_host_lists():
