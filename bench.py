@@ -242,6 +242,9 @@ def main():
     sharing = ({"appending": sharing_stages(scene, part, dev, prof_steps, True),
                 "copying": sharing_stages(scene, part, dev, prof_steps, False)} if part is not None else None)
 
+    # ---- the steps after the path: image loss with its gradient, and the optimiser step
+    after = training_stages(subs, H, W, dev, prof_steps) if do_backward else None
+
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
     cpu = None
     if not args.no_cpu_baseline:
@@ -259,7 +262,7 @@ def main():
                    "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
                    "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1)},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
-        "blend_work": evals, "sharing": sharing,
+        "blend_work": evals, "sharing": sharing, "loss_and_optimiser": after,
     }
     print(json.dumps(line))
 
@@ -314,6 +317,56 @@ def sharing_stages(scene, part, dev, repeats, append):
         out[name] = {"ms_per_pass": round(per, 4), "launches_per_pass": launches / repeats,
                      "achieved_GBps": round(alg[name] / (per * 1e-3) / 1e9, 1) if name in alg and per > 0 else None}
         if out[name]["achieved_GBps"] is not None:
+            out[name]["frac"] = round(out[name]["achieved_GBps"] / HBM_PEAK_GBS, 4)
+    return out
+
+
+def training_stages(subs, H, W, dev, repeats):
+    """Times the image loss (forward and backward) at the frame's size and one Adam step over the
+    59 trainable floats (+1 untrained placeholder) of every Gaussian the submodels own, in the
+    reference's seven parameter groups per submodel.  Not part of a step.  Algorithmic bytes: the
+    loss reads image and ground truth and writes three derivative maps (20 B per pixel and channel),
+    its backward reads the five and writes the gradient (24 B); Adam reads parameter, gradient and
+    two moments and writes three of them (28 B per float)."""
+    from retinags_amd import _capi
+    from retinags_amd.loss import l1_ssim_loss
+    from retinags_amd.optimizer import Adam
+    gen = torch.Generator().manual_seed(4)
+    gt = torch.rand(3, H, W, generator=gen).to(dev)
+    image = (gt * 0.8 + 0.1 * torch.rand(3, H, W, generator=gen).to(dev)).requires_grad_(True)
+    widths = [3, 3, 45, 1, 1, 3, 4]          # xyz, f_dc, f_rest, opacity, means2D_meta, scaling, rotation
+    lrs = [0.00016, 0.0025, 0.0025 / 20.0, 0.05, 0.0, 0.005, 0.001]
+    optimisers, floats = [], 0
+    for s in subs:
+        n = int(s.means3D.shape[0])
+        params = [torch.nn.Parameter(torch.randn(n, w, device=dev) * 0.1) for w in widths]
+        for p in params:
+            p.grad = torch.randn_like(p) * 1e-3
+        floats += n * sum(widths)
+        optimisers.append(Adam([{"params": [p], "lr": lr} for p, lr in zip(params, lrs)], lr=0.0, eps=1e-15))
+
+    def once():
+        loss, _ = l1_ssim_loss(image, gt, 0.2)
+        loss.backward()
+        image.grad = None
+        for o in optimisers:
+            o.step()
+
+    once()
+    torch.cuda.synchronize()
+    _capi.stage_timing(True)
+    for _ in range(repeats):
+        once()
+    ms = _capi.stage_timing_read()
+    _capi.stage_timing(False)
+    pixels = 3.0 * H * W
+    alg = {"l1_ssim_forward": 20.0 * pixels, "l1_ssim_backward": 24.0 * pixels, "adam_step": 28.0 * floats}
+    out = {"image": f"3x{H}x{W}", "adam_floats": floats}
+    for name, (total, launches) in ms.items():
+        per = total / repeats
+        out[name] = {"ms_per_pass": round(per, 4), "launches_per_pass": launches / repeats}
+        if name in alg and per > 0:
+            out[name]["achieved_GBps"] = round(alg[name] / (per * 1e-3) / 1e9, 1)
             out[name]["frac"] = round(out[name]["achieved_GBps"] / HBM_PEAK_GBS, 4)
     return out
 

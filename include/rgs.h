@@ -289,6 +289,43 @@ int rgs_merge_rows_backward(int n_segments, const rgs_shared_grads* segments, ui
                             const float* g_means3D, const float* g_means2D, const float* g_opacity,
                             const float* g_scales, const float* g_rotations, const float* g_shs, void* stream);
 
+/* ---- image loss ------------------------------------------------------------------------------
+ * loss = (1 - lambda_dssim) * mean|image - gt| + lambda_dssim * (1 - SSIM(image, gt)), what
+ * loss_local computes per camera (parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:
+ * 436-455) from l1_loss and ssim (utils/loss_utils.py:17-18, 39-63: 11x11 Gaussian window, sigma
+ * 1.5, zero padding, mean over all pixels and channels).  image, gt: (channels, height, width)
+ * on the device.  out receives 3 floats on the device: the loss, the L1 term, the SSIM.
+ * workspace: rgs_loss_workspace_bytes() bytes; with keep_for_backward it keeps what
+ * rgs_l1_ssim_backward needs until that call.  The backward writes d loss / d image scaled by
+ * *grad_loss (a device scalar; NULL means 1); image, gt and lambda_dssim must be the forward's. */
+size_t rgs_loss_workspace_bytes(int channels, int height, int width);
+int rgs_l1_ssim_forward(int channels, int height, int width, const float* image, const float* gt,
+                        float lambda_dssim, float* out, void* workspace, int keep_for_backward, void* stream);
+int rgs_l1_ssim_backward(int channels, int height, int width, const float* image, const float* gt,
+                         float lambda_dssim, const float* grad_loss, const void* workspace, float* d_image,
+                         void* stream);
+
+/* ---- optimiser step ---------------------------------------------------------------------------
+ * torch.optim.Adam without weight decay or amsgrad, as the reference sets it up per submodel
+ * (scene/gaussian_nn_module.py:429-444) and steps it once per iteration
+ * (trainer4tree_partition.py:662-666): for every tensor, with t = step (>= 1, the count
+ * including this update),
+ *   exp_avg = beta1 exp_avg + (1 - beta1) grad;  exp_avg_sq = beta2 exp_avg_sq + (1 - beta2) grad^2;
+ *   param -= lr / (1 - beta1^t) * exp_avg / (sqrt(exp_avg_sq) / sqrt(1 - beta2^t) + eps).
+ * `tensors` is a HOST array (one entry per parameter group member); all arrays on the device,
+ * n floats each.  Hyper-parameters are doubles, as torch holds them: 1 - beta and the bias
+ * corrections are formed in double and rounded to float once.  One launch per 16 tensors. */
+typedef struct rgs_adam_tensor {
+	float* param;
+	const float* grad;
+	float* exp_avg;
+	float* exp_avg_sq;
+	size_t n;
+	double lr;
+	int step;
+} rgs_adam_tensor;
+int rgs_adam_step(int n_tensors, const rgs_adam_tensor* tensors, double beta1, double beta2, double eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -34,6 +34,12 @@ class SharedGrads(C.Structure):
                 ("rotations", C.c_void_p), ("shs", C.c_void_p), ("rows", C.c_void_p), ("count", C.c_uint32)]
 
 
+class AdamTensor(C.Structure):
+    """rgs_adam_tensor of include/rgs.h."""
+    _fields_ = [("param", C.c_void_p), ("grad", C.c_void_p), ("exp_avg", C.c_void_p), ("exp_avg_sq", C.c_void_p),
+                ("n", C.c_size_t), ("lr", C.c_double), ("step", C.c_int)]
+
+
 class RgsError(RuntimeError):
     pass
 
@@ -74,13 +80,17 @@ def _load():
     lib.rgs_straddler_select.argtypes = [i, vp, vp, fp, fp, i, fp, fp, i, vp, vp, C.c_uint32, vp, vp]
     lib.rgs_merge_rows.argtypes = [i, C.POINTER(SharedRows), C.c_uint32, i, vp, vp, vp, vp, vp, vp]
     lib.rgs_merge_rows_backward.argtypes = [i, C.POINTER(SharedGrads), C.c_uint32, i, vp, vp, vp, vp, vp, vp, vp]
+    lib.rgs_loss_workspace_bytes.restype, lib.rgs_loss_workspace_bytes.argtypes = sz, [i, i, i]
+    lib.rgs_l1_ssim_forward.argtypes = [i, i, i, vp, vp, f, vp, vp, i, vp]
+    lib.rgs_l1_ssim_backward.argtypes = [i, i, i, vp, vp, f, vp, vp, vp, vp]
+    lib.rgs_adam_step.argtypes = [i, C.POINTER(AdamTensor), C.c_double, C.c_double, C.c_double, vp]
     lib.rgs_stage_timing.argtypes = [i]
     lib.rgs_stage_timing_read.argtypes = [i, C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.POINTER(C.c_int)]
     lib.rgs_blend_work_counters.argtypes = [i, i, i, i, f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
                  "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
                  "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
-                 "rgs_merge_rows_backward"):
+                 "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step"):
         getattr(lib, name).restype = i
     return lib
 
@@ -92,7 +102,8 @@ EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_byte
            "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
            "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward",
            "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",
-           "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward")
+           "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward", "rgs_loss_workspace_bytes",
+           "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step")
 WORK_COUNTERS = 7
 
 

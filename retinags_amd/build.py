@@ -31,6 +31,7 @@ SOURCES = {
     "blend.hip": ["-ffp-contract=off"],
     "composite.hip": [],
     "sharing.hip": ["-ffp-contract=off"],
+    "training.hip": [],
 }
 
 HEADERS = ["rgs_device.h", "rgs_kernels.h", os.path.join("..", "..", "include", "rgs.h")]

@@ -4,6 +4,7 @@
 #include "../../include/rgs.h"
 #include "rgs_kernels.h"
 
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -934,6 +935,120 @@ int rgs_merge_rows_backward(int n_segments, const rgs_shared_grads* segments, ui
 		}
 		rgs::launch_merge_rows_backward(a, blocks, wide, s);
 		RGS_STAGE("merge_rows_backward");
+	}
+	return 0;
+}
+
+namespace {
+
+size_t loss_map_floats(int C, int H, int W) { return (size_t)3 * C * H * W; }
+
+int fill_loss(rgs::LossArgs& a, const char* who, int C, int H, int W, const float* image, const float* gt, float lambda,
+              const void* workspace)
+{
+	RGS_REQUIRE(C >= 1 && H >= 1 && W >= 1, "%s: bad image size %dx%dx%d", who, C, H, W);
+	RGS_REQUIRE((size_t)C * H * W < (1ull << 31), "%s: image too large", who);
+	RGS_REQUIRE(image && gt && workspace, "%s: null pointer", who);
+	a.C = C; a.H = H; a.W = W;
+	a.x = image;
+	a.y = gt;
+	a.lambda = lambda;
+	// utils/loss_utils.py:23-25: exp in double, stored as float, normalised in float
+	float g[11], sum = 0.f;
+	for (int i = 0; i < 11; i++) {
+		g[i] = (float)exp(-(double)((i - 5) * (i - 5)) / (2.0 * 1.5 * 1.5));
+		sum += g[i];
+	}
+	for (int i = 0; i < 11; i++)
+		a.w[i] = g[i] / sum;
+	float* ws = static_cast<float*>(const_cast<void*>(workspace));
+	a.maps = ws;
+	a.partial = ws + loss_map_floats(C, H, W);
+	a.out = nullptr;
+	a.grad_loss = nullptr;
+	a.d_image = nullptr;
+	return 0;
+}
+
+}  // namespace
+
+size_t rgs_loss_workspace_bytes(int channels, int height, int width)
+{
+	if (channels < 1 || height < 1 || width < 1)
+		return 0;
+	return sizeof(float) * (loss_map_floats(channels, height, width) + 2 * (size_t)rgs::loss_blocks(channels, height, width));
+}
+
+int rgs_l1_ssim_forward(int channels, int height, int width, const float* image, const float* gt, float lambda_dssim,
+                        float* out, void* workspace, int keep_for_backward, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	rgs::LossArgs a;
+	if (int rc = fill_loss(a, "rgs_l1_ssim_forward", channels, height, width, image, gt, lambda_dssim, workspace))
+		return rc;
+	RGS_REQUIRE(out, "rgs_l1_ssim_forward: null output");
+	a.out = out;
+	if (!keep_for_backward)
+		a.maps = nullptr;
+	rgs::launch_l1_ssim_forward(a, s);
+	RGS_STAGE("l1_ssim_forward");
+	return 0;
+}
+
+int rgs_l1_ssim_backward(int channels, int height, int width, const float* image, const float* gt, float lambda_dssim,
+                         const float* grad_loss, const void* workspace, float* d_image, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	rgs::LossArgs a;
+	if (int rc = fill_loss(a, "rgs_l1_ssim_backward", channels, height, width, image, gt, lambda_dssim, workspace))
+		return rc;
+	RGS_REQUIRE(d_image, "rgs_l1_ssim_backward: null output");
+	a.grad_loss = grad_loss;
+	a.d_image = d_image;
+	rgs::launch_l1_ssim_backward(a, s);
+	RGS_STAGE("l1_ssim_backward");
+	return 0;
+}
+
+int rgs_adam_step(int n_tensors, const rgs_adam_tensor* tensors, double beta1, double beta2, double eps, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(n_tensors >= 0 && (n_tensors == 0 || tensors), "rgs_adam_step: bad tensor list");
+	for (int i = 0; i < n_tensors; i++) {
+		const rgs_adam_tensor& t = tensors[i];
+		RGS_REQUIRE(t.n == 0 || (t.param && t.grad && t.exp_avg && t.exp_avg_sq), "rgs_adam_step: null array in tensor %d", i);
+		RGS_REQUIRE(t.step >= 1, "rgs_adam_step: tensor %d has step %d; the count includes this update", i, t.step);
+	}
+	int i = 0;
+	while (i < n_tensors) {
+		rgs::AdamArgs a;
+		a.tensors = 0;
+		a.beta1 = (float)beta1; a.beta2 = (float)beta2; a.eps = (float)eps;
+		a.one_minus_beta1 = (float)(1.0 - beta1); a.one_minus_beta2 = (float)(1.0 - beta2);
+		uint32_t blocks = 0;
+		for (; i < n_tensors && a.tensors < rgs::kMaxAdamTensors; i++) {
+			const rgs_adam_tensor& t = tensors[i];
+			if (t.n == 0)
+				continue;
+			rgs::AdamTensor& k = a.t[a.tensors++];
+			k.param = t.param; k.grad = t.grad; k.exp_avg = t.exp_avg; k.exp_avg_sq = t.exp_avg_sq;
+			k.n = t.n;
+			// torch/optim/adam.py: bias corrections and step size in double, applied as floats
+			const double c1 = 1.0 - pow(beta1, (double)t.step), c2 = 1.0 - pow(beta2, (double)t.step);
+			k.step_size = (float)(t.lr / c1);
+			k.bias2_sqrt = (float)sqrt(c2);
+			k.block0 = blocks;
+			k.by_16_bytes = aligned16(t.param) && aligned16(t.grad) && aligned16(t.exp_avg) && aligned16(t.exp_avg_sq);
+			blocks += rgs::adam_blocks_for(t.n);
+		}
+		rgs::launch_adam_step(a, blocks, s);
+		RGS_STAGE("adam_step");
 	}
 	return 0;
 }

@@ -190,6 +190,38 @@ struct MergeBackwardArgs {
 	const float* shs;
 };
 
+// Image loss and optimiser step (training.hip).
+struct LossArgs {
+	int C, H, W;
+	const float* x;          // rendered image (C,H,W)
+	const float* y;          // ground truth
+	float w[11];             // normalised 1-D Gaussian window
+	float lambda;            // weight of (1 - SSIM)
+	float* maps;             // 3 x C x H x W derivative maps (may be null in the forward: no backward will follow)
+	float* partial;          // 2 floats per workgroup
+	float* out;              // loss, L1, SSIM
+	const float* grad_loss;  // backward: upstream gradient of the loss (device scalar) or null for 1
+	float* d_image;          // backward: gradient of the loss with respect to x
+};
+constexpr int kMaxAdamTensors = 16;
+struct AdamTensor {
+	float* param;
+	const float* grad;
+	float* exp_avg;
+	float* exp_avg_sq;
+	size_t n;
+	float step_size;         // lr / (1 - beta1^t)
+	float bias2_sqrt;        // sqrt(1 - beta2^t)
+	uint32_t block0;
+	int by_16_bytes;
+};
+struct AdamArgs {
+	AdamTensor t[kMaxAdamTensors];
+	int tensors;
+	float beta1, beta2, eps;
+	float one_minus_beta1, one_minus_beta2;   // formed in double by the host
+};
+
 // preprocess.hip
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s);
 void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s);
@@ -260,6 +292,13 @@ void launch_straddler_select(const StraddlerSelectArgs& a, hipStream_t s);
 uint32_t merge_blocks_for(uint32_t rows);   // workgroups one segment of that many rows takes
 void launch_merge_rows(const MergeArgs& a, uint32_t blocks, bool by_16_bytes, hipStream_t s);
 void launch_merge_rows_backward(const MergeBackwardArgs& a, uint32_t blocks, bool by_16_bytes, hipStream_t s);
+
+// training.hip
+uint32_t loss_blocks(int C, int H, int W);   // workgroups of the loss kernels = pairs of partial sums
+void launch_l1_ssim_forward(const LossArgs& a, hipStream_t s);
+void launch_l1_ssim_backward(const LossArgs& a, hipStream_t s);
+uint32_t adam_blocks_for(size_t n);
+void launch_adam_step(const AdamArgs& a, uint32_t blocks, hipStream_t s);
 
 // api.hip: optional stage timing.  A mark names the work launched after it.
 void stage_mark(const char* name, hipStream_t s);

@@ -1,0 +1,284 @@
+// The two steps either side of the renderer in a training iteration: the image loss
+// (1 - lambda) L1 + lambda (1 - SSIM) with its gradient, and the Adam update of the parameters.
+//
+// SSIM (utils/loss_utils.py:39-63): five zero-padded 11x11 Gaussian-window (sigma 1.5) means per
+// pixel and channel, of x, y, x^2, y^2 and xy, then
+//   f = (2 mu1 mu2 + C1)(2 s12 + C2) / ((mu1^2 + mu2^2 + C1)(s11 + s22 + C2)),  C1 = 0.01^2, C2 = 0.03^2.
+// The window is an outer product, so each mean is a row pass followed by a column pass.  A
+// workgroup produces a 32x16 tile of one channel: the 42x26 pixels it needs go to LDS once, the
+// row pass leaves 5 x 26 x 32 partial means in LDS, the column pass finishes them, and the
+// per-pixel SSIM and |x - y| are summed per workgroup (a second kernel adds the partial sums in a
+// fixed order, so the loss is reproducible).  For the backward the same kernel stores three
+// derivative maps per pixel,
+//   a = df/dmu1,  b = df/dE[x^2] = -f / B2,  c = df/dE[xy] = 2 A1 / (B1 B2),
+// and the gradient is their windowed means: dL/dx(q) = W*a (q) + 2 x(q) W*b (q) + y(q) W*c (q),
+// which the backward kernel computes with the same two passes.  Bound by HBM (44 bytes per pixel
+// and channel over both kernels) and by LDS reads.
+//
+// Adam (torch.optim.Adam as the reference configures it, scene/gaussian_nn_module.py:429-444:
+// eps 1e-15, no weight decay, no amsgrad): one pass over parameter, gradient and both moments.
+#include "rgs_device.h"
+#include "rgs_kernels.h"
+
+namespace rgs {
+
+namespace {
+
+constexpr int kLossTileW = 32, kLossTileH = 16;
+constexpr int kHalo = 5, kTaps = 11;
+constexpr int kRegionW = kLossTileW + 2 * kHalo, kRegionH = kLossTileH + 2 * kHalo;
+
+__device__ __forceinline__ float block256_sum(float v, float* lds)
+{
+	v = wave_sum_to_lane63(v);
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	if (lane == 63)
+		lds[wave] = v;
+	__syncthreads();
+	const float total = lds[0] + lds[1] + lds[2] + lds[3];
+	__syncthreads();
+	return total;
+}
+
+__global__ __launch_bounds__(256) void ssim_forward_kernel(LossArgs a)
+{
+	__shared__ float sx[kRegionH][kRegionW + 1];
+	__shared__ float sy[kRegionH][kRegionW + 1];
+	__shared__ float rows[5][kRegionH][kLossTileW + 1];
+	__shared__ float red[4];
+	const int tid = threadIdx.x;
+	const size_t plane = (size_t)blockIdx.z * a.H * a.W;
+	const int x0 = blockIdx.x * kLossTileW - kHalo, y0 = blockIdx.y * kLossTileH - kHalo;
+	for (int i = tid; i < kRegionH * kRegionW; i += 256) {
+		const int r = i / kRegionW, c = i % kRegionW;
+		const int gx = x0 + c, gy = y0 + r;
+		const bool inside = gx >= 0 && gx < a.W && gy >= 0 && gy < a.H;
+		const size_t at = plane + (size_t)gy * a.W + gx;
+		sx[r][c] = inside ? a.x[at] : 0.f;
+		sy[r][c] = inside ? a.y[at] : 0.f;
+	}
+	__syncthreads();
+	for (int i = tid; i < kRegionH * kLossTileW; i += 256) {
+		const int r = i / kLossTileW, c = i % kLossTileW;
+		float m1 = 0.f, m2 = 0.f, xx = 0.f, yy = 0.f, xy = 0.f;
+#pragma unroll
+		for (int k = 0; k < kTaps; k++) {
+			const float w = a.w[k], u = sx[r][c + k], v = sy[r][c + k];
+			m1 += w * u;
+			m2 += w * v;
+			xx += w * (u * u);
+			yy += w * (v * v);
+			xy += w * (u * v);
+		}
+		rows[0][r][c] = m1; rows[1][r][c] = m2; rows[2][r][c] = xx; rows[3][r][c] = yy; rows[4][r][c] = xy;
+	}
+	__syncthreads();
+	float ssim_sum = 0.f, l1_sum = 0.f;
+	for (int i = tid; i < kLossTileH * kLossTileW; i += 256) {
+		const int r = i / kLossTileW, c = i % kLossTileW;
+		const int gx = x0 + kHalo + c, gy = y0 + kHalo + r;
+		if (gx >= a.W || gy >= a.H)
+			continue;
+		float m1 = 0.f, m2 = 0.f, xx = 0.f, yy = 0.f, xy = 0.f;
+#pragma unroll
+		for (int k = 0; k < kTaps; k++) {
+			const float w = a.w[k];
+			m1 += w * rows[0][r + k][c];
+			m2 += w * rows[1][r + k][c];
+			xx += w * rows[2][r + k][c];
+			yy += w * rows[3][r + k][c];
+			xy += w * rows[4][r + k][c];
+		}
+		const float C1 = 0.01f * 0.01f, C2 = 0.03f * 0.03f;
+		const float m11 = m1 * m1, m22 = m2 * m2, m12 = m1 * m2;
+		const float s11 = xx - m11, s22 = yy - m22, s12 = xy - m12;
+		const float A1 = 2.f * m12 + C1, A2 = 2.f * s12 + C2, B1 = m11 + m22 + C1, B2 = s11 + s22 + C2;
+		const float inv = 1.f / (B1 * B2);
+		const float f = A1 * A2 * inv;
+		ssim_sum += f;
+		l1_sum += fabsf(sx[r + kHalo][c + kHalo] - sy[r + kHalo][c + kHalo]);
+		if (a.maps) {
+			const size_t n = (size_t)a.C * a.H * a.W;
+			const size_t at = plane + (size_t)gy * a.W + gx;
+			a.maps[at] = 2.f * m2 * (A2 - A1) * inv - 2.f * m1 * f * (1.f / B1 - 1.f / B2);
+			a.maps[n + at] = -f / B2;
+			a.maps[2 * n + at] = 2.f * A1 * inv;
+		}
+	}
+	ssim_sum = block256_sum(ssim_sum, red);
+	l1_sum = block256_sum(l1_sum, red);
+	if (tid == 0) {
+		const size_t block = ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+		a.partial[2 * block] = ssim_sum;
+		a.partial[2 * block + 1] = l1_sum;
+	}
+}
+
+// One workgroup: the partial sums in index order (double accumulators), then the three results.
+__global__ __launch_bounds__(256) void loss_finish_kernel(LossArgs a, uint32_t blocks)
+{
+	__shared__ double red[2][256];
+	double s = 0.0, l = 0.0;
+	for (uint32_t i = threadIdx.x; i < blocks; i += 256) {
+		s += (double)a.partial[2 * i];
+		l += (double)a.partial[2 * i + 1];
+	}
+	red[0][threadIdx.x] = s;
+	red[1][threadIdx.x] = l;
+	__syncthreads();
+	for (int step = 128; step > 0; step >>= 1) {
+		if ((int)threadIdx.x < step) {
+			red[0][threadIdx.x] += red[0][threadIdx.x + step];
+			red[1][threadIdx.x] += red[1][threadIdx.x + step];
+		}
+		__syncthreads();
+	}
+	if (threadIdx.x == 0) {
+		const double n = (double)a.C * a.H * a.W;
+		const float ssim = (float)(red[0][0] / n), l1 = (float)(red[1][0] / n);
+		a.out[0] = (1.0f - a.lambda) * l1 + a.lambda * (1.0f - ssim);
+		a.out[1] = l1;
+		a.out[2] = ssim;
+	}
+}
+
+__global__ __launch_bounds__(256) void ssim_backward_kernel(LossArgs a)
+{
+	__shared__ float sm[3][kRegionH][kRegionW + 1];
+	__shared__ float rows[3][kRegionH][kLossTileW + 1];
+	const int tid = threadIdx.x;
+	const size_t n = (size_t)a.C * a.H * a.W;
+	const size_t plane = (size_t)blockIdx.z * a.H * a.W;
+	const int x0 = blockIdx.x * kLossTileW - kHalo, y0 = blockIdx.y * kLossTileH - kHalo;
+	for (int i = tid; i < kRegionH * kRegionW; i += 256) {
+		const int r = i / kRegionW, c = i % kRegionW;
+		const int gx = x0 + c, gy = y0 + r;
+		const bool inside = gx >= 0 && gx < a.W && gy >= 0 && gy < a.H;
+		const size_t at = plane + (size_t)gy * a.W + gx;
+		sm[0][r][c] = inside ? a.maps[at] : 0.f;
+		sm[1][r][c] = inside ? a.maps[n + at] : 0.f;
+		sm[2][r][c] = inside ? a.maps[2 * n + at] : 0.f;
+	}
+	__syncthreads();
+	for (int i = tid; i < kRegionH * kLossTileW; i += 256) {
+		const int r = i / kLossTileW, c = i % kLossTileW;
+		float pa = 0.f, pb = 0.f, pc = 0.f;
+#pragma unroll
+		for (int k = 0; k < kTaps; k++) {
+			const float w = a.w[k];
+			pa += w * sm[0][r][c + k];
+			pb += w * sm[1][r][c + k];
+			pc += w * sm[2][r][c + k];
+		}
+		rows[0][r][c] = pa; rows[1][r][c] = pb; rows[2][r][c] = pc;
+	}
+	__syncthreads();
+	const float upstream = a.grad_loss ? a.grad_loss[0] : 1.0f;
+	const float l1_scale = upstream * (1.0f - a.lambda) / (float)n, ssim_scale = -upstream * a.lambda / (float)n;
+	for (int i = tid; i < kLossTileH * kLossTileW; i += 256) {
+		const int r = i / kLossTileW, c = i % kLossTileW;
+		const int gx = x0 + kHalo + c, gy = y0 + kHalo + r;
+		if (gx >= a.W || gy >= a.H)
+			continue;
+		float ca = 0.f, cb = 0.f, cc = 0.f;
+#pragma unroll
+		for (int k = 0; k < kTaps; k++) {
+			const float w = a.w[k];
+			ca += w * rows[0][r + k][c];
+			cb += w * rows[1][r + k][c];
+			cc += w * rows[2][r + k][c];
+		}
+		const size_t at = plane + (size_t)gy * a.W + gx;
+		const float x = a.x[at], y = a.y[at];
+		const float d = x - y;
+		const float sign = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
+		a.d_image[at] = l1_scale * sign + ssim_scale * (ca + 2.f * x * cb + y * cc);
+	}
+}
+
+// torch.optim.Adam's single-tensor update, in its order of operations:
+//   m = b1 m + (1 - b1) g;  v = b2 v + (1 - b2) g g;
+//   p = p - (lr / (1 - b1^t)) * m / (sqrt(v) / sqrt(1 - b2^t) + eps)
+// One launch updates every tensor of a parameter-group list; a workgroup takes kAdamBlock
+// consecutive elements of one tensor.
+constexpr int kAdamBlock = 4096;
+
+__device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, const AdamTensor& t, const AdamArgs& a)
+{
+	m = m * a.beta1 + g * a.one_minus_beta1;
+	v = v * a.beta2 + (g * g) * a.one_minus_beta2;
+	const float denom = sqrtf(v) / t.bias2_sqrt + a.eps;
+	p = p - t.step_size * (m / denom);
+}
+
+__global__ __launch_bounds__(256) void adam_step_kernel(AdamArgs a)
+{
+	int k = 0;
+	while (k + 1 < a.tensors && blockIdx.x >= a.t[k + 1].block0)
+		k++;
+	const AdamTensor& t = a.t[k];
+	const size_t base = (size_t)(blockIdx.x - t.block0) * kAdamBlock;
+#pragma unroll
+	for (int it = 0; it < kAdamBlock / 1024; it++) {
+		const size_t i = base + (size_t)it * 1024 + threadIdx.x * 4;
+		if (i >= t.n)
+			break;
+		if (i + 4 <= t.n && t.by_16_bytes) {
+			float4 p = *reinterpret_cast<float4*>(t.param + i);
+			const float4 g = *reinterpret_cast<const float4*>(t.grad + i);
+			float4 m = *reinterpret_cast<float4*>(t.exp_avg + i);
+			float4 v = *reinterpret_cast<float4*>(t.exp_avg_sq + i);
+			adam_one(p.x, g.x, m.x, v.x, t, a);
+			adam_one(p.y, g.y, m.y, v.y, t, a);
+			adam_one(p.z, g.z, m.z, v.z, t, a);
+			adam_one(p.w, g.w, m.w, v.w, t, a);
+			*reinterpret_cast<float4*>(t.param + i) = p;
+			*reinterpret_cast<float4*>(t.exp_avg + i) = m;
+			*reinterpret_cast<float4*>(t.exp_avg_sq + i) = v;
+		} else {
+			for (size_t j = i; j < t.n && j < i + 4; j++) {
+				float p = t.param[j], m = t.exp_avg[j], v = t.exp_avg_sq[j];
+				adam_one(p, t.grad[j], m, v, t, a);
+				t.param[j] = p;
+				t.exp_avg[j] = m;
+				t.exp_avg_sq[j] = v;
+			}
+		}
+	}
+}
+
+}  // namespace
+
+uint32_t loss_blocks(int C, int H, int W)
+{
+	return (uint32_t)(((W + kLossTileW - 1) / kLossTileW) * ((H + kLossTileH - 1) / kLossTileH) * C);
+}
+
+void launch_l1_ssim_forward(const LossArgs& a, hipStream_t s)
+{
+	stage_mark("l1_ssim_forward", s);
+	const dim3 grid((a.W + kLossTileW - 1) / kLossTileW, (a.H + kLossTileH - 1) / kLossTileH, a.C);
+	hipLaunchKernelGGL(ssim_forward_kernel, grid, dim3(256), 0, s, a);
+	hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(256), 0, s, a, loss_blocks(a.C, a.H, a.W));
+}
+
+void launch_l1_ssim_backward(const LossArgs& a, hipStream_t s)
+{
+	stage_mark("l1_ssim_backward", s);
+	const dim3 grid((a.W + kLossTileW - 1) / kLossTileW, (a.H + kLossTileH - 1) / kLossTileH, a.C);
+	hipLaunchKernelGGL(ssim_backward_kernel, grid, dim3(256), 0, s, a);
+}
+
+uint32_t adam_blocks_for(size_t n)
+{
+	return (uint32_t)((n + kAdamBlock - 1) / kAdamBlock);
+}
+
+void launch_adam_step(const AdamArgs& a, uint32_t blocks, hipStream_t s)
+{
+	stage_mark("adam_step", s);
+	if (blocks)
+		hipLaunchKernelGGL(adam_step_kernel, dim3(blocks), dim3(256), 0, s, a);
+}
+
+}  // namespace rgs
