@@ -54,6 +54,10 @@ def parse():
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--streams", type=int, default=4,
                     help="render the submodels of a frame on this many HIP streams (0: all on the current stream)")
+    ap.add_argument("--instance-room", type=float, default=0.0,
+                    help="if > 0: room for (Gaussian, tile) instances as a multiple of the first frame's count; the "
+                         "forward then runs without a host round trip and the count is checked after each frame "
+                         "(0: wait for every count before sorting, as the reference does; measured as fast)")
     ap.add_argument("--host-threads", action="store_true",
                     help="issue each stream's forward calls from a host thread of its own")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -112,14 +116,30 @@ def main():
     streams = ([torch.cuda.current_stream(dev)] + [torch.cuda.Stream(device=dev) for _ in range(args.streams - 1)]
                if args.streams > 0 else None)
 
-    def step(streams=streams):
-        for s in subs:
-            for p in s.parameters():
-                p.grad = None
-        out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=args.host_threads)
-        if do_backward:
-            torch.autograd.backward([out["render"]], [upstream])
-        return out
+    bounds = None   # room for each submodel's instances; None: wait for every count
+
+    def step(streams=streams, host_threads=args.host_threads):
+        nonlocal bounds
+        while True:
+            for s in subs:
+                for p in s.parameters():
+                    p.grad = None
+            out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=host_threads,
+                                        instance_bounds=bounds)
+            if do_backward:
+                torch.autograd.backward([out["render"]], [upstream])
+            if bounds is None:
+                return out
+            try:   # the counts have long arrived by now; a frame that ran out of room is rendered again
+                pipeline.check_instance_bounds(out)
+                return out
+            except pipeline.InstanceBoundExceeded as ex:
+                bounds.update({m: int(c * args.instance_room) + 4096 for m, c in ex.needed.items()})
+
+    if args.instance_room > 0:
+        first = step(host_threads=False)   # waits for the counts, and so learns them
+        bounds = {m: int(c * args.instance_room) + 4096 for m, c in pipeline.check_instance_bounds(first).items()}
+        del first
 
     for _ in range(args.warmup):
         step()
@@ -260,7 +280,9 @@ def main():
                                f"({K} of {len(subs)} submodels related), SH degree 3, "
                                f"{'fwd+bwd' if do_backward else 'fwd only'}",
                    "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
-                   "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1)},
+                   "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1),
+                   "instance_room": (f"{args.instance_room} x the first frame's count, checked after every frame"
+                                     if bounds is not None else "sized from each call's count (host waits)")},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
         "blend_work": evals, "sharing": sharing, "loss_and_optimiser": after,
     }

@@ -145,6 +145,23 @@ int rgs_forward_raster(int P, int R, int width, int height,
                        void* image_ws, size_t image_bytes,
                        float* out_color, float* out_depth, float* out_alpha, void* stream, int debug);
 
+/* rgs_forward_raster for a caller that does not wait for the instance count: R_bound sizes the
+ * binning workspace (rgs_binning_bytes(R_bound)) and the launches, and the kernels take the
+ * count the geometry stage left on the device.  The host never learns R before launching, so
+ * a frame's forward needs no round trip; the price is a check afterwards: if the count that
+ * rgs_forward_geom_enqueue delivered exceeds R_bound, instances beyond it were dropped, the images
+ * are wrong and the call must be repeated with a larger bound (nothing is written out of bounds).
+ * rgs_backward is then given R_bound as its R.  The reference has no counterpart: it sizes its
+ * buffers after a blocking read of the count (rasterizer_impl.cu:287-292), through callbacks that
+ * grow them (K/rasterize_points.cu:27-33). */
+int rgs_forward_raster_bounded(int P, int R_bound, int width, int height,
+                       const float* background, float tan_fovx, float tan_fovy,
+                       const float* projmatrix_inv, const float* range_low, const float* range_up,
+                       const float* colors_precomp, const int* radii,
+                       void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                       void* image_ws, size_t image_bytes,
+                       float* out_color, float* out_depth, float* out_alpha, void* stream, int debug);
+
 /* grad_accum is scratch for the backward pass: RGS_ACC_FLOATS floats per Gaussian in which
  * the backward blend accumulates its per-Gaussian sums atomically (one 48-byte row per
  * Gaussian, so that the adds a wavefront issues for one Gaussian share a cache line).  The

@@ -68,6 +68,7 @@ def _load():
     lib.rgs_forward_geom_enqueue.argtypes = lib.rgs_forward_geom.argtypes[:-2] + [vp, vp, i]
     lib.rgs_forward_raster.argtypes = [i, i, i, i, vp, f, f, vp, vp, vp, vp, vp, vp, sz, vp, sz, vp, sz,
                                        vp, vp, vp, vp, i]
+    lib.rgs_forward_raster_bounded.argtypes = lib.rgs_forward_raster.argtypes
     lib.rgs_backward.argtypes = [i, i, i, i, i, i, vp, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, vp, vp, vp,
                                  f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, i]
     lib.rgs_inclusive_sum.argtypes = [vp, vp, sz, vp, vp]
@@ -88,7 +89,7 @@ def _load():
     lib.rgs_stage_timing_read.argtypes = [i, C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.POINTER(C.c_int)]
     lib.rgs_blend_work_counters.argtypes = [i, i, i, i, f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
-                 "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
+                 "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_forward_raster_bounded", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
                  "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
                  "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step"):
         getattr(lib, name).restype = i
@@ -99,7 +100,7 @@ lib = _load()
 
 EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_bytes", "rgs_binning_bytes",
            "rgs_image_bytes", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
-           "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
+           "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_forward_raster_bounded", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
            "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward",
            "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",
            "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward", "rgs_loss_workspace_bytes",

@@ -467,13 +467,19 @@ int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
 }
 
 
-int rgs_forward_raster(int P, int R, int width, int height,
-                       const float* background, float tan_fovx, float tan_fovy,
-                       const float* projmatrix_inv, const float* range_low, const float* range_up,
-                       const float* colors_precomp, const int* radii,
-                       void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
-                       void* image_ws, size_t image_bytes,
-                       float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
+}  // extern "C"
+
+namespace {
+
+// `R` sizes the binning workspace and the launches.  With count_on_device the number of instances
+// is the smaller of R and the count the geometry stage left in its workspace, read by the kernels.
+int forward_raster(bool count_on_device, int P, int R, int width, int height,
+                   const float* background, float tan_fovx, float tan_fovy,
+                   const float* projmatrix_inv, const float* range_low, const float* range_up,
+                   const float* colors_precomp, const int* radii,
+                   void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                   void* image_ws, size_t image_bytes,
+                   float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
@@ -503,15 +509,16 @@ int rgs_forward_raster(int P, int R, int width, int height,
 		uint32_t* vals_b = at<uint32_t>(binning_ws, b.vals_b);
 		const uint32_t* order_status =
 		    rgs::sort_status_word(at<uint32_t>(at<char>(geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).sort_temp));
+		const uint32_t* count = count_on_device ? at<uint32_t>(geom_ws, goff[RGS_GEOM_TOTAL]) : nullptr;
 		rgs::launch_duplicate_with_keys(P, at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]),
 		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_DEPTH_ORDER]),
 		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_POINT_OFFSETS]), at<float2>(geom_ws, goff[RGS_GEOM_XY]),
-		                                radii, gx, gy, keys_a, vals_a, at<uint32_t>(binning_ws, b.temp),
+		                                radii, gx, gy, keys_a, vals_a, (uint32_t)R, at<uint32_t>(binning_ws, b.temp),
 		                                rgs::sort_clear_words((size_t)R, tile_key_bits(width, height)), s);
 		RGS_STAGE("duplicate_with_keys");
 		const int end_bit = tile_key_bits(width, height);
 		// the first kernel of the sort also clears the tile ranges (and the counters behind them)
-		rgs::launch_sort_pairs_u32(keys_a, keys_b, vals_a, vals_b, (size_t)R, nullptr, end_bit, at<uint32_t>(binning_ws, b.temp),
+		rgs::launch_sort_pairs_u32(keys_a, keys_b, vals_a, vals_b, (size_t)R, count, end_bit, at<uint32_t>(binning_ws, b.temp),
 		                           true, reinterpret_cast<uint32_t*>(ranges), (size_t)gx * gy * 2 + rgs::kRangeTailWords,
 		                           "sort", s);
 		RGS_STAGE("sort_pairs");
@@ -526,12 +533,12 @@ int rgs_forward_raster(int P, int R, int width, int height,
 			if (e != hipSuccess || status != 0)
 				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
 		}
-		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, ranges, gx * gy,
+		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, count, ranges, gx * gy,
 		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, true, s);
 		RGS_STAGE("tile_ranges");
 		point_list = sorted_in_a ? vals_a : vals_b;
 	} else {
-		rgs::launch_tile_ranges(nullptr, 0, ranges, gx * gy, nullptr, nullptr, false, s);
+		rgs::launch_tile_ranges(nullptr, 0, nullptr, ranges, gx * gy, nullptr, nullptr, false, s);
 		RGS_STAGE("tile_ranges");
 	}
 
@@ -557,6 +564,36 @@ int rgs_forward_raster(int P, int R, int width, int height,
 	rgs::launch_blend_forward(a, s);
 	RGS_STAGE("blend_forward");
 	return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rgs_forward_raster(int P, int R, int width, int height,
+                       const float* background, float tan_fovx, float tan_fovy,
+                       const float* projmatrix_inv, const float* range_low, const float* range_up,
+                       const float* colors_precomp, const int* radii,
+                       void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                       void* image_ws, size_t image_bytes,
+                       float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
+{
+	return forward_raster(false, P, R, width, height, background, tan_fovx, tan_fovy, projmatrix_inv, range_low, range_up,
+	                      colors_precomp, radii, geom_ws, geom_bytes, binning_ws, binning_bytes, image_ws, image_bytes,
+	                      out_color, out_depth, out_alpha, stream, debug);
+}
+
+int rgs_forward_raster_bounded(int P, int R_bound, int width, int height,
+                               const float* background, float tan_fovx, float tan_fovy,
+                               const float* projmatrix_inv, const float* range_low, const float* range_up,
+                               const float* colors_precomp, const int* radii,
+                               void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                               void* image_ws, size_t image_bytes,
+                               float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
+{
+	return forward_raster(true, P, R_bound, width, height, background, tan_fovx, tan_fovy, projmatrix_inv, range_low,
+	                      range_up, colors_precomp, radii, geom_ws, geom_bytes, binning_ws, binning_bytes, image_ws,
+	                      image_bytes, out_color, out_depth, out_alpha, stream, debug);
 }
 
 int rgs_backward(int P, int D, int M, int R, int width, int height,

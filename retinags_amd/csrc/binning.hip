@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t
                                                                    const float2* __restrict__ xy,
                                                                    const int* __restrict__ radii, int gx, int gy,
                                                                    uint32_t* __restrict__ keys,
-                                                                   uint32_t* __restrict__ values,
+                                                                   uint32_t* __restrict__ values, uint32_t capacity,
                                                                    uint32_t* __restrict__ clear, size_t clear_words)
 {
 	__shared__ uint32_t s_end[4][64];     // inclusive offset of each of the wavefront's Gaussians
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t
 	const uint32_t run_end = s_end[wave][63];
 	for (uint32_t base = run_begin; base < run_end; base += 64) {
 		const uint32_t pos = base + (uint32_t)lane;
-		if (pos < run_end) {
+		if (pos < run_end && pos < capacity) {  // positions beyond the room the caller gave are dropped
 			// the first Gaussian whose inclusive offset exceeds pos
 			int lo = 0;
 #pragma unroll
@@ -266,12 +266,12 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
 
 void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
                                 const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
-                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t* clear, size_t clear_words,
-                                hipStream_t s)
+                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t capacity, uint32_t* clear,
+                                size_t clear_words, hipStream_t s)
 {
 	stage_mark("duplicate_with_keys", s);
 	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, visible_count, order,
-	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values, clear, clear_words);
+	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values, capacity, clear, clear_words);
 }
 
 // ---- radix sort -------------------------------------------------------------------------------
@@ -316,7 +316,7 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const KeyT* _
 	for (size_t w = (size_t)blockIdx.x * 256 + threadIdx.x; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;  // an array that a later kernel of the same stream wants cleared
 	if (n_device)
-		n = *n_device;
+		n = min(n, (size_t)*n_device);
 #pragma unroll
 	for (int p = 0; p < kSortMaxPasses; p++)
 		s_hist[p][threadIdx.x] = 0;
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restri
 	const uint32_t tile = s_tile;
 	const size_t block_base = (size_t)tile * kSortBlock;
 	if (n_device)
-		n = *n_device;
+		n = min(n, (size_t)*n_device);
 	// launched for an upper bound of n: tiles beyond the data leave, and no tile waits for them
 	if (block_base >= n)
 		return;
@@ -582,11 +582,14 @@ void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 // The status words (may be null) are those of the two sorts: if either reported a failure the
 // ranges stay empty, so no later stage walks an unsorted list.
 __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __restrict__ keys, size_t n,
+                                                           const uint32_t* __restrict__ n_device,
                                                            uint2* __restrict__ ranges,
                                                            const uint32_t* __restrict__ sort_status,
                                                            const uint32_t* __restrict__ order_status)
 {
 	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if (n_device)
+		n = min(n, (size_t)*n_device);  // launched for an upper bound
 	if (idx >= n)
 		return;
 	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u))
@@ -605,16 +608,16 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __rest
 		ranges[cur].y = (uint32_t)n;
 }
 
-void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
-                        const uint32_t* order_status, bool ranges_cleared, hipStream_t s)
+void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device, uint2* ranges, int tiles,
+                        const uint32_t* sort_status, const uint32_t* order_status, bool ranges_cleared, hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
 	if (!ranges_cleared)
 		launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2 + kRangeTailWords, s);
 	if (n == 0)
 		return;
-	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, ranges,
-	                   sort_status, order_status);
+	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, n_device,
+	                   ranges, sort_status, order_status);
 }
 
 }  // namespace rgs

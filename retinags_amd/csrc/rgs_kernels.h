@@ -249,11 +249,12 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
                         uint32_t* visible_count, uint32_t* visible_list, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
                         uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
                         hipStream_t s);
-// Also sets clear[0..clear_words) to zero (the scratch of the sort that follows).
+// Also sets clear[0..clear_words) to zero (the scratch of the sort that follows).  Instances whose
+// position is `capacity` or more are not written.
 void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
                                 const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
-                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t* clear, size_t clear_words,
-                                hipStream_t s);
+                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t capacity, uint32_t* clear,
+                                size_t clear_words, hipStream_t s);
 size_t sort_clear_words(size_t n, int end_bit);    // words of the sort scratch that must be zero before a sort
 size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs*
 // Stable LSD radix sort on key bits [0, end_bit), ceil(end_bit/8) passes that ping-pong between
@@ -262,7 +263,7 @@ size_t sort_temp_words(size_t n);                 // u32 words of scratch for la
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s);
 // The same for 32-bit keys; with a null `stage` its kernels are not marked for the timing aid.
-// With a non-null n_device the number of pairs is read from there by the kernels and `n` is only
+// With a non-null n_device the number of pairs is min(n, *n_device), read by the kernels, and `n` is only
 // its upper bound (grids and scratch are sized for it).
 // temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of temp already.
 // also_clear: an array the first kernel sets to zero on the way (for a later stage), or null.
@@ -274,8 +275,9 @@ const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a fai
 // the kRangeTailWords words behind it (the strip class counters of the blend).
 constexpr int kRangeTailWords = 512;
 // ranges_cleared: an earlier kernel has done that clearing.
-void launch_tile_ranges(const uint32_t* keys, size_t n, uint2* ranges, int tiles, const uint32_t* sort_status,
-                        const uint32_t* order_status, bool ranges_cleared, hipStream_t s);
+// With a non-null n_device the number of keys is min(n, *n_device) and the launch is sized for n.
+void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device, uint2* ranges, int tiles,
+                        const uint32_t* sort_status, const uint32_t* order_status, bool ranges_cleared, hipStream_t s);
 
 // blend.hip
 void launch_blend_forward(const BlendArgs& a, hipStream_t s);

@@ -116,13 +116,34 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
             "depth": depth, "alpha": alpha, "num_rendered": -1}
 
 
-def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0, debug: bool = False):
+def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0, debug: bool = False,
+                   instance_bound: Optional[int] = None):
     """Enqueues the geometry stage of a submodel's forward on the current stream without waiting
     for its instance count; hand the result to render_submodel(..., started=...)."""
     rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug))
     geometry = rasterizer.enqueue_geometry(means3D=sub.means3D, opacities=sub.opacity, shs=sub.shs,
-                                           scales=sub.scales, rotations=sub.rotations)
+                                           scales=sub.scales, rotations=sub.rotations, instance_bound=instance_bound)
     return rasterizer, geometry
+
+
+class InstanceBoundExceeded(RuntimeError):
+    """A submodel had more (Gaussian, tile) instances than the room its forward was given;
+    `needed` maps submodel id to the count."""
+
+    def __init__(self, needed: Dict[int, int]):
+        super().__init__(f"instance bounds exceeded: {needed}")
+        self.needed = needed
+
+
+def check_instance_bounds(frame: dict) -> Dict[int, int]:
+    """For a frame rendered with instance_bounds: the instance count of every submodel; raises
+    InstanceBoundExceeded if any forward ran out of room (its images are then wrong and the
+    frame must be rendered again with larger bounds)."""
+    counts = {m: st.instances() if st.P else 0 for m, st in frame.get("stages", {}).items()}
+    over = {m: c for m, c in counts.items() if not frame["stages"][m].within_bound()}
+    if over:
+        raise InstanceBoundExceeded(over)
+    return counts
 
 
 _pools = {}
@@ -137,7 +158,8 @@ def _host_pool(n: int):
 
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
                  submodel_bg: Optional[torch.Tensor] = None,
-                 streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = False) -> dict:
+                 streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = False,
+                 instance_bounds: Optional[Dict[int, int]] = None) -> dict:
     """Render every related submodel (black background, as the trainer does:
     trainer4tree_partition.py:397) and composite the partial images in BVH order.
 
@@ -151,13 +173,54 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     With host_threads each stream's forward calls are instead issued by a host thread of their
     own (ctypes releases the interpreter lock inside the library); measured no faster, and less
     steady, than the two rounds: the threads contend for the interpreter between the calls.
+
+    instance_bounds (submodel id -> room for that many instances; with or without `streams`): the
+    forward of each submodel is issued in one go, without waiting for its instance count.  The
+    stages come back under "stages"; call check_instance_bounds(frame) before using the frame's
+    results (after the backward has been issued is early enough).
     """
     device = subs[0].means3D.device
     if submodel_bg is None:
         submodel_bg = torch.zeros(3, device=device)
     related = [m for m in range(len(subs)) if relation[m] >= 0]
-    if not streams:
-        partial = {m: render_submodel(cam, subs[m], submodel_bg) for m in related}
+    stages = {}
+    if instance_bounds is not None:
+        main = torch.cuda.current_stream(device)
+        lanes = streams if streams else [main]
+        for side in lanes[:len(related)]:
+            if side is not main:
+                side.wait_stream(main)
+        partial = {}
+
+        def forward_in_one_go(k, m):
+            with torch.cuda.device(device), torch.cuda.stream(lanes[k % len(lanes)]):
+                started = start_submodel(cam, subs[m], submodel_bg, instance_bound=instance_bounds.get(m))
+                return m, started[1], render_submodel(cam, subs[m], submodel_bg, started=started)
+
+        if host_threads and len(lanes) > 1:
+            # nothing waits for the device here, so a host thread per stream spends its time inside
+            # the library's launches, where it does not hold the interpreter lock
+            def lane_work(j):
+                return [forward_in_one_go(k, m) for k, m in enumerate(related) if k % len(lanes) == j]
+            done = [r for rs in _host_pool(len(lanes)).map(lane_work, range(min(len(lanes), len(related)))) for r in rs]
+        else:
+            done = [forward_in_one_go(k, m) for k, m in enumerate(related)]
+        for m, stage, res in sorted(done, key=lambda d: related.index(d[0])):
+            stages[m] = stage
+            partial[m] = res
+        for side in lanes[:len(related)]:
+            if side is not main:
+                main.wait_stream(side)
+        for res in partial.values():
+            for t in res.values():
+                if torch.is_tensor(t) and t.is_cuda:
+                    t.record_stream(main)
+    elif not streams:
+        partial = {}
+        for m in related:
+            started = start_submodel(cam, subs[m], submodel_bg)
+            stages[m] = started[1]
+            partial[m] = render_submodel(cam, subs[m], submodel_bg, started=started)
     else:
         main = torch.cuda.current_stream(device)
         for side in streams[:len(related)]:
@@ -183,6 +246,7 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
             for k, m in enumerate(related):
                 with torch.cuda.stream(streams[k % len(streams)]):
                     partial[m] = render_submodel(cam, subs[m], submodel_bg, started=started[m])
+                    stages[m] = started[m][1]
         for side in streams[:len(related)]:
             main.wait_stream(side)
         for res in partial.values():
@@ -191,4 +255,5 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
                     t.record_stream(main)
     out = blender_render_result(partial, relation, background)
     out["partial"] = partial
+    out["stages"] = stages
     return out

@@ -79,11 +79,31 @@ class GeometryStage:
     GaussianRasterizer.enqueue_geometry, consumed once by GaussianRasterizer.forward."""
 
     __slots__ = ("device", "stream", "P", "H", "W", "tensors", "settings", "radii", "geomBuffer", "geom_bytes",
-                 "count", "event", "source", "used")
+                 "count", "event", "source", "used", "instance_bound", "_instances")
 
     def matches(self, means3D, raster_settings) -> bool:
         return (self.source == (means3D.data_ptr(), int(means3D.shape[0])) and self.settings is raster_settings
                 and not self.used)
+
+    def instances(self) -> int:
+        """The number of (Gaussian, tile) instances of this call; waits for it if it is still on
+        its way.  A stage that was given an instance_bound must be asked once its forward has
+        been issued: a count above the bound means the images of that forward are wrong."""
+        if self._instances is None:
+            if self.count is None:
+                raise RuntimeError("the instance count of this stage has been handed on already")
+            if self.event is not None:
+                self.event.synchronize()
+                self._instances = int(self.count.item())
+                _free_count_slots[(self.device.type, self.device.index)].append((self.count, self.event))
+                self.event = None
+            else:
+                self._instances = int(self.count.item())
+            self.count = None
+        return self._instances
+
+    def within_bound(self) -> bool:
+        return self.instance_bound is None or self.P == 0 or self.instances() <= self.instance_bound
 
 
 _EMPTY = torch.Tensor([])  # stands for an absent input, as in the reference (it becomes a null pointer)
@@ -119,6 +139,8 @@ def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations,
     st.settings = None
     st.event = None
     st.count = None
+    st.instance_bound = None
+    st._instances = None
     byte = dict(dtype=torch.uint8, device=device)
     st.radii = torch.empty((st.P,), dtype=torch.int32, device=device)
     names = ("means3D", "colors_precomp", "opacities", "scales", "rotations", "cov3Ds_precomp", "sh", "bg",
@@ -175,19 +197,16 @@ def _forward_blend(st: GeometryStage):
     with torch.cuda.device(device):
         image_bytes = lib.rgs_image_bytes(W, H)
         imgBuffer = torch.empty(image_bytes, **byte)
-        if st.event is not None:
-            st.event.synchronize()
-            rendered = int(st.count.item())
-            _free_count_slots[(device.type, device.index)].append((st.count, st.event))
-            st.event = None
+        if st.instance_bound is not None:
+            # no wait: the kernels read the count on the device; the caller checks it afterwards
+            rendered, raster = int(st.instance_bound), lib.rgs_forward_raster_bounded
         else:
-            rendered = int(st.count.item())
-        st.count = None
+            rendered, raster = st.instances(), lib.rgs_forward_raster
         if rendered >= 1 << 30:
             raise _capi.RgsError(f"{rendered} (Gaussian, tile) instances exceed the 2^30 limit of the sort")
         binning_bytes = lib.rgs_binning_bytes(rendered) if rendered > 0 else 0
         binningBuffer = torch.empty(binning_bytes, **byte)
-        check(lib.rgs_forward_raster(
+        check(raster(
             P, rendered, W, H, ptr(t["bg"]), t["tanfovx"], t["tanfovy"], ptr(t["projmatrix_inv"]),
             ptr(t["range_low"]), ptr(t["range_up"]), ptr(t["colors_precomp"]), ptr(st.radii), ptr(st.geomBuffer),
             st.geom_bytes, ptr(binningBuffer), binning_bytes, ptr(imgBuffer), image_bytes, ptr(out_color),
@@ -451,13 +470,19 @@ class GaussianRasterizer(nn.Module):
                                    raster_settings, geometry)
 
     def enqueue_geometry(self, means3D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
-                         cov3D_precomp=None) -> GeometryStage:
+                         cov3D_precomp=None, instance_bound=None) -> GeometryStage:
         """Starts the first half of a forward call (preprocess and instance count) on the current
         stream and returns without waiting for it.  No counterpart in the reference, whose forward
         always blocks on the count (K/cuda_rasterizer_hgs/rasterizer_impl.cu:287): a caller that
         renders several submodels on separate streams enqueues every geometry stage first and
         then calls forward(..., geometry=stage) for each, on the stream the stage was enqueued
-        on, so that the host's wait for one count no longer holds back the other submodels."""
+        on, so that the host's wait for one count no longer holds back the other submodels.
+
+        instance_bound: room for that many (Gaussian, tile) instances is set aside and the forward
+        does not wait for the count at all (the reference grows its buffers on demand instead,
+        K/rasterize_points.cu:27-33).  The caller must then ask stage.within_bound() after the
+        forward has been issued (at the end of the iteration is early enough) and, if it is
+        false, repeat the forward with a bound of at least stage.instances()."""
         rs = self.raster_settings
         shs, colors_precomp, scales, rotations, cov3D_precomp = self._check_and_fill(
             shs, colors_precomp, scales, rotations, cov3D_precomp)
@@ -467,4 +492,8 @@ class GaussianRasterizer(nn.Module):
                 rs.viewmatrix, rs.projmatrix, rs.projmatrix_inv, rs.range_low, rs.range_up, rs.tanfovx, rs.tanfovy,
                 rs.image_height, rs.image_width, shs, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, wait=False)
         stage.settings = rs
+        if instance_bound is not None:
+            if int(instance_bound) < 0:
+                raise ValueError("instance_bound must not be negative")
+            stage.instance_bound = int(instance_bound)
         return stage

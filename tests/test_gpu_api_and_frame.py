@@ -240,6 +240,80 @@ def test_enqueued_geometry_stage_gives_the_same_forward_and_is_checked():
     torch.cuda.synchronize()
 
 
+def test_forward_with_an_instance_bound_needs_no_count_and_reports_overflow():
+    """enqueue_geometry(instance_bound=N) + forward: no wait for the instance count.  With room
+    enough the outputs and gradients are those of the ordinary call, bit for bit (gradients up to
+    the order of the atomic adds); with too little room the stage says so, nothing faults, and a
+    repeat with the count it reports is right again."""
+    from retinags_amd import GaussianRasterizer
+    scene, cam, low, up = _small_inputs(n=6000, seed=21)
+    r = GaussianRasterizer(_settings(oracle_settings(cam, low, up, torch.tensor([0.3, 0.2, 0.1]))))
+    leaves = {k: scene[n].to(DEV).requires_grad_(True) for k, n in
+              (("means3D", "xyz"), ("opacities", "opacity"), ("shs", "shs"), ("scales", "scales"), ("rotations", "rotations"))}
+    weight = torch.randn(3, cam.image_height, cam.image_width, generator=torch.Generator().manual_seed(4)).to(DEV)
+
+    def run(bound):
+        for t in leaves.values():
+            t.grad = None
+        stage = r.enqueue_geometry(instance_bound=bound, **leaves) if bound != "wait" else r.enqueue_geometry(**leaves)
+        out = r(means2D=torch.zeros_like(leaves["means3D"]), geometry=stage, **leaves)
+        (out[0] * weight).sum().backward()
+        torch.cuda.synchronize()
+        return stage, [o.detach().clone() for o in out], [t.grad.clone() for t in leaves.values()]
+
+    stage, ref_out, ref_grads = run("wait")
+    R = stage.instances()
+    assert R > 1000 and stage.within_bound()
+    for bound in (R, R + 1, 3 * R + 12345):
+        st, out, grads = run(bound)
+        assert st.within_bound() and st.instances() == R
+        assert all(torch.equal(a, b) for a, b in zip(ref_out, out))
+        assert all(rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-5 for a, b in zip(ref_grads, grads))
+    for bound in (R - 1, R // 2, 1, 0):
+        st, out, grads = run(bound)
+        assert not st.within_bound() and st.instances() == R
+        assert all(torch.isfinite(o.float()).all() for o in out) and all(torch.isfinite(g).all() for g in grads)
+    st, out, grads = run(stage.instances())
+    assert all(torch.equal(a, b) for a, b in zip(ref_out, out))
+
+
+def test_frame_with_instance_bounds_matches_the_waiting_frame():
+    from retinags_amd.harness import partition, pipeline
+    scene, cam, _ = scenes.make_config("C1", shrink=40, resolution_scale=0.5)
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    rel = partition.relation_vector(part, cam)
+    subs = [s.requires_grad_(True) for s in pipeline.submodels_from_partition(scene, part, DEV)]
+    up = (torch.randn(3, cam.image_height, cam.image_width, generator=torch.Generator().manual_seed(5)) * 1e-2).to(DEV)
+    bg = torch.tensor([0.2, 0.3, 0.4], device=DEV)
+    cam_d = cam.to(DEV)
+    streams = [torch.cuda.current_stream(DEV)] + [torch.cuda.Stream(device=DEV) for _ in range(3)]
+
+    def frame(bounds, lanes):
+        for s in subs:
+            for p in s.parameters():
+                p.grad = None
+        out = pipeline.render_frame(cam_d, subs, rel, bg, streams=lanes, instance_bounds=bounds)
+        torch.autograd.backward([out["render"]], [up])
+        counts = pipeline.check_instance_bounds(out)
+        torch.cuda.synchronize()
+        return out["render"].detach().clone(), counts, [[p.grad.clone() for p in s.parameters()] for s in subs]
+
+    ref_img, counts, ref_grads = frame(None, streams)
+    assert len(counts) >= 2 and min(counts.values()) > 0
+    for lanes in (streams, None):
+        img, again, grads = frame({m: c + 100 for m, c in counts.items()}, lanes)
+        assert again == counts and torch.equal(img, ref_img)
+        for ga, gb in zip(ref_grads, grads):
+            assert all(rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-4 for a, b in zip(ga, gb))
+    tight = dict(counts)
+    worst = max(counts, key=counts.get)
+    tight[worst] = counts[worst] // 3
+    with pytest.raises(pipeline.InstanceBoundExceeded) as info:
+        frame(tight, streams)
+    assert info.value.needed == {worst: counts[worst]}
+    torch.cuda.synchronize()
+
+
 def test_backward_clears_the_gradients_itself_when_the_caller_has_not():
     """The first backward of a forward call uses gradient tensors cleared during the forward;
     a second one over the retained graph has none and lets the library clear them.  Both give
