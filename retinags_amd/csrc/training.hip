@@ -27,6 +27,9 @@ namespace {
 constexpr int kLossTileW = 32, kLossTileH = 16;
 constexpr int kHalo = 5, kTaps = 11;
 constexpr int kRegionW = kLossTileW + 2 * kHalo, kRegionH = kLossTileH + 2 * kHalo;
+constexpr int kRowRun = 4;   // columns a thread takes in the row pass (26 x 8 runs for 256 threads)
+constexpr int kColRun = 2;   // rows a thread takes in the column pass (8 x 32 runs)
+static_assert(kRegionH * (kLossTileW / kRowRun) <= 256 && (kLossTileH / kColRun) * kLossTileW == 256, "pass shapes");
 
 __device__ __forceinline__ float block256_sum(float v, float* lds)
 {
@@ -40,6 +43,31 @@ __device__ __forceinline__ float block256_sum(float v, float* lds)
 	return total;
 }
 
+// Workgroups are dealt to the 8 XCDs in turn, and each XCD has its own L2.  Workgroup b therefore
+// takes tile (b % 8) * ceil(tiles / 8) + b / 8 of the row-major (channel, tile row, tile column)
+// order: an XCD gets a contiguous band of tiles, and the halo a tile shares with its neighbours is
+// fetched from memory once per band instead of once per tile.
+struct LossTile {
+	int channel, tx, ty;
+	uint32_t linear;
+	bool valid;
+};
+
+__device__ __forceinline__ LossTile loss_tile_of_block(const LossArgs& a)
+{
+	const uint32_t tiles_x = (a.W + kLossTileW - 1) / kLossTileW, tiles_y = (a.H + kLossTileH - 1) / kLossTileH;
+	const uint32_t total = tiles_x * tiles_y * (uint32_t)a.C;
+	const uint32_t per_xcd = (total + 7) / 8;
+	LossTile t;
+	t.linear = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+	t.valid = blockIdx.x / 8 < per_xcd && t.linear < total;
+	const uint32_t in_plane = t.linear % (tiles_x * tiles_y);
+	t.channel = (int)(t.linear / (tiles_x * tiles_y));
+	t.ty = (int)(in_plane / tiles_x);
+	t.tx = (int)(in_plane % tiles_x);
+	return t;
+}
+
 __global__ __launch_bounds__(256) void ssim_forward_kernel(LossArgs a)
 {
 	__shared__ float sx[kRegionH][kRegionW + 1];
@@ -47,8 +75,11 @@ __global__ __launch_bounds__(256) void ssim_forward_kernel(LossArgs a)
 	__shared__ float rows[5][kRegionH][kLossTileW + 1];
 	__shared__ float red[4];
 	const int tid = threadIdx.x;
-	const size_t plane = (size_t)blockIdx.z * a.H * a.W;
-	const int x0 = blockIdx.x * kLossTileW - kHalo, y0 = blockIdx.y * kLossTileH - kHalo;
+	const LossTile tile = loss_tile_of_block(a);
+	if (!tile.valid)
+		return;
+	const size_t plane = (size_t)tile.channel * a.H * a.W;
+	const int x0 = tile.tx * kLossTileW - kHalo, y0 = tile.ty * kLossTileH - kHalo;
 	for (int i = tid; i < kRegionH * kRegionW; i += 256) {
 		const int r = i / kRegionW, c = i % kRegionW;
 		const int gx = x0 + c, gy = y0 + r;
@@ -58,24 +89,45 @@ __global__ __launch_bounds__(256) void ssim_forward_kernel(LossArgs a)
 		sy[r][c] = inside ? a.y[at] : 0.f;
 	}
 	__syncthreads();
-	for (int i = tid; i < kRegionH * kLossTileW; i += 256) {
-		const int r = i / kLossTileW, c = i % kLossTileW;
-		float m1 = 0.f, m2 = 0.f, xx = 0.f, yy = 0.f, xy = 0.f;
+	// row pass: a thread takes 4 neighbouring columns of one row, so 14 pixels of each image
+	// feed 4 x 5 sums (28 LDS reads instead of 88)
+	if (tid < kRegionH * (kLossTileW / kRowRun)) {
+		const int r = tid / (kLossTileW / kRowRun), c0 = kRowRun * (tid % (kLossTileW / kRowRun));
+		float u[kTaps + kRowRun - 1], v[kTaps + kRowRun - 1];
 #pragma unroll
-		for (int k = 0; k < kTaps; k++) {
-			const float w = a.w[k], u = sx[r][c + k], v = sy[r][c + k];
-			m1 += w * u;
-			m2 += w * v;
-			xx += w * (u * u);
-			yy += w * (v * v);
-			xy += w * (u * v);
+		for (int k = 0; k < kTaps + kRowRun - 1; k++) {
+			u[k] = sx[r][c0 + k];
+			v[k] = sy[r][c0 + k];
 		}
-		rows[0][r][c] = m1; rows[1][r][c] = m2; rows[2][r][c] = xx; rows[3][r][c] = yy; rows[4][r][c] = xy;
+#pragma unroll
+		for (int o = 0; o < kRowRun; o++) {
+			float m1 = 0.f, m2 = 0.f, xx = 0.f, yy = 0.f, xy = 0.f;
+#pragma unroll
+			for (int k = 0; k < kTaps; k++) {
+				const float w = a.w[k];
+				m1 += w * u[o + k];
+				m2 += w * v[o + k];
+				xx += w * (u[o + k] * u[o + k]);
+				yy += w * (v[o + k] * v[o + k]);
+				xy += w * (u[o + k] * v[o + k]);
+			}
+			rows[0][r][c0 + o] = m1; rows[1][r][c0 + o] = m2; rows[2][r][c0 + o] = xx; rows[3][r][c0 + o] = yy;
+			rows[4][r][c0 + o] = xy;
+		}
 	}
 	__syncthreads();
 	float ssim_sum = 0.f, l1_sum = 0.f;
-	for (int i = tid; i < kLossTileH * kLossTileW; i += 256) {
-		const int r = i / kLossTileW, c = i % kLossTileW;
+	// column pass: a thread takes kColRun rows of one column
+	float part[5][kTaps + kColRun - 1];
+	const int col = tid % kLossTileW, row0 = kColRun * (tid / kLossTileW);
+#pragma unroll
+	for (int q = 0; q < 5; q++)
+#pragma unroll
+		for (int k = 0; k < kTaps + kColRun - 1; k++)
+			part[q][k] = rows[q][row0 + k][col];
+#pragma unroll
+	for (int o = 0; o < kColRun; o++) {
+		const int r = row0 + o, c = col;
 		const int gx = x0 + kHalo + c, gy = y0 + kHalo + r;
 		if (gx >= a.W || gy >= a.H)
 			continue;
@@ -83,11 +135,11 @@ __global__ __launch_bounds__(256) void ssim_forward_kernel(LossArgs a)
 #pragma unroll
 		for (int k = 0; k < kTaps; k++) {
 			const float w = a.w[k];
-			m1 += w * rows[0][r + k][c];
-			m2 += w * rows[1][r + k][c];
-			xx += w * rows[2][r + k][c];
-			yy += w * rows[3][r + k][c];
-			xy += w * rows[4][r + k][c];
+			m1 += w * part[0][o + k];
+			m2 += w * part[1][o + k];
+			xx += w * part[2][o + k];
+			yy += w * part[3][o + k];
+			xy += w * part[4][o + k];
 		}
 		const float C1 = 0.01f * 0.01f, C2 = 0.03f * 0.03f;
 		const float m11 = m1 * m1, m22 = m2 * m2, m12 = m1 * m2;
@@ -108,9 +160,8 @@ __global__ __launch_bounds__(256) void ssim_forward_kernel(LossArgs a)
 	ssim_sum = block256_sum(ssim_sum, red);
 	l1_sum = block256_sum(l1_sum, red);
 	if (tid == 0) {
-		const size_t block = ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-		a.partial[2 * block] = ssim_sum;
-		a.partial[2 * block + 1] = l1_sum;
+		a.partial[2 * (size_t)tile.linear] = ssim_sum;
+		a.partial[2 * (size_t)tile.linear + 1] = l1_sum;
 	}
 }
 
@@ -148,8 +199,11 @@ __global__ __launch_bounds__(256) void ssim_backward_kernel(LossArgs a)
 	__shared__ float rows[3][kRegionH][kLossTileW + 1];
 	const int tid = threadIdx.x;
 	const size_t n = (size_t)a.C * a.H * a.W;
-	const size_t plane = (size_t)blockIdx.z * a.H * a.W;
-	const int x0 = blockIdx.x * kLossTileW - kHalo, y0 = blockIdx.y * kLossTileH - kHalo;
+	const LossTile tile = loss_tile_of_block(a);
+	if (!tile.valid)
+		return;
+	const size_t plane = (size_t)tile.channel * a.H * a.W;
+	const int x0 = tile.tx * kLossTileW - kHalo, y0 = tile.ty * kLossTileH - kHalo;
 	for (int i = tid; i < kRegionH * kRegionW; i += 256) {
 		const int r = i / kRegionW, c = i % kRegionW;
 		const int gx = x0 + c, gy = y0 + r;
@@ -160,23 +214,37 @@ __global__ __launch_bounds__(256) void ssim_backward_kernel(LossArgs a)
 		sm[2][r][c] = inside ? a.maps[2 * n + at] : 0.f;
 	}
 	__syncthreads();
-	for (int i = tid; i < kRegionH * kLossTileW; i += 256) {
-		const int r = i / kLossTileW, c = i % kLossTileW;
-		float pa = 0.f, pb = 0.f, pc = 0.f;
+	if (tid < kRegionH * (kLossTileW / kRowRun)) {
+		const int r = tid / (kLossTileW / kRowRun), c0 = kRowRun * (tid % (kLossTileW / kRowRun));
 #pragma unroll
-		for (int k = 0; k < kTaps; k++) {
-			const float w = a.w[k];
-			pa += w * sm[0][r][c + k];
-			pb += w * sm[1][r][c + k];
-			pc += w * sm[2][r][c + k];
+		for (int q = 0; q < 3; q++) {
+			float u[kTaps + kRowRun - 1];
+#pragma unroll
+			for (int k = 0; k < kTaps + kRowRun - 1; k++)
+				u[k] = sm[q][r][c0 + k];
+#pragma unroll
+			for (int o = 0; o < kRowRun; o++) {
+				float acc = 0.f;
+#pragma unroll
+				for (int k = 0; k < kTaps; k++)
+					acc += a.w[k] * u[o + k];
+				rows[q][r][c0 + o] = acc;
+			}
 		}
-		rows[0][r][c] = pa; rows[1][r][c] = pb; rows[2][r][c] = pc;
 	}
 	__syncthreads();
 	const float upstream = a.grad_loss ? a.grad_loss[0] : 1.0f;
 	const float l1_scale = upstream * (1.0f - a.lambda) / (float)n, ssim_scale = -upstream * a.lambda / (float)n;
-	for (int i = tid; i < kLossTileH * kLossTileW; i += 256) {
-		const int r = i / kLossTileW, c = i % kLossTileW;
+	float part[3][kTaps + kColRun - 1];
+	const int col = tid % kLossTileW, row0 = kColRun * (tid / kLossTileW);
+#pragma unroll
+	for (int q = 0; q < 3; q++)
+#pragma unroll
+		for (int k = 0; k < kTaps + kColRun - 1; k++)
+			part[q][k] = rows[q][row0 + k][col];
+#pragma unroll
+	for (int o = 0; o < kColRun; o++) {
+		const int r = row0 + o, c = col;
 		const int gx = x0 + kHalo + c, gy = y0 + kHalo + r;
 		if (gx >= a.W || gy >= a.H)
 			continue;
@@ -184,9 +252,9 @@ __global__ __launch_bounds__(256) void ssim_backward_kernel(LossArgs a)
 #pragma unroll
 		for (int k = 0; k < kTaps; k++) {
 			const float w = a.w[k];
-			ca += w * rows[0][r + k][c];
-			cb += w * rows[1][r + k][c];
-			cc += w * rows[2][r + k][c];
+			ca += w * part[0][o + k];
+			cb += w * part[1][o + k];
+			cc += w * part[2][o + k];
 		}
 		const size_t at = plane + (size_t)gy * a.W + gx;
 		const float x = a.x[at], y = a.y[at];
@@ -257,16 +325,16 @@ uint32_t loss_blocks(int C, int H, int W)
 void launch_l1_ssim_forward(const LossArgs& a, hipStream_t s)
 {
 	stage_mark("l1_ssim_forward", s);
-	const dim3 grid((a.W + kLossTileW - 1) / kLossTileW, (a.H + kLossTileH - 1) / kLossTileH, a.C);
-	hipLaunchKernelGGL(ssim_forward_kernel, grid, dim3(256), 0, s, a);
+	const uint32_t grid = 8 * ((loss_blocks(a.C, a.H, a.W) + 7) / 8);
+	hipLaunchKernelGGL(ssim_forward_kernel, dim3(grid), dim3(256), 0, s, a);
 	hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(256), 0, s, a, loss_blocks(a.C, a.H, a.W));
 }
 
 void launch_l1_ssim_backward(const LossArgs& a, hipStream_t s)
 {
 	stage_mark("l1_ssim_backward", s);
-	const dim3 grid((a.W + kLossTileW - 1) / kLossTileW, (a.H + kLossTileH - 1) / kLossTileH, a.C);
-	hipLaunchKernelGGL(ssim_backward_kernel, grid, dim3(256), 0, s, a);
+	const uint32_t grid = 8 * ((loss_blocks(a.C, a.H, a.W) + 7) / 8);
+	hipLaunchKernelGGL(ssim_backward_kernel, dim3(grid), dim3(256), 0, s, a);
 }
 
 uint32_t adam_blocks_for(size_t n)
