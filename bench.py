@@ -36,9 +36,9 @@ FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
 # cannot be read from inside the process, so the figures are carried here; other workloads
 # report null.
 C1_TRAFFIC_MB_PER_LAUNCH = {
-    "preprocess_forward": 253.68, "duplicate_with_keys": 108.30, "sort_onesweep": 23.08, "tile_ranges": 13.22,
-    "blend_forward": 237.65, "composite_forward": 165.79, "composite_backward": 372.11, "blend_backward": 308.29,
-    "preprocess_backward": 370.17,
+    "preprocess_forward": 254.10, "duplicate_with_keys": 108.31, "sort_onesweep": 23.11, "tile_ranges": 13.22,
+    "blend_forward": 237.40, "composite_forward": 165.79, "composite_backward": 372.03, "blend_backward": 284.80,
+    "preprocess_backward": 370.26,
 }
 
 
