@@ -326,6 +326,9 @@ def sharing_stages(scene, part, dev, repeats, append):
     wall_ms = (time.perf_counter() - t0) * 1e3 / repeats
     ms = _capi.stage_timing_read()
     _capi.stage_timing(False)
+    torch_ms = None
+    if append:   # measured once, beside the appending variant
+        torch_ms = _timed_ms(lambda: _sharing_by_tensor_expressions(models, part.box_low, part.box_up, dev), repeats)
     owned = float(sum(table.own))
     lent = float(table.counts.sum())
     merged_rows = owned + lent
@@ -334,6 +337,10 @@ def sharing_stages(scene, part, dev, repeats, append):
            "merge_rows_backward": (248.0 + 2 * 248.0 + 4.0) * lent}
     out = {"owned_gaussians": int(owned), "lent_rows": int(lent), "submodels": K, "wall_ms_per_pass": round(wall_ms, 3),
            "own_rows": "in place, lent rows appended behind them" if append else "copied into the merged arrays"}
+    if torch_ms is not None:
+        # the same selection, merge and backward written as the reference writes them: boolean-mask
+        # indexing per (source, destination) pair and torch.cat per field, differentiated by autograd
+        out["tensor_expression_wall_ms_per_pass"] = round(torch_ms, 3)
     for name, (total, launches) in ms.items():
         per = total / repeats
         out[name] = {"ms_per_pass": round(per, 4), "launches_per_pass": launches / repeats,
@@ -341,6 +348,57 @@ def sharing_stages(scene, part, dev, repeats, append):
         if out[name]["achieved_GBps"] is not None:
             out[name]["frac"] = round(out[name]["achieved_GBps"] / HBM_PEAK_GBS, 4)
     return out
+
+
+def _timed_ms(fn, repeats):
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / repeats
+
+
+def _sharing_by_tensor_expressions(models, box_low, box_up, dev):
+    """What the kernels of the sharing stage replace, as stock tensor operations on the same GPU
+    (for the timing beside them only; the checker of the tests is elsewhere)."""
+    K = len(models)
+    low = [torch.tensor(box_low[k], device=dev) for k in range(K)]
+    up = [torch.tensor(box_up[k], device=dev) for k in range(K)]
+    parts = [[m.fields()] for m in models]           # own rows first
+    for s_id, m in enumerate(models):
+        reach = (m.scales.max(dim=-1, keepdim=True).values * 3).clamp(min=0)
+        hi, lo = m.means3D + reach, m.means3D - reach
+        cand = ((hi >= up[s_id]) | (lo <= low[s_id])).any(dim=-1)
+        cand_fields = [f[cand] for f in m.fields()]
+        hi_c, lo_c = hi[cand], lo[cand]
+        for d_id in range(K):
+            if d_id == s_id:
+                continue
+            meets = ((hi_c >= low[d_id]) & (lo_c <= up[d_id])).all(dim=-1)
+            parts[d_id].append([f[meets] for f in cand_fields])
+    merged = [[torch.cat([p[f] for p in parts[d_id]], dim=0) for f in range(6)] for d_id in range(K)]
+    outs = [t for m in merged for t in m]
+    torch.autograd.backward(outs, [torch.ones_like(t) for t in outs])
+    for m in models:
+        for t in m.fields():
+            t.grad = None
+
+
+def _loss_by_tensor_expressions(image, gt, lambda_dssim):
+    """L1 + SSIM as 11x11 grouped convolutions and elementwise operations, with autograd."""
+    import torch.nn.functional as F
+    g = torch.tensor([np.exp(-(x - 5) ** 2 / (2 * 1.5 ** 2)) for x in range(11)], dtype=torch.float32, device=image.device)
+    g = (g / g.sum()).unsqueeze(1)
+    window = (g @ g.t()).expand(3, 1, 11, 11).contiguous()
+    blur = lambda t: F.conv2d(t.unsqueeze(0), window, padding=5, groups=3)
+    mu1, mu2 = blur(image), blur(gt)
+    s11, s22, s12 = blur(image * image) - mu1 * mu1, blur(gt * gt) - mu2 * mu2, blur(image * gt) - mu1 * mu2
+    ssim = (((2 * mu1 * mu2 + 1e-4) * (2 * s12 + 9e-4)) / ((mu1 * mu1 + mu2 * mu2 + 1e-4) * (s11 + s22 + 9e-4))).mean()
+    loss = (1 - lambda_dssim) * (image - gt).abs().mean() + lambda_dssim * (1 - ssim)
+    loss.backward()
+    image.grad = None
 
 
 def training_stages(subs, H, W, dev, repeats):
@@ -381,9 +439,23 @@ def training_stages(subs, H, W, dev, repeats):
         once()
     ms = _capi.stage_timing_read()
     _capi.stage_timing(False)
+    loss_torch_ms = _timed_ms(lambda: _loss_by_tensor_expressions(image, gt, 0.2), repeats)
+
+    def loss_once():
+        loss, _ = l1_ssim_loss(image, gt, 0.2)
+        loss.backward()
+        image.grad = None
+    loss_ms = _timed_ms(loss_once, repeats)
+    adam_ms = _timed_ms(lambda: [o.step() for o in optimisers], repeats)
+    stock = [torch.optim.Adam(o.param_groups, lr=0.0, eps=1e-15) for o in optimisers]
+    adam_torch_ms = _timed_ms(lambda: [o.step() for o in stock], repeats)
     pixels = 3.0 * H * W
     alg = {"l1_ssim_forward": 20.0 * pixels, "l1_ssim_backward": 24.0 * pixels, "adam_step": 28.0 * floats}
-    out = {"image": f"3x{H}x{W}", "adam_floats": floats}
+    out = {"image": f"3x{H}x{W}", "adam_floats": floats,
+           # wall clock per pass, host included, beside the same step written with stock tensor operations
+           # (conv2d expression + autograd; torch.optim.Adam) on the same GPU
+           "loss_fwd_bwd_wall_ms": round(loss_ms, 3), "loss_tensor_expression_wall_ms": round(loss_torch_ms, 3),
+           "adam_wall_ms": round(adam_ms, 3), "adam_torch_optim_wall_ms": round(adam_torch_ms, 3)}
     for name, (total, launches) in ms.items():
         per = total / repeats
         out[name] = {"ms_per_pass": round(per, 4), "launches_per_pass": launches / repeats}

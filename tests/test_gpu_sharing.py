@@ -65,6 +65,45 @@ def test_truncated_lists_are_redone_with_room():
         assert torch.equal(rows, tight.rows[key])
 
 
+def test_one_submodel_empty_submodel_and_distant_boxes():
+    """Nothing to lend: a single submodel, a submodel without Gaussians, boxes that are far apart."""
+    from retinags_amd import sharing
+    g = torch.Generator().manual_seed(2)
+
+    def model(n, centre):
+        xyz = (torch.rand(n, 3, generator=g) - 0.5 + torch.tensor(centre)).to(DEV)
+        return sharing.SharedGSInfo(xyz, torch.zeros_like(xyz), torch.rand(n, 1, generator=g).to(DEV),
+                                    (torch.rand(n, 3, generator=g) * 0.01).to(DEV), torch.randn(n, 4, generator=g).to(DEV),
+                                    torch.randn(n, 16, 3, generator=g).to(DEV))
+
+    one = [model(500, (0.0, 0.0, 0.0))]
+    table = sharing.select_straddlers(one, [[-1, -1, -1]], [[1, 1, 1]])
+    assert table.counts.tolist() == [[0]] and not table.rows
+    merged = sharing.merge_shared(one, table)
+    assert all(torch.equal(a, b) for a, b in zip(merged[0].fields(), one[0].fields()))
+
+    models = [model(300, (0.0, 0.0, 0.0)), model(0, (10.0, 0.0, 0.0)), model(200, (20.0, 0.0, 0.0))]
+    low = [[-1, -1, -1], [9, -1, -1], [19, -1, -1]]
+    up = [[1, 1, 1], [11, 1, 1], [21, 1, 1]]
+    table = sharing.select_straddlers(models, low, up)
+    assert int(table.counts.sum()) == 0
+    for m in models:
+        for t in m.fields():
+            t.requires_grad_(True)
+    merged = sharing.merge_shared(models, table)
+    assert [len(m) for m in merged] == [300, 0, 200]
+    torch.autograd.backward([merged[0].shs, merged[2].means3D], [torch.ones_like(merged[0].shs), torch.ones_like(merged[2].means3D)])
+    assert float(models[0].shs.grad.min()) == 1.0 and float(models[2].means3D.grad.min()) == 1.0
+    assert models[1].shs.grad is None or models[1].shs.grad.numel() == 0
+    # a Gaussian of submodel 0 that reaches into submodel 2's box is lent to it and to nobody else
+    with torch.no_grad():
+        models[0].scales[7] = 7.0
+    table = sharing.select_straddlers(models, low, up)
+    assert table.counts.tolist() == [[0, 1, 1], [0, 0, 0], [0, 0, 0]]
+    assert table.rows[(0, 2)].tolist() == [7] and table.rows[(0, 1)].tolist() == [7]
+    torch.cuda.synchronize()
+
+
 def test_merge_and_its_backward_against_checker():
     from retinags_amd import sharing
     scene, cam, part, models = _setup(60, 2, 1.0)
