@@ -265,6 +265,9 @@ def main():
     # ---- the steps after the path: image loss with its gradient, and the optimiser step
     after = training_stages(subs, H, W, dev, prof_steps) if do_backward else None
 
+    # ---- everything together: one training iteration for this camera
+    whole = whole_iteration(scene, part, cam_d, rel, bg, streams, dev, args.steps) if (part is not None and do_backward) else None
+
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
     cpu = None
     if not args.no_cpu_baseline:
@@ -284,7 +287,7 @@ def main():
                    "instance_room": (f"{args.instance_room} x the first frame's count, checked after every frame"
                                      if bounds is not None else "sized from each call's count (host waits)")},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
-        "blend_work": evals, "sharing": sharing, "loss_and_optimiser": after,
+        "blend_work": evals, "sharing": sharing, "loss_and_optimiser": after, "training_iteration": whole,
     }
     print(json.dumps(line))
 
@@ -348,6 +351,25 @@ def sharing_stages(scene, part, dev, repeats, append):
         if out[name]["achieved_GBps"] is not None:
             out[name]["frac"] = round(out[name]["achieved_GBps"] / HBM_PEAK_GBS, 4)
     return out
+
+
+def whole_iteration(scene, part, cam_d, rel, bg, streams, dev, repeats):
+    """Share the boundary Gaussians, render and composite, L1 + SSIM loss, backward, Adam: wall clock
+    per iteration with the host included (learning rates scaled down so that the scene stays the
+    workload it is).  Not the metric of `value`, which is the rasterizer's forward + backward."""
+    from retinags_amd.harness import pipeline
+    models = pipeline.owned_models_from_partition(scene, part, dev, spare_fraction=0.1)
+    for m in models:
+        for t in m.fields():
+            t.requires_grad_(True)
+    rates = {n: r * 1e-3 for n, r in pipeline.REFERENCE_LEARNING_RATES.items()}
+    optimisers = pipeline.make_optimisers(models, rates)
+    H, W = cam_d.image_height, cam_d.image_width
+    gt = torch.rand(3, H, W, generator=torch.Generator().manual_seed(11)).to(dev)
+    run = lambda: pipeline.training_iteration(models, optimisers, part, cam_d, rel, gt, bg, streams=streams, append=True)
+    ms = _timed_ms(run, repeats)
+    return {"ms_per_iteration": round(ms, 3), "iterations_per_s": round(1e3 / ms, 2),
+            "steps": "select + merge straddlers (appended), render + composite, L1+SSIM loss, backward, Adam (28 tensors)"}
 
 
 def _timed_ms(fn, repeats):

@@ -257,3 +257,39 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     out["partial"] = partial
     out["stages"] = stages
     return out
+
+
+REFERENCE_LEARNING_RATES = {"means3D": 0.00016, "means2D": 0.0, "opacity": 0.05, "scales": 0.005, "rotations": 0.001,
+                            "shs": 0.0025}   # arguments/__init__.py:84-95 (one rate for all SH coefficients here)
+
+
+def make_optimisers(models: List["SharedGSInfo"], rates: Optional[Dict[str, float]] = None):
+    """One Adam per submodel with a parameter group per field, eps 1e-15, as the reference sets up
+    (scene/gaussian_nn_module.py:433-443).  The harness trains the activated values directly."""
+    from ..optimizer import Adam
+    from ..sharing import FIELDS
+    rates = REFERENCE_LEARNING_RATES if rates is None else rates
+    return [Adam([{"params": [getattr(m, n)], "lr": rates[n], "name": n} for n in FIELDS], lr=0.0, eps=1e-15)
+            for m in models]
+
+
+def training_iteration(models: List["SharedGSInfo"], optimisers, part: Partition, cam: Camera, relation: np.ndarray,
+                       gt_image: torch.Tensor, background: torch.Tensor, lambda_dssim: float = 0.2,
+                       streams: Optional[List["torch.cuda.Stream"]] = None, append: bool = False) -> dict:
+    """One iteration of the reference's training loop for one camera with every submodel on one GPU
+    (parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:596-666, without densification
+    and logging): share the boundary Gaussians, render every related submodel, composite, take the
+    L1 + SSIM loss against gt_image, differentiate back to every submodel's own Gaussians, step the
+    optimisers.  Returns the loss terms (device scalars) and the frame."""
+    from ..loss import l1_ssim_loss
+    from ..sharing import merge_shared, select_straddlers
+    device = models[0].means3D.device
+    table = select_straddlers(models, part.box_low, part.box_up)
+    merged = merge_shared(models, table, reuse_gradients=True, append=append)
+    frame = render_frame(cam, submodels_from_shared(merged, part, device), relation, background, streams=streams)
+    loss, l1 = l1_ssim_loss(frame["render"], gt_image, lambda_dssim)
+    loss.backward()
+    for opt in optimisers:
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    return {"loss": loss.detach(), "l1": l1, "frame": frame, "lent_rows": int(table.counts.sum())}

@@ -1,0 +1,105 @@
+"""A whole training iteration on the GPU (share boundary Gaussians, render the submodels, composite,
+L1 + SSIM loss, backward to every submodel's own Gaussians, Adam) against the chain of CPU checkers
+for its gradients, and over a few iterations for what it is for: the loss goes down."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import GRAD_TOL, IMAGE_TOL, np32, oracle_settings, orc, rel_l2, scenes
+from oracle import sharing_oracle as so
+from oracle import training_oracle as to
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+NAMES = ("means3D", "means2D", "opacity", "scales", "rotations", "shs")
+
+
+def _setup(spare=0.0):
+    from retinags_amd.harness import partition, pipeline
+    scene, cam, _ = scenes.make_config("C1", shrink=150, resolution_scale=0.25)
+    scene["scales"] = scene["scales"] * 2.0      # more boundary straddlers at this size
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    rel = partition.relation_vector(part, cam)
+    models = pipeline.owned_models_from_partition(scene, part, DEV, spare)
+    return scene, cam, part, rel, models
+
+
+def test_gradients_of_one_iteration_against_the_checker_chain():
+    from retinags_amd import sharing
+    from retinags_amd.harness import pipeline
+    from retinags_amd.loss import l1_ssim_loss
+    scene, cam, part, rel, models = _setup()
+    K = len(models)
+    H, W = cam.image_height, cam.image_width
+    gen = torch.Generator().manual_seed(9)
+    gt = torch.rand(3, H, W, generator=gen)
+    bg = torch.tensor([0.1, 0.1, 0.1])
+    for m in models:
+        for t in m.fields():
+            t.requires_grad_(True)
+    table = sharing.select_straddlers(models, part.box_low, part.box_up)
+    assert table.counts.sum() > 20
+    merged = sharing.merge_shared(models, table, reuse_gradients=True)
+    frame = pipeline.render_frame(cam.to(DEV), pipeline.submodels_from_shared(merged, part, DEV), rel, bg.to(DEV))
+    loss, l1 = l1_ssim_loss(frame["render"], gt.to(DEV), 0.2)
+    loss.backward()
+    torch.cuda.synchronize()
+
+    # the same on the CPU: checker of every stage, chained
+    host = [{n: np32(getattr(m, n)) for n in NAMES} for m in models]
+    lent = {(s, d): so.straddler_rows(host[s]["means3D"], host[s]["scales"], part.box_low[s], part.box_up[s],
+                                      part.box_low[d], part.box_up[d]) for s in range(K) for d in range(K) if s != d}
+    order = sorted((m for m in range(K) if rel[m] >= 0), key=lambda m: rel[m])
+    blocks = {d: so.merged_rows([len(h["means3D"]) for h in host], lent, d) for d in order}
+    inputs = {d: so.merge_fields(host, blocks[d]) for d in order}
+    states, sets = {}, {}
+    for d in order:
+        sets[d] = oracle_settings(cam, torch.from_numpy(part.box_low[d]), torch.from_numpy(part.box_up[d]), torch.zeros(3))
+        states[d] = orc.forward(sets[d], inputs[d]["means3D"], inputs[d]["opacity"], shs=inputs[d]["shs"],
+                                scales=inputs[d]["scales"], rotations=inputs[d]["rotations"])
+    imgs, deps, alps = ([states[d].color for d in order], [states[d].depth for d in order], [states[d].alpha for d in order])
+    image, _, _ = orc.composite_forward(imgs, deps, alps, np32(bg))
+    want_loss, want_l1, _, d_image = to.l1_ssim(image, gt.numpy(), 0.2)
+    assert abs(float(loss.detach()) - want_loss) < 1e-5 and abs(float(l1) - want_l1) < 1e-5
+    assert np.abs(frame["render"].detach().cpu().numpy() - image).mean() < IMAGE_TOL
+    d_img, d_dep, d_alp = orc.composite_backward(imgs, deps, alps, np32(bg), d_image.astype(np.float32))
+    shapes = [{n: v.shape for n, v in h.items()} for h in host]
+    want = [{n: np.zeros(s, np.float32) for n, s in sh.items()} for sh in shapes]
+    for k, d in enumerate(order):
+        g = orc.backward(sets[d], states[d], d_img[k], d_dep[k], d_alp[k])
+        grads = {"means3D": g["means3D"], "means2D": g["means2D"], "opacity": g["opacity"], "scales": g["scales"],
+                 "rotations": g["rotations"], "shs": g["sh"]}
+        back = so.merge_backward(grads, blocks[d], shapes)
+        for s in range(K):
+            for n in NAMES:
+                want[s][n] += back[s][n]
+    for s in range(K):
+        for n in NAMES:
+            got = getattr(models[s], n).grad.cpu().numpy()
+            assert rel_l2(got, want[s][n]) <= GRAD_TOL, (s, n)
+
+
+@pytest.mark.parametrize("append", [False, True])
+def test_the_loss_goes_down(append):
+    from retinags_amd.harness import pipeline
+    scene, cam, part, rel, models = _setup(spare=0.3 if append else 0.0)
+    cam_d = cam.to(DEV)
+    bg = torch.zeros(3, device=DEV)
+    with torch.no_grad():
+        target = pipeline.render_frame(cam_d, pipeline.submodels_from_partition(scene, part, DEV), rel, bg)["render"].clone()
+        gen = torch.Generator().manual_seed(3)
+        for m in models:                                   # start from disturbed colours and opacities
+            m.shs.add_((torch.randn(m.shs.shape, generator=gen) * 0.1).to(DEV))
+            m.opacity.mul_(0.8)
+    for m in models:
+        for t in m.fields():
+            t.requires_grad_(True)
+    optimisers = pipeline.make_optimisers(models)
+    streams = [torch.cuda.current_stream(DEV)] + [torch.cuda.Stream(device=DEV) for _ in range(3)]
+    losses = []
+    for _ in range(12):
+        step = pipeline.training_iteration(models, optimisers, part, cam_d, rel, target, bg, streams=streams, append=append)
+        losses.append(float(step["loss"]))
+        assert step["lent_rows"] > 0
+    assert all(np.isfinite(losses)) and losses[-1] < 0.8 * losses[0], losses
+    assert all(opt.state[p]["step"] == 12 for opt in optimisers for g in opt.param_groups for p in g["params"])
