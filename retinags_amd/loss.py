@@ -33,7 +33,7 @@ class _L1SSIM(torch.autograd.Function):
     @staticmethod
     def forward(ctx, image: torch.Tensor, gt: torch.Tensor, lambda_dssim: float):
         x, y, planes, H, W = _as_planes(image, gt)
-        keep = image.requires_grad
+        keep = bool(ctx.needs_input_grad[0])
         workspace = torch.empty(lib.rgs_loss_workspace_bytes(planes, H, W), dtype=torch.uint8, device=x.device)
         out = torch.empty(3, device=x.device)
         check(lib.rgs_l1_ssim_forward(planes, H, W, ptr(x), ptr(y), float(lambda_dssim), ptr(out), ptr(workspace),
