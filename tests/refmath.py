@@ -4,10 +4,10 @@ Nothing here is derived from the checker's source: projection is a plain matrix 
 the covariance is R diag(s^2) R^T pushed through the EWA Jacobian, spherical harmonics come
 from scipy's complex harmonics, tile coverage is brute force, and the renderer is a
 differentiable torch program whose gradients come from autograd.  Where the reference
-deliberately deviates from the true gradient (straight-through 0.99 clamp, guard-frustum
-clamp, 1e-7 in the determinant, un-normalised quaternion) the scenes used with this module
-stay away from the deviation, or the deviation is part of the forward function itself
-(the quaternion is used as given).
+deliberately deviates from the true gradient, the deviation is modelled here as what it is: the
+0.99 clamp as a straight-through estimator, the guard-frustum clamp as a constant to the backward
+pass (detached), the quaternion used as given; only the 1e-7 in the determinant's reciprocal is
+left out (scenes with determinants far above it).
 """
 import math
 
@@ -74,8 +74,12 @@ def ewa_cov2d(means, cov3d, view_t, W, H, tanx, tany):
     fx, fy = W / (2 * tanx), H / (2 * tany)
     lx, ly = 1.3 * tanx, 1.3 * tany
     tz = t[:, 2]
-    tx = torch.clamp(t[:, 0] / tz, -lx, lx) * tz
-    ty = torch.clamp(t[:, 1] / tz, -ly, ly) * tz
+    # Outside the guard band the clamped coordinate is a constant to the backward pass: no gradient
+    # to t.x (t.y), and none to t.z through it (K/cuda_rasterizer_hgs/backward.cu:168-176, 262-264).
+    rx, ry = t[:, 0] / tz, t[:, 1] / tz
+    cx, cy = torch.clamp(rx, -lx, lx), torch.clamp(ry, -ly, ly)
+    tx = torch.where(cx == rx, t[:, 0], (cx * tz).detach())
+    ty = torch.where(cy == ry, t[:, 1], (cy * tz).detach())
     zero = torch.zeros_like(tz)
     J = torch.stack([torch.stack([fx / tz, zero, -fx * tx / tz ** 2], -1),
                      torch.stack([zero, fy / tz, -fy * ty / tz ** 2], -1)], -2)   # (n,2,3)

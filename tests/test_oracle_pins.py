@@ -392,6 +392,28 @@ def test_backward_straight_through_clamp():
     assert max(errs.values()) < 1e-3, errs
 
 
+def test_backward_outside_the_guard_frustum():
+    """Gaussians whose centre lies beyond 1.3 x the field of view but whose footprint still reaches
+    the image: the forward clamps the view-space x / y it linearises around, and the backward treats
+    the clamped value as a constant (K/cuda_rasterizer_hgs/backward.cu:168-176, 262-264).  The
+    independent renderer models exactly that with a detached clamp."""
+    scene, cam = tiny_scene(24, seed=13, log_scale=-1.0)
+    with torch.no_grad():
+        z = scene["xyz"][:, 2]
+        # half of them far off to the sides and above / below, large enough to be seen
+        scene["xyz"][0:6, 0] = 1.6 * cam.tanfovx * z[0:6] * torch.tensor([1, -1, 1, -1, 1, -1.0])
+        scene["xyz"][6:12, 1] = 1.5 * cam.tanfovy * z[6:12] * torch.tensor([1, -1, 1, -1, 1, -1.0])
+        scene["scales"][0:12] = scene["scales"][0:12] * 2.5
+    view = np32(scene["xyz"]) @ cam.world_view_transform.numpy()[:3, :3] + cam.world_view_transform.numpy()[3, :3]
+    outside = (np.abs(view[:, 0] / view[:, 2]) > 1.3 * cam.tanfovx) | (np.abs(view[:, 1] / view[:, 2]) > 1.3 * cam.tanfovy)
+    errs, got, st = _oracle_vs_autograd(scene, cam, *big_box(), torch.tensor([0.2, 0.2, 0.2]), 4, True)
+    seen_outside = outside & (st.radii > 0)
+    assert seen_outside.sum() >= 6
+    # they do take part: their gradients are not zero
+    assert np.abs(got["means3D"][seen_outside]).sum() > 0 and np.abs(got["scales"][seen_outside]).sum() > 0
+    assert max(errs.values()) < 1e-3, errs
+
+
 # ---- compositor (parallel_utils/basic_parallel_trainer/result_aggregator.py:244-259) -------------------
 
 def _torch_composite(images, depths, alphas, bg):
