@@ -86,6 +86,26 @@ def whole_scene_submodel(scene: Dict[str, torch.Tensor], device, margin: float =
     return Submodel(mv(xyz), mv(scene["opacity"]), mv(scene["scales"]), mv(scene["rotations"]), mv(scene["shs"]), low, up)
 
 
+class GradNormHelper(torch.autograd.Function):
+    """The placeholder through which the reference collects the screen-space gradient norm that
+    densification reads (gaussian_renderer/render_half_gs.py:7-19): forward turns an (N,1) meta
+    tensor into the (N,3) zeros passed as means2D; backward hands the meta tensor the length of
+    each row's (x, y) gradient."""
+
+    @staticmethod
+    def forward(ctx, meta: torch.Tensor) -> torch.Tensor:
+        if meta.dim() != 2 or meta.shape[1] != 1:
+            raise RuntimeError("meta must have shape (N, 1)")
+        return torch.zeros((meta.shape[0], 3), dtype=meta.dtype, device=meta.device)
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor) -> torch.Tensor:
+        return torch.norm(grad_output[:, :2], dim=-1, keepdim=True)
+
+
+gradNormHelpFunction = GradNormHelper.apply
+
+
 def raster_settings(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0,
                     debug: bool = False) -> GaussianRasterizationSettings:
     return GaussianRasterizationSettings(

@@ -164,3 +164,16 @@ def test_banded_tile_order_is_a_bijection(tmp_path):
                     os.path.join(here, "tile_order_check.cpp"), "-o", exe], check=True)
     out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
     assert out.strip() == "ok"
+
+
+def test_grad_norm_helper_hands_back_the_screen_space_gradient_length():
+    """gaussian_renderer/render_half_gs.py:7-19."""
+    from retinags_amd.harness.pipeline import gradNormHelpFunction
+    meta = torch.zeros(5, 1, requires_grad=True)
+    means2D = gradNormHelpFunction(meta)
+    assert means2D.shape == (5, 3) and float(means2D.abs().sum()) == 0.0 and means2D.requires_grad
+    g = torch.tensor([[3.0, 4.0, 9.0], [0.0, 0.0, 1.0], [1.0, 0.0, 0.0], [-6.0, 8.0, 0.0], [0.5, 0.5, 0.5]])
+    means2D.backward(g)
+    assert torch.allclose(meta.grad[:, 0], torch.tensor([5.0, 0.0, 1.0, 10.0, 0.5 * 2 ** 0.5]))
+    with pytest.raises(RuntimeError):
+        gradNormHelpFunction(torch.zeros(5, 2))
