@@ -259,14 +259,24 @@ def main():
     }
 
     # ---- the step before the path: who lends which Gaussians to whom, and the merged inputs
-    sharing = ({"appending": sharing_stages(scene, part, dev, prof_steps, True),
-                "copying": sharing_stages(scene, part, dev, prof_steps, False)} if part is not None else None)
+    def aside(fn):
+        """The sections beside the metric must not take the metric's line with them."""
+        try:
+            return fn()
+        except Exception as ex:   # reported in the line instead
+            torch.cuda.synchronize()
+            return {"error": f"{type(ex).__name__}: {ex}"}
+
+    sharing = (aside(lambda: {"appending": sharing_stages(scene, part, dev, prof_steps, True),
+                              "copying": sharing_stages(scene, part, dev, prof_steps, False)})
+               if part is not None else None)
 
     # ---- the steps after the path: image loss with its gradient, and the optimiser step
-    after = training_stages(subs, H, W, dev, prof_steps) if do_backward else None
+    after = aside(lambda: training_stages(subs, H, W, dev, prof_steps)) if do_backward else None
 
     # ---- everything together: one training iteration for this camera
-    whole = whole_iteration(scene, part, cam_d, rel, bg, streams, dev, args.steps) if (part is not None and do_backward) else None
+    whole = (aside(lambda: whole_iteration(scene, part, cam_d, rel, bg, streams, dev, args.steps))
+             if (part is not None and do_backward) else None)
 
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
     cpu = None
