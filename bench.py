@@ -379,7 +379,8 @@ def whole_iteration(scene, part, cam_d, rel, bg, streams, dev, repeats):
     run = lambda: pipeline.training_iteration(models, optimisers, part, cam_d, rel, gt, bg, streams=streams, append=True)
     ms = _timed_ms(run, repeats)
     return {"ms_per_iteration": round(ms, 3), "iterations_per_s": round(1e3 / ms, 2),
-            "steps": "select + merge straddlers (appended), render + composite, L1+SSIM loss, backward, Adam (28 tensors)"}
+            "steps": f"select + merge straddlers (appended), render + composite, L1+SSIM loss, backward, "
+                     f"Adam ({6 * len(models)} tensors)"}
 
 
 def _timed_ms(fn, repeats):

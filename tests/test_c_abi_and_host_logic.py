@@ -171,9 +171,51 @@ def test_grad_norm_helper_hands_back_the_screen_space_gradient_length():
     from retinags_amd.harness.pipeline import gradNormHelpFunction
     meta = torch.zeros(5, 1, requires_grad=True)
     means2D = gradNormHelpFunction(meta)
-    assert means2D.shape == (5, 3) and float(means2D.abs().sum()) == 0.0 and means2D.requires_grad
+    assert means2D.shape == (5, 3) and float(means2D.detach().abs().sum()) == 0.0 and means2D.requires_grad
     g = torch.tensor([[3.0, 4.0, 9.0], [0.0, 0.0, 1.0], [1.0, 0.0, 0.0], [-6.0, 8.0, 0.0], [0.5, 0.5, 0.5]])
     means2D.backward(g)
     assert torch.allclose(meta.grad[:, 0], torch.tensor([5.0, 0.0, 1.0, 10.0, 0.5 * 2 ** 0.5]))
     with pytest.raises(RuntimeError):
         gradNormHelpFunction(torch.zeros(5, 2))
+
+
+def test_entry_points_refuse_bad_arguments_before_touching_the_gpu():
+    """Argument checks come first and report through rgs_last_error; none of these calls launches."""
+    import ctypes as C
+    from retinags_amd import _capi
+    lib = _capi.lib
+    null = C.c_void_p(0)
+    fp = C.POINTER(C.c_float)
+    three = (C.c_float * 3)(0, 0, 0)
+    boxes = (C.c_float * 6)(0, 0, 0, 1, 1, 1)
+    as_fp = lambda a: C.cast(a, fp)
+
+    def refused(rc, needle):
+        assert rc != 0
+        message = lib.rgs_last_error().decode()
+        assert needle in message, message
+
+    refused(lib.rgs_straddler_select(10, null, null, as_fp(three), as_fp(three), 0, as_fp(boxes), as_fp(boxes), -1,
+                                     null, null, 0, null, null), "n_boxes")
+    refused(lib.rgs_straddler_select(10, null, null, as_fp(three), as_fp(three), 65, as_fp(boxes), as_fp(boxes), -1,
+                                     null, null, 0, null, null), "n_boxes")
+    refused(lib.rgs_straddler_select(10, null, null, as_fp(three), as_fp(three), 2, as_fp(boxes), as_fp(boxes), 2,
+                                     null, null, 0, null, null), "skip")
+    refused(lib.rgs_straddler_select(-1, null, null, as_fp(three), as_fp(three), 2, as_fp(boxes), as_fp(boxes), 0,
+                                     null, null, 0, null, null), "negative")
+    seg = (_capi.SharedRows * 1)(_capi.SharedRows(None, None, None, None, None, None, 5))
+    refused(lib.rgs_merge_rows(1, seg, 0, 48, null, null, null, null, null, null), "null field")
+    refused(lib.rgs_merge_rows(1, seg, 0, -3, null, null, null, null, null, null), "sh_floats")
+    assert lib.rgs_merge_rows(0, None, 0, 48, null, null, null, null, null, null) == 0       # nothing to do
+    grads = (_capi.SharedGrads * 1)(_capi.SharedGrads(None, None, None, None, None, None, None, 5))
+    refused(lib.rgs_merge_rows_backward(1, grads, 0, 48, null, null, null, null, null, null, null), "row list")
+    refused(lib.rgs_l1_ssim_forward(3, 0, 10, null, null, 0.2, null, null, 1, null), "bad image size")
+    refused(lib.rgs_l1_ssim_forward(3, 10, 10, null, null, 0.2, null, null, 1, null), "null pointer")
+    refused(lib.rgs_l1_ssim_backward(3, 10, 10, null, null, 0.2, null, null, null, null), "null pointer")
+    assert lib.rgs_loss_workspace_bytes(3, 0, 5) == 0 and lib.rgs_loss_workspace_bytes(3, 16, 32) == 4 * (3 * 3 * 16 * 32 + 2 * 3)
+    t = (_capi.AdamTensor * 1)(_capi.AdamTensor(None, None, None, None, 8, 0.1, 1))
+    refused(lib.rgs_adam_step(1, t, 0.9, 0.999, 1e-8, null), "null array")
+    t[0].n, t[0].step = 0, 0
+    refused(lib.rgs_adam_step(1, t, 0.9, 0.999, 1e-8, null), "step")
+    assert lib.rgs_adam_step(0, None, 0.9, 0.999, 1e-8, null) == 0
+    assert lib.rgs_straddler_scratch_bytes(-1, 4) == 0 and lib.rgs_straddler_scratch_bytes(1025, 3) == 4 * 3 * 3
