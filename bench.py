@@ -150,6 +150,7 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t1
     ms_per_step = elapsed * 1e3 / args.steps
+    peak_gb = torch.cuda.max_memory_allocated(dev) / 1e9   # inputs, workspaces and gradients of the timed steps
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -242,7 +243,9 @@ def main():
                         "unit": "GB/s", "frac": d["frac"], "traffic": None}
         elif d.get("bound") == "valu":
             roofline = {"kernel": dominant, "bound": "valu", "achieved": d["achieved_TFLOPs"],
-                        "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": d["frac"], "traffic": None}
+                        "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": d["frac"], "traffic": None,
+                        "bound_note": "fp32 vector-ALU issue (per-pixel compare / exp / blend arithmetic, no dense "
+                                      "contraction, so no MFMA); peak is the published 157.3 TFLOP/s fp32 figure"}
         if roofline is not None:
             full_c1 = args.config == "C1" and args.shrink == 1.0 and args.resolution_scale == 1.0
             if full_c1 and dominant in C1_TRAFFIC_MB_PER_LAUNCH:
@@ -294,6 +297,7 @@ def main():
                                f"{'fwd+bwd' if do_backward else 'fwd only'}",
                    "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
                    "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1),
+                   "peak_device_memory_GB": round(peak_gb, 2),
                    "instance_room": (f"{args.instance_room} x the first frame's count, checked after every frame"
                                      if bounds is not None else "sized from each call's count (host waits)")},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
