@@ -114,3 +114,42 @@ def test_adam_handles_odd_sizes_and_many_tensors():
     for k, p in enumerate(ps):
         assert np.abs(p.detach().cpu().numpy() - want[k]).max() <= 2e-6, k
     assert float(base[0]) == 0.0 and float(base[at:].abs().max()) == 0.0     # nothing written outside the tensors
+
+
+def test_golden_vectors_of_the_neighbouring_steps():
+    """The committed fixtures (tests/golden/neighbouring_steps_small.npz) through the C ABI: row lists
+    bit for bit, loss and gradient, five Adam steps."""
+    import os
+    from helpers import ROOT
+    from retinags_amd import loss as L, sharing
+    from retinags_amd.optimizer import Adam
+    z = np.load(os.path.join(ROOT, "tests", "golden", "neighbouring_steps_small.npz"))
+    dev = lambda a: torch.tensor(a, device=DEV)
+    models = []
+    for m in range(3):
+        xyz = dev(z[f"share/xyz{m}"])
+        n = xyz.shape[0]
+        models.append(sharing.SharedGSInfo(xyz, torch.zeros_like(xyz), torch.zeros(n, 1, device=DEV), dev(z[f"share/scales{m}"]),
+                                           torch.zeros(n, 4, device=DEV), torch.zeros(n, 16, 3, device=DEV)))
+    table = sharing.select_straddlers(models, z["share/box_low"], z["share/box_up"])
+    for s in range(3):
+        for d in range(3):
+            if s != d:
+                want = z[f"share/rows_{s}_{d}"]
+                assert table.counts[s, d] == len(want)
+                if len(want):
+                    assert np.array_equal(table.rows[(s, d)].cpu().numpy().astype(np.int64), want)
+    x = dev(z["loss/image"]).requires_grad_(True)
+    loss, l1 = L.l1_ssim_loss(x, dev(z["loss/gt"]), 0.2)
+    loss.backward()
+    assert abs(float(loss.detach()) - z["loss/values"][0]) < 2e-6 and abs(float(l1) - z["loss/values"][1]) < 2e-6
+    assert rel_l2(x.grad.cpu().numpy(), z["loss/grad"]) < 1e-3
+    ps = [torch.nn.Parameter(dev(z[f"adam/param{k}"])) for k in range(4)]
+    opt = Adam([{"params": [p], "lr": float(lr)} for p, lr in zip(ps, z["adam/lrs"])], lr=0.0, eps=1e-15)
+    for t in range(5):
+        for k, p in enumerate(ps):
+            p.grad = dev(z[f"adam/grad{t}_{k}"])
+        opt.step()
+    for k, p in enumerate(ps):
+        assert rel_l2(p.detach().cpu().numpy(), z[f"adam/after{k}"]) < 1e-6
+        assert rel_l2(opt.state[p]["exp_avg_sq"].cpu().numpy(), z[f"adam/exp_avg_sq{k}"]) < 1e-6
