@@ -368,23 +368,59 @@ def sharing_stages(scene, part, dev, repeats, append):
 
 
 def whole_iteration(scene, part, cam_d, rel, bg, streams, dev, repeats):
-    """Share the boundary Gaussians, render and composite, L1 + SSIM loss, backward, Adam: wall clock
-    per iteration with the host included (learning rates scaled down so that the scene stays the
-    workload it is).  Not the metric of `value`, which is the rasterizer's forward + backward."""
+    """From the stored parameters and back to them: activation, sharing of the boundary Gaussians,
+    render and composite, L1 + SSIM loss, backward through all of it, Adam.  Wall clock per iteration
+    with the host included (learning rates scaled down so that the scene stays the workload it is);
+    the activation kernels' own times from the library's stage events.  Not the metric of `value`,
+    which is the rasterizer's forward + backward."""
+    from retinags_amd import _capi
     from retinags_amd.harness import pipeline
-    models = pipeline.owned_models_from_partition(scene, part, dev, spare_fraction=0.1)
+    models = pipeline.stored_models_from_partition(scene, part, dev, spare_fraction=0.1)
     for m in models:
-        for t in m.fields():
+        for t in m.parameters():
             t.requires_grad_(True)
-    rates = {n: r * 1e-3 for n, r in pipeline.REFERENCE_LEARNING_RATES.items()}
-    optimisers = pipeline.make_optimisers(models, rates)
+    optimisers = pipeline.make_stored_optimisers(models, scale=1e-3)
     H, W = cam_d.image_height, cam_d.image_width
     gt = torch.rand(3, H, W, generator=torch.Generator().manual_seed(11)).to(dev)
-    run = lambda: pipeline.training_iteration(models, optimisers, part, cam_d, rel, gt, bg, streams=streams, append=True)
+    run = lambda: pipeline.stored_training_iteration(models, optimisers, part, cam_d, rel, gt, bg, streams=streams)
     ms = _timed_ms(run, repeats)
-    return {"ms_per_iteration": round(ms, 3), "iterations_per_s": round(1e3 / ms, 2),
-            "steps": f"select + merge straddlers (appended), render + composite, L1+SSIM loss, backward, "
-                     f"Adam ({6 * len(models)} tensors)"}
+    _capi.stage_timing(True)
+    run()
+    stage = _capi.stage_timing_read()
+    _capi.stage_timing(False)
+    n = float(sum(int(m.xyz.shape[0]) for m in models))
+
+    def activations_by_tensor_expressions():
+        import torch.nn.functional as F
+        for m in models:
+            outs = [torch.cat((m.features_dc, m.features_rest), dim=1), torch.exp(m.scaling), F.normalize(m.rotation),
+                    torch.sigmoid(m.opacity)]
+            torch.autograd.backward(outs, [torch.ones_like(o) for o in outs])
+            for t in m.parameters():
+                t.grad = None
+
+    def activations_by_the_library():
+        for m in models:
+            shown = m.activated()
+            outs = [shown.shs, shown.scales, shown.rotations, shown.opacity]
+            torch.autograd.backward(outs, [torch.ones_like(o) for o in outs])
+            for t in m.parameters():
+                t.grad = None
+
+    out = {"ms_per_iteration": round(ms, 3), "iterations_per_s": round(1e3 / ms, 2),
+           "activation_fwd_bwd_wall_ms": round(_timed_ms(activations_by_the_library, repeats), 3),
+           "activation_tensor_expression_wall_ms": round(_timed_ms(activations_by_tensor_expressions, repeats), 3),
+           "steps": f"activate, select + merge straddlers (appended), render + composite, L1+SSIM loss, backward, "
+                    f"Adam ({7 * len(models)} tensors)"}
+    # algorithmic bytes: 224 in + 224 out per Gaussian forward (56 floats: SH, scale, rotation, opacity);
+    # backward reads their gradients, the stored rotation and the activated scale / opacity, writes 224
+    for name, per_gaussian in (("activate_forward", 448.0), ("activate_backward", 224.0 + 32.0 + 224.0)):
+        if name in stage and stage[name][0] > 0:
+            t = stage[name][0]
+            out[name] = {"ms_per_iteration": round(t, 4), "launches": stage[name][1],
+                         "achieved_GBps": round(per_gaussian * n / (t * 1e-3) / 1e9, 1),
+                         "frac": round(per_gaussian * n / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
 
 
 def _timed_ms(fn, repeats):

@@ -322,6 +322,24 @@ int rgs_l1_ssim_backward(int channels, int height, int width, const float* image
                          float lambda_dssim, const float* grad_loss, const void* workspace, float* d_image,
                          void* stream);
 
+/* ---- activation ------------------------------------------------------------------------------
+ * From a submodel's stored parameters to the tensors its renderer and its neighbours see
+ * (scene/gaussian_nn_module.py:373-394: get_scaling = exp, get_opacity = sigmoid, get_rotation =
+ * torch.nn.functional.normalize, get_features = cat(features_dc, features_rest); get_xyz is the
+ * stored tensor itself and has no part here).  features_dc (n,1,3), features_rest (n,rest,3),
+ * scaling (n,3), rotation (n,4), opacity (n,1) in; shs (n,1+rest,3), scales, rotations, opacities
+ * out; all on the device.  The backward turns the gradients of the four outputs (any may be NULL:
+ * that parameter's gradient is then not written) into gradients of the five stored tensors; it
+ * reads the stored rotation and the activated scales and opacities the forward wrote.  Every array
+ * except features_dc / features_rest and their gradients must start at a multiple of 16 bytes. */
+int rgs_activate_forward(int n, int rest, const float* features_dc, const float* features_rest, const float* scaling,
+                         const float* rotation, const float* opacity, float* shs, float* scales, float* rotations,
+                         float* opacities, void* stream);
+int rgs_activate_backward(int n, int rest, const float* rotation, const float* scales, const float* opacities,
+                          const float* g_shs, const float* g_scales, const float* g_rotations, const float* g_opacities,
+                          float* d_features_dc, float* d_features_rest, float* d_scaling, float* d_rotation,
+                          float* d_opacity, void* stream);
+
 /* ---- optimiser step ---------------------------------------------------------------------------
  * torch.optim.Adam without weight decay or amsgrad, as the reference sets it up per submodel
  * (scene/gaussian_nn_module.py:429-444) and steps it once per iteration

@@ -9,7 +9,8 @@ TEST INFRASTRUCTURE ONLY.  Tests, ``__graft_entry__.smoke()`` and the ``cpu_base
 convolution in float64; its gradient is autograd's.  Pinned by tests/test_training_cpu.py:
 SSIM against an implementation built on scipy.ndimage's separable Gaussian filter, SSIM(x, x) = 1,
 the gradient against central differences.  ``adam_reference`` IS torch.optim.Adam (the reference's
-optimiser, scene/gaussian_nn_module.py:443) run on the CPU, so it needs no pin.
+optimiser, scene/gaussian_nn_module.py:443) run on the CPU, so it needs no pin; ``activate_reference``
+likewise is the reference's own four tensor expressions with autograd.
 """
 from __future__ import annotations
 
@@ -56,6 +57,22 @@ def l1_ssim(image: np.ndarray, gt: np.ndarray, lambda_dssim: float = 0.2, want_g
         loss.backward()
         grad = x.grad.numpy()
     return float(loss.detach()), float(l1.detach()), float(s.detach()), grad
+
+
+def activate_reference(features_dc, features_rest, scaling, rotation, opacity, grads=None):
+    """The reference's activations as it writes them (scene/gaussian_nn_module.py:304-312, 373-394):
+    torch.exp, torch.sigmoid, torch.nn.functional.normalize, torch.cat, on the CPU in float32.
+    Returns (shs, scales, rotations, opacities) and, with `grads` (gradients of those four), the
+    gradients of the five inputs by autograd."""
+    leaves = [torch.tensor(np.asarray(a, dtype=np.float32), requires_grad=grads is not None)
+              for a in (features_dc, features_rest, scaling, rotation, opacity)]
+    dc, rest, sc, rot, op = leaves
+    outs = (torch.cat((dc, rest), dim=1), torch.exp(sc), F.normalize(rot), torch.sigmoid(op))
+    values = [o.detach().numpy().copy() for o in outs]
+    if grads is None:
+        return values, None
+    torch.autograd.backward(outs, [torch.tensor(np.asarray(g, dtype=np.float32)) for g in grads])
+    return values, [t.grad.numpy().copy() for t in leaves]
 
 
 def adam_reference(params: Sequence[np.ndarray], lrs: Sequence[float], grads_per_step: Sequence[Sequence[np.ndarray]],

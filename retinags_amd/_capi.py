@@ -84,6 +84,8 @@ def _load():
     lib.rgs_loss_workspace_bytes.restype, lib.rgs_loss_workspace_bytes.argtypes = sz, [i, i, i]
     lib.rgs_l1_ssim_forward.argtypes = [i, i, i, vp, vp, f, vp, vp, i, vp]
     lib.rgs_l1_ssim_backward.argtypes = [i, i, i, vp, vp, f, vp, vp, vp, vp]
+    lib.rgs_activate_forward.argtypes = [i, i] + [vp] * 10
+    lib.rgs_activate_backward.argtypes = [i, i] + [vp] * 13
     lib.rgs_adam_step.argtypes = [i, C.POINTER(AdamTensor), C.c_double, C.c_double, C.c_double, vp]
     lib.rgs_stage_timing.argtypes = [i]
     lib.rgs_stage_timing_read.argtypes = [i, C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.POINTER(C.c_int)]
@@ -91,7 +93,8 @@ def _load():
     for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
                  "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_forward_raster_bounded", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
                  "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
-                 "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step"):
+                 "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step",
+                 "rgs_activate_forward", "rgs_activate_backward"):
         getattr(lib, name).restype = i
     return lib
 
@@ -104,7 +107,8 @@ EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_byte
            "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward",
            "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",
            "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward", "rgs_loss_workspace_bytes",
-           "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step")
+           "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step", "rgs_activate_forward",
+           "rgs_activate_backward")
 WORK_COUNTERS = 7
 
 

@@ -1051,6 +1051,62 @@ int rgs_l1_ssim_backward(int channels, int height, int width, const float* image
 	return 0;
 }
 
+int rgs_activate_forward(int n, int rest, const float* features_dc, const float* features_rest, const float* scaling,
+                         const float* rotation, const float* opacity, float* shs, float* scales, float* rotations,
+                         float* opacities, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(n >= 0 && rest >= 0, "rgs_activate_forward: bad sizes n=%d rest=%d", n, rest);
+	if (n == 0)
+		return 0;
+	RGS_REQUIRE(features_dc && (features_rest || rest == 0) && scaling && rotation && opacity && shs && scales && rotations &&
+	                opacities,
+	            "rgs_activate_forward: null pointer");
+	RGS_REQUIRE(aligned16(scaling) && aligned16(rotation) && aligned16(opacity) && aligned16(shs) && aligned16(scales) &&
+	                aligned16(rotations) && aligned16(opacities),
+	            "rgs_activate_forward: arrays must start at multiples of 16 bytes");
+	rgs::ActivateArgs a;
+	a.n = n; a.rest = rest;
+	a.features_dc = features_dc; a.features_rest = features_rest; a.scaling = scaling; a.rotation = rotation;
+	a.opacity = opacity;
+	a.shs = shs; a.scales = scales; a.rotations = rotations; a.opacities = opacities;
+	rgs::launch_activate_forward(a, s);
+	RGS_STAGE("activate_forward");
+	return 0;
+}
+
+int rgs_activate_backward(int n, int rest, const float* rotation, const float* scales, const float* opacities,
+                          const float* g_shs, const float* g_scales, const float* g_rotations, const float* g_opacities,
+                          float* d_features_dc, float* d_features_rest, float* d_scaling, float* d_rotation,
+                          float* d_opacity, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(n >= 0 && rest >= 0, "rgs_activate_backward: bad sizes n=%d rest=%d", n, rest);
+	if (n == 0)
+		return 0;
+	RGS_REQUIRE(!g_shs || (d_features_dc && (d_features_rest || rest == 0)), "rgs_activate_backward: no room for the SH gradients");
+	RGS_REQUIRE(!g_scales || (scales && d_scaling), "rgs_activate_backward: scales or their gradient missing");
+	RGS_REQUIRE(!g_rotations || (rotation && d_rotation), "rgs_activate_backward: rotation or its gradient missing");
+	RGS_REQUIRE(!g_opacities || (opacities && d_opacity), "rgs_activate_backward: opacities or their gradient missing");
+	RGS_REQUIRE(aligned16(rotation) && aligned16(scales) && aligned16(opacities) && aligned16(g_shs) && aligned16(g_scales) &&
+	                aligned16(g_rotations) && aligned16(g_opacities) && aligned16(d_scaling) && aligned16(d_rotation) &&
+	                aligned16(d_opacity),
+	            "rgs_activate_backward: arrays must start at multiples of 16 bytes");
+	rgs::ActivateBackwardArgs a;
+	a.n = n; a.rest = rest;
+	a.rotation = rotation; a.scales = scales; a.opacities = opacities;
+	a.g_shs = g_shs; a.g_scales = g_scales; a.g_rotations = g_rotations; a.g_opacities = g_opacities;
+	a.d_features_dc = d_features_dc; a.d_features_rest = d_features_rest; a.d_scaling = d_scaling;
+	a.d_rotation = d_rotation; a.d_opacity = d_opacity;
+	rgs::launch_activate_backward(a, s);
+	RGS_STAGE("activate_backward");
+	return 0;
+}
+
 int rgs_adam_step(int n_tensors, const rgs_adam_tensor* tensors, double beta1, double beta2, double eps, void* stream)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);

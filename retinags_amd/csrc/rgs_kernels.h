@@ -203,6 +203,33 @@ struct LossArgs {
 	const float* grad_loss;  // backward: upstream gradient of the loss (device scalar) or null for 1
 	float* d_image;          // backward: gradient of the loss with respect to x
 };
+struct ActivateArgs {
+	int n, rest;                 // Gaussians; SH coefficients beyond the first (15 at degree 3)
+	const float* features_dc;    // (n,1,3)
+	const float* features_rest;  // (n,rest,3)
+	const float* scaling;        // (n,3) log of the scales
+	const float* rotation;       // (n,4) as stored
+	const float* opacity;        // (n,1) logit
+	float* shs;                  // (n,1+rest,3)
+	float* scales;
+	float* rotations;
+	float* opacities;
+};
+struct ActivateBackwardArgs {
+	int n, rest;
+	const float* rotation;       // stored quaternions
+	const float* scales;         // activated values, as the forward wrote them
+	const float* opacities;
+	const float* g_shs;          // gradients of the activated tensors; any may be null (that output is left alone)
+	const float* g_scales;
+	const float* g_rotations;
+	const float* g_opacities;
+	float* d_features_dc;
+	float* d_features_rest;
+	float* d_scaling;
+	float* d_rotation;
+	float* d_opacity;
+};
 constexpr int kMaxAdamTensors = 16;
 struct AdamTensor {
 	float* param;
@@ -299,6 +326,8 @@ void launch_merge_rows_backward(const MergeBackwardArgs& a, uint32_t blocks, boo
 uint32_t loss_blocks(int C, int H, int W);   // workgroups of the loss kernels = pairs of partial sums
 void launch_l1_ssim_forward(const LossArgs& a, hipStream_t s);
 void launch_l1_ssim_backward(const LossArgs& a, hipStream_t s);
+void launch_activate_forward(const ActivateArgs& a, hipStream_t s);
+void launch_activate_backward(const ActivateBackwardArgs& a, hipStream_t s);
 uint32_t adam_blocks_for(size_t n);
 void launch_adam_step(const AdamArgs& a, uint32_t blocks, hipStream_t s);
 

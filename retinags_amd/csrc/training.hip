@@ -15,6 +15,10 @@
 // which the backward kernel computes with the same two passes.  Bound by HBM (44 bytes per pixel
 // and channel over both kernels) and by LDS reads.
 //
+// Activation (scene/gaussian_nn_module.py:373-394): what a submodel's renderer and neighbours see
+// is exp of the stored scales, sigmoid of the stored opacities, the normalised quaternions and the
+// two SH parameter tensors joined: one flat pass forward and one backward.
+//
 // Adam (torch.optim.Adam as the reference configures it, scene/gaussian_nn_module.py:429-444:
 // eps 1e-15, no weight decay, no amsgrad): one pass over parameter, gradient and both moments.
 #include "rgs_device.h"
@@ -315,7 +319,192 @@ __global__ __launch_bounds__(256) void adam_step_kernel(AdamArgs a)
 	}
 }
 
+// Both activation kernels are flat passes over four arrays; a workgroup works on one of them
+// (its part is the same for all its threads), 1024 sixteen-byte units per workgroup, so every
+// store is a full 16 bytes to consecutive addresses.  The SH rows are the one place where that
+// takes care: a row of the joined tensor is 3 floats of one source followed by 3 * rest of the
+// other, so the 16-byte units of the output (or of its gradient) straddle the two sources and
+// are put together from 4-byte accesses on the source side.
+constexpr int kActUnits = 1024;   // 16-byte units per workgroup: 4 per thread
+
+struct ActParts {
+	uint32_t sh_blocks, rot_blocks, scale_blocks, opacity_blocks;
+};
+
+__host__ __device__ inline ActParts act_parts(int n, int rest)
+{
+	const size_t sh_floats = 3 * (size_t)(1 + rest);
+	auto blocks = [](size_t units) { return (uint32_t)((units + kActUnits - 1) / kActUnits); };
+	ActParts p;
+	p.sh_blocks = blocks(((size_t)n * sh_floats + 3) / 4);
+	p.rot_blocks = blocks((size_t)n);
+	p.scale_blocks = blocks(((size_t)n * 3 + 3) / 4);
+	p.opacity_blocks = blocks(((size_t)n + 3) / 4);
+	return p;
+}
+
+// floats [4u, 4u+4) of a flat array of `total` floats, element by element where the array ends
+template <typename F>
+__device__ __forceinline__ void flat_unit(size_t u, size_t total, const float* __restrict__ in, float* __restrict__ out, F f)
+{
+	if (4 * u + 4 <= total) {
+		const float4 v = reinterpret_cast<const float4*>(in)[u];
+		reinterpret_cast<float4*>(out)[u] = float4{f(v.x, 4 * u), f(v.y, 4 * u + 1), f(v.z, 4 * u + 2), f(v.w, 4 * u + 3)};
+	} else {
+		for (size_t k = 4 * u; k < total; k++)
+			out[k] = f(in[k], k);
+	}
+}
+
+__global__ __launch_bounds__(256) void activate_forward_kernel(ActivateArgs a, ActParts parts)
+{
+	uint32_t block = blockIdx.x;
+	const size_t n = (size_t)a.n;
+	if (block < parts.sh_blocks) {
+		const size_t sh_floats = 3 * (size_t)(1 + a.rest), rest_floats = 3 * (size_t)a.rest, total = n * sh_floats;
+		for (int it = 0; it < kActUnits / 256; it++) {
+			const size_t u = (size_t)block * kActUnits + it * 256 + threadIdx.x;
+			if (4 * u >= total)
+				break;
+			float v[4];
+#pragma unroll
+			for (int k = 0; k < 4; k++) {
+				const size_t at = 4 * u + k;
+				if (at < total) {
+					const size_t row = at / sh_floats, col = at - row * sh_floats;
+					v[k] = col < 3 ? a.features_dc[3 * row + col] : a.features_rest[rest_floats * row + (col - 3)];
+				} else {
+					v[k] = 0.f;
+				}
+			}
+			if (4 * u + 4 <= total)
+				reinterpret_cast<float4*>(a.shs)[u] = float4{v[0], v[1], v[2], v[3]};
+			else
+				for (size_t k = 4 * u; k < total; k++)
+					a.shs[k] = v[k - 4 * u];
+		}
+		return;
+	}
+	block -= parts.sh_blocks;
+	if (block < parts.rot_blocks) {
+		for (int it = 0; it < kActUnits / 256; it++) {
+			const size_t i = (size_t)block * kActUnits + it * 256 + threadIdx.x;
+			if (i >= n)
+				break;
+			const float4 q = reinterpret_cast<const float4*>(a.rotation)[i];
+			const float len = fmaxf(sqrtf(q.x * q.x + q.y * q.y + q.z * q.z + q.w * q.w), 1e-12f);  // torch.nn.functional.normalize
+			reinterpret_cast<float4*>(a.rotations)[i] = float4{q.x / len, q.y / len, q.z / len, q.w / len};
+		}
+		return;
+	}
+	block -= parts.rot_blocks;
+	if (block < parts.scale_blocks) {
+		for (int it = 0; it < kActUnits / 256; it++)
+			flat_unit((size_t)block * kActUnits + it * 256 + threadIdx.x, 3 * n, a.scaling, a.scales,
+			          [](float v, size_t) { return expf(v); });
+		return;
+	}
+	block -= parts.scale_blocks;
+	for (int it = 0; it < kActUnits / 256; it++)
+		flat_unit((size_t)block * kActUnits + it * 256 + threadIdx.x, n, a.opacity, a.opacities,
+		          [](float v, size_t) { return 1.0f / (1.0f + expf(-v)); });
+}
+
+__global__ __launch_bounds__(256) void activate_backward_kernel(ActivateBackwardArgs a, ActParts parts)
+{
+	uint32_t block = blockIdx.x;
+	const size_t n = (size_t)a.n;
+	if (block < parts.sh_blocks) {
+		if (!a.g_shs)
+			return;
+		const size_t sh_floats = 3 * (size_t)(1 + a.rest), rest_floats = 3 * (size_t)a.rest, total = n * sh_floats;
+		for (int it = 0; it < kActUnits / 256; it++) {
+			const size_t u = (size_t)block * kActUnits + it * 256 + threadIdx.x;
+			if (4 * u >= total)
+				break;
+			float v[4] = {0.f, 0.f, 0.f, 0.f};
+			if (4 * u + 4 <= total) {
+				const float4 g = reinterpret_cast<const float4*>(a.g_shs)[u];
+				v[0] = g.x; v[1] = g.y; v[2] = g.z; v[3] = g.w;
+			} else {
+				for (size_t k = 4 * u; k < total; k++)
+					v[k - 4 * u] = a.g_shs[k];
+			}
+#pragma unroll
+			for (int k = 0; k < 4; k++) {
+				const size_t at = 4 * u + k;
+				if (at < total) {
+					const size_t row = at / sh_floats, col = at - row * sh_floats;
+					if (col < 3)
+						a.d_features_dc[3 * row + col] = v[k];
+					else
+						a.d_features_rest[rest_floats * row + (col - 3)] = v[k];
+				}
+			}
+		}
+		return;
+	}
+	block -= parts.sh_blocks;
+	if (block < parts.rot_blocks) {
+		if (!a.g_rotations)
+			return;
+		for (int it = 0; it < kActUnits / 256; it++) {
+			const size_t i = (size_t)block * kActUnits + it * 256 + threadIdx.x;
+			if (i >= n)
+				break;
+			// d/dq of q / |q|: (g - u (u . g)) / |q| with u = q / |q|
+			const float4 q = reinterpret_cast<const float4*>(a.rotation)[i];
+			const float4 g = reinterpret_cast<const float4*>(a.g_rotations)[i];
+			const float len = fmaxf(sqrtf(q.x * q.x + q.y * q.y + q.z * q.z + q.w * q.w), 1e-12f);
+			const float u0 = q.x / len, u1 = q.y / len, u2 = q.z / len, u3 = q.w / len;
+			const float along = u0 * g.x + u1 * g.y + u2 * g.z + u3 * g.w;
+			reinterpret_cast<float4*>(a.d_rotation)[i] =
+			    float4{(g.x - u0 * along) / len, (g.y - u1 * along) / len, (g.z - u2 * along) / len, (g.w - u3 * along) / len};
+		}
+		return;
+	}
+	block -= parts.rot_blocks;
+	if (block < parts.scale_blocks) {
+		if (!a.g_scales)
+			return;
+		const float* scales = a.scales;
+		for (int it = 0; it < kActUnits / 256; it++)
+			flat_unit((size_t)block * kActUnits + it * 256 + threadIdx.x, 3 * n, a.g_scales, a.d_scaling,
+			          [scales](float g, size_t k) { return g * scales[k]; });
+		return;
+	}
+	block -= parts.scale_blocks;
+	if (!a.g_opacities)
+		return;
+	const float* opacities = a.opacities;
+	for (int it = 0; it < kActUnits / 256; it++)
+		flat_unit((size_t)block * kActUnits + it * 256 + threadIdx.x, n, a.g_opacities, a.d_opacity, [opacities](float g, size_t k) {
+			const float o = opacities[k];
+			return g * (o * (1.0f - o));
+		});
+}
+
 }  // namespace
+
+void launch_activate_forward(const ActivateArgs& a, hipStream_t s)
+{
+	stage_mark("activate_forward", s);
+	if (a.n <= 0)
+		return;
+	const ActParts p = act_parts(a.n, a.rest);
+	hipLaunchKernelGGL(activate_forward_kernel, dim3(p.sh_blocks + p.rot_blocks + p.scale_blocks + p.opacity_blocks), dim3(256),
+	                   0, s, a, p);
+}
+
+void launch_activate_backward(const ActivateBackwardArgs& a, hipStream_t s)
+{
+	stage_mark("activate_backward", s);
+	if (a.n <= 0)
+		return;
+	const ActParts p = act_parts(a.n, a.rest);
+	hipLaunchKernelGGL(activate_backward_kernel, dim3(p.sh_blocks + p.rot_blocks + p.scale_blocks + p.opacity_blocks), dim3(256),
+	                   0, s, a, p);
+}
 
 uint32_t loss_blocks(int C, int H, int W)
 {

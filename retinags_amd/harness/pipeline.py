@@ -313,3 +313,98 @@ def training_iteration(models: List["SharedGSInfo"], optimisers, part: Partition
         opt.step()
         opt.zero_grad(set_to_none=True)
     return {"loss": loss.detach(), "l1": l1, "frame": frame, "lent_rows": int(table.counts.sum())}
+
+
+@dataclass
+class StoredModel:
+    """A submodel's trainable tensors as the reference stores them (scene/gaussian_nn_module.py:420-426):
+    positions, first and remaining SH coefficients, log scales, quaternions, opacity logits, and the
+    (N,1) placeholder whose gradient densification reads."""
+    xyz: torch.Tensor
+    features_dc: torch.Tensor
+    features_rest: torch.Tensor
+    scaling: torch.Tensor
+    rotation: torch.Tensor
+    opacity: torch.Tensor
+    means2D_meta: torch.Tensor
+    spare_rows: int = 0
+
+    def parameters(self) -> List[torch.Tensor]:
+        return [self.xyz, self.features_dc, self.features_rest, self.opacity, self.means2D_meta, self.scaling, self.rotation]
+
+    def activated(self) -> "SharedGSInfo":
+        """get_xyz, get_opacity, get_scaling, get_rotation, get_features and the means2D placeholder
+        (parallel_utils/basic_parallel_trainer/result_aggregator.py:40-52)."""
+        from ..activation import activate_gaussians
+        means2D = gradNormHelpFunction(self.means2D_meta)
+        if self.spare_rows:
+            means2D = _RoomBehind.apply(means2D, self.spare_rows)
+        return activate_gaussians(self.xyz, self.features_dc, self.features_rest, self.scaling, self.rotation,
+                                  self.opacity, means2D=means2D, spare_rows=self.spare_rows)
+
+
+class _RoomBehind(torch.autograd.Function):
+    """Identity that moves a tensor to the start of an allocation with spare rows behind it."""
+
+    @staticmethod
+    def forward(ctx, t: torch.Tensor, spare: int) -> torch.Tensor:
+        from ..sharing import with_spare_rows
+        return with_spare_rows(t, spare).detach()
+
+    @staticmethod
+    def backward(ctx, g: torch.Tensor):
+        return g, None
+
+
+def stored_models_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device,
+                                 spare_fraction: float = 0.0) -> List[StoredModel]:
+    """Every submodel's own Gaussians in stored form: log of the scene's scales, logit of its
+    opacities, its SH coefficients split into the first and the rest."""
+    from ..sharing import with_spare_rows
+    out = []
+    for k in range(len(part.leaves)):
+        idx = torch.from_numpy(np.nonzero(part.owner == k)[0])
+        spare = int(len(idx) * spare_fraction) + 4096 if spare_fraction > 0 else 0
+        pick = lambda t: t[idx].to(device).contiguous()
+        opacity = pick(scene["opacity"]).clamp(1e-6, 1 - 1e-6)
+        shs = pick(scene["shs"])
+        out.append(StoredModel(
+            xyz=with_spare_rows(pick(scene["xyz"]), spare), features_dc=shs[:, :1].contiguous(),
+            features_rest=shs[:, 1:].contiguous(), scaling=torch.log(pick(scene["scales"])), rotation=pick(scene["rotations"]),
+            opacity=torch.log(opacity / (1 - opacity)), means2D_meta=torch.zeros(len(idx), 1, device=device),
+            spare_rows=spare))
+    return out
+
+
+def make_stored_optimisers(models: List[StoredModel], scale: float = 1.0):
+    """The reference's seven parameter groups per submodel (scene/gaussian_nn_module.py:433-443)."""
+    from ..optimizer import Adam
+    lr = REFERENCE_LEARNING_RATES
+    out = []
+    for m in models:
+        groups = [(m.xyz, lr["means3D"], "xyz"), (m.features_dc, lr["shs"], "f_dc"), (m.features_rest, lr["shs"] / 20.0, "f_rest"),
+                  (m.opacity, lr["opacity"], "opacity"), (m.means2D_meta, 0.0, "means2D_meta"), (m.scaling, lr["scales"], "scaling"),
+                  (m.rotation, lr["rotations"], "rotation")]
+        out.append(Adam([{"params": [p], "lr": r * scale, "name": n} for p, r, n in groups], lr=0.0, eps=1e-15))
+    return out
+
+
+def stored_training_iteration(models: List[StoredModel], optimisers, part: Partition, cam: Camera, relation: np.ndarray,
+                              gt_image: torch.Tensor, background: torch.Tensor, lambda_dssim: float = 0.2,
+                              streams: Optional[List["torch.cuda.Stream"]] = None) -> dict:
+    """training_iteration from the stored parameters: activation first, and its backward last, so the
+    optimisers step what the reference's step (log scales, opacity logits, raw quaternions, split
+    SH coefficients).  Lent rows are appended when the models were made with spare rows."""
+    from ..loss import l1_ssim_loss
+    from ..sharing import merge_shared, select_straddlers
+    device = models[0].xyz.device
+    shown = [m.activated() for m in models]
+    table = select_straddlers(shown, part.box_low, part.box_up)
+    merged = merge_shared(shown, table, reuse_gradients=True, append=all(m.spare_rows > 0 for m in models))
+    frame = render_frame(cam, submodels_from_shared(merged, part, device), relation, background, streams=streams)
+    loss, l1 = l1_ssim_loss(frame["render"], gt_image, lambda_dssim)
+    loss.backward()
+    for opt in optimisers:
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    return {"loss": loss.detach(), "l1": l1, "frame": frame, "lent_rows": int(table.counts.sum())}

@@ -103,3 +103,50 @@ def test_the_loss_goes_down(append):
         assert step["lent_rows"] > 0
     assert all(np.isfinite(losses)) and losses[-1] < 0.8 * losses[0], losses
     assert all(opt.state[p]["step"] == 12 for opt in optimisers for g in opt.param_groups for p in g["params"])
+
+
+@pytest.mark.parametrize("spare", [0.0, 0.3])
+def test_the_loss_goes_down_from_stored_parameters(spare):
+    """The same loop from the parameters as the reference stores them (log scales, opacity logits, split SH
+    coefficients) through the activation kernels; the screen-space gradient reaches the (N,1) placeholder."""
+    from retinags_amd.harness import partition, pipeline
+    scene, cam, _ = scenes.make_config("C1", shrink=150, resolution_scale=0.25)
+    scene["scales"] = scene["scales"] * 2.0
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    rel = partition.relation_vector(part, cam)
+    cam_d = cam.to(DEV)
+    bg = torch.zeros(3, device=DEV)
+    with torch.no_grad():
+        target = pipeline.render_frame(cam_d, pipeline.submodels_from_partition(scene, part, DEV), rel, bg)["render"].clone()
+    models = pipeline.stored_models_from_partition(scene, part, DEV, spare)
+    # stored form and activation are inverse to each other: the untouched models render the target
+    with torch.no_grad():
+        shown = [m.activated() for m in models]
+        from retinags_amd import sharing
+        table = sharing.select_straddlers(shown, part.box_low, part.box_up)
+        merged = sharing.merge_shared(shown, table, append=spare > 0)
+        again = pipeline.render_frame(cam_d, pipeline.submodels_from_shared(merged, part, DEV), rel, bg)["render"]
+        assert float((again - target).abs().max()) < 2e-3
+        gen = torch.Generator().manual_seed(3)
+        for m in models:
+            m.features_dc.add_((torch.randn(m.features_dc.shape, generator=gen) * 0.1).to(DEV))
+            m.opacity.sub_(0.5)
+    for m in models:
+        for t in m.parameters():
+            t.requires_grad_(True)
+    optimisers = pipeline.make_stored_optimisers(models)
+    streams = [torch.cuda.current_stream(DEV)] + [torch.cuda.Stream(device=DEV) for _ in range(3)]
+    losses, seen_meta_grad = [], False
+    for it in range(12):
+        if it == 11:      # look at the gradients of the last iteration before the step clears them
+            for opt in optimisers:
+                opt.zero_grad = lambda set_to_none=True: None
+        step = pipeline.stored_training_iteration(models, optimisers, part, cam_d, rel, target, bg, streams=streams)
+        losses.append(float(step["loss"]))
+    assert all(np.isfinite(losses)) and losses[-1] < 0.8 * losses[0], losses
+    for m in models:
+        g = m.means2D_meta.grad
+        assert g is not None and g.shape == m.means2D_meta.shape and float(g.min()) >= 0.0
+        seen_meta_grad = seen_meta_grad or float(g.max()) > 0.0
+        assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+    assert seen_meta_grad

@@ -153,3 +153,40 @@ def test_golden_vectors_of_the_neighbouring_steps():
     for k, p in enumerate(ps):
         assert rel_l2(p.detach().cpu().numpy(), z[f"adam/after{k}"]) < 1e-6
         assert rel_l2(opt.state[p]["exp_avg_sq"].cpu().numpy(), z[f"adam/exp_avg_sq{k}"]) < 1e-6
+
+
+def test_activation_and_its_backward_against_the_tensor_expressions():
+    """rgs_activate_forward / rgs_activate_backward against exp, sigmoid, normalize and cat with autograd
+    (scene/gaussian_nn_module.py:373-394), incl. a zero quaternion, rows behind for appending, and
+    outputs without a gradient."""
+    from retinags_amd.activation import activate_gaussians
+    rng = np.random.default_rng(14)
+    for n, rest, spare in ((1003, 15, 0), (257, 15, 64), (64, 0, 8), (5, 8, 0)):
+        dc = rng.normal(size=(n, 1, 3)).astype(np.float32)
+        fr = rng.normal(size=(n, rest, 3)).astype(np.float32)
+        sc = rng.normal(-4, 1, size=(n, 3)).astype(np.float32)
+        rot = rng.normal(size=(n, 4)).astype(np.float32)
+        rot[0] = 0.0                                   # normalize leaves a zero vector at zero
+        op = rng.normal(0, 2, size=(n, 1)).astype(np.float32)
+        g = [rng.normal(size=s).astype(np.float32) for s in ((n, 1 + rest, 3), (n, 3), (n, 4), (n, 1))]
+        want, want_grads = to.activate_reference(dc, fr, sc, rot, op, g)
+        leaves = [torch.tensor(a, device=DEV, requires_grad=True) for a in (dc, fr, sc, rot, op)]
+        xyz = torch.zeros(n, 3, device=DEV)
+        info = activate_gaussians(xyz, *leaves, spare_rows=spare)
+        got = [info.shs, info.scales, info.rotations, info.opacity]
+        assert info.means3D is xyz and float(info.means2D.abs().sum()) == 0.0
+        assert np.array_equal(got[0].detach().cpu().numpy(), want[0])
+        for a, b in zip(got[1:], want[1:]):
+            assert np.abs(a.detach().cpu().numpy() - b).max() <= 2e-6 * max(1.0, np.abs(b).max())
+        if spare:
+            assert all(t.untyped_storage().nbytes() >= (n + spare) * t[0].numel() * 4 for t in got)
+        torch.autograd.backward(got, [torch.tensor(x, device=DEV) for x in g])
+        for leaf, w in zip(leaves, want_grads):
+            assert rel_l2(leaf.grad.cpu().numpy()[1:], w[1:]) < 1e-5      # row 0: the zero quaternion
+        assert torch.isfinite(leaves[3].grad[0]).all()
+    # only some outputs take part in the loss
+    leaves = [torch.tensor(a, device=DEV, requires_grad=True) for a in (dc, fr, sc, rot, op)]
+    info = activate_gaussians(torch.zeros(n, 3, device=DEV), *leaves)
+    info.scales.sum().backward()
+    assert leaves[0].grad is None and leaves[3].grad is None
+    assert torch.allclose(leaves[2].grad, torch.exp(leaves[2].detach()), rtol=1e-5)
