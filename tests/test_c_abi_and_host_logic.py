@@ -218,4 +218,12 @@ def test_entry_points_refuse_bad_arguments_before_touching_the_gpu():
     t[0].n, t[0].step = 0, 0
     refused(lib.rgs_adam_step(1, t, 0.9, 0.999, 1e-8, null), "step")
     assert lib.rgs_adam_step(0, None, 0.9, 0.999, 1e-8, null) == 0
+    refused(lib.rgs_activate_forward(-1, 15, *([null] * 10)), "bad sizes")
+    refused(lib.rgs_activate_forward(8, 15, *([null] * 10)), "null pointer")
+    odd = C.c_void_p(0x1004)
+    even = C.c_void_p(0x1000)
+    refused(lib.rgs_activate_forward(8, 15, even, even, odd, even, even, even, even, even, even, null), "16 bytes")
+    refused(lib.rgs_activate_backward(8, 15, null, null, null, even, null, null, null, null, null, null, null, null, null),
+            "no room for the SH gradients")
+    assert lib.rgs_activate_forward(0, 15, *([null] * 10)) == 0 and lib.rgs_activate_backward(0, 15, *([null] * 13)) == 0
     assert lib.rgs_straddler_scratch_bytes(-1, 4) == 0 and lib.rgs_straddler_scratch_bytes(1025, 3) == 4 * 3 * 3
