@@ -131,7 +131,7 @@ def test_garden_odd_resolution():
     _check_forward_stages(_scene_sub(scene), cam, torch.tensor([1.0, 1.0, 1.0]))
 
 
-def _check_backward(sub, cam, bg, seed, with_depth_alpha):
+def _check_backward(sub, cam, bg, seed, with_depth_alpha, sh_degree=3, scale_modifier=1.0):
     from retinags_amd import GaussianRasterizationSettings, GaussianRasterizer
     dev = torch.device("cuda:0")
     H, W = cam.image_height, cam.image_width
@@ -140,7 +140,7 @@ def _check_backward(sub, cam, bg, seed, with_depth_alpha):
     g_depth = torch.randn(1, H, W, generator=gen) * 1e-2 if with_depth_alpha else None
     g_alpha = torch.randn(1, H, W, generator=gen) * 1e-2 if with_depth_alpha else None
 
-    s = oracle_settings(cam, sub["low"], sub["up"], bg)
+    s = oracle_settings(cam, sub["low"], sub["up"], bg, sh_degree, scale_modifier)
     st = orc.forward(s, np32(sub["xyz"]), np32(sub["opacity"]), shs=np32(sub["shs"]), scales=np32(sub["scales"]),
                      rotations=np32(sub["rotations"]))
     want = orc.backward(s, st, np32(g_color), None if g_depth is None else np32(g_depth),
@@ -149,10 +149,11 @@ def _check_backward(sub, cam, bg, seed, with_depth_alpha):
     leaf = {k: sub[k].to(dev).clone().requires_grad_(True) for k in ("xyz", "opacity", "scales", "rotations", "shs")}
     means2D = torch.zeros_like(leaf["xyz"], requires_grad=True)
     settings = GaussianRasterizationSettings(
-        image_height=H, image_width=W, tanfovx=cam.tanfovx, tanfovy=cam.tanfovy, bg=bg.to(dev), scale_modifier=1.0,
+        image_height=H, image_width=W, tanfovx=cam.tanfovx, tanfovy=cam.tanfovy, bg=bg.to(dev),
+        scale_modifier=scale_modifier,
         viewmatrix=cam.world_view_transform.to(dev), projmatrix=cam.full_proj_transform.to(dev),
         projmatrix_inv=cam.projection_matrix_inv.to(dev), range_low=sub["low"].to(dev), range_up=sub["up"].to(dev),
-        sh_degree=3, campos=cam.camera_center.to(dev), prefiltered=False, debug=False)
+        sh_degree=sh_degree, campos=cam.camera_center.to(dev), prefiltered=False, debug=False)
     color, radii, depth, alpha = GaussianRasterizer(settings)(
         means3D=leaf["xyz"], means2D=means2D, opacities=leaf["opacity"], shs=leaf["shs"], scales=leaf["scales"],
         rotations=leaf["rotations"])
@@ -186,3 +187,15 @@ def test_cube_backward_all_outputs_with_background_and_box():
 def test_garden_backward():
     scene, cam, _ = scenes.make_config("C1", shrink=400, resolution_scale=0.2)
     _check_backward(_scene_sub(scene), cam, torch.zeros(3), seed=9, with_depth_alpha=True)
+
+
+@pytest.mark.parametrize("degree,stored", [(0, 16), (1, 16), (2, 16), (1, 4), (0, 1), (2, 9)])
+def test_backward_at_lower_sh_degrees_and_fewer_stored_coefficients(degree, stored):
+    """The active SH degree may be below 3 (the reference raises it during training,
+    scene/gaussian_nn_module.py:399-401) and the SH tensor may hold fewer than 16 coefficients
+    (M = sh.size(1), K/rasterize_points.cu:85-89); coefficients beyond the active degree get no gradient."""
+    scene, cam, _ = scenes.make_config("C0", shrink=40, resolution_scale=0.4)
+    sub = _scene_sub(scene)
+    sub["shs"] = sub["shs"][:, :stored].contiguous()
+    _check_backward(sub, cam, torch.tensor([0.1, 0.2, 0.3]), seed=10 + degree, with_depth_alpha=True, sh_degree=degree,
+                    scale_modifier=0.8)
