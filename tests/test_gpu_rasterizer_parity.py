@@ -199,3 +199,14 @@ def test_backward_at_lower_sh_degrees_and_fewer_stored_coefficients(degree, stor
     sub["shs"] = sub["shs"][:, :stored].contiguous()
     _check_backward(sub, cam, torch.tensor([0.1, 0.2, 0.3]), seed=10 + degree, with_depth_alpha=True, sh_degree=degree,
                     scale_modifier=0.8)
+
+
+@pytest.mark.parametrize("width,height,n", [(9, 7, 50), (16, 16, 1), (17, 33, 300), (1, 1, 20), (130, 5, 200)])
+def test_tiny_images_and_few_gaussians(width, height, n):
+    """One tile, one pixel, one Gaussian, a strip of tiles: every stage and every gradient as at full size."""
+    scene = scenes.cube_scene(n, seed=width * 100 + height)
+    scene["scales"] = scene["scales"] * 6.0      # wide enough to be seen at these sizes
+    cam = scenes.look_at_camera((0.0, 0.0, 0.0), (0.0, 0.0, 4.0), (0, -1, 0), width, height, 60.0)
+    sub = _scene_sub(scene)
+    _check_forward_stages(sub, cam, torch.tensor([0.2, 0.1, 0.05]))
+    _check_backward(sub, cam, torch.tensor([0.2, 0.1, 0.05]), seed=3, with_depth_alpha=True)
