@@ -51,6 +51,8 @@ def parse():
     ap.add_argument("--shrink", type=float, default=1.0, help="divide the Gaussian count (debugging only)")
     ap.add_argument("--resolution-scale", type=float, default=1.0, help="scale the image size (debugging only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--forward-only", action="store_true",
+                    help="render and composite only (the ms/frame figure; ms_per_step is then the render time)")
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--streams", type=int, default=4,
                     help="render the submodels of a frame on this many HIP streams (0: all on the current stream)")
@@ -101,7 +103,7 @@ def main():
         members = [np.arange(scene["xyz"].shape[0])]
     cam_d = cam.to(dev)
     H, W = cam.image_height, cam.image_width
-    do_backward = bool(cfg["backward"])
+    do_backward = bool(cfg["backward"]) and not args.forward_only
     if do_backward:
         for s in subs:
             s.requires_grad_(True)
@@ -290,8 +292,8 @@ def main():
         cpu = cpu_baseline(scene, members, part, cam, rel, related, upstream.cpu().numpy(), do_backward, args)
 
     line = {
-        "metric": "fwd+bwd iterations/s, 5.6M Gaussians, 1600x1036, 4 composited submodels" if args.config == "C1"
-        else f"fwd{'+bwd' if do_backward else ''} iterations/s, config {args.config}",
+        "metric": "fwd+bwd iterations/s, 5.6M Gaussians, 1600x1036, 4 composited submodels"
+        if (args.config == "C1" and do_backward) else f"fwd{'+bwd' if do_backward else ''} iterations/s, config {args.config}",
         "value": round(args.steps / elapsed, 4), "unit": "it/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
