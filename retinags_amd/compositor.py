@@ -61,9 +61,12 @@ class _CompositePartialImages(torch.autograd.Function):
         g_image = torch.zeros((3, H, W), **f32) if g_image is None else _prep(g_image, device, (3, H, W))
         g_depth = None if g_depth is None else _prep(g_depth, device, (1, H, W))
         g_alpha = None if g_alpha is None else _prep(g_alpha, device, (1, H, W))
-        d_images = [torch.empty((3, H, W), **f32) for _ in range(K)]
-        d_depths = [torch.empty((1, H, W), **f32) for _ in range(K)]
-        d_alphas = [torch.empty((1, H, W), **f32) for _ in range(K)]
+        # a layer's three gradients in one (5,H,W) block, the layout of RenderResult.zip_grad
+        # (parallel_utils/basic_parallel_trainer/task_utils.py:187-195)
+        blocks = [torch.empty((5, H, W), **f32) for _ in range(K)]
+        d_images = [b[0:3] for b in blocks]
+        d_depths = [b[3:4] for b in blocks]
+        d_alphas = [b[4:5] for b in blocks]
         with torch.cuda.device(device):
             check(lib.rgs_composite_backward(
                 K, H, W, ptr_table(images), ptr_table(depths), ptr_table(alphas), ptr(bg), ptr(g_image), ptr(g_depth),
@@ -112,3 +115,26 @@ def blender_render_result(render_results: Dict[int, dict], relation_vector, back
     image, depth, alpha = composite_partial_images([p["render"] for p in pk], [p["depth"] for p in pk],
                                                    [p["alpha"] for p in pk], bkg)
     return {"render": image, "depth": depth, "alpha": alpha}
+
+
+def partial_image_package(render: torch.Tensor, depth: torch.Tensor, alpha: torch.Tensor) -> torch.Tensor:
+    """The (5,H,W) tensor in which the reference ships a partial image or its gradient between ranks
+    (RenderResult.zip_content / zip_grad, parallel_utils/basic_parallel_trainer/task_utils.py:156-163,
+    187-195): colour, depth, alpha stacked.  The rasterizer and the compositor's backward of this
+    package already write the three into one such block, so this returns that block itself when it is
+    given them (no copy), and concatenates otherwise."""
+    base = render._base
+    if (base is not None and depth._base is base and alpha._base is base and tuple(base.shape) == (5,) + tuple(render.shape[1:])
+            and base.is_contiguous() and render.data_ptr() == base.data_ptr()
+            and depth.data_ptr() == base[3:4].data_ptr() and alpha.data_ptr() == base[4:5].data_ptr()):
+        return base.detach()
+    with torch.no_grad():
+        return torch.cat([render, depth, alpha], dim=0).to(dtype=torch.float32)
+
+
+def unpack_partial_image(package: torch.Tensor):
+    """Views of a (5,H,W) package: colour (3,H,W), depth (1,H,W), alpha (1,H,W)
+    (RenderResult.unzip_content / unzip_grad, task_utils.py:176-185, 206-214, without the copies)."""
+    if package.dim() != 3 or package.shape[0] != 5:
+        raise RuntimeError("a partial-image package has shape (5, H, W)")
+    return package[0:3], package[3:4], package[4:5]

@@ -186,9 +186,11 @@ def _forward_blend(st: GeometryStage):
     byte = dict(dtype=torch.uint8, device=device)
     if torch.cuda.current_stream(device).cuda_stream != st.stream:
         raise RuntimeError("the geometry stage was enqueued on another stream than the one current now")
-    out_color = torch.empty((3, H, W), **f32)
-    out_depth = torch.empty((1, H, W), **f32)
-    out_alpha = torch.empty((1, H, W), **f32)
+    # One (5,H,W) block: colour, depth, accumulated alpha in the order in which the reference packs a
+    # partial image for transport (RenderResult.zip_content,
+    # parallel_utils/basic_parallel_trainer/task_utils.py:156-163); see compositor.partial_image_package.
+    package = torch.empty((5, H, W), **f32)
+    out_color, out_depth, out_alpha = package[0:3], package[3:4], package[4:5]
     if P == 0:
         out_color.zero_(); out_depth.zero_(); out_alpha.zero_()
         empty = torch.empty(0, **byte)

@@ -336,3 +336,37 @@ def test_backward_clears_the_gradients_itself_when_the_caller_has_not():
     for a, b in zip(first, second):
         assert rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-4
         assert torch.equal((a == 0).all(dim=tuple(range(1, a.ndim))), (b == 0).all(dim=tuple(range(1, b.ndim))))
+
+
+def test_partial_images_and_their_gradients_come_packed_for_transport():
+    """Colour, depth and alpha of a submodel's render, and their gradients from the compositor, each sit in
+    one (5,H,W) block in the reference's wire order (task_utils.py:156-163, 187-195): packing is free."""
+    from retinags_amd import GaussianRasterizer
+    from retinags_amd.compositor import composite_partial_images, partial_image_package, unpack_partial_image
+    scene, cam, low, up = _small_inputs(n=3000, seed=5)
+    r = GaussianRasterizer(_settings(oracle_settings(cam, low, up, torch.zeros(3))))
+    xyz = scene["xyz"].to(DEV).requires_grad_(True)
+    color, radii, depth, alpha = r(means3D=xyz, means2D=torch.zeros_like(xyz), opacities=scene["opacity"].to(DEV),
+                                   shs=scene["shs"].to(DEV), scales=scene["scales"].to(DEV), rotations=scene["rotations"].to(DEV))
+    package = partial_image_package(color, depth, alpha)
+    assert package.shape == (5, cam.image_height, cam.image_width) and package.data_ptr() == color.data_ptr()
+    assert torch.equal(package, torch.cat([color, depth, alpha]).detach())
+    c, d, a = unpack_partial_image(package)
+    assert torch.equal(c, color.detach()) and torch.equal(d, depth.detach()) and torch.equal(a, alpha.detach())
+    # tensors that are not one block are concatenated
+    other = partial_image_package(color.detach().clone(), depth.detach().clone(), alpha.detach().clone())
+    assert torch.equal(other, package) and other.data_ptr() != package.data_ptr()
+    # gradients of a layer out of the compositor
+    # (as they leave the compositor's backward; a leaf's .grad is a copy that autograd makes of a view)
+    layers = [t.detach().clone().requires_grad_(True) for t in (color, depth, alpha)]
+    arrived = {}
+    for name, t in zip(("render", "depth", "alpha"), layers):
+        t.register_hook(lambda g, name=name: arrived.__setitem__(name, g))
+    image, dep, alp = composite_partial_images([layers[0]], [layers[1]], [layers[2]], torch.tensor([0.1, 0.2, 0.3], device=DEV))
+    (image.sum() + 2 * dep.sum() + 3 * alp.sum()).backward()
+    g = partial_image_package(arrived["render"], arrived["depth"], arrived["alpha"])
+    assert g.data_ptr() == arrived["render"].data_ptr() and g.shape[0] == 5
+    assert torch.equal(g[3:4], layers[1].grad) and torch.equal(g[0:3], layers[0].grad)
+    # the rasterizer's backward takes the views as they are
+    (color.sum() + depth.sum() + alpha.sum()).backward()
+    assert torch.isfinite(xyz.grad).all() and float(xyz.grad.abs().sum()) > 0
