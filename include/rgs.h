@@ -11,6 +11,19 @@
  * Functions return 0 on success; on failure they return non-zero and
  * rgs_last_error() gives the reason for the calling thread.
  *
+ * Limits: a call handles fewer than 2^30 (Gaussian, tile) instances (the radix sorts pack a
+ * count and two flag bits into one word); rgs_forward_geom reports a larger count as an error.
+ *
+ * A sort that gives up: the radix sorts wait for neighbouring workgroups with a bounded number
+ * of polls.  Should such a wait ever run out (never observed), every later kernel of that call
+ * still runs to its end inside its buffers, the call's tile lists are left empty (the images show
+ * the background only, the gradients are zero) and a word of pinned host memory is set, which
+ * rgs_forward_geom*, rgs_forward_raster*, rgs_backward and rgs_sort_fault look at when they are
+ * called: the next of these calls on that device then fails with a message that says so, without
+ * doing its work, and clears the report.  A caller that wants to know before its next call asks
+ * rgs_sort_fault, which waits for the stream first.  The reference's cub::DeviceRadixSort has no
+ * such state (K/cuda_rasterizer_hgs/rasterizer_impl.cu:312-317).
+ *
  * Citations name the interface of the reference that each entry point replaces,
  * with K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian.
  */
@@ -206,8 +219,9 @@ int rgs_stage_timing_read(int max_stages, const char** names, float* total_ms, i
  * re-walks every tile exactly like the forward blend and writes RGS_WORK_COUNTERS uint64 sums
  * to `counters` (device memory): [0] list entries visited by a live pixel, [1] of those with
  * power <= 0, [2] with alpha >= 1/255, [3] inside the submodel box, [4] blended; [5], [6] are
- * [1], [2] restricted to entries up to each pixel's last blended one (the backward's share). */
-#define RGS_WORK_COUNTERS 7
+ * [1], [2] restricted to entries up to each pixel's last blended one (the backward's share), and
+ * [7] is [0] restricted the same way. */
+#define RGS_WORK_COUNTERS 8
 int rgs_blend_work_counters(int P, int R, int width, int height, float tan_fovx, float tan_fovy,
                             const float* projmatrix_inv, const float* range_low, const float* range_up,
                             const float* colors_precomp, const void* geom_ws, const void* binning_ws,
@@ -226,6 +240,15 @@ int rgs_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, void* temp, v
 size_t rgs_sort_temp_bytes(size_t n);
 int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                    int end_bit, void* temp, void* stream);
+
+/* Waits for `stream`, then returns non-zero (and clears the report) if a sort of an earlier call on
+ * the current device gave up; see the note at the top. */
+int rgs_sort_fault(void* stream);
+
+/* Test hook: the number of polls a look-back of the sorts allows before it gives up (0 restores
+ * the default of 2^18; a negative value makes every look-back give up at once, which drives the
+ * give-up path from the host while every kernel still runs to its end).  Process-wide. */
+int rgs_set_lookback_spin_limit(int polls);
 
 /* ---- partial-image compositor ------------------------------------------------------------
  * Replaces the tensor expression in blender_render_result

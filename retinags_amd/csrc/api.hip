@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -82,6 +83,59 @@ struct EntryScope {
 	explicit EntryScope(hipStream_t stream) : s(stream) {}
 	~EntryScope() { timer_record(nullptr, s); }
 };
+
+// ---- sticky report of a sort that gave up ------------------------------------------------------
+// One word of pinned host memory per device, which the device can write: the kernel that reads the
+// sorts' status words sets it, and every rasterizer entry point looks at it (a plain host read) when
+// it is called, so a give-up surfaces as an error of the next call on that device without any
+// additional synchronisation.
+constexpr int kMaxDevices = 64;
+std::mutex g_device_mutex;
+uint32_t* g_fault_word[kMaxDevices] = {};
+
+int current_device()
+{
+	int dev = 0;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+		return -1;
+	return dev;
+}
+
+// The current device's word; allocated on first use unless `allocate` is false (then null if absent).
+uint32_t* fault_word(bool allocate)
+{
+	const int dev = current_device();
+	if (dev < 0)
+		return nullptr;
+	std::lock_guard<std::mutex> lock(g_device_mutex);
+	if (!g_fault_word[dev] && allocate) {
+		void* p = nullptr;
+		if (hipHostMalloc(&p, 64, hipHostMallocDefault) == hipSuccess && p) {
+			memset(p, 0, 64);
+			g_fault_word[dev] = static_cast<uint32_t*>(p);
+		} else {
+			(void)hipGetLastError();
+		}
+	}
+	return g_fault_word[dev];
+}
+
+// Non-zero (with the error set) if a sort of an earlier call on this device gave up; clears the report.
+int take_sort_fault(const char* who)
+{
+	uint32_t* w = fault_word(false);
+	if (!w || __atomic_load_n(w, __ATOMIC_RELAXED) == 0u)
+		return 0;
+	__atomic_store_n(w, 0u, __ATOMIC_RELAXED);
+	return fail("%s: a radix sort of an earlier call on this device gave up waiting for a neighbouring workgroup; "
+	            "that call left empty tile lists (background-only images, zero gradients) and must be repeated", who);
+}
+
+#define RGS_TAKE_SORT_FAULT(who)                   \
+	do {                                           \
+		if (int rc_ = take_sort_fault(who))        \
+			return rc_;                            \
+	} while (0)
 
 constexpr size_t kAlign = 256;
 
@@ -360,6 +414,7 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 	(void)prefiltered;
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
+	RGS_TAKE_SORT_FAULT(who);
 	RGS_REQUIRE(P > 0, "%s: P must be positive (the caller short-circuits P == 0)", who);
 	RGS_REQUIRE(width > 0 && height > 0, "%s: bad image size %dx%d", who, width, height);
 	RGS_REQUIRE(means3D && opacities && viewmatrix && projmatrix && cam_pos && radii && geom_ws && num_rendered_host,
@@ -483,6 +538,7 @@ int forward_raster(bool count_on_device, int P, int R, int width, int height,
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
+	RGS_TAKE_SORT_FAULT("rgs_forward_raster");
 	RGS_REQUIRE(P > 0 && R >= 0, "rgs_forward_raster: bad sizes P=%d R=%d", P, R);
 	RGS_REQUIRE(R < 0x40000000, "rgs_forward_raster: %d (Gaussian, tile) instances exceed the 2^30 limit of the sort", R);
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_raster: bad image size %dx%d", width, height);
@@ -534,11 +590,11 @@ int forward_raster(bool count_on_device, int P, int R, int width, int height,
 				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
 		}
 		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, count, ranges, gx * gy,
-		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, true, s);
+		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, fault_word(true), true, s);
 		RGS_STAGE("tile_ranges");
 		point_list = sorted_in_a ? vals_a : vals_b;
 	} else {
-		rgs::launch_tile_ranges(nullptr, 0, nullptr, ranges, gx * gy, nullptr, nullptr, false, s);
+		rgs::launch_tile_ranges(nullptr, 0, nullptr, ranges, gx * gy, nullptr, nullptr, nullptr, false, s);
 		RGS_STAGE("tile_ranges");
 	}
 
@@ -610,6 +666,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
+	RGS_TAKE_SORT_FAULT("rgs_backward");
 	RGS_REQUIRE(P > 0 && R >= 0, "rgs_backward: bad sizes P=%d R=%d", P, R);
 	RGS_REQUIRE(width > 0 && height > 0, "rgs_backward: bad image size %dx%d", width, height);
 	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
@@ -748,28 +805,51 @@ size_t rgs_sort_temp_bytes(size_t n)
 	return 4 * rgs::sort_temp_words(n);
 }
 
-int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                   int end_bit, void* temp, void* stream)
+static int sort_pairs_u64(const char* who, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
+                          size_t n, int end_bit, uint32_t* temp, uint32_t* fault, hipStream_t s)
 {
-	hipStream_t s = static_cast<hipStream_t>(stream);
-	EntryScope scope_(s);
 	const int debug = 0;
-	RGS_REQUIRE(end_bit >= 1 && end_bit <= 64, "rgs_sort_pairs: end_bit %d out of range", end_bit);
-	if (n == 0)
-		return 0;
-	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out && temp, "rgs_sort_pairs: null pointer");
-	RGS_REQUIRE(n < 0x40000000ull, "rgs_sort_pairs: 2^30 pairs or more");
-	rgs::launch_sort_pairs(keys_in, keys_out, vals_in, vals_out, n, end_bit, static_cast<uint32_t*>(temp), s);
+	rgs::launch_sort_pairs(keys_in, keys_out, vals_in, vals_out, n, end_bit, temp, s);
 	RGS_STAGE("sort_pairs");
+	rgs::launch_report_sort_status(temp, fault, s);
 	if ((((end_bit + 7) / 8) % 2) == 0) {
 		// An even number of passes leaves the result in the input buffers; hand it over.
 		hipError_t e = hipMemcpyAsync(keys_out, keys_in, n * sizeof(uint64_t), hipMemcpyDeviceToDevice, s);
 		if (e == hipSuccess)
 			e = hipMemcpyAsync(vals_out, vals_in, n * sizeof(uint32_t), hipMemcpyDeviceToDevice, s);
 		if (e != hipSuccess)
-			return fail("rgs_sort_pairs: copy failed: %s", hipGetErrorString(e));
+			return fail("%s: copy failed: %s", who, hipGetErrorString(e));
 	}
 	return 0;
+}
+
+int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                   int end_bit, void* temp, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	RGS_REQUIRE(end_bit >= 1 && end_bit <= 64, "rgs_sort_pairs: end_bit %d out of range", end_bit);
+	if (n == 0)
+		return 0;
+	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out && temp, "rgs_sort_pairs: null pointer");
+	RGS_REQUIRE(n < 0x40000000ull, "rgs_sort_pairs: 2^30 pairs or more");
+	return sort_pairs_u64("rgs_sort_pairs", keys_in, keys_out, vals_in, vals_out, n, end_bit, static_cast<uint32_t*>(temp),
+	                      fault_word(true), s);
+}
+
+int rgs_set_lookback_spin_limit(int polls)
+{
+	rgs::set_lookback_spin_limit(polls);
+	return 0;
+}
+
+int rgs_sort_fault(void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const hipError_t e = hipStreamSynchronize(s);
+	if (e != hipSuccess)
+		return fail("rgs_sort_fault: %s", hipGetErrorString(e));
+	return take_sort_fault("rgs_sort_fault");
 }
 
 static int fill_composite(rgs::CompositeArgs& a, int K, int height, int width, const float* const* images,

@@ -15,6 +15,8 @@
 // depth and break ties by Gaussian index (a Gaussian touches a tile at most once).
 #include "rgs_kernels.h"
 
+#include <atomic>
+
 namespace rgs {
 
 // ---- prefix sums ---------------------------------------------------------------------------
@@ -160,17 +162,19 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __
 }
 
 // out[k] = in[index[k]] for k below the count on the device, and the sum of every 256 of them
-// (the first level of the scan that follows).
+// (the first level of the scan that follows).  `in` has in_size entries; an index beyond it (only
+// possible in what a sort that gave up left behind) reads the last entry instead.
 __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ n_device,
                                                           const uint32_t* __restrict__ index,
-                                                          const uint32_t* __restrict__ in, uint32_t* __restrict__ out,
+                                                          const uint32_t* __restrict__ in, uint32_t in_size,
+                                                          uint32_t* __restrict__ out,
                                                           uint32_t* __restrict__ block_totals)
 {
 	__shared__ uint32_t lds[8];
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
 	uint32_t v = 0;
 	if (k < *n_device) {
-		v = in[index[k]];
+		v = in[min(index[k], in_size - 1u)];
 		out[k] = v;
 	}
 	uint32_t total;
@@ -186,7 +190,9 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restr
 // inclusive offsets, then the tile from the position inside that Gaussian's rectangle.  (With
 // one thread per Gaussian every store touched 64 different cache lines, and a Gaussian that
 // covers hundreds of tiles kept its wavefront busy alone.)
-__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t* __restrict__ visible_count,
+// `order` is the output of a sort: should that sort ever have given up, its entries may be anything, so
+// they are clamped to the P Gaussians there are (the tile ranges then stay empty and nothing reads the result).
+__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(uint32_t P, const uint32_t* __restrict__ visible_count,
                                                                    const uint32_t* __restrict__ order,
                                                                    const uint32_t* __restrict__ offsets,
                                                                    const float2* __restrict__ xy,
@@ -204,14 +210,14 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(const uint32_t
 	// the scratch of the sort that follows is cleared here, which saves a launch
 	for (size_t w = k; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;
-	const uint32_t n = *visible_count;
+	const uint32_t n = min(*visible_count, P);
 	const uint32_t k0 = k - (uint32_t)lane;  // the wavefront's first Gaussian
 	if (k0 >= n)
 		return;
 	const uint32_t run_begin = k0 == 0u ? 0u : offsets[k0 - 1];
 	uint32_t end = 0, origin = 0, width = 1, idx = 0;
 	if (k < n) {
-		idx = order[k];
+		idx = min(order[k], P - 1u);
 		end = offsets[k];
 		const float2 p = xy[idx];
 		const TileRect rc = tile_rect(p.x, p.y, radii[idx], gx, gy);
@@ -256,7 +262,7 @@ void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touche
 	// 4 passes: the sorted pairs end up in the first buffer pair again
 	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, true, nullptr, 0, nullptr,
 	                      s);
-	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched,
+	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched, (uint32_t)P,
 	                   tiles_in_order, scan_temp);
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan_temp, (size_t)nb,
 	                   visible_count, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr);
@@ -270,7 +276,7 @@ void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint
                                 size_t clear_words, hipStream_t s)
 {
 	stage_mark("duplicate_with_keys", s);
-	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, visible_count, order,
+	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, (uint32_t)P, visible_count, order,
 	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values, capacity, clear, clear_words);
 }
 
@@ -290,14 +296,22 @@ void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint
 //   [2056]         status: non-zero if a look-back ever gave up waiting (never expected)
 //   [kSortHeader + pass * 256 * tiles + tile * 256 + digit]  look-back words
 
-constexpr int kSortMaxPasses = 8;
 constexpr uint32_t kSortCounters = 2048;
 constexpr uint32_t kSortStatus = 2056;
-constexpr uint32_t kSortHeader = 2112;
 constexpr uint32_t kFlagAggregate = 1u << 30;  // word holds this tile's own digit count
 constexpr uint32_t kFlagInclusive = 2u << 30;  // word holds the count of this and all earlier tiles
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
 constexpr int kLookbackSpinLimit = 1 << 18;
+
+// How many times a look-back polls a word that has not been published yet before it gives up.
+// A negative value makes every look-back give up at once: the way a test drives the give-up
+// path from the host (every kernel still runs to its end).
+static std::atomic<int> g_lookback_spin_limit{kLookbackSpinLimit};
+
+void set_lookback_spin_limit(int polls)
+{
+	g_lookback_spin_limit.store(polls == 0 ? kLookbackSpinLimit : polls);
+}
 
 template <typename KeyT>
 __device__ __forceinline__ uint32_t digit_of(KeyT key, int shift, uint32_t mask)
@@ -346,7 +360,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restri
                                                              uint32_t mask, const uint32_t* __restrict__ digit_count,
                                                              uint32_t* __restrict__ lookback,
                                                              uint32_t* __restrict__ tile_counter,
-                                                             uint32_t* __restrict__ status)
+                                                             uint32_t* __restrict__ status, int spin_limit)
 {
 	__shared__ KeyT s_keys[kSortBlock];
 	__shared__ uint32_t s_vals[kSortBlock];
@@ -436,14 +450,14 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restri
 		} else {
 			__hip_atomic_store(my_word, count | kFlagAggregate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 			uint32_t t = tile;
-			bool gave_up = false;
-			while (true) {
+			bool gave_up = spin_limit < 0;
+			while (!gave_up) {
 				t--;
 				const uint32_t* word = lookback + (size_t)t * 256 + tid;
 				uint32_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 				for (int spins = 0; (v >> 30) == 0u; spins++) {
 					// give up after a bounded wait, or as soon as any other look-back has
-					if (spins >= kLookbackSpinLimit ||
+					if (spins >= spin_limit ||
 					    ((spins & 255) == 255 &&
 					     __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
 						gave_up = true;
@@ -501,8 +515,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restri
 
 size_t sort_temp_words(size_t n)
 {
-	const size_t tiles = (n + kSortBlock - 1) / kSortBlock;
-	return kSortHeader + (size_t)kSortMaxPasses * 256 * (tiles > 0 ? tiles : 1);
+	return sort_temp_words_for(n);
 }
 
 const uint32_t* sort_status_word(const uint32_t* temp)
@@ -543,7 +556,7 @@ static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_
 		hipLaunchKernelGGL(sort_onesweep_kernel<KeyT>, dim3(tiles), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, n_device, shift,
 		                   mask,
 		                   temp + p * 256, temp + kSortHeader + (size_t)p * 256 * tiles, temp + kSortCounters + p,
-		                   temp + kSortStatus);
+		                   temp + kSortStatus, g_lookback_spin_limit.load());
 		KeyT* tk = ksrc; ksrc = kdst; kdst = tk;
 		uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
 	}
@@ -580,19 +593,24 @@ void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 }
 
 // The status words (may be null) are those of the two sorts: if either reported a failure the
-// ranges stay empty, so no later stage walks an unsorted list.
+// ranges stay empty, so no later stage walks an unsorted list, and *fault (host memory that the
+// device can write, may be null) is set for the host to find.
 __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __restrict__ keys, size_t n,
                                                            const uint32_t* __restrict__ n_device,
                                                            uint2* __restrict__ ranges,
                                                            const uint32_t* __restrict__ sort_status,
-                                                           const uint32_t* __restrict__ order_status)
+                                                           const uint32_t* __restrict__ order_status,
+                                                           uint32_t* __restrict__ fault)
 {
 	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u)) {
+		if (idx == 0 && fault)
+			__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+		return;
+	}
 	if (n_device)
 		n = min(n, (size_t)*n_device);  // launched for an upper bound
 	if (idx >= n)
-		return;
-	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u))
 		return;
 	const uint32_t cur = keys[idx];
 	if (idx == 0) {
@@ -608,8 +626,21 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __rest
 		ranges[cur].y = (uint32_t)n;
 }
 
+__global__ void report_sort_status_kernel(const uint32_t* __restrict__ status, uint32_t* __restrict__ fault)
+{
+	if (threadIdx.x == 0 && *status != 0u)
+		__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_t s)
+{
+	if (fault)
+		hipLaunchKernelGGL(report_sort_status_kernel, dim3(1), dim3(64), 0, s, temp + kSortStatus, fault);
+}
+
 void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device, uint2* ranges, int tiles,
-                        const uint32_t* sort_status, const uint32_t* order_status, bool ranges_cleared, hipStream_t s)
+                        const uint32_t* sort_status, const uint32_t* order_status, uint32_t* fault, bool ranges_cleared,
+                        hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
 	if (!ranges_cleared)
@@ -617,7 +648,7 @@ void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device
 	if (n == 0)
 		return;
 	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, n_device,
-	                   ranges, sort_status, order_status);
+	                   ranges, sort_status, order_status, fault);
 }
 
 }  // namespace rgs

@@ -427,7 +427,7 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 
 // Work accounting: the reference loop taken literally, one list entry at a time with no
 // filter, counting over all pixels the entries visited by a live pixel (A), those with
-// power <= 0 (B), with alpha >= 1/255 (C), inside the box (D), blended (E), and B and C
+// power <= 0 (B), with alpha >= 1/255 (C), inside the box (D), blended (E), and B, C and A
 // restricted to entries up to each pixel's last blended one (the backward's share).
 __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 {
@@ -450,7 +450,7 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 
 	bool done = !inside;
 	float T = 1.0f;
-	uint32_t nA = 0, nB = 0, nC = 0, nD = 0, nE = 0, nB_last = 0, nC_last = 0;
+	uint32_t nA = 0, nB = 0, nC = 0, nD = 0, nE = 0, nA_last = 0, nB_last = 0, nC_last = 0;
 	for (int i = 0; i < rounds; i++, todo -= 256) {
 		__syncthreads();
 		const uint32_t src = range.x + (uint32_t)i * 256 + tid;
@@ -484,14 +484,15 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 				continue;
 			}
 			nE++;
+			nA_last = nA;
 			nB_last = nB;
 			nC_last = nC;
 			T = test_T;
 		}
 	}
-	const uint32_t c[7] = {nA, nB, nC, nD, nE, nB_last, nC_last};
+	const uint32_t c[8] = {nA, nB, nC, nD, nE, nB_last, nC_last, nA_last};
 #pragma unroll
-	for (int q = 0; q < 7; q++) {
+	for (int q = 0; q < 8; q++) {
 		const uint32_t tot = wave_inclusive_scan_u32(c[q]);
 		if (lane == 63)
 			atomicAdd(reinterpret_cast<unsigned long long*>(a.counters) + q, (unsigned long long)tot);

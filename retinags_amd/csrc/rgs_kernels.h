@@ -283,7 +283,13 @@ void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint
                                 int grid_y, uint32_t* keys, uint32_t* values, uint32_t capacity, uint32_t* clear,
                                 size_t clear_words, hipStream_t s);
 size_t sort_clear_words(size_t n, int end_bit);    // words of the sort scratch that must be zero before a sort
-size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs*
+constexpr int kSortMaxPasses = 8;                 // radix passes the scratch has room for (64-bit keys)
+constexpr uint32_t kSortHeader = 2112;            // words ahead of the look-back words: histograms, counters, status
+constexpr size_t sort_temp_words_for(size_t n)
+{
+	return kSortHeader + (size_t)kSortMaxPasses * 256 * ((n + kSortBlock - 1) / kSortBlock > 0 ? (n + kSortBlock - 1) / kSortBlock : 1);
+}
+size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs* (= sort_temp_words_for)
 // Stable LSD radix sort on key bits [0, end_bit), ceil(end_bit/8) passes that ping-pong between
 // the two buffer pairs starting in -> out: an odd pass count leaves the result in
 // keys_out/vals_out, an even one in keys_in/vals_in.
@@ -298,13 +304,20 @@ void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals
                            const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, uint32_t* also_clear,
                            size_t also_clear_words, const char* stage, hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
+// Polls a look-back allows before it gives up (0 restores the default; negative: give up at once,
+// which is how a test exercises the give-up path with every kernel still running to its end).
+void set_lookback_spin_limit(int polls);
+// Sets *fault (host memory the device can write; null: nothing is launched) if the sort that used `temp` gave up.
+void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_t s);
 // Either status word (may be null) being non-zero leaves every range empty.  Clears `ranges` and
 // the kRangeTailWords words behind it (the strip class counters of the blend).
 constexpr int kRangeTailWords = 512;
 // ranges_cleared: an earlier kernel has done that clearing.
 // With a non-null n_device the number of keys is min(n, *n_device) and the launch is sized for n.
+// A non-zero status also sets *fault (host memory the device can write, may be null).
 void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device, uint2* ranges, int tiles,
-                        const uint32_t* sort_status, const uint32_t* order_status, bool ranges_cleared, hipStream_t s);
+                        const uint32_t* sort_status, const uint32_t* order_status, uint32_t* fault, bool ranges_cleared,
+                        hipStream_t s);
 
 // blend.hip
 void launch_blend_forward(const BlendArgs& a, hipStream_t s);

@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import threading
 from typing import NamedTuple
 
 import torch
@@ -44,16 +45,19 @@ class GaussianRasterizationSettings(NamedTuple):
     debug: bool
 
 
-_pinned_words = {}
+_pinned_words = threading.local()
 
 
 def _pinned_word(device: torch.device) -> torch.Tensor:
-    """One pinned uint32 per device: the landing spot of the instance count."""
+    """One pinned uint32 per host thread and device: the landing spot of the instance count of a
+    call that waits for it.  The count is copied out before the call returns, so calls of one
+    thread can share the word; another thread has its own."""
+    words = _pinned_words.__dict__.setdefault("words", {})
     key = (device.type, device.index)
-    t = _pinned_words.get(key)
+    t = words.get(key)
     if t is None:
         t = torch.zeros(1, dtype=torch.int32).pin_memory()
-        _pinned_words[key] = t
+        words[key] = t
     return t
 
 
@@ -95,7 +99,7 @@ class GeometryStage:
             if self.event is not None:
                 self.event.synchronize()
                 self._instances = int(self.count.item())
-                _free_count_slots[(self.device.type, self.device.index)].append((self.count, self.event))
+                _free_count_slots.setdefault((self.device.type, self.device.index), []).append((self.count, self.event))
                 self.event = None
             else:
                 self._instances = int(self.count.item())
@@ -163,12 +167,15 @@ def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations,
                 float(tanfovx), float(tanfovy), int(bool(prefiltered)), ptr(st.radii), ptr(st.geomBuffer),
                 st.geom_bytes)
         if wait:
-            st.count = _pinned_word(device)
-            check(lib.rgs_forward_geom(*args, C.c_void_p(st.count.data_ptr()), C.c_void_p(st.stream),
+            word = _pinned_word(device)
+            check(lib.rgs_forward_geom(*args, C.c_void_p(word.data_ptr()), C.c_void_p(st.stream),
                                        int(bool(debug))))
+            st._instances = int(word.item())   # the call returned with the count in place
         else:
-            free = _free_count_slots.setdefault((device.type, device.index), [])
-            st.count, st.event = free.pop() if free else _new_count_slot(device)
+            try:   # list.pop is atomic: two threads never get the same slot
+                st.count, st.event = _free_count_slots.setdefault((device.type, device.index), []).pop()
+            except IndexError:
+                st.count, st.event = _new_count_slot(device)
             check(lib.rgs_forward_geom_enqueue(*args, C.c_void_p(st.count.data_ptr()),
                                                C.c_void_p(st.event.cuda_event), C.c_void_p(st.stream),
                                                int(bool(debug))))
@@ -223,18 +230,22 @@ def _rasterize_forward(*args):
 
 
 def _gradient_outputs(P, M, has_scales, device, make):
-    """The eight dense gradient tensors of K/rasterize_points.cu:165-174 and the backward's
-    scratch for the per-Gaussian sums, carved out of one allocation made with `make`
-    (torch.empty or torch.zeros: one fill instead of nine);
-    without scales the scale / rotation gradients are zeros in either case."""
+    """The eight dense gradient tensors of K/rasterize_points.cu:165-174, carved out of one
+    allocation made with `make` (torch.empty or torch.zeros: one fill instead of eight), and the
+    backward's scratch for the per-Gaussian sums in an allocation of its own, so that a gradient
+    the caller keeps (the means2D gradient, say, for densification statistics) does not hold on to
+    the scratch.  The eight do share one block: keeping any of them keeps all (about 280 bytes
+    per Gaussian with SH degree 3).  Without scales the scale / rotation gradients are zeros in
+    either case."""
     shapes = {"means2D": (P, 3), "opacity": (P, 1), "colors": (P, 3), "means3D": (P, 3), "cov3D": (P, 6),
-              "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4), "sums": (P, _capi.ACC_FLOATS)}
+              "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4)}
     sizes = {k: (math.prod(v) + 63) // 64 * 64 for k, v in shapes.items()}  # 256-byte aligned parts
     flat = make((sum(sizes.values()),), dtype=torch.float32, device=device)
     out, at = {}, 0
     for k, shape in shapes.items():
         out[k] = flat[at:at + math.prod(shape)].view(shape)
         at += sizes[k]
+    out["sums"] = make((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
     if not has_scales and make is not torch.zeros:
         out["scales"].zero_()
         out["rotations"].zero_()

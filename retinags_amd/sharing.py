@@ -211,7 +211,10 @@ def merge_shared(models: Sequence[SharedGSInfo], table: StraddlerTable, reuse_gr
     the memory right behind them and return tensors over both.  Every field of every submodel
     must then sit in an allocation with that much room behind its rows (with_spare_rows makes
     such tensors); the merged tensors alias the submodel's own, and the room behind is
-    overwritten by every merge.
+    overwritten by every merge.  Autograd does not know of that aliasing (the merged tensors are
+    built over the inputs' storage, so the inputs' version counters do not guard them): the
+    inputs must not be updated in place, and no other merge may run, between this call and the
+    backward of everything that was rendered from its result.
 
     reuse_gradients: the backward returns the incoming gradient buffers of the merged arrays,
     with the borrowers' rows added in place, instead of copies.  Only for callers that do not

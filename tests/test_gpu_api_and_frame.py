@@ -370,3 +370,41 @@ def test_partial_images_and_their_gradients_come_packed_for_transport():
     # the rasterizer's backward takes the views as they are
     (color.sum() + depth.sum() + alpha.sum()).backward()
     assert torch.isfinite(xyz.grad).all() and float(xyz.grad.abs().sum()) > 0
+
+
+def test_a_sort_that_gives_up_is_reported_by_the_next_call():
+    """The radix sorts wait for neighbouring workgroups with a bounded number of polls.  With the limit
+    set below zero from the host every such wait gives up at once (every kernel still runs to its end):
+    the forward must then leave a background-only image, stay inside its buffers, and the next call
+    into the library on this device must fail with a message that says so; after that, and with the
+    limit restored, the same forward is correct again."""
+    import ctypes as C
+    from retinags_amd import _capi, GaussianRasterizer
+    scene, cam, low, up = _small_inputs(n=30000)
+    cam_d = cam.to(DEV)
+    s = oracle_settings(cam, low, up, torch.tensor([0.2, 0.4, 0.6]))
+    settings = _settings(s)
+    args = dict(means3D=scene["xyz"].to(DEV), means2D=torch.zeros(scene["xyz"].shape[0], 3, device=DEV),
+                opacities=scene["opacity"].to(DEV), shs=scene["shs"].to(DEV), scales=scene["scales"].to(DEV),
+                rotations=scene["rotations"].to(DEV))
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    good, radii, _, _ = GaussianRasterizer(settings)(**args)
+    torch.cuda.synchronize()
+    assert _capi.lib.rgs_sort_fault(stream) == 0
+    assert int((radii > 0).sum()) > 8192      # more than one block of the depth sort, so a look-back happens
+    try:
+        _capi.check(_capi.lib.rgs_set_lookback_spin_limit(-1))
+        color, radii2, depth, alpha = GaussianRasterizer(settings)(**args)
+        torch.cuda.synchronize()
+    finally:
+        _capi.check(_capi.lib.rgs_set_lookback_spin_limit(0))
+    assert torch.equal(radii, radii2)                        # the geometry stage does not depend on the sorts
+    assert float(alpha.abs().max()) == 0.0                   # empty tile lists: nothing was blended
+    assert torch.allclose(color, torch.tensor([0.2, 0.4, 0.6], device=DEV).view(3, 1, 1).expand_as(color))
+    with pytest.raises(_capi.RgsError, match="gave up"):
+        GaussianRasterizer(settings)(**args)                 # the report surfaces here, and is cleared
+    assert _capi.lib.rgs_sort_fault(stream) == 0
+    again, _, _, _ = GaussianRasterizer(settings)(**args)
+    torch.cuda.synchronize()
+    assert torch.equal(again, good)
+    assert _capi.lib.rgs_sort_fault(stream) == 0
