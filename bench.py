@@ -30,16 +30,25 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
 
-# HBM bytes per launch of each stage's kernels on the default workload (C1 at full size), from
-# rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this script scaled by what the same counters read
-# for a 1 GiB copy (x2.000 and x1.000 to KiB); mean over the launches of a step.  Counters
-# cannot be read from inside the process, so the figures are carried here; other workloads
-# report null.
-C1_TRAFFIC_MB_PER_LAUNCH = {
-    "preprocess_forward": 254.10, "duplicate_with_keys": 108.31, "sort_onesweep": 23.11, "tile_ranges": 13.22,
-    "blend_forward": 237.40, "composite_forward": 165.79, "composite_backward": 372.03, "blend_backward": 284.80,
-    "preprocess_backward": 370.26,
-}
+def load_traffic_table():
+    """HBM bytes per launch of each stage's kernels on the default workload (C1 at full size), measured with
+    rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this script.  Counters cannot be read from inside the process, so
+    the figures are kept in a small text file beside the profile summaries, which also names the commit they
+    were taken at; without that file the line reports null."""
+    path = os.path.join(ROOT, "profiles", "c1_hbm_traffic_per_launch.txt")
+    table, commit = {}, None
+    try:
+        for raw in open(path):
+            line = raw.strip()
+            if line.startswith("# commit:"):
+                commit = line.split(":", 1)[1].strip()
+            if not line or line.startswith("#"):
+                continue
+            name, mb = line.split()[:2]
+            table[name] = float(mb)
+    except (OSError, ValueError):
+        return {}, None
+    return table, commit
 
 
 def parse():
@@ -64,6 +73,12 @@ def parse():
                     help="issue each stream's forward calls from a host thread of its own")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 1 GiB device-to-device copy, the known-size reference for HBM traffic counters")
+    ap.add_argument("--scene-on", default="auto", choices=["auto", "host", "device"],
+                    help="where the synthetic scene is generated and partitioned (auto: C3 and C4 on the device, "
+                         "where it takes seconds; the others on the host, so that the CPU baseline sees the same values)")
+    ap.add_argument("--no-render-metric", action="store_true",
+                    help="skip the second half of the metric (render-only ms/frame at C3 and C4) in the default run")
+    ap.add_argument("--no-asides", action="store_true", help="skip the stages beside the metric (sharing, loss, optimiser)")
     return ap.parse_args()
 
 
@@ -84,15 +99,42 @@ def main():
         print("bench.py needs a GPU (the HIP library is the only implementation).", file=sys.stderr)
         sys.exit(2)
     ensure_built()
+    default_run = (args.config == "C1" and not args.forward_only and args.shrink == 1.0 and args.resolution_scale == 1.0)
+    line = measure(args, args.config, args.forward_only, asides=not args.no_asides, cpu=not args.no_cpu_baseline)
+    if default_run and not args.no_render_metric:
+        # the second half of the metric: render only (every related submodel's forward and the compositing)
+        for name in ("C3", "C4"):
+            try:
+                sub = measure(args, name, True, asides=False, cpu=False)
+                line[f"render_ms_per_frame_{name.lower()}"] = {
+                    "value": sub["ms_per_step"], "unit": "ms/frame", "ms_per_frame_one_stream": sub["ms_per_step_one_stream"],
+                    "workload": sub["config"]["workload"], "instances": sub["config"]["instances"],
+                    "visible": sub["config"]["visible"], "setup_s": sub["config"]["setup_s"],
+                    "peak_device_memory_GB": sub["config"]["peak_device_memory_GB"], "roofline": sub["roofline"],
+                    "blend_forward": sub["stages"].get("blend_forward"), "stages_ms": {k: v["ms_per_step"] for k, v in sub["stages"].items()},
+                    "blend_work": sub["blend_work"]}
+            except Exception as ex:   # the first half of the metric must not be lost with the second
+                torch.cuda.synchronize()
+                line[f"render_ms_per_frame_{name.lower()}"] = {"error": f"{type(ex).__name__}: {ex}"}
+    print(json.dumps(line))
+
+
+def measure(args, config, forward_only, asides, cpu):
+    """Times `config` and returns the JSON line's dictionary."""
     from retinags_amd import _capi, rasterizer as R
     from retinags_amd.harness import scenes, partition, pipeline
 
     dev = torch.device("cuda:0")
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats(dev)
     t0 = time.time()
-    scene, cam, cfg = scenes.make_config(args.config, "cpu", args.shrink, args.resolution_scale)
+    on_device = args.scene_on == "device" or (args.scene_on == "auto" and config in ("C3", "C4"))
+    scene, cam, cfg = scenes.make_config(config, dev if on_device else "cpu", args.shrink, args.resolution_scale)
     depth = cfg["bvh_depth"]
     if depth > 0:
-        part = partition.partition_scene(scene["xyz"], scene["scales"], depth)
+        split = partition.partition_scene_on_device if on_device else partition.partition_scene
+        part = split(scene["xyz"], scene["scales"], depth)
         rel = partition.relation_vector(part, cam)
         subs = pipeline.submodels_from_partition(scene, part, dev)
         members = part.members
@@ -101,9 +143,12 @@ def main():
         rel = np.zeros(1, dtype=np.int64)
         subs = [pipeline.whole_scene_submodel(scene, dev)]
         members = [np.arange(scene["xyz"].shape[0])]
+    if on_device:
+        scene = None   # the submodels hold their own copies; the CPU baseline is not run on such scenes
+        torch.cuda.empty_cache()
     cam_d = cam.to(dev)
     H, W = cam.image_height, cam.image_width
-    do_backward = bool(cfg["backward"]) and not args.forward_only
+    do_backward = bool(cfg["backward"]) and not forward_only
     if do_backward:
         for s in subs:
             s.requires_grad_(True)
@@ -111,6 +156,7 @@ def main():
     gen = torch.Generator().manual_seed(cfg["seed"] + 77)
     upstream = (torch.randn(3, H, W, generator=gen) * 1e-2).to(dev)
     related = [m for m in range(len(subs)) if rel[m] >= 0]
+    torch.cuda.synchronize()
     setup_s = time.time() - t0
 
     # the current stream counts as one of them: a process has 4 hardware queues here, and a fifth
@@ -126,10 +172,14 @@ def main():
             for s in subs:
                 for p in s.parameters():
                     p.grad = None
-            out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=host_threads,
-                                        instance_bounds=bounds)
             if do_backward:
+                out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=host_threads,
+                                            instance_bounds=bounds)
                 torch.autograd.backward([out["render"]], [upstream])
+            else:
+                with torch.no_grad():
+                    out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=host_threads,
+                                                instance_bounds=bounds)
             if bounds is None:
                 return out
             try:   # the counts have long arrived by now; a frame that ran out of room is rendered again
@@ -143,15 +193,20 @@ def main():
         bounds = {m: int(c * args.instance_room) + 4096 for m, c in pipeline.check_instance_bounds(first).items()}
         del first
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t1
+    def timed(**kw):
+        for _ in range(args.warmup):
+            step(**kw)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step(**kw)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t1
+
+    elapsed = timed()
     ms_per_step = elapsed * 1e3 / args.steps
+    # the same steps with every submodel on the caller's stream, one after the other
+    elapsed_one = timed(streams=None) if streams is not None else elapsed
     peak_gb = torch.cuda.max_memory_allocated(dev) / 1e9   # inputs, workspaces and gradients of the timed steps
 
     if args.calibrate_copy:
@@ -194,15 +249,14 @@ def main():
                 _capi.ptr(img), _capi.ptr(cnt), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
             counters += cnt.cpu().numpy().astype(np.uint64)
             del outs, geom, binning, img
-    nA, nB, nC, nD, nE, nBl, nCl = (float(v) for v in counters)
+    nA, nB, nC, nD, nE, nBl, nCl, nAl = (float(v) for v in counters)
     K = len(related)
     T = ((W + 15) // 16) * ((H + 15) // 16)
     N = W * H
     passes = (int(_capi.lib.rgs_get_higher_msb(T)) + 7) // 8   # of the instance sort, on the tile key
-    # Per-pixel entries the backward revisits: everything up to the last blended entry.
-    # It is not counted separately; the forward visit count bounds it from above.
+    # The backward revisits, per pixel, the entries up to the last blended one: nAl of the nA visits.
     flops_fwd = 12 * nA + 3 * nB + 27 * nC + 3 * nD + 14 * nE
-    flops_bwd = 12 * nA + 3 * nBl + 27 * nCl + 80 * nE
+    flops_bwd = 12 * nAl + 3 * nBl + 27 * nCl + 80 * nE
     # Algorithmic bytes per frame of every HBM-bound stage (one launch per submodel; the sort
     # kernels run `passes` times per submodel).
     alg_bytes = {
@@ -252,16 +306,18 @@ def main():
                                       "off, so full-rate issue of fused multiply-adds is 78.6 TFLOP/s",
                         "frac_of_unpacked_fp32_issue_peak": round(d["achieved_TFLOPs"] / (FP32_PEAK_TFLOPS / 2), 4)}
         if roofline is not None:
-            full_c1 = args.config == "C1" and args.shrink == 1.0 and args.resolution_scale == 1.0
-            if full_c1 and dominant in C1_TRAFFIC_MB_PER_LAUNCH:
-                roofline["traffic"] = C1_TRAFFIC_MB_PER_LAUNCH[dominant] * 1e6  # bytes per launch
+            full_c1 = config == "C1" and args.shrink == 1.0 and args.resolution_scale == 1.0
+            traffic, commit = load_traffic_table()
+            if full_c1 and dominant in traffic:
+                roofline["traffic"] = traffic[dominant] * 1e6  # bytes per launch
+                roofline["traffic_measured_at_commit"] = commit
             roofline["timing"] = "HIP events on the launching stream, all submodels on one stream"
             roofline["avg_launch_ms"] = d["avg_launch_ms"]
             roofline["launches_per_step"] = d["launches_per_step"]
 
     gpu_stage_ms = sum(v["ms_per_step"] for v in stages.values())
     evals = {
-        "visits_per_frame": nA, "exp_per_frame": nB, "blended_per_frame": nE,
+        "visits_per_frame": nA, "exp_per_frame": nB, "blended_per_frame": nE, "backward_visits_per_frame": nAl,
         "fwd_visits_per_s": round(nA / (stages["blend_forward"]["ms_per_step"] * 1e-3), 1)
         if "blend_forward" in stages and stages["blend_forward"]["ms_per_step"] > 0 else None,
     }
@@ -275,40 +331,45 @@ def main():
             torch.cuda.synchronize()
             return {"error": f"{type(ex).__name__}: {ex}"}
 
+    asides = asides and scene is not None
     sharing = (aside(lambda: {"appending": sharing_stages(scene, part, dev, prof_steps, True),
                               "copying": sharing_stages(scene, part, dev, prof_steps, False)})
-               if part is not None else None)
+               if (part is not None and asides) else None)
 
     # ---- the steps after the path: image loss with its gradient, and the optimiser step
-    after = aside(lambda: training_stages(subs, H, W, dev, prof_steps)) if do_backward else None
+    after = aside(lambda: training_stages(subs, H, W, dev, prof_steps)) if (do_backward and asides) else None
 
     # ---- everything together: one training iteration for this camera
     whole = (aside(lambda: whole_iteration(scene, part, cam_d, rel, bg, streams, dev, args.steps))
-             if (part is not None and do_backward) else None)
+             if (part is not None and do_backward and asides) else None)
 
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
-    cpu = None
-    if not args.no_cpu_baseline:
-        cpu = cpu_baseline(scene, members, part, cam, rel, related, upstream.cpu().numpy(), do_backward, args)
+    cpu_line = None
+    if cpu and scene is not None:
+        cpu_line = cpu_baseline(scene, members, part, cam, rel, related, upstream.cpu().numpy(), do_backward, args)
 
-    line = {
+    return {
         "metric": "fwd+bwd iterations/s, 5.6M Gaussians, 1600x1036, 4 composited submodels"
-        if (args.config == "C1" and do_backward) else f"fwd{'+bwd' if do_backward else ''} iterations/s, config {args.config}",
+        if (config == "C1" and do_backward) else f"fwd{'+bwd' if do_backward else ''} iterations/s, config {config}",
         "value": round(args.steps / elapsed, 4), "unit": "it/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.config}: {cfg['n']} Gaussians, {W}x{H}, bvh_depth={depth} "
+        # every submodel on one stream, rendered strictly one after the other (`value` offers the independent
+        # submodels to the GPU on several HIP streams; no work differs)
+        "value_one_stream": round(args.steps / elapsed_one, 4), "ms_per_step_one_stream": round(elapsed_one * 1e3 / args.steps, 3),
+        "config": {"workload": f"{config}: {cfg['n']} Gaussians, {W}x{H}, bvh_depth={depth} "
                                f"({K} of {len(subs)} submodels related), SH degree 3, "
                                f"{'fwd+bwd' if do_backward else 'fwd only'}",
                    "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
                    "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1),
+                   "scene_generated_on": "device" if on_device else "host",
+                   "streams": args.streams,
                    "peak_device_memory_GB": round(peak_gb, 2),
                    "instance_room": (f"{args.instance_room} x the first frame's count, checked after every frame"
                                      if bounds is not None else "sized from each call's count (host waits)")},
-        "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
+        "roofline": roofline, "cpu_baseline": cpu_line, "stages": stages, "gpu_kernel_ms_per_step": round(gpu_stage_ms, 3),
         "blend_work": evals, "sharing": sharing, "loss_and_optimiser": after, "training_iteration": whole,
     }
-    print(json.dumps(line))
 
 
 def sharing_stages(scene, part, dev, repeats, append):

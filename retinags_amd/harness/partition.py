@@ -57,6 +57,7 @@ class Partition:
     owner: np.ndarray             # (N,) submodel id of every Gaussian
     members: List[np.ndarray]     # per submodel: indices into the scene, own Gaussians first,
                                   # then straddlers from other submodels in ascending source id
+    # partition_scene_on_device leaves owner and members as tensors on the scene's device
 
 
 def build_grid(xyz: np.ndarray, scales_activated: np.ndarray) -> Grid:
@@ -143,6 +144,74 @@ def partition_scene(xyz: torch.Tensor, scales_activated: torch.Tensor, depth: in
             reach = np.all((p + r[:, None] >= box_low[dst]) & (p - r[:, None] <= box_up[dst]), axis=1)
             parts.append(ids[cand & reach])
         members.append(np.concatenate(parts))
+    return Partition(grid, nodes, leaves, box_low, box_up, owner, members)
+
+
+def _grid_from_extent(xyz_min: np.ndarray, xyz_max: np.ndarray, scale_max: np.ndarray):
+    """low, up, voxel, size of build_grid from the three per-axis extremes (float32, as there)."""
+    pad = 3.0 * scale_max.astype(np.float32)
+    low = xyz_min.astype(np.float32) - pad
+    up = xyz_max.astype(np.float32) + pad
+    voxel = (up - low) / np.asarray(SCENE_GRID_SIZE, dtype=low.dtype) - 1e-7
+    low, up, voxel = (np.asarray(v, dtype=np.float32) for v in (low, up, voxel))
+    size = tuple(max(int((up[i] - low[i]) // voxel[i]), 1) for i in range(3))
+    return low, up, voxel, size
+
+
+def partition_scene_on_device(xyz: torch.Tensor, scales_activated: torch.Tensor, depth: int,
+                              rows_per_pass: int = 1 << 24) -> Partition:
+    """partition_scene for scenes too large to take through the host (tens to hundreds of millions
+    of Gaussians): the per-Gaussian work (voxel histogram, ownership, straddler selection) is done
+    with tensor operations on the device the scene lives on, in float32 like the numpy version, and
+    gives the same grid, boxes, owners and member lists; the tree itself (a 2048 x 2048 histogram)
+    is split on the host.  owner and members come back as tensors on that device."""
+    dev = xyz.device
+    N = int(xyz.shape[0])
+    f32 = lambda t: t.detach().cpu().numpy().astype(np.float32)
+    low, up, voxel, size = _grid_from_extent(f32(xyz.min(dim=0).values), f32(xyz.max(dim=0).values),
+                                             f32(scales_activated.max(dim=0).values))
+    low_t, voxel_t = torch.from_numpy(low).to(dev), torch.from_numpy(voxel).to(dev)
+    size_t = torch.tensor(size, device=dev)
+    cells = size[0] * size[1] * size[2]
+    load = torch.zeros(cells, dtype=torch.int64, device=dev)
+    for at in range(0, N, rows_per_pass):
+        idx = torch.floor_divide(xyz[at:at + rows_per_pass] - low_t, voxel_t).long()
+        ok = ((idx >= 0) & (idx < size_t)).all(dim=1)
+        flat = ((idx[:, 0] * size[1] + idx[:, 1]) * size[2] + idx[:, 2])[ok]
+        load += torch.bincount(flat, minlength=cells)
+    grid = Grid(low, up, voxel, size, load.reshape(size).double().cpu().numpy())
+    nodes = build_bvh(grid, depth)
+    leaves = sorted((n for n in nodes.values() if n.is_leaf), key=lambda n: n.path)
+    K = len(leaves)
+    box_low = np.stack([np.asarray(n.low) * grid.voxel.astype(np.float64) + grid.low for n in leaves]).astype(np.float32)
+    box_up = np.stack([np.asarray(n.up) * grid.voxel.astype(np.float64) + grid.low for n in leaves]).astype(np.float32)
+    lows, ups = torch.from_numpy(box_low).to(dev), torch.from_numpy(box_up).to(dev)
+
+    owner = torch.full((N,), -1, dtype=torch.int64, device=dev)
+    for at in range(0, N, rows_per_pass):
+        p = xyz[at:at + rows_per_pass]
+        part = owner[at:at + rows_per_pass]
+        for k in range(K):  # later ids overwrite earlier ones on ties
+            part[((p >= lows[k]) & (p <= ups[k])).all(dim=1)] = k
+    if bool((owner < 0).any()):
+        raise RuntimeError("a Gaussian fell outside every submodel box")
+
+    own = [torch.nonzero(owner == k).squeeze(1) for k in range(K)]
+    lent = [[None] * K for _ in range(K)]   # lent[dst][src]
+    for src in range(K):
+        ids = own[src]
+        if ids.numel() == 0:
+            continue
+        p = xyz[ids]
+        r = (3.0 * scales_activated[ids].max(dim=1).values).clamp(min=0.0).unsqueeze(1)
+        hi, lo = p + r, p - r
+        cand = ((hi >= ups[src]) | (lo <= lows[src])).any(dim=1)
+        ids, hi, lo = ids[cand], hi[cand], lo[cand]
+        for dst in range(K):
+            if dst != src:
+                lent[dst][src] = ids[((hi >= lows[dst]) & (lo <= ups[dst])).all(dim=1)]
+    members = [torch.cat([own[dst]] + [lent[dst][src] for src in range(K) if src != dst and lent[dst][src] is not None])
+               for dst in range(K)]
     return Partition(grid, nodes, leaves, box_low, box_up, owner, members)
 
 

@@ -45,8 +45,8 @@ class Submodel:
 def submodels_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device) -> List[Submodel]:
     subs = []
     for k, ids in enumerate(part.members):
-        idx = torch.from_numpy(ids)
-        pick = lambda t: t[idx].to(device).contiguous()
+        idx = ids if torch.is_tensor(ids) else torch.from_numpy(ids)
+        pick = lambda t: t[idx.to(t.device)].to(device).contiguous()
         subs.append(Submodel(pick(scene["xyz"]), pick(scene["opacity"]), pick(scene["scales"]),
                              pick(scene["rotations"]), pick(scene["shs"]),
                              torch.from_numpy(part.box_low[k]).to(device), torch.from_numpy(part.box_up[k]).to(device)))

@@ -88,30 +88,36 @@ def look_at_camera(eye, target, up, width: int, height: int, fovx_deg: float) ->
     return camera_from_w2c(w2c, width, height, math.radians(fovx_deg))
 
 
-def _attributes(n: int, gen: torch.Generator, device, scale_shift: float = 0.0) -> Dict[str, torch.Tensor]:
+def _attributes(n: int, gen: torch.Generator, device, scale_shift: float = 0.0,
+                geometry_only: bool = False) -> Dict[str, torch.Tensor]:
     """Scales exp(N(-4, 0.5^2)) (+ scale_shift in log space), unit quaternions, opacity
-    sigmoid(N(0,1)), SH degree 3: DC ~ N(0.5, 0.2^2), 45 remaining coefficients ~ N(0, 0.2^2)."""
+    sigmoid(N(0,1)), SH degree 3: DC ~ N(0.5, 0.2^2), 45 remaining coefficients ~ N(0, 0.2^2).
+    geometry_only stops after the scales (the first draw), which with the positions is all a
+    partition needs."""
     kw = dict(generator=gen, device=device, dtype=torch.float32)
-    scales = torch.exp(torch.randn(n, 3, **kw) * 0.5 - 4.0 + scale_shift)
+    scales = torch.exp(torch.randn(n, 3, **kw).mul_(0.5).add_(-4.0 + scale_shift))
+    if geometry_only:
+        return dict(scales=scales)
     rot = torch.randn(n, 4, **kw)
     rot = rot / rot.norm(dim=1, keepdim=True)
     opacity = torch.sigmoid(torch.randn(n, 1, **kw))
-    shs = torch.randn(n, 16, 3, **kw) * 0.2
+    shs = torch.randn(n, 16, 3, **kw).mul_(0.2)
     shs[:, 0, :] += 0.5
     return dict(scales=scales, rotations=rot, opacity=opacity, shs=shs)
 
 
-def cube_scene(n: int, seed: int, device="cpu") -> Dict[str, torch.Tensor]:
+def cube_scene(n: int, seed: int, device="cpu", geometry_only: bool = False) -> Dict[str, torch.Tensor]:
     """Config 0: positions uniform in [-1,1]^3 centred 4 units down +z."""
     gen = torch.Generator(device=device).manual_seed(seed)
     xyz = torch.rand(n, 3, generator=gen, device=device) * 2.0 - 1.0
     xyz[:, 2] += 4.0
-    out = _attributes(n, gen, device)
+    out = _attributes(n, gen, device, geometry_only=geometry_only)
     out["xyz"] = xyz
     return out
 
 
-def garden_scene(n: int, seed: int, device="cpu", scale_shift: float = 0.0) -> Dict[str, torch.Tensor]:
+def garden_scene(n: int, seed: int, device="cpu", scale_shift: float = 0.0,
+                 geometry_only: bool = False) -> Dict[str, torch.Tensor]:
     """Configs 1-3: 70 % on a noisy ground plane (x,y uniform over 20x20, z ~ N(0,0.05^2)),
     30 % on an upper hemisphere shell of radius 10 with N(0,0.3^2) radial jitter."""
     gen = torch.Generator(device=device).manual_seed(seed)
@@ -126,12 +132,13 @@ def garden_scene(n: int, seed: int, device="cpu", scale_shift: float = 0.0) -> D
     d[:, 2] = d[:, 2].abs()
     radius = 10.0 + torch.randn(n_shell, 1, **kw) * 0.3
     shell = d * radius
-    out = _attributes(n, gen, device, scale_shift)
+    out = _attributes(n, gen, device, scale_shift, geometry_only)
     out["xyz"] = torch.cat([ground, shell], dim=0)
     return out
 
 
-def city_scene(n: int, seed: int, device="cpu", blocks_per_side: int = 40) -> Dict[str, torch.Tensor]:
+def city_scene(n: int, seed: int, device="cpu", blocks_per_side: int = 40,
+               geometry_only: bool = False) -> Dict[str, torch.Tensor]:
     """Config 4: axis-aligned building boxes on a 2 km x 2 km grid (heights ~ U(5,120) m,
     Gaussians on the box surfaces) plus a ground plane (30 % of the Gaussians)."""
     gen = torch.Generator(device=device).manual_seed(seed)
@@ -157,7 +164,8 @@ def city_scene(n: int, seed: int, device="cpu", blocks_per_side: int = 40) -> Di
     py = torch.where(face == 2, torch.full_like(py, half), torch.where(face == 3, torch.full_like(py, -half), py))
     pz = torch.where(face == 4, heights[which], pz)
     blocks = torch.stack([cx + px, cy + py, pz], dim=1)
-    out = _attributes(n, gen, device)
+    del u, face, which, px, py, pz, cx, cy
+    out = _attributes(n, gen, device, geometry_only=geometry_only)
     out["xyz"] = torch.cat([ground, blocks], dim=0)
     return out
 
@@ -172,10 +180,13 @@ CONFIGS = {
 }
 
 
-def make_config(name: str, device="cpu", shrink: float = 1.0, resolution_scale: float = 1.0):
+def make_config(name: str, device="cpu", shrink: float = 1.0, resolution_scale: float = 1.0,
+                geometry_only: bool = False):
     """Returns (scene dict, Camera, config dict).  `shrink` divides the Gaussian count and
     `resolution_scale` multiplies the image size, for tests that need a small instance of
-    the same distribution."""
+    the same distribution.  The generator lives on `device`: a scene made on the GPU has the same
+    distribution as, but other values than, the one made on the host from the same seed.
+    geometry_only: positions and scales alone (the same values as in the full scene)."""
     cfg = dict(CONFIGS[name])
     cfg["name"] = name
     n = max(16, int(cfg["n"] / shrink))
@@ -183,16 +194,16 @@ def make_config(name: str, device="cpu", shrink: float = 1.0, resolution_scale: 
     h = max(16, int(round(cfg["height"] * resolution_scale)))
     cfg.update(n=n, width=w, height=h)
     if name == "C0":
-        scene = cube_scene(n, cfg["seed"], device)
+        scene = cube_scene(n, cfg["seed"], device, geometry_only=geometry_only)
         cam = look_at_camera((0, 0, 0), (0, 0, 1), (0, -1, 0), w, h, 60.0)
     elif name in ("C1", "C2"):
-        scene = garden_scene(n, cfg["seed"], device)
+        scene = garden_scene(n, cfg["seed"], device, geometry_only=geometry_only)
         cam = look_at_camera((6.0, 0.0, 2.0), (0, 0, 0), (0, 0, 1), w, h, 60.0)
     elif name == "C3":
-        scene = garden_scene(n, cfg["seed"], device, scale_shift=-math.log(math.sqrt(11.0)))
+        scene = garden_scene(n, cfg["seed"], device, scale_shift=-math.log(math.sqrt(11.0)), geometry_only=geometry_only)
         cam = look_at_camera((6.0, 0.0, 2.0), (0, 0, 0), (0, 0, 1), w, h, 60.0)
     elif name == "C4":
-        scene = city_scene(n, cfg["seed"], device)
+        scene = city_scene(n, cfg["seed"], device, geometry_only=geometry_only)
         cam = look_at_camera((0.0, -300.0, 300.0), (0, 0, 0), (0, 0, 1), w, h, 60.0)
     else:
         raise KeyError(name)

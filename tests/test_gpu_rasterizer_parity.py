@@ -25,7 +25,7 @@ def _run_gpu_forward(sub, cam, bg, dev, sh_degree=3, scale_modifier=1.0, debug=F
         cam.image_height, cam.image_width, sub["shs"].to(dev), sh_degree, cam.camera_center.to(dev), False, debug)
 
 
-def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
+def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0, max_borderline=MAX_BORDERLINE_FRACTION):
     from retinags_amd import _capi
     dev = torch.device("cuda:0")
     s = oracle_settings(cam, sub["low"], sub["up"], bg, sh_degree, scale_modifier)
@@ -84,7 +84,7 @@ def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0):
     # ---- blend: tolerance, away from decision thresholds
     n_contrib = view_ws(img, im["n_contrib"], H * W, np.uint32)
     safe = (st.margin > DECISION_MARGIN).reshape(H, W)
-    assert (~safe).mean() <= MAX_BORDERLINE_FRACTION
+    assert (~safe).mean() <= max_borderline
     for got, want in ((color, st.color), (depth, st.depth), (alpha, st.alpha)):
         diff = np.abs(got.cpu().numpy() - want)
         assert diff[:, safe].max() <= IMAGE_TOL
@@ -108,6 +108,21 @@ def _scene_sub(scene, low=None, up=None):
 def test_cube_forward_stages():
     scene, cam, _ = scenes.make_config("C0", shrink=5, resolution_scale=0.5)
     _check_forward_stages(_scene_sub(scene), cam, torch.tensor([0.1, 0.2, 0.3]))
+
+
+def test_cube_at_full_size_forward_and_backward():
+    """Config C0 whole: 100 000 Gaussians at 512x512, one submodel, every stage and every gradient."""
+    import os
+    scene, cam, cfg = scenes.make_config("C0")
+    assert cfg["n"] == 100_000 and (cam.image_width, cam.image_height) == (512, 512)
+    orc.set_threads(min(16, orc.max_threads(), os.cpu_count() or 1))
+    try:
+        # a pixel walks some 500 list entries here, each a chance to sit within 2e-5 of a threshold
+        st = _check_forward_stages(_scene_sub(scene), cam, torch.tensor([0.1, 0.2, 0.3]), max_borderline=1e-3)
+        assert st.R > 400_000
+        _check_backward(_scene_sub(scene), cam, torch.tensor([0.1, 0.2, 0.3]), seed=21, with_depth_alpha=True)
+    finally:
+        orc.set_threads(1)
 
 
 def test_cube_forward_lower_sh_degrees_and_scale_modifier():

@@ -221,3 +221,16 @@ def test_merge_of_the_checker_and_its_adjoint():
         lhs = sum(float((merged[n].astype(np.float64) * g[n]).sum()) for n in merged)
         rhs = sum(float((models[s][n].astype(np.float64) * back[s][n]).sum()) for s in range(3) for n in merged)
         assert abs(lhs - rhs) < 1e-4 * max(1.0, abs(lhs))
+
+
+def test_partition_by_tensor_operations_matches_the_numpy_partition():
+    """partition_scene_on_device (used for the scenes too large for the host) on the CPU device: same
+    grid loads, boxes, owners and member lists as partition_scene, also when taken in several passes."""
+    for name, shrink in (("C1", 100.0), ("C3", 600.0), ("C4", 2000.0)):
+        scene, _, cfg = scenes.make_config(name, "cpu", shrink, geometry_only=True)
+        host = partition.partition_scene(scene["xyz"], scene["scales"], cfg["bvh_depth"])
+        other = partition.partition_scene_on_device(scene["xyz"], scene["scales"], cfg["bvh_depth"], rows_per_pass=20_000)
+        assert np.array_equal(host.grid.load, other.grid.load)
+        assert np.array_equal(host.box_low, other.box_low) and np.array_equal(host.box_up, other.box_up)
+        assert np.array_equal(host.owner, other.owner.numpy())
+        assert all(np.array_equal(a, b.numpy()) for a, b in zip(host.members, other.members))
