@@ -250,6 +250,18 @@ int rgs_sort_fault(void* stream);
  * give-up path from the host while every kernel still runs to its end).  Process-wide. */
 int rgs_set_lookback_spin_limit(int polls);
 
+/* rgs_sort_pairs for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it): the same sort with the same results, whose
+ * scratch is an array the library itself holds on every device it runs on (about 8.4 MB, until
+ * the process ends), so no workspace is passed.  No counterpart in the reference, whose
+ * cub::DeviceRadixSort::SortPairs always works in a buffer the caller grows
+ * (K/cuda_rasterizer_hgs/rasterizer_impl.cu:188-194, 312-317).  n <= RGS_STATIC_SORT_MAX_PAIRS, else the
+ * call fails.  It calls no allocation routine; all calls on one device share the one array, so
+ * calls that overlap on a device (two streams, two threads) race: issue them on one stream. */
+#define RGS_STATIC_SORT_MAX_PAIRS (1 << 22)
+int rgs_sort_pairs_static(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                          int end_bit, void* stream);
+
 /* ---- partial-image compositor ------------------------------------------------------------
  * Replaces the tensor expression in blender_render_result
  * (parallel_utils/basic_parallel_trainer/result_aggregator.py:244-259) and its autograd

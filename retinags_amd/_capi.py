@@ -73,6 +73,7 @@ def _load():
                                  f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, i]
     lib.rgs_inclusive_sum.argtypes = [vp, vp, sz, vp, vp]
     lib.rgs_sort_pairs.argtypes = [vp, vp, vp, vp, sz, i, vp, vp]
+    lib.rgs_sort_pairs_static.argtypes = [vp, vp, vp, vp, sz, i, vp]
     lib.rgs_sort_fault.argtypes = [vp]
     lib.rgs_set_lookback_spin_limit.argtypes = [i]
     pp = C.POINTER(vp)
@@ -96,7 +97,7 @@ def _load():
                  "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_forward_raster_bounded", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
                  "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
                  "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step",
-                 "rgs_activate_forward", "rgs_activate_backward", "rgs_sort_fault",
+                 "rgs_activate_forward", "rgs_activate_backward", "rgs_sort_pairs_static", "rgs_sort_fault",
                  "rgs_set_lookback_spin_limit"):
         getattr(lib, name).restype = i
     return lib
@@ -111,7 +112,8 @@ EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_byte
            "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",
            "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward", "rgs_loss_workspace_bytes",
            "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step", "rgs_activate_forward",
-           "rgs_activate_backward", "rgs_sort_fault", "rgs_set_lookback_spin_limit")
+           "rgs_activate_backward", "rgs_sort_pairs_static", "rgs_sort_fault", "rgs_set_lookback_spin_limit")
+STATIC_SORT_MAX_PAIRS = 1 << 22
 WORK_COUNTERS = 8
 
 

@@ -12,6 +12,13 @@
 #include <string>
 #include <vector>
 
+// Scratch of rgs_sort_pairs_static, the entry point that allocates nothing: digit histograms, tile
+// counters and look-back words of a sort of up to RGS_STATIC_SORT_MAX_PAIRS pairs.  Every device the
+// library runs on holds its own copy until the process ends.  In host code this name is only a handle
+// for hipGetSymbolAddress; the address the kernels get is looked up once per device (static_sort_scratch).
+constexpr size_t kStaticSortWords = rgs::sort_temp_words_for(RGS_STATIC_SORT_MAX_PAIRS);
+static __device__ __align__(256) uint32_t scratch[kStaticSortWords];
+
 namespace {
 
 thread_local char g_error[512] = "";
@@ -92,6 +99,7 @@ struct EntryScope {
 constexpr int kMaxDevices = 64;
 std::mutex g_device_mutex;
 uint32_t* g_fault_word[kMaxDevices] = {};
+uint32_t* g_static_scratch[kMaxDevices] = {};
 
 int current_device()
 {
@@ -136,6 +144,24 @@ int take_sort_fault(const char* who)
 		if (int rc_ = take_sort_fault(who))        \
 			return rc_;                            \
 	} while (0)
+
+// Device address of this device's copy of `scratch`, looked up once per device with that device current.
+int static_sort_scratch(uint32_t** out)
+{
+	const int dev = current_device();
+	if (dev < 0)
+		return fail("rgs_sort_pairs_static: no current device");
+	std::lock_guard<std::mutex> lock(g_device_mutex);
+	if (!g_static_scratch[dev]) {
+		void* p = nullptr;
+		const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+		if (e != hipSuccess || !p)
+			return fail("rgs_sort_pairs_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+		g_static_scratch[dev] = static_cast<uint32_t*>(p);
+	}
+	*out = g_static_scratch[dev];
+	return 0;
+}
 
 constexpr size_t kAlign = 256;
 
@@ -835,6 +861,26 @@ int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uin
 	RGS_REQUIRE(n < 0x40000000ull, "rgs_sort_pairs: 2^30 pairs or more");
 	return sort_pairs_u64("rgs_sort_pairs", keys_in, keys_out, vals_in, vals_out, n, end_bit, static_cast<uint32_t*>(temp),
 	                      fault_word(true), s);
+}
+
+int rgs_sort_pairs_static(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
+                          int end_bit, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	RGS_REQUIRE(end_bit >= 1 && end_bit <= 64, "rgs_sort_pairs_static: end_bit %d out of range", end_bit);
+	RGS_REQUIRE(n <= (size_t)RGS_STATIC_SORT_MAX_PAIRS,
+	            "rgs_sort_pairs_static: %zu pairs exceed the %d the library's own scratch has room for (use rgs_sort_pairs "
+	            "with a workspace)", n, RGS_STATIC_SORT_MAX_PAIRS);
+	if (n == 0)
+		return 0;
+	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out, "rgs_sort_pairs_static: null pointer");
+	RGS_REQUIRE(rgs::sort_temp_words(n) <= kStaticSortWords, "rgs_sort_pairs_static: scratch layout mismatch");
+	uint32_t* temp = nullptr;
+	if (int rc = static_sort_scratch(&temp))
+		return rc;
+	// the report word is only used if an earlier call has set it up: nothing is allocated here
+	return sort_pairs_u64("rgs_sort_pairs_static", keys_in, keys_out, vals_in, vals_out, n, end_bit, temp, fault_word(false), s);
 }
 
 int rgs_set_lookback_spin_limit(int polls)
