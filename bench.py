@@ -78,6 +78,9 @@ def parse():
                          "where it takes seconds; the others on the host, so that the CPU baseline sees the same values)")
     ap.add_argument("--no-render-metric", action="store_true",
                     help="skip the second half of the metric (render-only ms/frame at C3 and C4) in the default run")
+    ap.add_argument("--apart", action="store_true",
+                    help="one rasterizer call per submodel, as the reference issues them (default: the submodels of a frame "
+                         "go through one call that blends them in one launch per direction)")
     ap.add_argument("--no-asides", action="store_true", help="skip the stages beside the metric (sharing, loss, optimiser)")
     return ap.parse_args()
 
@@ -165,6 +168,7 @@ def measure(args, config, forward_only, asides, cpu):
                if args.streams > 0 else None)
 
     bounds = None   # room for each submodel's instances; None: wait for every count
+    together = not args.apart and args.instance_room <= 0 and not args.host_threads
 
     def step(streams=streams, host_threads=args.host_threads):
         nonlocal bounds
@@ -174,12 +178,12 @@ def measure(args, config, forward_only, asides, cpu):
                     p.grad = None
             if do_backward:
                 out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=host_threads,
-                                            instance_bounds=bounds)
+                                            instance_bounds=bounds, together=together)
                 torch.autograd.backward([out["render"]], [upstream])
             else:
                 with torch.no_grad():
                     out = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, host_threads=host_threads,
-                                                instance_bounds=bounds)
+                                                instance_bounds=bounds, together=together)
             if bounds is None:
                 return out
             try:   # the counts have long arrived by now; a frame that ran out of room is rendered again
@@ -193,6 +197,8 @@ def measure(args, config, forward_only, asides, cpu):
         bounds = {m: int(c * args.instance_room) + 4096 for m, c in pipeline.check_instance_bounds(first).items()}
         del first
 
+    host_ms = {}
+
     def timed(**kw):
         for _ in range(args.warmup):
             step(**kw)
@@ -200,8 +206,11 @@ def measure(args, config, forward_only, asides, cpu):
         t1 = time.perf_counter()
         for _ in range(args.steps):
             step(**kw)
+        t2 = time.perf_counter()   # everything is queued; what is left is the device catching up
         torch.cuda.synchronize()
-        return time.perf_counter() - t1
+        t3 = time.perf_counter()
+        host_ms["one_stream" if kw.get("streams", streams) is None else "streams"] = (t2 - t1) * 1e3 / args.steps
+        return t3 - t1
 
     elapsed = timed()
     ms_per_step = elapsed * 1e3 / args.steps
@@ -268,6 +277,10 @@ def measure(args, config, forward_only, asides, cpu):
         "sort_setup": 4.0 * R_tot,
         "sort_onesweep": 16.0 * R_tot * passes,
         "tile_ranges": 4.0 * R_tot + 16.0 * T * K,
+        # the sorted keys in, the filed positions out (at most four per instance; counted as one)
+        "strip_filing": 8.0 * R_tot + 16.0 * T * K,
+        # the eight gradient tensors and the rows of sums, written once
+        "clear_gradients": (4.0 * (3 + 1 + 3 + 3 + 6 + 48 + 3 + 4) + 48.0) * P_tot,
         # rows of the rendered Gaussians only: sums, mean, covariance, SH, scale, rotation in;
         # the eight gradient rows out
         "preprocess_backward": (309.0 + 284.0) * P_vis,
@@ -357,6 +370,8 @@ def measure(args, config, forward_only, asides, cpu):
         # every submodel on one stream, rendered strictly one after the other (`value` offers the independent
         # submodels to the GPU on several HIP streams; no work differs)
         "value_one_stream": round(args.steps / elapsed_one, 4), "ms_per_step_one_stream": round(elapsed_one * 1e3 / args.steps, 3),
+        # how long the host takes to queue a step (the forward's waits for the instance counts included)
+        "host_ms_per_step": {k: round(v, 3) for k, v in host_ms.items()},
         "config": {"workload": f"{config}: {cfg['n']} Gaussians, {W}x{H}, bvh_depth={depth} "
                                f"({K} of {len(subs)} submodels related), SH degree 3, "
                                f"{'fwd+bwd' if do_backward else 'fwd only'}",
@@ -364,6 +379,7 @@ def measure(args, config, forward_only, asides, cpu):
                    "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1),
                    "scene_generated_on": "device" if on_device else "host",
                    "streams": args.streams,
+                   "submodels_of_a_frame": "one call, blended in one launch per direction" if together else "one call each",
                    "peak_device_memory_GB": round(peak_gb, 2),
                    "instance_room": (f"{args.instance_room} x the first frame's count, checked after every frame"
                                      if bounds is not None else "sized from each call's count (host waits)")},

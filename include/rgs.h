@@ -13,6 +13,8 @@
  *
  * Limits: a call handles fewer than 2^30 (Gaussian, tile) instances (the radix sorts pack a
  * count and two flag bits into one word); rgs_forward_geom reports a larger count as an error.
+ * An image has fewer than 2^24 tiles of 16x16 pixels (the tile shares its 32-bit sort key with
+ * eight strip bits); rgs_forward_raster refuses a larger one.
  *
  * A sort that gives up: the radix sorts wait for neighbouring workgroups with a bounded number
  * of polls.  Should such a wait ever run out (never observed), every later kernel of that call
@@ -73,7 +75,7 @@ enum {
 	RGS_GEOM_TOTAL,             /* uint32     number of (Gaussian, tile) instances */
 	RGS_GEOM_BLEND_RECORD,      /* float[16P] one 64-byte record per Gaussian with everything the blend reads:
 	                               x, y, exponent floor, clip w | conic xx, xy, yy, opacity | r, g, b, depth |
-	                               half-width, half-height of the alpha >= 1/255 ellipse's bounding box, 0, 0 */
+	                               half-width, half-height of the alpha >= 1/255 ellipse's bounding box, the radius (int32 bits), 0 */
 	RGS_GEOM_DEPTH_ORDER,       /* uint32[P]  the Gaussians that touch a tile by increasing depth, ties by index;
 	                               entries from RGS_GEOM_VISIBLE_COUNT on are unused */
 	RGS_GEOM_BLOCK_VISIBLE,     /* uint32[ceil(P/256)+1] */
@@ -83,12 +85,14 @@ enum {
 	RGS_GEOM_FIELDS
 };
 enum {
-	RGS_BIN_KEYS_UNSORTED = 0,  /* uint32[R]  tile of each instance, emitted Gaussian after Gaussian in depth order */
+	RGS_BIN_KEYS_UNSORTED = 0,  /* uint32[R]  key of each instance, emitted Gaussian after Gaussian in depth order: the tile in
+	                               the low 24 bits; above it, per 16x4 strip s of the tile, bit 24+s = the instance can
+	                               matter to the strip, bit 28+s = that strip lies inside the submodel box */
 	RGS_BIN_KEYS_SORTED,        /* uint32[R]  the same after the stable sort by tile */
 	RGS_BIN_VALUES_UNSORTED,    /* uint32[R]  Gaussian index */
 	RGS_BIN_VALUES_SORTED,      /* uint32[R]  the per-tile Gaussian lists, tile after tile */
 	RGS_BIN_SORT_TEMP,          /* uint32[..] */
-	RGS_BIN_STRIP_LISTS,        /* uint32[4R] written by the forward blend: for strip s of a tile with list [x, x+n), from
+	RGS_BIN_STRIP_LISTS,        /* uint32[4R] written ahead of the forward blend: for strip s of a tile with list [x, x+n), from
 	                               4x + s*n on, the list positions that can matter to the strip (bit 31: strip inside the box) */
 	RGS_BIN_FIELDS
 };
@@ -97,6 +101,8 @@ enum {
 	RGS_IMG_N_CONTRIB,          /* uint32[H*W]   list position of the last blended Gaussian */
 	RGS_IMG_STRIP_FILED,        /* uint32[4*tiles] per 16x4 strip (tile * 4 + strip): entries of RGS_BIN_STRIP_LISTS the backward walks */
 	RGS_IMG_STRIP_ORDER,        /* uint32[4*tiles] the strips by decreasing RGS_IMG_STRIP_FILED: the order the backward blend takes them in */
+	RGS_IMG_STRIP_TOTAL,        /* uint32[4*tiles] per strip: entries of RGS_BIN_STRIP_LISTS in all */
+	RGS_IMG_STRIP_ORDER_FORWARD,/* uint32[4*tiles] the strips by decreasing RGS_IMG_STRIP_TOTAL: the order the forward blend takes them in */
 	RGS_IMG_FIELDS
 };
 int rgs_geom_layout(int P, size_t offsets[RGS_GEOM_FIELDS]);
@@ -203,6 +209,75 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
                  float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int outputs_zeroed, void* stream,
                  int debug);
+
+/* ---- the submodels of a frame in one go ----------------------------------------------------------
+ * The reference renders the submodels that a camera sees one call after the other
+ * (gather_RenderResult_pool, parallel_utils/basic_parallel_trainer/result_aggregator.py:22-38) and hands
+ * each its gradient in turn (trainer4tree_partition.py:505-514).  These two entry points take all of them
+ * ("layers": same camera, same image size) so that the per-tile blends, whose launches end with a few
+ * long tiles each, run as one launch per frame in which the layers' tails overlap.  A layer's fields are
+ * the arguments of rgs_forward_raster / rgs_backward with the same meaning; the geometry stage of every
+ * layer (rgs_forward_geom or rgs_forward_geom_enqueue) comes first and supplies R.  Results are those of
+ * the per-layer calls, bit for bit in the forward. */
+#define RGS_MAX_FRAME_LAYERS 64
+typedef struct rgs_frame_view {
+	int width, height;
+	float tan_fovx, tan_fovy;
+	const float* viewmatrix;
+	const float* projmatrix;
+	const float* projmatrix_inv;
+	const float* cam_pos;
+} rgs_frame_view;
+typedef struct rgs_frame_layer {
+	int P, D, M, R;
+	const float* means3D;
+	const float* shs;
+	const float* colors_precomp;
+	const float* opacities;
+	const float* scales;
+	const float* rotations;
+	const float* cov3D_precomp;
+	float scale_modifier;
+	const float* background;
+	const float* range_low;
+	const float* range_up;
+	const int* radii;
+	void* geom_ws;
+	void* binning_ws;
+	void* image_ws;
+	size_t geom_bytes, binning_bytes, image_bytes;
+	float* out_color;          /* forward outputs; the backward reads out_alpha */
+	float* out_depth;
+	float* out_alpha;
+	const float* dL_dpix;      /* backward inputs; depth / alpha may be NULL */
+	const float* dL_dpix_depth;
+	const float* dL_dalphas;
+	float* grad_accum;         /* backward scratch and outputs, as in rgs_backward */
+	float* dL_dmean2D;
+	float* dL_dopacity;
+	float* dL_dcolor;
+	float* dL_dmean3D;
+	float* dL_dcov3D;
+	float* dL_dsh;
+	float* dL_dscale;
+	float* dL_drot;
+	int outputs_zeroed;
+	void* clear[2];            /* rgs_frame_forward_raster: up to two device buffers (NULL: none) that it sets to zero (sizes */
+	size_t clear_bytes[2];     /* multiples of 4 bytes): the gradient tensors, cleared beside the blend on the layer's own stream */
+	void* stream;              /* the layer's own HIP stream, or NULL for the frame's: its geometry stage was enqueued
+	                              there, and the stages that run once per layer (binning; per-Gaussian backward) follow
+	                              on it, beside the other layers'; the frame's stream waits for them and is waited for */
+} rgs_frame_layer;
+/* rgs_forward_geom for every layer (P > 0 each): every geometry stage is queued (on the layer's stream) before
+ * the host waits for the first instance count; returns when all counts have arrived in counts_pinned[0..K)
+ * (pinned host memory), which is also where the layers' R for the next call is read from. */
+int rgs_frame_forward_geom(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, uint32_t* counts_pinned,
+                           void* stream, int debug);
+/* rgs_forward_raster for every layer (P > 0 each): per layer the key duplication, sort, ranges and strip
+ * lists, then one blend launch for all.  `layers` and `view` are HOST structures. */
+int rgs_frame_forward_raster(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug);
+/* rgs_backward for every layer: one blend-backward launch for all, then each layer's per-Gaussian backward. */
+int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug);
 
 /* ---- measurement aids (no counterpart in the reference, which times whole iterations
  * with CUDA events: parallel_utils/basic_parallel_trainer/trainer4tree_partition.py:590-643) -- */

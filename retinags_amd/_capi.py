@@ -16,7 +16,7 @@ GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles
                "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
                "visible_list", "order_scratch")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp", "strip_lists")
-IMG_FIELDS = ("ranges", "n_contrib", "strip_filed", "strip_order")
+IMG_FIELDS = ("ranges", "n_contrib", "strip_filed", "strip_order", "strip_total", "strip_order_forward")
 ACC_FLOATS = 12
 MAX_COMPOSITE = 64
 MAX_SHARE_BOXES = 64
@@ -38,6 +38,30 @@ class AdamTensor(C.Structure):
     """rgs_adam_tensor of include/rgs.h."""
     _fields_ = [("param", C.c_void_p), ("grad", C.c_void_p), ("exp_avg", C.c_void_p), ("exp_avg_sq", C.c_void_p),
                 ("n", C.c_size_t), ("lr", C.c_double), ("step", C.c_int)]
+
+
+class FrameView(C.Structure):
+    """rgs_frame_view of include/rgs.h."""
+    _fields_ = [("width", C.c_int), ("height", C.c_int), ("tan_fovx", C.c_float), ("tan_fovy", C.c_float),
+                ("viewmatrix", C.c_void_p), ("projmatrix", C.c_void_p), ("projmatrix_inv", C.c_void_p),
+                ("cam_pos", C.c_void_p)]
+
+
+class FrameLayer(C.Structure):
+    """rgs_frame_layer of include/rgs.h."""
+    _fields_ = [("P", C.c_int), ("D", C.c_int), ("M", C.c_int), ("R", C.c_int),
+                ("means3D", C.c_void_p), ("shs", C.c_void_p), ("colors_precomp", C.c_void_p), ("opacities", C.c_void_p),
+                ("scales", C.c_void_p), ("rotations", C.c_void_p), ("cov3D_precomp", C.c_void_p),
+                ("scale_modifier", C.c_float),
+                ("background", C.c_void_p), ("range_low", C.c_void_p), ("range_up", C.c_void_p), ("radii", C.c_void_p),
+                ("geom_ws", C.c_void_p), ("binning_ws", C.c_void_p), ("image_ws", C.c_void_p),
+                ("geom_bytes", C.c_size_t), ("binning_bytes", C.c_size_t), ("image_bytes", C.c_size_t),
+                ("out_color", C.c_void_p), ("out_depth", C.c_void_p), ("out_alpha", C.c_void_p),
+                ("dL_dpix", C.c_void_p), ("dL_dpix_depth", C.c_void_p), ("dL_dalphas", C.c_void_p),
+                ("grad_accum", C.c_void_p), ("dL_dmean2D", C.c_void_p), ("dL_dopacity", C.c_void_p),
+                ("dL_dcolor", C.c_void_p), ("dL_dmean3D", C.c_void_p), ("dL_dcov3D", C.c_void_p), ("dL_dsh", C.c_void_p),
+                ("dL_dscale", C.c_void_p), ("dL_drot", C.c_void_p), ("outputs_zeroed", C.c_int),
+                ("clear", C.c_void_p * 2), ("clear_bytes", C.c_size_t * 2), ("stream", C.c_void_p)]
 
 
 class RgsError(RuntimeError):
@@ -74,6 +98,9 @@ def _load():
     lib.rgs_inclusive_sum.argtypes = [vp, vp, sz, vp, vp]
     lib.rgs_sort_pairs.argtypes = [vp, vp, vp, vp, sz, i, vp, vp]
     lib.rgs_sort_pairs_static.argtypes = [vp, vp, vp, vp, sz, i, vp]
+    lib.rgs_frame_forward_geom.argtypes = [i, C.POINTER(FrameLayer), C.POINTER(FrameView), vp, vp, i]
+    lib.rgs_frame_forward_raster.argtypes = [i, C.POINTER(FrameLayer), C.POINTER(FrameView), vp, i]
+    lib.rgs_frame_backward.argtypes = [i, C.POINTER(FrameLayer), C.POINTER(FrameView), vp, i]
     lib.rgs_sort_fault.argtypes = [vp]
     lib.rgs_set_lookback_spin_limit.argtypes = [i]
     pp = C.POINTER(vp)
@@ -98,7 +125,8 @@ def _load():
                  "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
                  "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step",
                  "rgs_activate_forward", "rgs_activate_backward", "rgs_sort_pairs_static", "rgs_sort_fault",
-                 "rgs_set_lookback_spin_limit"):
+                 "rgs_set_lookback_spin_limit", "rgs_frame_forward_geom", "rgs_frame_forward_raster",
+                 "rgs_frame_backward"):
         getattr(lib, name).restype = i
     return lib
 
@@ -112,7 +140,9 @@ EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_byte
            "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",
            "rgs_straddler_select", "rgs_merge_rows", "rgs_merge_rows_backward", "rgs_loss_workspace_bytes",
            "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step", "rgs_activate_forward",
-           "rgs_activate_backward", "rgs_sort_pairs_static", "rgs_sort_fault", "rgs_set_lookback_spin_limit")
+           "rgs_activate_backward", "rgs_sort_pairs_static", "rgs_sort_fault", "rgs_set_lookback_spin_limit",
+           "rgs_frame_forward_geom", "rgs_frame_forward_raster", "rgs_frame_backward")
+MAX_FRAME_LAYERS = 64
 STATIC_SORT_MAX_PAIRS = 1 << 22
 WORK_COUNTERS = 8
 

@@ -212,7 +212,7 @@ size_t geom_layout(size_t P, size_t* off)
 	off[RGS_GEOM_POINT_OFFSETS] = c.take(4 * P);
 	off[RGS_GEOM_CLAMPED] = c.take(P);
 	off[RGS_GEOM_BLOCK_SUMS] = c.take(4 * ((P + 255) / 256 + 1));
-	off[RGS_GEOM_TOTAL] = c.take(4);
+	off[RGS_GEOM_TOTAL] = c.take(4 * (1 + RGS_MAX_FRAME_LAYERS));  // + where the first layer of a frame gathers every layer's count
 	off[RGS_GEOM_BLEND_RECORD] = c.take(64 * P);
 	off[RGS_GEOM_DEPTH_ORDER] = c.take(4 * P);
 	off[RGS_GEOM_BLOCK_VISIBLE] = c.take(4 * ((P + 255) / 256 + 1));
@@ -231,7 +231,7 @@ int tile_key_bits(int width, int height)
 
 // Physical buffers: A receives the duplicated keys, B is its ping-pong partner.
 struct BinningPhysical {
-	size_t keys_a, keys_b, vals_a, vals_b, temp, strip_lists, total;
+	size_t keys_a, keys_b, vals_a, vals_b, temp, strip_lists, file_tail, total;
 };
 
 BinningPhysical binning_physical(size_t R)
@@ -244,6 +244,7 @@ BinningPhysical binning_physical(size_t R)
 	b.vals_b = c.take(4 * R);
 	b.temp = c.take(4 * rgs::sort_temp_words(R));
 	b.strip_lists = c.take(16 * R);
+	b.file_tail = c.take(16 * ((R + 255) / 256));
 	b.total = c.cursor;
 	return b;
 }
@@ -252,10 +253,13 @@ size_t image_layout(int width, int height, size_t* off)
 {
 	const size_t tiles = (size_t)((width + rgs::kTile - 1) / rgs::kTile) * (size_t)((height + rgs::kTile - 1) / rgs::kTile);
 	Carver c;
-	off[RGS_IMG_RANGES] = c.take(8 * tiles + 4 * rgs::kRangeTailWords);  // + the strip class counters, cleared with it
+	// the ranges, the strip class counters and the strips' totals lie one behind the other: they are cleared together
+	off[RGS_IMG_RANGES] = c.take(8 * tiles + 4 * rgs::kRangeTailWords + 4 * 4 * tiles);
+	off[RGS_IMG_STRIP_TOTAL] = off[RGS_IMG_RANGES] + 8 * tiles + 4 * rgs::kRangeTailWords;
 	off[RGS_IMG_N_CONTRIB] = c.take(4 * (size_t)width * height);
 	off[RGS_IMG_STRIP_FILED] = c.take(4 * 4 * tiles);
 	off[RGS_IMG_STRIP_ORDER] = c.take(4 * 4 * tiles);
+	off[RGS_IMG_STRIP_ORDER_FORWARD] = c.take(4 * 4 * tiles);
 	return c.cursor;
 }
 
@@ -426,98 +430,120 @@ static hipEvent_t count_event_of_this_thread()
 	return events[dev];
 }
 
-static int forward_geom(bool wait_for_count, void* count_ready_event, const char* who, int P, int D, int M, int width, int height,
-                        const float* means3D, const float* shs, const float* colors_precomp, const float* opacities,
-                        const float* scales, float scale_modifier, const float* rotations, const float* cov3D_precomp,
-                        const float* viewmatrix, const float* projmatrix, const float* cam_pos,
-                        float tan_fovx, float tan_fovy, int prefiltered,
-                        int* radii, void* geom_ws, size_t geom_bytes,
-                        uint32_t* num_rendered_host, void* stream, int debug)
+// One layer's arguments of the geometry stage.
+struct GeomCall {
+	int P, D, M;
+	const float* means3D;
+	const float* shs;
+	const float* colors_precomp;
+	const float* opacities;
+	const float* scales;
+	float scale_modifier;
+	const float* rotations;
+	const float* cov3D_precomp;
+	int* radii;
+	void* geom_ws;
+	size_t geom_bytes;
+};
+
+// The geometry stage of `K` layers that share a camera, every kernel launched once for all of them: preprocess,
+// the instance counts (one copy to counts_host[0..K)), and, behind that copy, the depth order.
+static int forward_geom(bool wait_for_count, void* count_ready_event, const char* who, int K, const GeomCall* calls,
+                        int width, int height, const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                        float tan_fovx, float tan_fovy, uint32_t* counts_host, void* stream, int debug)
 {
-	// `prefiltered` promises that no Gaussian is culled; the reference traps the device when
-	// the promise is broken (K/cuda_rasterizer_hgs/auxiliary.h:172-176).  Here a culled
-	// Gaussian is simply skipped.
-	(void)prefiltered;
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
 	RGS_TAKE_SORT_FAULT(who);
-	RGS_REQUIRE(P > 0, "%s: P must be positive (the caller short-circuits P == 0)", who);
 	RGS_REQUIRE(width > 0 && height > 0, "%s: bad image size %dx%d", who, width, height);
-	RGS_REQUIRE(means3D && opacities && viewmatrix && projmatrix && cam_pos && radii && geom_ws && num_rendered_host,
-	            "%s: null pointer", who);
-	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr),
-	            "%s: provide exactly one of SHs or precomputed colours", who);
-	RGS_REQUIRE(((scales != nullptr) && (rotations != nullptr)) != (cov3D_precomp != nullptr) &&
-	                ((scales != nullptr) == (rotations != nullptr)),
-	            "%s: provide exactly one of scale/rotation or precomputed 3D covariance", who);
-	RGS_REQUIRE(D >= 0 && D <= 3, "%s: SH degree %d out of range", who, D);
-	RGS_REQUIRE(!shs || M >= (D + 1) * (D + 1), "%s: %d SH coefficients cannot hold degree %d", who, M, D);
-	RGS_REQUIRE(geom_bytes >= rgs_geom_bytes(P), "%s: geometry workspace too small", who);
-	RGS_REQUIRE((reinterpret_cast<uintptr_t>(geom_ws) & 15) == 0, "%s: workspace must be 16-byte aligned", who);
+	RGS_REQUIRE(viewmatrix && projmatrix && cam_pos && counts_host, "%s: null pointer", who);
+	std::vector<rgs::PreprocessArgs> pre((size_t)K);
+	std::vector<rgs::TotalsJob> totals((size_t)K);
+	std::vector<rgs::DepthOrderJob> orders((size_t)K);
+	uint32_t* frame_counts = nullptr;  // K words in the first layer's workspace, so that one copy brings all counts
+	for (int k = 0; k < K; k++) {
+		const GeomCall& c = calls[k];
+		RGS_REQUIRE(c.P > 0, "%s: P must be positive (the caller short-circuits P == 0)", who);
+		RGS_REQUIRE(c.means3D && c.opacities && c.radii && c.geom_ws, "%s: null pointer", who);
+		RGS_REQUIRE((c.shs != nullptr) != (c.colors_precomp != nullptr),
+		            "%s: provide exactly one of SHs or precomputed colours", who);
+		RGS_REQUIRE(((c.scales != nullptr) && (c.rotations != nullptr)) != (c.cov3D_precomp != nullptr) &&
+		                ((c.scales != nullptr) == (c.rotations != nullptr)),
+		            "%s: provide exactly one of scale/rotation or precomputed 3D covariance", who);
+		RGS_REQUIRE(c.D >= 0 && c.D <= 3, "%s: SH degree %d out of range", who, c.D);
+		RGS_REQUIRE(!c.shs || c.M >= (c.D + 1) * (c.D + 1), "%s: %d SH coefficients cannot hold degree %d", who, c.M, c.D);
+		RGS_REQUIRE(c.geom_bytes >= rgs_geom_bytes(c.P), "%s: geometry workspace too small", who);
+		RGS_REQUIRE((reinterpret_cast<uintptr_t>(c.geom_ws) & 15) == 0, "%s: workspace must be 16-byte aligned", who);
 
-	size_t off[RGS_GEOM_FIELDS];
-	geom_layout((size_t)P, off);
+		size_t off[RGS_GEOM_FIELDS];
+		geom_layout((size_t)c.P, off);
+		void* ws = c.geom_ws;
+		if (k == 0)
+			frame_counts = at<uint32_t>(ws, off[RGS_GEOM_TOTAL]) + 1;
+		rgs::PreprocessArgs& a = pre[(size_t)k];
+		a.P = c.P; a.D = c.D; a.M = c.M;
+		a.means = c.means3D; a.scales = c.scales; a.scale_modifier = c.scale_modifier; a.rotations = c.rotations;
+		a.opacities = c.opacities; a.shs = c.shs; a.cov3D_precomp = c.cov3D_precomp; a.colors_precomp = c.colors_precomp;
+		a.view = viewmatrix; a.proj = projmatrix; a.campos = cam_pos;
+		a.W = width; a.H = height;
+		a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
+		// K/cuda_rasterizer_hgs/rasterizer_impl.cu:227-228
+		a.focal_y = height / (2.0f * tan_fovy);
+		a.focal_x = width / (2.0f * tan_fovx);
+		a.grid_x = (width + rgs::kTile - 1) / rgs::kTile;
+		a.grid_y = (height + rgs::kTile - 1) / rgs::kTile;
+		a.radii = c.radii;
+		a.xy = at<float2>(ws, off[RGS_GEOM_XY]);
+		a.clip_w = at<float>(ws, off[RGS_GEOM_CLIP_W]);
+		a.depths = at<float>(ws, off[RGS_GEOM_DEPTHS]);
+		a.cov3D = at<float>(ws, off[RGS_GEOM_COV3D]);
+		a.rgb = at<float>(ws, off[RGS_GEOM_RGB]);
+		a.conic_opacity = at<float4>(ws, off[RGS_GEOM_CONIC_OPACITY]);
+		a.tiles_touched = at<uint32_t>(ws, off[RGS_GEOM_TILES_TOUCHED]);
+		a.clamped = at<uint8_t>(ws, off[RGS_GEOM_CLAMPED]);
+		a.block_sums = at<uint32_t>(ws, off[RGS_GEOM_BLOCK_SUMS]);
+		a.blend_record = at<float4>(ws, off[RGS_GEOM_BLEND_RECORD]);
+		a.block_visible = at<uint32_t>(ws, off[RGS_GEOM_BLOCK_VISIBLE]);
+		a.sh_rows_by_16_bytes = sh_rows_by_16_bytes(c.shs, c.M, c.D);
+		const OrderScratch o = order_scratch((size_t)c.P);
+		char* scratch = at<char>(ws, off[RGS_GEOM_ORDER_SCRATCH]);
+		a.clear = at<uint32_t>(scratch, o.sort_temp);
+		a.clear_words = rgs::sort_clear_words((size_t)c.P, 32);
 
-	rgs::PreprocessArgs a;
-	a.P = P; a.D = D; a.M = M;
-	a.means = means3D; a.scales = scales; a.scale_modifier = scale_modifier; a.rotations = rotations;
-	a.opacities = opacities; a.shs = shs; a.cov3D_precomp = cov3D_precomp; a.colors_precomp = colors_precomp;
-	a.view = viewmatrix; a.proj = projmatrix; a.campos = cam_pos;
-	a.W = width; a.H = height;
-	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
-	// K/cuda_rasterizer_hgs/rasterizer_impl.cu:227-228
-	a.focal_y = height / (2.0f * tan_fovy);
-	a.focal_x = width / (2.0f * tan_fovx);
-	a.grid_x = (width + rgs::kTile - 1) / rgs::kTile;
-	a.grid_y = (height + rgs::kTile - 1) / rgs::kTile;
-	a.radii = radii;
-	a.xy = at<float2>(geom_ws, off[RGS_GEOM_XY]);
-	a.clip_w = at<float>(geom_ws, off[RGS_GEOM_CLIP_W]);
-	a.depths = at<float>(geom_ws, off[RGS_GEOM_DEPTHS]);
-	a.cov3D = at<float>(geom_ws, off[RGS_GEOM_COV3D]);
-	a.rgb = at<float>(geom_ws, off[RGS_GEOM_RGB]);
-	a.conic_opacity = at<float4>(geom_ws, off[RGS_GEOM_CONIC_OPACITY]);
-	a.tiles_touched = at<uint32_t>(geom_ws, off[RGS_GEOM_TILES_TOUCHED]);
-	a.clamped = at<uint8_t>(geom_ws, off[RGS_GEOM_CLAMPED]);
-	a.block_sums = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_SUMS]);
-	a.blend_record = at<float4>(geom_ws, off[RGS_GEOM_BLEND_RECORD]);
-	a.block_visible = at<uint32_t>(geom_ws, off[RGS_GEOM_BLOCK_VISIBLE]);
-	a.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D);
-
-	const OrderScratch order = order_scratch((size_t)P);
-	a.clear = at<uint32_t>(at<char>(geom_ws, off[RGS_GEOM_ORDER_SCRATCH]), order.sort_temp);
-	a.clear_words = rgs::sort_clear_words((size_t)P, 32);
-	rgs::launch_preprocess_forward(a, s);
+		totals[(size_t)k] = rgs::TotalsJob{a.block_sums, a.block_visible, c.P, at<uint32_t>(ws, off[RGS_GEOM_TOTAL]),
+		                                   frame_counts + k, at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_COUNT])};
+		rgs::DepthOrderJob& d = orders[(size_t)k];
+		d.P = c.P;
+		d.depths = a.depths; d.tiles_touched = a.tiles_touched; d.block_visible = a.block_visible;
+		d.visible_count = at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_COUNT]);
+		d.visible_list = at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_LIST]);
+		d.keys_a = at<uint32_t>(scratch, o.keys_a); d.keys_b = at<uint32_t>(scratch, o.keys_b);
+		d.order = at<uint32_t>(ws, off[RGS_GEOM_DEPTH_ORDER]); d.vals_b = at<uint32_t>(scratch, o.vals_b);
+		d.tiles_in_order = at<uint32_t>(scratch, o.tiles_in_order);
+		d.offsets_in_order = at<uint32_t>(ws, off[RGS_GEOM_POINT_OFFSETS]);
+		d.sort_temp = at<uint32_t>(scratch, o.sort_temp); d.scan_temp = at<uint32_t>(scratch, o.scan_temp);
+	}
+	rgs::launch_preprocess_forward(pre.data(), K, s);
 	RGS_STAGE("preprocess");
-	rgs::launch_totals_from_block_sums(a.block_sums, a.block_visible, P, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]),
-	                                   at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_COUNT]), s);
+	rgs::launch_totals_from_block_sums(totals.data(), K, s);
 	RGS_STAGE("instance count");
-	hipError_t e = hipMemcpyAsync(num_rendered_host, at<uint32_t>(geom_ws, off[RGS_GEOM_TOTAL]), sizeof(uint32_t),
-	                              hipMemcpyDeviceToHost, s);
-	// the host only needs the count: it waits for this event, not for the kernels queued below
+	hipError_t e = hipMemcpyAsync(counts_host, frame_counts, sizeof(uint32_t) * (size_t)K, hipMemcpyDeviceToHost, s);
+	// the host only needs the counts: it waits for this event, not for the kernels queued below
 	hipEvent_t ready = wait_for_count ? count_event_of_this_thread() : static_cast<hipEvent_t>(count_ready_event);
 	if (e == hipSuccess && ready)
 		e = hipEventRecord(ready, s);
-	{
-		// depth order of the Gaussians and the offsets of their instances in that order: needs
-		// nothing from the host, so it is queued behind the count's copy
-		const OrderScratch& o = order;
-		char* scratch = at<char>(geom_ws, off[RGS_GEOM_ORDER_SCRATCH]);
-		rgs::launch_depth_order(P, a.depths, a.tiles_touched, a.block_visible, at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_COUNT]),
-		                        at<uint32_t>(geom_ws, off[RGS_GEOM_VISIBLE_LIST]),
-		                        at<uint32_t>(scratch, o.keys_a), at<uint32_t>(scratch, o.keys_b),
-		                        at<uint32_t>(geom_ws, off[RGS_GEOM_DEPTH_ORDER]), at<uint32_t>(scratch, o.vals_b),
-		                        at<uint32_t>(scratch, o.tiles_in_order), at<uint32_t>(geom_ws, off[RGS_GEOM_POINT_OFFSETS]),
-		                        at<uint32_t>(scratch, o.sort_temp), at<uint32_t>(scratch, o.scan_temp), s);
-		RGS_STAGE("depth order");
-	}
+	// depth order of the Gaussians and the offsets of their instances in that order: needs
+	// nothing from the host, so it is queued behind the counts' copy
+	rgs::launch_depth_order(orders.data(), K, s);
+	RGS_STAGE("depth order");
 	if (e == hipSuccess && wait_for_count)
 		e = ready ? hipEventSynchronize(ready) : hipStreamSynchronize(s);
 	if (e != hipSuccess)
 		return fail("%s: reading the instance count failed: %s", who, hipGetErrorString(e));
 	if (wait_for_count)
-		RGS_REQUIRE(*num_rendered_host < 0x40000000u,
-		            "%s: %u (Gaussian, tile) instances exceed the 2^30 limit of the sort", who, *num_rendered_host);
+		for (int k = 0; k < K; k++)
+			RGS_REQUIRE(counts_host[k] < 0x40000000u, "%s: %u (Gaussian, tile) instances exceed the 2^30 limit of the sort", who,
+			            counts_host[k]);
 	return 0;
 }
 
@@ -529,9 +555,16 @@ int rgs_forward_geom(int P, int D, int M, int width, int height,
                      int* radii, void* geom_ws, size_t geom_bytes,
                      uint32_t* num_rendered_host, void* stream, int debug)
 {
-	return forward_geom(true, nullptr, "rgs_forward_geom", P, D, M, width, height, means3D, shs, colors_precomp, opacities, scales,
-	                    scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, cam_pos, tan_fovx, tan_fovy,
-	                    prefiltered, radii, geom_ws, geom_bytes, num_rendered_host, stream, debug);
+	// `prefiltered` promises that no Gaussian is culled; the reference traps the device when
+	// the promise is broken (K/cuda_rasterizer_hgs/auxiliary.h:172-176).  Here a culled
+	// Gaussian is simply skipped.
+	(void)prefiltered;
+	RGS_REQUIRE(P > 0, "rgs_forward_geom: P must be positive (the caller short-circuits P == 0)");
+	RGS_REQUIRE(num_rendered_host, "rgs_forward_geom: null pointer");
+	const GeomCall c = {P, D, M, means3D, shs, colors_precomp, opacities, scales, scale_modifier, rotations, cov3D_precomp, radii,
+	                    geom_ws, geom_bytes};
+	return forward_geom(true, nullptr, "rgs_forward_geom", 1, &c, width, height, viewmatrix, projmatrix, cam_pos, tan_fovx,
+	                    tan_fovy, num_rendered_host, stream, debug);
 }
 
 int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
@@ -542,9 +575,13 @@ int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
                              int* radii, void* geom_ws, size_t geom_bytes,
                              uint32_t* num_rendered_pinned, void* count_ready_event, void* stream, int debug)
 {
-	return forward_geom(false, count_ready_event, "rgs_forward_geom_enqueue", P, D, M, width, height, means3D, shs, colors_precomp, opacities,
-	                    scales, scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, cam_pos, tan_fovx,
-	                    tan_fovy, prefiltered, radii, geom_ws, geom_bytes, num_rendered_pinned, stream, debug);
+	(void)prefiltered;
+	RGS_REQUIRE(P > 0, "rgs_forward_geom_enqueue: P must be positive (the caller short-circuits P == 0)");
+	RGS_REQUIRE(num_rendered_pinned, "rgs_forward_geom_enqueue: null pointer");
+	const GeomCall c = {P, D, M, means3D, shs, colors_precomp, opacities, scales, scale_modifier, rotations, cov3D_precomp, radii,
+	                    geom_ws, geom_bytes};
+	return forward_geom(false, count_ready_event, "rgs_forward_geom_enqueue", 1, &c, width, height, viewmatrix, projmatrix, cam_pos,
+	                    tan_fovx, tan_fovy, num_rendered_pinned, stream, debug);
 }
 
 
@@ -552,82 +589,18 @@ int rgs_forward_geom_enqueue(int P, int D, int M, int width, int height,
 
 namespace {
 
-// `R` sizes the binning workspace and the launches.  With count_on_device the number of instances
-// is the smaller of R and the count the geometry stage left in its workspace, read by the kernels.
-int forward_raster(bool count_on_device, int P, int R, int width, int height,
-                   const float* background, float tan_fovx, float tan_fovy,
-                   const float* projmatrix_inv, const float* range_low, const float* range_up,
-                   const float* colors_precomp, const int* radii,
-                   void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
-                   void* image_ws, size_t image_bytes,
-                   float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
+// The blend kernels' view of one call's workspaces (everything but the outputs and the gradients).
+void fill_blend_args(rgs::BlendArgs& a, int P, int R, int width, int height, float tan_fovx, float tan_fovy,
+                     const float* background, const float* projmatrix_inv, const float* range_low, const float* range_up,
+                     const float* colors_precomp, const void* geom_ws, const void* binning_ws, const void* image_ws)
 {
-	hipStream_t s = static_cast<hipStream_t>(stream);
-	EntryScope scope_(s);
-	RGS_TAKE_SORT_FAULT("rgs_forward_raster");
-	RGS_REQUIRE(P > 0 && R >= 0, "rgs_forward_raster: bad sizes P=%d R=%d", P, R);
-	RGS_REQUIRE(R < 0x40000000, "rgs_forward_raster: %d (Gaussian, tile) instances exceed the 2^30 limit of the sort", R);
-	RGS_REQUIRE(width > 0 && height > 0, "rgs_forward_raster: bad image size %dx%d", width, height);
-	RGS_REQUIRE(background && projmatrix_inv && range_low && range_up && radii && geom_ws && image_ws && out_color &&
-	                out_depth && out_alpha,
-	            "rgs_forward_raster: null pointer");
-	RGS_REQUIRE(R == 0 || binning_ws, "rgs_forward_raster: null binning workspace");
-	RGS_REQUIRE(geom_bytes >= rgs_geom_bytes(P), "rgs_forward_raster: geometry workspace too small");
-	RGS_REQUIRE(R == 0 || binning_bytes >= rgs_binning_bytes(R), "rgs_forward_raster: binning workspace too small");
-	RGS_REQUIRE(image_bytes >= rgs_image_bytes(width, height), "rgs_forward_raster: image workspace too small");
-
 	size_t goff[RGS_GEOM_FIELDS], ioff[RGS_IMG_FIELDS];
 	geom_layout((size_t)P, goff);
 	image_layout(width, height, ioff);
 	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
-	uint2* ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
-	const uint32_t* point_list = nullptr;
-
-	if (R > 0) {
-		const BinningPhysical b = binning_physical((size_t)R);
-		uint32_t* keys_a = at<uint32_t>(binning_ws, b.keys_a);
-		uint32_t* keys_b = at<uint32_t>(binning_ws, b.keys_b);
-		uint32_t* vals_a = at<uint32_t>(binning_ws, b.vals_a);
-		uint32_t* vals_b = at<uint32_t>(binning_ws, b.vals_b);
-		const uint32_t* order_status =
-		    rgs::sort_status_word(at<uint32_t>(at<char>(geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).sort_temp));
-		const uint32_t* count = count_on_device ? at<uint32_t>(geom_ws, goff[RGS_GEOM_TOTAL]) : nullptr;
-		rgs::launch_duplicate_with_keys(P, at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]),
-		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_DEPTH_ORDER]),
-		                                at<uint32_t>(geom_ws, goff[RGS_GEOM_POINT_OFFSETS]), at<float2>(geom_ws, goff[RGS_GEOM_XY]),
-		                                radii, gx, gy, keys_a, vals_a, (uint32_t)R, at<uint32_t>(binning_ws, b.temp),
-		                                rgs::sort_clear_words((size_t)R, tile_key_bits(width, height)), s);
-		RGS_STAGE("duplicate_with_keys");
-		const int end_bit = tile_key_bits(width, height);
-		// the first kernel of the sort also clears the tile ranges (and the counters behind them)
-		rgs::launch_sort_pairs_u32(keys_a, keys_b, vals_a, vals_b, (size_t)R, count, end_bit, at<uint32_t>(binning_ws, b.temp),
-		                           true, reinterpret_cast<uint32_t*>(ranges), (size_t)gx * gy * 2 + rgs::kRangeTailWords,
-		                           "sort", s);
-		RGS_STAGE("sort_pairs");
-		const bool sorted_in_a = (((end_bit + 7) / 8) % 2) == 0;
-		if (debug) {
-			uint32_t status = 0, status2 = 0;
-			hipError_t e = hipMemcpy(&status, rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), sizeof(status),
-			                         hipMemcpyDeviceToHost);
-			if (e == hipSuccess)
-				e = hipMemcpy(&status2, order_status, sizeof(status2), hipMemcpyDeviceToHost);
-			status |= status2;
-			if (e != hipSuccess || status != 0)
-				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
-		}
-		rgs::launch_tile_ranges(sorted_in_a ? keys_a : keys_b, (size_t)R, count, ranges, gx * gy,
-		                        rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp)), order_status, fault_word(true), true, s);
-		RGS_STAGE("tile_ranges");
-		point_list = sorted_in_a ? vals_a : vals_b;
-	} else {
-		rgs::launch_tile_ranges(nullptr, 0, nullptr, ranges, gx * gy, nullptr, nullptr, nullptr, false, s);
-		RGS_STAGE("tile_ranges");
-	}
-
-	rgs::BlendArgs a;
 	memset(&a, 0, sizeof(a));
-	a.ranges = ranges;
-	a.point_list = point_list;
+	void* img = const_cast<void*>(image_ws);
+	a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
 	a.W = width; a.H = height; a.grid_x = gx; a.grid_y = gy;
 	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
 	a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up; a.bg = background;
@@ -637,14 +610,275 @@ int forward_raster(bool count_on_device, int P, int R, int width, int height,
 	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
 	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
 	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
+	a.n_contrib = at<uint32_t>(img, ioff[RGS_IMG_N_CONTRIB]);
+	a.strip_filed = at<uint32_t>(img, ioff[RGS_IMG_STRIP_FILED]);
+	a.strip_order = at<uint32_t>(img, ioff[RGS_IMG_STRIP_ORDER]);
+	a.strip_order_forward = at<uint32_t>(img, ioff[RGS_IMG_STRIP_ORDER_FORWARD]);
+	a.strip_total = at<uint32_t>(img, ioff[RGS_IMG_STRIP_TOTAL]);
+	a.strip_classes = reinterpret_cast<uint32_t*>(at<uint2>(img, ioff[RGS_IMG_RANGES])) + 2 * (size_t)gx * gy;
+	a.capacity = (uint32_t)R;
+	if (R > 0) {
+		const BinningPhysical b = binning_physical((size_t)R);
+		const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
+		void* bin = const_cast<void*>(binning_ws);
+		a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
+		a.tile_keys = at<uint32_t>(binning_ws, sorted_in_a ? b.keys_a : b.keys_b);
+		a.strip_lists = at<uint32_t>(bin, b.strip_lists);
+		a.file_tail = at<uint4>(binning_ws, b.file_tail);
+		a.sort_status = rgs::sort_status_word(at<uint32_t>(binning_ws, b.temp));
+		a.order_status = rgs::sort_status_word(at<uint32_t>(at<char>(geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).sort_temp));
+	}
+}
+
+// One layer's arguments of the second half of the forward.
+struct RasterCall {
+	int P, R;
+	const float* background;
+	const float* range_low;
+	const float* range_up;
+	const float* colors_precomp;
+	void* geom_ws;
+	size_t geom_bytes;
+	void* binning_ws;
+	size_t binning_bytes;
+	void* image_ws;
+	size_t image_bytes;
+};
+
+// Second half of the forward up to the blend, for `K` layers that share a camera, every kernel launched once for
+// all of them: key duplication, the instance sort, tile ranges, the strips' lists.  A layer's R sizes its binning
+// workspace and its share of the launches.  With count_on_device the number of instances is the smaller of R and
+// the count the geometry stage left in the layer's workspace, read by the kernels.  Fills jobs[k] for the blend.
+int forward_binning(const char* who, bool count_on_device, int K, const RasterCall* calls, int width, int height,
+                    float tan_fovx, float tan_fovy, const float* projmatrix_inv, rgs::BlendArgs* jobs, hipStream_t s, int debug)
+{
+	RGS_TAKE_SORT_FAULT(who);
+	RGS_REQUIRE(width > 0 && height > 0, "%s: bad image size %dx%d", who, width, height);
+	RGS_REQUIRE((uint64_t)((width + rgs::kTile - 1) / rgs::kTile) * (uint64_t)((height + rgs::kTile - 1) / rgs::kTile) <
+	                (1ull << rgs::kKeyTileBits),
+	            "%s: a %dx%d image has 2^%d tiles or more", who, width, height, rgs::kKeyTileBits);
+	RGS_REQUIRE(projmatrix_inv, "%s: null pointer", who);
+	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
+	const int end_bit = tile_key_bits(width, height);
+	// the tile ranges, the strip class counters and the strips' totals, cleared together
+	const size_t clear_words = (size_t)gx * gy * 2 + rgs::kRangeTailWords + (size_t)gx * gy * 4;
+	std::vector<rgs::DuplicateJob> dups;
+	std::vector<rgs::SortJob<uint32_t>> sorts;
+	std::vector<rgs::TileRangesJob> ranges_jobs;
+	std::vector<int> with_instances;
+	uint32_t* fault = fault_word(true);
+	for (int k = 0; k < K; k++) {
+		const RasterCall& c = calls[k];
+		const int P = c.P, R = c.R;
+		RGS_REQUIRE(P > 0 && R >= 0, "%s: bad sizes P=%d R=%d", who, P, R);
+		RGS_REQUIRE(R < 0x40000000, "%s: %d (Gaussian, tile) instances exceed the 2^30 limit of the sort", who, R);
+		RGS_REQUIRE(c.background && c.range_low && c.range_up && c.geom_ws && c.image_ws, "%s: null pointer", who);
+		RGS_REQUIRE(R == 0 || c.binning_ws, "%s: null binning workspace", who);
+		RGS_REQUIRE(c.geom_bytes >= rgs_geom_bytes(P), "%s: geometry workspace too small", who);
+		RGS_REQUIRE(R == 0 || c.binning_bytes >= rgs_binning_bytes(R), "%s: binning workspace too small", who);
+		RGS_REQUIRE(c.image_bytes >= rgs_image_bytes(width, height), "%s: image workspace too small", who);
+		rgs::BlendArgs& a = jobs[k];
+		fill_blend_args(a, P, R, width, height, tan_fovx, tan_fovy, c.background, projmatrix_inv, c.range_low, c.range_up,
+		                c.colors_precomp, c.geom_ws, c.binning_ws, c.image_ws);
+		uint2* ranges = const_cast<uint2*>(a.ranges);
+		if (R == 0) {
+			rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, clear_words, s);
+			RGS_STAGE("tile_ranges");
+			continue;
+		}
+		size_t goff[RGS_GEOM_FIELDS];
+		geom_layout((size_t)P, goff);
+		const BinningPhysical b = binning_physical((size_t)R);
+		uint32_t* keys_a = at<uint32_t>(c.binning_ws, b.keys_a);
+		uint32_t* keys_b = at<uint32_t>(c.binning_ws, b.keys_b);
+		uint32_t* vals_a = at<uint32_t>(c.binning_ws, b.vals_a);
+		uint32_t* vals_b = at<uint32_t>(c.binning_ws, b.vals_b);
+		uint32_t* temp = at<uint32_t>(c.binning_ws, b.temp);
+		const uint32_t* count = count_on_device ? at<uint32_t>(c.geom_ws, goff[RGS_GEOM_TOTAL]) : nullptr;
+		a.count_device = count;
+		rgs::DuplicateJob d;
+		d.P = P;
+		d.visible_count = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
+		d.order = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_DEPTH_ORDER]);
+		d.offsets = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_POINT_OFFSETS]);
+		d.filing.record = a.record;
+		d.filing.projinv = projmatrix_inv; d.filing.range_low = c.range_low; d.filing.range_up = c.range_up;
+		d.filing.tanfovx = tan_fovx; d.filing.tanfovy = tan_fovy;
+		d.filing.W = width; d.filing.H = height;
+		d.keys = keys_a; d.values = vals_a; d.capacity = (uint32_t)R;
+		d.clear = temp; d.clear_words = rgs::sort_clear_words((size_t)R, end_bit);
+		dups.push_back(d);
+		// the first kernel of the sort also clears the tile ranges (and the counters and totals behind them)
+		sorts.push_back(rgs::SortJob<uint32_t>{keys_a, keys_b, vals_a, vals_b, (size_t)R, count, temp,
+		                                       reinterpret_cast<uint32_t*>(ranges), clear_words});
+		ranges_jobs.push_back(rgs::TileRangesJob{a.tile_keys, (size_t)R, count, ranges, a.sort_status, a.order_status, fault,
+		                                         at<uint4>(c.binning_ws, b.file_tail)});
+		with_instances.push_back(k);
+	}
+	if (with_instances.empty())
+		return 0;
+	const int n = (int)with_instances.size();
+	rgs::launch_duplicate_with_keys(dups.data(), n, gx, gy, s);
+	RGS_STAGE("duplicate_with_keys");
+	rgs::launch_sort_pairs_u32(sorts.data(), n, end_bit, true, "sort", s);
+	RGS_STAGE("sort_pairs");
+	if (debug)
+		for (int k : with_instances) {
+			uint32_t status = 0, status2 = 0;
+			hipError_t e = hipMemcpy(&status, jobs[k].sort_status, sizeof(status), hipMemcpyDeviceToHost);
+			if (e == hipSuccess)
+				e = hipMemcpy(&status2, jobs[k].order_status, sizeof(status2), hipMemcpyDeviceToHost);
+			status |= status2;
+			if (e != hipSuccess || status != 0)
+				return fail("sort_pairs: %s", e != hipSuccess ? hipGetErrorString(e) : "a look-back wait timed out");
+		}
+	rgs::launch_tile_ranges(ranges_jobs.data(), n, s);
+	RGS_STAGE("tile_ranges");
+	std::vector<rgs::BlendArgs> filing((size_t)n);
+	for (int i = 0; i < n; i++)
+		filing[(size_t)i] = jobs[with_instances[(size_t)i]];
+	rgs::launch_strip_filing(filing.data(), n, s);
+	RGS_STAGE("strip_filing");
+	return 0;
+}
+
+int forward_raster(bool count_on_device, int P, int R, int width, int height,
+                   const float* background, float tan_fovx, float tan_fovy,
+                   const float* projmatrix_inv, const float* range_low, const float* range_up,
+                   const float* colors_precomp, const int* radii,
+                   void* geom_ws, size_t geom_bytes, void* binning_ws, size_t binning_bytes,
+                   void* image_ws, size_t image_bytes,
+                   float* out_color, float* out_depth, float* out_alpha, void* stream, int debug)
+{
+	(void)radii;  // the key duplication reads the radius from the Gaussian's packed record
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	RGS_REQUIRE(out_color && out_depth && out_alpha, "rgs_forward_raster: null pointer");
+	rgs::BlendArgs a;
+	const RasterCall c = {P, R, background, range_low, range_up, colors_precomp, geom_ws, geom_bytes, binning_ws, binning_bytes,
+	                      image_ws, image_bytes};
+	if (int rc = forward_binning("rgs_forward_raster", count_on_device, 1, &c, width, height, tan_fovx, tan_fovy, projmatrix_inv,
+	                             &a, s, debug))
+		return rc;
 	a.out_color = out_color; a.out_depth = out_depth; a.out_alpha = out_alpha;
-	a.n_contrib = at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]);
-	a.strip_filed = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_FILED]);
-	a.strip_order = at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_ORDER]);
-	a.strip_lists = R > 0 ? at<uint32_t>(binning_ws, binning_physical((size_t)R).strip_lists) : nullptr;
-	a.strip_classes = reinterpret_cast<uint32_t*>(ranges) + 2 * (size_t)gx * gy;
-	rgs::launch_blend_forward(a, s);
+	rgs::launch_blend_forward(&a, 1, s);
 	RGS_STAGE("blend_forward");
+	return 0;
+}
+
+// The per-Gaussian half of the backward: fused cov2D / preprocess backward over the rendered Gaussians.
+void fill_backward_geometry(rgs::PreprocessBackwardArgs& p, int P, int D, int M, int width, int height, const float* means3D,
+                            const float* shs, const float* scales, float scale_modifier, const float* rotations,
+                            const float* cov3D_precomp, const float* viewmatrix, const float* projmatrix, const float* cam_pos,
+                            float tan_fovx, float tan_fovy, const int* radii, const void* geom_ws, const float* grad_accum,
+                            float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D, float* dL_dcov3D,
+                            float* dL_dsh, float* dL_dscale, float* dL_drot)
+{
+	size_t goff[RGS_GEOM_FIELDS];
+	geom_layout((size_t)P, goff);
+	memset(&p, 0, sizeof(p));
+	p.P = P; p.D = D; p.M = M;
+	p.means = means3D; p.radii = radii; p.shs = shs;
+	p.clamped = at<uint8_t>(geom_ws, goff[RGS_GEOM_CLAMPED]);
+	p.scales = scales; p.rotations = rotations; p.scale_modifier = scale_modifier;
+	p.cov3D = cov3D_precomp ? cov3D_precomp : at<float>(geom_ws, goff[RGS_GEOM_COV3D]);
+	p.view = viewmatrix; p.proj = projmatrix; p.campos = cam_pos;
+	p.focal_y = height / (2.0f * tan_fovy);
+	p.focal_x = width / (2.0f * tan_fovx);
+	p.tanfovx = tan_fovx; p.tanfovy = tan_fovy;
+	p.sums = grad_accum;
+	p.dL_dmean2D = dL_dmean2D; p.dL_dopacity = dL_dopacity; p.dL_dcolor = dL_dcolor;
+	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
+	p.visible_list = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_LIST]);
+	p.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D) && (reinterpret_cast<uintptr_t>(dL_dsh) & 15) == 0;
+	p.visible_count = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
+}
+
+// Events for ordering a frame's stream against its layers' own streams: a few per host thread and device, reused.
+hipEvent_t frame_event(size_t i)
+{
+	static thread_local std::vector<hipEvent_t> events[kMaxDevices];
+	const int dev = current_device();
+	if (dev < 0)
+		return nullptr;
+	std::vector<hipEvent_t>& v = events[dev];
+	while (v.size() <= i) {
+		hipEvent_t e = nullptr;
+		if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess)
+			return nullptr;
+		v.push_back(e);
+	}
+	return v[i];
+}
+
+// The distinct streams among the layers' own that are not the frame's.
+std::vector<hipStream_t> side_streams(int K, const rgs_frame_layer* layers, hipStream_t frame)
+{
+	std::vector<hipStream_t> out;
+	for (int k = 0; k < K; k++) {
+		hipStream_t ls = static_cast<hipStream_t>(layers[k].stream);
+		if (!ls || ls == frame)
+			continue;
+		bool seen = false;
+		for (hipStream_t o : out)
+			seen = seen || o == ls;
+		if (!seen)
+			out.push_back(ls);
+	}
+	return out;
+}
+
+// Work queued on the layers' streams from here on starts after what the frame's stream holds now.
+int side_streams_wait_for(int K, const rgs_frame_layer* layers, hipStream_t frame, const char* who)
+{
+	const std::vector<hipStream_t> sides = side_streams(K, layers, frame);
+	if (sides.empty())
+		return 0;
+	hipEvent_t e = frame_event(0);
+	hipError_t rc = e ? hipEventRecord(e, frame) : hipErrorUnknown;
+	for (size_t i = 0; rc == hipSuccess && i < sides.size(); i++)
+		rc = hipStreamWaitEvent(sides[i], e, 0);
+	if (rc != hipSuccess)
+		return fail("%s: ordering the layers' streams failed: %s", who, hipGetErrorString(rc));
+	return 0;
+}
+
+// Work queued on the frame's stream from here on starts after what the layers' streams hold now.
+int wait_for_side_streams(int K, const rgs_frame_layer* layers, hipStream_t frame, const char* who)
+{
+	const std::vector<hipStream_t> sides = side_streams(K, layers, frame);
+	hipError_t rc = hipSuccess;
+	for (size_t i = 0; rc == hipSuccess && i < sides.size(); i++) {
+		hipEvent_t e = frame_event(1 + i);
+		rc = e ? hipEventRecord(e, sides[i]) : hipErrorUnknown;
+		if (rc == hipSuccess)
+			rc = hipStreamWaitEvent(frame, e, 0);
+	}
+	if (rc != hipSuccess)
+		return fail("%s: ordering the layers' streams failed: %s", who, hipGetErrorString(rc));
+	return 0;
+}
+
+int check_backward_pointers(const char* who, int P, int R, int width, int height, const float* background,
+                            const float* means3D, const float* shs, const float* colors_precomp, const float* alphas,
+                            const float* scales, const float* rotations, const float* cov3D_precomp, const float* viewmatrix,
+                            const float* projmatrix, const float* projmatrix_inv, const float* range_low,
+                            const float* range_up, const float* cam_pos, const int* radii, const void* geom_ws,
+                            const void* binning_ws, const void* image_ws, const float* dL_dpix, const float* grad_accum,
+                            const float* dL_dmean2D, const float* dL_dopacity, const float* dL_dcolor, const float* dL_dmean3D,
+                            const float* dL_dcov3D, const float* dL_dsh, const float* dL_dscale, const float* dL_drot)
+{
+	RGS_REQUIRE(P > 0 && R >= 0, "%s: bad sizes P=%d R=%d", who, P, R);
+	RGS_REQUIRE(width > 0 && height > 0, "%s: bad image size %dx%d", who, width, height);
+	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
+	                cam_pos && radii && geom_ws && image_ws && dL_dpix && grad_accum &&
+	                dL_dmean2D && dL_dopacity && dL_dcolor && dL_dmean3D && dL_dcov3D,
+	            "%s: null pointer", who);
+	RGS_REQUIRE(R == 0 || binning_ws, "%s: null binning workspace", who);
+	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr), "%s: provide exactly one of SHs or colours", who);
+	RGS_REQUIRE(!shs || dL_dsh, "%s: dL_dsh is required with SHs", who);
+	RGS_REQUIRE(!scales || (rotations && dL_dscale && dL_drot), "%s: scale/rotation outputs missing", who);
+	RGS_REQUIRE(scales || cov3D_precomp, "%s: neither scales nor precomputed covariance", who);
 	return 0;
 }
 
@@ -693,75 +927,145 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	hipStream_t s = static_cast<hipStream_t>(stream);
 	EntryScope scope_(s);
 	RGS_TAKE_SORT_FAULT("rgs_backward");
-	RGS_REQUIRE(P > 0 && R >= 0, "rgs_backward: bad sizes P=%d R=%d", P, R);
-	RGS_REQUIRE(width > 0 && height > 0, "rgs_backward: bad image size %dx%d", width, height);
-	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
-	                cam_pos && radii && geom_ws && image_ws && dL_dpix && grad_accum &&
-	                dL_dmean2D && dL_dopacity && dL_dcolor && dL_dmean3D && dL_dcov3D,
-	            "rgs_backward: null pointer");
-	RGS_REQUIRE(R == 0 || binning_ws, "rgs_backward: null binning workspace");
-	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr), "rgs_backward: provide exactly one of SHs or colours");
-	RGS_REQUIRE(!shs || dL_dsh, "rgs_backward: dL_dsh is required with SHs");
-	RGS_REQUIRE(!scales || (rotations && dL_dscale && dL_drot), "rgs_backward: scale/rotation outputs missing");
-	RGS_REQUIRE(scales || cov3D_precomp, "rgs_backward: neither scales nor precomputed covariance");
-
-	size_t goff[RGS_GEOM_FIELDS], ioff[RGS_IMG_FIELDS];
-	geom_layout((size_t)P, goff);
-	image_layout(width, height, ioff);
-	const int gx = (width + rgs::kTile - 1) / rgs::kTile, gy = (height + rgs::kTile - 1) / rgs::kTile;
-	const size_t n = (size_t)P;
-
+	if (int rc = check_backward_pointers("rgs_backward", P, R, width, height, background, means3D, shs, colors_precomp, alphas,
+	                                     scales, rotations, cov3D_precomp, viewmatrix, projmatrix, projmatrix_inv, range_low,
+	                                     range_up, cam_pos, radii, geom_ws, binning_ws, image_ws, dL_dpix, grad_accum, dL_dmean2D,
+	                                     dL_dopacity, dL_dcolor, dL_dmean3D, dL_dcov3D, dL_dsh, dL_dscale, dL_drot))
+		return rc;
 	if (!outputs_zeroed) {
-		rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, (size_t)RGS_ACC_FLOATS * n, s);
+		rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, (size_t)RGS_ACC_FLOATS * (size_t)P, s);
 		RGS_STAGE("clear gradient sums");
 	}
-
-	const float* colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
 	if (R > 0) {
-		const BinningPhysical b = binning_physical((size_t)R);
-		const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
 		rgs::BlendArgs a;
-		memset(&a, 0, sizeof(a));
-		a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
-		a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
-		a.W = width; a.H = height; a.grid_x = gx; a.grid_y = gy;
-		a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
-		a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up; a.bg = background;
-		a.xy = at<float2>(geom_ws, goff[RGS_GEOM_XY]);
-		a.clip_w = at<float>(geom_ws, goff[RGS_GEOM_CLIP_W]);
-		a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
-		a.colors = colors;
-		a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
-		a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
+		fill_blend_args(a, P, R, width, height, tan_fovx, tan_fovy, background, projmatrix_inv, range_low, range_up, colors_precomp,
+		                geom_ws, binning_ws, image_ws);
 		a.out_alpha = const_cast<float*>(alphas);
-		a.n_contrib = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_N_CONTRIB]));
-		a.strip_filed = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_FILED]));
-		a.strip_order = const_cast<uint32_t*>(at<uint32_t>(image_ws, ioff[RGS_IMG_STRIP_ORDER]));
-		a.strip_lists = const_cast<uint32_t*>(at<uint32_t>(binning_ws, b.strip_lists));
 		a.dL_dpix = dL_dpix; a.dL_dpix_depth = dL_dpix_depth; a.dL_dalpha = dL_dalphas;
 		a.sums = grad_accum;
-		rgs::launch_blend_backward(a, s);
+		rgs::launch_blend_backward(&a, 1, s);
 		RGS_STAGE("blend_backward");
 	}
-
 	rgs::PreprocessBackwardArgs p;
-	memset(&p, 0, sizeof(p));
-	p.P = P; p.D = D; p.M = M;
-	p.means = means3D; p.radii = radii; p.shs = shs;
-	p.clamped = at<uint8_t>(geom_ws, goff[RGS_GEOM_CLAMPED]);
-	p.scales = scales; p.rotations = rotations; p.scale_modifier = scale_modifier;
-	p.cov3D = cov3D_precomp ? cov3D_precomp : at<float>(geom_ws, goff[RGS_GEOM_COV3D]);
-	p.view = viewmatrix; p.proj = projmatrix; p.campos = cam_pos;
-	p.focal_y = height / (2.0f * tan_fovy);
-	p.focal_x = width / (2.0f * tan_fovx);
-	p.tanfovx = tan_fovx; p.tanfovy = tan_fovy;
-	p.sums = grad_accum;
-	p.dL_dmean2D = dL_dmean2D; p.dL_dopacity = dL_dopacity; p.dL_dcolor = dL_dcolor;
-	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
-	p.visible_list = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_LIST]);
-	p.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D) && (reinterpret_cast<uintptr_t>(dL_dsh) & 15) == 0;
-	p.visible_count = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
-	rgs::launch_preprocess_backward(p, outputs_zeroed != 0, s);
+	fill_backward_geometry(p, P, D, M, width, height, means3D, shs, scales, scale_modifier, rotations, cov3D_precomp, viewmatrix,
+	                       projmatrix, cam_pos, tan_fovx, tan_fovy, radii, geom_ws, grad_accum, dL_dmean2D, dL_dopacity,
+	                       dL_dcolor, dL_dmean3D, dL_dcov3D, dL_dsh, dL_dscale, dL_drot);
+	rgs::launch_preprocess_backward(&p, &outputs_zeroed, 1, s);
+	RGS_STAGE("preprocess_backward");
+	return 0;
+}
+
+int rgs_frame_forward_geom(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, uint32_t* counts_pinned,
+                           void* stream, int debug)
+{
+	RGS_REQUIRE(K >= 1 && K <= RGS_MAX_FRAME_LAYERS && layers && view && counts_pinned,
+	            "rgs_frame_forward_geom: K = %d outside 1..%d, or null", K, RGS_MAX_FRAME_LAYERS);
+	std::vector<GeomCall> calls((size_t)K);
+	for (int k = 0; k < K; k++) {
+		const rgs_frame_layer& l = layers[k];
+		calls[(size_t)k] = GeomCall{l.P, l.D, l.M, l.means3D, l.shs, l.colors_precomp, l.opacities, l.scales, l.scale_modifier,
+		                            l.rotations, l.cov3D_precomp, const_cast<int*>(l.radii), l.geom_ws, l.geom_bytes};
+	}
+	return forward_geom(true, nullptr, "rgs_frame_forward_geom", K, calls.data(), view->width, view->height, view->viewmatrix,
+	                    view->projmatrix, view->cam_pos, view->tan_fovx, view->tan_fovy, counts_pinned, stream, debug);
+}
+
+int rgs_frame_forward_raster(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	RGS_REQUIRE(K >= 1 && K <= RGS_MAX_FRAME_LAYERS && layers && view, "rgs_frame_forward_raster: K = %d outside 1..%d, or null", K,
+	            RGS_MAX_FRAME_LAYERS);
+	std::vector<rgs::BlendArgs> jobs((size_t)K);
+	std::vector<RasterCall> calls((size_t)K);
+	for (int k = 0; k < K; k++) {
+		const rgs_frame_layer& l = layers[k];
+		RGS_REQUIRE(l.out_color && l.out_depth && l.out_alpha, "rgs_frame_forward_raster: layer %d has a null output", k);
+		calls[(size_t)k] = RasterCall{l.P, l.R, l.background, l.range_low, l.range_up, l.colors_precomp, l.geom_ws, l.geom_bytes,
+		                              l.binning_ws, l.binning_bytes, l.image_ws, l.image_bytes};
+	}
+	if (int rc = forward_binning("rgs_frame_forward_raster", false, K, calls.data(), view->width, view->height, view->tan_fovx,
+	                             view->tan_fovy, view->projmatrix_inv, jobs.data(), s, debug))
+		return rc;
+	for (int k = 0; k < K; k++) {
+		jobs[(size_t)k].out_color = layers[k].out_color;
+		jobs[(size_t)k].out_depth = layers[k].out_depth;
+		jobs[(size_t)k].out_alpha = layers[k].out_alpha;
+	}
+	// Clearing the gradient buffers is pure memory traffic and the blend is bound by instruction issue: on a
+	// layer's own stream the clearing runs beside the blend (rgs_frame_backward waits for it), else behind it.
+	if (int rc = side_streams_wait_for(K, layers, s, "rgs_frame_forward_raster"))
+		return rc;
+	for (int pass = 0; pass < 2; pass++) {
+		if (pass == 1) {
+			rgs::launch_blend_forward(jobs.data(), K, s);
+			RGS_STAGE("blend_forward");
+		}
+		for (int k = 0; k < K; k++) {
+			const rgs_frame_layer& l = layers[k];
+			const bool own_stream = l.stream && static_cast<hipStream_t>(l.stream) != s;
+			if (own_stream != (pass == 0))
+				continue;
+			for (int c = 0; c < 2; c++)
+				if (l.clear[c] && l.clear_bytes[c] != 0) {
+					RGS_REQUIRE((l.clear_bytes[c] & 3) == 0, "rgs_frame_forward_raster: clear_bytes must be a multiple of 4");
+					if (!own_stream)
+						rgs::stage_mark("clear_gradients", s);
+					rgs::launch_fill_u32(static_cast<uint32_t*>(l.clear[c]), 0u, l.clear_bytes[c] / 4,
+					                     own_stream ? static_cast<hipStream_t>(l.stream) : s);
+					RGS_STAGE("clear gradients");
+				}
+		}
+	}
+	return 0;
+}
+
+int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	RGS_TAKE_SORT_FAULT("rgs_frame_backward");
+	RGS_REQUIRE(K >= 1 && K <= RGS_MAX_FRAME_LAYERS && layers && view, "rgs_frame_backward: K = %d outside 1..%d, or null", K,
+	            RGS_MAX_FRAME_LAYERS);
+	// what the forward left running on the layers' own streams (the clearing of the gradient buffers) comes first
+	if (int rc = wait_for_side_streams(K, layers, s, "rgs_frame_backward"))
+		return rc;
+	std::vector<rgs::BlendArgs> jobs;
+	std::vector<rgs::PreprocessBackwardArgs> geometry((size_t)K);
+	std::vector<int> zeroed((size_t)K);
+	for (int k = 0; k < K; k++) {
+		const rgs_frame_layer& l = layers[k];
+		if (int rc = check_backward_pointers("rgs_frame_backward", l.P, l.R, view->width, view->height, l.background, l.means3D,
+		                                     l.shs, l.colors_precomp, l.out_alpha, l.scales, l.rotations, l.cov3D_precomp,
+		                                     view->viewmatrix, view->projmatrix, view->projmatrix_inv, l.range_low, l.range_up,
+		                                     view->cam_pos, l.radii, l.geom_ws, l.binning_ws, l.image_ws, l.dL_dpix, l.grad_accum,
+		                                     l.dL_dmean2D, l.dL_dopacity, l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh,
+		                                     l.dL_dscale, l.dL_drot))
+			return rc;
+		if (!l.outputs_zeroed) {
+			rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(l.grad_accum), 0u, (size_t)RGS_ACC_FLOATS * (size_t)l.P, s);
+			RGS_STAGE("clear gradient sums");
+		}
+		if (l.R > 0) {
+			rgs::BlendArgs a;
+			fill_blend_args(a, l.P, l.R, view->width, view->height, view->tan_fovx, view->tan_fovy, l.background,
+			                view->projmatrix_inv, l.range_low, l.range_up, l.colors_precomp, l.geom_ws, l.binning_ws, l.image_ws);
+			a.out_alpha = l.out_alpha;
+			a.dL_dpix = l.dL_dpix; a.dL_dpix_depth = l.dL_dpix_depth; a.dL_dalpha = l.dL_dalphas;
+			a.sums = l.grad_accum;
+			jobs.push_back(a);
+		}
+		fill_backward_geometry(geometry[(size_t)k], l.P, l.D, l.M, view->width, view->height, l.means3D, l.shs, l.scales,
+		                       l.scale_modifier, l.rotations, l.cov3D_precomp, view->viewmatrix, view->projmatrix, view->cam_pos,
+		                       view->tan_fovx, view->tan_fovy, l.radii, l.geom_ws, l.grad_accum, l.dL_dmean2D, l.dL_dopacity,
+		                       l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh, l.dL_dscale, l.dL_drot);
+		zeroed[(size_t)k] = l.outputs_zeroed;
+	}
+	if (!jobs.empty()) {
+		rgs::launch_blend_backward(jobs.data(), (int)jobs.size(), s);
+		RGS_STAGE("blend_backward");
+	}
+	rgs::launch_preprocess_backward(geometry.data(), zeroed.data(), K, s);
 	RGS_STAGE("preprocess_backward");
 	return 0;
 }
@@ -777,32 +1081,14 @@ int rgs_blend_work_counters(int P, int R, int width, int height, float tan_fovx,
 	RGS_REQUIRE(P > 0 && R >= 0 && width > 0 && height > 0, "rgs_blend_work_counters: bad sizes");
 	RGS_REQUIRE(projmatrix_inv && range_low && range_up && geom_ws && image_ws && counters && (R == 0 || binning_ws),
 	            "rgs_blend_work_counters: null pointer");
-	size_t goff[RGS_GEOM_FIELDS], ioff[RGS_IMG_FIELDS];
-	geom_layout((size_t)P, goff);
-	image_layout(width, height, ioff);
 	rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(counters), 0u, 2 * RGS_WORK_COUNTERS, s);
 	if (R == 0)
 		return 0;
-	const BinningPhysical b = binning_physical((size_t)R);
-	const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
 	rgs::BlendArgs a;
-	memset(&a, 0, sizeof(a));
-	a.ranges = at<uint2>(image_ws, ioff[RGS_IMG_RANGES]);
-	a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
-	a.W = width; a.H = height;
-	a.grid_x = (width + rgs::kTile - 1) / rgs::kTile;
-	a.grid_y = (height + rgs::kTile - 1) / rgs::kTile;
-	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
-	a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up;
-	a.bg = range_low;  // unused by the counting kernel
-	a.xy = at<float2>(geom_ws, goff[RGS_GEOM_XY]);
-	a.clip_w = at<float>(geom_ws, goff[RGS_GEOM_CLIP_W]);
-	a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
-	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
-	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
-	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
+	fill_blend_args(a, P, R, width, height, tan_fovx, tan_fovy, range_low /* unused by the counting kernel */, projmatrix_inv,
+	                range_low, range_up, colors_precomp, geom_ws, binning_ws, image_ws);
 	a.counters = counters;
-	rgs::launch_blend_forward(a, s);
+	rgs::launch_blend_count(a, s);
 	RGS_STAGE("blend_count");
 	return 0;
 }

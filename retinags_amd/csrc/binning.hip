@@ -14,6 +14,7 @@
 // of instances emitted in (depth, index) order give the same list: within a tile both order by
 // depth and break ties by Gaussian index (a Gaussian touches a tile at most once).
 #include "rgs_kernels.h"
+#include "strip_filing.h"
 
 #include <atomic>
 
@@ -43,19 +44,34 @@ __global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __res
 }
 
 // In-place exclusive scan of `data[0..n)` by one block of 1024 threads; the grand total goes
-// to *total_out (if non-null).
-// Block 1, if launched, does the same for a second array of the same length.
-__global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(uint32_t* __restrict__ data, size_t n,
-                                                                            const uint32_t* __restrict__ n_device,
-                                                                            uint32_t* __restrict__ total_out,
-                                                                            uint32_t* __restrict__ data_b,
-                                                                            uint32_t* __restrict__ total_out_b)
+// to *total_out and *total_copy (if non-null).  Block 1, if launched, does the same for a second
+// array of the same length.  blockIdx.y selects the job.
+struct BlockScanJob {
+	uint32_t* data;
+	size_t n;
+	const uint32_t* n_device;
+	uint32_t* total_out;
+	uint32_t* total_copy;
+	uint32_t* data_b;
+	uint32_t* total_out_b;
+};
+
+__global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(Batch<BlockScanJob> batch)
 {
 	__shared__ uint32_t wave_tot[16];
+	const BlockScanJob& j = batch.job[blockIdx.y];
+	uint32_t* data = j.data;
+	size_t n = j.n;
+	const uint32_t* n_device = j.n_device;
+	uint32_t* total_out = j.total_out;
+	uint32_t* total_copy = j.total_copy;
 	if (blockIdx.x == 1) {
-		data = data_b;
-		total_out = total_out_b;
+		data = j.data_b;
+		total_out = j.total_out_b;
+		total_copy = nullptr;
 	}
+	if (!data)
+		return;
 	if (n_device)
 		n = ((size_t)*n_device + 255) / 256;  // one entry per 256 elements
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -85,16 +101,30 @@ __global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(uint3
 	}
 	if (tid == 0 && total_out)
 		*total_out = total;
+	if (tid == 0 && total_copy)
+		*total_copy = total;
 }
 
-__global__ __launch_bounds__(256) void block_inclusive_scan_kernel(const uint32_t* __restrict__ in,
-                                                                    const uint32_t* __restrict__ block_base, size_t n,
-                                                                    const uint32_t* __restrict__ n_device,
-                                                                    uint32_t* __restrict__ out)
+struct BlockInclusiveJob {
+	const uint32_t* in;
+	const uint32_t* block_base;
+	size_t n;
+	const uint32_t* n_device;
+	uint32_t* out;
+};
+
+__global__ __launch_bounds__(256) void block_inclusive_scan_kernel(Batch<BlockInclusiveJob> batch)
 {
 	__shared__ uint32_t lds[8];
-	if (n_device)
-		n = *n_device;
+	const BlockInclusiveJob& j = batch.job[blockIdx.y];
+	const uint32_t* __restrict__ in = j.in;
+	const uint32_t* __restrict__ block_base = j.block_base;
+	uint32_t* __restrict__ out = j.out;
+	size_t n = j.n;
+	if (j.n_device)
+		n = *j.n_device;
+	if ((size_t)blockIdx.x * 256 >= n)
+		return;
 	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
 	const uint32_t v = i < n ? in[i] : 0u;
 	uint32_t total;
@@ -113,9 +143,12 @@ static void inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, const uin
 {
 	const size_t nb = (n + 255) / 256;
 	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, n_device, temp);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, temp, nb, n_device,
-	                   (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr);
-	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, temp, n, n_device, out);
+	Batch<BlockScanJob> scan = {};
+	scan.job[0] = BlockScanJob{temp, nb, n_device, nullptr, nullptr, nullptr, nullptr};
+	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan);
+	Batch<BlockInclusiveJob> inc = {};
+	inc.job[0] = BlockInclusiveJob{in, temp, n, n_device, out};
+	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, inc);
 }
 
 void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, const char* stage,
@@ -128,13 +161,19 @@ void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t*
 	inclusive_sum(in, out, n, nullptr, temp, s);
 }
 
-void launch_totals_from_block_sums(uint32_t* block_sums, uint32_t* block_visible, int P, uint32_t* total_out,
-                                   uint32_t* visible_count, hipStream_t s)
+void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t s)
 {
-	const size_t nb = ((size_t)P + 255) / 256;
 	stage_mark("offset_scan", s);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(2), dim3(1024), 0, s, block_sums, nb,
-	                   (const uint32_t*)nullptr, total_out, block_visible, visible_count);
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<BlockScanJob> b = {};
+		for (int k = 0; k < nj; k++) {
+			const TotalsJob& t = jobs[at + k];
+			b.job[k] = BlockScanJob{t.block_sums, ((size_t)t.P + 255) / 256, nullptr, t.total_out, t.total_copy, t.block_visible,
+			                        t.visible_count};
+		}
+		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(2, (unsigned)nj), dim3(1024), 0, s, b);
+	}
 }
 
 // ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------
@@ -142,13 +181,19 @@ void launch_totals_from_block_sums(uint32_t* block_sums, uint32_t* block_visible
 // (depth bits, index) pairs of the Gaussians that touch a tile, compacted in index order:
 // block b of 256 Gaussians writes from visible_base[b] on.  Depths of rendered Gaussians are
 // positive floats (> 0.2), whose bit patterns order like the values.
-__global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __restrict__ depths,
-                                                           const uint32_t* __restrict__ tiles_touched,
-                                                           const uint32_t* __restrict__ visible_base,
-                                                           uint32_t* __restrict__ keys, uint32_t* __restrict__ values,
-                                                           uint32_t* __restrict__ visible_list)
+__global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
+	const DepthOrderJob& j = batch.job[blockIdx.y];
+	const int P = j.P;
+	if ((int)blockIdx.x * 256 >= P)
+		return;
+	const float* __restrict__ depths = j.depths;
+	const uint32_t* __restrict__ tiles_touched = j.tiles_touched;
+	const uint32_t* __restrict__ visible_base = j.block_visible;
+	uint32_t* __restrict__ keys = j.keys_a;
+	uint32_t* __restrict__ values = j.order;
+	uint32_t* __restrict__ visible_list = j.visible_list;
 	const int idx = blockIdx.x * 256 + threadIdx.x;
 	const bool visible = idx < P && tiles_touched[idx] != 0u;
 	uint32_t total;
@@ -164,13 +209,18 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(int P, const float* __
 // out[k] = in[index[k]] for k below the count on the device, and the sum of every 256 of them
 // (the first level of the scan that follows).  `in` has in_size entries; an index beyond it (only
 // possible in what a sort that gave up left behind) reads the last entry instead.
-__global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ n_device,
-                                                          const uint32_t* __restrict__ index,
-                                                          const uint32_t* __restrict__ in, uint32_t in_size,
-                                                          uint32_t* __restrict__ out,
-                                                          uint32_t* __restrict__ block_totals)
+__global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
+	const DepthOrderJob& j = batch.job[blockIdx.y];
+	if ((int)blockIdx.x * 256 >= j.P)
+		return;
+	const uint32_t* __restrict__ n_device = j.visible_count;
+	const uint32_t* __restrict__ index = j.order;
+	const uint32_t* __restrict__ in = j.tiles_touched;
+	const uint32_t in_size = (uint32_t)j.P;
+	uint32_t* __restrict__ out = j.tiles_in_order;
+	uint32_t* __restrict__ block_totals = j.scan_temp;
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
 	uint32_t v = 0;
 	if (k < *n_device) {
@@ -184,100 +234,209 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restr
 }
 
 // Instances of the Gaussians in depth order, tiles row by row like the reference, at the offsets
-// of the scan taken in that same order.  A wavefront takes 64 Gaussians; their instances form one
-// contiguous run of the output, which the wavefront writes 64 consecutive entries at a time:
-// each lane finds the Gaussian its output position belongs to by a binary search over the 64
-// inclusive offsets, then the tile from the position inside that Gaussian's rectangle.  (With
-// one thread per Gaussian every store touched 64 different cache lines, and a Gaussian that
-// covers hundreds of tiles kept its wavefront busy alone.)
+// of the scan taken in that same order.  The work is dealt out by output position, not by Gaussian:
+// a workgroup writes kDupPositions consecutive instances, whichever Gaussians they belong to (one
+// that covers thousands of tiles is shared by several workgroups, a thousand that cover one tile
+// each are taken by one).  It finds the first Gaussian of its range by a 64-ary search over the
+// inclusive offsets, stages the Gaussians of its range in LDS 256 at a time (offset, tile rectangle,
+// the tile-independent part of the strip tests) and lets every thread find the Gaussian of its
+// output position by a binary search over those 256 offsets, then the tile from the position
+// inside that Gaussian's rectangle; stores are contiguous.  The thread also decides which of the
+// tile's four strips the instance can matter to (strip_filing.h) and puts those bits above the
+// tile in the key: the sort only looks at the tile bits, so they travel with the instance for free.
 // `order` is the output of a sort: should that sort ever have given up, its entries may be anything, so
 // they are clamped to the P Gaussians there are (the tile ranges then stay empty and nothing reads the result).
-__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(uint32_t P, const uint32_t* __restrict__ visible_count,
-                                                                   const uint32_t* __restrict__ order,
-                                                                   const uint32_t* __restrict__ offsets,
-                                                                   const float2* __restrict__ xy,
-                                                                   const int* __restrict__ radii, int gx, int gy,
-                                                                   uint32_t* __restrict__ keys,
-                                                                   uint32_t* __restrict__ values, uint32_t capacity,
-                                                                   uint32_t* __restrict__ clear, size_t clear_words)
+constexpr int kDupPositions = 1024;
+
+struct DuplicateStage {
+	uint32_t end[256];     // inclusive offset of each staged Gaussian
+	uint32_t origin[256];  // first tile of its rectangle
+	uint32_t width[256];   // tiles per row of its rectangle
+	uint32_t index[256];
+	StripTests tests[256]; // the tile-independent part of its strip tests
+};
+
+// Floats of LDS for the NDC tables of a grid of tiles: 2 per tile column (rounded up to a multiple of 4), 8 per tile row.
+static inline size_t ndc_table_floats(int gx, int gy)
 {
-	__shared__ uint32_t s_end[4][64];     // inclusive offset of each of the wavefront's Gaussians
-	__shared__ uint32_t s_origin[4][64];  // first tile of its rectangle
-	__shared__ uint32_t s_width[4][64];   // tiles per row of its rectangle
-	__shared__ uint32_t s_index[4][64];
-	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
+	return (size_t)((2 * gx + 3) & ~3) + 8 * (size_t)gy;
+}
+constexpr size_t kNdcTableMaxFloats = 8192;  // larger grids compute the coordinates per instance
+
+__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<DuplicateJob> batch, int gx, int gy, int ndc_in_lds)
+{
+	__shared__ DuplicateStage st;
+	__shared__ uint32_t s_first;
+	extern __shared__ __align__(16) float s_ndc[];  // NDC of every tile column's first and last pixel, then of every strip's first and last row
+	const DuplicateJob& job = batch.job[blockIdx.y];
+	const uint32_t P = (uint32_t)job.P;
+	const uint32_t* __restrict__ visible_count = job.visible_count;
+	const uint32_t* __restrict__ order = job.order;
+	const uint32_t* __restrict__ offsets = job.offsets;
+	const FilingArgs& filing = job.filing;
+	uint32_t* __restrict__ keys = job.keys;
+	uint32_t* __restrict__ values = job.values;
+	const uint32_t capacity = job.capacity;
+	uint32_t* __restrict__ clear = job.clear;
+	const size_t clear_words = job.clear_words;
+	const int tid = threadIdx.x, lane = tid & 63;
 	// the scratch of the sort that follows is cleared here, which saves a launch
-	for (size_t w = k; w < clear_words; w += (size_t)gridDim.x * 256)
+	for (size_t w = (size_t)blockIdx.x * 256 + tid; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;
 	const uint32_t n = min(*visible_count, P);
-	const uint32_t k0 = k - (uint32_t)lane;  // the wavefront's first Gaussian
-	if (k0 >= n)
+	if (n == 0u)
 		return;
-	const uint32_t run_begin = k0 == 0u ? 0u : offsets[k0 - 1];
-	uint32_t end = 0, origin = 0, width = 1, idx = 0;
-	if (k < n) {
-		idx = min(order[k], P - 1u);
-		end = offsets[k];
-		const float2 p = xy[idx];
-		const TileRect rc = tile_rect(p.x, p.y, radii[idx], gx, gy);
-		origin = rc.y0 * (uint32_t)gx + rc.x0;
-		width = rc.x1 - rc.x0;
-	} else {
-		end = offsets[n - 1];  // no instances of its own
-	}
-	s_end[wave][lane] = end;
-	s_origin[wave][lane] = origin;
-	s_width[wave][lane] = width;
-	s_index[wave][lane] = idx;
-	__builtin_amdgcn_wave_barrier();
-	const uint32_t run_end = s_end[wave][63];
-	for (uint32_t base = run_begin; base < run_end; base += 64) {
-		const uint32_t pos = base + (uint32_t)lane;
-		if (pos < run_end && pos < capacity) {  // positions beyond the room the caller gave are dropped
-			// the first Gaussian whose inclusive offset exceeds pos
-			int lo = 0;
-#pragma unroll
-			for (int step = 32; step > 0; step >>= 1)
-				if (s_end[wave][lo + step - 1] <= pos)
-					lo += step;
-			const uint32_t first = lo == 0 ? run_begin : s_end[wave][lo - 1];
-			const uint32_t t = pos - first, w = s_width[wave][lo];
-			const uint32_t row = t / w;
-			keys[pos] = s_origin[wave][lo] + row * (uint32_t)gx + (t - row * w);
-			values[pos] = s_index[wave][lo];
+	const uint32_t total = offsets[n - 1];
+	const uint32_t limit = min(total, capacity);  // positions beyond the room the caller gave are dropped
+	const uint32_t start = blockIdx.x * (uint32_t)kDupPositions;
+	if (start >= limit)
+		return;
+	const uint32_t stop = min(start + (uint32_t)kDupPositions, limit);
+
+	const int rows_at = (2 * gx + 3) & ~3;
+	if (ndc_in_lds) {
+		for (int c = tid; c < gx; c += 256) {
+			const float2 v = tile_column_ndc(c, filing.W);
+			s_ndc[2 * c] = v.x;
+			s_ndc[2 * c + 1] = v.y;
+		}
+		for (int r = tid; r < 4 * gy; r += 256) {
+			const float2 v = strip_rows_ndc(r >> 2, r & 3, filing.H);
+			s_ndc[rows_at + 2 * r] = v.x;
+			s_ndc[rows_at + 2 * r + 1] = v.y;
 		}
 	}
+	// the first Gaussian whose inclusive offset exceeds `start`: 64-ary search by the first wavefront
+	if (tid < 64) {
+		uint32_t lo = 0, hi = n;  // the answer lies in [lo, hi]
+		while (lo < hi) {
+			const uint32_t step = (hi - lo + 63u) / 64u;
+			const uint32_t probe = lo + (uint32_t)lane * step;
+			const bool below = probe < hi && offsets[probe] <= start;
+			const uint32_t c = (uint32_t)__popcll(__ballot(below));  // the predicate is monotone: the first c probes hold
+			if (c == 0u) {
+				hi = lo;
+			} else {
+				const uint32_t last_true = lo + (c - 1u) * step;
+				lo = last_true + 1u;
+				hi = min(last_true + step, hi);
+			}
+		}
+		if (lane == 0)
+			s_first = lo;
+	}
+	__syncthreads();
+	const BoxFrame box = load_box_frame(filing.projinv, filing.range_low, filing.range_up, filing.tanfovx, filing.tanfovy);
+
+	for (uint32_t g0 = s_first; g0 < n; g0 += 256) {
+		// stage Gaussians g0 .. g0 + 255 (in depth order)
+		const uint32_t g = g0 + (uint32_t)tid;
+		uint32_t end = total, origin = 0, width = 1, idx = 0;
+		if (g < n) {
+			idx = min(order[g], P - 1u);
+			end = offsets[g];
+			// everything else comes from the Gaussian's 64-byte record: pixel centre, conic, extents, radius
+			const float4* rec = filing.record + 4 * (size_t)idx;
+			const float4 g4 = rec[0], h = rec[3];
+			const TileRect rc = tile_rect(g4.x, g4.y, __float_as_int(h.z), gx, gy);
+			origin = rc.y0 * (uint32_t)gx + rc.x0;
+			width = max(rc.x1 - rc.x0, 1u);
+			st.tests[tid] = prepare_strip_tests(FiledGeometry{g4, rec[1], float2{h.x, h.y}}, box);
+		}
+		st.end[tid] = end;
+		st.origin[tid] = origin;
+		st.width[tid] = width;
+		st.index[tid] = idx;
+		__syncthreads();
+		const uint32_t staged_begin = g0 == 0u ? 0u : offsets[g0 - 1];
+		const uint32_t staged_end = st.end[255];
+		const uint32_t from = max(start, staged_begin), to = min(stop, staged_end);
+		for (uint32_t pos = from + (uint32_t)tid; pos < to; pos += 256) {
+			// the first staged Gaussian whose inclusive offset exceeds pos
+			int lo = 0;
+#pragma unroll
+			for (int step = 128; step > 0; step >>= 1)
+				if (st.end[lo + step - 1] <= pos)
+					lo += step;
+			const uint32_t first = lo == 0 ? staged_begin : st.end[lo - 1];
+			const uint32_t t = pos - first, w = st.width[lo];
+			const uint32_t row = t / w;
+			const uint32_t tile = st.origin[lo] + row * (uint32_t)gx + (t - row * w);
+			const int tx = (int)(tile % (uint32_t)gx), ty = (int)(tile / (uint32_t)gx);
+			float2 nx;
+			float ny[8];
+			if (ndc_in_lds) {
+				nx = float2{s_ndc[2 * tx], s_ndc[2 * tx + 1]};
+				const float4 r0 = *reinterpret_cast<const float4*>(s_ndc + rows_at + 8 * ty);
+				const float4 r1 = *reinterpret_cast<const float4*>(s_ndc + rows_at + 8 * ty + 4);
+				ny[0] = r0.x; ny[1] = r0.y; ny[2] = r0.z; ny[3] = r0.w;
+				ny[4] = r1.x; ny[5] = r1.y; ny[6] = r1.z; ny[7] = r1.w;
+			} else {
+				nx = tile_column_ndc(tx, filing.W);
+#pragma unroll
+				for (int q = 0; q < 4; q++) {
+					const float2 v = strip_rows_ndc(ty, q, filing.H);
+					ny[2 * q] = v.x;
+					ny[2 * q + 1] = v.y;
+				}
+			}
+			const uint32_t strips = strips_filed_for(st.tests[lo], (float)(tx * kTile), (float)(ty * kTile), nx, ny, box);
+			keys[pos] = tile | (strips << kKeyTileBits);
+			values[pos] = st.index[lo];
+		}
+		if (staged_end >= stop)
+			break;
+		__syncthreads();
+	}
 }
 
-void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touched, uint32_t* block_visible,
-                        uint32_t* visible_count, uint32_t* visible_list, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
-                        uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
-                        hipStream_t s)
+void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)
 {
-	const unsigned nb = (unsigned)((P + 255) / 256);
 	stage_mark("depth_order", s);
-	hipLaunchKernelGGL(depth_pairs_kernel, dim3(nb), dim3(256), 0, s, P, depths, tiles_touched, block_visible, keys_a,
-	                   order, visible_list);
-	// 4 passes: the sorted pairs end up in the first buffer pair again
-	launch_sort_pairs_u32(keys_a, keys_b, order, vals_b, (size_t)P, visible_count, 32, sort_temp, true, nullptr, 0, nullptr,
-	                      s);
-	hipLaunchKernelGGL(gather_u32_kernel, dim3(nb), dim3(256), 0, s, visible_count, order, tiles_touched, (uint32_t)P,
-	                   tiles_in_order, scan_temp);
-	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan_temp, (size_t)nb,
-	                   visible_count, (uint32_t*)nullptr, (uint32_t*)nullptr, (uint32_t*)nullptr);
-	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3(nb), dim3(256), 0, s, tiles_in_order, scan_temp, (size_t)P,
-	                   visible_count, offsets_in_order);
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<DepthOrderJob> b = {};
+		Batch<BlockScanJob> scan = {};
+		Batch<BlockInclusiveJob> inc = {};
+		SortJob<uint32_t> sorts[kMaxBatch];
+		int max_p = 0;
+		for (int k = 0; k < nj; k++) {
+			const DepthOrderJob& j = jobs[at + k];
+			b.job[k] = j;
+			max_p = j.P > max_p ? j.P : max_p;
+			// 4 passes: the sorted pairs end up in the first buffer pair again
+			sorts[k] = SortJob<uint32_t>{j.keys_a, j.keys_b, j.order, j.vals_b, (size_t)j.P, j.visible_count, j.sort_temp, nullptr, 0};
+			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + 255) / 256, j.visible_count, nullptr, nullptr, nullptr, nullptr};
+			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order};
+		}
+		const dim3 grid((unsigned)((max_p + 255) / 256), (unsigned)nj);
+		hipLaunchKernelGGL(depth_pairs_kernel, grid, dim3(256), 0, s, b);
+		launch_sort_pairs_u32(sorts, nj, 32, true, nullptr, s);
+		hipLaunchKernelGGL(gather_u32_kernel, grid, dim3(256), 0, s, b);
+		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1, (unsigned)nj), dim3(1024), 0, s, scan);
+		hipLaunchKernelGGL(block_inclusive_scan_kernel, grid, dim3(256), 0, s, inc);
+	}
 }
 
-void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
-                                const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
-                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t capacity, uint32_t* clear,
-                                size_t clear_words, hipStream_t s)
+void launch_duplicate_with_keys(const DuplicateJob* jobs, int count, int grid_x, int grid_y, hipStream_t s)
 {
 	stage_mark("duplicate_with_keys", s);
-	hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + 255) / 256), dim3(256), 0, s, (uint32_t)P, visible_count, order,
-	                   offsets_in_order, xy, radii, grid_x, grid_y, keys, values, capacity, clear, clear_words);
+	const size_t table = ndc_table_floats(grid_x, grid_y);
+	const int ndc_in_lds = table <= kNdcTableMaxFloats ? 1 : 0;
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<DuplicateJob> b = {};
+		size_t blocks = 1;
+		for (int k = 0; k < nj; k++) {
+			b.job[k] = jobs[at + k];
+			// sized for the positions there is room for; at least enough workgroups to clear the sort's scratch at a decent rate
+			const size_t need = max((size_t)(b.job[k].capacity + kDupPositions - 1) / kDupPositions,
+			                        min((b.job[k].clear_words + 4095) / 4096, (size_t)1024));
+			blocks = need > blocks ? need : blocks;
+		}
+		hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((unsigned)blocks, (unsigned)nj), dim3(256),
+		                   ndc_in_lds ? table * sizeof(float) : 0, s, b, grid_x, grid_y, ndc_in_lds);
+	}
 }
 
 // ---- radix sort -------------------------------------------------------------------------------
@@ -320,13 +479,16 @@ __device__ __forceinline__ uint32_t digit_of(KeyT key, int shift, uint32_t mask)
 }
 
 template <typename KeyT>
-__global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const KeyT* __restrict__ keys, size_t n,
-                                                                    const uint32_t* __restrict__ n_device,
-                                                                    int passes, int end_bit,
-                                                                    uint32_t* __restrict__ hist,
-                                                                    uint32_t* __restrict__ clear, size_t clear_words)
+__global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob<KeyT>> batch, int passes, int end_bit)
 {
 	__shared__ uint32_t s_hist[kSortMaxPasses][256];
+	const SortJob<KeyT>& j = batch.job[blockIdx.y];
+	const KeyT* __restrict__ keys = j.keys_in;
+	size_t n = j.n;
+	const uint32_t* __restrict__ n_device = j.n_device;
+	uint32_t* __restrict__ hist = j.temp;
+	uint32_t* __restrict__ clear = j.also_clear;
+	const size_t clear_words = j.also_clear_words;
 	for (size_t w = (size_t)blockIdx.x * 256 + threadIdx.x; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;  // an array that a later kernel of the same stream wants cleared
 	if (n_device)
@@ -352,16 +514,24 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(const KeyT* _
 }
 
 template <typename KeyT>
-__global__ __launch_bounds__(256) void sort_onesweep_kernel(const KeyT* __restrict__ keys_in,
-                                                             const uint32_t* __restrict__ vals_in,
-                                                             KeyT* __restrict__ keys_out,
-                                                             uint32_t* __restrict__ vals_out, size_t n,
-                                                             const uint32_t* __restrict__ n_device, int shift,
-                                                             uint32_t mask, const uint32_t* __restrict__ digit_count,
-                                                             uint32_t* __restrict__ lookback,
-                                                             uint32_t* __restrict__ tile_counter,
-                                                             uint32_t* __restrict__ status, int spin_limit)
+__global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>> batch, int pass, int shift, uint32_t mask,
+                                                             int spin_limit)
 {
+	const SortJob<KeyT>& j = batch.job[blockIdx.y];
+	// the passes ping-pong between the two buffer pairs, starting in -> out
+	const KeyT* __restrict__ keys_in = (pass & 1) ? j.keys_out : j.keys_in;
+	const uint32_t* __restrict__ vals_in = (pass & 1) ? j.vals_out : j.vals_in;
+	KeyT* __restrict__ keys_out = (pass & 1) ? j.keys_in : j.keys_out;
+	uint32_t* __restrict__ vals_out = (pass & 1) ? j.vals_in : j.vals_out;
+	size_t n = j.n;
+	const uint32_t* __restrict__ n_device = j.n_device;
+	const size_t job_tiles = (j.n + kSortBlock - 1) / kSortBlock;
+	if (blockIdx.x >= job_tiles)
+		return;  // the launch is sized for the job with the most tiles
+	const uint32_t* __restrict__ digit_count = j.temp + pass * 256;
+	uint32_t* __restrict__ lookback = j.temp + kSortHeader + (size_t)pass * 256 * job_tiles;
+	uint32_t* __restrict__ tile_counter = j.temp + kSortCounters + pass;
+	uint32_t* __restrict__ status = j.temp + kSortStatus;
 	__shared__ KeyT s_keys[kSortBlock];
 	__shared__ uint32_t s_vals[kSortBlock];
 	__shared__ uint32_t s_wave_hist[4][256];  // per-wave digit counts, then exclusive prefix over waves
@@ -530,79 +700,103 @@ size_t sort_clear_words(size_t n, int end_bit)
 }
 
 template <typename KeyT>
-static void sort_pairs(KeyT* keys_in, KeyT* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                       const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, bool mark_stages,
-                       uint32_t* also_clear, size_t also_clear_words, hipStream_t s)
+static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool temp_cleared, bool mark_stages, hipStream_t s)
 {
-	if (n == 0)
-		return;
-	const uint32_t tiles = (uint32_t)((n + kSortBlock - 1) / kSortBlock);
 	const int passes = (end_bit + 7) / 8;
-	if (mark_stages)
-		stage_mark("sort_setup", s);
-	if (!temp_cleared)
-		launch_fill_u32(temp, 0u, sort_clear_words(n, end_bit), s);
-	const uint32_t hist_blocks = tiles < 2048u ? tiles : 2048u;
-	hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks), dim3(256), 0, s, keys_in, n, n_device, passes,
-	                   end_bit, temp, also_clear, also_clear_words);
-	KeyT *ksrc = keys_in, *kdst = keys_out;
-	uint32_t *vsrc = vals_in, *vdst = vals_out;
-	for (int p = 0; p < passes; p++) {
-		const int shift = 8 * p;
-		const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
-		const uint32_t mask = (1u << bits) - 1u;
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<SortJob<KeyT>> b = {};
+		uint32_t max_tiles = 0;
+		int live = 0;
+		for (int k = 0; k < nj; k++) {
+			const SortJob<KeyT>& j = jobs[at + k];
+			if (j.n == 0)
+				continue;
+			b.job[live++] = j;
+			const uint32_t tiles = (uint32_t)((j.n + kSortBlock - 1) / kSortBlock);
+			max_tiles = tiles > max_tiles ? tiles : max_tiles;
+			if (!temp_cleared)
+				launch_fill_u32(j.temp, 0u, sort_clear_words(j.n, end_bit), s);
+		}
+		if (live == 0)
+			continue;
 		if (mark_stages)
-			stage_mark("sort_onesweep", s);
-		hipLaunchKernelGGL(sort_onesweep_kernel<KeyT>, dim3(tiles), dim3(256), 0, s, ksrc, vsrc, kdst, vdst, n, n_device, shift,
-		                   mask,
-		                   temp + p * 256, temp + kSortHeader + (size_t)p * 256 * tiles, temp + kSortCounters + p,
-		                   temp + kSortStatus, g_lookback_spin_limit.load());
-		KeyT* tk = ksrc; ksrc = kdst; kdst = tk;
-		uint32_t* tv = vsrc; vsrc = vdst; vdst = tv;
+			stage_mark("sort_setup", s);
+		const uint32_t hist_blocks = max_tiles < 2048u ? max_tiles : 2048u;
+		hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
+		for (int p = 0; p < passes; p++) {
+			const int shift = 8 * p;
+			const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+			const uint32_t mask = (1u << bits) - 1u;
+			if (mark_stages)
+				stage_mark("sort_onesweep", s);
+			hipLaunchKernelGGL(sort_onesweep_kernel<KeyT>, dim3(max_tiles, (unsigned)live), dim3(256), 0, s, b, p, shift, mask,
+			                   g_lookback_spin_limit.load());
+		}
 	}
 }
 
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s)
 {
-	sort_pairs<uint64_t>(keys_in, keys_out, vals_in, vals_out, n, nullptr, end_bit, temp, false, true, nullptr, 0, s);
+	const SortJob<uint64_t> job = {keys_in, keys_out, vals_in, vals_out, n, nullptr, temp, nullptr, 0};
+	sort_pairs<uint64_t>(&job, 1, end_bit, false, true, s);
 }
 
-void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                           const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, uint32_t* also_clear,
-                           size_t also_clear_words, const char* stage, hipStream_t s)
+void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, const char* stage,
+                           hipStream_t s)
 {
-	sort_pairs<uint32_t>(keys_in, keys_out, vals_in, vals_out, n, n_device, end_bit, temp, temp_cleared, stage != nullptr,
-	                     also_clear, also_clear_words, s);
+	sort_pairs<uint32_t>(jobs, count, end_bit, temp_cleared, stage != nullptr, s);
 }
 
-// ---- tile ranges (K/cuda_rasterizer_hgs/rasterizer_impl.cu:116-138 and the memset at :319) ----
-
+// Sets n words to v, 16 bytes per store where the address allows; a capped grid walks the array.
 __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t v, size_t n)
 {
-	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-	if (i < n)
-		p[i] = v;
+	const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, threads = (size_t)gridDim.x * 256;
+	// words up to the first 16-byte boundary, whole 16-byte groups, the rest
+	const size_t head = min(n, (size_t)((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4);
+	const size_t groups = (n - head) / 4;
+	if (tid < head)
+		p[tid] = v;
+	uint4* q = reinterpret_cast<uint4*>(p + head);
+	const uint4 vv = {v, v, v, v};
+	for (size_t g = tid; g < groups; g += threads)
+		q[g] = vv;
+	const size_t done = head + 4 * groups;
+	if (tid < n - done)
+		p[done + tid] = v;
 }
 
 void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 {
 	if (n == 0)
 		return;
-	hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, v, n);
+	const size_t blocks = (n / 4 + 255) / 256 + 1;
+	hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, s, p, v, n);
 }
 
 // The status words (may be null) are those of the two sorts: if either reported a failure the
 // ranges stay empty, so no later stage walks an unsorted list, and *fault (host memory that the
-// device can write, may be null) is set for the host to find.
-__global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __restrict__ keys, size_t n,
-                                                           const uint32_t* __restrict__ n_device,
-                                                           uint2* __restrict__ ranges,
-                                                           const uint32_t* __restrict__ sort_status,
-                                                           const uint32_t* __restrict__ order_status,
-                                                           uint32_t* __restrict__ fault)
+// device can write, may be null) is set for the host to find.  The keys carry strip bits above the
+// tile (key_strips); per workgroup of kFileBlock keys, file_tail (may be null) receives how many keys
+// of the tile of its last key have each of the four "filed" bits set, which is what the kernel that
+// places the entries in their strips' lists needs from the workgroups ahead of its own.
+__global__ __launch_bounds__(kFileBlock) void tile_ranges_kernel(Batch<TileRangesJob> batch)
 {
-	const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+	__shared__ uint32_t s_tail[4][4];  // [wave][strip]
+	__shared__ uint32_t s_last_tile;
+	const TileRangesJob& j = batch.job[blockIdx.y];
+	const uint32_t* __restrict__ keys = j.keys;
+	size_t n = j.n;
+	const uint32_t* __restrict__ n_device = j.n_device;
+	uint2* __restrict__ ranges = j.ranges;
+	const uint32_t* __restrict__ sort_status = j.sort_status;
+	const uint32_t* __restrict__ order_status = j.order_status;
+	uint32_t* __restrict__ fault = j.fault;
+	uint4* __restrict__ file_tail = j.file_tail;
+	if ((size_t)blockIdx.x * kFileBlock >= j.n)
+		return;  // the launch is sized for the job with the most keys
+	const size_t idx = (size_t)blockIdx.x * kFileBlock + threadIdx.x;
 	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u)) {
 		if (idx == 0 && fault)
 			__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -610,20 +804,47 @@ __global__ __launch_bounds__(256) void tile_ranges_kernel(const uint32_t* __rest
 	}
 	if (n_device)
 		n = min(n, (size_t)*n_device);  // launched for an upper bound
-	if (idx >= n)
+	if ((size_t)blockIdx.x * kFileBlock >= n)
 		return;
-	const uint32_t cur = keys[idx];
-	if (idx == 0) {
-		ranges[cur].x = 0;
-	} else {
-		const uint32_t prev = keys[idx - 1];
-		if (cur != prev) {
-			ranges[prev].y = (uint32_t)idx;
-			ranges[cur].x = (uint32_t)idx;
+	const bool valid = idx < n;
+	const uint32_t key = valid ? keys[idx] : 0u;
+	const uint32_t cur = key_tile(key);
+	if (valid) {
+		if (idx == 0) {
+			ranges[cur].x = 0;
+		} else {
+			const uint32_t prev = key_tile(keys[idx - 1]);
+			if (cur != prev) {
+				ranges[prev].y = (uint32_t)idx;
+				ranges[cur].x = (uint32_t)idx;
+			}
 		}
+		if (idx == n - 1)
+			ranges[cur].y = (uint32_t)n;
 	}
-	if (idx == n - 1)
-		ranges[cur].y = (uint32_t)n;
+	if (!file_tail)
+		return;
+	const size_t last = min(n, ((size_t)blockIdx.x + 1) * kFileBlock) - 1;
+	if (idx == last)
+		s_last_tile = cur;
+	__syncthreads();
+	const bool counted = valid && cur == s_last_tile;  // sorted: these are the workgroup's last keys
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+	for (int s = 0; s < 4; s++) {
+		const uint64_t m = __ballot(counted && ((key_strips(key) >> s) & 1u));
+		if (lane == 0)
+			s_tail[wave][s] = (uint32_t)__popcll(m);
+	}
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		uint4 t;
+		t.x = s_tail[0][0] + s_tail[1][0] + s_tail[2][0] + s_tail[3][0];
+		t.y = s_tail[0][1] + s_tail[1][1] + s_tail[2][1] + s_tail[3][1];
+		t.z = s_tail[0][2] + s_tail[1][2] + s_tail[2][2] + s_tail[3][2];
+		t.w = s_tail[0][3] + s_tail[1][3] + s_tail[2][3] + s_tail[3][3];
+		file_tail[blockIdx.x] = t;
+	}
 }
 
 __global__ void report_sort_status_kernel(const uint32_t* __restrict__ status, uint32_t* __restrict__ fault)
@@ -638,17 +859,24 @@ void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_
 		hipLaunchKernelGGL(report_sort_status_kernel, dim3(1), dim3(64), 0, s, temp + kSortStatus, fault);
 }
 
-void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device, uint2* ranges, int tiles,
-                        const uint32_t* sort_status, const uint32_t* order_status, uint32_t* fault, bool ranges_cleared,
-                        hipStream_t s)
+void launch_tile_ranges(const TileRangesJob* jobs, int count, hipStream_t s)
 {
 	stage_mark("tile_ranges", s);
-	if (!ranges_cleared)
-		launch_fill_u32(reinterpret_cast<uint32_t*>(ranges), 0u, (size_t)tiles * 2 + kRangeTailWords, s);
-	if (n == 0)
-		return;
-	hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, keys, n, n_device,
-	                   ranges, sort_status, order_status, fault);
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<TileRangesJob> b = {};
+		size_t max_n = 0;
+		int live = 0;
+		for (int k = 0; k < nj; k++) {
+			if (jobs[at + k].n == 0)
+				continue;
+			b.job[live++] = jobs[at + k];
+			max_n = jobs[at + k].n > max_n ? jobs[at + k].n : max_n;
+		}
+		if (live)
+			hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((max_n + kFileBlock - 1) / kFileBlock), (unsigned)live),
+			                   dim3(kFileBlock), 0, s, b);
+	}
 }
 
 }  // namespace rgs

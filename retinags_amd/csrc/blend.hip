@@ -1,8 +1,7 @@
 // Per-tile alpha blending, forward and backward.  A 16x16 tile is four strips of 16x4 pixels;
-// a wavefront owns one strip, one pixel per lane.  The forward runs a tile's four wavefronts
-// in one 256-thread block, the backward launches every strip as a block of its own (strips
-// end at very different times there, and a wave slot should not idle until its tile's longest
-// strip is done), longest strips first.
+// a wavefront owns one strip, one pixel per lane, and every strip is a workgroup of its own
+// (strips end at very different times, and a wave slot should not idle until its tile's longest
+// strip is done); the backward takes the longest strips first.
 //
 // Compiled with -ffp-contract=off: every per-pixel decision (power > 0, alpha < 1/255,
 // the half-Gaussian box test, T(1-alpha) < 1e-4) is evaluated with the unfused
@@ -10,27 +9,23 @@
 // (K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian), so a pixel
 // can only differ from that evaluation through the last-bit behaviour of exp().
 //
-// The four wavefronts of a block never synchronise with each other: measured per wave, more
-// than half of a heavy tile's time used to go into waiting for the slowest strip at the
-// end-of-batch barrier.  Each wavefront instead streams the tile's list by itself in chunks
-// of 64 entries (lane l takes entry l of the chunk; the next chunk's records and the ids of
-// the one after are already in flight while the current chunk is processed), keeps the
-// entries that can matter to its strip in a wave-private LDS list, and walks that list.
-// The forward also writes those entries' list positions out, strip by strip; the backward
-// walks exactly them (up to the last one any pixel blended) and repeats none of the filtering.
+// Blending front to back gives a strip no parallelism beyond its 64 pixels, but deciding which
+// entries of a tile's list can matter to a strip needs no order at all.  So the work is split:
+// the kernel that emits the (Gaussian, tile) instances decides for each of them which of the
+// tile's four strips it can matter to (strip_filing.h) and sends that along with the tile key
+// through the sort; a placing kernel turns the sorted bits into one list per strip (the list
+// positions that matter to it, in list order); the blend kernels then walk only those, in chunks
+// of 64 (lane l takes entry l of the chunk; the next chunk's records, the ids of the one after and
+// the positions of the one after that are already in flight while the current chunk is
+// processed).  With many small Gaussians a tile's list runs to tens of thousands of entries of
+// which a strip needs a few thousand at most.  The backward walks the same filed lists, up to the
+// last entry any pixel blended.
 //
-// Most (pixel, Gaussian) visits of the reference loop end at "alpha < 1/255" or at the box
-// test.  Three conservative filters remove such visits without changing any result:
-//  * alpha >= 1/255 needs power >= -ln(255 * opacity); that floor (minus a margin) is stored
-//    with the Gaussian, and a group of entries is skipped with one ballot when no live lane
-//    reaches it, before exp() is evaluated.
-//  * power >= floor is an ellipse around the Gaussian's centre; an entry whose ellipse (first
-//    its bounding box, then the ellipse itself) misses the strip's rectangle is not filed at all.
-//  * the world-space ray sample is affine in the pixel, so its extremes over the strip are at
-//    the strip's corner pixels: an entry whose corners are all outside the submodel box is not
-//    filed, one whose corners are all inside skips the per-pixel box test.
-// All three only drop work that the exact evaluation would have skipped too.
+// Inside the walk, alpha >= 1/255 needs power >= -ln(255 * opacity); that floor (minus a margin) is
+// stored with the Gaussian, and a group of four entries is skipped with one ballot when no live
+// lane reaches it, before exp() is evaluated.
 #include "rgs_kernels.h"
+#include "strip_filing.h"
 #include "tile_order.h"
 
 namespace rgs {
@@ -39,33 +34,9 @@ struct PixelRay {
 	float ndc_x, ndc_y;  // pixel centre in NDC
 };
 
-__device__ __forceinline__ float wave_uniform(float v)
-{
-	return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
-}
-
-// What the half-Gaussian test needs besides the pixel: rows 0..2 of the inverse projection
-// (column-major 4x4, m[c][r] = element (r, c)) and the submodel box.  Read once per wavefront
-// into scalar registers; the test itself runs for every blended sample.
-struct BoxFrame {
-	float m[4][3];
-	float3 lo, hi;
-	float tanx, tany;
-};
-
 __device__ __forceinline__ BoxFrame load_box_frame(const BlendArgs& a)
 {
-	BoxFrame b;
-#pragma unroll
-	for (int c = 0; c < 4; c++)
-#pragma unroll
-		for (int r = 0; r < 3; r++)
-			b.m[c][r] = wave_uniform(a.projinv[4 * c + r]);
-	b.lo = float3{wave_uniform(a.range_low[0]), wave_uniform(a.range_low[1]), wave_uniform(a.range_low[2])};
-	b.hi = float3{wave_uniform(a.range_up[0]), wave_uniform(a.range_up[1]), wave_uniform(a.range_up[2])};
-	b.tanx = a.tanfovx;
-	b.tany = a.tanfovy;
-	return b;
+	return load_box_frame(a.projinv, a.range_low, a.range_up, a.tanfovx, a.tanfovy);
 }
 
 // World-space point of the pixel's ray at clip-w `w`, tested against the submodel box
@@ -93,117 +64,12 @@ __device__ __forceinline__ float exp_of_exponent(float x)
 	return __builtin_fmaf(e, r * 0.693147182f, e);
 }
 
-// True if some pixel of the strip whose first pixel is (x0, ya) (16 wide, 4 high) may reach
-// power >= floor, judged by the bounding box (half-widths hx, hy) of that ellipse.  Written so
-// that NaN keeps the entry.
-__device__ __forceinline__ bool reaches_strip(float gx, float gy, float hx, float hy, float floor, float x0, float ya)
-{
-	if (floor > 0.f)
-		return false;  // even power = 0 gives alpha < 1/255
-	return !((gx + hx < x0) || (gx - hx > x0 + 15.f) || (gy + hy < ya) || (gy - hy > ya + 3.f));
-}
-
-// The same question answered with the ellipse itself: the smallest value over the strip's
-// rectangle of q(d) = a dx^2 + 2 b dx dy + c dy^2 (d = centre - pixel, conic = (a, b, c)), against
-// the -2 floor that power = -q / 2 >= floor allows.  With the centre outside the rectangle the
-// minimum of the convex q lies on one of the four edges, where it is a clamped parabola vertex.
-// Conservative: the rectangle contains the pixels, and the comparison leaves room for the
-// rounding of q (relative to its largest terms).  Anything that is not an ellipse, or NaN, is kept.
-__device__ __forceinline__ bool ellipse_reaches_strip(float gx, float gy, const float4 co, float floor, float x0, float ya)
-{
-	const float a = co.x, b = co.y, c = co.z;
-	if (!(a > 0.f) || !(c > 0.f) || !(a * c - b * b > 0.f))
-		return true;
-	const float dxl = gx - (x0 + 15.f), dxh = gx - x0, dyl = gy - (ya + 3.f), dyh = gy - ya;
-	if (!(dxl > 0.f) && !(dxh < 0.f) && !(dyl > 0.f) && !(dyh < 0.f))
-		return true;  // the centre lies within the strip
-	float qmin = INFINITY;
-#pragma unroll
-	for (int edge = 0; edge < 2; edge++) {
-		const float dy = edge ? dyh : dyl;
-		const float dx = fminf(dxh, fmaxf(dxl, -b * dy / a));
-		qmin = fminf(qmin, (a * dx + 2.f * b * dy) * dx + c * dy * dy);
-	}
-#pragma unroll
-	for (int edge = 0; edge < 2; edge++) {
-		const float dx = edge ? dxh : dxl;
-		const float dy = fminf(dyh, fmaxf(dyl, -b * dx / c));
-		qmin = fminf(qmin, (c * dy + 2.f * b * dx) * dy + a * dx * dx);
-	}
-	const float largest = a * fmaxf(dxl * dxl, dxh * dxh) + c * fmaxf(dyl * dyl, dyh * dyh);
-	const float limit = -2.f * floor;
-	return !(qmin > limit + (1e-3f + 1e-4f * limit + 1e-5f * largest));
-}
-
-// Where the rays of a whole strip, sampled at clip-w `w`, fall relative to the submodel box.
-// With a tolerance far above the rounding error of the affine map: kBoxInside = every pixel's
-// exact test passes, kBoxOutside = every pixel's exact test fails, kBoxMixed = decide per pixel.
-enum { kBoxMixed = 0, kBoxInside = 1, kBoxOutside = 2 };
-
-struct StripCorners {
-	float nx0, nx1, ny0, ny1;  // NDC of the strip's first/last pixel column and row
-};
-
-__device__ __forceinline__ int classify_strip_against_box(float w, const StripCorners& sc, const BoxFrame& b)
-{
-	float pmin[3] = {INFINITY, INFINITY, INFINITY}, pmax[3] = {-INFINITY, -INFINITY, -INFINITY};
-#pragma unroll
-	for (int c = 0; c < 4; c++) {
-		const float nx = (c & 1) ? sc.nx1 : sc.nx0;
-		const float ny = (c & 2) ? sc.ny1 : sc.ny0;
-		const float3 ph = {nx * (w + 0.0000001f) * b.tanx, ny * (w + 0.0000001f) * b.tany, w};
-		const float q[3] = {b.m[0][0] * ph.x + b.m[1][0] * ph.y + b.m[2][0] * ph.z + b.m[3][0],
-		                    b.m[0][1] * ph.x + b.m[1][1] * ph.y + b.m[2][1] * ph.z + b.m[3][1],
-		                    b.m[0][2] * ph.x + b.m[1][2] * ph.y + b.m[2][2] * ph.z + b.m[3][2]};
-#pragma unroll
-		for (int k = 0; k < 3; k++) {
-			pmin[k] = fminf(pmin[k], q[k]);
-			pmax[k] = fmaxf(pmax[k], q[k]);
-		}
-	}
-	const float lov[3] = {b.lo.x, b.lo.y, b.lo.z}, hiv[3] = {b.hi.x, b.hi.y, b.hi.z};
-	bool inside = true, outside = false;
-#pragma unroll
-	for (int k = 0; k < 3; k++) {
-		const float tol = 1e-4f * fmaxf(fmaxf(fabsf(pmin[k]), fabsf(pmax[k])), 1.f);
-		inside = inside && (pmin[k] > lov[k] + tol) && (pmax[k] < hiv[k] - tol);
-		outside = outside || (pmax[k] < lov[k] - tol) || (pmin[k] > hiv[k] + tol);
-	}
-	// a NaN can set neither flag, which leaves the decision to the per-pixel test
-	return outside ? kBoxOutside : (inside ? kBoxInside : kBoxMixed);
-}
-
 // Launch-order classes of the backward's strips, by the number of entries they have to walk.
 constexpr int kStripClasses = 256;
 __device__ __forceinline__ uint32_t strip_class(uint32_t filed) { return 255u - min(filed >> 3, 255u); }
 
 constexpr int kPerLane = 1;             // list entries per lane and step (2 was measured slower)
 constexpr int kChunk = 64 * kPerLane;   // list entries a wavefront takes per step
-
-// One entry of the tile list as a lane holds it between the load and the filter.
-struct LoadedEntry {
-	float4 geom, conic, cd, half;
-	uint32_t id;
-};
-
-__device__ __forceinline__ LoadedEntry load_entry(const BlendArgs& a, uint32_t id, bool in_range)
-{
-	LoadedEntry e;
-	e.id = id;
-	if (in_range) {
-		const float4* rec = a.record + 4 * (size_t)id;
-		e.geom = rec[0];
-		e.conic = rec[1];
-		e.cd = rec[2];
-		e.half = rec[3];
-	} else {
-		e.geom = float4{0.f, 0.f, INFINITY, 0.f};  // floor = +inf: never filed
-		e.conic = float4{0.f, 0.f, 0.f, 0.f};
-		e.cd = float4{0.f, 0.f, 0.f, 0.f};
-		e.half = float4{0.f, 0.f, 0.f, 0.f};
-	}
-	return e;
-}
 
 // What the backward reads of a record: it takes the forward's word for which entries matter.
 struct LoadedRecord {
@@ -228,35 +94,100 @@ __device__ __forceinline__ LoadedRecord load_record(const BlendArgs& a, uint32_t
 	return e;
 }
 
-// The last two words of a record are padding.  Registers that a load in flight will write
-// cannot be reused, but the compiler would hand these two to the walk as temporaries, and the
-// walk would then wait for the very prefetch it is meant to overlap; naming them as used after
-// the walk keeps them reserved.
-__device__ __forceinline__ void keep_padding_registers(const LoadedEntry& e)
-{
-	asm volatile("" ::"v"(e.half.z), "v"(e.half.w));
-}
-
-// Decides whether the lane's entry is filed for this strip; a filed entry whose strip lies
-// entirely inside the box gets a NaN clip-w, which tells the walk to skip the per-pixel test.
-__device__ __forceinline__ bool file_entry(LoadedEntry& e, float x0, float ya, const StripCorners& sc, const BoxFrame& box)
-{
-	if (!reaches_strip(e.geom.x, e.geom.y, e.half.x, e.half.y, e.geom.z, x0, ya))
-		return false;
-	if (!ellipse_reaches_strip(e.geom.x, e.geom.y, e.conic, e.geom.z, x0, ya))
-		return false;
-	const int where = classify_strip_against_box(e.geom.w, sc, box);
-	if (where == kBoxOutside)
-		return false;
-	if (where == kBoxInside)
-		e.geom.w = __int_as_float(0x7FC00000);
-	return true;
-}
-
 __device__ __forceinline__ float exponent_of(const float4 g, const float4 co, const float2 pixf, float2& d)
 {
 	d = float2{g.x - pixf.x, g.y - pixf.y};
 	return -0.5f * (co.x * d.x * d.x + co.z * d.y * d.y) - co.y * d.x * d.y;
+}
+
+// ---- filing ------------------------------------------------------------------------------------
+// The sorted keys carry, above the tile, one bit per strip the entry is filed for and one per strip
+// that lies inside the box (key_strips).  A workgroup takes 256 consecutive positions of the sorted
+// list, whichever tiles they belong to.  An entry's rank in its strip's list is the number of filed
+// entries of its tile before it: those inside the workgroup are counted from the ballots, those in
+// earlier workgroups (only the tile of the workgroup's first entry can have any) are the sum, over
+// the workgroups since that tile began, of what each filed for the tile of its LAST entry, which the
+// tile-range kernel has left in file_tail.  The thread that holds a tile's last entry also writes
+// the strips' totals.
+
+struct FileBallots {
+	uint64_t set[4][4];  // [wave][strip]
+};
+
+// Number of set bits of strip s among threads [0, i) of the workgroup.
+__device__ __forceinline__ uint32_t filed_before(const FileBallots& b, int s, int i)
+{
+	uint32_t n = 0;
+	const int w = i >> 6;
+#pragma unroll
+	for (int k = 0; k < 4; k++)
+		if (k < w)
+			n += (uint32_t)__popcll(b.set[k][s]);
+	if (w < 4)
+		n += (uint32_t)__popcll(b.set[w][s] & ((1ull << (i & 63)) - 1ull));
+	return n;
+}
+
+__global__ __launch_bounds__(kFileBlock) void strip_file_place_kernel(BlendBatch batch)
+{
+	__shared__ FileBallots s_ballots;
+	__shared__ uint32_t s_carry[4][4];  // [wave][strip] partial sums of the earlier workgroups' counts
+	const BlendArgs& a = batch.job[blockIdx.y];
+	const uint32_t capacity = a.capacity;
+	const uint32_t R = a.count_device ? min(capacity, *a.count_device) : capacity;
+	const uint32_t first = blockIdx.x * kFileBlock;
+	// after a sort that gave up the list is not sorted and the tile ranges are empty: nothing to place
+	if (first >= R || (a.sort_status && *a.sort_status != 0u) || (a.order_status && *a.order_status != 0u))
+		return;
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const uint32_t pos = first + (uint32_t)tid;
+	const bool valid = pos < R;
+	const uint32_t key = valid ? a.tile_keys[pos] : 0u;
+	const uint32_t bits = key_strips(key), tile = key_tile(key);
+	const uint2 range = valid ? a.ranges[tile] : uint2{0u, 0u};
+#pragma unroll
+	for (int s = 0; s < 4; s++) {
+		const uint64_t m = __ballot((bits >> s) & 1u);
+		if (lane == 0)
+			s_ballots.set[wave][s] = m;
+	}
+	// what the tile of this workgroup's first entry filed in the workgroups before this one
+	{
+		const uint32_t begin0 = a.ranges[key_tile(a.tile_keys[first])].x;
+		uint4 sum = {0u, 0u, 0u, 0u};
+		if (begin0 < first)
+			for (uint32_t g = begin0 / kFileBlock + (uint32_t)tid; g < blockIdx.x; g += kFileBlock) {
+				const uint4 t = a.file_tail[g];
+				sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+			}
+		uint32_t v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+		for (int s = 0; s < 4; s++) {
+			const uint32_t tot = wave_inclusive_scan_u32(v[s]);
+			if (lane == 63)
+				s_carry[wave][s] = tot;
+		}
+	}
+	__syncthreads();
+	if (!valid)
+		return;
+	const bool continues = range.x < first;  // the tile began in an earlier workgroup
+	const int begin = (int)(max(range.x, first) - first);
+	const uint32_t n = range.y - range.x, e = pos - range.x;
+	uint32_t* lists = a.strip_lists + 4 * (size_t)range.x;
+	uint32_t rank[4];
+#pragma unroll
+	for (int s = 0; s < 4; s++) {
+		const uint32_t carry = continues ? s_carry[0][s] + s_carry[1][s] + s_carry[2][s] + s_carry[3][s] : 0u;
+		rank[s] = carry + filed_before(s_ballots, s, tid) - filed_before(s_ballots, s, begin);
+		if ((bits >> s) & 1u)
+			lists[(size_t)s * n + rank[s]] = e | (((bits >> (4 + s)) & 1u) ? 0x80000000u : 0u);
+	}
+	if (pos + 1u == range.y) {  // the tile's last entry: its ranks plus itself are the strips' totals
+		uint4 total = {rank[0] + (bits & 1u), rank[1] + ((bits >> 1) & 1u), rank[2] + ((bits >> 2) & 1u),
+		               rank[3] + ((bits >> 3) & 1u)};
+		reinterpret_cast<uint4*>(a.strip_total)[tile] = total;
+	}
 }
 
 // ---- forward (K/cuda_rasterizer_hgs/forward.cu:263-405) ---------------------------------------
@@ -268,7 +199,7 @@ struct ForwardPixel {
 	uint32_t last_filed;  // like last_contributor, but counted in entries filed for the strip
 };
 
-struct ForwardStage {  // wave-private
+struct ForwardStage {  // one per workgroup (a single wavefront)
 	float4 geom[kChunk + 3];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
 	float4 conic[kChunk + 3];  // conic xx, xy, yy, opacity
 	float4 cd[kChunk];         // r, g, b, view depth
@@ -305,14 +236,17 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 	}
 }
 
-__global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
+__global__ __launch_bounds__(64) void blend_forward_kernel(BlendBatch batch)
 {
-	__shared__ ForwardStage s_stage[4];
+	__shared__ ForwardStage st;
 
-	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const int tile = tile_of_block((int)blockIdx.x, a.grid_x, a.grid_y);
-	if (tile < 0)
-		return;
+	const int lane = threadIdx.x;
+	// The jobs of a batch (the submodels of a frame) take turns, each handing out its strips longest
+	// list first: a long strip that starts late is what a launch waits for, and with several jobs in one
+	// launch there is other work to run beside the longest strips of each.
+	const BlendArgs& a = batch.job[blockIdx.x % (uint32_t)batch.count];
+	const uint32_t strip_id = a.strip_order_forward[blockIdx.x / (uint32_t)batch.count];
+	const int tile = (int)(strip_id >> 2), wave = (int)(strip_id & 3u);  // wave: which strip of the tile
 	const uint2 range = a.ranges[tile];
 	const uint32_t n = range.y - range.x;
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
@@ -322,64 +256,49 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 	const float2 pixf = {(float)px, (float)py};
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
 	const BoxFrame box = load_box_frame(a);
-	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
-	const StripCorners sc = {pix_to_ndc(strip_x0, a.W), pix_to_ndc(strip_x0 + 15.f, a.W), pix_to_ndc(strip_y0, a.H),
-	                         pix_to_ndc(strip_y0 + 3.f, a.H)};
-	ForwardStage& st = s_stage[wave];
-	const uint64_t below = (1ull << lane) - 1ull;
 
 	ForwardPixel p = {!inside, 1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u, 0u};
 	uint64_t live = __ballot(!p.done);
-	// The entries filed for this strip are also written out, for the backward pass: their list
-	// positions in order, bit 31 set where the strip lies inside the box.  The backward needs
-	// them up to the last one that some pixel blended (the largest last_filed of the strip).
-	uint32_t* filed_list = a.strip_lists + 4 * (size_t)range.x + (size_t)wave * n;
-	uint32_t filed_total = 0;
+	// the entries filed for this strip, in list order: list position, bit 31 = strip inside the box
+	const uint32_t filed = a.strip_total[strip_id];
 
-	if (n != 0u && live != 0ull) {
+	if (filed != 0u && live != 0ull) {
 		const uint32_t* list = a.point_list + range.x;
-		// lane l holds entries first + 64 e + l (e < kPerLane) of the chunk; the next chunk's records
-		// and the ids of the chunk after it are in flight while the current one is walked
-		LoadedEntry cur[kPerLane];
-		uint32_t id_next[kPerLane];
-#pragma unroll
-		for (int e = 0; e < kPerLane; e++) {
-			const uint32_t i0 = 64 * e + lane, i1 = kChunk + i0;
-			cur[e] = load_entry(a, i0 < n ? list[i0] : 0u, i0 < n);
-			id_next[e] = i1 < n ? list[i1] : 0u;
-		}
+		const uint32_t* filed_list = a.strip_lists + 4 * (size_t)range.x + (size_t)wave * n;
+		constexpr uint32_t kNone = 0xFFFFFFFFu, kPosition = 0x7FFFFFFFu;
+		// Lane l of the chunk that starts at filed entry `first` takes entry first + l: its list
+		// position (and box flag), through that the Gaussian's index, through that its record.
+		// Three chunks are in flight: the records of the next one, the indices of the one after,
+		// the positions of the one after that.
+		uint32_t pos_cur = (uint32_t)lane < filed ? filed_list[lane] : kNone;
+		uint32_t pos_next = (uint32_t)(64 + lane) < filed ? filed_list[64 + lane] : kNone;
+		uint32_t pos_after = (uint32_t)(128 + lane) < filed ? filed_list[128 + lane] : kNone;
+		LoadedRecord cur = load_record(a, pos_cur != kNone ? list[pos_cur & kPosition] : 0u, pos_cur != kNone);
+		uint32_t id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
 
-		for (uint32_t first = 0; first < n && live != 0ull; first += kChunk) {
-			int count = 0;
-#pragma unroll
-			for (int e = 0; e < kPerLane; e++) {
-				const bool filed = file_entry(cur[e], strip_x0, strip_y0, sc, box);
-				const uint64_t m = __ballot(filed);
-				if (filed) {
-					const int slot = count + __popcll(m & below);
-					st.geom[slot] = cur[e].geom;
-					st.conic[slot] = cur[e].conic;
-					st.cd[slot] = cur[e].cd;
-					st.position[slot] = first + 64 * e + lane + 1;
-					const bool strip_inside_box = cur[e].geom.w != cur[e].geom.w;
-					filed_list[filed_total + slot] = (first + 64 * e + lane) | (strip_inside_box ? 0x80000000u : 0u);
-				}
-				count += __popcll(m);
+		for (uint32_t first = 0; first < filed && live != 0ull; first += 64) {
+			const int count = (int)min(filed - first, 64u);
+			if (lane < count) {
+				float4 g = cur.geom;
+				if (pos_cur & 0x80000000u)
+					g.w = __int_as_float(0x7FC00000);  // the strip lies inside the box: no per-pixel test
+				st.geom[lane] = g;
+				st.conic[lane] = cur.conic;
+				st.cd[lane] = cur.cd;
+				st.position[lane] = (pos_cur & kPosition) + 1u;
 			}
-			const uint32_t chunk_base = filed_total;
-			filed_total += (uint32_t)count;
 			if (lane < 3) {  // pad to a multiple of four with entries that never pass the floor test
 				st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
 				st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
 			}
 			__builtin_amdgcn_wave_barrier();
 			// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
-#pragma unroll
-			for (int e = 0; e < kPerLane; e++) {
-				const uint32_t i1 = first + kChunk + 64 * e + lane, i2 = i1 + kChunk;
-				cur[e] = load_entry(a, id_next[e], i1 < n);
-				id_next[e] = i2 < n ? list[i2] : 0u;
-			}
+			cur = load_record(a, id_next, pos_next != kNone);
+			pos_cur = pos_next;
+			pos_next = pos_after;
+			id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
+			const uint32_t e3 = first + 192 + (uint32_t)lane;
+			pos_after = e3 < filed ? filed_list[e3] : kNone;
 
 			for (int k = 0; k < count && live != 0ull; k += 4) {
 				const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
@@ -392,7 +311,7 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
 				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
 					continue;
-				const uint32_t f = chunk_base + (uint32_t)k;
+				const uint32_t f = first + (uint32_t)k;
 				forward_visit(p, q0, w0, g0, c0, st, k, f + 1, ray, box);
 				forward_visit(p, q1, w1, g1, c1, st, k + 1, f + 2, ray, box);
 				forward_visit(p, q2, w2, g2, c2, st, k + 2, f + 3, ray, box);
@@ -400,19 +319,17 @@ __global__ __launch_bounds__(256) void blend_forward_kernel(BlendArgs a)
 				live = __ballot(!p.done);
 			}
 			__builtin_amdgcn_wave_barrier();
-#pragma unroll
-			for (int e = 0; e < kPerLane; e++)
-				keep_padding_registers(cur[e]);
 		}
 	}
 
 	{
+		// how many of the filed entries the backward has to walk: up to the last one some pixel blended
 		uint32_t upto = inside ? p.last_filed : 0u;
 #pragma unroll
 		for (int off = 32; off > 0; off >>= 1)
 			upto = max(upto, (uint32_t)__shfl_xor((int)upto, off));
 		if (lane == 0)
-			a.strip_filed[4 * tile + wave] = upto;
+			a.strip_filed[strip_id] = upto;
 	}
 	if (inside) {
 		const size_t plane = (size_t)a.H * a.W;
@@ -669,13 +586,15 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	}
 }
 
-__global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
+__global__ __launch_bounds__(64) void blend_backward_kernel(BlendBatch batch)
 {
 	__shared__ BackwardStage s_stage;
 
 	const int lane = threadIdx.x;
-	// strips with the most entries first: a long strip that starts late is what the whole launch waits for
-	const uint32_t strip_id = a.strip_order[blockIdx.x];
+	// the jobs of the batch take turns; each hands out its strips with the most entries first: a long
+	// strip that starts late is what the whole launch waits for
+	const BlendArgs& a = batch.job[blockIdx.x % (uint32_t)batch.count];
+	const uint32_t strip_id = a.strip_order[blockIdx.x / (uint32_t)batch.count];
 	const int tile = (int)(strip_id >> 2), wave = (int)(strip_id & 3u);  // wave: which strip of the tile
 	const uint2 range = a.ranges[tile];
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
@@ -781,73 +700,129 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendArgs a)
 		flush_rows(st, rows, frame, a, lane);
 }
 
-// Strips by decreasing number of filed entries, in kStripClasses classes of 8 (longer ones share
+// Strips by decreasing number of entries to walk, in kStripClasses classes of 8 (longer ones share
 // the first class); the order inside a class is whatever the atomics give, which is all a
-// launch order needs.  Two small kernels: count the strips of every class, then place them.
-// Both aggregate in LDS first: most strips fall into one class (nothing to walk), and
-// thousands of global atomics on one word would take longer than the blend itself.
-__global__ __launch_bounds__(256) void strip_count_kernel(const uint32_t* __restrict__ filed, uint32_t n,
-                                                           uint32_t* __restrict__ class_count)
+// launch order needs.  Two small kernels: count the strips of every class, then place them; one
+// launch of each serves every job of a batch (blockIdx.y).  Both aggregate in LDS first: most
+// strips fall into one class (nothing to walk), and thousands of global atomics on one word would
+// take longer than the blend itself.
+struct StripOrderJob {
+	const uint32_t* length;  // per strip
+	uint32_t* classes;       // kStripClasses counters and as many placement cursors, zero beforehand
+	uint32_t* order;
+};
+struct StripOrderBatch {
+	StripOrderJob job[kMaxBlendBatch];
+	uint32_t strips;
+};
+
+__global__ __launch_bounds__(256) void strip_count_kernel(StripOrderBatch batch)
 {
 	__shared__ uint32_t s_count[kStripClasses];
+	const StripOrderJob& j = batch.job[blockIdx.y];
 	s_count[threadIdx.x] = 0;
 	__syncthreads();
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
-	if (k < n)
-		atomicAdd(&s_count[strip_class(filed[k])], 1u);
+	if (k < batch.strips)
+		atomicAdd(&s_count[strip_class(j.length[k])], 1u);
 	__syncthreads();
 	if (s_count[threadIdx.x] != 0u)
-		atomicAdd(&class_count[threadIdx.x], s_count[threadIdx.x]);
+		atomicAdd(&j.classes[threadIdx.x], s_count[threadIdx.x]);
 }
 
-__global__ __launch_bounds__(256) void strip_place_kernel(const uint32_t* __restrict__ filed, uint32_t n,
-                                                           const uint32_t* __restrict__ class_count,
-                                                           uint32_t* __restrict__ class_cursor,
-                                                           uint32_t* __restrict__ order)
+__global__ __launch_bounds__(256) void strip_place_kernel(StripOrderBatch batch)
 {
 	__shared__ uint32_t s_count[kStripClasses];  // strips of this block per class, then where they go
 	__shared__ uint32_t s_scan[8];
+	const StripOrderJob& j = batch.job[blockIdx.y];
 	s_count[threadIdx.x] = 0;
 	__syncthreads();
 	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
 	uint32_t c = 0, rank = 0;
-	if (k < n) {
-		c = strip_class(filed[k]);
+	if (k < batch.strips) {
+		c = strip_class(j.length[k]);
 		rank = atomicAdd(&s_count[c], 1u);
 	}
 	__syncthreads();
 	uint32_t total;
-	const uint32_t start = block256_exclusive_scan_u32(class_count[threadIdx.x], s_scan, total);
+	const uint32_t start = block256_exclusive_scan_u32(j.classes[threadIdx.x], s_scan, total);
 	const uint32_t mine = s_count[threadIdx.x];
 	__syncthreads();
-	s_count[threadIdx.x] = start + (mine != 0u ? atomicAdd(&class_cursor[threadIdx.x], mine) : 0u);
+	s_count[threadIdx.x] = start + (mine != 0u ? atomicAdd(&j.classes[kStripClasses + threadIdx.x], mine) : 0u);
 	__syncthreads();
-	if (k < n)
-		order[s_count[c] + rank] = k;
+	if (k < batch.strips)
+		j.order[s_count[c] + rank] = k;
 }
 
-void launch_blend_forward(const BlendArgs& a, hipStream_t s)
+// which: 0 = the forward's order (by the entries filed), 1 = the backward's (by the entries up to the last one blended)
+static void launch_strip_order(const BlendArgs* jobs, int count, int which, hipStream_t s)
 {
-	stage_mark(a.counters ? "blend_count" : "blend_forward", s);
-	if (a.counters)
-		hipLaunchKernelGGL(blend_count_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
-	else
-	{
-		hipLaunchKernelGGL(blend_forward_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
-		// the order in which the backward will take the strips (longest first was measured no
-		// faster for the forward's tiles, whose length is only known as the list length)
-		const uint32_t strips = (uint32_t)(4 * a.grid_x * a.grid_y);
-		hipLaunchKernelGGL(strip_count_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_filed, strips,
-		                   a.strip_classes);
-		hipLaunchKernelGGL(strip_place_kernel, dim3((strips + 255) / 256), dim3(256), 0, s, a.strip_filed, strips,
-		                   a.strip_classes, a.strip_classes + kStripClasses, a.strip_order);
+	StripOrderBatch b;
+	b.strips = (uint32_t)(4 * jobs[0].grid_x * jobs[0].grid_y);
+	for (int k = 0; k < count; k++) {
+		b.job[k].length = which == 0 ? jobs[k].strip_total : jobs[k].strip_filed;
+		b.job[k].classes = jobs[k].strip_classes + (which == 0 ? 2 * kStripClasses : 0);
+		b.job[k].order = which == 0 ? jobs[k].strip_order_forward : jobs[k].strip_order;
+	}
+	const dim3 grid((b.strips + 255) / 256, (unsigned)count);
+	hipLaunchKernelGGL(strip_count_kernel, grid, dim3(256), 0, s, b);
+	hipLaunchKernelGGL(strip_place_kernel, grid, dim3(256), 0, s, b);
+}
+
+void launch_blend_count(const BlendArgs& a, hipStream_t s)
+{
+	stage_mark("blend_count", s);
+	hipLaunchKernelGGL(blend_count_kernel, dim3(tile_order_blocks(a.grid_x, a.grid_y)), dim3(256), 0, s, a);
+}
+
+void launch_strip_filing(const BlendArgs* jobs, int count, hipStream_t s)
+{
+	stage_mark("strip_filing", s);
+	for (int at = 0; at < count; at += kMaxBlendBatch) {
+		BlendBatch batch;
+		batch.count = 0;
+		uint32_t most = 0;
+		for (int k = at; k < count && k < at + kMaxBlendBatch; k++)
+			if (jobs[k].capacity != 0u) {
+				batch.job[batch.count++] = jobs[k];
+				most = jobs[k].capacity > most ? jobs[k].capacity : most;
+			}
+		if (batch.count)
+			hipLaunchKernelGGL(strip_file_place_kernel, dim3((most + kFileBlock - 1) / kFileBlock, (unsigned)batch.count),
+			                   dim3(kFileBlock), 0, s, batch);
 	}
 }
 
-void launch_blend_backward(const BlendArgs& a, hipStream_t s)
+// All jobs share the image size (they are the submodels of one frame, or a single call).
+void launch_blend_forward(const BlendArgs* jobs, int count, hipStream_t s)
 {
+	const unsigned strips = (unsigned)(4 * jobs[0].grid_x * jobs[0].grid_y);
+	for (int at = 0; at < count; at += kMaxBlendBatch) {
+		BlendBatch batch;
+		batch.count = count - at < kMaxBlendBatch ? count - at : kMaxBlendBatch;
+		for (int k = 0; k < batch.count; k++)
+			batch.job[k] = jobs[at + k];
+		stage_mark("strip_order", s);
+		launch_strip_order(jobs + at, batch.count, 0, s);
+		stage_mark("blend_forward", s);
+		hipLaunchKernelGGL(blend_forward_kernel, dim3(strips * (unsigned)batch.count), dim3(64), 0, s, batch);
+		// the order in which the backward will take the strips
+		stage_mark("strip_order", s);
+		launch_strip_order(jobs + at, batch.count, 1, s);
+	}
+}
+
+void launch_blend_backward(const BlendArgs* jobs, int count, hipStream_t s)
+{
+	const unsigned strips = (unsigned)(4 * jobs[0].grid_x * jobs[0].grid_y);
 	stage_mark("blend_backward", s);
-	hipLaunchKernelGGL(blend_backward_kernel, dim3(4 * a.grid_x * a.grid_y), dim3(64), 0, s, a);
+	for (int at = 0; at < count; at += kMaxBlendBatch) {
+		BlendBatch batch;
+		batch.count = count - at < kMaxBlendBatch ? count - at : kMaxBlendBatch;
+		for (int k = 0; k < batch.count; k++)
+			batch.job[k] = jobs[at + k];
+		hipLaunchKernelGGL(blend_backward_kernel, dim3(strips * (unsigned)batch.count), dim3(64), 0, s, batch);
+	}
 }
 
 }  // namespace rgs

@@ -139,13 +139,16 @@ __device__ __forceinline__ void load_sh_row(const float* __restrict__ row, int d
 
 // ---- forward preprocess (K/cuda_rasterizer_hgs/forward.cu:155-258) -------------------------
 
-__global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs a)
+__global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<PreprocessArgs> batch)
 {
 	__shared__ uint32_t s_scan[8];
+	const PreprocessArgs& a = batch.job[blockIdx.y];  // one job per submodel of the frame
 	const int idx = blockIdx.x * 256 + threadIdx.x;
 	// the scratch of the depth sort that follows is cleared here, which saves a launch
 	for (size_t w = (size_t)idx; w < a.clear_words; w += (size_t)gridDim.x * 256)
 		a.clear[w] = 0u;
+	if ((int)blockIdx.x * 256 >= a.P)
+		return;  // the launch is sized for the job with the most Gaussians
 	uint32_t touched = 0;
 
 	if (idx < a.P) {
@@ -242,7 +245,8 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(PreprocessArgs 
 				rec[0] = float4{pix.x, pix.y, floor, p_hom.w};
 				rec[1] = conic_o;
 				rec[2] = float4{col.x, col.y, col.z, p_view.z};
-				rec[3] = float4{half.x, half.y, 0.f, 0.f};
+				// the third word is the integer radius (as bits): the key duplication reads the tile rectangle's inputs from here
+				rec[3] = float4{half.x, half.y, __int_as_float((int)my_radius), 0.f};
 			}
 			radius_out = (int)my_radius;
 			touched = ntiles;
@@ -329,8 +333,9 @@ __device__ __forceinline__ void sh_backward_channel(int deg, float x, float y, f
 
 constexpr int kBwdShMax = 48;  // SH gradient floats kept in registers until they are stored
 
-__global__ __launch_bounds__(128) void preprocess_backward_kernel(PreprocessBackwardArgs a)
+__global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<PreprocessBackwardArgs> batch)
 {
+	const PreprocessBackwardArgs& a = batch.job[blockIdx.y];
 	const uint32_t k_vis = blockIdx.x * 128 + threadIdx.x;
 	if (k_vis >= *a.visible_count)
 		return;
@@ -562,31 +567,51 @@ void launch_mark_visible(int P, const float* means, const float* view, uint8_t* 
 	hipLaunchKernelGGL(mark_visible_kernel, dim3((P + 255) / 256), dim3(256), 0, s, P, means, view, present);
 }
 
-void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s)
+void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_t s)
 {
 	stage_mark("preprocess_forward", s);
-	hipLaunchKernelGGL(preprocess_forward_kernel, dim3((a.P + 255) / 256), dim3(256), 0, s, a);
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<PreprocessArgs> b = {};
+		int max_p = 0;
+		for (int k = 0; k < nj; k++) {
+			b.job[k] = jobs[at + k];
+			max_p = b.job[k].P > max_p ? b.job[k].P : max_p;
+		}
+		hipLaunchKernelGGL(preprocess_forward_kernel, dim3((unsigned)((max_p + 255) / 256), (unsigned)nj), dim3(256), 0, s, b);
+	}
 }
 
-void launch_preprocess_backward(const PreprocessBackwardArgs& a, bool outputs_zeroed, hipStream_t s)
+void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, const int* outputs_zeroed, int count, hipStream_t s)
 {
-	if (!outputs_zeroed) {
-		stage_mark("clear_gradients", s);
-		const size_t n = (size_t)a.P;
-		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmean2D), 0u, 3 * n, s);
-		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dopacity), 0u, n, s);
-		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcolor), 0u, 3 * n, s);
-		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmeans), 0u, 3 * n, s);
-		launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcov3D), 0u, 6 * n, s);
-		if (a.shs)
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dsh), 0u, (size_t)a.M * 3 * n, s);
-		if (a.scales) {
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dscale), 0u, 3 * n, s);
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_drot), 0u, 4 * n, s);
+	for (int k = 0; k < count; k++)
+		if (!outputs_zeroed[k]) {
+			const PreprocessBackwardArgs& a = jobs[k];
+			stage_mark("clear_gradients", s);
+			const size_t n = (size_t)a.P;
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmean2D), 0u, 3 * n, s);
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dopacity), 0u, n, s);
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcolor), 0u, 3 * n, s);
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmeans), 0u, 3 * n, s);
+			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcov3D), 0u, 6 * n, s);
+			if (a.shs)
+				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dsh), 0u, (size_t)a.M * 3 * n, s);
+			if (a.scales) {
+				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dscale), 0u, 3 * n, s);
+				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_drot), 0u, 4 * n, s);
+			}
 		}
-	}
 	stage_mark("preprocess_backward", s);
-	hipLaunchKernelGGL(preprocess_backward_kernel, dim3((a.P + 127) / 128), dim3(128), 0, s, a);
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<PreprocessBackwardArgs> b = {};
+		int max_p = 0;
+		for (int k = 0; k < nj; k++) {
+			b.job[k] = jobs[at + k];
+			max_p = b.job[k].P > max_p ? b.job[k].P : max_p;
+		}
+		hipLaunchKernelGGL(preprocess_backward_kernel, dim3((unsigned)((max_p + 127) / 128), (unsigned)nj), dim3(128), 0, s, b);
+	}
 }
 
 }  // namespace rgs

@@ -7,6 +7,14 @@ namespace rgs {
 
 constexpr int kMaxComposite = 64;  // most partial images one composite call can take
 
+// Jobs of one launch: kernels that run once per submodel take the submodels of a frame together, the job in
+// blockIdx.y; the arguments travel by value.  More jobs than kMaxBatch take several launches.
+constexpr int kMaxBatch = 8;
+template <typename T>
+struct Batch {
+	T job[kMaxBatch];
+};
+
 struct PreprocessArgs {
 	int P, D, M;
 	const float* means;
@@ -90,11 +98,20 @@ struct BlendArgs {
 	float* out_depth;
 	float* out_alpha;
 	uint32_t* n_contrib;
-	uint32_t* strip_lists;  // 4 R words: for strip s of a tile whose list is [x, x + n), the entries the forward
-	                        // filed for it, at 4 x + s n: list position, bit 31 = strip inside the box
-	uint32_t* strip_filed;  // per 16x4 strip (tile * 4 + strip): how many of them, up to the last one blended
+	uint32_t* strip_lists;  // 4 R words: for strip s of a tile whose list is [x, x + n), the entries filed
+	                        // for it, at 4 x + s n: list position, bit 31 = strip inside the box
+	uint32_t* strip_total;  // per 16x4 strip (tile * 4 + strip): how many entries are filed for it; zero before the filing
+	uint32_t* strip_filed;  // per strip: how many of them the backward walks, i.e. up to the last one blended
+	const uint32_t* tile_keys;    // the sorted key of every list position: tile and strip bits (key_tile, key_strips)
+	const uint32_t* count_device; // non-null: the number of instances is min(capacity, *count_device)
+	uint32_t capacity;      // instances the launch is sized for
+	const uint4* file_tail; // per kFileBlock list positions: entries filed per strip for the tile of the last of them
+	const uint32_t* sort_status;   // status words of the two sorts (may be null): non-zero = the sort gave up
+	const uint32_t* order_status;
 	uint32_t* strip_order;  // strips by decreasing strip_filed, written behind the forward blend
-	uint32_t* strip_classes;  // 2 x 256 words, zero before the forward blend: strips per class of strip_filed, placement cursors
+	uint32_t* strip_order_forward;  // strips by decreasing strip_total, written ahead of the forward blend
+	uint32_t* strip_classes;  // 4 x 256 words, zero before the forward blend: strips per class and placement cursors,
+	                          // for strip_order and then for strip_order_forward
 	uint64_t* counters;  // non-null selects the work-accounting twin of the forward blend (7 sums)
 	// backward
 	const float* dL_dpix;
@@ -249,11 +266,29 @@ struct AdamArgs {
 	float one_minus_beta1, one_minus_beta2;   // formed in double by the host
 };
 
+// An instance's sort key: the tile in the low kKeyTileBits bits (all the sort looks at) and above them
+// what strip_filing.h decides for the four strips of that tile: bits 0-3 filed, bits 4-7 inside the box.
+constexpr int kKeyTileBits = 24;
+__host__ __device__ inline uint32_t key_tile(uint32_t key) { return key & ((1u << kKeyTileBits) - 1u); }
+__host__ __device__ inline uint32_t key_strips(uint32_t key) { return key >> kKeyTileBits; }
+constexpr int kFileBlock = 256;   // list positions per workgroup of the kernels that file entries for strips
+
+// What the key duplication needs to decide the strips: the packed records and the submodel box test's frame.
+struct FilingArgs {
+	const float4* record;      // 4 float4 per Gaussian: pixel centre, conic, ellipse extents and the integer radius among them
+	const float* projinv;
+	const float* range_low;
+	const float* range_up;
+	float tanfovx, tanfovy;
+	int W, H;
+};
+
 // preprocess.hip
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s);
-void launch_preprocess_forward(const PreprocessArgs& a, hipStream_t s);
-// With outputs_zeroed false the eight output arrays are cleared first.
-void launch_preprocess_backward(const PreprocessBackwardArgs& a, bool outputs_zeroed, hipStream_t s);
+// `jobs` are host arrays: the submodels of a frame in one launch (kMaxBatch of them at a time).
+void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_t s);
+// Where outputs_zeroed[k] is 0 the eight output arrays of job k are cleared first.
+void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, const int* outputs_zeroed, int count, hipStream_t s);
 
 // binning.hip
 constexpr int kSortItems = 16;                    // keys per thread in one sort block
@@ -263,25 +298,54 @@ size_t scan_temp_words(size_t n);                 // u32 words of scratch for la
 void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, const char* stage,
                           hipStream_t s);
 // Scans the per-256 block sums of the tile counts and of the visible flags in place;
-// *total_out = number of instances, *visible_count = number of Gaussians that touch a tile.
-void launch_totals_from_block_sums(uint32_t* block_sums, uint32_t* block_visible, int P, uint32_t* total_out,
-                                   uint32_t* visible_count, hipStream_t s);
+// *total_out (and *total_copy, if non-null) = number of instances, *visible_count = number of Gaussians that touch a tile.
+struct TotalsJob {
+	uint32_t* block_sums;
+	uint32_t* block_visible;
+	int P;
+	uint32_t* total_out;
+	uint32_t* total_copy;
+	uint32_t* visible_count;
+};
+void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t s);
 // Depth order of the Gaussians that touch a tile.  block_visible holds the exclusive scan of
 // their count per 256 Gaussians and *visible_count the total; sort_temp has been cleared
 // (sort_clear_words(P, 32) words).  On return order[0..count)
 // lists them by increasing depth, ties by index, and offsets_in_order is the inclusive scan of
 // their tile counts in that order; visible_list keeps them in index order.  The count stays on the device: every kernel is launched
 // for P elements and reads it.
-void launch_depth_order(int P, const float* depths, const uint32_t* tiles_touched, uint32_t* block_visible,
-                        uint32_t* visible_count, uint32_t* visible_list, uint32_t* keys_a, uint32_t* keys_b, uint32_t* order, uint32_t* vals_b,
-                        uint32_t* tiles_in_order, uint32_t* offsets_in_order, uint32_t* sort_temp, uint32_t* scan_temp,
-                        hipStream_t s);
+struct DepthOrderJob {
+	int P;
+	const float* depths;
+	const uint32_t* tiles_touched;
+	uint32_t* block_visible;
+	uint32_t* visible_count;
+	uint32_t* visible_list;
+	uint32_t* keys_a;
+	uint32_t* keys_b;
+	uint32_t* order;
+	uint32_t* vals_b;
+	uint32_t* tiles_in_order;
+	uint32_t* offsets_in_order;
+	uint32_t* sort_temp;
+	uint32_t* scan_temp;
+};
+void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 // Also sets clear[0..clear_words) to zero (the scratch of the sort that follows).  Instances whose
 // position is `capacity` or more are not written.
-void launch_duplicate_with_keys(int P, const uint32_t* visible_count, const uint32_t* order,
-                                const uint32_t* offsets_in_order, const float2* xy, const int* radii, int grid_x,
-                                int grid_y, uint32_t* keys, uint32_t* values, uint32_t capacity, uint32_t* clear,
-                                size_t clear_words, hipStream_t s);
+struct DuplicateJob {
+	int P;
+	const uint32_t* visible_count;
+	const uint32_t* order;
+	const uint32_t* offsets;   // inclusive, in depth order
+	FilingArgs filing;
+	uint32_t* keys;
+	uint32_t* values;
+	uint32_t capacity;
+	uint32_t* clear;
+	size_t clear_words;
+};
+void launch_duplicate_with_keys(const DuplicateJob* jobs, int count, int grid_x, int grid_y, hipStream_t s);
 size_t sort_clear_words(size_t n, int end_bit);    // words of the sort scratch that must be zero before a sort
 constexpr int kSortMaxPasses = 8;                 // radix passes the scratch has room for (64-bit keys)
 constexpr uint32_t kSortHeader = 2112;            // words ahead of the look-back words: histograms, counters, status
@@ -295,33 +359,59 @@ size_t sort_temp_words(size_t n);                 // u32 words of scratch for la
 // keys_out/vals_out, an even one in keys_in/vals_in.
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s);
-// The same for 32-bit keys; with a null `stage` its kernels are not marked for the timing aid.
-// With a non-null n_device the number of pairs is min(n, *n_device), read by the kernels, and `n` is only
-// its upper bound (grids and scratch are sized for it).
-// temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of temp already.
-// also_clear: an array the first kernel sets to zero on the way (for a later stage), or null.
-void launch_sort_pairs_u32(uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
-                           const uint32_t* n_device, int end_bit, uint32_t* temp, bool temp_cleared, uint32_t* also_clear,
-                           size_t also_clear_words, const char* stage, hipStream_t s);
+// One sort of a batch.  With a non-null n_device the number of pairs is min(n, *n_device), read by the kernels, and
+// `n` is only its upper bound (grids and scratch are sized for it).  also_clear: an array the first kernel sets to
+// zero on the way (for a later stage), or null.
+template <typename KeyT>
+struct SortJob {
+	KeyT* keys_in;
+	KeyT* keys_out;
+	uint32_t* vals_in;
+	uint32_t* vals_out;
+	size_t n;
+	const uint32_t* n_device;
+	uint32_t* temp;
+	uint32_t* also_clear;
+	size_t also_clear_words;
+};
+// The same for 32-bit keys, every job in one launch per kernel; with a null `stage` its kernels are not marked for
+// the timing aid.  temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of every temp already.
+void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, const char* stage,
+                           hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
 // Polls a look-back allows before it gives up (0 restores the default; negative: give up at once,
 // which is how a test exercises the give-up path with every kernel still running to its end).
 void set_lookback_spin_limit(int polls);
 // Sets *fault (host memory the device can write; null: nothing is launched) if the sort that used `temp` gave up.
 void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_t s);
-// Either status word (may be null) being non-zero leaves every range empty.  Clears `ranges` and
-// the kRangeTailWords words behind it (the strip class counters of the blend).
-constexpr int kRangeTailWords = 512;
-// ranges_cleared: an earlier kernel has done that clearing.
-// With a non-null n_device the number of keys is min(n, *n_device) and the launch is sized for n.
-// A non-zero status also sets *fault (host memory the device can write, may be null).
-void launch_tile_ranges(const uint32_t* keys, size_t n, const uint32_t* n_device, uint2* ranges, int tiles,
-                        const uint32_t* sort_status, const uint32_t* order_status, uint32_t* fault, bool ranges_cleared,
-                        hipStream_t s);
+// The tile ranges from the sorted keys.  Either status word (may be null) being non-zero leaves every range empty
+// and sets *fault (host memory the device can write, may be null).  The caller has cleared `ranges`.  With a non-null
+// n_device the number of keys is min(n, *n_device) and the launch is sized for n.  file_tail (may be null)
+// receives, per kFileBlock keys, how many entries of the tile of the last of them have each strip bit set.
+constexpr int kRangeTailWords = 1024;   // words behind the ranges: the strip class counters of the blend
+struct TileRangesJob {
+	const uint32_t* keys;
+	size_t n;
+	const uint32_t* n_device;
+	uint2* ranges;
+	const uint32_t* sort_status;
+	const uint32_t* order_status;
+	uint32_t* fault;
+	uint4* file_tail;
+};
+void launch_tile_ranges(const TileRangesJob* jobs, int count, hipStream_t s);
 
 // blend.hip
-void launch_blend_forward(const BlendArgs& a, hipStream_t s);
-void launch_blend_backward(const BlendArgs& a, hipStream_t s);
+constexpr int kMaxBlendBatch = 8;   // jobs one launch of a blend kernel can take (their arguments travel by value)
+struct BlendBatch {
+	BlendArgs job[kMaxBlendBatch];
+	int count;
+};
+void launch_strip_filing(const BlendArgs* jobs, int count, hipStream_t s);   // the per-strip lists, from the sorted keys' strip bits
+// `jobs` (host array) share one image size; more than kMaxBlendBatch take several launches.
+void launch_blend_forward(const BlendArgs* jobs, int count, hipStream_t s);
+void launch_blend_backward(const BlendArgs* jobs, int count, hipStream_t s);
+void launch_blend_count(const BlendArgs& a, hipStream_t s);    // the work-accounting twin of the forward (a.counters)
 
 // composite.hip
 void launch_composite_forward(const CompositeArgs& a, hipStream_t s);

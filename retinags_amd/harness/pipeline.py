@@ -13,7 +13,7 @@ from typing import Dict, List, Optional
 import numpy as np
 import torch
 
-from ..rasterizer import GaussianRasterizationSettings, GaussianRasterizer
+from ..rasterizer import GaussianRasterizationSettings, GaussianRasterizer, rasterize_frame
 from ..compositor import blender_render_result
 from .partition import Partition, partition_scene, relation_vector
 from .scenes import Camera
@@ -137,12 +137,13 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
 
 
 def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0, debug: bool = False,
-                   instance_bound: Optional[int] = None):
+                   instance_bound: Optional[int] = None, clear_gradients: bool = False):
     """Enqueues the geometry stage of a submodel's forward on the current stream without waiting
     for its instance count; hand the result to render_submodel(..., started=...)."""
     rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug))
     geometry = rasterizer.enqueue_geometry(means3D=sub.means3D, opacities=sub.opacity, shs=sub.shs,
-                                           scales=sub.scales, rotations=sub.rotations, instance_bound=instance_bound)
+                                           scales=sub.scales, rotations=sub.rotations, instance_bound=instance_bound,
+                                           clear_gradients=clear_gradients)
     return rasterizer, geometry
 
 
@@ -179,7 +180,7 @@ def _host_pool(n: int):
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
                  submodel_bg: Optional[torch.Tensor] = None,
                  streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = False,
-                 instance_bounds: Optional[Dict[int, int]] = None) -> dict:
+                 instance_bounds: Optional[Dict[int, int]] = None, together: bool = False) -> dict:
     """Render every related submodel (black background, as the trainer does:
     trainer4tree_partition.py:397) and composite the partial images in BVH order.
 
@@ -194,6 +195,10 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     own (ctypes releases the interpreter lock inside the library); measured no faster, and less
     steady, than the two rounds: the threads contend for the interpreter between the calls.
 
+    together: the related submodels go through rasterize_frame: three library calls per frame, which blend all
+    submodels in one launch per direction (the stages that run once per submodel are queued on `streams`, if
+    given, beside each other); same results.
+
     instance_bounds (submodel id -> room for that many instances; with or without `streams`): the
     forward of each submodel is issued in one go, without waiting for its instance count.  The
     stages come back under "stages"; call check_instance_bounds(frame) before using the frame's
@@ -204,7 +209,28 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
         submodel_bg = torch.zeros(3, device=device)
     related = [m for m in range(len(subs)) if relation[m] >= 0]
     stages = {}
-    if instance_bounds is not None:
+    if together:
+        if instance_bounds is not None or host_threads:
+            raise ValueError("together=True takes neither instance_bounds nor host_threads")
+        main = torch.cuda.current_stream(device)
+        lanes = streams if streams else [main]
+        rasterizers, inputs = [], []
+        for m in related:
+            sub = subs[m]
+            means2D = sub.means2D
+            if means2D is None:
+                means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
+            rasterizers.append(GaussianRasterizer(raster_settings=raster_settings(cam, sub, submodel_bg)))
+            inputs.append(dict(means3D=sub.means3D, means2D=means2D, shs=sub.shs, opacities=sub.opacity, scales=sub.scales,
+                               rotations=sub.rotations))
+        outs = rasterize_frame(rasterizers, inputs,
+                               streams=[lanes[k % len(lanes)].cuda_stream for k in range(len(related))] if streams else None)
+        partial = {}
+        for k, m in enumerate(related):
+            color, radii, depth, alpha = outs[k]
+            partial[m] = {"render": color, "viewspace_points": inputs[k]["means2D"], "visibility_filter": radii > 0,
+                          "radii": radii, "depth": depth, "alpha": alpha, "num_rendered": -1}
+    elif instance_bounds is not None:
         main = torch.cuda.current_stream(device)
         lanes = streams if streams else [main]
         for side in lanes[:len(related)]:

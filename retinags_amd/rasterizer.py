@@ -83,7 +83,7 @@ class GeometryStage:
     GaussianRasterizer.enqueue_geometry, consumed once by GaussianRasterizer.forward."""
 
     __slots__ = ("device", "stream", "P", "H", "W", "tensors", "settings", "radii", "geomBuffer", "geom_bytes",
-                 "count", "event", "source", "used", "instance_bound", "_instances")
+                 "count", "event", "source", "used", "instance_bound", "_instances", "cleared")
 
     def matches(self, means3D, raster_settings) -> bool:
         return (self.source == (means3D.data_ptr(), int(means3D.shape[0])) and self.settings is raster_settings
@@ -145,6 +145,7 @@ def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations,
     st.count = None
     st.instance_bound = None
     st._instances = None
+    st.cleared = None
     byte = dict(dtype=torch.uint8, device=device)
     st.radii = torch.empty((st.P,), dtype=torch.int32, device=device)
     names = ("means3D", "colors_precomp", "opacities", "scales", "rotations", "cov3Ds_precomp", "sh", "bg",
@@ -437,6 +438,220 @@ class _RasterizeGaussians(torch.autograd.Function):
         return grads
 
 
+class _RasterizeFrame(torch.autograd.Function):
+    """The submodels that a camera sees ("layers"), rasterized together: what the reference does with one
+    _RasterizeGaussians call per submodel (gather_RenderResult_pool,
+    parallel_utils/basic_parallel_trainer/result_aggregator.py:22-38), as three library calls per frame
+    (every layer's geometry stage, then binning and one blend launch for all, and for the backward one
+    blend launch for all and every layer's per-Gaussian backward).
+
+    apply(settings, streams, *flat): `settings` a tuple of K GaussianRasterizationSettings (same camera and
+    image size), `streams` None or a tuple of K HIP stream handles (a layer's own stream, on which the
+    stages that run once per layer are queued, beside the other layers'), flat = for every layer
+    (means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp).
+    Returns for every layer (color, radii, depth, alpha)."""
+
+    FIELDS = 8
+
+    @staticmethod
+    def forward(ctx, settings, streams, *flat):
+        K = len(settings)
+        if K == 0 or len(flat) != _RasterizeFrame.FIELDS * K:
+            raise RuntimeError("rasterize_frame: one group of eight tensors per layer is needed")
+        if K > _capi.MAX_FRAME_LAYERS:
+            raise RuntimeError(f"rasterize_frame: at most {_capi.MAX_FRAME_LAYERS} layers")
+        rs0 = settings[0]
+        H, W = int(rs0.image_height), int(rs0.image_width)
+        device = flat[0].device
+        if not flat[0].is_cuda:
+            raise RuntimeError("the rasterizer needs its inputs on a GPU (device memory)")
+        f32 = dict(dtype=torch.float32, device=device)
+        byte = dict(dtype=torch.uint8, device=device)
+        main = torch.cuda.current_stream(device).cuda_stream
+        debug = int(bool(rs0.debug))
+        view_t = {n: _dev_f32(v, device, n) for n, v in (("viewmatrix", rs0.viewmatrix), ("projmatrix", rs0.projmatrix),
+                                                          ("projmatrix_inv", rs0.projmatrix_inv), ("campos", rs0.campos))}
+        view = _capi.FrameView(W, H, float(rs0.tanfovx), float(rs0.tanfovy), ptr(view_t["viewmatrix"]),
+                               ptr(view_t["projmatrix"]), ptr(view_t["projmatrix_inv"]), ptr(view_t["campos"]))
+        arr = (_capi.FrameLayer * K)()
+        records, live = [], []
+        with torch.cuda.device(device):
+            image_bytes = lib.rgs_image_bytes(W, H)
+            for k, rs in enumerate(settings):
+                means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds = flat[8 * k:8 * k + 8]
+                if int(rs.image_height) != H or int(rs.image_width) != W:
+                    raise RuntimeError("rasterize_frame: the layers of a frame share one image size")
+                if means3D.ndim != 2 or means3D.shape[1] != 3:
+                    raise RuntimeError("means3D must have dimensions (num_points, 3)")
+                P = int(means3D.shape[0])
+                M = int(sh.shape[1]) if sh.numel() != 0 else 0
+                package = torch.empty((5, H, W), **f32)
+                t = {n: _dev_f32(v, device, n) for n, v in (
+                    ("means3D", means3D), ("sh", sh), ("colors_precomp", colors_precomp), ("opacities", opacities),
+                    ("scales", scales), ("rotations", rotations), ("cov3Ds_precomp", cov3Ds), ("bg", rs.bg),
+                    ("range_low", rs.range_low), ("range_up", rs.range_up))}
+                rec = dict(P=P, M=M, t=t, package=package, radii=torch.empty((P,), dtype=torch.int32, device=device),
+                           rendered=0, geom=torch.empty(0, **byte), binning=torch.empty(0, **byte), img=torch.empty(0, **byte),
+                           cleared=None)
+                records.append(rec)
+                if P == 0:
+                    package.zero_()
+                    continue
+                needs = ctx.needs_input_grad[2 + 8 * k:2 + 8 * (k + 1)]
+                L = arr[len(live)]
+                live.append(k)
+                L.P, L.D, L.M = P, int(rs.sh_degree), M
+                L.means3D, L.shs, L.colors_precomp, L.opacities = ptr(t["means3D"]), ptr(t["sh"]), ptr(t["colors_precomp"]), ptr(t["opacities"])
+                L.scales, L.rotations, L.cov3D_precomp = ptr(t["scales"]), ptr(t["rotations"]), ptr(t["cov3Ds_precomp"])
+                L.scale_modifier = float(rs.scale_modifier)
+                L.background, L.range_low, L.range_up = ptr(t["bg"]), ptr(t["range_low"]), ptr(t["range_up"])
+                L.radii = ptr(rec["radii"])
+                geom_bytes = lib.rgs_geom_bytes(P)
+                rec["geom"] = torch.empty(geom_bytes, **byte)
+                rec["img"] = torch.empty(image_bytes, **byte)
+                L.geom_ws, L.image_ws = ptr(rec["geom"]), ptr(rec["img"])
+                L.geom_bytes, L.image_bytes = geom_bytes, image_bytes
+                L.out_color, L.out_depth, L.out_alpha = ptr(package[0:3]), ptr(package[3:4]), ptr(package[4:5])
+                L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
+                if any(needs):
+                    # Only rendered Gaussians get their gradient rows written; the library clears the rest behind
+                    # the layer's geometry stage, where that pure memory traffic runs beside the other layers' short kernels.
+                    cleared = _gradient_outputs(P, M, scales.numel() != 0, device, torch.empty)
+                    rec["cleared"] = cleared
+                    base = cleared["means2D"]
+                    span = cleared["rotations"].data_ptr() + cleared["rotations"].numel() * 4 - base.data_ptr()
+                    L.clear[0], L.clear_bytes[0] = base.data_ptr(), span
+                    L.clear[1], L.clear_bytes[1] = cleared["sums"].data_ptr(), cleared["sums"].numel() * 4
+            if live:
+                counts = _frame_counts(device, len(live))
+                check(lib.rgs_frame_forward_geom(len(live), arr, C.byref(view), C.c_void_p(counts.data_ptr()), C.c_void_p(main), debug))
+                got = counts[:len(live)].tolist()
+                for j, k in enumerate(live):
+                    rec = records[k]
+                    rec["rendered"] = int(got[j])
+                    binning_bytes = lib.rgs_binning_bytes(rec["rendered"]) if rec["rendered"] > 0 else 0
+                    rec["binning"] = torch.empty(binning_bytes, **byte)
+                    arr[j].R = rec["rendered"]
+                    arr[j].binning_ws, arr[j].binning_bytes = ptr(rec["binning"]), binning_bytes
+                check(lib.rgs_frame_forward_raster(len(live), arr, C.byref(view), C.c_void_p(main), debug))
+        ctx.settings = settings
+        ctx.streams = streams
+        ctx.meta = []
+        saved, outs = [], []
+        for k, rec in enumerate(records):
+            t = rec["t"]
+            ctx.meta.append(dict(rendered=rec["rendered"], cleared=rec["cleared"]))
+            saved += [t["colors_precomp"], t["means3D"], t["scales"], t["rotations"], t["cov3Ds_precomp"], rec["radii"], t["sh"],
+                      rec["geom"], rec["binning"], rec["img"], rec["package"][4:5]]
+            outs += [rec["package"][0:3], rec["radii"], rec["package"][3:4], rec["package"][4:5]]
+        ctx.save_for_backward(*saved)
+        ctx.mark_non_differentiable(*[outs[4 * k + 1] for k in range(K)])
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        settings, streams = ctx.settings, ctx.streams
+        K = len(settings)
+        saved = ctx.saved_tensors
+        rs0 = settings[0]
+        H, W = int(rs0.image_height), int(rs0.image_width)
+        device = saved[1].device
+        main = torch.cuda.current_stream(device).cuda_stream
+        arr = (_capi.FrameLayer * K)()
+        keep, results, live = [], [], 0
+        view = None
+        for k in range(K):
+            (colors_precomp, means3D, scales, rotations, cov3Ds, radii, sh, geomBuffer, binningBuffer, imgBuffer,
+             alpha) = saved[11 * k:11 * (k + 1)]
+            rs, meta = settings[k], ctx.meta[k]
+            g_color, _, g_depth, g_alpha = grads[4 * k:4 * (k + 1)]
+            P = int(means3D.shape[0])
+            M = int(sh.shape[1]) if sh.numel() != 0 else 0
+            f32 = dict(dtype=torch.float32, device=device)
+            if P == 0:
+                z = lambda *shape: torch.zeros(shape, **f32)
+                results.append((z(0, 3), z(0, 3), z(0, 1), z(0, 3), z(0, 6), z(0, M, 3), z(0, 3), z(0, 4)))
+                continue
+            if g_color is None:
+                g_color = torch.zeros((3, H, W), **f32)
+            has_scales = scales.numel() != 0
+            out = meta["cleared"] if meta["cleared"] is not None else _gradient_outputs(P, M, has_scales, device, torch.empty)
+            t = dict(bg=_dev_f32(rs.bg, device, "bg"), low=_dev_f32(rs.range_low, device, "range_low"),
+                     up=_dev_f32(rs.range_up, device, "range_up"), g_color=_dev_f32(g_color, device, "grad_color"),
+                     g_depth=None if g_depth is None else _dev_f32(g_depth, device, "grad_depth"),
+                     g_alpha=None if g_alpha is None else _dev_f32(g_alpha, device, "grad_alpha"))
+            keep.append(t)
+            if view is None:
+                vt = dict(v=_dev_f32(rs.viewmatrix, device, "viewmatrix"), p=_dev_f32(rs.projmatrix, device, "projmatrix"),
+                          pi=_dev_f32(rs.projmatrix_inv, device, "projmatrix_inv"), c=_dev_f32(rs.campos, device, "campos"))
+                keep.append(vt)
+                view = _capi.FrameView(W, H, float(rs.tanfovx), float(rs.tanfovy), ptr(vt["v"]), ptr(vt["p"]), ptr(vt["pi"]),
+                                       ptr(vt["c"]))
+            L = arr[live]
+            live += 1
+            L.P, L.D, L.M, L.R = P, int(rs.sh_degree), M, int(meta["rendered"])
+            L.means3D, L.shs, L.colors_precomp = ptr(means3D), ptr(sh), ptr(colors_precomp)
+            L.scales, L.rotations, L.cov3D_precomp = ptr(scales), ptr(rotations), ptr(cov3Ds)
+            L.scale_modifier = float(rs.scale_modifier)
+            L.background, L.range_low, L.range_up = ptr(t["bg"]), ptr(t["low"]), ptr(t["up"])
+            L.radii = ptr(radii)
+            L.geom_ws, L.binning_ws, L.image_ws = ptr(geomBuffer), ptr(binningBuffer), ptr(imgBuffer)
+            L.out_alpha = ptr(alpha)
+            L.dL_dpix, L.dL_dpix_depth, L.dL_dalphas = ptr(t["g_color"]), ptr(t["g_depth"]), ptr(t["g_alpha"])
+            L.grad_accum = ptr(out["sums"])
+            L.dL_dmean2D, L.dL_dopacity, L.dL_dcolor = ptr(out["means2D"]), ptr(out["opacity"]), ptr(out["colors"])
+            L.dL_dmean3D, L.dL_dcov3D, L.dL_dsh = ptr(out["means3D"]), ptr(out["cov3D"]), ptr(out["sh"])
+            L.dL_dscale = ptr(out["scales"]) if has_scales else C.c_void_p(0)
+            L.dL_drot = ptr(out["rotations"]) if has_scales else C.c_void_p(0)
+            L.outputs_zeroed = int(meta["cleared"] is not None)
+            L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
+            results.append((out["means2D"], out["colors"], out["opacity"], out["means3D"], out["cov3D"], out["sh"],
+                            out["scales"], out["rotations"]))
+        if live:
+            with torch.cuda.device(device):
+                check(lib.rgs_frame_backward(live, arr, C.byref(view), C.c_void_p(main), int(bool(rs0.debug))))
+        ctx.meta = None
+        flat = []
+        for k in range(K):
+            (colors_precomp, means3D, scales, rotations, cov3Ds, radii, sh) = saved[11 * k:11 * k + 7]
+            g_means2D, g_colors, g_opacity, g_means3D, g_cov3D, g_sh, g_scales, g_rot = results[k]
+            flat += [g_means3D, g_means2D, g_sh if sh.numel() else None, g_colors if colors_precomp.numel() else None,
+                     g_opacity, g_scales if scales.numel() else None, g_rot if rotations.numel() else None,
+                     g_cov3D if cov3Ds.numel() else None]
+        return (None, None, *flat)
+
+
+_frame_count_words = threading.local()
+
+
+def _frame_counts(device: torch.device, n: int) -> torch.Tensor:
+    """Pinned words for the layers' instance counts, per host thread and device; read before the call returns."""
+    words = _frame_count_words.__dict__.setdefault("words", {})
+    key = (device.type, device.index)
+    t = words.get(key)
+    if t is None or t.numel() < n:
+        t = torch.zeros(max(n, _capi.MAX_FRAME_LAYERS), dtype=torch.int32).pin_memory()
+        words[key] = t
+    return t
+
+
+def rasterize_frame(rasterizers, inputs, streams=None):
+    """All layers of a frame through one call.  `rasterizers`: K GaussianRasterizer (their settings share the
+    camera and the image size); `inputs`: K dicts with the keyword arguments of GaussianRasterizer.forward
+    (means3D, means2D, opacities, shs / colors_precomp, scales + rotations / cov3D_precomp); `streams`: None,
+    or for every layer the handle of a HIP stream on which the stages that run once per layer are queued (the
+    caller's stream waits for them).  Returns K tuples (color, radii, depth, alpha), the results of K
+    forward calls, and differentiates like them."""
+    flat = []
+    for rz, kw in zip(rasterizers, inputs):
+        shs, colors_precomp, scales, rotations, cov3D = GaussianRasterizer._check_and_fill(
+            kw.get("shs"), kw.get("colors_precomp"), kw.get("scales"), kw.get("rotations"), kw.get("cov3D_precomp"))
+        flat += [kw["means3D"], kw["means2D"], shs, colors_precomp, kw["opacities"], scales, rotations, cov3D]
+    outs = _RasterizeFrame.apply(tuple(rz.raster_settings for rz in rasterizers),
+                                 None if streams is None else tuple(streams), *flat)
+    return [tuple(outs[4 * k:4 * k + 4]) for k in range(len(rasterizers))]
+
+
 class GaussianRasterizer(nn.Module):
     """K/diff_gaussian_rasterization_half_gaussian/__init__.py:183-232."""
 
@@ -483,7 +698,7 @@ class GaussianRasterizer(nn.Module):
                                    raster_settings, geometry)
 
     def enqueue_geometry(self, means3D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
-                         cov3D_precomp=None, instance_bound=None) -> GeometryStage:
+                         cov3D_precomp=None, instance_bound=None, clear_gradients=False) -> GeometryStage:
         """Starts the first half of a forward call (preprocess and instance count) on the current
         stream and returns without waiting for it.  No counterpart in the reference, whose forward
         always blocks on the count (K/cuda_rasterizer_hgs/rasterizer_impl.cu:287): a caller that
@@ -495,7 +710,12 @@ class GaussianRasterizer(nn.Module):
         does not wait for the count at all (the reference grows its buffers on demand instead,
         K/rasterize_points.cu:27-33).  The caller must then ask stage.within_bound() after the
         forward has been issued (at the end of the iteration is early enough) and, if it is
-        false, repeat the forward with a bound of at least stage.instances()."""
+        false, repeat the forward with a bound of at least stage.instances().
+
+        clear_gradients: also allocates and clears, on this stream and right away, the gradient tensors the
+        backward of this call will fill (only rendered Gaussians get rows written; the rest must be zero):
+        pure memory traffic that then runs beside the other layers' short kernels instead of behind the
+        blend.  Used by rasterize_frame; a plain forward(..., geometry=stage) clears its own."""
         rs = self.raster_settings
         shs, colors_precomp, scales, rotations, cov3D_precomp = self._check_and_fill(
             shs, colors_precomp, scales, rotations, cov3D_precomp)
@@ -505,6 +725,9 @@ class GaussianRasterizer(nn.Module):
                 rs.viewmatrix, rs.projmatrix, rs.projmatrix_inv, rs.range_low, rs.range_up, rs.tanfovx, rs.tanfovy,
                 rs.image_height, rs.image_width, shs, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, wait=False)
         stage.settings = rs
+        if clear_gradients and stage.P > 0:
+            M = int(shs.shape[1]) if shs.numel() != 0 else 0
+            stage.cleared = _gradient_outputs(stage.P, M, scales.numel() != 0, means3D.device, torch.zeros)
         if instance_bound is not None:
             if int(instance_bound) < 0:
                 raise ValueError("instance_bound must not be negative")

@@ -67,7 +67,7 @@ def check_binning_against(st, geom, binning, P, R, W, H):
     if R == 0:
         return
     b = _capi.binning_layout(R, W, H)
-    tiles = view_ws(binning, b["keys_sorted"], R, np.uint32)
+    tiles = view_ws(binning, b["keys_sorted"], R, np.uint32) & np.uint32(0xFFFFFF)   # strip bits ride above the tile
     vals = view_ws(binning, b["values_sorted"], R, np.uint32)
     assert np.array_equal(vals, st.point_list)
     assert np.array_equal((tiles.astype(np.uint64) << np.uint64(32)) | depth_bits[vals].astype(np.uint64), st.keys)

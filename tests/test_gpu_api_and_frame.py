@@ -408,3 +408,61 @@ def test_a_sort_that_gives_up_is_reported_by_the_next_call():
     torch.cuda.synchronize()
     assert torch.equal(again, good)
     assert _capi.lib.rgs_sort_fault(stream) == 0
+
+
+@pytest.mark.parametrize("with_streams", [False, True])
+def test_frame_rendered_together_matches_one_call_per_submodel(with_streams):
+    """render_frame(together=True) sends the related submodels through rgs_frame_forward_raster /
+    rgs_frame_backward (one blend launch per direction for all of them): images bit for bit those of one
+    call per submodel, gradients equal up to the order of the atomic sums."""
+    from retinags_amd.harness import partition, pipeline
+    scene, cam, _ = scenes.make_config("C1", shrink=300, resolution_scale=0.25)
+    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    rel = partition.relation_vector(part, cam)
+    H, W = cam.image_height, cam.image_width
+    g = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(2)) * 1e-2).to(DEV)
+    bg = torch.tensor([0.3, 0.1, 0.2], device=DEV)
+    results = []
+    for together in (False, True):
+        subs = [s.requires_grad_(True) for s in pipeline.submodels_from_partition(scene, part, DEV)]
+        for s in subs:
+            s.means2D = torch.zeros_like(s.means3D, requires_grad=True)
+        streams = ([torch.cuda.current_stream()] + [torch.cuda.Stream() for _ in range(2)]) if with_streams else None
+        out = pipeline.render_frame(cam.to(DEV), subs, rel, bg, streams=streams, together=together)
+        torch.autograd.backward([out["render"]], [g])
+        torch.cuda.synchronize()
+        results.append((out, subs))
+    (a, subs_a), (b, subs_b) = results
+    for key in ("render", "depth", "alpha"):
+        assert torch.equal(a[key], b[key]), key
+    for m in a["partial"]:
+        for key in ("render", "depth", "alpha", "radii"):
+            assert torch.equal(a["partial"][m][key], b["partial"][m][key]), (m, key)
+    for sa, sb in zip(subs_a, subs_b):
+        for ta, tb in zip(sa.parameters() + [sa.means2D], sb.parameters() + [sb.means2D]):
+            assert (ta.grad is None) == (tb.grad is None)
+            if ta.grad is not None:
+                assert rel_l2(ta.grad.cpu().numpy(), tb.grad.cpu().numpy()) <= 1e-5
+
+
+def test_rasterize_frame_with_an_empty_layer_and_without_stages():
+    """rasterize_frame called directly, one layer of which has no Gaussians."""
+    from retinags_amd import GaussianRasterizer
+    from retinags_amd.rasterizer import rasterize_frame
+    scene, cam, low, up = _small_inputs(n=2000)
+    s = oracle_settings(cam, low, up, torch.tensor([0.2, 0.4, 0.6]))
+    settings = _settings(s)
+    full = dict(means3D=scene["xyz"].to(DEV).requires_grad_(True), means2D=torch.zeros(scene["xyz"].shape[0], 3, device=DEV),
+                opacities=scene["opacity"].to(DEV), shs=scene["shs"].to(DEV), scales=scene["scales"].to(DEV),
+                rotations=scene["rotations"].to(DEV))
+    empty = dict(means3D=torch.zeros(0, 3, device=DEV, requires_grad=True), means2D=torch.zeros(0, 3, device=DEV),
+                 opacities=torch.zeros(0, 1, device=DEV), shs=torch.zeros(0, 16, 3, device=DEV),
+                 scales=torch.zeros(0, 3, device=DEV), rotations=torch.zeros(0, 4, device=DEV))
+    rz = GaussianRasterizer(settings)
+    (c0, r0, d0, a0), (c1, r1, d1, a1) = rasterize_frame([rz, rz], [full, empty])
+    want = rz(**{k: (v.detach() if k == "means3D" else v) for k, v in full.items()})
+    assert torch.equal(c0, want[0]) and torch.equal(r0, want[1]) and torch.equal(d0, want[2]) and torch.equal(a0, want[3])
+    assert r1.numel() == 0 and float(c1.abs().max()) == 0.0 and float(a1.abs().max()) == 0.0
+    (c0.sum() + c1.sum()).backward()
+    assert full["means3D"].grad is not None and float(full["means3D"].grad.abs().sum()) > 0
+    assert empty["means3D"].grad is not None and empty["means3D"].grad.shape == (0, 3)

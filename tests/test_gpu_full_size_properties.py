@@ -47,7 +47,7 @@ def _check_binning_structure(outs, P, W, H):
     b = _capi.binning_layout(Rn, W, H)
     vals = view_ws(binning, b["values_sorted"], Rn, np.uint32)
     # the reference's 64-bit keys, rebuilt: the tile the sort used and the Gaussian's depth bits
-    keys = (view_ws(binning, b["keys_sorted"], Rn, np.uint32).astype(np.uint64) << np.uint64(32)) | \
+    keys = ((view_ws(binning, b["keys_sorted"], Rn, np.uint32) & np.uint32(0xFFFFFF)).astype(np.uint64) << np.uint64(32)) | \
         depth_bits[vals].astype(np.uint64)
     assert (np.diff(keys.astype(np.uint64).view(np.int64)) >= 0).all()          # sorted (keys < 2^63)
     same = keys[1:] == keys[:-1]
