@@ -262,11 +262,11 @@ typedef struct rgs_frame_layer {
 	float* dL_dscale;
 	float* dL_drot;
 	int outputs_zeroed;
-	void* clear[2];            /* rgs_frame_forward_raster: up to two device buffers (NULL: none) that it sets to zero (sizes */
-	size_t clear_bytes[2];     /* multiples of 4 bytes): the gradient tensors, cleared beside the blend on the layer's own stream */
-	void* stream;              /* the layer's own HIP stream, or NULL for the frame's: its geometry stage was enqueued
-	                              there, and the stages that run once per layer (binning; per-Gaussian backward) follow
-	                              on it, beside the other layers'; the frame's stream waits for them and is waited for */
+	void* grad_block;          /* with outputs_zeroed = 0: NULL, or one block of grad_block_bytes (a multiple of 4) that holds the */
+	size_t grad_block_bytes;   /* eight gradient arrays and nothing that must survive: cleared in one go instead of array by array */
+	void* stream;              /* NULL, or a second HIP stream for the backward: work that is bound by memory bandwidth (clearing
+	                              the gradient arrays, the per-Gaussian backward of the layers whose blend is done) then runs on it
+	                              beside the blend, which is bound by instruction issue; the frame's stream waits for it */
 } rgs_frame_layer;
 /* rgs_forward_geom for every layer (P > 0 each): every geometry stage is queued (on the layer's stream) before
  * the host waits for the first instance count; returns when all counts have arrived in counts_pinned[0..K)
@@ -276,7 +276,9 @@ int rgs_frame_forward_geom(int K, const rgs_frame_layer* layers, const rgs_frame
 /* rgs_forward_raster for every layer (P > 0 each): per layer the key duplication, sort, ranges and strip
  * lists, then one blend launch for all.  `layers` and `view` are HOST structures. */
 int rgs_frame_forward_raster(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug);
-/* rgs_backward for every layer: one blend-backward launch for all, then each layer's per-Gaussian backward. */
+/* rgs_backward for every layer: the blend backward of all layers in one launch (two, one behind the other, when a
+ * layer names a second stream, so that the first half's per-Gaussian backward runs beside the second half's blend),
+ * then each layer's per-Gaussian backward. */
 int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug);
 
 /* ---- measurement aids (no counterpart in the reference, which times whole iterations

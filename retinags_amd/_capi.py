@@ -61,7 +61,7 @@ class FrameLayer(C.Structure):
                 ("grad_accum", C.c_void_p), ("dL_dmean2D", C.c_void_p), ("dL_dopacity", C.c_void_p),
                 ("dL_dcolor", C.c_void_p), ("dL_dmean3D", C.c_void_p), ("dL_dcov3D", C.c_void_p), ("dL_dsh", C.c_void_p),
                 ("dL_dscale", C.c_void_p), ("dL_drot", C.c_void_p), ("outputs_zeroed", C.c_int),
-                ("clear", C.c_void_p * 2), ("clear_bytes", C.c_size_t * 2), ("stream", C.c_void_p)]
+                ("grad_block", C.c_void_p), ("grad_block_bytes", C.c_size_t), ("stream", C.c_void_p)]
 
 
 class RgsError(RuntimeError):

@@ -992,31 +992,8 @@ int rgs_frame_forward_raster(int K, const rgs_frame_layer* layers, const rgs_fra
 		jobs[(size_t)k].out_depth = layers[k].out_depth;
 		jobs[(size_t)k].out_alpha = layers[k].out_alpha;
 	}
-	// Clearing the gradient buffers is pure memory traffic and the blend is bound by instruction issue: on a
-	// layer's own stream the clearing runs beside the blend (rgs_frame_backward waits for it), else behind it.
-	if (int rc = side_streams_wait_for(K, layers, s, "rgs_frame_forward_raster"))
-		return rc;
-	for (int pass = 0; pass < 2; pass++) {
-		if (pass == 1) {
-			rgs::launch_blend_forward(jobs.data(), K, s);
-			RGS_STAGE("blend_forward");
-		}
-		for (int k = 0; k < K; k++) {
-			const rgs_frame_layer& l = layers[k];
-			const bool own_stream = l.stream && static_cast<hipStream_t>(l.stream) != s;
-			if (own_stream != (pass == 0))
-				continue;
-			for (int c = 0; c < 2; c++)
-				if (l.clear[c] && l.clear_bytes[c] != 0) {
-					RGS_REQUIRE((l.clear_bytes[c] & 3) == 0, "rgs_frame_forward_raster: clear_bytes must be a multiple of 4");
-					if (!own_stream)
-						rgs::stage_mark("clear_gradients", s);
-					rgs::launch_fill_u32(static_cast<uint32_t*>(l.clear[c]), 0u, l.clear_bytes[c] / 4,
-					                     own_stream ? static_cast<hipStream_t>(l.stream) : s);
-					RGS_STAGE("clear gradients");
-				}
-		}
-	}
+	rgs::launch_blend_forward(jobs.data(), K, s);
+	RGS_STAGE("blend_forward");
 	return 0;
 }
 
@@ -1027,12 +1004,11 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 	RGS_TAKE_SORT_FAULT("rgs_frame_backward");
 	RGS_REQUIRE(K >= 1 && K <= RGS_MAX_FRAME_LAYERS && layers && view, "rgs_frame_backward: K = %d outside 1..%d, or null", K,
 	            RGS_MAX_FRAME_LAYERS);
-	// what the forward left running on the layers' own streams (the clearing of the gradient buffers) comes first
-	if (int rc = wait_for_side_streams(K, layers, s, "rgs_frame_backward"))
-		return rc;
+	const std::vector<hipStream_t> sides = side_streams(K, layers, s);
+	hipStream_t beside = sides.empty() ? s : sides[0];  // where the bandwidth-bound work goes
 	std::vector<rgs::BlendArgs> jobs;
+	std::vector<int> job_layer;
 	std::vector<rgs::PreprocessBackwardArgs> geometry((size_t)K);
-	std::vector<int> zeroed((size_t)K);
 	for (int k = 0; k < K; k++) {
 		const rgs_frame_layer& l = layers[k];
 		if (int rc = check_backward_pointers("rgs_frame_backward", l.P, l.R, view->width, view->height, l.background, l.means3D,
@@ -1042,7 +1018,9 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		                                     l.dL_dmean2D, l.dL_dopacity, l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh,
 		                                     l.dL_dscale, l.dL_drot))
 			return rc;
-		if (!l.outputs_zeroed) {
+		RGS_REQUIRE(!l.grad_block || (l.grad_block_bytes & 3) == 0, "rgs_frame_backward: grad_block_bytes must be a multiple of 4");
+		if (!l.outputs_zeroed) {  // the blend adds into the rows of sums: they come first, on the frame's stream
+			rgs::stage_mark("clear_gradients", s);
 			rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(l.grad_accum), 0u, (size_t)RGS_ACC_FLOATS * (size_t)l.P, s);
 			RGS_STAGE("clear gradient sums");
 		}
@@ -1054,19 +1032,79 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 			a.dL_dpix = l.dL_dpix; a.dL_dpix_depth = l.dL_dpix_depth; a.dL_dalpha = l.dL_dalphas;
 			a.sums = l.grad_accum;
 			jobs.push_back(a);
+			job_layer.push_back(k);
 		}
 		fill_backward_geometry(geometry[(size_t)k], l.P, l.D, l.M, view->width, view->height, l.means3D, l.shs, l.scales,
 		                       l.scale_modifier, l.rotations, l.cov3D_precomp, view->viewmatrix, view->projmatrix, view->cam_pos,
 		                       view->tan_fovx, view->tan_fovy, l.radii, l.geom_ws, l.grad_accum, l.dL_dmean2D, l.dL_dopacity,
 		                       l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh, l.dL_dscale, l.dL_drot);
-		zeroed[(size_t)k] = l.outputs_zeroed;
 	}
-	if (!jobs.empty()) {
-		rgs::launch_blend_backward(jobs.data(), (int)jobs.size(), s);
-		RGS_STAGE("blend_backward");
+	// The gradient arrays are cleared (pure memory traffic) beside the blend (instruction issue) when there is a second stream.
+	hipError_t e = hipSuccess;
+	if (beside != s) {
+		hipEvent_t begun = frame_event(0);
+		e = begun ? hipEventRecord(begun, s) : hipErrorUnknown;
+		if (e == hipSuccess)
+			e = hipStreamWaitEvent(beside, begun, 0);
+		if (e != hipSuccess)
+			return fail("rgs_frame_backward: ordering the streams failed: %s", hipGetErrorString(e));
 	}
-	rgs::launch_preprocess_backward(geometry.data(), zeroed.data(), K, s);
-	RGS_STAGE("preprocess_backward");
+	std::vector<int> already((size_t)K, 1);  // as far as launch_preprocess_backward is concerned: cleared here, or by the caller
+	for (int k = 0; k < K; k++) {
+		const rgs_frame_layer& l = layers[k];
+		if (l.outputs_zeroed)
+			continue;
+		if (l.grad_block) {
+			if (beside == s)
+				rgs::stage_mark("clear_gradients", s);
+			rgs::launch_fill_u32(static_cast<uint32_t*>(l.grad_block), 0u, l.grad_block_bytes / 4, beside);
+			RGS_STAGE("clear gradients");
+		} else {
+			already[(size_t)k] = 0;
+		}
+	}
+	// With a second stream the blend goes in two halves, so that the per-Gaussian backward of the first half's layers
+	// (memory bandwidth) runs beside the blend of the second half.  Layers without instances go with the last half.
+	const int n_jobs = (int)jobs.size();
+	const int halves = (beside != s && n_jobs >= 2) ? 2 : 1;
+	const int first_half = halves == 2 ? (n_jobs + 1) / 2 : n_jobs;
+	std::vector<char> in_first((size_t)K, 0);
+	for (int i = 0; i < first_half; i++)
+		in_first[(size_t)job_layer[(size_t)i]] = 1;
+	for (int half = 0; half < halves; half++) {
+		const int from = half == 0 ? 0 : first_half, to = half == 0 ? first_half : n_jobs;
+		if (to > from) {
+			rgs::launch_blend_backward(jobs.data() + from, to - from, s);
+			RGS_STAGE("blend_backward");
+		}
+		std::vector<rgs::PreprocessBackwardArgs> part;
+		std::vector<int> part_zeroed;
+		for (int k = 0; k < K; k++)
+			if (halves == 1 || (in_first[(size_t)k] != 0) == (half == 0)) {
+				part.push_back(geometry[(size_t)k]);
+				part_zeroed.push_back(already[(size_t)k]);
+			}
+		if (part.empty())
+			continue;
+		if (beside != s) {
+			hipEvent_t blended = frame_event((size_t)(1 + half));
+			e = blended ? hipEventRecord(blended, s) : hipErrorUnknown;
+			if (e == hipSuccess)
+				e = hipStreamWaitEvent(beside, blended, 0);
+			if (e != hipSuccess)
+				return fail("rgs_frame_backward: ordering the streams failed: %s", hipGetErrorString(e));
+		}
+		rgs::launch_preprocess_backward(part.data(), part_zeroed.data(), (int)part.size(), beside);
+		RGS_STAGE("preprocess_backward");
+	}
+	if (beside != s) {
+		hipEvent_t done = frame_event(3);
+		e = done ? hipEventRecord(done, beside) : hipErrorUnknown;
+		if (e == hipSuccess)
+			e = hipStreamWaitEvent(s, done, 0);
+		if (e != hipSuccess)
+			return fail("rgs_frame_backward: ordering the streams failed: %s", hipGetErrorString(e));
+	}
 	return 0;
 }
 

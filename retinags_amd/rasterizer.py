@@ -446,8 +446,8 @@ class _RasterizeFrame(torch.autograd.Function):
     blend launch for all and every layer's per-Gaussian backward).
 
     apply(settings, streams, *flat): `settings` a tuple of K GaussianRasterizationSettings (same camera and
-    image size), `streams` None or a tuple of K HIP stream handles (a layer's own stream, on which the
-    stages that run once per layer are queued, beside the other layers'), flat = for every layer
+    image size), `streams` None or a tuple of K HIP stream handles (the first that differs from the current
+    stream serves the backward as a second stream for its memory-bound work), flat = for every layer
     (means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp).
     Returns for every layer (color, radii, depth, alpha)."""
 
@@ -491,13 +491,11 @@ class _RasterizeFrame(torch.autograd.Function):
                     ("scales", scales), ("rotations", rotations), ("cov3Ds_precomp", cov3Ds), ("bg", rs.bg),
                     ("range_low", rs.range_low), ("range_up", rs.range_up))}
                 rec = dict(P=P, M=M, t=t, package=package, radii=torch.empty((P,), dtype=torch.int32, device=device),
-                           rendered=0, geom=torch.empty(0, **byte), binning=torch.empty(0, **byte), img=torch.empty(0, **byte),
-                           cleared=None)
+                           rendered=0, geom=torch.empty(0, **byte), binning=torch.empty(0, **byte), img=torch.empty(0, **byte))
                 records.append(rec)
                 if P == 0:
                     package.zero_()
                     continue
-                needs = ctx.needs_input_grad[2 + 8 * k:2 + 8 * (k + 1)]
                 L = arr[len(live)]
                 live.append(k)
                 L.P, L.D, L.M = P, int(rs.sh_degree), M
@@ -512,16 +510,6 @@ class _RasterizeFrame(torch.autograd.Function):
                 L.geom_ws, L.image_ws = ptr(rec["geom"]), ptr(rec["img"])
                 L.geom_bytes, L.image_bytes = geom_bytes, image_bytes
                 L.out_color, L.out_depth, L.out_alpha = ptr(package[0:3]), ptr(package[3:4]), ptr(package[4:5])
-                L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
-                if any(needs):
-                    # Only rendered Gaussians get their gradient rows written; the library clears the rest behind
-                    # the layer's geometry stage, where that pure memory traffic runs beside the other layers' short kernels.
-                    cleared = _gradient_outputs(P, M, scales.numel() != 0, device, torch.empty)
-                    rec["cleared"] = cleared
-                    base = cleared["means2D"]
-                    span = cleared["rotations"].data_ptr() + cleared["rotations"].numel() * 4 - base.data_ptr()
-                    L.clear[0], L.clear_bytes[0] = base.data_ptr(), span
-                    L.clear[1], L.clear_bytes[1] = cleared["sums"].data_ptr(), cleared["sums"].numel() * 4
             if live:
                 counts = _frame_counts(device, len(live))
                 check(lib.rgs_frame_forward_geom(len(live), arr, C.byref(view), C.c_void_p(counts.data_ptr()), C.c_void_p(main), debug))
@@ -540,7 +528,7 @@ class _RasterizeFrame(torch.autograd.Function):
         saved, outs = [], []
         for k, rec in enumerate(records):
             t = rec["t"]
-            ctx.meta.append(dict(rendered=rec["rendered"], cleared=rec["cleared"]))
+            ctx.meta.append(dict(rendered=rec["rendered"]))
             saved += [t["colors_precomp"], t["means3D"], t["scales"], t["rotations"], t["cov3Ds_precomp"], rec["radii"], t["sh"],
                       rec["geom"], rec["binning"], rec["img"], rec["package"][4:5]]
             outs += [rec["package"][0:3], rec["radii"], rec["package"][3:4], rec["package"][4:5]]
@@ -575,7 +563,10 @@ class _RasterizeFrame(torch.autograd.Function):
             if g_color is None:
                 g_color = torch.zeros((3, H, W), **f32)
             has_scales = scales.numel() != 0
-            out = meta["cleared"] if meta["cleared"] is not None else _gradient_outputs(P, M, has_scales, device, torch.empty)
+            # Only rendered Gaussians get their gradient rows written; the library clears the rest (beside the blend,
+            # on the second stream, if it is given one).
+            out = _gradient_outputs(P, M, has_scales, device, torch.empty)
+            keep.append(out)   # its scratch rows must outlive the library call below
             t = dict(bg=_dev_f32(rs.bg, device, "bg"), low=_dev_f32(rs.range_low, device, "range_low"),
                      up=_dev_f32(rs.range_up, device, "range_up"), g_color=_dev_f32(g_color, device, "grad_color"),
                      g_depth=None if g_depth is None else _dev_f32(g_depth, device, "grad_depth"),
@@ -603,7 +594,10 @@ class _RasterizeFrame(torch.autograd.Function):
             L.dL_dmean3D, L.dL_dcov3D, L.dL_dsh = ptr(out["means3D"]), ptr(out["cov3D"]), ptr(out["sh"])
             L.dL_dscale = ptr(out["scales"]) if has_scales else C.c_void_p(0)
             L.dL_drot = ptr(out["rotations"]) if has_scales else C.c_void_p(0)
-            L.outputs_zeroed = int(meta["cleared"] is not None)
+            L.outputs_zeroed = 0
+            base = out["means2D"]
+            L.grad_block = base.data_ptr()
+            L.grad_block_bytes = out["rotations"].data_ptr() + out["rotations"].numel() * 4 - base.data_ptr()
             L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
             results.append((out["means2D"], out["colors"], out["opacity"], out["means3D"], out["cov3D"], out["sh"],
                             out["scales"], out["rotations"]))
@@ -639,8 +633,8 @@ def rasterize_frame(rasterizers, inputs, streams=None):
     """All layers of a frame through one call.  `rasterizers`: K GaussianRasterizer (their settings share the
     camera and the image size); `inputs`: K dicts with the keyword arguments of GaussianRasterizer.forward
     (means3D, means2D, opacities, shs / colors_precomp, scales + rotations / cov3D_precomp); `streams`: None,
-    or for every layer the handle of a HIP stream on which the stages that run once per layer are queued (the
-    caller's stream waits for them).  Returns K tuples (color, radii, depth, alpha), the results of K
+    or for every layer the handle of a HIP stream; the first that is not the current stream is used by the
+    backward for its memory-bound work, beside the blend (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
     forward calls, and differentiates like them."""
     flat = []
     for rz, kw in zip(rasterizers, inputs):
