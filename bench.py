@@ -269,7 +269,9 @@ def measure(args, config, forward_only, asides, cpu):
     # Algorithmic bytes per frame of every HBM-bound stage (one launch per submodel; the sort
     # kernels run `passes` times per submodel).
     alg_bytes = {
-        "preprocess_forward": 20.0 * P_tot + 299.0 * P_vis,
+        # mean in, radius and tile count out for all; scale, rotation, opacity, SH row in and depth, clamp flags,
+        # 64-byte record out for the rendered ones
+        "preprocess_forward": 20.0 * P_tot + (224.0 + 69.0) * P_vis,
         # tile counts and depths of all, then 4 passes over the (depth, index) pairs of the visible
         # ones, the gathered tile counts and their scan
         "depth_order": 8.0 * P_tot + (12.0 + 4 * 16.0 + 16.0) * P_vis,
@@ -281,9 +283,9 @@ def measure(args, config, forward_only, asides, cpu):
         "strip_filing": 8.0 * R_tot + 16.0 * T * K,
         # the eight gradient tensors and the rows of sums, written once
         "clear_gradients": (4.0 * (3 + 1 + 3 + 3 + 6 + 48 + 3 + 4) + 48.0) * P_tot,
-        # rows of the rendered Gaussians only: sums, mean, covariance, SH, scale, rotation in;
+        # rows of the rendered Gaussians only: sums, mean, SH, scale, rotation in;
         # the eight gradient rows out
-        "preprocess_backward": (309.0 + 284.0) * P_vis,
+        "preprocess_backward": (285.0 + 284.0) * P_vis,
         "composite_forward": (20.0 * K + 20.0) * N,
         "composite_backward": (40.0 * K + 20.0) * N,
     }

@@ -62,11 +62,6 @@ size_t rgs_image_bytes(int width, int height);
  * look at intermediate results.  The workspaces are otherwise opaque. */
 enum {
 	RGS_GEOM_DEPTHS = 0,        /* float[P]   view-space z */
-	RGS_GEOM_XY,                /* float2[P]  pixel centre */
-	RGS_GEOM_CLIP_W,            /* float[P]   clip-space w */
-	RGS_GEOM_COV3D,             /* float[6P] */
-	RGS_GEOM_CONIC_OPACITY,     /* float4[P] */
-	RGS_GEOM_RGB,               /* float[3P] */
 	RGS_GEOM_TILES_TOUCHED,     /* uint32[P] */
 	RGS_GEOM_POINT_OFFSETS,     /* uint32[P]  inclusive prefix sum of the tile counts of the Gaussians in
 	                               RGS_GEOM_DEPTH_ORDER (as many entries as that has) */
@@ -75,7 +70,9 @@ enum {
 	RGS_GEOM_TOTAL,             /* uint32     number of (Gaussian, tile) instances */
 	RGS_GEOM_BLEND_RECORD,      /* float[16P] one 64-byte record per Gaussian with everything the blend reads:
 	                               x, y, exponent floor, clip w | conic xx, xy, yy, opacity | r, g, b, depth |
-	                               half-width, half-height of the alpha >= 1/255 ellipse's bounding box, the radius (int32 bits), 0 */
+	                               half-width, half-height of the alpha >= 1/255 ellipse's bounding box, the radius (int32 bits), 0.
+	                               The pixel centre, clip w, conic, opacity and colour of a Gaussian are kept here only; its
+	                               3D covariance is not kept at all (the backward computes it again from scale and rotation) */
 	RGS_GEOM_DEPTH_ORDER,       /* uint32[P]  the Gaussians that touch a tile by increasing depth, ties by index;
 	                               entries from RGS_GEOM_VISIBLE_COUNT on are unused */
 	RGS_GEOM_BLOCK_VISIBLE,     /* uint32[ceil(P/256)+1] */
@@ -119,6 +116,12 @@ int rgs_image_layout(int width, int height, size_t offsets[RGS_IMG_FIELDS]);
  * rasterizer_impl.cu:141-153) behind _C.mark_visible (K/ext.cpp:18). */
 int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const float* projmatrix,
                      uint8_t* present, void* stream);
+
+/* cov3D[6 i .. 6 i + 5] = the upper triangle of R S S^T R^T of Gaussian i (S = scale_modifier * scales, R from the
+ * quaternion), exactly as the forward and the backward compute it for themselves: neither keeps it in a workspace.
+ * Restates computeCov3D (K/cuda_rasterizer_hgs/forward.cu:117-152), which the reference reaches only from inside
+ * preprocessCUDA; offered for callers and tests that want the values. */
+int rgs_covariance3d(int P, const float* scales, float scale_modifier, const float* rotations, float* cov3D, void* stream);
 
 /* First half of Rasterizer::forward (K/cuda_rasterizer_hgs/rasterizer.h:29-58,
  * rasterizer_impl.cu:198-287): per-Gaussian preprocess and the prefix sum of the tile

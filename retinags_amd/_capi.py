@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # RGS_LIBRARY selects another build of the same library (used when comparing kernel variants)
 LIB_PATH = os.environ.get("RGS_LIBRARY") or os.path.join(_HERE, "librgs_gfx950.so")
 
-GEOM_FIELDS = ("depths", "xy", "clip_w", "cov3D", "conic_opacity", "rgb", "tiles_touched", "point_offsets",
+GEOM_FIELDS = ("depths", "tiles_touched", "point_offsets",
                "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
                "visible_list", "order_scratch")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp", "strip_lists")
@@ -87,6 +87,7 @@ def _load():
     lib.rgs_binning_layout.argtypes = [i, i, i, C.POINTER(sz)]
     lib.rgs_image_layout.argtypes = [i, i, C.POINTER(sz)]
     lib.rgs_mark_visible.argtypes = [i, vp, vp, vp, vp, vp]
+    lib.rgs_covariance3d.argtypes = [i, vp, f, vp, vp, vp]
     lib.rgs_forward_geom.argtypes = [i, i, i, i, i, vp, vp, vp, vp, vp, f, vp, vp, vp, vp, vp, f, f, i,
                                      vp, vp, sz, vp, vp, i]
     lib.rgs_forward_geom_enqueue.argtypes = lib.rgs_forward_geom.argtypes[:-2] + [vp, vp, i]
@@ -120,7 +121,7 @@ def _load():
     lib.rgs_stage_timing.argtypes = [i]
     lib.rgs_stage_timing_read.argtypes = [i, C.POINTER(C.c_char_p), C.POINTER(C.c_float), C.POINTER(C.c_int)]
     lib.rgs_blend_work_counters.argtypes = [i, i, i, i, f, f, vp, vp, vp, vp, vp, vp, vp, vp, vp]
-    for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
+    for name in ("rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible", "rgs_covariance3d",
                  "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_forward_raster_bounded", "rgs_backward", "rgs_inclusive_sum", "rgs_sort_pairs",
                  "rgs_composite_forward", "rgs_composite_backward", "rgs_straddler_select", "rgs_merge_rows",
                  "rgs_merge_rows_backward", "rgs_l1_ssim_forward", "rgs_l1_ssim_backward", "rgs_adam_step",
@@ -134,7 +135,7 @@ def _load():
 lib = _load()
 
 EXPORTS = ("rgs_version", "rgs_last_error", "rgs_get_higher_msb", "rgs_geom_bytes", "rgs_binning_bytes",
-           "rgs_image_bytes", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible",
+           "rgs_image_bytes", "rgs_geom_layout", "rgs_binning_layout", "rgs_image_layout", "rgs_mark_visible", "rgs_covariance3d",
            "rgs_forward_geom", "rgs_forward_geom_enqueue", "rgs_forward_raster", "rgs_forward_raster_bounded", "rgs_backward", "rgs_scan_temp_bytes", "rgs_inclusive_sum",
            "rgs_sort_temp_bytes", "rgs_sort_pairs", "rgs_composite_forward", "rgs_composite_backward",
            "rgs_stage_timing", "rgs_stage_timing_read", "rgs_blend_work_counters", "rgs_straddler_scratch_bytes",

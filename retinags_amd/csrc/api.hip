@@ -203,11 +203,6 @@ size_t geom_layout(size_t P, size_t* off)
 {
 	Carver c;
 	off[RGS_GEOM_DEPTHS] = c.take(4 * P);
-	off[RGS_GEOM_XY] = c.take(8 * P);
-	off[RGS_GEOM_CLIP_W] = c.take(4 * P);
-	off[RGS_GEOM_COV3D] = c.take(24 * P);
-	off[RGS_GEOM_CONIC_OPACITY] = c.take(16 * P);
-	off[RGS_GEOM_RGB] = c.take(12 * P);
 	off[RGS_GEOM_TILES_TOUCHED] = c.take(4 * P);
 	off[RGS_GEOM_POINT_OFFSETS] = c.take(4 * P);
 	off[RGS_GEOM_CLAMPED] = c.take(P);
@@ -409,6 +404,21 @@ int rgs_mark_visible(int P, const float* means3D, const float* viewmatrix, const
 	return 0;
 }
 
+int rgs_covariance3d(int P, const float* scales, float scale_modifier, const float* rotations, float* cov3D, void* stream)
+{
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	EntryScope scope_(s);
+	const int debug = 0;
+	RGS_REQUIRE(P >= 0, "rgs_covariance3d: negative P");
+	if (P == 0)
+		return 0;
+	RGS_REQUIRE(scales && rotations && cov3D, "rgs_covariance3d: null pointer");
+	RGS_REQUIRE((reinterpret_cast<uintptr_t>(rotations) & 15) == 0, "rgs_covariance3d: rotations must be 16-byte aligned");
+	rgs::launch_covariance3d(P, scales, scale_modifier, rotations, cov3D, s);
+	RGS_STAGE("covariance3d");
+	return 0;
+}
+
 // Whether SH rows can be moved 16 bytes at a time: aligned base, row length a multiple of four
 // floats, at most 48 of them, and enough of them for the degree's rounded-up count.
 static bool sh_rows_by_16_bytes(const float* shs, int M, int D)
@@ -493,12 +503,7 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 		a.grid_x = (width + rgs::kTile - 1) / rgs::kTile;
 		a.grid_y = (height + rgs::kTile - 1) / rgs::kTile;
 		a.radii = c.radii;
-		a.xy = at<float2>(ws, off[RGS_GEOM_XY]);
-		a.clip_w = at<float>(ws, off[RGS_GEOM_CLIP_W]);
 		a.depths = at<float>(ws, off[RGS_GEOM_DEPTHS]);
-		a.cov3D = at<float>(ws, off[RGS_GEOM_COV3D]);
-		a.rgb = at<float>(ws, off[RGS_GEOM_RGB]);
-		a.conic_opacity = at<float4>(ws, off[RGS_GEOM_CONIC_OPACITY]);
 		a.tiles_touched = at<uint32_t>(ws, off[RGS_GEOM_TILES_TOUCHED]);
 		a.clamped = at<uint8_t>(ws, off[RGS_GEOM_CLAMPED]);
 		a.block_sums = at<uint32_t>(ws, off[RGS_GEOM_BLOCK_SUMS]);
@@ -604,11 +609,6 @@ void fill_blend_args(rgs::BlendArgs& a, int P, int R, int width, int height, flo
 	a.W = width; a.H = height; a.grid_x = gx; a.grid_y = gy;
 	a.tanfovx = tan_fovx; a.tanfovy = tan_fovy;
 	a.projinv = projmatrix_inv; a.range_low = range_low; a.range_up = range_up; a.bg = background;
-	a.xy = at<float2>(geom_ws, goff[RGS_GEOM_XY]);
-	a.clip_w = at<float>(geom_ws, goff[RGS_GEOM_CLIP_W]);
-	a.conic_opacity = at<float4>(geom_ws, goff[RGS_GEOM_CONIC_OPACITY]);
-	a.colors = colors_precomp ? colors_precomp : at<float>(geom_ws, goff[RGS_GEOM_RGB]);
-	a.depths = at<float>(geom_ws, goff[RGS_GEOM_DEPTHS]);
 	a.record = at<float4>(geom_ws, goff[RGS_GEOM_BLEND_RECORD]);
 	a.n_contrib = at<uint32_t>(img, ioff[RGS_IMG_N_CONTRIB]);
 	a.strip_filed = at<uint32_t>(img, ioff[RGS_IMG_STRIP_FILED]);
@@ -781,7 +781,7 @@ void fill_backward_geometry(rgs::PreprocessBackwardArgs& p, int P, int D, int M,
 	p.means = means3D; p.radii = radii; p.shs = shs;
 	p.clamped = at<uint8_t>(geom_ws, goff[RGS_GEOM_CLAMPED]);
 	p.scales = scales; p.rotations = rotations; p.scale_modifier = scale_modifier;
-	p.cov3D = cov3D_precomp ? cov3D_precomp : at<float>(geom_ws, goff[RGS_GEOM_COV3D]);
+	p.cov3D_precomp = cov3D_precomp;
 	p.view = viewmatrix; p.proj = projmatrix; p.campos = cam_pos;
 	p.focal_y = height / (2.0f * tan_fovy);
 	p.focal_x = width / (2.0f * tan_fovx);

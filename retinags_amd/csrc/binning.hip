@@ -497,12 +497,23 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 	for (int p = 0; p < kSortMaxPasses; p++)
 		s_hist[p][threadIdx.x] = 0;
 	__syncthreads();
-	for (size_t k = (size_t)blockIdx.x * 256 + threadIdx.x; k < n; k += (size_t)gridDim.x * 256) {
-		const KeyT key = keys[k];
-		for (int p = 0; p < passes; p++) {
-			const int shift = 8 * p;
-			const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
-			atomicAdd(&s_hist[p][digit_of(key, shift, (1u << bits) - 1u)], 1u);
+	// four keys per thread and round, requested together: one key at a time the loop waits for
+	// memory once per key and the kernel takes as long as a pass of the sort
+	const size_t threads = (size_t)gridDim.x * 256;
+	for (size_t k = (size_t)blockIdx.x * 256 + threadIdx.x; k < n; k += 4 * threads) {
+		KeyT key[4];
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+			key[q] = k + q * threads < n ? keys[k + q * threads] : (KeyT)0;
+#pragma unroll
+		for (int q = 0; q < 4; q++) {
+			if (k + q * threads >= n)
+				break;
+			for (int p = 0; p < passes; p++) {
+				const int shift = 8 * p;
+				const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+				atomicAdd(&s_hist[p][digit_of(key[q], shift, (1u << bits) - 1u)], 1u);
+			}
 		}
 	}
 	__syncthreads();

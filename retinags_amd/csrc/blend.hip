@@ -373,9 +373,9 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 		const uint32_t src = range.x + (uint32_t)i * 256 + tid;
 		if (src < range.y) {
 			const uint32_t id = a.point_list[src];
-			const float2 xy = a.xy[id];
-			s_geom[tid] = float4{xy.x, xy.y, 0.f, a.clip_w[id]};
-			s_conic[tid] = a.conic_opacity[id];
+			const float4 r0 = a.record[4 * (size_t)id];
+			s_geom[tid] = float4{r0.x, r0.y, 0.f, r0.w};
+			s_conic[tid] = a.record[4 * (size_t)id + 1];
 		}
 		__syncthreads();
 		const int count = todo < 256 ? todo : 256;

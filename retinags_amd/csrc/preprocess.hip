@@ -191,7 +191,11 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<Preproces
 			if (ntiles == 0)
 				break;
 
-			if (!a.colors_precomp) {
+			float3 col;
+			if (a.colors_precomp) {
+				col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
+				             a.colors_precomp[3 * (size_t)idx + 2]};
+			} else {
 				const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
 				const float3 dir = {p.x - cam.x, p.y - cam.y, p.z - cam.z};
 				const float len = sqrtf(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
@@ -216,29 +220,15 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<Preproces
 					clamp_bits |= (v < 0) ? (1u << ch) : 0u;
 					rgb[ch] = fmaxf(v, 0.0f);
 				}
-				a.rgb[3 * (size_t)idx + 0] = rgb[0];
-				a.rgb[3 * (size_t)idx + 1] = rgb[1];
-				a.rgb[3 * (size_t)idx + 2] = rgb[2];
+				col = float3{rgb[0], rgb[1], rgb[2]};
 				a.clamped[idx] = (uint8_t)clamp_bits;
 			}
-			if (!a.cov3D_precomp) {
-#pragma unroll
-				for (int i = 0; i < 6; i++)
-					a.cov3D[6 * (size_t)idx + i] = cov6[i];
-			}
 			a.depths[idx] = p_view.z;
-			a.xy[idx] = pix;
-			a.clip_w[idx] = p_hom.w;
-			a.conic_opacity[idx] = conic_o;
 			{
-				// Packed copy for the blend kernels, which gather per-Gaussian data in depth order:
-				// one 64-byte record instead of one cache line from each of five arrays.
-				float3 col;
-				if (a.colors_precomp)
-					col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
-					             a.colors_precomp[3 * (size_t)idx + 2]};
-				else
-					col = float3{a.rgb[3 * (size_t)idx], a.rgb[3 * (size_t)idx + 1], a.rgb[3 * (size_t)idx + 2]};
+				// Everything later stages read of a rendered Gaussian goes into one 64-byte record: a
+				// gather by index then costs one cache line, and nothing is written a second time into
+				// arrays of their own, where a rendered Gaussian among unrendered ones dirties a whole
+				// line for a few bytes.  The 3D covariance is not kept: the backward computes it again.
 				const float floor = exponent_floor(conic_o.w);
 				const float2 half = alpha_ellipse_half_extent(conic_o, floor);
 				float4* rec = a.blend_record + 4 * (size_t)idx;
@@ -352,7 +342,6 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	const float* __restrict__ view = a.view;
 	const float* __restrict__ proj = a.proj;
 	const float3 mean = {a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
-	const float* cov6 = a.cov3D + 6 * i;
 	const float4* sums = reinterpret_cast<const float4*>(a.sums + kSumCols * i);
 	const float4 sum0 = sums[0], sum1 = sums[1], sum2v = sums[2];
 	const float3 dLc = {sum0.z, sum0.w, sum1.x};  // kSumConicXX, kSumConicXY, kSumConicYY
@@ -366,9 +355,15 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 
 	// -- conic -> cov2D -> cov3D and mean (backward.cu:144-274)
 	float cov6r[6];
+	if (a.cov3D_precomp) {
 #pragma unroll
-	for (int k = 0; k < 6; k++)
-		cov6r[k] = cov6[k];
+		for (int k = 0; k < 6; k++)
+			cov6r[k] = a.cov3D_precomp[6 * i + k];
+	} else {
+		// the same arithmetic as the forward's, which did not keep its result
+		const float3 sc = {a.scales[3 * i], a.scales[3 * i + 1], a.scales[3 * i + 2]};
+		covariance3d(sc, a.scale_modifier, reinterpret_cast<const float4*>(a.rotations)[i], cov6r);
+	}
 	Ewa e = ewa_project(mean, a.focal_x, a.focal_y, a.tanfovx, a.tanfovy, cov6r, view);
 	const float x_grad_mul = (e.txtz < -e.limx || e.txtz > e.limx) ? 0.f : 1.f;
 	const float y_grad_mul = (e.tytz < -e.limy || e.tytz > e.limy) ? 0.f : 1.f;
@@ -560,6 +555,25 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 }
 
 // ---- launchers -----------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void covariance3d_kernel(int P, const float* __restrict__ scales, float mod,
+                                                            const float* __restrict__ rotations, float* __restrict__ cov3D)
+{
+	const int idx = blockIdx.x * 256 + threadIdx.x;
+	if (idx >= P)
+		return;
+	const float3 sc = {scales[3 * (size_t)idx], scales[3 * (size_t)idx + 1], scales[3 * (size_t)idx + 2]};
+	float cov6[6];
+	covariance3d(sc, mod, reinterpret_cast<const float4*>(rotations)[idx], cov6);
+#pragma unroll
+	for (int i = 0; i < 6; i++)
+		cov3D[6 * (size_t)idx + i] = cov6[i];
+}
+
+void launch_covariance3d(int P, const float* scales, float scale_modifier, const float* rotations, float* cov3D, hipStream_t s)
+{
+	hipLaunchKernelGGL(covariance3d_kernel, dim3((P + 255) / 256), dim3(256), 0, s, P, scales, scale_modifier, rotations, cov3D);
+}
 
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s)
 {

@@ -33,12 +33,7 @@ struct PreprocessArgs {
 	int grid_x, grid_y;
 	// outputs
 	int* radii;
-	float2* xy;
-	float* clip_w;
 	float* depths;
-	float* cov3D;
-	float* rgb;
-	float4* conic_opacity;
 	uint32_t* tiles_touched;
 	uint8_t* clamped;
 	uint32_t* block_sums;  // one per 256 Gaussians
@@ -58,7 +53,7 @@ struct PreprocessBackwardArgs {
 	const float* scales;   // may be null
 	const float* rotations;
 	float scale_modifier;
-	const float* cov3D;
+	const float* cov3D_precomp;  // may be null: then the 3D covariance is computed from scale and rotation, as the forward did
 	const float* view;
 	const float* proj;
 	const float* campos;
@@ -87,12 +82,7 @@ struct BlendArgs {
 	const float* range_low;
 	const float* range_up;
 	const float* bg;
-	const float2* xy;
-	const float* clip_w;
-	const float4* conic_opacity;
-	const float* colors;  // (P,3)
-	const float* depths;
-	const float4* record;  // 4 float4 per Gaussian: the packed copy of the arrays above that the blend gathers
+	const float4* record;  // 4 float4 per Gaussian: everything the blend reads of it
 	// forward outputs / backward inputs
 	float* out_color;
 	float* out_depth;
@@ -285,6 +275,7 @@ struct FilingArgs {
 
 // preprocess.hip
 void launch_mark_visible(int P, const float* means, const float* view, uint8_t* present, hipStream_t s);
+void launch_covariance3d(int P, const float* scales, float scale_modifier, const float* rotations, float* cov3D, hipStream_t s);
 // `jobs` are host arrays: the submodels of a frame in one launch (kMaxBatch of them at a time).
 void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_t s);
 // Where outputs_zeroed[k] is 0 the eight output arrays of job k are cleared first.

@@ -43,8 +43,7 @@ def test_workspace_sizes_and_layouts_are_consistent():
     for P in (1, 255, 256, 257, 100_000):
         lay = _capi.geom_layout(P)
         total = _capi.lib.rgs_geom_bytes(P)
-        sizes = dict(depths=4 * P, xy=8 * P, clip_w=4 * P, cov3D=24 * P, conic_opacity=16 * P, rgb=12 * P,
-                     tiles_touched=4 * P, point_offsets=4 * P, clamped=P, block_sums=4 * ((P + 255) // 256 + 1), total=4,
+        sizes = dict(depths=4 * P, tiles_touched=4 * P, point_offsets=4 * P, clamped=P, block_sums=4 * ((P + 255) // 256 + 1), total=4,
                      blend_record=64 * P, depth_order=4 * P, block_visible=4 * ((P + 255) // 256 + 1),
                      visible_count=4, order_scratch=16 * P)
         spans = sorted((lay[k], lay[k] + sizes[k]) for k in sizes)

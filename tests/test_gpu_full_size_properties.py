@@ -186,7 +186,7 @@ def _sh_linearity(cam, subs, rel, which, seed):
     from retinags_amd import _capi
     P = sub.means3D.shape[0]
     raw = _forward_raw(sub, cam_d, cam, bg)
-    rgb = torch.from_numpy(view_ws(raw[5], _capi.geom_layout(P)["rgb"], 3 * P, np.float32).reshape(P, 3).copy()).to(DEV)
+    rgb = torch.from_numpy(view_ws(raw[5], _capi.geom_layout(P)["blend_record"], 16 * P, np.float32).reshape(P, 16)[:, 8:11].copy()).to(DEV)
     safe = rendered & (rgb.min(dim=1).values > 0.05)
     del raw
     assert int(safe.sum()) > 100

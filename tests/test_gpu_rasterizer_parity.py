@@ -5,6 +5,8 @@ Gaussians and their offsets, the sorted (tile, depth) keys (rebuilt from the lib
 keys and depth bits), per-tile Gaussian lists, tile ranges.  Within 1e-4 max-abs:
 rendered colour, depth and alpha planes.  Within 1e-3 relative L2: every gradient.
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -43,16 +45,21 @@ def _check_forward_stages(sub, cam, bg, sh_degree=3, scale_modifier=1.0, max_bor
     vis = st.radii > 0
     g = _capi.geom_layout(P)
     assert np.array_equal(view_ws(geom, g["tiles_touched"], P, np.uint32), st.tiles_touched)
-    xy = view_ws(geom, g["xy"], 2 * P, np.float32).reshape(P, 2)
-    assert np.array_equal(xy[vis].view(np.uint32), st.xy[vis].view(np.uint32))
     assert np.array_equal(view_ws(geom, g["depths"], P, np.uint32)[vis], st.depths.view(np.uint32)[vis])
-    assert np.array_equal(view_ws(geom, g["clip_w"], P, np.uint32)[vis], st.zw[:, 1].copy().view(np.uint32)[vis])
-    co = view_ws(geom, g["conic_opacity"], 4 * P, np.float32).reshape(P, 4)
-    assert np.array_equal(co[vis].view(np.uint32), st.conic_opacity[vis].view(np.uint32))
-    cov = view_ws(geom, g["cov3D"], 6 * P, np.float32).reshape(P, 6)
-    assert np.array_equal(cov[vis].view(np.uint32), st.cov3D[vis].view(np.uint32))
-    rgb = view_ws(geom, g["rgb"], 3 * P, np.float32).reshape(P, 3)
-    assert np.array_equal(rgb[vis].view(np.uint32), st.rgb[vis].view(np.uint32))
+    # pixel centre, clip w, conic, opacity and colour live in the Gaussian's 64-byte record only
+    rec = view_ws(geom, g["blend_record"], 16 * P, np.uint32).reshape(P, 16)[vis]
+    assert np.array_equal(rec[:, 0:2], st.xy[vis].view(np.uint32))
+    assert np.array_equal(rec[:, 3], st.zw[:, 1].copy().view(np.uint32)[vis])
+    assert np.array_equal(rec[:, 4:8], st.conic_opacity[vis].view(np.uint32))
+    assert np.array_equal(rec[:, 8:11], st.rgb[vis].view(np.uint32))
+    assert np.array_equal(rec[:, 11], st.depths.view(np.uint32)[vis])
+    assert np.array_equal(rec[:, 14], st.radii[vis].astype(np.int32).view(np.uint32))
+    # the 3D covariance is kept nowhere: forward and backward compute it with the function behind this entry point
+    cov = torch.empty((P, 6), device=dev)
+    scales_d, rot_d = sub["scales"].to(dev).contiguous(), sub["rotations"].to(dev).contiguous()
+    _capi.check(_capi.lib.rgs_covariance3d(P, _capi.ptr(scales_d), scale_modifier, _capi.ptr(rot_d), _capi.ptr(cov),
+                                           ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)))
+    assert np.array_equal(cov.cpu().numpy()[vis].view(np.uint32), st.cov3D[vis].view(np.uint32))
     clamped = view_ws(geom, g["clamped"], P, np.uint8)
     packed = st.clamped[:, 0] | (st.clamped[:, 1] << 1) | (st.clamped[:, 2] << 2)
     assert np.array_equal(clamped[vis], packed[vis])
