@@ -461,6 +461,7 @@ constexpr uint32_t kFlagAggregate = 1u << 30;  // word holds this tile's own dig
 constexpr uint32_t kFlagInclusive = 2u << 30;  // word holds the count of this and all earlier tiles
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
 constexpr int kLookbackSpinLimit = 1 << 18;
+constexpr int kLookBatch = 8;  // earlier tiles a look-back reads at once
 
 // How many times a look-back polls a word that has not been published yet before it gives up.
 // A negative value makes every look-back give up at once: the way a test drives the give-up
@@ -630,28 +631,46 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 			__hip_atomic_store(my_word, count | kFlagInclusive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		} else {
 			__hip_atomic_store(my_word, count | kFlagAggregate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			// Words of the tiles below t are still to be added.  Up to kLookBatch of them are requested
+			// together: walked one load at a time, the chain of tiles and not memory sets the pace of a pass.
 			uint32_t t = tile;
-			bool gave_up = spin_limit < 0;
-			while (!gave_up) {
-				t--;
-				const uint32_t* word = lookback + (size_t)t * 256 + tid;
-				uint32_t v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-				for (int spins = 0; (v >> 30) == 0u; spins++) {
-					// give up after a bounded wait, or as soon as any other look-back has
-					if (spins >= spin_limit ||
-					    ((spins & 255) == 255 &&
-					     __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
-						gave_up = true;
-						break;
+			bool gave_up = spin_limit < 0, done = false;
+			while (!gave_up && !done) {
+				uint32_t v[kLookBatch];
+#pragma unroll
+				for (int q = 0; q < kLookBatch; q++)
+					v[q] = (uint32_t)q < t ? __hip_atomic_load(lookback + (size_t)(t - 1u - (uint32_t)q) * 256 + tid, __ATOMIC_RELAXED,
+					                                           __HIP_MEMORY_SCOPE_AGENT)
+					                       : kFlagInclusive;  // below the first tile there is nothing
+				uint32_t used = 0;
+#pragma unroll
+				for (int q = 0; q < kLookBatch; q++) {
+					// a word counts once every nearer one has been published and none of them closed the sum
+					if (!done && used == (uint32_t)q && (v[q] >> 30) != 0u) {
+						exclusive += v[q] & kValueMask;
+						used = (uint32_t)q + 1u;
+						done = (v[q] & kFlagInclusive) != 0u;
 					}
-					__builtin_amdgcn_s_sleep(1);
-					v = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 				}
-				if (gave_up)
-					break;
-				exclusive += v & kValueMask;
-				if ((v & kFlagInclusive) || t == 0)
-					break;
+				t -= used < t ? used : t;
+				if (t == 0u)
+					done = true;
+				if (!done && used < (uint32_t)kLookBatch) {
+					// tile t - 1 has not published yet: wait for its word, then look again from there
+					const uint32_t* word = lookback + (size_t)(t - 1u) * 256 + tid;
+					uint32_t w = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+					for (int spins = 0; (w >> 30) == 0u; spins++) {
+						// give up after a bounded wait, or as soon as any other look-back has
+						if (spins >= spin_limit ||
+						    ((spins & 255) == 255 &&
+						     __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
+							gave_up = true;
+							break;
+						}
+						__builtin_amdgcn_s_sleep(1);
+						w = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+					}
+				}
 			}
 			if (gave_up)
 				atomicOr(status, 1u);
@@ -733,7 +752,10 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 			continue;
 		if (mark_stages)
 			stage_mark("sort_setup", s);
-		const uint32_t hist_blocks = max_tiles < 2048u ? max_tiles : 2048u;
+		// every block ends with an atomic add per digit and pass into its job's counts: a few hundred blocks per
+		// job read the keys as fast as thousands would, and queue far fewer adds on the same words
+		const uint32_t most_blocks = live >= 8 ? 256u : 2048u / (uint32_t)live;
+		const uint32_t hist_blocks = max_tiles < most_blocks ? max_tiles : most_blocks;
 		hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
 		for (int p = 0; p < passes; p++) {
 			const int shift = 8 * p;
