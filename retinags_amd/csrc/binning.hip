@@ -238,10 +238,10 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> ba
 // a workgroup writes kDupPositions consecutive instances, whichever Gaussians they belong to (one
 // that covers thousands of tiles is shared by several workgroups, a thousand that cover one tile
 // each are taken by one).  It finds the first Gaussian of its range by a 64-ary search over the
-// inclusive offsets, stages the Gaussians of its range in LDS 256 at a time (offset, tile rectangle,
-// the tile-independent part of the strip tests) and lets every thread find the Gaussian of its
-// output position by a binary search over those 256 offsets, then the tile from the position
-// inside that Gaussian's rectangle; stores are contiguous.  The thread also decides which of the
+// inclusive offsets, stages the offsets and indices of the Gaussians of its range in LDS 256 at a time
+// and lets every thread find the Gaussian of its output position by a binary search over those 256
+// offsets, read that Gaussian's 64-byte record, and take the tile from the position inside the
+// record's rectangle; stores are contiguous.  The thread also decides which of the
 // tile's four strips the instance can matter to (strip_filing.h) and puts those bits above the
 // tile in the key: the sort only looks at the tile bits, so they travel with the instance for free.
 // `order` is the output of a sort: should that sort ever have given up, its entries may be anything, so
@@ -250,10 +250,7 @@ constexpr int kDupPositions = 1024;
 
 struct DuplicateStage {
 	uint32_t end[256];     // inclusive offset of each staged Gaussian
-	uint32_t origin[256];  // first tile of its rectangle
-	uint32_t width[256];   // tiles per row of its rectangle
 	uint32_t index[256];
-	StripTests tests[256]; // the tile-independent part of its strip tests
 };
 
 // Floats of LDS for the NDC tables of a grid of tiles: 2 per tile column (rounded up to a multiple of 4), 8 per tile row.
@@ -329,60 +326,71 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	const BoxFrame box = load_box_frame(filing.projinv, filing.range_low, filing.range_up, filing.tanfovx, filing.tanfovy);
 
 	for (uint32_t g0 = s_first; g0 < n; g0 += 256) {
-		// stage Gaussians g0 .. g0 + 255 (in depth order)
+		// stage the offsets and indices of Gaussians g0 .. g0 + 255 (in depth order)
 		const uint32_t g = g0 + (uint32_t)tid;
-		uint32_t end = total, origin = 0, width = 1, idx = 0;
-		if (g < n) {
-			idx = min(order[g], P - 1u);
-			end = offsets[g];
-			// everything else comes from the Gaussian's 64-byte record: pixel centre, conic, extents, radius
-			const float4* rec = filing.record + 4 * (size_t)idx;
-			const float4 g4 = rec[0], h = rec[3];
-			const TileRect rc = tile_rect(g4.x, g4.y, __float_as_int(h.z), gx, gy);
-			origin = rc.y0 * (uint32_t)gx + rc.x0;
-			width = max(rc.x1 - rc.x0, 1u);
-			st.tests[tid] = prepare_strip_tests(FiledGeometry{g4, rec[1], float2{h.x, h.y}}, box);
-		}
-		st.end[tid] = end;
-		st.origin[tid] = origin;
-		st.width[tid] = width;
-		st.index[tid] = idx;
+		st.end[tid] = g < n ? offsets[g] : total;
+		st.index[tid] = g < n ? min(order[g], P - 1u) : 0u;
 		__syncthreads();
 		const uint32_t staged_begin = g0 == 0u ? 0u : offsets[g0 - 1];
 		const uint32_t staged_end = st.end[255];
 		const uint32_t from = max(start, staged_begin), to = min(stop, staged_end);
-		for (uint32_t pos = from + (uint32_t)tid; pos < to; pos += 256) {
-			// the first staged Gaussian whose inclusive offset exceeds pos
-			int lo = 0;
+		// Up to kDupPositions / 256 positions per thread.  First all of them find their Gaussian and ask for its
+		// record (pixel centre, conic, extents, radius: everything else follows from those), then each is finished:
+		// the records of a thread arrive together, not one wait after another.
+		constexpr int kPerThread = kDupPositions / 256;
+		uint32_t first[kPerThread], index[kPerThread];
+		float4 r0[kPerThread], r1[kPerThread], r3[kPerThread];
 #pragma unroll
-			for (int step = 128; step > 0; step >>= 1)
-				if (st.end[lo + step - 1] <= pos)
-					lo += step;
-			const uint32_t first = lo == 0 ? staged_begin : st.end[lo - 1];
-			const uint32_t t = pos - first, w = st.width[lo];
+		for (int q = 0; q < kPerThread; q++) {
+			const uint32_t pos = from + (uint32_t)tid + 256u * (uint32_t)q;
+			first[q] = 0u;
+			index[q] = 0u;
+			if (pos < to) {
+				// the first staged Gaussian whose inclusive offset exceeds pos
+				int lo = 0;
+#pragma unroll
+				for (int step = 128; step > 0; step >>= 1)
+					if (st.end[lo + step - 1] <= pos)
+						lo += step;
+				first[q] = lo == 0 ? staged_begin : st.end[lo - 1];
+				index[q] = st.index[lo];
+				const float4* rec = filing.record + 4 * (size_t)index[q];
+				r0[q] = rec[0];
+				r1[q] = rec[1];
+				r3[q] = rec[3];
+			}
+		}
+#pragma unroll
+		for (int q = 0; q < kPerThread; q++) {
+			const uint32_t pos = from + (uint32_t)tid + 256u * (uint32_t)q;
+			if (pos >= to)
+				continue;
+			const TileRect rc = tile_rect(r0[q].x, r0[q].y, __float_as_int(r3[q].z), gx, gy);
+			const uint32_t t = pos - first[q], w = max(rc.x1 - rc.x0, 1u);
 			const uint32_t row = t / w;
-			const uint32_t tile = st.origin[lo] + row * (uint32_t)gx + (t - row * w);
-			const int tx = (int)(tile % (uint32_t)gx), ty = (int)(tile / (uint32_t)gx);
+			const int tx = (int)(rc.x0 + (t - row * w)), ty = (int)(rc.y0 + row);
+			const uint32_t tile = (uint32_t)ty * (uint32_t)gx + (uint32_t)tx;
 			float2 nx;
 			float ny[8];
 			if (ndc_in_lds) {
 				nx = float2{s_ndc[2 * tx], s_ndc[2 * tx + 1]};
-				const float4 r0 = *reinterpret_cast<const float4*>(s_ndc + rows_at + 8 * ty);
-				const float4 r1 = *reinterpret_cast<const float4*>(s_ndc + rows_at + 8 * ty + 4);
-				ny[0] = r0.x; ny[1] = r0.y; ny[2] = r0.z; ny[3] = r0.w;
-				ny[4] = r1.x; ny[5] = r1.y; ny[6] = r1.z; ny[7] = r1.w;
+				const float4 y0 = *reinterpret_cast<const float4*>(s_ndc + rows_at + 8 * ty);
+				const float4 y1 = *reinterpret_cast<const float4*>(s_ndc + rows_at + 8 * ty + 4);
+				ny[0] = y0.x; ny[1] = y0.y; ny[2] = y0.z; ny[3] = y0.w;
+				ny[4] = y1.x; ny[5] = y1.y; ny[6] = y1.z; ny[7] = y1.w;
 			} else {
 				nx = tile_column_ndc(tx, filing.W);
 #pragma unroll
-				for (int q = 0; q < 4; q++) {
-					const float2 v = strip_rows_ndc(ty, q, filing.H);
-					ny[2 * q] = v.x;
-					ny[2 * q + 1] = v.y;
+				for (int h = 0; h < 4; h++) {
+					const float2 v = strip_rows_ndc(ty, h, filing.H);
+					ny[2 * h] = v.x;
+					ny[2 * h + 1] = v.y;
 				}
 			}
-			const uint32_t strips = strips_filed_for(st.tests[lo], (float)(tx * kTile), (float)(ty * kTile), nx, ny, box);
+			const StripTests tests = prepare_strip_tests(FiledGeometry{r0[q], r1[q], float2{r3[q].x, r3[q].y}}, box);
+			const uint32_t strips = strips_filed_for(tests, (float)(tx * kTile), (float)(ty * kTile), nx, ny, box);
 			keys[pos] = tile | (strips << kKeyTileBits);
-			values[pos] = st.index[lo];
+			values[pos] = index[q];
 		}
 		if (staged_end >= stop)
 			break;
