@@ -561,6 +561,8 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 	__shared__ uint32_t s_tile;
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	// asked for before anything else: needed only after the look-back, by when it has long arrived
+	const uint32_t digit_total = digit_count[tid];
 	// Tiles are handed out in arrival order, so every tile a block waits for below belongs to
 	// a block that is already running.
 	if (tid == 0)
@@ -616,29 +618,57 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 	}
 	__syncthreads();
 
-	// Thread d owns digit d: prefix over the 4 waves, publish the tile's count, look back.
+	// Thread d owns digit d: prefix over the 4 waves, publish the tile's count.
+	const size_t remaining = n - block_base;
+	const uint32_t valid = remaining < (size_t)kSortBlock ? (uint32_t)remaining : (uint32_t)kSortBlock;
+	uint32_t* const my_word = lookback + (size_t)tile * 256 + tid;
+	uint32_t count, digit_start;
 	{
-		const size_t remaining = n - block_base;
-		const uint32_t valid = remaining < (size_t)kSortBlock ? (uint32_t)remaining : (uint32_t)kSortBlock;
 		const uint32_t c0 = s_wave_hist[0][tid], c1 = s_wave_hist[1][tid], c2 = s_wave_hist[2][tid],
 		               c3 = s_wave_hist[3][tid];
 		s_wave_hist[0][tid] = 0;
 		s_wave_hist[1][tid] = c0;
 		s_wave_hist[2][tid] = c0 + c1;
 		s_wave_hist[3][tid] = c0 + c1 + c2;
-		uint32_t count = c0 + c1 + c2 + c3;
+		count = c0 + c1 + c2 + c3;
 		uint32_t total;
 		const uint32_t ex = block256_exclusive_scan_u32(count, s_scan, total);
 		s_digit_base[tid] = ex;
 		if (tid == 255)
 			count -= (uint32_t)kSortBlock - valid;  // padding is not published
+		__hip_atomic_store(my_word, count | (tile == 0 ? kFlagInclusive : kFlagAggregate), __ATOMIC_RELAXED,
+		                   __HIP_MEMORY_SCOPE_AGENT);
+		// where the digit's run starts in the whole array: the exclusive scan of the digit counts
+		uint32_t all;
+		digit_start = block256_exclusive_scan_u32(digit_total, s_scan, all);
+	}
 
-		uint32_t* my_word = lookback + (size_t)tile * 256 + tid;
+	// The tile's pairs in digit order, through LDS.  None of this needs the tiles before this one: by the time
+	// the look-back below starts, more of them have finished theirs and it has fewer words to read.
+#pragma unroll
+	for (int i = 0; i < kSortItems; i++) {
+		const size_t k = wave_base + (size_t)i * 64 + lane;
+		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : 255u;
+		const uint32_t pos = s_digit_base[d] + s_wave_hist[wave][d] + rank[i];
+		s_keys[pos] = key[i];
+		s_vals[pos] = val[i];
+	}
+	__syncthreads();
+	// every LDS read of the thread is asked for before anything needs one
+	KeyT out_key[kSortItems];
+	uint32_t out_val[kSortItems];
+#pragma unroll
+	for (int i = 0; i < kSortItems; i++) {
+		const uint32_t p = (uint32_t)i * 256 + tid;
+		const uint32_t q = p < valid ? p : 0u;
+		out_key[i] = s_keys[q];
+		out_val[i] = s_vals[q];
+	}
+
+	// Look back: the pairs of this digit in all earlier tiles.
+	{
 		uint32_t exclusive = 0;
-		if (tile == 0) {
-			__hip_atomic_store(my_word, count | kFlagInclusive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-		} else {
-			__hip_atomic_store(my_word, count | kFlagAggregate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		if (tile != 0) {
 			// Words of the tiles below t are still to be added.  Up to kLookBatch of them are requested
 			// together: walked one load at a time, the chain of tiles and not memory sets the pace of a pass.
 			uint32_t t = tile;
@@ -687,36 +717,22 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 			__hip_atomic_store(my_word, ((exclusive + count) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
 			                   __HIP_MEMORY_SCOPE_AGENT);
 		}
-		// where the digit's run starts in the whole array: the exclusive scan of the digit counts
-		uint32_t all;
-		const uint32_t digit_start = block256_exclusive_scan_u32(digit_count[tid], s_scan, all);
 		s_global_base[tid] = digit_start + exclusive;
 	}
 	__syncthreads();
 
+	size_t out_at[kSortItems];
 #pragma unroll
 	for (int i = 0; i < kSortItems; i++) {
-		const size_t k = wave_base + (size_t)i * 64 + lane;
-		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : 255u;
-		const uint32_t pos = s_digit_base[d] + s_wave_hist[wave][d] + rank[i];
-		s_keys[pos] = key[i];
-		s_vals[pos] = val[i];
-	}
-	__syncthreads();
-
-	const size_t remaining = n - block_base;
-	const uint32_t valid = remaining < (size_t)kSortBlock ? (uint32_t)remaining : (uint32_t)kSortBlock;
-#pragma unroll 4
-	for (int i = 0; i < kSortItems; i++) {
 		const uint32_t p = (uint32_t)i * 256 + tid;
-		if (p < valid) {
-			const KeyT kk = s_keys[p];
-			const uint32_t d = digit_of(kk, shift, mask);
-			const size_t dst = (size_t)s_global_base[d] + (p - s_digit_base[d]);
-			if (dst < n) {
-				keys_out[dst] = kk;
-				vals_out[dst] = s_vals[p];
-			}
+		const uint32_t d = digit_of(out_key[i], shift, mask);
+		out_at[i] = p < valid ? (size_t)s_global_base[d] + (p - s_digit_base[d]) : n;
+	}
+#pragma unroll
+	for (int i = 0; i < kSortItems; i++) {
+		if (out_at[i] < n) {
+			keys_out[out_at[i]] = out_key[i];
+			vals_out[out_at[i]] = out_val[i];
 		}
 	}
 }
