@@ -8,8 +8,9 @@ namespace rgs {
 constexpr int kMaxComposite = 64;  // most partial images one composite call can take
 
 // Jobs of one launch: kernels that run once per submodel take the submodels of a frame together, the job in
-// blockIdx.y; the arguments travel by value.  More jobs than kMaxBatch take several launches.
-constexpr int kMaxBatch = 8;
+// blockIdx.y; the arguments travel by value.  More jobs than kMaxBatch take several launches.  16 of the largest
+// job (248 bytes) stay inside the 4096 bytes a launch can carry.
+constexpr int kMaxBatch = 16;
 template <typename T>
 struct Batch {
 	T job[kMaxBatch];
@@ -393,7 +394,7 @@ struct TileRangesJob {
 void launch_tile_ranges(const TileRangesJob* jobs, int count, hipStream_t s);
 
 // blend.hip
-constexpr int kMaxBlendBatch = 8;   // jobs one launch of a blend kernel can take (their arguments travel by value)
+constexpr int kMaxBlendBatch = 16;   // jobs one launch of a blend kernel can take (their arguments travel by value)
 struct BlendBatch {
 	BlendArgs job[kMaxBlendBatch];
 	int count;
