@@ -275,7 +275,8 @@ def measure(args, config, forward_only, asides, cpu):
         # tile counts and depths of all, then 4 passes over the (depth, index) pairs of the visible
         # ones, the gathered tile counts and their scan
         "depth_order": 8.0 * P_tot + (12.0 + 4 * 16.0 + 16.0) * P_vis,
-        "duplicate_with_keys": 20.0 * P_vis + 8.0 * R_tot,
+        # per rendered Gaussian its place in the depth order, its offset and its 64-byte record in; key and index out per instance
+        "duplicate_with_keys": 72.0 * P_vis + 8.0 * R_tot,
         "sort_setup": 4.0 * R_tot,
         "sort_onesweep": 16.0 * R_tot * passes,
         "tile_ranges": 4.0 * R_tot + 16.0 * T * K,
