@@ -68,6 +68,7 @@ __device__ __forceinline__ float exp_of_exponent(float x)
 constexpr int kStripClasses = 256;
 __device__ __forceinline__ uint32_t strip_class(uint32_t filed) { return 255u - min(filed >> 3, 255u); }
 
+constexpr uint32_t kLongList = 2048;    // filed entries from which a strip's wavefront takes the highest issue priority
 constexpr int kPerLane = 1;             // list entries per lane and step (2 was measured slower)
 constexpr int kChunk = 64 * kPerLane;   // list entries a wavefront takes per step
 
@@ -261,6 +262,12 @@ __global__ __launch_bounds__(64) void blend_forward_kernel(BlendBatch batch)
 	uint64_t live = __ballot(!p.done);
 	// the entries filed for this strip, in list order: list position, bit 31 = strip inside the box
 	const uint32_t filed = a.strip_total[strip_id];
+	// A long list is a long chain of dependent steps: its wavefront goes first where it shares a SIMD with
+	// wavefronts of short lists, which lose little by waiting and would otherwise stretch the launch's longest walk.
+	if (filed > kLongList)
+		__builtin_amdgcn_s_setprio(3);
+	else if (filed > kLongList / 4)
+		__builtin_amdgcn_s_setprio(2);
 
 	if (filed != 0u && live != 0ull) {
 		const uint32_t* list = a.point_list + range.x;
