@@ -237,7 +237,7 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 	}
 }
 
-__global__ __launch_bounds__(64) void blend_forward_kernel(BlendBatch batch)
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) void blend_forward_kernel(BlendBatch batch)
 {
 	__shared__ ForwardStage st;
 
