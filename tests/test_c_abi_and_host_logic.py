@@ -79,6 +79,20 @@ def test_entry_points_reject_bad_arguments_without_launching():
     rc = lib.rgs_forward_geom(0, 3, 16, 64, 64, null, null, null, null, null, 1.0, null, null, null, null, null,
                               1.0, 1.0, 0, null, null, 0, null, null, 0)
     assert rc != 0 and b"P must be positive" in lib.rgs_last_error()
+    assert lib.rgs_covariance3d(-1, null, 1.0, null, null, null) != 0
+    assert lib.rgs_covariance3d(0, null, 1.0, null, null, null) == 0
+    # the frame entry points: layer counts outside 1..RGS_MAX_FRAME_LAYERS, null tables
+    layers = (_capi.FrameLayer * 1)()
+    view = _capi.FrameView()
+    for K in (0, _capi.MAX_FRAME_LAYERS + 1):
+        assert lib.rgs_frame_forward_geom(K, layers, ctypes.byref(view), null, null, 0) != 0
+        assert b"outside" in lib.rgs_last_error()
+        assert lib.rgs_frame_forward_raster(K, layers, ctypes.byref(view), null, 0) != 0
+        assert lib.rgs_frame_backward(K, layers, ctypes.byref(view), null, 0) != 0
+    assert lib.rgs_frame_forward_geom(1, None, ctypes.byref(view), null, null, 0) != 0
+    # the sort that allocates nothing refuses more pairs than its array holds, before it touches a device
+    assert lib.rgs_sort_pairs_static(null, null, null, null, _capi.STATIC_SORT_MAX_PAIRS + 1, 32, null) != 0
+    assert b"pairs" in lib.rgs_last_error()
 
 
 def test_rasterizer_argument_validation_matches_reference():
