@@ -521,7 +521,18 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 			for (int p = 0; p < passes; p++) {
 				const int shift = 8 * p;
 				const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
-				atomicAdd(&s_hist[p][digit_of(key[q], shift, (1u << bits) - 1u)], 1u);
+				const uint32_t d = digit_of(key[q], shift, (1u << bits) - 1u);
+				if (bits <= 2) {
+					// a digit of one or two bits: every lane would add to one of a few words, one after the
+					// other; count the lanes of each value instead
+					for (uint32_t v = 0; v < (1u << bits); v++) {
+						const uint32_t c = (uint32_t)__popcll(__ballot(d == v));
+						if ((threadIdx.x & 63) == 0 && c != 0u)
+							atomicAdd(&s_hist[p][v], c);
+					}
+				} else {
+					atomicAdd(&s_hist[p][d], 1u);
+				}
 			}
 		}
 	}
