@@ -332,7 +332,7 @@ def training_iteration(models: List["SharedGSInfo"], optimisers, part: Partition
     device = models[0].means3D.device
     table = select_straddlers(models, part.box_low, part.box_up)
     merged = merge_shared(models, table, reuse_gradients=True, append=append)
-    frame = render_frame(cam, submodels_from_shared(merged, part, device), relation, background, streams=streams)
+    frame = render_frame(cam, submodels_from_shared(merged, part, device), relation, background, streams=streams, together=True)
     loss, l1 = l1_ssim_loss(frame["render"], gt_image, lambda_dssim)
     loss.backward()
     for opt in optimisers:
@@ -427,7 +427,7 @@ def stored_training_iteration(models: List[StoredModel], optimisers, part: Parti
     shown = [m.activated() for m in models]
     table = select_straddlers(shown, part.box_low, part.box_up)
     merged = merge_shared(shown, table, reuse_gradients=True, append=all(m.spare_rows > 0 for m in models))
-    frame = render_frame(cam, submodels_from_shared(merged, part, device), relation, background, streams=streams)
+    frame = render_frame(cam, submodels_from_shared(merged, part, device), relation, background, streams=streams, together=True)
     loss, l1 = l1_ssim_loss(frame["render"], gt_image, lambda_dssim)
     loss.backward()
     for opt in optimisers:
