@@ -219,7 +219,14 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
             sub = subs[m]
             means2D = sub.means2D
             if means2D is None:
-                means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
+                if sub.means3D.requires_grad:
+                    means2D = torch.zeros_like(sub.means3D, requires_grad=True)
+                else:
+                    # nothing reads or writes the placeholder without a backward: one zero tensor serves every frame
+                    means2D = getattr(sub, "_still_means2D", None)
+                    if means2D is None or means2D.shape != sub.means3D.shape or means2D.device != sub.means3D.device:
+                        means2D = torch.zeros_like(sub.means3D)
+                        sub._still_means2D = means2D
             rasterizers.append(GaussianRasterizer(raster_settings=raster_settings(cam, sub, submodel_bg)))
             inputs.append(dict(means3D=sub.means3D, means2D=means2D, shs=sub.shs, opacities=sub.opacity, scales=sub.scales,
                                rotations=sub.rotations))
