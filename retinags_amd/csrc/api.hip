@@ -828,37 +828,6 @@ std::vector<hipStream_t> side_streams(int K, const rgs_frame_layer* layers, hipS
 	return out;
 }
 
-// Work queued on the layers' streams from here on starts after what the frame's stream holds now.
-int side_streams_wait_for(int K, const rgs_frame_layer* layers, hipStream_t frame, const char* who)
-{
-	const std::vector<hipStream_t> sides = side_streams(K, layers, frame);
-	if (sides.empty())
-		return 0;
-	hipEvent_t e = frame_event(0);
-	hipError_t rc = e ? hipEventRecord(e, frame) : hipErrorUnknown;
-	for (size_t i = 0; rc == hipSuccess && i < sides.size(); i++)
-		rc = hipStreamWaitEvent(sides[i], e, 0);
-	if (rc != hipSuccess)
-		return fail("%s: ordering the layers' streams failed: %s", who, hipGetErrorString(rc));
-	return 0;
-}
-
-// Work queued on the frame's stream from here on starts after what the layers' streams hold now.
-int wait_for_side_streams(int K, const rgs_frame_layer* layers, hipStream_t frame, const char* who)
-{
-	const std::vector<hipStream_t> sides = side_streams(K, layers, frame);
-	hipError_t rc = hipSuccess;
-	for (size_t i = 0; rc == hipSuccess && i < sides.size(); i++) {
-		hipEvent_t e = frame_event(1 + i);
-		rc = e ? hipEventRecord(e, sides[i]) : hipErrorUnknown;
-		if (rc == hipSuccess)
-			rc = hipStreamWaitEvent(frame, e, 0);
-	}
-	if (rc != hipSuccess)
-		return fail("%s: ordering the layers' streams failed: %s", who, hipGetErrorString(rc));
-	return 0;
-}
-
 int check_backward_pointers(const char* who, int P, int R, int width, int height, const float* background,
                             const float* means3D, const float* shs, const float* colors_precomp, const float* alphas,
                             const float* scales, const float* rotations, const float* cov3D_precomp, const float* viewmatrix,

@@ -137,13 +137,12 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
 
 
 def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0, debug: bool = False,
-                   instance_bound: Optional[int] = None, clear_gradients: bool = False):
+                   instance_bound: Optional[int] = None):
     """Enqueues the geometry stage of a submodel's forward on the current stream without waiting
     for its instance count; hand the result to render_submodel(..., started=...)."""
     rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, debug))
     geometry = rasterizer.enqueue_geometry(means3D=sub.means3D, opacities=sub.opacity, shs=sub.shs,
-                                           scales=sub.scales, rotations=sub.rotations, instance_bound=instance_bound,
-                                           clear_gradients=clear_gradients)
+                                           scales=sub.scales, rotations=sub.rotations, instance_bound=instance_bound)
     return rasterizer, geometry
 
 

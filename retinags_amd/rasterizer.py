@@ -83,7 +83,7 @@ class GeometryStage:
     GaussianRasterizer.enqueue_geometry, consumed once by GaussianRasterizer.forward."""
 
     __slots__ = ("device", "stream", "P", "H", "W", "tensors", "settings", "radii", "geomBuffer", "geom_bytes",
-                 "count", "event", "source", "used", "instance_bound", "_instances", "cleared")
+                 "count", "event", "source", "used", "instance_bound", "_instances")
 
     def matches(self, means3D, raster_settings) -> bool:
         return (self.source == (means3D.data_ptr(), int(means3D.shape[0])) and self.settings is raster_settings
@@ -145,7 +145,6 @@ def _forward_geometry(bg, means3D, colors_precomp, opacities, scales, rotations,
     st.count = None
     st.instance_bound = None
     st._instances = None
-    st.cleared = None
     byte = dict(dtype=torch.uint8, device=device)
     st.radii = torch.empty((st.P,), dtype=torch.int32, device=device)
     names = ("means3D", "colors_precomp", "opacities", "scales", "rotations", "cov3Ds_precomp", "sh", "bg",
@@ -692,7 +691,7 @@ class GaussianRasterizer(nn.Module):
                                    raster_settings, geometry)
 
     def enqueue_geometry(self, means3D, opacities, shs=None, colors_precomp=None, scales=None, rotations=None,
-                         cov3D_precomp=None, instance_bound=None, clear_gradients=False) -> GeometryStage:
+                         cov3D_precomp=None, instance_bound=None) -> GeometryStage:
         """Starts the first half of a forward call (preprocess and instance count) on the current
         stream and returns without waiting for it.  No counterpart in the reference, whose forward
         always blocks on the count (K/cuda_rasterizer_hgs/rasterizer_impl.cu:287): a caller that
@@ -704,12 +703,7 @@ class GaussianRasterizer(nn.Module):
         does not wait for the count at all (the reference grows its buffers on demand instead,
         K/rasterize_points.cu:27-33).  The caller must then ask stage.within_bound() after the
         forward has been issued (at the end of the iteration is early enough) and, if it is
-        false, repeat the forward with a bound of at least stage.instances().
-
-        clear_gradients: also allocates and clears, on this stream and right away, the gradient tensors the
-        backward of this call will fill (only rendered Gaussians get rows written; the rest must be zero):
-        pure memory traffic that then runs beside the other layers' short kernels instead of behind the
-        blend.  Used by rasterize_frame; a plain forward(..., geometry=stage) clears its own."""
+        false, repeat the forward with a bound of at least stage.instances()."""
         rs = self.raster_settings
         shs, colors_precomp, scales, rotations, cov3D_precomp = self._check_and_fill(
             shs, colors_precomp, scales, rotations, cov3D_precomp)
@@ -719,9 +713,6 @@ class GaussianRasterizer(nn.Module):
                 rs.viewmatrix, rs.projmatrix, rs.projmatrix_inv, rs.range_low, rs.range_up, rs.tanfovx, rs.tanfovy,
                 rs.image_height, rs.image_width, shs, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, wait=False)
         stage.settings = rs
-        if clear_gradients and stage.P > 0:
-            M = int(shs.shape[1]) if shs.numel() != 0 else 0
-            stage.cleared = _gradient_outputs(stage.P, M, scales.numel() != 0, means3D.device, torch.zeros)
         if instance_bound is not None:
             if int(instance_bound) < 0:
                 raise ValueError("instance_bound must not be negative")
