@@ -410,15 +410,17 @@ def test_a_sort_that_gives_up_is_reported_by_the_next_call():
     assert _capi.lib.rgs_sort_fault(stream) == 0
 
 
-@pytest.mark.parametrize("with_streams", [False, True])
-def test_frame_rendered_together_matches_one_call_per_submodel(with_streams):
+@pytest.mark.parametrize("with_streams,bvh_depth", [(False, 2), (True, 2), (False, 5), (True, 5)])
+def test_frame_rendered_together_matches_one_call_per_submodel(with_streams, bvh_depth):
     """render_frame(together=True) sends the related submodels through rgs_frame_forward_raster /
     rgs_frame_backward (one blend launch per direction for all of them): images bit for bit those of one
-    call per submodel, gradients equal up to the order of the atomic sums."""
+    call per submodel, gradients equal up to the order of the atomic sums.  With 32 submodels a frame has more
+    layers than one launch takes (16), so every stage goes in two launches."""
     from retinags_amd.harness import partition, pipeline
     scene, cam, _ = scenes.make_config("C1", shrink=300, resolution_scale=0.25)
-    part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
+    part = partition.partition_scene(scene["xyz"], scene["scales"], bvh_depth)
     rel = partition.relation_vector(part, cam)
+    assert bvh_depth < 5 or int((rel >= 0).sum()) > 16
     H, W = cam.image_height, cam.image_width
     g = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(2)) * 1e-2).to(DEV)
     bg = torch.tensor([0.3, 0.1, 0.2], device=DEV)
