@@ -260,7 +260,7 @@ static inline size_t ndc_table_floats(int gx, int gy)
 }
 constexpr size_t kNdcTableMaxFloats = 8192;  // larger grids compute the coordinates per instance
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 5))) void duplicate_with_keys_kernel(Batch<DuplicateJob> batch, int gx, int gy, int ndc_in_lds)
+__global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<DuplicateJob> batch, int gx, int gy, int ndc_in_lds)
 {
 	__shared__ DuplicateStage st;
 	__shared__ uint32_t s_first;

@@ -140,6 +140,21 @@ __device__ __forceinline__ uint32_t strips_filed_for(const StripTests& t, float 
 	}
 	const float lov[3] = {box.lo.x, box.lo.y, box.lo.z}, hiv[3] = {box.hi.x, box.hi.y, box.hi.z};
 
+	// The same box test for the whole tile first (rows from the first of strip 0 to the last of strip 3): a product
+	// with a constant is monotone in the row coordinate, so the tile's range contains every strip's, and a tile that
+	// lies inside (outside) the box has all four strips inside (outside) by the very comparisons made below.  Most
+	// Gaussians are far from their submodel's faces, and three of the four evaluations go.
+	bool tile_inside = true, tile_outside = false;
+#pragma unroll
+	for (int k = 0; k < 3; k++) {
+		const float q0 = t.B[k] * ny[0], q1 = t.B[k] * ny[7];
+		const float pmin = xlo[k] + fminf(q0, q1), pmax = xhi[k] + fmaxf(q0, q1);
+		tile_inside = tile_inside && (pmin > lov[k] + t.tol[k]) && (pmax < hiv[k] - t.tol[k]);
+		tile_outside = tile_outside || (pmax < lov[k] - t.tol[k]) || (pmin > hiv[k] + t.tol[k]);
+	}
+	if (tile_outside)
+		return 0u;
+
 	uint32_t bits = 0;
 #pragma unroll
 	for (int s = 0; s < 4; s++) {
@@ -170,12 +185,14 @@ __device__ __forceinline__ uint32_t strips_filed_for(const StripTests& t, float 
 				continue;
 		}
 		bool inside = true, outside = false;
+		if (!tile_inside) {
 #pragma unroll
-		for (int k = 0; k < 3; k++) {
-			const float q0 = t.B[k] * ny[2 * s], q1 = t.B[k] * ny[2 * s + 1];
-			const float pmin = xlo[k] + fminf(q0, q1), pmax = xhi[k] + fmaxf(q0, q1);
-			inside = inside && (pmin > lov[k] + t.tol[k]) && (pmax < hiv[k] - t.tol[k]);
-			outside = outside || (pmax < lov[k] - t.tol[k]) || (pmin > hiv[k] + t.tol[k]);
+			for (int k = 0; k < 3; k++) {
+				const float q0 = t.B[k] * ny[2 * s], q1 = t.B[k] * ny[2 * s + 1];
+				const float pmin = xlo[k] + fminf(q0, q1), pmax = xhi[k] + fmaxf(q0, q1);
+				inside = inside && (pmin > lov[k] + t.tol[k]) && (pmax < hiv[k] - t.tol[k]);
+				outside = outside || (pmax < lov[k] - t.tol[k]) || (pmin > hiv[k] + t.tol[k]);
+			}
 		}
 		// a NaN can set neither flag, which leaves the decision to the per-pixel test
 		if (outside)
