@@ -603,7 +603,6 @@ class _RasterizeFrame(torch.autograd.Function):
         if live:
             with torch.cuda.device(device):
                 check(lib.rgs_frame_backward(live, arr, C.byref(view), C.c_void_p(main), int(bool(rs0.debug))))
-        ctx.meta = None
         flat = []
         for k in range(K):
             (colors_precomp, means3D, scales, rotations, cov3Ds, radii, sh) = saved[11 * k:11 * k + 7]

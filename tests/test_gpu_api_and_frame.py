@@ -465,6 +465,10 @@ def test_rasterize_frame_with_an_empty_layer_and_without_stages():
     want = rz(**{k: (v.detach() if k == "means3D" else v) for k, v in full.items()})
     assert torch.equal(c0, want[0]) and torch.equal(r0, want[1]) and torch.equal(d0, want[2]) and torch.equal(a0, want[3])
     assert r1.numel() == 0 and float(c1.abs().max()) == 0.0 and float(a1.abs().max()) == 0.0
-    (c0.sum() + c1.sum()).backward()
+    (c0.sum() + c1.sum()).backward(retain_graph=True)
     assert full["means3D"].grad is not None and float(full["means3D"].grad.abs().sum()) > 0
     assert empty["means3D"].grad is not None and empty["means3D"].grad.shape == (0, 3)
+    # a second backward of the same graph adds the same gradient again
+    once = full["means3D"].grad.clone()
+    (c0.sum() + c1.sum()).backward()
+    assert rel_l2(full["means3D"].grad.cpu().numpy(), 2.0 * once.cpu().numpy()) <= 1e-5
