@@ -86,6 +86,44 @@ def test_precomputed_colours_and_covariance_modes():
     assert rel_l2(opa.grad.cpu().numpy(), want["opacity"]) <= GRAD_TOL
 
 
+def test_frame_layers_with_different_input_modes():
+    """rasterize_frame with one layer given SHs and scale/rotation and one given precomputed colours and 3D
+    covariances: each layer's images and gradients are those of a call of its own."""
+    from retinags_amd import GaussianRasterizer
+    from retinags_amd.rasterizer import rasterize_frame
+    scene, cam, low, up = _small_inputs()
+    s = oracle_settings(cam, low, up, torch.tensor([0.2, 0.1, 0.4]))
+    st = orc.forward(s, np32(scene["xyz"]), np32(scene["opacity"]), shs=np32(scene["shs"]),
+                     scales=np32(scene["scales"]), rotations=np32(scene["rotations"]))
+    rz = GaussianRasterizer(_settings(s))
+    H, W = cam.image_height, cam.image_width
+    g = (torch.randn(2, 3, H, W, generator=torch.Generator().manual_seed(4)) * 1e-2).to(DEV)
+
+    def inputs():
+        leaf = lambda t: t.to(DEV).clone().requires_grad_(True)
+        a = dict(means3D=leaf(scene["xyz"]), means2D=torch.zeros(scene["xyz"].shape[0], 3, device=DEV),
+                 opacities=leaf(scene["opacity"]), shs=leaf(scene["shs"]), scales=leaf(scene["scales"]),
+                 rotations=leaf(scene["rotations"]))
+        b = dict(means3D=leaf(scene["xyz"]), means2D=torch.zeros(scene["xyz"].shape[0], 3, device=DEV),
+                 opacities=leaf(scene["opacity"]), colors_precomp=leaf(torch.from_numpy(st.rgb.copy())),
+                 cov3D_precomp=leaf(torch.from_numpy(st.cov3D.copy())))
+        return a, b
+
+    a, b = inputs()
+    outs = rasterize_frame([rz, rz], [a, b])
+    torch.autograd.backward([outs[0][0], outs[1][0]], [g[0], g[1]])
+    a1, b1 = inputs()
+    alone = [rz(**a1), rz(**b1)]
+    torch.autograd.backward([alone[0][0], alone[1][0]], [g[0], g[1]])
+    for got, want in zip(outs, alone):
+        for x, y in zip(got, want):
+            assert torch.equal(x, y)
+    for together, apart in ((a, a1), (b, b1)):
+        for name in together:
+            if together[name].requires_grad:
+                assert rel_l2(together[name].grad.cpu().numpy(), apart[name].grad.cpu().numpy()) <= 1e-5, name
+
+
 def test_empty_input_and_nothing_visible():
     from retinags_amd import GaussianRasterizer
     scene, cam, low, up = _small_inputs(64)
