@@ -182,7 +182,7 @@ struct Carver {
 
 // Scratch of the depth sort of the Gaussians, inside the geometry workspace.
 struct OrderScratch {
-	size_t keys_a, keys_b, vals_b, tiles_in_order, sort_temp, scan_temp, total;
+	size_t keys_a, keys_b, vals_b, tiles_in_order, sort_temp, scan_temp, dup_first, total;
 };
 
 OrderScratch order_scratch(size_t P)
@@ -195,6 +195,7 @@ OrderScratch order_scratch(size_t P)
 	o.tiles_in_order = c.take(4 * P);
 	o.sort_temp = c.take(4 * rgs::sort_temp_words(P));
 	o.scan_temp = c.take(4 * rgs::scan_temp_words(P));
+	o.dup_first = c.take(4 * rgs::dup_first_words(P));
 	o.total = c.cursor;
 	return o;
 }
@@ -527,6 +528,7 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 		d.tiles_in_order = at<uint32_t>(scratch, o.tiles_in_order);
 		d.offsets_in_order = at<uint32_t>(ws, off[RGS_GEOM_POINT_OFFSETS]);
 		d.sort_temp = at<uint32_t>(scratch, o.sort_temp); d.scan_temp = at<uint32_t>(scratch, o.scan_temp);
+		d.dup_first = at<uint32_t>(scratch, o.dup_first);
 	}
 	rgs::launch_preprocess_forward(pre.data(), K, s);
 	RGS_STAGE("preprocess");
@@ -701,6 +703,8 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 		d.visible_count = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
 		d.order = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_DEPTH_ORDER]);
 		d.offsets = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_POINT_OFFSETS]);
+		d.total = at<uint32_t>(c.geom_ws, goff[RGS_GEOM_TOTAL]);
+		d.first_of_block = at<uint32_t>(at<char>(c.geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).dup_first);
 		d.filing.record = a.record;
 		d.filing.projinv = projmatrix_inv; d.filing.range_low = c.range_low; d.filing.range_up = c.range_up;
 		d.filing.tanfovx = tan_fovx; d.filing.tanfovy = tan_fovy;

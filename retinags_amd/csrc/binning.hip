@@ -111,6 +111,8 @@ struct BlockInclusiveJob {
 	size_t n;
 	const uint32_t* n_device;
 	uint32_t* out;
+	uint32_t* first_of_block;  // may be null; see DuplicateJob
+	uint32_t first_of_block_words;
 };
 
 __global__ __launch_bounds__(256) void block_inclusive_scan_kernel(Batch<BlockInclusiveJob> batch)
@@ -129,8 +131,17 @@ __global__ __launch_bounds__(256) void block_inclusive_scan_kernel(Batch<BlockIn
 	const uint32_t v = i < n ? in[i] : 0u;
 	uint32_t total;
 	const uint32_t ex = block256_exclusive_scan_u32(v, lds, total);
-	if (i < n)
-		out[i] = block_base[blockIdx.x] + ex + v;
+	if (i < n) {
+		const uint32_t begin = block_base[blockIdx.x] + ex, end = begin + v;
+		out[i] = end;
+		if (j.first_of_block) {
+			// entry i covers positions [begin, end): it is where every workgroup of the key duplication starts whose
+			// first position, a multiple of kDupPositions, lies among them
+			for (uint32_t b = (begin + (uint32_t)kDupPositions - 1u) / (uint32_t)kDupPositions;
+			     b < j.first_of_block_words && (uint64_t)b * (uint64_t)kDupPositions < (uint64_t)end; b++)
+				j.first_of_block[b] = (uint32_t)i;
+		}
+	}
 }
 
 size_t scan_temp_words(size_t n)
@@ -147,7 +158,7 @@ static void inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, const uin
 	scan.job[0] = BlockScanJob{temp, nb, n_device, nullptr, nullptr, nullptr, nullptr};
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan);
 	Batch<BlockInclusiveJob> inc = {};
-	inc.job[0] = BlockInclusiveJob{in, temp, n, n_device, out};
+	inc.job[0] = BlockInclusiveJob{in, temp, n, n_device, out, nullptr, 0u};
 	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, inc);
 }
 
@@ -246,8 +257,6 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> ba
 // tile in the key: the sort only looks at the tile bits, so they travel with the instance for free.
 // `order` is the output of a sort: should that sort ever have given up, its entries may be anything, so
 // they are clamped to the P Gaussians there are (the tile ranges then stay empty and nothing reads the result).
-constexpr int kDupPositions = 1024;
-
 struct DuplicateStage {
 	uint32_t end[256];     // inclusive offset of each staged Gaussian
 	uint32_t index[256];
@@ -281,9 +290,11 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	for (size_t w = (size_t)blockIdx.x * 256 + tid; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;
 	const uint32_t n = min(*visible_count, P);
+	const uint32_t total = *job.total;
+	const bool listed = blockIdx.x < (uint32_t)dup_first_words((size_t)P);
+	const uint32_t listed_first = listed ? job.first_of_block[blockIdx.x] : 0u;  // only meaningful below `total`
 	if (n == 0u)
 		return;
-	const uint32_t total = offsets[n - 1];
 	const uint32_t limit = min(total, capacity);  // positions beyond the room the caller gave are dropped
 	const uint32_t start = blockIdx.x * (uint32_t)kDupPositions;
 	if (start >= limit)
@@ -303,8 +314,11 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 			s_ndc[rows_at + 2 * r + 1] = v.y;
 		}
 	}
-	// the first Gaussian whose inclusive offset exceeds `start`: 64-ary search by the first wavefront
-	if (tid < 64) {
+	// the first Gaussian whose inclusive offset exceeds `start`: from the table, or by a 64-ary search of the first wavefront
+	if (listed) {
+		if (tid == 0)
+			s_first = min(listed_first, n - 1u);
+	} else if (tid < 64) {
 		uint32_t lo = 0, hi = n;  // the answer lies in [lo, hi]
 		while (lo < hi) {
 			const uint32_t step = (hi - lo + 63u) / 64u;
@@ -415,7 +429,8 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)
 			// 4 passes: the sorted pairs end up in the first buffer pair again
 			sorts[k] = SortJob<uint32_t>{j.keys_a, j.keys_b, j.order, j.vals_b, (size_t)j.P, j.visible_count, j.sort_temp, nullptr, 0};
 			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + 255) / 256, j.visible_count, nullptr, nullptr, nullptr, nullptr};
-			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order};
+			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order, j.dup_first,
+			                               (uint32_t)dup_first_words((size_t)j.P)};
 		}
 		const dim3 grid((unsigned)((max_p + 255) / 256), (unsigned)nj);
 		hipLaunchKernelGGL(depth_pairs_kernel, grid, dim3(256), 0, s, b);

@@ -19,7 +19,9 @@
 // the positions of the one after that are already in flight while the current chunk is
 // processed).  With many small Gaussians a tile's list runs to tens of thousands of entries of
 // which a strip needs a few thousand at most.  The backward walks the same filed lists, up to the
-// last entry any pixel blended.
+// last entry any pixel blended.  The forward narrows a step further: of each chunk it packs, per
+// 8-pixel-wide half of the strip, the entries whose ellipse reaches that half, and the lanes of
+// each half walk their own packed entries side by side (as many steps as the longer of the two).
 //
 // Inside the walk, alpha >= 1/255 needs power >= -ln(255 * opacity); that floor (minus a margin) is
 // stored with the Gaussian, and a group of four entries is skipped with one ballot when no live
@@ -201,43 +203,61 @@ struct ForwardPixel {
 };
 
 struct ForwardStage {  // one per workgroup (a single wavefront)
-	float4 geom[kChunk + 3];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
-	float4 conic[kChunk + 3];  // conic xx, xy, yy, opacity
-	float4 cd[kChunk];         // r, g, b, view depth
-	uint32_t position[kChunk]; // 1-based position in the tile list
+	// The chunk's entries once per 8-pixel-wide half of the strip they can reach, each half's packed to the front:
+	float4 geom[2][kChunk + 3];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
+	float4 conic[2][kChunk + 3];  // conic xx, xy, yy, opacity
+	uint8_t entry[2][kChunk + 4]; // which entry of the chunk a packed slot holds
+	// and once per entry of the chunk, what only a blended sample reads:
+	float4 cd[kChunk];            // r, g, b, view depth
+	uint32_t position[kChunk];    // 1-based position in the tile list
 };
 
-// `filed_index` is the entry's 1-based number among those filed for the strip.
+// `first` is the number of entries filed for the strip ahead of the chunk; `slot` is the packed slot in the
+// pixel's half.
 __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, float power, const float4 g,
-                                              const float4 co, const ForwardStage& st, int slot, uint32_t filed_index,
+                                              const float4 co, const ForwardStage& st, int half, int slot, uint32_t first,
                                               const PixelRay& ray, const BoxFrame& box)
 {
 	candidate = candidate && !p.done;
 	if (__ballot(candidate) == 0ull)
 		return;
-	const float clip_w = wave_uniform(g.w);  // NaN: the whole strip is inside the box
 	if (candidate) {
+		const float clip_w = g.w;  // NaN: the whole strip is inside the box
 		const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
 		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, box))) {
 			const float test_T = p.T * (1 - alpha);
 			if (test_T < 0.0001f) {
 				p.done = true;
 			} else {
-				const float4 cd = st.cd[slot];
+				const uint32_t entry = st.entry[half][slot];
+				const float4 cd = st.cd[entry];
 				p.C0 += cd.x * alpha * p.T;
 				p.C1 += cd.y * alpha * p.T;
 				p.C2 += cd.z * alpha * p.T;
 				p.weight += alpha * p.T;
 				p.D += cd.w * alpha * p.T;
 				p.T = test_T;
-				p.last_contributor = st.position[slot];
-				p.last_filed = filed_index;
+				p.last_contributor = st.position[entry];
+				p.last_filed = first + entry + 1u;
 			}
 		}
 	}
 }
 
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) void blend_forward_kernel(BlendBatch batch)
+// Number of set bits of a ballot below the calling lane.
+__device__ __forceinline__ uint32_t lanes_below(uint64_t ballot)
+{
+	return __builtin_amdgcn_mbcnt_hi((uint32_t)(ballot >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)ballot, 0u));
+}
+
+// Whether the ellipse power >= floor of a filed entry can reach pixel columns [xa, xa + 7] (x relative to the
+// Gaussian's centre: dxa = centre - xa).  `reach` is the ellipse's half extent in x, with room for rounding.
+__device__ __forceinline__ bool reaches_columns(float dxa, float reach)
+{
+	return !(dxa + reach < 0.f) && !(dxa - reach > 7.f);
+}
+
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void blend_forward_kernel(BlendBatch batch)
 {
 	__shared__ ForwardStage st;
 
@@ -283,20 +303,61 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) void
 		LoadedRecord cur = load_record(a, pos_cur != kNone ? list[pos_cur & kPosition] : 0u, pos_cur != kNone);
 		uint32_t id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
 
+		const int half = (lane >> 3) & 1;
+		const float x0 = (float)(tx * kTile), ya = (float)(ty * kTile + wave * 4);
 		for (uint32_t first = 0; first < filed && live != 0ull; first += 64) {
 			const int count = (int)min(filed - first, 64u);
+			// Which 8-pixel-wide halves of the strip the entry's ellipse power >= floor can reach: its half extent
+			// in x is sqrt(limit c / (a c - b^2)) with limit = -2 floor, here with room for the rounding of the
+			// exponent the pixels evaluate (relative to its largest terms over the strip) and of the determinant.
+			// A half that cannot be reached holds no pixel that would pass the floor test below, so leaving the
+			// entry out of that half's walk changes no result.
+			bool left = false, right = false;
+			if (lane < count) {
+				const float ca = cur.conic.x, cb = cur.conic.y, cc = cur.conic.z;
+				const float dxa = cur.geom.x - x0, dya = cur.geom.y - ya;
+				const float limit = -2.f * cur.geom.z;
+				const float far_x = fmaxf(fabsf(dxa), fabsf(dxa - 15.f)), far_y = fmaxf(fabsf(dya), fabsf(dya - 3.f));
+				const float allowed = limit + (1e-3f + 1e-4f * limit + 1e-5f * (ca * far_x * far_x + cc * far_y * far_y));
+				const float det = ca * cc - cb * cb - 1e-6f * ca * cc;
+				float reach = INFINITY;
+				if ((ca > 0.f) && (cc > 0.f) && (det > 0.f))
+					reach = __builtin_sqrtf(allowed * cc / det) * 1.001f + 0.01f;
+				if (!(reach == reach))
+					reach = INFINITY;
+				left = reaches_columns(dxa, reach);
+				right = reaches_columns(dxa - 8.f, reach);
+			}
+			const uint64_t in_left = __ballot(left), in_right = __ballot(right);
+			const int n_left = __popcll(in_left), n_right = __popcll(in_right);
+			const int steps = max(n_left, n_right), padded = (steps + 3) & ~3;
 			if (lane < count) {
 				float4 g = cur.geom;
 				if (pos_cur & 0x80000000u)
 					g.w = __int_as_float(0x7FC00000);  // the strip lies inside the box: no per-pixel test
-				st.geom[lane] = g;
-				st.conic[lane] = cur.conic;
 				st.cd[lane] = cur.cd;
 				st.position[lane] = (pos_cur & kPosition) + 1u;
+				if (left) {
+					const uint32_t r = lanes_below(in_left);
+					st.geom[0][r] = g;
+					st.conic[0][r] = cur.conic;
+					st.entry[0][r] = (uint8_t)lane;
+				}
+				if (right) {
+					const uint32_t r = lanes_below(in_right);
+					st.geom[1][r] = g;
+					st.conic[1][r] = cur.conic;
+					st.entry[1][r] = (uint8_t)lane;
+				}
 			}
-			if (lane < 3) {  // pad to a multiple of four with entries that never pass the floor test
-				st.geom[count + lane] = float4{0.f, 0.f, INFINITY, 0.f};
-				st.conic[count + lane] = float4{0.f, 0.f, 0.f, 0.f};
+			// both halves are walked for `padded` slots: the rest get entries that never pass the floor test
+			if (lane >= n_left && lane < padded) {
+				st.geom[0][lane] = float4{0.f, 0.f, INFINITY, 0.f};
+				st.conic[0][lane] = float4{0.f, 0.f, 0.f, 0.f};
+			}
+			if (lane >= n_right && lane < padded) {
+				st.geom[1][lane] = float4{0.f, 0.f, INFINITY, 0.f};
+				st.conic[1][lane] = float4{0.f, 0.f, 0.f, 0.f};
 			}
 			__builtin_amdgcn_wave_barrier();
 			// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
@@ -307,9 +368,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) void
 			const uint32_t e3 = first + 192 + (uint32_t)lane;
 			pos_after = e3 < filed ? filed_list[e3] : kNone;
 
-			for (int k = 0; k < count && live != 0ull; k += 4) {
-				const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
-				const float4 c0 = st.conic[k], c1 = st.conic[k + 1], c2 = st.conic[k + 2], c3 = st.conic[k + 3];
+			const float4* geom = st.geom[half];
+			const float4* conic = st.conic[half];
+			for (int k = 0; k < steps && live != 0ull; k += 4) {
+				const float4 g0 = geom[k], g1 = geom[k + 1], g2 = geom[k + 2], g3 = geom[k + 3];
+				const float4 c0 = conic[k], c1 = conic[k + 1], c2 = conic[k + 2], c3 = conic[k + 3];
 				float2 d;
 				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
 				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
@@ -318,11 +381,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(7, 7))) void
 				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
 				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
 					continue;
-				const uint32_t f = first + (uint32_t)k;
-				forward_visit(p, q0, w0, g0, c0, st, k, f + 1, ray, box);
-				forward_visit(p, q1, w1, g1, c1, st, k + 1, f + 2, ray, box);
-				forward_visit(p, q2, w2, g2, c2, st, k + 2, f + 3, ray, box);
-				forward_visit(p, q3, w3, g3, c3, st, k + 3, f + 4, ray, box);
+				forward_visit(p, q0, w0, g0, c0, st, half, k, first, ray, box);
+				forward_visit(p, q1, w1, g1, c1, st, half, k + 1, first, ray, box);
+				forward_visit(p, q2, w2, g2, c2, st, half, k + 2, first, ray, box);
+				forward_visit(p, q3, w3, g3, c3, st, half, k + 3, first, ray, box);
 				live = __ballot(!p.done);
 			}
 			__builtin_amdgcn_wave_barrier();

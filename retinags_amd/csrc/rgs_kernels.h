@@ -321,15 +321,24 @@ struct DepthOrderJob {
 	uint32_t* offsets_in_order;
 	uint32_t* sort_temp;
 	uint32_t* scan_temp;
+	uint32_t* dup_first;       // dup_first_words(P) words: see launch_duplicate_with_keys
 };
 void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 // Also sets clear[0..clear_words) to zero (the scratch of the sort that follows).  Instances whose
 // position is `capacity` or more are not written.
+// Output positions a workgroup of the key duplication writes, and the table that tells each such workgroup at
+// which Gaussian (of the depth order) its positions begin: entry b = the Gaussian whose instances include position
+// b * kDupPositions.  The scan that produces the offsets fills it; it has room for dup_first_words(P) workgroups,
+// those beyond (more than 16 instances per Gaussian on average) search the offsets instead.
+constexpr int kDupPositions = 1024;
+constexpr size_t dup_first_words(size_t P) { return P / 64 + 2; }
 struct DuplicateJob {
 	int P;
 	const uint32_t* visible_count;
 	const uint32_t* order;
 	const uint32_t* offsets;   // inclusive, in depth order
+	const uint32_t* total;     // the last of them
+	const uint32_t* first_of_block;  // dup_first_words(P) words
 	FilingArgs filing;
 	uint32_t* keys;
 	uint32_t* values;
