@@ -4,7 +4,7 @@
  * Every entry point takes plain device pointers, sizes and a HIP stream (as void*;
  * NULL = the default stream).  The library never allocates or frees device memory:
  * the caller sizes the three workspaces with the rgs_*_bytes() functions and owns
- * them.  All float data is fp32, contiguous, on the device the stream belongs to.
+ * them; a workspace starts at a multiple of 16 bytes.  All float data is fp32, contiguous, on the device the stream belongs to.
  * Matrices are 16 floats in the reference's layout (row-vector convention, i.e.
  * element [4*c + r] is row r, column c of the usual column-vector matrix).
  *

@@ -240,7 +240,7 @@ BinningPhysical binning_physical(size_t R)
 	b.vals_b = c.take(4 * R);
 	b.temp = c.take(4 * rgs::sort_temp_words(R));
 	b.strip_lists = c.take(16 * R);
-	b.file_tail = c.take(16 * ((R + 255) / 256));
+	b.file_tail = c.take(16 * ((R + rgs::kFileGroup - 1) / rgs::kFileGroup));
 	b.total = c.cursor;
 	return b;
 }
@@ -676,6 +676,8 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 		RGS_REQUIRE(R < 0x40000000, "%s: %d (Gaussian, tile) instances exceed the 2^30 limit of the sort", who, R);
 		RGS_REQUIRE(c.background && c.range_low && c.range_up && c.geom_ws && c.image_ws, "%s: null pointer", who);
 		RGS_REQUIRE(R == 0 || c.binning_ws, "%s: null binning workspace", who);
+		RGS_REQUIRE((reinterpret_cast<uintptr_t>(c.binning_ws) & 15) == 0 && (reinterpret_cast<uintptr_t>(c.image_ws) & 15) == 0,
+		            "%s: workspaces must be 16-byte aligned", who);
 		RGS_REQUIRE(c.geom_bytes >= rgs_geom_bytes(P), "%s: geometry workspace too small", who);
 		RGS_REQUIRE(R == 0 || c.binning_bytes >= rgs_binning_bytes(R), "%s: binning workspace too small", who);
 		RGS_REQUIRE(c.image_bytes >= rgs_image_bytes(width, height), "%s: image workspace too small", who);

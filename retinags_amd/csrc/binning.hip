@@ -861,12 +861,13 @@ void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 // The status words (may be null) are those of the two sorts: if either reported a failure the
 // ranges stay empty, so no later stage walks an unsorted list, and *fault (host memory that the
 // device can write, may be null) is set for the host to find.  The keys carry strip bits above the
-// tile (key_strips); per workgroup of kFileBlock keys, file_tail (may be null) receives how many keys
-// of the tile of its last key have each of the four "filed" bits set, which is what the kernel that
-// places the entries in their strips' lists needs from the workgroups ahead of its own.
+// tile (key_strips); per workgroup of kFileGroup keys (four neighbouring keys per thread), file_tail
+// (may be null) receives how many keys of the tile of its last key have each of the four "filed" bits
+// set, which is what the kernel that places the entries in their strips' lists needs from the
+// workgroups ahead of its own.
 __global__ __launch_bounds__(kFileBlock) void tile_ranges_kernel(Batch<TileRangesJob> batch)
 {
-	__shared__ uint32_t s_tail[4][4];  // [wave][strip]
+	__shared__ uint2 s_tail[4];  // per wave, the four strips' counts packed 16 bits each
 	__shared__ uint32_t s_last_tile;
 	const TileRangesJob& j = batch.job[blockIdx.y];
 	const uint32_t* __restrict__ keys = j.keys;
@@ -877,56 +878,70 @@ __global__ __launch_bounds__(kFileBlock) void tile_ranges_kernel(Batch<TileRange
 	const uint32_t* __restrict__ order_status = j.order_status;
 	uint32_t* __restrict__ fault = j.fault;
 	uint4* __restrict__ file_tail = j.file_tail;
-	if ((size_t)blockIdx.x * kFileBlock >= j.n)
+	const size_t first = (size_t)blockIdx.x * kFileGroup;
+	if (first >= j.n)
 		return;  // the launch is sized for the job with the most keys
-	const size_t idx = (size_t)blockIdx.x * kFileBlock + threadIdx.x;
 	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u)) {
-		if (idx == 0 && fault)
+		if (blockIdx.x == 0 && threadIdx.x == 0 && fault)
 			__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 		return;
 	}
 	if (n_device)
 		n = min(n, (size_t)*n_device);  // launched for an upper bound
-	if ((size_t)blockIdx.x * kFileBlock >= n)
+	if (first >= n)
 		return;
-	const bool valid = idx < n;
-	const uint32_t key = valid ? keys[idx] : 0u;
-	const uint32_t cur = key_tile(key);
-	if (valid) {
-		if (idx == 0) {
-			ranges[cur].x = 0;
-		} else {
-			const uint32_t prev = key_tile(keys[idx - 1]);
-			if (cur != prev) {
+	const size_t idx0 = first + 4 * (size_t)threadIdx.x;
+	uint32_t key[4] = {0u, 0u, 0u, 0u};
+	if (idx0 + 3 < n) {
+		const uint4 k4 = *reinterpret_cast<const uint4*>(keys + idx0);
+		key[0] = k4.x; key[1] = k4.y; key[2] = k4.z; key[3] = k4.w;
+	} else {
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+			if (idx0 + q < n)
+				key[q] = keys[idx0 + q];
+	}
+	uint32_t prev = (idx0 > 0 && idx0 < n) ? key_tile(keys[idx0 - 1]) : 0u;
+	const size_t last = min(n, first + kFileGroup) - 1;
+#pragma unroll
+	for (int q = 0; q < 4; q++) {
+		const size_t idx = idx0 + q;
+		const uint32_t cur = key_tile(key[q]);
+		if (idx < n) {
+			if (idx == 0) {
+				ranges[cur].x = 0;
+			} else if (cur != prev) {
 				ranges[prev].y = (uint32_t)idx;
 				ranges[cur].x = (uint32_t)idx;
 			}
+			if (idx == n - 1)
+				ranges[cur].y = (uint32_t)n;
+			if (idx == last)
+				s_last_tile = cur;
 		}
-		if (idx == n - 1)
-			ranges[cur].y = (uint32_t)n;
+		prev = cur;
 	}
 	if (!file_tail)
 		return;
-	const size_t last = min(n, ((size_t)blockIdx.x + 1) * kFileBlock) - 1;
-	if (idx == last)
-		s_last_tile = cur;
 	__syncthreads();
-	const bool counted = valid && cur == s_last_tile;  // sorted: these are the workgroup's last keys
-	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const uint32_t last_tile = s_last_tile;
+	uint2 own = {0u, 0u};
 #pragma unroll
-	for (int s = 0; s < 4; s++) {
-		const uint64_t m = __ballot(counted && ((key_strips(key) >> s) & 1u));
-		if (lane == 0)
-			s_tail[wave][s] = (uint32_t)__popcll(m);
-	}
+	for (int q = 0; q < 4; q++)
+		if (idx0 + q < n && key_tile(key[q]) == last_tile) {  // sorted: these are the workgroup's last keys
+			const uint32_t bits = key_strips(key[q]);
+			own.x += (bits & 1u) | ((bits & 2u) << 15);
+			own.y += ((bits >> 2) & 1u) | ((bits & 8u) << 13);
+		}
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const uint2 inc = {wave_inclusive_scan_u32(own.x), wave_inclusive_scan_u32(own.y)};
+	if (lane == 63)
+		s_tail[wave] = inc;
 	__syncthreads();
 	if (threadIdx.x == 0) {
-		uint4 t;
-		t.x = s_tail[0][0] + s_tail[1][0] + s_tail[2][0] + s_tail[3][0];
-		t.y = s_tail[0][1] + s_tail[1][1] + s_tail[2][1] + s_tail[3][1];
-		t.z = s_tail[0][2] + s_tail[1][2] + s_tail[2][2] + s_tail[3][2];
-		t.w = s_tail[0][3] + s_tail[1][3] + s_tail[2][3] + s_tail[3][3];
-		file_tail[blockIdx.x] = t;
+		const uint32_t x = s_tail[0].x + s_tail[1].x + s_tail[2].x + s_tail[3].x;
+		const uint32_t y = s_tail[0].y + s_tail[1].y + s_tail[2].y + s_tail[3].y;
+		file_tail[blockIdx.x] = uint4{x & 0xFFFFu, x >> 16, y & 0xFFFFu, y >> 16};
 	}
 }
 
@@ -957,7 +972,7 @@ void launch_tile_ranges(const TileRangesJob* jobs, int count, hipStream_t s)
 			max_n = jobs[at + k].n > max_n ? jobs[at + k].n : max_n;
 		}
 		if (live)
-			hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((max_n + kFileBlock - 1) / kFileBlock), (unsigned)live),
+			hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((max_n + kFileGroup - 1) / kFileGroup), (unsigned)live),
 			                   dim3(kFileBlock), 0, s, b);
 	}
 }

@@ -105,61 +105,90 @@ __device__ __forceinline__ float exponent_of(const float4 g, const float4 co, co
 
 // ---- filing ------------------------------------------------------------------------------------
 // The sorted keys carry, above the tile, one bit per strip the entry is filed for and one per strip
-// that lies inside the box (key_strips).  A workgroup takes 256 consecutive positions of the sorted
-// list, whichever tiles they belong to.  An entry's rank in its strip's list is the number of filed
-// entries of its tile before it: those inside the workgroup are counted from the ballots, those in
-// earlier workgroups (only the tile of the workgroup's first entry can have any) are the sum, over
-// the workgroups since that tile began, of what each filed for the tile of its LAST entry, which the
-// tile-range kernel has left in file_tail.  The thread that holds a tile's last entry also writes
-// the strips' totals.
+// that lies inside the box (key_strips).  A workgroup takes kFileGroup consecutive positions of the
+// sorted list, whichever tiles they belong to, four neighbouring positions per thread.  An entry's rank
+// in its strip's list is the number of filed entries of its tile before it: those inside the workgroup
+// follow from a prefix count over the workgroup (per thread in LDS, four strips packed 16 bits each),
+// taken at the entry and at the place where its tile begins; those in earlier workgroups (only the
+// tile of the workgroup's first entry can have any) are the sum, over the workgroups since that tile
+// began, of what each filed for the tile of its LAST entry, which the tile-range kernel has left in
+// file_tail.  The thread that holds a tile's last entry also writes the strips' totals.
 
-struct FileBallots {
-	uint64_t set[4][4];  // [wave][strip]
+// Counts of the four strips packed in two words, 16 bits each (a workgroup files at most kFileGroup per strip).
+__device__ __forceinline__ uint2 packed_strip_bits(uint32_t bits)
+{
+	return uint2{(bits & 1u) | ((bits & 2u) << 15), ((bits >> 2) & 1u) | ((bits & 8u) << 13)};
+}
+
+struct FileStage {
+	uint2 before[kFileBlock];   // entries filed by the threads before this one
+	uint16_t bits[kFileBlock];  // the filed bits of the thread's four positions, four bits each
+	uint2 wave_total[4];
+	uint32_t carry[4][4];       // [wave][strip] partial sums of the earlier workgroups' counts
 };
 
-// Number of set bits of strip s among threads [0, i) of the workgroup.
-__device__ __forceinline__ uint32_t filed_before(const FileBallots& b, int s, int i)
+// Entries filed at positions [0, i) of the workgroup.
+__device__ __forceinline__ uint2 filed_before(const FileStage& st, uint32_t i)
 {
-	uint32_t n = 0;
-	const int w = i >> 6;
+	const uint32_t t = i >> 2, q = i & 3u;
+	uint2 n = st.before[t];
+	const uint32_t bits = st.bits[t];
 #pragma unroll
-	for (int k = 0; k < 4; k++)
-		if (k < w)
-			n += (uint32_t)__popcll(b.set[k][s]);
-	if (w < 4)
-		n += (uint32_t)__popcll(b.set[w][s] & ((1ull << (i & 63)) - 1ull));
+	for (uint32_t k = 0; k < 3; k++)
+		if (k < q) {
+			const uint2 c = packed_strip_bits((bits >> (4 * k)) & 0xFu);
+			n.x += c.x;
+			n.y += c.y;
+		}
 	return n;
 }
 
 __global__ __launch_bounds__(kFileBlock) void strip_file_place_kernel(BlendBatch batch)
 {
-	__shared__ FileBallots s_ballots;
-	__shared__ uint32_t s_carry[4][4];  // [wave][strip] partial sums of the earlier workgroups' counts
+	__shared__ FileStage st;
 	const BlendArgs& a = batch.job[blockIdx.y];
 	const uint32_t capacity = a.capacity;
 	const uint32_t R = a.count_device ? min(capacity, *a.count_device) : capacity;
-	const uint32_t first = blockIdx.x * kFileBlock;
+	const uint32_t first = blockIdx.x * (uint32_t)kFileGroup;
 	// after a sort that gave up the list is not sorted and the tile ranges are empty: nothing to place
 	if (first >= R || (a.sort_status && *a.sort_status != 0u) || (a.order_status && *a.order_status != 0u))
 		return;
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const uint32_t pos = first + (uint32_t)tid;
-	const bool valid = pos < R;
-	const uint32_t key = valid ? a.tile_keys[pos] : 0u;
-	const uint32_t bits = key_strips(key), tile = key_tile(key);
-	const uint2 range = valid ? a.ranges[tile] : uint2{0u, 0u};
+	const uint32_t pos0 = first + 4u * (uint32_t)tid;
+	uint32_t key[4] = {0u, 0u, 0u, 0u};
+	if (pos0 + 3u < R) {
+		const uint4 k4 = *reinterpret_cast<const uint4*>(a.tile_keys + pos0);
+		key[0] = k4.x; key[1] = k4.y; key[2] = k4.z; key[3] = k4.w;
+	} else {
 #pragma unroll
-	for (int s = 0; s < 4; s++) {
-		const uint64_t m = __ballot((bits >> s) & 1u);
-		if (lane == 0)
-			s_ballots.set[wave][s] = m;
+		for (int q = 0; q < 4; q++)
+			if (pos0 + (uint32_t)q < R)
+				key[q] = a.tile_keys[pos0 + q];
 	}
+	uint2 range[4];
+	uint32_t filed[4];
+	uint2 own = {0u, 0u};
+	uint32_t all = 0;
+#pragma unroll
+	for (int q = 0; q < 4; q++) {
+		const bool valid = pos0 + (uint32_t)q < R;
+		range[q] = valid ? a.ranges[key_tile(key[q])] : uint2{0u, 0u};
+		filed[q] = valid ? (key_strips(key[q]) & 0xFu) : 0u;
+		const uint2 c = packed_strip_bits(filed[q]);
+		own.x += c.x;
+		own.y += c.y;
+		all |= filed[q] << (4 * q);
+	}
+	const uint2 inc = {wave_inclusive_scan_u32(own.x), wave_inclusive_scan_u32(own.y)};
+	if (lane == 63)
+		st.wave_total[wave] = inc;
+	st.bits[tid] = (uint16_t)all;
 	// what the tile of this workgroup's first entry filed in the workgroups before this one
 	{
 		const uint32_t begin0 = a.ranges[key_tile(a.tile_keys[first])].x;
 		uint4 sum = {0u, 0u, 0u, 0u};
 		if (begin0 < first)
-			for (uint32_t g = begin0 / kFileBlock + (uint32_t)tid; g < blockIdx.x; g += kFileBlock) {
+			for (uint32_t g = begin0 / (uint32_t)kFileGroup + (uint32_t)tid; g < blockIdx.x; g += kFileBlock) {
 				const uint4 t = a.file_tail[g];
 				sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
 			}
@@ -168,28 +197,57 @@ __global__ __launch_bounds__(kFileBlock) void strip_file_place_kernel(BlendBatch
 		for (int s = 0; s < 4; s++) {
 			const uint32_t tot = wave_inclusive_scan_u32(v[s]);
 			if (lane == 63)
-				s_carry[wave][s] = tot;
+				st.carry[wave][s] = tot;
 		}
 	}
 	__syncthreads();
-	if (!valid)
-		return;
-	const bool continues = range.x < first;  // the tile began in an earlier workgroup
-	const int begin = (int)(max(range.x, first) - first);
-	const uint32_t n = range.y - range.x, e = pos - range.x;
-	uint32_t* lists = a.strip_lists + 4 * (size_t)range.x;
-	uint32_t rank[4];
+	uint2 mine = {inc.x - own.x, inc.y - own.y};  // filed before this thread's first position
 #pragma unroll
-	for (int s = 0; s < 4; s++) {
-		const uint32_t carry = continues ? s_carry[0][s] + s_carry[1][s] + s_carry[2][s] + s_carry[3][s] : 0u;
-		rank[s] = carry + filed_before(s_ballots, s, tid) - filed_before(s_ballots, s, begin);
-		if ((bits >> s) & 1u)
-			lists[(size_t)s * n + rank[s]] = e | (((bits >> (4 + s)) & 1u) ? 0x80000000u : 0u);
-	}
-	if (pos + 1u == range.y) {  // the tile's last entry: its ranks plus itself are the strips' totals
-		uint4 total = {rank[0] + (bits & 1u), rank[1] + ((bits >> 1) & 1u), rank[2] + ((bits >> 2) & 1u),
-		               rank[3] + ((bits >> 3) & 1u)};
-		reinterpret_cast<uint4*>(a.strip_total)[tile] = total;
+	for (int w = 0; w < 3; w++)
+		if (w < wave) {
+			mine.x += st.wave_total[w].x;
+			mine.y += st.wave_total[w].y;
+		}
+	st.before[tid] = mine;
+	__syncthreads();
+	uint32_t carry[4];
+#pragma unroll
+	for (int s = 0; s < 4; s++)
+		carry[s] = st.carry[0][s] + st.carry[1][s] + st.carry[2][s] + st.carry[3][s];
+
+	uint32_t begin_of = 0xFFFFFFFFu;  // the tile start the last `from` was taken at
+	uint2 from = {0u, 0u};
+#pragma unroll
+	for (int q = 0; q < 4; q++) {
+		const uint32_t pos = pos0 + (uint32_t)q;
+		if (pos < R) {
+			const uint2 r = range[q];
+			const bool continues = r.x < first;  // the tile began in an earlier workgroup
+			const uint32_t begin = max(r.x, first) - first;
+			if (begin != begin_of) {
+				from = begin == 0u ? uint2{0u, 0u} : filed_before(st, begin);
+				begin_of = begin;
+			}
+			const uint32_t n = r.y - r.x, e = pos - r.x, bits = key_strips(key[q]);
+			uint32_t* lists = a.strip_lists + 4 * (size_t)r.x;
+			const uint32_t at[4] = {mine.x & 0xFFFFu, mine.x >> 16, mine.y & 0xFFFFu, mine.y >> 16};
+			const uint32_t base[4] = {from.x & 0xFFFFu, from.x >> 16, from.y & 0xFFFFu, from.y >> 16};
+			uint32_t rank[4];
+#pragma unroll
+			for (int s = 0; s < 4; s++) {
+				rank[s] = (continues ? carry[s] : 0u) + at[s] - base[s];
+				if ((bits >> s) & 1u)
+					lists[(size_t)s * n + rank[s]] = e | (((bits >> (4 + s)) & 1u) ? 0x80000000u : 0u);
+			}
+			if (pos + 1u == r.y) {  // the tile's last entry: its ranks plus itself are the strips' totals
+				uint4 total = {rank[0] + (bits & 1u), rank[1] + ((bits >> 1) & 1u), rank[2] + ((bits >> 2) & 1u),
+				               rank[3] + ((bits >> 3) & 1u)};
+				reinterpret_cast<uint4*>(a.strip_total)[key_tile(key[q])] = total;
+			}
+		}
+		const uint2 c = packed_strip_bits(filed[q]);
+		mine.x += c.x;
+		mine.y += c.y;
 	}
 }
 
@@ -857,7 +915,7 @@ void launch_strip_filing(const BlendArgs* jobs, int count, hipStream_t s)
 				most = jobs[k].capacity > most ? jobs[k].capacity : most;
 			}
 		if (batch.count)
-			hipLaunchKernelGGL(strip_file_place_kernel, dim3((most + kFileBlock - 1) / kFileBlock, (unsigned)batch.count),
+			hipLaunchKernelGGL(strip_file_place_kernel, dim3((most + kFileGroup - 1) / kFileGroup, (unsigned)batch.count),
 			                   dim3(kFileBlock), 0, s, batch);
 	}
 }

@@ -96,7 +96,7 @@ struct BlendArgs {
 	const uint32_t* tile_keys;    // the sorted key of every list position: tile and strip bits (key_tile, key_strips)
 	const uint32_t* count_device; // non-null: the number of instances is min(capacity, *count_device)
 	uint32_t capacity;      // instances the launch is sized for
-	const uint4* file_tail; // per kFileBlock list positions: entries filed per strip for the tile of the last of them
+	const uint4* file_tail; // per kFileGroup list positions: entries filed per strip for the tile of the last of them
 	const uint32_t* sort_status;   // status words of the two sorts (may be null): non-zero = the sort gave up
 	const uint32_t* order_status;
 	uint32_t* strip_order;  // strips by decreasing strip_filed, written behind the forward blend
@@ -262,7 +262,8 @@ struct AdamArgs {
 constexpr int kKeyTileBits = 24;
 __host__ __device__ inline uint32_t key_tile(uint32_t key) { return key & ((1u << kKeyTileBits) - 1u); }
 __host__ __device__ inline uint32_t key_strips(uint32_t key) { return key >> kKeyTileBits; }
-constexpr int kFileBlock = 256;   // list positions per workgroup of the kernels that file entries for strips
+constexpr int kFileBlock = 256;   // threads of a workgroup of the kernels that file entries for strips
+constexpr int kFileGroup = 1024;  // list positions such a workgroup takes, four neighbouring ones per thread
 
 // What the key duplication needs to decide the strips: the packed records and the submodel box test's frame.
 struct FilingArgs {
@@ -388,7 +389,7 @@ void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_
 // The tile ranges from the sorted keys.  Either status word (may be null) being non-zero leaves every range empty
 // and sets *fault (host memory the device can write, may be null).  The caller has cleared `ranges`.  With a non-null
 // n_device the number of keys is min(n, *n_device) and the launch is sized for n.  file_tail (may be null)
-// receives, per kFileBlock keys, how many entries of the tile of the last of them have each strip bit set.
+// receives, per kFileGroup keys, how many entries of the tile of the last of them have each strip bit set.
 constexpr int kRangeTailWords = 1024;   // words behind the ranges: the strip class counters of the blend
 struct TileRangesJob {
 	const uint32_t* keys;
