@@ -49,7 +49,8 @@ __global__ __launch_bounds__(256) void block_totals_kernel(const uint32_t* __res
 struct BlockScanJob {
 	uint32_t* data;
 	size_t n;
-	const uint32_t* n_device;
+	const uint32_t* n_device;  // if non-null: the number of elements behind the entries, `per_entry` of them to an entry
+	uint32_t per_entry;
 	uint32_t* total_out;
 	uint32_t* total_copy;
 	uint32_t* data_b;
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(1024) void single_block_exclusive_scan_kernel(Batch
 	if (!data)
 		return;
 	if (n_device)
-		n = ((size_t)*n_device + 255) / 256;  // one entry per 256 elements
+		n = ((size_t)*n_device + j.per_entry - 1) / j.per_entry;
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const size_t chunk = (n + 1023) / 1024;
 	const size_t lo = (size_t)tid * chunk;
@@ -115,9 +116,13 @@ struct BlockInclusiveJob {
 	uint32_t first_of_block_words;
 };
 
+// kPer consecutive elements per thread; with kPer = 4 `in` and `out` are 16-byte aligned and moved 16 bytes at a time.
+constexpr int kScanGroup = 1024;  // elements per workgroup of the four-per-thread kernels of the depth order
+template <int kPer>
 __global__ __launch_bounds__(256) void block_inclusive_scan_kernel(Batch<BlockInclusiveJob> batch)
 {
 	__shared__ uint32_t lds[8];
+	constexpr size_t kGroup = 256 * (size_t)kPer;
 	const BlockInclusiveJob& j = batch.job[blockIdx.y];
 	const uint32_t* __restrict__ in = j.in;
 	const uint32_t* __restrict__ block_base = j.block_base;
@@ -125,22 +130,56 @@ __global__ __launch_bounds__(256) void block_inclusive_scan_kernel(Batch<BlockIn
 	size_t n = j.n;
 	if (j.n_device)
 		n = *j.n_device;
-	if ((size_t)blockIdx.x * 256 >= n)
+	if ((size_t)blockIdx.x * kGroup >= n)
 		return;
-	const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-	const uint32_t v = i < n ? in[i] : 0u;
+	const size_t i0 = (size_t)blockIdx.x * kGroup + (size_t)kPer * threadIdx.x;
+	uint32_t v[kPer];
+	const bool whole = i0 + kPer <= n;
+	bool loaded = false;
+	if constexpr (kPer == 4) {
+		if (whole) {
+			const uint4 v4 = *reinterpret_cast<const uint4*>(in + i0);
+			v[0] = v4.x; v[1] = v4.y; v[2] = v4.z; v[3] = v4.w;
+			loaded = true;
+		}
+	}
+	if (!loaded) {
+#pragma unroll
+		for (int q = 0; q < kPer; q++)
+			v[q] = i0 + q < n ? in[i0 + q] : 0u;
+	}
+	uint32_t sum = 0;
+#pragma unroll
+	for (int q = 0; q < kPer; q++)
+		sum += v[q];
 	uint32_t total;
-	const uint32_t ex = block256_exclusive_scan_u32(v, lds, total);
-	if (i < n) {
-		const uint32_t begin = block_base[blockIdx.x] + ex, end = begin + v;
-		out[i] = end;
-		if (j.first_of_block) {
-			// entry i covers positions [begin, end): it is where every workgroup of the key duplication starts whose
+	uint32_t run = block_base[blockIdx.x] + block256_exclusive_scan_u32(sum, lds, total);
+	uint32_t end[kPer];
+#pragma unroll
+	for (int q = 0; q < kPer; q++) {
+		const uint32_t begin = run;
+		run += v[q];
+		end[q] = run;
+		if (j.first_of_block && i0 + q < n) {
+			// element i covers positions [begin, end): it is where every workgroup of the key duplication starts whose
 			// first position, a multiple of kDupPositions, lies among them
 			for (uint32_t b = (begin + (uint32_t)kDupPositions - 1u) / (uint32_t)kDupPositions;
-			     b < j.first_of_block_words && (uint64_t)b * (uint64_t)kDupPositions < (uint64_t)end; b++)
-				j.first_of_block[b] = (uint32_t)i;
+			     b < j.first_of_block_words && (uint64_t)b * (uint64_t)kDupPositions < (uint64_t)run; b++)
+				j.first_of_block[b] = (uint32_t)(i0 + q);
 		}
+	}
+	bool stored = false;
+	if constexpr (kPer == 4) {
+		if (whole) {
+			*reinterpret_cast<uint4*>(out + i0) = uint4{end[0], end[1], end[2], end[3]};
+			stored = true;
+		}
+	}
+	if (!stored) {
+#pragma unroll
+		for (int q = 0; q < kPer; q++)
+			if (i0 + q < n)
+				out[i0 + q] = end[q];
 	}
 }
 
@@ -155,11 +194,11 @@ static void inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, const uin
 	const size_t nb = (n + 255) / 256;
 	hipLaunchKernelGGL(block_totals_kernel, dim3((unsigned)nb), dim3(256), 0, s, in, n, n_device, temp);
 	Batch<BlockScanJob> scan = {};
-	scan.job[0] = BlockScanJob{temp, nb, n_device, nullptr, nullptr, nullptr, nullptr};
+	scan.job[0] = BlockScanJob{temp, nb, n_device, 256u, nullptr, nullptr, nullptr, nullptr};
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan);
 	Batch<BlockInclusiveJob> inc = {};
 	inc.job[0] = BlockInclusiveJob{in, temp, n, n_device, out, nullptr, 0u};
-	hipLaunchKernelGGL(block_inclusive_scan_kernel, dim3((unsigned)nb), dim3(256), 0, s, inc);
+	hipLaunchKernelGGL(block_inclusive_scan_kernel<1>, dim3((unsigned)nb), dim3(256), 0, s, inc);
 }
 
 void launch_inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, uint32_t* temp, const char* stage,
@@ -180,7 +219,7 @@ void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t
 		Batch<BlockScanJob> b = {};
 		for (int k = 0; k < nj; k++) {
 			const TotalsJob& t = jobs[at + k];
-			b.job[k] = BlockScanJob{t.block_sums, ((size_t)t.P + 255) / 256, nullptr, t.total_out, t.total_copy, t.block_visible,
+			b.job[k] = BlockScanJob{t.block_sums, ((size_t)t.P + 255) / 256, nullptr, 256u, t.total_out, t.total_copy, t.block_visible,
 			                        t.visible_count};
 		}
 		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(2, (unsigned)nj), dim3(1024), 0, s, b);
@@ -189,15 +228,16 @@ void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t
 
 // ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------
 
-// (depth bits, index) pairs of the Gaussians that touch a tile, compacted in index order:
-// block b of 256 Gaussians writes from visible_base[b] on.  Depths of rendered Gaussians are
+// (depth bits, index) pairs of the Gaussians that touch a tile, compacted in index order: the
+// workgroup that takes Gaussians [kScanGroup b, kScanGroup (b + 1)), four neighbouring ones per thread,
+// writes from visible_base[4 b] on (the bases are per 256 Gaussians).  Depths of rendered Gaussians are
 // positive floats (> 0.2), whose bit patterns order like the values.
 __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
 	const DepthOrderJob& j = batch.job[blockIdx.y];
-	const int P = j.P;
-	if ((int)blockIdx.x * 256 >= P)
+	const size_t P = (size_t)j.P;
+	if ((size_t)blockIdx.x * kScanGroup >= P)
 		return;
 	const float* __restrict__ depths = j.depths;
 	const uint32_t* __restrict__ tiles_touched = j.tiles_touched;
@@ -205,41 +245,73 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 	uint32_t* __restrict__ keys = j.keys_a;
 	uint32_t* __restrict__ values = j.order;
 	uint32_t* __restrict__ visible_list = j.visible_list;
-	const int idx = blockIdx.x * 256 + threadIdx.x;
-	const bool visible = idx < P && tiles_touched[idx] != 0u;
-	uint32_t total;
-	const uint32_t rank = block256_exclusive_scan_u32(visible ? 1u : 0u, lds, total);
-	if (visible) {
-		const uint32_t at = visible_base[blockIdx.x] + rank;
-		keys[at] = __float_as_uint(depths[idx]);
-		values[at] = (uint32_t)idx;
-		visible_list[at] = (uint32_t)idx;  // the sort reorders `values`; this copy stays in index order
+	const size_t idx0 = (size_t)blockIdx.x * kScanGroup + 4 * (size_t)threadIdx.x;
+	uint32_t touched[4] = {0u, 0u, 0u, 0u};
+	float depth[4] = {0.f, 0.f, 0.f, 0.f};
+	if (idx0 + 4 <= P) {
+		const uint4 t4 = *reinterpret_cast<const uint4*>(tiles_touched + idx0);
+		const float4 d4 = *reinterpret_cast<const float4*>(depths + idx0);
+		touched[0] = t4.x; touched[1] = t4.y; touched[2] = t4.z; touched[3] = t4.w;
+		depth[0] = d4.x; depth[1] = d4.y; depth[2] = d4.z; depth[3] = d4.w;
+	} else {
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+			if (idx0 + q < P) {
+				touched[q] = tiles_touched[idx0 + q];
+				depth[q] = depths[idx0 + q];
+			}
 	}
+	uint32_t mine = 0;
+#pragma unroll
+	for (int q = 0; q < 4; q++)
+		mine += touched[q] != 0u ? 1u : 0u;
+	uint32_t total;
+	uint32_t at = visible_base[4 * blockIdx.x] + block256_exclusive_scan_u32(mine, lds, total);
+#pragma unroll
+	for (int q = 0; q < 4; q++)
+		if (touched[q] != 0u) {
+			keys[at] = __float_as_uint(depth[q]);
+			values[at] = (uint32_t)(idx0 + q);
+			visible_list[at] = (uint32_t)(idx0 + q);  // the sort reorders `values`; this copy stays in index order
+			at++;
+		}
 }
 
-// out[k] = in[index[k]] for k below the count on the device, and the sum of every 256 of them
-// (the first level of the scan that follows).  `in` has in_size entries; an index beyond it (only
-// possible in what a sort that gave up left behind) reads the last entry instead.
+// out[k] = in[index[k]] for k below the count on the device, and the sum of every kScanGroup of them
+// (the first level of the scan that follows), four neighbouring k per thread.  `in` has in_size entries;
+// an index beyond it (only possible in what a sort that gave up left behind) reads the last entry instead.
 __global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
 	const DepthOrderJob& j = batch.job[blockIdx.y];
-	if ((int)blockIdx.x * 256 >= j.P)
+	const size_t n = min((size_t)*j.visible_count, (size_t)j.P);
+	if ((size_t)blockIdx.x * kScanGroup >= n)
 		return;
-	const uint32_t* __restrict__ n_device = j.visible_count;
 	const uint32_t* __restrict__ index = j.order;
 	const uint32_t* __restrict__ in = j.tiles_touched;
 	const uint32_t in_size = (uint32_t)j.P;
 	uint32_t* __restrict__ out = j.tiles_in_order;
 	uint32_t* __restrict__ block_totals = j.scan_temp;
-	const uint32_t k = blockIdx.x * 256 + threadIdx.x;
-	uint32_t v = 0;
-	if (k < *n_device) {
-		v = in[min(index[k], in_size - 1u)];
-		out[k] = v;
+	const size_t k0 = (size_t)blockIdx.x * kScanGroup + 4 * (size_t)threadIdx.x;
+	uint32_t v[4] = {0u, 0u, 0u, 0u};
+	const bool whole = k0 + 4 <= n;
+	if (whole) {
+		const uint4 i4 = *reinterpret_cast<const uint4*>(index + k0);
+		v[0] = in[min(i4.x, in_size - 1u)];
+		v[1] = in[min(i4.y, in_size - 1u)];
+		v[2] = in[min(i4.z, in_size - 1u)];
+		v[3] = in[min(i4.w, in_size - 1u)];
+		*reinterpret_cast<uint4*>(out + k0) = uint4{v[0], v[1], v[2], v[3]};
+	} else {
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+			if (k0 + q < n) {
+				v[q] = in[min(index[k0 + q], in_size - 1u)];
+				out[k0 + q] = v[q];
+			}
 	}
 	uint32_t total;
-	(void)block256_exclusive_scan_u32(v, lds, total);
+	(void)block256_exclusive_scan_u32(v[0] + v[1] + v[2] + v[3], lds, total);
 	if (threadIdx.x == 0)
 		block_totals[blockIdx.x] = total;
 }
@@ -428,16 +500,17 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)
 			max_p = j.P > max_p ? j.P : max_p;
 			// 4 passes: the sorted pairs end up in the first buffer pair again
 			sorts[k] = SortJob<uint32_t>{j.keys_a, j.keys_b, j.order, j.vals_b, (size_t)j.P, j.visible_count, j.sort_temp, nullptr, 0};
-			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + 255) / 256, j.visible_count, nullptr, nullptr, nullptr, nullptr};
+			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + kScanGroup - 1) / kScanGroup, j.visible_count, (uint32_t)kScanGroup, nullptr, nullptr,
+			                           nullptr, nullptr};
 			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order, j.dup_first,
 			                               (uint32_t)dup_first_words((size_t)j.P)};
 		}
-		const dim3 grid((unsigned)((max_p + 255) / 256), (unsigned)nj);
+		const dim3 grid((unsigned)((max_p + kScanGroup - 1) / kScanGroup), (unsigned)nj);
 		hipLaunchKernelGGL(depth_pairs_kernel, grid, dim3(256), 0, s, b);
 		launch_sort_pairs_u32(sorts, nj, 32, true, nullptr, s);
 		hipLaunchKernelGGL(gather_u32_kernel, grid, dim3(256), 0, s, b);
 		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1, (unsigned)nj), dim3(1024), 0, s, scan);
-		hipLaunchKernelGGL(block_inclusive_scan_kernel, grid, dim3(256), 0, s, inc);
+		hipLaunchKernelGGL(block_inclusive_scan_kernel<4>, grid, dim3(256), 0, s, inc);
 	}
 }
 
