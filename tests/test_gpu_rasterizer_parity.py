@@ -234,16 +234,19 @@ def test_tiny_images_and_few_gaussians(width, height, n):
     _check_backward(sub, cam, torch.tensor([0.2, 0.1, 0.05]), seed=3, with_depth_alpha=True)
 
 
-def test_gaussians_that_cover_the_whole_image():
+@pytest.mark.parametrize("width,height", [(400, 272), (1040, 784)])
+def test_gaussians_that_cover_the_whole_image(width, height):
     """Footprints of hundreds of tiles each (one Gaussian keeps a wavefront of the key duplication busy),
-    mixed with small ones; faint enough that the lists are walked to the end."""
+    mixed with small ones; faint enough that the lists are walked to the end.  At the larger size a footprint
+    has more tiles than one workgroup of the key duplication writes, so several workgroups start inside the
+    same Gaussian."""
     scene = scenes.cube_scene(400, seed=77)
     with torch.no_grad():
         scene["scales"][:40] = scene["scales"][:40] * 150.0
         scene["opacity"][:40] = 0.02
-    cam = scenes.look_at_camera((0.0, 0.0, 0.0), (0.0, 0.0, 4.0), (0, -1, 0), 400, 272, 60.0)
+    cam = scenes.look_at_camera((0.0, 0.0, 0.0), (0.0, 0.0, 4.0), (0, -1, 0), width, height, 60.0)
     sub = _scene_sub(scene)
     st = _check_forward_stages(sub, cam, torch.tensor([0.0, 0.0, 0.0]))
-    tiles = (400 // 16) * (272 // 16)
+    tiles = (width // 16) * (height // 16)
     assert (st.tiles_touched[:40] >= tiles // 2).sum() >= 20
     _check_backward(sub, cam, torch.zeros(3), seed=5, with_depth_alpha=True)
