@@ -726,7 +726,7 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 	const int n = (int)with_instances.size();
 	rgs::launch_duplicate_with_keys(dups.data(), n, gx, gy, s);
 	RGS_STAGE("duplicate_with_keys");
-	rgs::launch_sort_pairs_u32(sorts.data(), n, end_bit, true, "sort", s);
+	rgs::launch_sort_pairs_u32(sorts.data(), n, end_bit, true, false, "sort", s);
 	RGS_STAGE("sort_pairs");
 	if (debug)
 		for (int k : with_instances) {

@@ -114,6 +114,9 @@ struct BlockInclusiveJob {
 	uint32_t* out;
 	uint32_t* first_of_block;  // may be null; see DuplicateJob
 	uint32_t first_of_block_words;
+	// non-zero: block_base holds the totals of the workgroups' elements, not yet scanned: a workgroup adds up those
+	// ahead of its own itself (for a few thousand workgroups at most, which saves the launch that scans them)
+	uint32_t base_from_totals;
 };
 
 // kPer consecutive elements per thread; with kPer = 4 `in` and `out` are 16-byte aligned and moved 16 bytes at a time.
@@ -153,7 +156,16 @@ __global__ __launch_bounds__(256) void block_inclusive_scan_kernel(Batch<BlockIn
 	for (int q = 0; q < kPer; q++)
 		sum += v[q];
 	uint32_t total;
-	uint32_t run = block_base[blockIdx.x] + block256_exclusive_scan_u32(sum, lds, total);
+	uint32_t base = 0;
+	if (j.base_from_totals) {
+		uint32_t ahead = 0;
+		for (uint32_t b = threadIdx.x; b < blockIdx.x; b += 256)
+			ahead += block_base[b];
+		(void)block256_exclusive_scan_u32(ahead, lds, base);
+	} else {
+		base = block_base[blockIdx.x];
+	}
+	uint32_t run = base + block256_exclusive_scan_u32(sum, lds, total);
 	uint32_t end[kPer];
 #pragma unroll
 	for (int q = 0; q < kPer; q++) {
@@ -197,7 +209,7 @@ static void inclusive_sum(const uint32_t* in, uint32_t* out, size_t n, const uin
 	scan.job[0] = BlockScanJob{temp, nb, n_device, 256u, nullptr, nullptr, nullptr, nullptr};
 	hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1), dim3(1024), 0, s, scan);
 	Batch<BlockInclusiveJob> inc = {};
-	inc.job[0] = BlockInclusiveJob{in, temp, n, n_device, out, nullptr, 0u};
+	inc.job[0] = BlockInclusiveJob{in, temp, n, n_device, out, nullptr, 0u, 0u};
 	hipLaunchKernelGGL(block_inclusive_scan_kernel<1>, dim3((unsigned)nb), dim3(256), 0, s, inc);
 }
 
@@ -229,12 +241,16 @@ void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t
 // ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------
 
 // (depth bits, index) pairs of the Gaussians that touch a tile, compacted in index order: the
-// workgroup that takes Gaussians [kScanGroup b, kScanGroup (b + 1)), four neighbouring ones per thread,
-// writes from visible_base[4 b] on (the bases are per 256 Gaussians).  Depths of rendered Gaussians are
-// positive floats (> 0.2), whose bit patterns order like the values.
+// group of Gaussians [kScanGroup b, kScanGroup (b + 1)), four neighbouring ones per thread, is written
+// from visible_base[4 b] on (the bases are per 256 Gaussians).  Depths of rendered Gaussians are
+// positive floats (> 0.2), whose bit patterns order like the values.  A workgroup takes every
+// gridDim.x-th group and counts the four digits of the keys it writes on the way: at the end it adds
+// its counts to the digit histograms the sort of these pairs starts from (cleared beforehand), which
+// saves that sort its own pass over the keys.
 __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
+	__shared__ uint32_t s_hist[4][256];
 	const DepthOrderJob& j = batch.job[blockIdx.y];
 	const size_t P = (size_t)j.P;
 	if ((size_t)blockIdx.x * kScanGroup >= P)
@@ -245,36 +261,53 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 	uint32_t* __restrict__ keys = j.keys_a;
 	uint32_t* __restrict__ values = j.order;
 	uint32_t* __restrict__ visible_list = j.visible_list;
-	const size_t idx0 = (size_t)blockIdx.x * kScanGroup + 4 * (size_t)threadIdx.x;
-	uint32_t touched[4] = {0u, 0u, 0u, 0u};
-	float depth[4] = {0.f, 0.f, 0.f, 0.f};
-	if (idx0 + 4 <= P) {
-		const uint4 t4 = *reinterpret_cast<const uint4*>(tiles_touched + idx0);
-		const float4 d4 = *reinterpret_cast<const float4*>(depths + idx0);
-		touched[0] = t4.x; touched[1] = t4.y; touched[2] = t4.z; touched[3] = t4.w;
-		depth[0] = d4.x; depth[1] = d4.y; depth[2] = d4.z; depth[3] = d4.w;
-	} else {
+#pragma unroll
+	for (int p = 0; p < 4; p++)
+		s_hist[p][threadIdx.x] = 0u;
+	__syncthreads();
+	for (size_t group = blockIdx.x; group * kScanGroup < P; group += gridDim.x) {
+		const size_t idx0 = group * kScanGroup + 4 * (size_t)threadIdx.x;
+		uint32_t touched[4] = {0u, 0u, 0u, 0u};
+		float depth[4] = {0.f, 0.f, 0.f, 0.f};
+		if (idx0 + 4 <= P) {
+			const uint4 t4 = *reinterpret_cast<const uint4*>(tiles_touched + idx0);
+			const float4 d4 = *reinterpret_cast<const float4*>(depths + idx0);
+			touched[0] = t4.x; touched[1] = t4.y; touched[2] = t4.z; touched[3] = t4.w;
+			depth[0] = d4.x; depth[1] = d4.y; depth[2] = d4.z; depth[3] = d4.w;
+		} else {
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				if (idx0 + q < P) {
+					touched[q] = tiles_touched[idx0 + q];
+					depth[q] = depths[idx0 + q];
+				}
+		}
+		uint32_t mine = 0;
 #pragma unroll
 		for (int q = 0; q < 4; q++)
-			if (idx0 + q < P) {
-				touched[q] = tiles_touched[idx0 + q];
-				depth[q] = depths[idx0 + q];
+			mine += touched[q] != 0u ? 1u : 0u;
+		uint32_t total;
+		uint32_t at = visible_base[4 * group] + block256_exclusive_scan_u32(mine, lds, total);
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+			if (touched[q] != 0u) {
+				const uint32_t key = __float_as_uint(depth[q]);
+				keys[at] = key;
+				values[at] = (uint32_t)(idx0 + q);
+				visible_list[at] = (uint32_t)(idx0 + q);  // the sort reorders `values`; this copy stays in index order
+				at++;
+#pragma unroll
+				for (int p = 0; p < 4; p++)
+					atomicAdd(&s_hist[p][(key >> (8 * p)) & 255u], 1u);
 			}
 	}
-	uint32_t mine = 0;
+	__syncthreads();
 #pragma unroll
-	for (int q = 0; q < 4; q++)
-		mine += touched[q] != 0u ? 1u : 0u;
-	uint32_t total;
-	uint32_t at = visible_base[4 * blockIdx.x] + block256_exclusive_scan_u32(mine, lds, total);
-#pragma unroll
-	for (int q = 0; q < 4; q++)
-		if (touched[q] != 0u) {
-			keys[at] = __float_as_uint(depth[q]);
-			values[at] = (uint32_t)(idx0 + q);
-			visible_list[at] = (uint32_t)(idx0 + q);  // the sort reorders `values`; this copy stays in index order
-			at++;
-		}
+	for (int p = 0; p < 4; p++) {
+		const uint32_t c = s_hist[p][threadIdx.x];
+		if (c)
+			atomicAdd(&j.sort_temp[p * 256 + threadIdx.x], c);
+	}
 }
 
 // out[k] = in[index[k]] for k below the count on the device, and the sum of every kScanGroup of them
@@ -494,22 +527,27 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)
 		Batch<BlockInclusiveJob> inc = {};
 		SortJob<uint32_t> sorts[kMaxBatch];
 		int max_p = 0;
+		for (int k = 0; k < nj; k++)
+			max_p = jobs[at + k].P > max_p ? jobs[at + k].P : max_p;
+		const bool few_groups = ((size_t)max_p + kScanGroup - 1) / kScanGroup <= 4096;
 		for (int k = 0; k < nj; k++) {
 			const DepthOrderJob& j = jobs[at + k];
 			b.job[k] = j;
-			max_p = j.P > max_p ? j.P : max_p;
 			// 4 passes: the sorted pairs end up in the first buffer pair again
 			sorts[k] = SortJob<uint32_t>{j.keys_a, j.keys_b, j.order, j.vals_b, (size_t)j.P, j.visible_count, j.sort_temp, nullptr, 0};
 			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + kScanGroup - 1) / kScanGroup, j.visible_count, (uint32_t)kScanGroup, nullptr, nullptr,
 			                           nullptr, nullptr};
 			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order, j.dup_first,
-			                               (uint32_t)dup_first_words((size_t)j.P)};
+			                               (uint32_t)dup_first_words((size_t)j.P), few_groups ? 1u : 0u};
 		}
 		const dim3 grid((unsigned)((max_p + kScanGroup - 1) / kScanGroup), (unsigned)nj);
-		hipLaunchKernelGGL(depth_pairs_kernel, grid, dim3(256), 0, s, b);
-		launch_sort_pairs_u32(sorts, nj, 32, true, nullptr, s);
+		// few workgroups per job, each over many groups: every one ends with an atomic add per digit into its job's counts
+		const unsigned most = nj >= 8 ? 256u : 2048u / (unsigned)nj;
+		hipLaunchKernelGGL(depth_pairs_kernel, dim3(grid.x < most ? grid.x : most, (unsigned)nj), dim3(256), 0, s, b);
+		launch_sort_pairs_u32(sorts, nj, 32, true, true, nullptr, s);
 		hipLaunchKernelGGL(gather_u32_kernel, grid, dim3(256), 0, s, b);
-		hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1, (unsigned)nj), dim3(1024), 0, s, scan);
+		if (!few_groups)
+			hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1, (unsigned)nj), dim3(1024), 0, s, scan);
 		hipLaunchKernelGGL(block_inclusive_scan_kernel<4>, grid, dim3(256), 0, s, inc);
 	}
 }
@@ -853,7 +891,8 @@ size_t sort_clear_words(size_t n, int end_bit)
 }
 
 template <typename KeyT>
-static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool temp_cleared, bool mark_stages, hipStream_t s)
+static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done, bool mark_stages,
+                       hipStream_t s)
 {
 	const int passes = (end_bit + 7) / 8;
 	for (int at = 0; at < count; at += kMaxBatch) {
@@ -879,7 +918,8 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 		// job read the keys as fast as thousands would, and queue far fewer adds on the same words
 		const uint32_t most_blocks = live >= 8 ? 256u : 2048u / (uint32_t)live;
 		const uint32_t hist_blocks = max_tiles < most_blocks ? max_tiles : most_blocks;
-		hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
+		if (!histograms_done)
+			hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
 		for (int p = 0; p < passes; p++) {
 			const int shift = 8 * p;
 			const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
@@ -896,13 +936,13 @@ void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in,
                        int end_bit, uint32_t* temp, hipStream_t s)
 {
 	const SortJob<uint64_t> job = {keys_in, keys_out, vals_in, vals_out, n, nullptr, temp, nullptr, 0};
-	sort_pairs<uint64_t>(&job, 1, end_bit, false, true, s);
+	sort_pairs<uint64_t>(&job, 1, end_bit, false, false, true, s);
 }
 
-void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, const char* stage,
-                           hipStream_t s)
+void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done,
+                           const char* stage, hipStream_t s)
 {
-	sort_pairs<uint32_t>(jobs, count, end_bit, temp_cleared, stage != nullptr, s);
+	sort_pairs<uint32_t>(jobs, count, end_bit, temp_cleared, histograms_done, stage != nullptr, s);
 }
 
 // Sets n words to v, 16 bytes per store where the address allows; a capped grid walks the array.

@@ -378,8 +378,10 @@ struct SortJob {
 };
 // The same for 32-bit keys, every job in one launch per kernel; with a null `stage` its kernels are not marked for
 // the timing aid.  temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of every temp already.
-void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, const char* stage,
-                           hipStream_t s);
+// histograms_done: the kernel that wrote keys_in has also added every key's digits to the counts at the start of temp
+// (temp[256 p + d] = keys whose bits [8 p, 8 p + 8) are d), so the sort need not read the keys for that.
+void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done,
+                           const char* stage, hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)
 // Polls a look-back allows before it gives up (0 restores the default; negative: give up at once,
 // which is how a test exercises the give-up path with every kernel still running to its end).

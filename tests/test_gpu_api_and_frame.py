@@ -278,6 +278,39 @@ def test_enqueued_geometry_stage_gives_the_same_forward_and_is_checked():
     torch.cuda.synchronize()
 
 
+def test_a_workspace_off_a_16_byte_boundary_is_refused():
+    """The binning kernels move keys 16 bytes at a time: rgs_forward_raster refuses a workspace that does not
+    start at a multiple of 16 bytes, before anything is launched, and accepts the same one when aligned."""
+    import ctypes as C
+    from retinags_amd import GaussianRasterizer, _capi
+    from retinags_amd.rasterizer import ptr
+    lib = _capi.lib
+    scene, cam, low, up = _small_inputs(n=3000, seed=5)
+    r = GaussianRasterizer(_settings(oracle_settings(cam, low, up, torch.zeros(3))))
+    stage = r.enqueue_geometry(means3D=scene["xyz"].to(DEV), opacities=scene["opacity"].to(DEV), shs=scene["shs"].to(DEV),
+                               scales=scene["scales"].to(DEV), rotations=scene["rotations"].to(DEV))
+    R, t = stage.instances(), stage.tensors
+    assert R > 0
+    H, W = stage.H, stage.W
+    byte = dict(dtype=torch.uint8, device=DEV)
+    binning = torch.empty(lib.rgs_binning_bytes(R) + 16, **byte)
+    image = torch.empty(lib.rgs_image_bytes(W, H), **byte)
+    color, depth, alpha = (torch.empty(c, H, W, device=DEV) for c in (3, 1, 1))
+
+    def raster(binning_at):
+        return lib.rgs_forward_raster(
+            stage.P, R, W, H, ptr(t["bg"]), t["tanfovx"], t["tanfovy"], ptr(t["projmatrix_inv"]), ptr(t["range_low"]),
+            ptr(t["range_up"]), ptr(t["colors_precomp"]), ptr(stage.radii), ptr(stage.geomBuffer), stage.geom_bytes,
+            C.c_void_p(binning.data_ptr() + binning_at), lib.rgs_binning_bytes(R), ptr(image), image.numel(), ptr(color),
+            ptr(depth), ptr(alpha), C.c_void_p(stage.stream), 0)
+
+    assert raster(4) != 0
+    assert "16-byte aligned" in lib.rgs_last_error().decode()
+    assert raster(0) == 0
+    torch.cuda.synchronize()
+    assert float(alpha.max()) > 0.0
+
+
 def test_forward_with_an_instance_bound_needs_no_count_and_reports_overflow():
     """enqueue_geometry(instance_bound=N) + forward: no wait for the instance count.  With room
     enough the outputs and gradients are those of the ordinary call, bit for bit (gradients up to
