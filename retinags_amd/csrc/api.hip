@@ -182,7 +182,7 @@ struct Carver {
 
 // Scratch of the depth sort of the Gaussians, inside the geometry workspace.
 struct OrderScratch {
-	size_t keys_a, keys_b, vals_b, tiles_in_order, sort_temp, scan_temp, dup_first, total;
+	size_t keys_a, keys_b, vals_b, tiles_in_order, sort_temp, scan_temp, dup_first, tile_digits, total;
 };
 
 OrderScratch order_scratch(size_t P)
@@ -196,6 +196,7 @@ OrderScratch order_scratch(size_t P)
 	o.sort_temp = c.take(4 * rgs::sort_temp_words(P));
 	o.scan_temp = c.take(4 * rgs::scan_temp_words(P));
 	o.dup_first = c.take(4 * rgs::dup_first_words(P));
+	o.tile_digits = c.take(4 * rgs::kTileDigitWords);
 	o.total = c.cursor;
 	return o;
 }
@@ -529,6 +530,7 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 		d.offsets_in_order = at<uint32_t>(ws, off[RGS_GEOM_POINT_OFFSETS]);
 		d.sort_temp = at<uint32_t>(scratch, o.sort_temp); d.scan_temp = at<uint32_t>(scratch, o.scan_temp);
 		d.dup_first = at<uint32_t>(scratch, o.dup_first);
+		d.tile_digits = at<uint32_t>(scratch, o.tile_digits);
 	}
 	rgs::launch_preprocess_forward(pre.data(), K, s);
 	RGS_STAGE("preprocess");
@@ -713,12 +715,15 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 		d.filing.W = width; d.filing.H = height;
 		d.keys = keys_a; d.values = vals_a; d.capacity = (uint32_t)R;
 		d.clear = temp; d.clear_words = rgs::sort_clear_words((size_t)R, end_bit);
+		// it also clears the tile ranges (and the counters and totals behind them) and counts the digits of the tiles
+		// it writes, so the sort starts with its passes
+		uint32_t* tile_digits = at<uint32_t>(at<char>(c.geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).tile_digits);
+		d.tile_digits = tile_digits; d.end_bit = end_bit;
+		d.also_clear = reinterpret_cast<uint32_t*>(ranges); d.also_clear_words = clear_words;
 		dups.push_back(d);
-		// the first kernel of the sort also clears the tile ranges (and the counters and totals behind them)
-		sorts.push_back(rgs::SortJob<uint32_t>{keys_a, keys_b, vals_a, vals_b, (size_t)R, count, temp,
-		                                       reinterpret_cast<uint32_t*>(ranges), clear_words});
+		sorts.push_back(rgs::SortJob<uint32_t>{keys_a, keys_b, vals_a, vals_b, (size_t)R, count, temp, nullptr, 0, tile_digits});
 		ranges_jobs.push_back(rgs::TileRangesJob{a.tile_keys, (size_t)R, count, ranges, a.sort_status, a.order_status, fault,
-		                                         at<uint4>(c.binning_ws, b.file_tail)});
+		                                         at<uint4>(c.binning_ws, b.file_tail), tile_digits});
 		with_instances.push_back(k);
 	}
 	if (with_instances.empty())
@@ -726,7 +731,7 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 	const int n = (int)with_instances.size();
 	rgs::launch_duplicate_with_keys(dups.data(), n, gx, gy, s);
 	RGS_STAGE("duplicate_with_keys");
-	rgs::launch_sort_pairs_u32(sorts.data(), n, end_bit, true, false, "sort", s);
+	rgs::launch_sort_pairs_u32(sorts.data(), n, end_bit, true, true, "sort", s);
 	RGS_STAGE("sort_pairs");
 	if (debug)
 		for (int k : with_instances) {

@@ -317,6 +317,9 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> ba
 {
 	__shared__ uint32_t lds[8];
 	const DepthOrderJob& j = batch.job[blockIdx.y];
+	if (blockIdx.x == 0)  // what the key duplication will count the digits of its tiles into
+		for (int w = threadIdx.x; w < kTileDigitWords; w += 256)
+			j.tile_digits[w] = 0u;
 	const size_t n = min((size_t)*j.visible_count, (size_t)j.P);
 	if ((size_t)blockIdx.x * kScanGroup >= n)
 		return;
@@ -351,15 +354,18 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> ba
 
 // Instances of the Gaussians in depth order, tiles row by row like the reference, at the offsets
 // of the scan taken in that same order.  The work is dealt out by output position, not by Gaussian:
-// a workgroup writes kDupPositions consecutive instances, whichever Gaussians they belong to (one
-// that covers thousands of tiles is shared by several workgroups, a thousand that cover one tile
-// each are taken by one).  It finds the first Gaussian of its range by a 64-ary search over the
-// inclusive offsets, stages the offsets and indices of the Gaussians of its range in LDS 256 at a time
+// a workgroup writes runs of kDupPositions consecutive instances, whichever Gaussians they belong to (one
+// that covers thousands of tiles is shared by several runs, a thousand that cover one tile
+// each are taken by one).  It takes the first Gaussian of a run from the table the offset scan has filled
+// (beyond that table, from a 64-ary search over the inclusive offsets), stages the offsets and indices of
+// the Gaussians of the run in LDS 256 at a time
 // and lets every thread find the Gaussian of its output position by a binary search over those 256
 // offsets, read that Gaussian's 64-byte record, and take the tile from the position inside the
 // record's rectangle; stores are contiguous.  The thread also decides which of the
 // tile's four strips the instance can matter to (strip_filing.h) and puts those bits above the
 // tile in the key: the sort only looks at the tile bits, so they travel with the instance for free.
+// On the way the workgroup counts the digits of the tiles it writes (what the sort's passes start from:
+// the sort then has no pass of its own over the keys) and it clears the sort's scratch and the tile ranges.
 // `order` is the output of a sort: should that sort ever have given up, its entries may be anything, so
 // they are clamped to the P Gaussians there are (the tile ranges then stay empty and nothing reads the result).
 struct DuplicateStage {
@@ -378,6 +384,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 {
 	__shared__ DuplicateStage st;
 	__shared__ uint32_t s_first;
+	__shared__ uint32_t s_digits[kTileDigitWords];  // digit counts of the tiles this workgroup writes
 	extern __shared__ __align__(16) float s_ndc[];  // NDC of every tile column's first and last pixel, then of every strip's first and last row
 	const DuplicateJob& job = batch.job[blockIdx.y];
 	const uint32_t P = (uint32_t)job.P;
@@ -394,17 +401,18 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	// the scratch of the sort that follows is cleared here, which saves a launch
 	for (size_t w = (size_t)blockIdx.x * 256 + tid; w < clear_words; w += (size_t)gridDim.x * 256)
 		clear[w] = 0u;
+	for (size_t w = (size_t)blockIdx.x * 256 + tid; w < job.also_clear_words; w += (size_t)gridDim.x * 256)
+		job.also_clear[w] = 0u;
 	const uint32_t n = min(*visible_count, P);
 	const uint32_t total = *job.total;
-	const bool listed = blockIdx.x < (uint32_t)dup_first_words((size_t)P);
-	const uint32_t listed_first = listed ? job.first_of_block[blockIdx.x] : 0u;  // only meaningful below `total`
 	if (n == 0u)
 		return;
 	const uint32_t limit = min(total, capacity);  // positions beyond the room the caller gave are dropped
-	const uint32_t start = blockIdx.x * (uint32_t)kDupPositions;
-	if (start >= limit)
+	if (blockIdx.x * (uint32_t)kDupPositions >= limit)
 		return;
-	const uint32_t stop = min(start + (uint32_t)kDupPositions, limit);
+	const int passes = (job.end_bit + 7) / 8;
+	for (int w = tid; w < kTileDigitWords; w += 256)
+		s_digits[w] = 0u;
 
 	const int rows_at = (2 * gx + 3) & ~3;
 	if (ndc_in_lds) {
@@ -419,10 +427,18 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 			s_ndc[rows_at + 2 * r + 1] = v.y;
 		}
 	}
+	const BoxFrame box = load_box_frame(filing.projinv, filing.range_low, filing.range_up, filing.tanfovx, filing.tanfovy);
+
+	// A workgroup takes every gridDim.x-th run of kDupPositions positions: the tables above are set up once, and the
+	// digit counts of many runs leave with one atomic add per digit.
+	for (uint32_t run = blockIdx.x; (uint64_t)run * kDupPositions < (uint64_t)limit; run += gridDim.x) {
+	const uint32_t start = run * (uint32_t)kDupPositions;
+	const uint32_t stop = min(start + (uint32_t)kDupPositions, limit);
+	__syncthreads();  // the previous run is done with s_first and the staged Gaussians; the tables are written
 	// the first Gaussian whose inclusive offset exceeds `start`: from the table, or by a 64-ary search of the first wavefront
-	if (listed) {
+	if (run < (uint32_t)dup_first_words((size_t)P)) {
 		if (tid == 0)
-			s_first = min(listed_first, n - 1u);
+			s_first = min(job.first_of_block[run], n - 1u);
 	} else if (tid < 64) {
 		uint32_t lo = 0, hi = n;  // the answer lies in [lo, hi]
 		while (lo < hi) {
@@ -442,7 +458,6 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 			s_first = lo;
 	}
 	__syncthreads();
-	const BoxFrame box = load_box_frame(filing.projinv, filing.range_low, filing.range_up, filing.tanfovx, filing.tanfovy);
 
 	for (uint32_t g0 = s_first; g0 < n; g0 += 256) {
 		// stage the offsets and indices of Gaussians g0 .. g0 + 255 (in depth order)
@@ -479,9 +494,11 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 				r3[q] = rec[3];
 			}
 		}
+		uint32_t tile_of[kPerThread];
 #pragma unroll
 		for (int q = 0; q < kPerThread; q++) {
 			const uint32_t pos = from + (uint32_t)tid + 256u * (uint32_t)q;
+			tile_of[q] = 0xFFFFFFFFu;
 			if (pos >= to)
 				continue;
 			const TileRect rc = tile_rect(r0[q].x, r0[q].y, __float_as_int(r3[q].z), gx, gy);
@@ -510,10 +527,38 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 			const uint32_t strips = strips_filed_for(tests, (float)(tx * kTile), (float)(ty * kTile), nx, ny, box);
 			keys[pos] = tile | (strips << kKeyTileBits);
 			values[pos] = index[q];
+			tile_of[q] = tile;
+		}
+		// the digits of the tiles just written, for the sort (every lane comes here: the narrow digits are counted by ballot)
+#pragma unroll
+		for (int q = 0; q < kPerThread; q++) {
+			const bool have = tile_of[q] != 0xFFFFFFFFu;
+			for (int p = 0; p < passes; p++) {
+				const int shift = 8 * p;
+				const int bits = job.end_bit - shift < 8 ? job.end_bit - shift : 8;
+				const uint32_t d = (tile_of[q] >> shift) & ((1u << bits) - 1u);
+				if (bits <= 2) {
+					// a digit of one or two bits: every lane would add to one of a few words, one after the other
+					for (uint32_t v = 0; v < (1u << bits); v++) {
+						const uint32_t c = (uint32_t)__popcll(__ballot(have && d == v));
+						if (lane == 0 && c != 0u)
+							atomicAdd(&s_digits[256 * p + v], c);
+					}
+				} else if (have) {
+					atomicAdd(&s_digits[256 * p + d], 1u);
+				}
+			}
 		}
 		if (staged_end >= stop)
 			break;
 		__syncthreads();
+	}
+	}
+	__syncthreads();
+	for (int w = tid; w < 256 * passes; w += 256) {
+		const uint32_t c = s_digits[w];
+		if (c)
+			atomicAdd(&job.tile_digits[w], c);
 	}
 }
 
@@ -568,6 +613,10 @@ void launch_duplicate_with_keys(const DuplicateJob* jobs, int count, int grid_x,
 			                        min((b.job[k].clear_words + 4095) / 4096, (size_t)1024));
 			blocks = need > blocks ? need : blocks;
 		}
+		// every workgroup ends with an atomic add per digit into its job's counts: enough of them to fill the GPU several
+		// times over, each over many runs of positions, rather than one per run
+		const size_t most = nj >= 8 ? 512 : 4096 / (size_t)nj;  // twice and four times as many were measured slower
+		blocks = blocks < most ? blocks : most;
 		hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((unsigned)blocks, (unsigned)nj), dim3(256),
 		                   ndc_in_lds ? table * sizeof(float) : 0, s, b, grid_x, grid_y, ndc_in_lds);
 	}
@@ -685,7 +734,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 	const size_t job_tiles = (j.n + kSortBlock - 1) / kSortBlock;
 	if (blockIdx.x >= job_tiles)
 		return;  // the launch is sized for the job with the most tiles
-	const uint32_t* __restrict__ digit_count = j.temp + pass * 256;
+	const uint32_t* __restrict__ digit_count = (j.digit_counts ? j.digit_counts : j.temp) + pass * 256;
 	uint32_t* __restrict__ lookback = j.temp + kSortHeader + (size_t)pass * 256 * job_tiles;
 	uint32_t* __restrict__ tile_counter = j.temp + kSortCounters + pass;
 	uint32_t* __restrict__ status = j.temp + kSortStatus;
@@ -912,7 +961,7 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 		}
 		if (live == 0)
 			continue;
-		if (mark_stages)
+		if (mark_stages && !histograms_done)
 			stage_mark("sort_setup", s);
 		// every block ends with an atomic add per digit and pass into its job's counts: a few hundred blocks per
 		// job read the keys as fast as thousands would, and queue far fewer adds on the same words
@@ -994,6 +1043,9 @@ __global__ __launch_bounds__(kFileBlock) void tile_ranges_kernel(Batch<TileRange
 	const size_t first = (size_t)blockIdx.x * kFileGroup;
 	if (first >= j.n)
 		return;  // the launch is sized for the job with the most keys
+	if (blockIdx.x == 0 && j.rezero)  // the sort has read its digit counts: zero again for the next to count into them
+		for (int w = threadIdx.x; w < kTileDigitWords; w += kFileBlock)
+			j.rezero[w] = 0u;
 	if ((sort_status && *sort_status != 0u) || (order_status && *order_status != 0u)) {
 		if (blockIdx.x == 0 && threadIdx.x == 0 && fault)
 			__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);

@@ -323,6 +323,7 @@ struct DepthOrderJob {
 	uint32_t* sort_temp;
 	uint32_t* scan_temp;
 	uint32_t* dup_first;       // dup_first_words(P) words: see launch_duplicate_with_keys
+	uint32_t* tile_digits;     // kTileDigitWords words, left zero: see DuplicateJob
 };
 void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 // Also sets clear[0..clear_words) to zero (the scratch of the sort that follows).  Instances whose
@@ -333,6 +334,10 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 // those beyond (more than 16 instances per Gaussian on average) search the offsets instead.
 constexpr int kDupPositions = 1024;
 constexpr size_t dup_first_words(size_t P) { return P / 64 + 2; }
+// The key duplication also counts the digits of the tiles it writes, which is what the sort of its keys starts
+// from: counts[256 p + d] = keys whose tile bits [8 p, 8 p + 8) are d, in kTileDigitWords words that are zero when it
+// starts (the depth order leaves them so, and so does the tile-range kernel, the last to run after they were read).
+constexpr int kTileDigitWords = 3 * 256;  // tiles have at most 24 bits
 struct DuplicateJob {
 	int P;
 	const uint32_t* visible_count;
@@ -340,6 +345,10 @@ struct DuplicateJob {
 	const uint32_t* offsets;   // inclusive, in depth order
 	const uint32_t* total;     // the last of them
 	const uint32_t* first_of_block;  // dup_first_words(P) words
+	uint32_t* tile_digits;     // kTileDigitWords words, zero beforehand
+	int end_bit;               // bits of the tile the sort will look at
+	uint32_t* also_clear;      // a second array to clear (the tile ranges and what lies behind them)
+	size_t also_clear_words;
 	FilingArgs filing;
 	uint32_t* keys;
 	uint32_t* values;
@@ -375,6 +384,7 @@ struct SortJob {
 	uint32_t* temp;
 	uint32_t* also_clear;
 	size_t also_clear_words;
+	const uint32_t* digit_counts;  // null: the counts are at the start of temp
 };
 // The same for 32-bit keys, every job in one launch per kernel; with a null `stage` its kernels are not marked for
 // the timing aid.  temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of every temp already.
@@ -402,6 +412,7 @@ struct TileRangesJob {
 	const uint32_t* order_status;
 	uint32_t* fault;
 	uint4* file_tail;
+	uint32_t* rezero;  // may be null: kTileDigitWords words set to zero (the digit counts the sort has read)
 };
 void launch_tile_ranges(const TileRangesJob* jobs, int count, hipStream_t s);
 

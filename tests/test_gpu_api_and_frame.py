@@ -309,6 +309,14 @@ def test_a_workspace_off_a_16_byte_boundary_is_refused():
     assert raster(0) == 0
     torch.cuda.synchronize()
     assert float(alpha.max()) > 0.0
+    # the second half of the forward may run again on the same geometry state (its counters are left as it found them)
+    first = (color.clone(), depth.clone(), alpha.clone())
+    for out in (color, depth, alpha):
+        out.fill_(-1.0)
+    assert raster(0) == 0
+    torch.cuda.synchronize()
+    for a, b in zip(first, (color, depth, alpha)):
+        assert torch.equal(a, b)
 
 
 def test_forward_with_an_instance_bound_needs_no_count_and_reports_overflow():
