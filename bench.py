@@ -29,6 +29,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_PEAK_TFLOPS = 157.3   # MI355X fp32 vector
+SIMDS = 256 * 4            # compute units x SIMDs
+CLOCK_HZ = 2.4e9           # peak engine clock
 
 def load_traffic_table():
     """HBM bytes per launch of each stage's kernels on the default workload (C1 at full size), measured with
@@ -46,6 +48,26 @@ def load_traffic_table():
                 continue
             name, mb = line.split()[:2]
             table[name] = float(mb)
+    except (OSError, ValueError):
+        return {}, None
+    return table, commit
+
+
+def load_valu_table():
+    """Wave-level vector-ALU instructions per launch of the kernels that are bound by instruction issue, on the
+    default workload (C1 at full size), from a rocprofv3 SQ_INSTS_VALU run of this script; kept like the traffic
+    figures in a small text file that names the commit it was taken at."""
+    path = os.path.join(ROOT, "profiles", "c1_valu_instructions_per_launch.txt")
+    table, commit = {}, None
+    try:
+        for raw in open(path):
+            line = raw.strip()
+            if line.startswith("# commit:"):
+                commit = line.split(":", 1)[1].strip()
+            if not line or line.startswith("#"):
+                continue
+            name, millions = line.split()[:2]
+            table[name] = float(millions) * 1e6
     except (OSError, ValueError):
         return {}, None
     return table, commit
@@ -327,6 +349,13 @@ def measure(args, config, forward_only, asides, cpu):
             if full_c1 and dominant in traffic:
                 roofline["traffic"] = traffic[dominant] * 1e6  # bytes per launch
                 roofline["traffic_measured_at_commit"] = commit
+            valu, valu_commit = load_valu_table()
+            if full_c1 and dominant in valu and d.get("bound") == "valu":
+                # a SIMD has 16 lanes: a wave-level instruction occupies it for 4 cycles
+                issue_ms = valu[dominant] * 4 / (SIMDS * CLOCK_HZ) * 1e3
+                roofline["valu_issue"] = {"wave_instructions": valu[dominant], "issue_ms": round(issue_ms, 4),
+                                          "frac_of_launch": round(issue_ms / d["avg_launch_ms"], 4),
+                                          "simds": SIMDS, "clock_GHz": CLOCK_HZ / 1e9, "measured_at_commit": valu_commit}
             roofline["timing"] = "HIP events on the launching stream, all submodels on one stream"
             roofline["avg_launch_ms"] = d["avg_launch_ms"]
             roofline["launches_per_step"] = d["launches_per_step"]
