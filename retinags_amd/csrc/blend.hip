@@ -568,8 +568,7 @@ __device__ __forceinline__ int row_column(int pixel) { return pixel + (pixel >> 
 
 struct BackwardPixel {
 	float T, T_final;
-	float accum_r, accum_g, accum_b, accum_depth, accum_alpha;
-	float last_alpha, last_r, last_g, last_b, last_depth;
+	float behind_r, behind_g, behind_b, behind_depth, behind_alpha;
 	float g_r, g_g, g_b, g_depth, g_alpha;
 	float bg_dot_dpixel;
 };
@@ -675,24 +674,23 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 			p.T = p.T * inv_one_minus_alpha;
 			aT = alpha * p.T;
 			const float4 cd = st.cd[slot];
-			const float keep = 1.f - p.last_alpha;
+			// p.behind_* is what the entries behind this one (already visited) add up to, per unit of transmittance:
+			// the reference forms it at the next entry from this entry's alpha and colour (K/cuda_rasterizer_hgs/backward.cu:568-592:
+			// accum_rec = last_alpha * last_color + (1 - last_alpha) * accum_rec); formed here, right after its use,
+			// the same expression needs no copy of this entry's alpha and colour kept for the next visit.
+			const float keep = 1.f - alpha;
 			float dL_dopa = 0.0f;
-			p.accum_r = p.last_alpha * p.last_r + keep * p.accum_r;
-			p.last_r = cd.x;
-			dL_dopa += (cd.x - p.accum_r) * p.g_r;
-			p.accum_g = p.last_alpha * p.last_g + keep * p.accum_g;
-			p.last_g = cd.y;
-			dL_dopa += (cd.y - p.accum_g) * p.g_g;
-			p.accum_b = p.last_alpha * p.last_b + keep * p.accum_b;
-			p.last_b = cd.z;
-			dL_dopa += (cd.z - p.accum_b) * p.g_b;
-			p.accum_depth = p.last_alpha * p.last_depth + keep * p.accum_depth;
-			p.last_depth = cd.w;
-			dL_dopa += (cd.w - p.accum_depth) * p.g_depth;
-			p.accum_alpha = p.last_alpha + keep * p.accum_alpha;
-			dL_dopa += (1 - p.accum_alpha) * p.g_alpha;
+			dL_dopa += (cd.x - p.behind_r) * p.g_r;
+			dL_dopa += (cd.y - p.behind_g) * p.g_g;
+			dL_dopa += (cd.z - p.behind_b) * p.g_b;
+			dL_dopa += (cd.w - p.behind_depth) * p.g_depth;
+			dL_dopa += (1 - p.behind_alpha) * p.g_alpha;
 			dL_dopa *= p.T;
-			p.last_alpha = alpha;
+			p.behind_r = alpha * cd.x + keep * p.behind_r;
+			p.behind_g = alpha * cd.y + keep * p.behind_g;
+			p.behind_b = alpha * cd.z + keep * p.behind_b;
+			p.behind_depth = alpha * cd.w + keep * p.behind_depth;
+			p.behind_alpha = alpha + keep * p.behind_alpha;
 			dL_dopa += (-p.T_final * inv_one_minus_alpha) * p.bg_dot_dpixel;
 			u = G * dL_dopa;
 		}
@@ -747,8 +745,7 @@ __global__ __launch_bounds__(64) void blend_backward_kernel(BlendBatch batch)
 	BackwardPixel p;
 	p.T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
 	p.T = p.T_final;
-	p.accum_r = p.accum_g = p.accum_b = p.accum_depth = p.accum_alpha = 0.f;
-	p.last_alpha = p.last_r = p.last_g = p.last_b = p.last_depth = 0.f;
+	p.behind_r = p.behind_g = p.behind_b = p.behind_depth = p.behind_alpha = 0.f;
 	p.g_r = p.g_g = p.g_b = p.g_depth = p.g_alpha = 0.f;
 	if (inside) {
 		p.g_r = a.dL_dpix[pix_id];
