@@ -1019,7 +1019,9 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		                       view->tan_fovx, view->tan_fovy, l.radii, l.geom_ws, l.grad_accum, l.dL_dmean2D, l.dL_dopacity,
 		                       l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh, l.dL_dscale, l.dL_drot);
 	}
-	// The gradient arrays are cleared (pure memory traffic) beside the blend (instruction issue) when there is a second stream.
+	// Gradient arrays that the caller has not cleared are cleared here, on the second stream if there is one (a caller
+	// with a second stream does better to clear them there during the forward: the backward blend fills every SIMD's
+	// registers, and stores beside it were measured to slow it down by as much as they take).
 	hipError_t e = hipSuccess;
 	if (beside != s) {
 		hipEvent_t begun = frame_event(0);

@@ -550,18 +550,19 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 //  * pixel-parallel part (lane = pixel, as in the forward): the per-pixel recurrences of the
 //    reference loop give, for an entry, two numbers per pixel: u = G dL/dalpha-term and
 //    aT = alpha T.  They are parked in one LDS row per entry.
-//  * entry-parallel part, run whenever 16 rows are full (lane = (entry, strip row)): each lane
-//    sweeps the 16 pixels of its strip row and accumulates sum u, sum u dx, sum u dx^2 and
+//  * entry-parallel part, run whenever 8 rows are full (lane = (entry, strip row, half of the row)):
+//    each lane sweeps 8 pixels and accumulates sum u, sum u dx, sum u dx^2 and
 //    sum aT g_{r,g,b,depth}; dy is constant along a strip row, so the y moments follow from
-//    those; two exchanges inside each quad of lanes finish the sums, and the quad adds its
-//    entry's ten sums into the Gaussian's row of `sums`, four neighbouring columns per atomic
-//    instruction.
+//    those; three exchanges inside each group of eight lanes finish the sums, and the group adds its
+//    entry's ten sums into the Gaussian's row of `sums`, eight neighbouring columns in one atomic
+//    instruction and the last two in another.  Eight rows rather than sixteen keep the wavefront's
+//    LDS under 10 KB, which is what lets sixteen of them share a CU.
 // All ten sums of the reference (mean2D x/y, conic xx/xy/yy, opacity, colour r/g/b, depth)
 // are linear in u and aT, which is what makes the split possible.
 
-constexpr int kRows = 16;     // entries gathered before the entry-parallel part runs
+constexpr int kRows = 8;      // entries gathered before the entry-parallel part runs
 // Pixel p of the strip sits in column p + (p >> 5) of a row of kRowStride words: with these two
-// numbers neither the per-pixel writes nor the per-(entry, strip row) reads below hit an LDS
+// numbers neither the per-pixel writes nor the per-(entry, strip row, half row) reads below hit an LDS
 // bank twice within a half wavefront.
 constexpr int kRowStride = 66;
 __device__ __forceinline__ int row_column(int pixel) { return pixel + (pixel >> 5); }
@@ -592,32 +593,34 @@ struct StripFrame {
 	float ddelx_dx, ddely_dy;
 };
 
-template <int QuadPerm>
-__device__ __forceinline__ float quad_exchange_add(float v)
+template <int DppCtrl>
+__device__ __forceinline__ float dpp_exchange_add(float v)
 {
-	const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), QuadPerm, 0xF, 0xF, true);
+	const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), DppCtrl, 0xF, 0xF, true);
 	return v + __builtin_bit_cast(float, moved);
 }
 
-// Entry-parallel part for the first `rows` rows.  Lane (e = lane >> 2, h = lane & 3) sums row e
-// over the 16 pixels of strip row h; the four lanes of a quad then hold one entry and add the
-// entry's ten sums into the Gaussian's row of `sums`, four neighbouring columns per instruction.
+// Entry-parallel part for the first `rows` rows.  Lane (e = lane >> 3, h = (lane >> 1) & 3, half = lane & 1)
+// sums row e over the 8 pixels of one half of strip row h; the eight lanes of an entry then add up what
+// they hold (three exchanges inside their group of eight) and add the entry's ten sums into the Gaussian's
+// row of `sums`: eight neighbouring columns in one atomic instruction, the last two in a second.
 __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, const StripFrame& f, const BlendArgs& a,
                                            int lane)
 {
 #pragma clang fp contract(fast)
 	__builtin_amdgcn_wave_barrier();
-	const int e = lane >> 2, h = lane & 3;
+	const int e = lane >> 3, h = (lane >> 1) & 3, half = lane & 1, j = lane & 7;
 	const float2 xy = st.row_xy[e];
 	const float dy = xy.y - (f.y0 + (float)h);
+	const float x_first = f.x0 + (float)(8 * half);
 	float s0 = 0.f, sx = 0.f, sxx = 0.f, cr = 0.f, cg = 0.f, cb = 0.f, cdp = 0.f;
-	const int col0 = row_column(h * 16);
+	const int col0 = row_column(h * 16 + 8 * half);
 	const float* urow = st.u + e * kRowStride + col0;
 	const float* arow = st.at + e * kRowStride + col0;
 #pragma unroll
-	for (int step = 0; step < 16; step++) {
+	for (int step = 0; step < 8; step++) {
 		const float uu = urow[step], tt = arow[step];
-		const float dx = xy.x - (f.x0 + (float)step);
+		const float dx = xy.x - (x_first + (float)step);
 		const float t = uu * dx;
 		s0 += uu;
 		sx += t;
@@ -627,11 +630,16 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 		cb += tt * st.upstream[2][col0 + step];
 		cdp += tt * st.upstream[3][col0 + step];
 	}
-	float v[10] = {s0, sx, dy * s0, sxx, dy * sx, dy * dy * s0, cr, cg, cb, cdp};
+	// the two halves of the strip row first (dy is theirs in common), then the four strip rows
+	float w[7] = {s0, sx, sxx, cr, cg, cb, cdp};
+#pragma unroll
+	for (int q = 0; q < 7; q++)
+		w[q] = dpp_exchange_add<0xB1>(w[q]);  // quad_perm:[1,0,3,2]
+	float v[10] = {w[0], w[1], dy * w[0], w[2], dy * w[1], dy * dy * w[0], w[3], w[4], w[5], w[6]};
 #pragma unroll
 	for (int q = 0; q < 10; q++) {
-		v[q] = quad_exchange_add<0xB1>(v[q]);  // quad_perm:[1,0,3,2]
-		v[q] = quad_exchange_add<0x4E>(v[q]);  // quad_perm:[2,3,0,1]
+		v[q] = dpp_exchange_add<0x4E>(v[q]);   // quad_perm:[2,3,0,1]
+		v[q] = dpp_exchange_add<0x141>(v[q]);  // row_half_mirror: the other quad of the eight
 	}
 	if (e < rows) {
 		const float4 co = st.row_conic[e];
@@ -639,14 +647,12 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 		const float m0 = -co.w * f.ddelx_dx * (co.x * Sx + co.y * Sy);
 		const float m1 = -co.w * f.ddely_dy * (co.z * Sy + co.y * Sx);
 		const float k0 = -0.5f * co.w * Sxx, k1 = -0.5f * co.w * Sxy, k3 = -0.5f * co.w * Syy;
-		// column 4 j + h of the row: see SumCol
-		const float w0 = h == 0 ? m0 : h == 1 ? m1 : h == 2 ? k0 : k1;
-		const float w1 = h == 0 ? k3 : h == 1 ? S0 : h == 2 ? v[6] : v[7];
-		const float w2 = h == 0 ? v[8] : h == 1 ? v[9] : 0.f;
-		float* row = a.sums + (size_t)kSumCols * st.row_id[e] + h;
-		if (w0 != 0.f) unsafeAtomicAdd(row, w0);
-		if (w1 != 0.f) unsafeAtomicAdd(row + 4, w1);
-		if (w2 != 0.f) unsafeAtomicAdd(row + 8, w2);
+		// lane j of the eight takes column j of the row, lanes 0 and 1 also columns 8 and 9: see SumCol
+		const float first = j == 0 ? m0 : j == 1 ? m1 : j == 2 ? k0 : j == 3 ? k1 : j == 4 ? k3 : j == 5 ? S0 : j == 6 ? v[6] : v[7];
+		const float second = j == 0 ? v[8] : j == 1 ? v[9] : 0.f;
+		float* row = a.sums + (size_t)kSumCols * st.row_id[e] + j;
+		if (first != 0.f) unsafeAtomicAdd(row, first);
+		if (second != 0.f) unsafeAtomicAdd(row + 8, second);
 	}
 	__builtin_amdgcn_wave_barrier();
 }
@@ -711,7 +717,9 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	}
 }
 
-__global__ __launch_bounds__(64) void blend_backward_kernel(BlendBatch batch)
+// 128 registers and under 10 KB of LDS: four wavefronts per SIMD (three, as the compiler chooses by itself, were
+// measured 19 % slower; five spill)
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void blend_backward_kernel(BlendBatch batch)
 {
 	__shared__ BackwardStage s_stage;
 

@@ -245,6 +245,7 @@ def _gradient_outputs(P, M, has_scales, device, make):
     for k, shape in shapes.items():
         out[k] = flat[at:at + math.prod(shape)].view(shape)
         at += sizes[k]
+    out["block"] = flat  # the eight above as one tensor
     out["sums"] = make((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
     if not has_scales and make is not torch.zeros:
         out["scales"].zero_()
@@ -520,7 +521,28 @@ class _RasterizeFrame(torch.autograd.Function):
                     rec["binning"] = torch.empty(binning_bytes, **byte)
                     arr[j].R = rec["rendered"]
                     arr[j].binning_ws, arr[j].binning_bytes = ptr(rec["binning"]), binning_bytes
+                # With a second stream and a backward to come, the gradient tensors are made now and cleared on that
+                # stream while this stream bins and blends (the backward blend leaves the clearing no room beside it).
+                cleared, cleared_event = None, None
+                side = next((h for h in streams if h != main), None) if streams is not None else None
+                if side is not None and any(ctx.needs_input_grad[2:]):
+                    cleared = {}
+                    for k in live:
+                        rec = records[k]
+                        cleared[k] = _gradient_outputs(rec["P"], rec["M"], rec["t"]["scales"].numel() != 0, device, torch.empty)
+                    begun = torch.cuda.Event()
+                    begun.record(torch.cuda.current_stream(device))
+                    side_stream = torch.cuda.ExternalStream(side, device=device)
+                    side_stream.wait_event(begun)  # whatever used this memory before did so ahead of this point
+                    with torch.cuda.stream(side_stream):
+                        for out in cleared.values():
+                            for name in ("block", "sums"):
+                                out[name].zero_()
+                                out[name].record_stream(side_stream)  # not to be handed out again before this is done
+                        cleared_event = torch.cuda.Event()
+                        cleared_event.record(side_stream)
                 check(lib.rgs_frame_forward_raster(len(live), arr, C.byref(view), C.c_void_p(main), debug))
+        ctx.cleared, ctx.cleared_event = (cleared, cleared_event) if live else (None, None)
         ctx.settings = settings
         ctx.streams = streams
         ctx.meta = []
@@ -564,7 +586,8 @@ class _RasterizeFrame(torch.autograd.Function):
             has_scales = scales.numel() != 0
             # Only rendered Gaussians get their gradient rows written; the library clears the rest (beside the blend,
             # on the second stream, if it is given one).
-            out = _gradient_outputs(P, M, has_scales, device, torch.empty)
+            ready = ctx.cleared.pop(k, None) if ctx.cleared else None  # made and cleared during the forward; used once
+            out = ready if ready is not None else _gradient_outputs(P, M, has_scales, device, torch.empty)
             keep.append(out)   # its scratch rows must outlive the library call below
             t = dict(bg=_dev_f32(rs.bg, device, "bg"), low=_dev_f32(rs.range_low, device, "range_low"),
                      up=_dev_f32(rs.range_up, device, "range_up"), g_color=_dev_f32(g_color, device, "grad_color"),
@@ -593,7 +616,7 @@ class _RasterizeFrame(torch.autograd.Function):
             L.dL_dmean3D, L.dL_dcov3D, L.dL_dsh = ptr(out["means3D"]), ptr(out["cov3D"]), ptr(out["sh"])
             L.dL_dscale = ptr(out["scales"]) if has_scales else C.c_void_p(0)
             L.dL_drot = ptr(out["rotations"]) if has_scales else C.c_void_p(0)
-            L.outputs_zeroed = 0
+            L.outputs_zeroed = 1 if ready is not None else 0
             base = out["means2D"]
             L.grad_block = base.data_ptr()
             L.grad_block_bytes = out["rotations"].data_ptr() + out["rotations"].numel() * 4 - base.data_ptr()
@@ -602,6 +625,8 @@ class _RasterizeFrame(torch.autograd.Function):
                             out["scales"], out["rotations"]))
         if live:
             with torch.cuda.device(device):
+                if ctx.cleared_event is not None:
+                    torch.cuda.current_stream(device).wait_event(ctx.cleared_event)
                 check(lib.rgs_frame_backward(live, arr, C.byref(view), C.c_void_p(main), int(bool(rs0.debug))))
         flat = []
         for k in range(K):
