@@ -511,16 +511,6 @@ class _RasterizeFrame(torch.autograd.Function):
                 L.geom_bytes, L.image_bytes = geom_bytes, image_bytes
                 L.out_color, L.out_depth, L.out_alpha = ptr(package[0:3]), ptr(package[3:4]), ptr(package[4:5])
             if live:
-                counts = _frame_counts(device, len(live))
-                check(lib.rgs_frame_forward_geom(len(live), arr, C.byref(view), C.c_void_p(counts.data_ptr()), C.c_void_p(main), debug))
-                got = counts[:len(live)].tolist()
-                for j, k in enumerate(live):
-                    rec = records[k]
-                    rec["rendered"] = int(got[j])
-                    binning_bytes = lib.rgs_binning_bytes(rec["rendered"]) if rec["rendered"] > 0 else 0
-                    rec["binning"] = torch.empty(binning_bytes, **byte)
-                    arr[j].R = rec["rendered"]
-                    arr[j].binning_ws, arr[j].binning_bytes = ptr(rec["binning"]), binning_bytes
                 # With a second stream and a backward to come, the gradient tensors are made now and cleared on that
                 # stream while this stream bins and blends (the backward blend leaves the clearing no room beside it).
                 cleared, cleared_event = None, None
@@ -541,6 +531,16 @@ class _RasterizeFrame(torch.autograd.Function):
                                 out[name].record_stream(side_stream)  # not to be handed out again before this is done
                         cleared_event = torch.cuda.Event()
                         cleared_event.record(side_stream)
+                counts = _frame_counts(device, len(live))
+                check(lib.rgs_frame_forward_geom(len(live), arr, C.byref(view), C.c_void_p(counts.data_ptr()), C.c_void_p(main), debug))
+                got = counts[:len(live)].tolist()
+                for j, k in enumerate(live):
+                    rec = records[k]
+                    rec["rendered"] = int(got[j])
+                    binning_bytes = lib.rgs_binning_bytes(rec["rendered"]) if rec["rendered"] > 0 else 0
+                    rec["binning"] = torch.empty(binning_bytes, **byte)
+                    arr[j].R = rec["rendered"]
+                    arr[j].binning_ws, arr[j].binning_bytes = ptr(rec["binning"]), binning_bytes
                 check(lib.rgs_frame_forward_raster(len(live), arr, C.byref(view), C.c_void_p(main), debug))
         ctx.cleared, ctx.cleared_event = (cleared, cleared_event) if live else (None, None)
         ctx.settings = settings
