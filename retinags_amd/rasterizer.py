@@ -656,8 +656,10 @@ def rasterize_frame(rasterizers, inputs, streams=None):
     """All layers of a frame through one call.  `rasterizers`: K GaussianRasterizer (their settings share the
     camera and the image size); `inputs`: K dicts with the keyword arguments of GaussianRasterizer.forward
     (means3D, means2D, opacities, shs / colors_precomp, scales + rotations / cov3D_precomp); `streams`: None,
-    or for every layer the handle of a HIP stream; the first that is not the current stream is used by the
-    backward for its memory-bound work, beside the blend (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
+    or for every layer the handle of a HIP stream; the first that is not the current stream takes memory-bound work
+    beside the kernels of the current one: if a backward is to come, the gradient tensors are made and cleared on it
+    during the forward, and the backward runs the per-Gaussian part of the layers whose blend is done on it
+    (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
     forward calls, and differentiates like them."""
     flat = []
     for rz, kw in zip(rasterizers, inputs):
