@@ -615,7 +615,7 @@ void launch_duplicate_with_keys(const DuplicateJob* jobs, int count, int grid_x,
 		}
 		// every workgroup ends with an atomic add per digit into its job's counts: enough of them to fill the GPU several
 		// times over, each over many runs of positions, rather than one per run
-		const size_t most = nj >= 8 ? 512 : 4096 / (size_t)nj;  // twice and four times as many were measured slower
+		const size_t most = nj >= 8 ? 512 : nj >= 4 ? 4096 / (size_t)nj : 1024;  // twice and four times as many were measured slower
 		blocks = blocks < most ? blocks : most;
 		hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((unsigned)blocks, (unsigned)nj), dim3(256),
 		                   ndc_in_lds ? table * sizeof(float) : 0, s, b, grid_x, grid_y, ndc_in_lds);

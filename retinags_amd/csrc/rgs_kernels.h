@@ -331,9 +331,11 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 // Output positions a workgroup of the key duplication writes, and the table that tells each such workgroup at
 // which Gaussian (of the depth order) its positions begin: entry b = the Gaussian whose instances include position
 // b * kDupPositions.  The scan that produces the offsets fills it; it has room for dup_first_words(P) workgroups,
-// those beyond (more than 16 instances per Gaussian on average) search the offsets instead.
-constexpr int kDupPositions = 1024;
-constexpr size_t dup_first_words(size_t P) { return P / 64 + 2; }
+// those beyond (more than 16 instances per Gaussian on average) search the offsets instead.  One position per thread:
+// with 1 024 positions (four per thread) the kernel held 117 registers and 4 wavefronts per SIMD; with 256 it holds
+// 79 and 6, and is 22 % faster where the Gaussians are small.
+constexpr int kDupPositions = 256;
+constexpr size_t dup_first_words(size_t P) { return P / 16 + 2; }
 // The key duplication also counts the digits of the tiles it writes, which is what the sort of its keys starts
 // from: counts[256 p + d] = keys whose tile bits [8 p, 8 p + 8) are d, in kTileDigitWords words that are zero when it
 // starts (the depth order leaves them so, and so does the tile-range kernel, the last to run after they were read).
