@@ -582,9 +582,6 @@ struct BackwardStage {  // wave-private
 	uint32_t id[kChunk];
 	float u[kRows * kRowStride];   // [row][row_column(pixel)]
 	float at[kRows * kRowStride];  // [row][row_column(pixel)]
-	float4 row_conic[kRows];
-	float2 row_xy[kRows];
-	uint32_t row_id[kRows];
 	float upstream[4][kRowStride];  // dL/dpixel r, g, b, depth of the strip's 64 pixels, by row_column
 };
 
@@ -604,13 +601,17 @@ __device__ __forceinline__ float dpp_exchange_add(float v)
 // sums row e over the 8 pixels of one half of strip row h; the eight lanes of an entry then add up what
 // they hold (three exchanges inside their group of eight) and add the entry's ten sums into the Gaussian's
 // row of `sums`: eight neighbouring columns in one atomic instruction, the last two in a second.
-__device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, const StripFrame& f, const BlendArgs& a,
-                                           int lane)
+// `row_slots` holds, one byte per row, which staged entry of the current chunk the row belongs to: the entry's centre,
+// conic and Gaussian are read from where the chunk was staged (so the rows are flushed before the next chunk is).
+__device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, uint64_t row_slots, const StripFrame& f,
+                                           const BlendArgs& a, int lane)
 {
 #pragma clang fp contract(fast)
 	__builtin_amdgcn_wave_barrier();
 	const int e = lane >> 3, h = (lane >> 1) & 3, half = lane & 1, j = lane & 7;
-	const float2 xy = st.row_xy[e];
+	const int slot = (int)((row_slots >> (8 * e)) & 0xFFull);
+	const float4 centre = st.geom[slot];
+	const float2 xy = {centre.x, centre.y};
 	const float dy = xy.y - (f.y0 + (float)h);
 	const float x_first = f.x0 + (float)(8 * half);
 	float s0 = 0.f, sx = 0.f, sxx = 0.f, cr = 0.f, cg = 0.f, cb = 0.f, cdp = 0.f;
@@ -642,7 +643,7 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 		v[q] = dpp_exchange_add<0x141>(v[q]);  // row_half_mirror: the other quad of the eight
 	}
 	if (e < rows) {
-		const float4 co = st.row_conic[e];
+		const float4 co = st.conic[slot];
 		const float S0 = v[0], Sx = v[1], Sy = v[2], Sxx = v[3], Sxy = v[4], Syy = v[5];
 		const float m0 = -co.w * f.ddelx_dx * (co.x * Sx + co.y * Sy);
 		const float m1 = -co.w * f.ddely_dy * (co.z * Sy + co.y * Sx);
@@ -650,7 +651,7 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 		// lane j of the eight takes column j of the row, lanes 0 and 1 also columns 8 and 9: see SumCol
 		const float first = j == 0 ? m0 : j == 1 ? m1 : j == 2 ? k0 : j == 3 ? k1 : j == 4 ? k3 : j == 5 ? S0 : j == 6 ? v[6] : v[7];
 		const float second = j == 0 ? v[8] : j == 1 ? v[9] : 0.f;
-		float* row = a.sums + (size_t)kSumCols * st.row_id[e] + j;
+		float* row = a.sums + (size_t)kSumCols * st.id[slot] + j;
 		if (first != 0.f) unsafeAtomicAdd(row, first);
 		if (second != 0.f) unsafeAtomicAdd(row + 8, second);
 	}
@@ -659,7 +660,7 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, co
 
 // Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
 __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
-                                               const float4 co, BackwardStage& st, int slot, int& rows,
+                                               const float4 co, BackwardStage& st, int slot, int& rows, uint64_t& row_slots,
                                                const StripFrame& f, const PixelRay& ray, const BlendArgs& a,
                                                const BoxFrame& box, int lane)
 {
@@ -705,15 +706,12 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 		return;
 	st.u[rows * kRowStride + row_column(lane)] = u;
 	st.at[rows * kRowStride + row_column(lane)] = aT;
-	if (lane == 0) {
-		st.row_conic[rows] = co;
-		st.row_xy[rows] = float2{g.x, g.y};
-		st.row_id[rows] = st.id[slot];
-	}
+	row_slots |= (uint64_t)slot << (8 * rows);
 	rows++;
 	if (rows == kRows) {
-		flush_rows(st, kRows, f, a, lane);
+		flush_rows(st, kRows, row_slots, f, a, lane);
 		rows = 0;
+		row_slots = 0ull;
 	}
 }
 
@@ -768,6 +766,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 	st.upstream[2][row_column(lane)] = p.g_b;
 	st.upstream[3][row_column(lane)] = p.g_depth;
 	int rows = 0;
+	uint64_t row_slots = 0ull;
 
 	// Lane l of the chunk that starts `first` entries from the back takes filed entry
 	// filed-1-first-l: its list position (and box flag), through that the Gaussian's index,
@@ -821,15 +820,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 			           q3 = (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
 			if (__ballot(q0 | q1 | q2 | q3) == 0ull)
 				continue;
-			backward_visit(p, q0, w0, g0, c0, st, k, rows, frame, ray, a, box, lane);
-			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, frame, ray, a, box, lane);
-			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, frame, ray, a, box, lane);
-			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, frame, ray, a, box, lane);
+			backward_visit(p, q0, w0, g0, c0, st, k, rows, row_slots, frame, ray, a, box, lane);
+			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, row_slots, frame, ray, a, box, lane);
+			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, row_slots, frame, ray, a, box, lane);
+			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, row_slots, frame, ray, a, box, lane);
+		}
+		// the rows point into this chunk's staged entries: they go before the next chunk takes their place
+		if (rows > 0) {
+			flush_rows(st, rows, row_slots, frame, a, lane);
+			rows = 0;
+			row_slots = 0ull;
 		}
 		__builtin_amdgcn_wave_barrier();
 	}
-	if (rows > 0)
-		flush_rows(st, rows, frame, a, lane);
 }
 
 // Strips by decreasing number of entries to walk, in kStripClasses classes of 8 (longer ones share
