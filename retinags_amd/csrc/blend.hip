@@ -658,6 +658,13 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 	__builtin_amdgcn_wave_barrier();
 }
 
+// behind = keep * behind + add, in the register that holds `behind`: written as an expression, the compiler forms the
+// sum in the register of `add` and copies it over afterwards, one more instruction per colour channel and visit.
+__device__ __forceinline__ void update_behind(float& behind, float keep, float add)
+{
+	asm("v_fma_f32 %0, %1, %0, %2" : "+v"(behind) : "v"(keep), "v"(add));
+}
+
 // Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
 __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
                                                const float4 co, BackwardStage& st, int slot, int& rows, uint64_t& row_slots,
@@ -693,11 +700,11 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 			dL_dopa += (cd.w - p.behind_depth) * p.g_depth;
 			dL_dopa += (1 - p.behind_alpha) * p.g_alpha;
 			dL_dopa *= p.T;
-			p.behind_r = alpha * cd.x + keep * p.behind_r;
-			p.behind_g = alpha * cd.y + keep * p.behind_g;
-			p.behind_b = alpha * cd.z + keep * p.behind_b;
-			p.behind_depth = alpha * cd.w + keep * p.behind_depth;
-			p.behind_alpha = alpha + keep * p.behind_alpha;
+			update_behind(p.behind_r, keep, alpha * cd.x);
+			update_behind(p.behind_g, keep, alpha * cd.y);
+			update_behind(p.behind_b, keep, alpha * cd.z);
+			update_behind(p.behind_depth, keep, alpha * cd.w);
+			update_behind(p.behind_alpha, keep, alpha);
 			dL_dopa += (-p.T_final * inv_one_minus_alpha) * p.bg_dot_dpixel;
 			u = G * dL_dopa;
 		}
