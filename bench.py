@@ -304,8 +304,9 @@ def measure(args, config, forward_only, asides, cpu):
         "tile_ranges": 4.0 * R_tot + 16.0 * T * K,
         # the sorted keys in, the filed positions out (at most four per instance; counted as one)
         "strip_filing": 8.0 * R_tot + 16.0 * T * K,
-        # the eight gradient tensors and the rows of sums, written once
-        "clear_gradients": (4.0 * (3 + 1 + 3 + 3 + 6 + 48 + 3 + 4) + 48.0) * P_tot,
+        # the six gradient tensors a frame hands out (mean2D, opacity, mean3D, SH, scale, rotation) and the rows of sums,
+        # written once
+        "clear_gradients": (4.0 * (3 + 1 + 3 + 48 + 3 + 4) + 48.0) * P_tot,
         # rows of the rendered Gaussians only: sums, mean, SH, scale, rotation in;
         # the eight gradient rows out
         "preprocess_backward": (285.0 + 284.0) * P_vis,

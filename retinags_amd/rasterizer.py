@@ -229,23 +229,27 @@ def _rasterize_forward(*args):
     return _forward_blend(_forward_geometry(*args, wait=True))
 
 
-def _gradient_outputs(P, M, has_scales, device, make):
+def _gradient_outputs(P, M, has_scales, device, make, scratch=()):
     """The eight dense gradient tensors of K/rasterize_points.cu:165-174, carved out of one
     allocation made with `make` (torch.empty or torch.zeros: one fill instead of eight), and the
     backward's scratch for the per-Gaussian sums in an allocation of its own, so that a gradient
     the caller keeps (the means2D gradient, say, for densification statistics) does not hold on to
     the scratch.  The eight do share one block: keeping any of them keeps all (about 280 bytes
     per Gaussian with SH degree 3).  Without scales the scale / rotation gradients are zeros in
-    either case."""
+    either case.  `scratch` names those of the eight that the caller hands to nobody (the colour
+    gradient when the colours come from SH, the covariance gradient when it comes from scale and
+    rotation): they lie behind the others, and out["block"], the part that has to be zero where
+    no Gaussian was rendered, ends before them."""
     shapes = {"means2D": (P, 3), "opacity": (P, 1), "colors": (P, 3), "means3D": (P, 3), "cov3D": (P, 6),
               "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4)}
+    order = [k for k in shapes if k not in scratch] + [k for k in shapes if k in scratch]
     sizes = {k: (math.prod(v) + 63) // 64 * 64 for k, v in shapes.items()}  # 256-byte aligned parts
     flat = make((sum(sizes.values()),), dtype=torch.float32, device=device)
     out, at = {}, 0
-    for k, shape in shapes.items():
-        out[k] = flat[at:at + math.prod(shape)].view(shape)
+    for k in order:
+        out[k] = flat[at:at + math.prod(shapes[k])].view(shapes[k])
         at += sizes[k]
-    out["block"] = flat  # the eight above as one tensor
+    out["block"] = flat[:sum(sizes[k] for k in order if k not in scratch)]  # what has to be cleared, as one tensor
     out["sums"] = make((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
     if not has_scales and make is not torch.zeros:
         out["scales"].zero_()
@@ -519,7 +523,9 @@ class _RasterizeFrame(torch.autograd.Function):
                     cleared = {}
                     for k in live:
                         rec = records[k]
-                        cleared[k] = _gradient_outputs(rec["P"], rec["M"], rec["t"]["scales"].numel() != 0, device, torch.empty)
+                        t_k = rec["t"]
+                        cleared[k] = _gradient_outputs(rec["P"], rec["M"], t_k["scales"].numel() != 0, device, torch.empty,
+                                                       scratch=_frame_scratch(t_k["colors_precomp"], t_k["cov3Ds_precomp"]))
                     begun = torch.cuda.Event()
                     begun.record(torch.cuda.current_stream(device))
                     side_stream = torch.cuda.ExternalStream(side, device=device)
@@ -587,7 +593,8 @@ class _RasterizeFrame(torch.autograd.Function):
             # Only rendered Gaussians get their gradient rows written; the library clears the rest (beside the blend,
             # on the second stream, if it is given one).
             ready = ctx.cleared.pop(k, None) if ctx.cleared else None  # made and cleared during the forward; used once
-            out = ready if ready is not None else _gradient_outputs(P, M, has_scales, device, torch.empty)
+            out = ready if ready is not None else _gradient_outputs(P, M, has_scales, device, torch.empty,
+                                                                    scratch=_frame_scratch(colors_precomp, cov3Ds))
             keep.append(out)   # its scratch rows must outlive the library call below
             t = dict(bg=_dev_f32(rs.bg, device, "bg"), low=_dev_f32(rs.range_low, device, "range_low"),
                      up=_dev_f32(rs.range_up, device, "range_up"), g_color=_dev_f32(g_color, device, "grad_color"),
@@ -617,9 +624,8 @@ class _RasterizeFrame(torch.autograd.Function):
             L.dL_dscale = ptr(out["scales"]) if has_scales else C.c_void_p(0)
             L.dL_drot = ptr(out["rotations"]) if has_scales else C.c_void_p(0)
             L.outputs_zeroed = 1 if ready is not None else 0
-            base = out["means2D"]
-            L.grad_block = base.data_ptr()
-            L.grad_block_bytes = out["rotations"].data_ptr() + out["rotations"].numel() * 4 - base.data_ptr()
+            L.grad_block = out["block"].data_ptr()
+            L.grad_block_bytes = out["block"].numel() * 4
             L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
             results.append((out["means2D"], out["colors"], out["opacity"], out["means3D"], out["cov3D"], out["sh"],
                             out["scales"], out["rotations"]))
@@ -636,6 +642,11 @@ class _RasterizeFrame(torch.autograd.Function):
                      g_opacity, g_scales if scales.numel() else None, g_rot if rotations.numel() else None,
                      g_cov3D if cov3Ds.numel() else None]
         return (None, None, *flat)
+
+
+def _frame_scratch(colors_precomp, cov3Ds_precomp):
+    """Which gradient arrays of a frame's layer nobody gets to see: see _gradient_outputs."""
+    return tuple(name for name, given in (("colors", colors_precomp), ("cov3D", cov3Ds_precomp)) if given.numel() == 0)
 
 
 _frame_count_words = threading.local()
