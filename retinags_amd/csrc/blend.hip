@@ -289,11 +289,14 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 			} else {
 				const uint32_t entry = st.entry[half][slot];
 				const float4 cd = st.cd[entry];
-				p.C0 += cd.x * alpha * p.T;
-				p.C1 += cd.y * alpha * p.T;
-				p.C2 += cd.z * alpha * p.T;
-				p.weight += alpha * p.T;
-				p.D += cd.w * alpha * p.T;
+				// The sums feed no decision (the images are compared by tolerance): one product alpha T and a fused
+				// multiply-add per channel instead of the reference's two products and an add each (forward.cu:378-385).
+				const float weight = alpha * p.T;
+				p.C0 = __builtin_fmaf(cd.x, weight, p.C0);
+				p.C1 = __builtin_fmaf(cd.y, weight, p.C1);
+				p.C2 = __builtin_fmaf(cd.z, weight, p.C2);
+				p.weight += weight;
+				p.D = __builtin_fmaf(cd.w, weight, p.D);
 				p.T = test_T;
 				p.last_contributor = st.position[entry];
 				p.last_filed = first + entry + 1u;
