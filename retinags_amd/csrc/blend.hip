@@ -564,11 +564,13 @@ __global__ __launch_bounds__(256) void blend_count_kernel(BlendArgs a)
 // are linear in u and aT, which is what makes the split possible.
 
 constexpr int kRows = 8;      // entries gathered before the entry-parallel part runs
-// Pixel p of the strip sits in column p + (p >> 5) of a row of kRowStride words: with these two
-// numbers neither the per-pixel writes nor the per-(entry, strip row, half row) reads below hit an LDS
-// bank twice within a half wavefront.
-constexpr int kRowStride = 66;
-__device__ __forceinline__ int row_column(int pixel) { return pixel + (pixel >> 5); }
+// Pixel p of the strip sits in column p + (p >> 4) of a row of kRowStride (u, alpha T) pairs, and its four upstream
+// gradients in element p + (p >> 3) of their array: the LDS has 32 banks of 4 bytes, an 8-byte access is served 16
+// lanes at a time and a 16-byte access 8 lanes at a time, and with these numbers neither the per-pixel writes nor
+// the per-(entry, strip row, half row) reads below hit a bank twice within such a group.
+constexpr int kRowStride = 68;
+__device__ __forceinline__ int row_column(int pixel) { return pixel + (pixel >> 4); }
+__device__ __forceinline__ int upstream_column(int pixel) { return pixel + (pixel >> 3); }
 
 struct BackwardPixel {
 	float T, T_final;
@@ -583,9 +585,8 @@ struct BackwardStage {  // wave-private
 	float4 cd[kChunk];
 	uint32_t entry[kChunk + 3];  // 0-based position in the tile list
 	uint32_t id[kChunk];
-	float u[kRows * kRowStride];   // [row][row_column(pixel)]
-	float at[kRows * kRowStride];  // [row][row_column(pixel)]
-	float upstream[4][kRowStride];  // dL/dpixel r, g, b, depth of the strip's 64 pixels, by row_column
+	float2 u_at[kRows * kRowStride];  // [row][row_column(pixel)]: (u, alpha T)
+	float4 upstream[72];              // dL/dpixel r, g, b, depth of the strip's 64 pixels, by upstream_column
 };
 
 struct StripFrame {
@@ -619,20 +620,22 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 	const float x_first = f.x0 + (float)(8 * half);
 	float s0 = 0.f, sx = 0.f, sxx = 0.f, cr = 0.f, cg = 0.f, cb = 0.f, cdp = 0.f;
 	const int col0 = row_column(h * 16 + 8 * half);
-	const float* urow = st.u + e * kRowStride + col0;
-	const float* arow = st.at + e * kRowStride + col0;
+	const float2* row = st.u_at + e * kRowStride + col0;
+	const float4* upstream = st.upstream + upstream_column(h * 16 + 8 * half);
 #pragma unroll
 	for (int step = 0; step < 8; step++) {
-		const float uu = urow[step], tt = arow[step];
+		const float2 ua = row[step];
+		const float4 g = upstream[step];
+		const float uu = ua.x, tt = ua.y;
 		const float dx = xy.x - (x_first + (float)step);
 		const float t = uu * dx;
 		s0 += uu;
 		sx += t;
 		sxx += t * dx;
-		cr += tt * st.upstream[0][col0 + step];
-		cg += tt * st.upstream[1][col0 + step];
-		cb += tt * st.upstream[2][col0 + step];
-		cdp += tt * st.upstream[3][col0 + step];
+		cr += tt * g.x;
+		cg += tt * g.y;
+		cb += tt * g.z;
+		cdp += tt * g.w;
 	}
 	// the two halves of the strip row first (dy is theirs in common), then the four strip rows
 	float w[7] = {s0, sx, sxx, cr, cg, cb, cdp};
@@ -714,8 +717,7 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	}
 	if (__ballot(valid) == 0ull)
 		return;
-	st.u[rows * kRowStride + row_column(lane)] = u;
-	st.at[rows * kRowStride + row_column(lane)] = aT;
+	st.u_at[rows * kRowStride + row_column(lane)] = float2{u, aT};
 	row_slots |= (uint64_t)slot << (8 * rows);
 	rows++;
 	if (rows == kRows) {
@@ -771,10 +773,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 		p.g_alpha = a.dL_dalpha ? a.dL_dalpha[pix_id] : 0.f;
 	}
 	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
-	st.upstream[0][row_column(lane)] = p.g_r;
-	st.upstream[1][row_column(lane)] = p.g_g;
-	st.upstream[2][row_column(lane)] = p.g_b;
-	st.upstream[3][row_column(lane)] = p.g_depth;
+	st.upstream[upstream_column(lane)] = float4{p.g_r, p.g_g, p.g_b, p.g_depth};
 	int rows = 0;
 	uint64_t row_slots = 0ull;
 
