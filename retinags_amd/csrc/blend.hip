@@ -674,8 +674,7 @@ __device__ __forceinline__ void update_behind(float& behind, float keep, float a
 // Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
 __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
                                                const float4 co, BackwardStage& st, int slot, int& rows, uint64_t& row_slots,
-                                               const StripFrame& f, const PixelRay& ray, const BlendArgs& a,
-                                               const BoxFrame& box, int lane)
+                                               const StripFrame& f, const PixelRay& ray, const BlendArgs& a, int lane)
 {
 	if (__ballot(candidate) == 0ull)
 		return;
@@ -685,7 +684,9 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	if (candidate) {
 		const float G = exp_of_exponent(power);
 		const float alpha = fminf(0.99f, co.w * G);
-		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, box))) {
+		// the box and the inverse projection are read where they are needed (few strips straddle a face of their
+		// box): kept in scalar registers for the whole walk they crowd out the candidate masks of a step
+		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, load_box_frame(a)))) {
 			// From here on nothing feeds a decision: gradients are compared by tolerance, so the
 			// compiler may contract multiply-adds and the divisions use the hardware reciprocal.
 #pragma clang fp contract(fast)
@@ -746,7 +747,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 	const uint32_t pix_id = (uint32_t)a.W * py + px;
 	const float2 pixf = {(float)px, (float)py};
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
-	const BoxFrame box = load_box_frame(a);
 	const size_t plane = (size_t)a.H * a.W;
 	const float strip_x0 = (float)(tx * kTile), strip_y0 = (float)(ty * kTile + wave * 4);
 	const StripFrame frame = {strip_x0, strip_y0, (float)(0.5 * a.W), (float)(0.5 * a.H)};
@@ -829,10 +829,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 			           q3 = (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
 			if (__ballot(q0 | q1 | q2 | q3) == 0ull)
 				continue;
-			backward_visit(p, q0, w0, g0, c0, st, k, rows, row_slots, frame, ray, a, box, lane);
-			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, row_slots, frame, ray, a, box, lane);
-			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, row_slots, frame, ray, a, box, lane);
-			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, row_slots, frame, ray, a, box, lane);
+			backward_visit(p, q0, w0, g0, c0, st, k, rows, row_slots, frame, ray, a, lane);
+			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, row_slots, frame, ray, a, lane);
+			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, row_slots, frame, ray, a, lane);
+			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, row_slots, frame, ray, a, lane);
 		}
 		// the rows point into this chunk's staged entries: they go before the next chunk takes their place
 		if (rows > 0) {
