@@ -823,16 +823,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 			float2 d;
 			const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
 			            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
-			const bool q0 = (p0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z),
-			           q1 = (p1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z),
-			           q2 = (p2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z),
-			           q3 = (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z);
-			if (__ballot(q0 | q1 | q2 | q3) == 0ull)
-				continue;
-			backward_visit(p, q0, w0, g0, c0, st, k, rows, row_slots, frame, ray, a, lane);
-			backward_visit(p, q1, w1, g1, c1, st, k + 1, rows, row_slots, frame, ray, a, lane);
-			backward_visit(p, q2, w2, g2, c2, st, k + 2, rows, row_slots, frame, ray, a, lane);
-			backward_visit(p, q3, w3, g3, c3, st, k + 3, rows, row_slots, frame, ray, a, lane);
+			// Each entry's candidates are formed right where its visit looks at them (the visit starts with their
+			// ballot): nearly every walked entry has some, so a test for the four together would save little, and
+			// four sets of flags kept alive across the visits are packed into a byte mask by the compiler, a dozen
+			// vector instructions per step.
+			backward_visit(p, (p0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z), w0, g0, c0, st, k, rows, row_slots, frame,
+			               ray, a, lane);
+			backward_visit(p, (p1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z), w1, g1, c1, st, k + 1, rows, row_slots,
+			               frame, ray, a, lane);
+			backward_visit(p, (p2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z), w2, g2, c2, st, k + 2, rows, row_slots,
+			               frame, ray, a, lane);
+			backward_visit(p, (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z), w3, g3, c3, st, k + 3, rows, row_slots,
+			               frame, ray, a, lane);
 		}
 		// the rows point into this chunk's staged entries: they go before the next chunk takes their place
 		if (rows > 0) {
