@@ -45,6 +45,7 @@ class _CompositePartialImages(torch.autograd.Function):
             check(lib.rgs_composite_forward(
                 K, H, W, ptr_table(images), ptr_table(depths), ptr_table(alphas), ptr(bg), ptr(out_image),
                 ptr(out_depth), ptr(out_alpha), C.c_void_p(torch.cuda.current_stream(device).cuda_stream)))
+        ctx.set_materialize_grads(False)  # absent depth / alpha gradients come back as None and go down as null pointers
         ctx.K, ctx.hw = K, (H, W)
         ctx.has_bg = bg is not None
         ctx.save_for_backward(*(images + depths + alphas + ([bg] if bg is not None else [])))

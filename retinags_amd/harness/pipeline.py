@@ -132,8 +132,21 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
     color, radii, depth, alpha = rasterizer(
         means3D=sub.means3D, means2D=means2D, shs=sub.shs, colors_precomp=None, opacities=sub.opacity,
         scales=sub.scales, rotations=sub.rotations, cov3D_precomp=None, geometry=geometry)
-    return {"render": color, "viewspace_points": means2D, "visibility_filter": radii > 0, "radii": radii,
-            "depth": depth, "alpha": alpha, "num_rendered": -1}
+    return RenderResult({"render": color, "viewspace_points": means2D, "radii": radii,
+                         "depth": depth, "alpha": alpha, "num_rendered": -1})
+
+
+class RenderResult(dict):
+    """What the reference's render() returns for a submodel (gaussian_renderer/__init__.py: "render",
+    "viewspace_points", "visibility_filter", "radii", "depth", "alpha", "num_rendered").  The visibility filter
+    (radii > 0) is formed when somebody asks for it: a training iteration that does not densify never does."""
+
+    def __missing__(self, key):
+        if key == "visibility_filter":
+            value = self["radii"] > 0
+            self[key] = value
+            return value
+        raise KeyError(key)
 
 
 def start_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0, debug: bool = False,
@@ -234,8 +247,8 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
         partial = {}
         for k, m in enumerate(related):
             color, radii, depth, alpha = outs[k]
-            partial[m] = {"render": color, "viewspace_points": inputs[k]["means2D"], "visibility_filter": radii > 0,
-                          "radii": radii, "depth": depth, "alpha": alpha, "num_rendered": -1}
+            partial[m] = RenderResult({"render": color, "viewspace_points": inputs[k]["means2D"], "radii": radii,
+                                       "depth": depth, "alpha": alpha, "num_rendered": -1})
     elif instance_bounds is not None:
         main = torch.cuda.current_stream(device)
         lanes = streams if streams else [main]

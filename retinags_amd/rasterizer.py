@@ -373,6 +373,7 @@ class _RasterizeGaussians(torch.autograd.Function):
     def _finish_forward(ctx, outs, raster_settings, colors_precomp, means3D, scales, rotations, cov3Ds_precomp, sh):
         num_rendered, color, depth, alpha, radii, geomBuffer, binningBuffer, imgBuffer = outs
 
+        ctx.set_materialize_grads(False)  # an output that took no part in the loss comes back as None, not as a tensor of zeros
         ctx.raster_settings = raster_settings
         ctx.num_rendered = num_rendered
         # Only rendered Gaussians get non-zero gradients and the library writes just those rows;
@@ -549,6 +550,7 @@ class _RasterizeFrame(torch.autograd.Function):
                     arr[j].binning_ws, arr[j].binning_bytes = ptr(rec["binning"]), binning_bytes
                 check(lib.rgs_frame_forward_raster(len(live), arr, C.byref(view), C.c_void_p(main), debug))
         ctx.cleared, ctx.cleared_event = (cleared, cleared_event) if live else (None, None)
+        ctx.set_materialize_grads(False)  # an output that took no part in the loss comes back as None, not as a tensor of zeros
         ctx.settings = settings
         ctx.streams = streams
         ctx.meta = []
