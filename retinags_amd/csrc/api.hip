@@ -989,6 +989,7 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 	std::vector<rgs::BlendArgs> jobs;
 	std::vector<int> job_layer;
 	std::vector<rgs::PreprocessBackwardArgs> geometry((size_t)K);
+	std::vector<rgs::FillJob> sums_to_clear, blocks_to_clear;
 	for (int k = 0; k < K; k++) {
 		const rgs_frame_layer& l = layers[k];
 		if (int rc = check_backward_pointers("rgs_frame_backward", l.P, l.R, view->width, view->height, l.background, l.means3D,
@@ -999,11 +1000,8 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		                                     l.dL_dscale, l.dL_drot))
 			return rc;
 		RGS_REQUIRE(!l.grad_block || (l.grad_block_bytes & 3) == 0, "rgs_frame_backward: grad_block_bytes must be a multiple of 4");
-		if (!l.outputs_zeroed) {  // the blend adds into the rows of sums: they come first, on the frame's stream
-			rgs::stage_mark("clear_gradients", s);
-			rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(l.grad_accum), 0u, (size_t)RGS_ACC_FLOATS * (size_t)l.P, s);
-			RGS_STAGE("clear gradient sums");
-		}
+		if (!l.outputs_zeroed)  // the blend adds into the rows of sums: they come first, on the frame's stream
+			sums_to_clear.push_back(rgs::FillJob{reinterpret_cast<uint32_t*>(l.grad_accum), (size_t)RGS_ACC_FLOATS * (size_t)l.P});
 		if (l.R > 0) {
 			rgs::BlendArgs a;
 			fill_blend_args(a, l.P, l.R, view->width, view->height, view->tan_fovx, view->tan_fovy, l.background,
@@ -1018,6 +1016,11 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		                       l.scale_modifier, l.rotations, l.cov3D_precomp, view->viewmatrix, view->projmatrix, view->cam_pos,
 		                       view->tan_fovx, view->tan_fovy, l.radii, l.geom_ws, l.grad_accum, l.dL_dmean2D, l.dL_dopacity,
 		                       l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh, l.dL_dscale, l.dL_drot);
+	}
+	if (!sums_to_clear.empty()) {
+		rgs::stage_mark("clear_gradients", s);
+		rgs::launch_fill_many(sums_to_clear.data(), (int)sums_to_clear.size(), 0u, s);
+		RGS_STAGE("clear gradient sums");
 	}
 	// Gradient arrays that the caller has not cleared are cleared here, on the second stream if there is one (a caller
 	// with a second stream does better to clear them there during the forward: the backward blend fills every SIMD's
@@ -1036,14 +1039,16 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		const rgs_frame_layer& l = layers[k];
 		if (l.outputs_zeroed)
 			continue;
-		if (l.grad_block) {
-			if (beside == s)
-				rgs::stage_mark("clear_gradients", s);
-			rgs::launch_fill_u32(static_cast<uint32_t*>(l.grad_block), 0u, l.grad_block_bytes / 4, beside);
-			RGS_STAGE("clear gradients");
-		} else {
+		if (l.grad_block)
+			blocks_to_clear.push_back(rgs::FillJob{static_cast<uint32_t*>(l.grad_block), l.grad_block_bytes / 4});
+		else
 			already[(size_t)k] = 0;
-		}
+	}
+	if (!blocks_to_clear.empty()) {  // one launch for every layer's block
+		if (beside == s)
+			rgs::stage_mark("clear_gradients", s);
+		rgs::launch_fill_many(blocks_to_clear.data(), (int)blocks_to_clear.size(), 0u, beside);
+		RGS_STAGE("clear gradients");
 	}
 	// With a second stream the blend goes in two halves, so that the per-Gaussian backward of the first half's layers
 	// (memory bandwidth) runs beside the blend of the second half.  Layers without instances go with the last half.

@@ -1012,6 +1012,42 @@ __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p,
 		p[done + tid] = v;
 }
 
+// The same for several arrays in one launch (the array in blockIdx.y).
+__global__ __launch_bounds__(256) void fill_many_kernel(Batch<FillJob> batch, uint32_t v)
+{
+	uint32_t* __restrict__ p = batch.job[blockIdx.y].p;
+	const size_t n = batch.job[blockIdx.y].n;
+	const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, threads = (size_t)gridDim.x * 256;
+	const size_t head = min(n, (size_t)((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4);
+	const size_t groups = (n - head) / 4;
+	if (tid < head)
+		p[tid] = v;
+	uint4* q = reinterpret_cast<uint4*>(p + head);
+	const uint4 vv = {v, v, v, v};
+	for (size_t g = tid; g < groups; g += threads)
+		q[g] = vv;
+	const size_t done = head + 4 * groups;
+	if (tid < n - done)
+		p[done + tid] = v;
+}
+
+void launch_fill_many(const FillJob* jobs, int count, uint32_t v, hipStream_t s)
+{
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<FillJob> b = {};
+		size_t most = 0;
+		for (int k = 0; k < nj; k++) {
+			b.job[k] = jobs[at + k];
+			most = b.job[k].n > most ? b.job[k].n : most;
+		}
+		if (most == 0)
+			continue;
+		const size_t blocks = (most / 4 + 255) / 256 + 1, cap = 4096 / (size_t)nj + 1;
+		hipLaunchKernelGGL(fill_many_kernel, dim3((unsigned)(blocks < cap ? blocks : cap), (unsigned)nj), dim3(256), 0, s, b, v);
+	}
+}
+
 void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
 {
 	if (n == 0)

@@ -434,6 +434,11 @@ void launch_blend_count(const BlendArgs& a, hipStream_t s);    // the work-accou
 void launch_composite_forward(const CompositeArgs& a, hipStream_t s);
 void launch_composite_backward(const CompositeArgs& a, hipStream_t s);
 void launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s);
+struct FillJob {
+	uint32_t* p;
+	size_t n;  // words
+};
+void launch_fill_many(const FillJob* jobs, int count, uint32_t v, hipStream_t s);  // every array in one launch
 
 // sharing.hip
 uint32_t straddler_select_blocks(int n);
