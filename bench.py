@@ -308,8 +308,8 @@ def measure(args, config, forward_only, asides, cpu):
         # written once
         "clear_gradients": (4.0 * (3 + 1 + 3 + 48 + 3 + 4) + 48.0) * P_tot,
         # rows of the rendered Gaussians only: sums, mean, SH, scale, rotation in;
-        # the eight gradient rows out
-        "preprocess_backward": (285.0 + 284.0) * P_vis,
+        # the six gradient rows a frame hands out (mean2D, opacity, mean3D, SH, scale, rotation)
+        "preprocess_backward": (285.0 + 248.0) * P_vis,
         "composite_forward": (20.0 * K + 20.0) * N,
         "composite_backward": (40.0 * K + 20.0) * N,
     }

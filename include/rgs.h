@@ -199,7 +199,9 @@ enum { RGS_ACC_FLOATS = 12 };
  * zero.  With outputs_zeroed = 0 the library clears the eight arrays and grad_accum itself,
  * like the reference's shim; a caller that hands over all nine already cleared (say, while
  * the forward pass was still running) passes 1 and saves that pass over them.  dL_dsh /
- * dL_dscale / dL_drot may be NULL when shs / scales are NULL; dL_dpix_depth / dL_dalphas
+ * dL_dscale / dL_drot may be NULL when shs / scales are NULL; dL_dcolor may be NULL when shs
+ * are given and dL_dcov3D when scales are (they are intermediates then: the reference fills
+ * them, a caller that hands them to nobody saves their traffic); dL_dpix_depth / dL_dalphas
  * may be NULL when no gradient arrived for the depth / alpha image (taken as zero). */
 int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const float* background, const float* means3D, const float* shs, const float* colors_precomp,

@@ -852,8 +852,10 @@ int check_backward_pointers(const char* who, int P, int R, int width, int height
 	RGS_REQUIRE(width > 0 && height > 0, "%s: bad image size %dx%d", who, width, height);
 	RGS_REQUIRE(background && means3D && alphas && viewmatrix && projmatrix && projmatrix_inv && range_low && range_up &&
 	                cam_pos && radii && geom_ws && image_ws && dL_dpix && grad_accum &&
-	                dL_dmean2D && dL_dopacity && dL_dcolor && dL_dmean3D && dL_dcov3D,
+	                dL_dmean2D && dL_dopacity && dL_dmean3D,
 	            "%s: null pointer", who);
+	RGS_REQUIRE(!colors_precomp || dL_dcolor, "%s: dL_dcolor is required with precomputed colours", who);
+	RGS_REQUIRE(!cov3D_precomp || dL_dcov3D, "%s: dL_dcov3D is required with a precomputed covariance", who);
 	RGS_REQUIRE(R == 0 || binning_ws, "%s: null binning workspace", who);
 	RGS_REQUIRE((shs != nullptr) != (colors_precomp != nullptr), "%s: provide exactly one of SHs or colours", who);
 	RGS_REQUIRE(!shs || dL_dsh, "%s: dL_dsh is required with SHs", who);

@@ -392,9 +392,11 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 		for (int k = 0; k < 6; k++)
 			dcov[k] = 0.f;
 	}
+	if (a.dL_dcov3D) {  // null when the covariance comes from scale and rotation and nobody asks for this intermediate
 #pragma unroll
-	for (int k = 0; k < 6; k++)
-		a.dL_dcov3D[6 * i + k] = dcov[k];
+		for (int k = 0; k < 6; k++)
+			a.dL_dcov3D[6 * i + k] = dcov[k];
+	}
 
 	const float dL_dT00 = 2 * (TM(0, 0) * VM(0, 0) + TM(0, 1) * VM(0, 1) + TM(0, 2) * VM(0, 2)) * dL_da +
 	                      (TM(1, 0) * VM(0, 0) + TM(1, 1) * VM(0, 1) + TM(1, 2) * VM(0, 2)) * dL_db;
@@ -549,9 +551,11 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	a.dL_dmean2D[3 * i + 0] = mean2d_x;
 	a.dL_dmean2D[3 * i + 1] = mean2d_y;
 	a.dL_dopacity[i] = opacity_sum;
-	a.dL_dcolor[3 * i + 0] = color_sum[0];
-	a.dL_dcolor[3 * i + 1] = color_sum[1];
-	a.dL_dcolor[3 * i + 2] = color_sum[2];
+	if (a.dL_dcolor) {  // null when the colours come from SH and nobody asks for this intermediate
+		a.dL_dcolor[3 * i + 0] = color_sum[0];
+		a.dL_dcolor[3 * i + 1] = color_sum[1];
+		a.dL_dcolor[3 * i + 2] = color_sum[2];
+	}
 }
 
 // ---- launchers -----------------------------------------------------------------------------
@@ -605,9 +609,11 @@ void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, const int* o
 			const size_t n = (size_t)a.P;
 			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmean2D), 0u, 3 * n, s);
 			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dopacity), 0u, n, s);
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcolor), 0u, 3 * n, s);
+			if (a.dL_dcolor)
+				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcolor), 0u, 3 * n, s);
 			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmeans), 0u, 3 * n, s);
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcov3D), 0u, 6 * n, s);
+			if (a.dL_dcov3D)
+				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcov3D), 0u, 6 * n, s);
 			if (a.shs)
 				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dsh), 0u, (size_t)a.M * 3 * n, s);
 			if (a.scales) {

@@ -238,18 +238,17 @@ def _gradient_outputs(P, M, has_scales, device, make, scratch=()):
     per Gaussian with SH degree 3).  Without scales the scale / rotation gradients are zeros in
     either case.  `scratch` names those of the eight that the caller hands to nobody (the colour
     gradient when the colours come from SH, the covariance gradient when it comes from scale and
-    rotation): they lie behind the others, and out["block"], the part that has to be zero where
-    no Gaussian was rendered, ends before them."""
+    rotation): they are not made at all (None), and the library does not write them."""
     shapes = {"means2D": (P, 3), "opacity": (P, 1), "colors": (P, 3), "means3D": (P, 3), "cov3D": (P, 6),
               "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4)}
-    order = [k for k in shapes if k not in scratch] + [k for k in shapes if k in scratch]
+    order = [k for k in shapes if k not in scratch]
     sizes = {k: (math.prod(v) + 63) // 64 * 64 for k, v in shapes.items()}  # 256-byte aligned parts
-    flat = make((sum(sizes.values()),), dtype=torch.float32, device=device)
-    out, at = {}, 0
+    flat = make((sum(sizes[k] for k in order),), dtype=torch.float32, device=device)
+    out, at = {k: None for k in scratch}, 0
     for k in order:
         out[k] = flat[at:at + math.prod(shapes[k])].view(shapes[k])
         at += sizes[k]
-    out["block"] = flat[:sum(sizes[k] for k in order if k not in scratch)]  # what has to be cleared, as one tensor
+    out["block"] = flat  # what has to be cleared, as one tensor
     out["sums"] = make((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
     if not has_scales and make is not torch.zeros:
         out["scales"].zero_()
