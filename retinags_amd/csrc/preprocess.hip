@@ -139,9 +139,27 @@ __device__ __forceinline__ void load_sh_row(const float* __restrict__ row, int d
 
 // ---- forward preprocess (K/cuda_rasterizer_hgs/forward.cu:155-258) -------------------------
 
+// SH rows through LDS: a wavefront reads the rows of its rendered Gaussians together, 16 lanes
+// per row and 16 bytes per lane (a load instruction then covers four rows instead of one piece of
+// 64), parks them in LDS and every lane picks up its own row.  32 rows at a time.
+constexpr int kRecordStride = 5;  // float4 per parked record: 20 words, so 8 lanes' 16-byte writes meet no bank twice
+static_assert(64 * kRecordStride <= 32 * 13, "the parked records share the rows' space");
+
+__device__ __forceinline__ void wave_lds_fence()
+{
+	// orders the LDS traffic of one wavefront around a hand-over between its lanes
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+	__builtin_amdgcn_wave_barrier();
+	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+constexpr int kShRowStride = 13;  // float4 per parked row: 52 words, so 8 lanes' 16-byte reads meet no bank twice
+
 __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<PreprocessArgs> batch)
 {
 	__shared__ uint32_t s_scan[8];
+	__shared__ float4 s_rows[4][32 * kShRowStride];
+	__shared__ uint8_t s_listed[4][64];
 	const PreprocessArgs& a = batch.job[blockIdx.y];  // one job per submodel of the frame
 	const int idx = blockIdx.x * 256 + threadIdx.x;
 	// the scratch of the depth sort that follows is cleared here, which saves a launch
@@ -150,11 +168,15 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<Preproces
 	if ((int)blockIdx.x * 256 >= a.P)
 		return;  // the launch is sized for the job with the most Gaussians
 	uint32_t touched = 0;
+	bool rendered = false;
+	float2 pix = {0.f, 0.f};
+	float4 conic_o = {0.f, 0.f, 0.f, 0.f};
+	float hom_w = 0.f, view_z = 0.f, my_radius = 0.f;
+	float3 p = {0.f, 0.f, 0.f};
 
 	if (idx < a.P) {
-		int radius_out = 0;
 		do {
-			const float3 p = {a.means[3 * (size_t)idx], a.means[3 * (size_t)idx + 1], a.means[3 * (size_t)idx + 2]};
+			p = float3{a.means[3 * (size_t)idx], a.means[3 * (size_t)idx + 1], a.means[3 * (size_t)idx + 2]};
 			const float3 p_view = xform_point_4x3(p, a.view);
 			if (p_view.z <= 0.2f)
 				break;
@@ -179,70 +201,138 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<Preproces
 			if (det == 0.0f)
 				break;
 			const float det_inv = 1.f / det;
-			const float4 conic_o = {cz * det_inv, -cy * det_inv, cx * det_inv, a.opacities[idx]};
 
 			const float mid = 0.5f * (cx + cz);
 			const float lambda1 = mid + sqrtf(fmaxf(0.1f, mid * mid - det));
 			const float lambda2 = mid - sqrtf(fmaxf(0.1f, mid * mid - det));
-			const float my_radius = ceilf(3.f * sqrtf(fmaxf(lambda1, lambda2)));
-			const float2 pix = {ndc_to_pix(p_proj.x, a.W), ndc_to_pix(p_proj.y, a.H)};
-			const TileRect rc = tile_rect(pix.x, pix.y, (int)my_radius, a.grid_x, a.grid_y);
+			const float radius = ceilf(3.f * sqrtf(fmaxf(lambda1, lambda2)));
+			const float2 at = {ndc_to_pix(p_proj.x, a.W), ndc_to_pix(p_proj.y, a.H)};
+			const TileRect rc = tile_rect(at.x, at.y, (int)radius, a.grid_x, a.grid_y);
 			const uint32_t ntiles = (rc.x1 - rc.x0) * (rc.y1 - rc.y0);
 			if (ntiles == 0)
 				break;
+			conic_o = float4{cz * det_inv, -cy * det_inv, cx * det_inv, a.opacities[idx]};
+			pix = at;
+			hom_w = p_hom.w;
+			view_z = p_view.z;
+			my_radius = radius;
+			touched = ntiles;
+			rendered = true;
+		} while (false);
+	}
 
-			float3 col;
-			if (a.colors_precomp) {
-				col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
-				             a.colors_precomp[3 * (size_t)idx + 2]};
-			} else {
-				const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
-				const float3 dir = {p.x - cam.x, p.y - cam.y, p.z - cam.z};
-				const float len = sqrtf(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
-				const float dx = dir.x / len, dy = dir.y / len, dz = dir.z / len;
-				const float* sh = a.shs + (size_t)idx * a.M * 3;
-				uint32_t clamp_bits = 0;
-				float rgb[3], raw[3];
-				if (a.sh_rows_by_16_bytes) {
+	// the rendered Gaussians of the wavefront, listed in lane order
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const uint64_t seen = __ballot(rendered);
+	const int n_seen = __popcll(seen);
+	const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(seen >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)seen, 0u));
+	float4* parked = s_rows[wave];
+	uint8_t* listed = s_listed[wave];
+	if (rendered)
+		listed[rank] = (uint8_t)lane;
+	wave_lds_fence();
+
+	float3 col = {0.f, 0.f, 0.f};
+	uint32_t clamp_bits = 0;
+	if (a.colors_precomp) {
+		if (rendered)
+			col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
+			             a.colors_precomp[3 * (size_t)idx + 2]};
+	} else {
+		const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
+		const float3 dir = {p.x - cam.x, p.y - cam.y, p.z - cam.z};
+		const float len = sqrtf(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
+		const float dx = dir.x / len, dy = dir.y / len, dz = dir.z / len;
+		float raw[3] = {0.f, 0.f, 0.f};
+		if (a.sh_rows_by_16_bytes) {
+			const int piece = lane & 15, sub = lane >> 4;
+			const int row_pieces = a.M * 3 / 4;
+			const int needed = 3 * (a.D + 1) * (a.D + 1);
+			const float4* __restrict__ rows =
+			    reinterpret_cast<const float4*>(a.shs) + (size_t)(idx - lane) * row_pieces;
+			for (int base = 0; base < n_seen; base += 32) {
+				float4 v[8];
+#pragma unroll
+				for (int r = 0; r < 8; r++) {
+					const int slot = base + 4 * r + sub;
+					v[r] = float4{0.f, 0.f, 0.f, 0.f};
+					if (4 * piece < needed && slot < n_seen)
+						v[r] = rows[(size_t)listed[slot] * row_pieces + piece];
+				}
+#pragma unroll
+				for (int r = 0; r < 8; r++)
+					if (piece < 12)
+						parked[(4 * r + sub) * kShRowStride + piece] = v[r];
+				wave_lds_fence();
+				if (rendered && rank >= base && rank < base + 32) {
 					float row[kShRegs];
-					load_sh_row(sh, a.D, row);
+					const float4* mine = parked + (rank - base) * kShRowStride;
+#pragma unroll
+					for (int k = 0; k < kShRegs; k += 4) {
+						float4 q = {0.f, 0.f, 0.f, 0.f};
+						if (k < needed)
+							q = mine[k / 4];
+						row[k] = q.x;
+						row[k + 1] = q.y;
+						row[k + 2] = q.z;
+						row[k + 3] = q.w;
+					}
 #pragma unroll
 					for (int ch = 0; ch < 3; ch++)
 						raw[ch] = sh_channel(a.D, dx, dy, dz, row + ch);
-				} else {
-#pragma unroll
-					for (int ch = 0; ch < 3; ch++)
-						raw[ch] = sh_channel(a.D, dx, dy, dz, sh + ch);
 				}
+				wave_lds_fence();
+			}
+		} else if (rendered) {
+			const float* sh = a.shs + (size_t)idx * a.M * 3;
 #pragma unroll
-				for (int ch = 0; ch < 3; ch++) {
-					const float v = raw[ch];
-					clamp_bits |= (v < 0) ? (1u << ch) : 0u;
-					rgb[ch] = fmaxf(v, 0.0f);
-				}
-				col = float3{rgb[0], rgb[1], rgb[2]};
+			for (int ch = 0; ch < 3; ch++)
+				raw[ch] = sh_channel(a.D, dx, dy, dz, sh + ch);
+		}
+		float rgb[3];
+#pragma unroll
+		for (int ch = 0; ch < 3; ch++) {
+			const float v = raw[ch];
+			clamp_bits |= (v < 0) ? (1u << ch) : 0u;
+			rgb[ch] = fmaxf(v, 0.0f);
+		}
+		col = float3{rgb[0], rgb[1], rgb[2]};
+	}
+
+	if (idx < a.P) {
+		if (rendered) {
+			if (!a.colors_precomp)
 				a.clamped[idx] = (uint8_t)clamp_bits;
-			}
-			a.depths[idx] = p_view.z;
-			{
-				// Everything later stages read of a rendered Gaussian goes into one 64-byte record: a
-				// gather by index then costs one cache line, and nothing is written a second time into
-				// arrays of their own, where a rendered Gaussian among unrendered ones dirties a whole
-				// line for a few bytes.  The 3D covariance is not kept: the backward computes it again.
-				const float floor = exponent_floor(conic_o.w);
-				const float2 half = alpha_ellipse_half_extent(conic_o, floor);
-				float4* rec = a.blend_record + 4 * (size_t)idx;
-				rec[0] = float4{pix.x, pix.y, floor, p_hom.w};
-				rec[1] = conic_o;
-				rec[2] = float4{col.x, col.y, col.z, p_view.z};
-				// the third word is the integer radius (as bits): the key duplication reads the tile rectangle's inputs from here
-				rec[3] = float4{half.x, half.y, __int_as_float((int)my_radius), 0.f};
-			}
-			radius_out = (int)my_radius;
-			touched = ntiles;
-		} while (false);
-		a.radii[idx] = radius_out;
+			a.depths[idx] = view_z;
+		}
+		a.radii[idx] = (int)my_radius;
 		a.tiles_touched[idx] = touched;
+	}
+	{
+		// Everything later stages read of a rendered Gaussian goes into one 64-byte record: a
+		// gather by index then costs one cache line, and nothing is written a second time into
+		// arrays of their own, where a rendered Gaussian among unrendered ones dirties a whole
+		// line for a few bytes.  The 3D covariance is not kept: the backward computes it again.
+		// The records leave through LDS, four lanes to a record, so that a store instruction
+		// writes 16 whole records and not a quarter of 64.
+		wave_lds_fence();
+		if (rendered) {
+			const float floor = exponent_floor(conic_o.w);
+			const float2 half = alpha_ellipse_half_extent(conic_o, floor);
+			float4* rec = parked + rank * kRecordStride;
+			rec[0] = float4{pix.x, pix.y, floor, hom_w};
+			rec[1] = conic_o;
+			rec[2] = float4{col.x, col.y, col.z, view_z};
+			// the third word is the integer radius (as bits): the key duplication reads the tile rectangle's inputs from here
+			rec[3] = float4{half.x, half.y, __int_as_float((int)my_radius), 0.f};
+		}
+		wave_lds_fence();
+		float4* records = a.blend_record + 4 * (size_t)(idx - lane);
+		for (int base = 0; base < n_seen; base += 16) {
+			const int slot = base + (lane >> 2);
+			if (slot < n_seen)
+				records[4 * (size_t)listed[slot] + (lane & 3)] = parked[slot * kRecordStride + (lane & 3)];
+		}
 	}
 
 	// Per-block total of tiles_touched: the first level of the offset scan.
