@@ -411,21 +411,25 @@ __device__ __forceinline__ void sh_backward_channel(int deg, float x, float y, f
 	ddz += dRGBdz * g;
 }
 
-constexpr int kBwdShMax = 48;  // SH gradient floats kept in registers until they are stored
-
+#ifndef RGS_PB_WAVES
+#define RGS_PB_WAVES 4
+#endif
+__attribute__((amdgpu_waves_per_eu(RGS_PB_WAVES, RGS_PB_WAVES)))
 __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<PreprocessBackwardArgs> batch)
 {
+	__shared__ float4 s_rows[2][32 * kShRowStride];
+	__shared__ uint32_t s_index[2][64];
 	const PreprocessBackwardArgs& a = batch.job[blockIdx.y];
-	const uint32_t k_vis = blockIdx.x * 128 + threadIdx.x;
-	if (k_vis >= *a.visible_count)
-		return;
+	const uint32_t listed = *a.visible_count;
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const uint32_t k_first = blockIdx.x * 128 + wave * 64;
+	if (k_first >= listed)
+		return;  // the whole wavefront
+	// Spare lanes of the list's last wavefront repeat its last Gaussian (the same values go to the
+	// same places), so that the whole wavefront takes part where its lanes share the work.
+	const uint32_t k_vis = min(k_first + (uint32_t)lane, listed - 1u);
 	const size_t i = (size_t)a.visible_list[k_vis];
 	const int n_sh = a.shs ? a.M * 3 : 0;
-	const bool sh_in_regs = n_sh <= kBwdShMax;
-	float shg[kBwdShMax];
-#pragma unroll
-	for (int k = 0; k < kBwdShMax; k++)
-		shg[k] = 0.f;
 	float mean2d_x = 0.f, mean2d_y = 0.f, opacity_sum = 0.f, color_sum[3] = {0.f, 0.f, 0.f};
 
 	{
@@ -442,6 +446,116 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	color_sum[0] = sum_color[0];
 	color_sum[1] = sum_color[1];
 	color_sum[2] = sum_color[2];
+
+	// (ahead of the rest, while few other values are held)
+	float3 sh_dmean = {0.f, 0.f, 0.f};
+	// -- SH colour and the view direction's dependence on the mean (backward.cu:20-139)
+	if (a.shs) {
+		const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
+		const float3 d0 = {mean.x - cam.x, mean.y - cam.y, mean.z - cam.z};
+		const float len = sqrtf(d0.x * d0.x + d0.y * d0.y + d0.z * d0.z);
+		const float x = d0.x / len, y = d0.y / len, z = d0.z / len;
+		const uint32_t cl = a.clamped[i];
+		const float* sh = a.shs + i * n_sh;
+		float ddx = 0.f, ddy = 0.f, ddz = 0.f;
+		if (a.sh_rows_by_16_bytes) {
+			// The usual case.  The wavefront reads the SH rows of its Gaussians together, 16 lanes
+			// to a row and 16 bytes a lane, parks them in LDS (32 rows at a time) where each lane
+			// picks up its own; the rows of dL_dsh leave the same way.
+			const int piece = lane & 15, sub = lane >> 4;
+			const int row_pieces = n_sh / 4;
+			const int needed = 3 * (a.D + 1) * (a.D + 1);
+			const int needed_pieces = (needed + 3) / 4;
+			float4* parked = s_rows[wave];
+			uint32_t* index = s_index[wave];
+			index[lane] = (uint32_t)i;
+			wave_lds_fence();
+			const float4* __restrict__ rows = reinterpret_cast<const float4*>(a.shs);
+			float4* __restrict__ grads = reinterpret_cast<float4*>(a.dL_dsh);
+			float g[3];
+#pragma unroll
+			for (int ch = 0; ch < 3; ch++)
+				g[ch] = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
+			for (int h = 0; h < 2; h++) {
+				float4* mine = parked + (lane & 31) * kShRowStride;
+				// (what a lane computes here does not depend on the turn; made opaque so that it is
+				// computed in its turn and not kept in registers across both)
+				float xo = x, yo = y, zo = z, go[3] = {g[0], g[1], g[2]};
+				asm volatile("" : "+v"(xo), "+v"(yo), "+v"(zo), "+v"(go[0]), "+v"(go[1]), "+v"(go[2]));
+				if ((lane >> 5) == h) {
+					// the rows of dL_dsh, which do not depend on the coefficients
+					float none[kShRegs], out[kShRegs];
+#pragma unroll
+					for (int k = 0; k < kShRegs; k++) {
+						none[k] = 0.f;
+						out[k] = 0.f;
+					}
+					float t0 = 0.f, t1 = 0.f, t2 = 0.f;
+#pragma unroll
+					for (int ch = 0; ch < 3; ch++)
+						sh_backward_channel(a.D, xo, yo, zo, none + ch, go[ch], out + ch, t0, t1, t2);
+#pragma unroll
+					for (int k = 0; k < kShRegs; k += 4)
+						if (k < needed)
+							mine[k / 4] = float4{out[k], out[k + 1], out[k + 2], out[k + 3]};
+				}
+				wave_lds_fence();
+				__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+				for (int r = 0; r < 8; r++)
+					if (piece < needed_pieces)
+						grads[(size_t)index[32 * h + 4 * r + sub] * row_pieces + piece] =
+						    parked[(4 * r + sub) * kShRowStride + piece];
+				wave_lds_fence();
+				{
+					float4 v[8];
+#pragma unroll
+					for (int r = 0; r < 8; r++) {
+						v[r] = float4{0.f, 0.f, 0.f, 0.f};
+						if (piece < needed_pieces)
+							v[r] = rows[(size_t)index[32 * h + 4 * r + sub] * row_pieces + piece];
+					}
+#pragma unroll
+					for (int r = 0; r < 8; r++)
+						if (piece < 12)
+							parked[(4 * r + sub) * kShRowStride + piece] = v[r];
+				}
+				wave_lds_fence();
+				__builtin_amdgcn_sched_barrier(0);
+				if ((lane >> 5) == h) {
+					// the coefficients' part in the gradient of the view direction
+					float row[kShRegs], unused[kShRegs];
+#pragma unroll
+					for (int k = 0; k < kShRegs; k += 4) {
+						float4 q = {0.f, 0.f, 0.f, 0.f};
+						if (k < needed)
+							q = mine[k / 4];
+						row[k] = q.x;
+						row[k + 1] = q.y;
+						row[k + 2] = q.z;
+						row[k + 3] = q.w;
+					}
+#pragma unroll
+					for (int ch = 0; ch < 3; ch++)
+						sh_backward_channel(a.D, xo, yo, zo, row + ch, go[ch], unused + ch, ddx, ddy, ddz);
+				}
+				wave_lds_fence();
+				__builtin_amdgcn_sched_barrier(0);
+			}
+		} else {
+#pragma unroll
+			for (int ch = 0; ch < 3; ch++) {
+				const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
+				sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
+			}
+		}
+		// normalisation Jacobian (auxiliary.h:123-133)
+		const float sum2 = d0.x * d0.x + d0.y * d0.y + d0.z * d0.z;
+		const float invsum32 = 1.0f / sqrtf(sum2 * sum2 * sum2);
+		sh_dmean.x = ((+sum2 - d0.x * d0.x) * ddx - d0.y * d0.x * ddy - d0.z * d0.x * ddz) * invsum32;
+		sh_dmean.y = (-d0.x * d0.y * ddx + (sum2 - d0.y * d0.y) * ddy - d0.z * d0.y * ddz) * invsum32;
+		sh_dmean.z = (-d0.x * d0.z * ddx - d0.y * d0.z * ddy + (sum2 - d0.z * d0.z) * ddz) * invsum32;
+	}
 
 	// -- conic -> cov2D -> cov3D and mean (backward.cu:144-274)
 	float cov6r[6];
@@ -536,40 +650,9 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	dmean.y += (view[6] - view[7] * mul3) * gd;
 	dmean.z += (view[10] - view[11] * mul3) * gd;
 
-	// -- SH colour and the view direction's dependence on the mean (backward.cu:20-139)
-	if (a.shs) {
-		const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
-		const float3 d0 = {mean.x - cam.x, mean.y - cam.y, mean.z - cam.z};
-		const float len = sqrtf(d0.x * d0.x + d0.y * d0.y + d0.z * d0.z);
-		const float x = d0.x / len, y = d0.y / len, z = d0.z / len;
-		const uint32_t cl = a.clamped[i];
-		const float* sh = a.shs + i * n_sh;
-		float ddx = 0.f, ddy = 0.f, ddz = 0.f;
-		if (a.sh_rows_by_16_bytes) {  // the usual case: rows are read and written 16 bytes at a time
-			float row[kShRegs];
-			load_sh_row(sh, a.D, row);
-#pragma unroll
-			for (int ch = 0; ch < 3; ch++) {
-				const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-				sh_backward_channel(a.D, x, y, z, row + ch, g, shg + ch, ddx, ddy, ddz);
-			}
-		} else {
-#pragma unroll
-			for (int ch = 0; ch < 3; ch++) {
-				const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-				if (sh_in_regs)
-					sh_backward_channel(a.D, x, y, z, sh + ch, g, shg + ch, ddx, ddy, ddz);
-				else
-					sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
-			}
-		}
-		// normalisation Jacobian (auxiliary.h:123-133)
-		const float sum2 = d0.x * d0.x + d0.y * d0.y + d0.z * d0.z;
-		const float invsum32 = 1.0f / sqrtf(sum2 * sum2 * sum2);
-		dmean.x += ((+sum2 - d0.x * d0.x) * ddx - d0.y * d0.x * ddy - d0.z * d0.x * ddz) * invsum32;
-		dmean.y += (-d0.x * d0.y * ddx + (sum2 - d0.y * d0.y) * ddy - d0.z * d0.y * ddz) * invsum32;
-		dmean.z += (-d0.x * d0.z * ddx - d0.y * d0.z * ddy + (sum2 - d0.z * d0.z) * ddz) * invsum32;
-	}
+	dmean.x += sh_dmean.x;
+	dmean.y += sh_dmean.y;
+	dmean.z += sh_dmean.z;
 	a.dL_dmeans[3 * i + 0] = dmean.x;
 	a.dL_dmeans[3 * i + 1] = dmean.y;
 	a.dL_dmeans[3 * i + 2] = dmean.z;
@@ -623,20 +706,6 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	}
 	}
 
-	if (n_sh > 0 && sh_in_regs) {
-		float* dst = a.dL_dsh + i * n_sh;
-		if ((n_sh & 3) == 0) {
-#pragma unroll
-			for (int k = 0; k < kBwdShMax; k += 4)
-				if (k < n_sh)
-					*reinterpret_cast<float4*>(dst + k) = float4{shg[k], shg[k + 1], shg[k + 2], shg[k + 3]};
-		} else {
-#pragma unroll
-			for (int k = 0; k < kBwdShMax; k++)
-				if (k < n_sh)
-					dst[k] = shg[k];
-		}
-	}
 	// the sums that are gradients as they stand
 	a.dL_dmean2D[3 * i + 0] = mean2d_x;
 	a.dL_dmean2D[3 * i + 1] = mean2d_y;
