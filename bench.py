@@ -296,7 +296,7 @@ def measure(args, config, forward_only, asides, cpu):
         "preprocess_forward": 20.0 * P_tot + (224.0 + 69.0) * P_vis,
         # tile counts and depths of all, then 4 passes over the (depth, index) pairs of the visible
         # ones, the gathered tile counts and their scan
-        "depth_order": 8.0 * P_tot + (12.0 + 4 * 16.0 + 16.0) * P_vis,
+        "depth_order": 8.0 * P_tot + (8.0 + 4 * 16.0 + 16.0) * P_vis,
         # per rendered Gaussian its place in the depth order, its offset and its 64-byte record in; key and index out per instance
         "duplicate_with_keys": 72.0 * P_vis + 8.0 * R_tot,
         "sort_setup": 4.0 * R_tot,
@@ -304,12 +304,12 @@ def measure(args, config, forward_only, asides, cpu):
         "tile_ranges": 4.0 * R_tot + 16.0 * T * K,
         # the sorted keys in, the filed positions out (at most four per instance; counted as one)
         "strip_filing": 8.0 * R_tot + 16.0 * T * K,
-        # the six gradient tensors a frame hands out (mean2D, opacity, mean3D, SH, scale, rotation) and the rows of sums,
-        # written once
-        "clear_gradients": (4.0 * (3 + 1 + 3 + 48 + 3 + 4) + 48.0) * P_tot,
-        # rows of the rendered Gaussians only: sums, mean, SH, scale, rotation in;
-        # the six gradient rows a frame hands out (mean2D, opacity, mean3D, SH, scale, rotation)
-        "preprocess_backward": (285.0 + 248.0) * P_vis,
+        # the rows of sums the backward blend adds into (the gradient tensors themselves need no clearing)
+        "clear_gradients": 48.0 * P_tot,
+        # the radius of every Gaussian in; sums, mean, SH, scale, rotation, clamp flags of the rendered ones in; for every
+        # Gaussian the six gradient rows a frame hands out (mean2D, opacity, mean3D, SH, scale, rotation: zeros for the
+        # ones that were not rendered)
+        "preprocess_backward": 285.0 * P_vis + (4.0 + 248.0) * P_tot,
         "composite_forward": (20.0 * K + 20.0) * N,
         "composite_backward": (40.0 * K + 20.0) * N,
     }

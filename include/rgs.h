@@ -77,7 +77,6 @@ enum {
 	                               entries from RGS_GEOM_VISIBLE_COUNT on are unused */
 	RGS_GEOM_BLOCK_VISIBLE,     /* uint32[ceil(P/256)+1] */
 	RGS_GEOM_VISIBLE_COUNT,     /* uint32     number of Gaussians that touch a tile */
-	RGS_GEOM_VISIBLE_LIST,      /* uint32[P]  their indices in increasing order (as many entries as the count) */
 	RGS_GEOM_ORDER_SCRATCH,     /* scratch of the depth sort */
 	RGS_GEOM_FIELDS
 };
@@ -195,14 +194,16 @@ enum { RGS_ACC_FLOATS = 12 };
  * together with the zero-initialisation done by its torch shim
  * (K/rasterize_points.cu:165-174).  grad_accum is RGS_ACC_FLOATS*P floats.  dL_dmean2D (P,3; third column 0), dL_dopacity (P), dL_dcolor (P,3),
  * dL_dmean3D (P,3), dL_dcov3D (P,6), dL_dsh (P,M,3), dL_dscale (P,3), dL_drot (P,4) are
- * complete when the call has run: rows of rendered Gaussians are computed, all others are
- * zero.  With outputs_zeroed = 0 the library clears the eight arrays and grad_accum itself,
- * like the reference's shim; a caller that hands over all nine already cleared (say, while
- * the forward pass was still running) passes 1 and saves that pass over them.  dL_dsh /
- * dL_dscale / dL_drot may be NULL when shs / scales are NULL; dL_dcolor may be NULL when shs
- * are given and dL_dcov3D when scales are (they are intermediates then: the reference fills
- * them, a caller that hands them to nobody saves their traffic); dL_dpix_depth / dL_dalphas
- * may be NULL when no gradient arrived for the depth / alpha image (taken as zero). */
+ * complete when the call has run: every row is written, those of Gaussians that were not
+ * rendered as zeros, so the arrays may arrive uninitialised (the reference's shim clears them
+ * first and writes the rendered rows).  Only grad_accum has to be zero when the blend starts:
+ * with accum_zeroed = 0 the library clears it, a caller that hands it over cleared (say, while
+ * the forward pass was still running) passes 1.  dL_dsh / dL_dscale / dL_drot may be NULL when
+ * shs / scales are NULL (given without scales, dL_dscale and dL_drot are filled with zeros);
+ * dL_dcolor may be NULL when shs are given and dL_dcov3D when scales are (they are
+ * intermediates then: the reference fills them, a caller that hands them to nobody saves their
+ * traffic); dL_dpix_depth / dL_dalphas may be NULL when no gradient arrived for the depth /
+ * alpha image (taken as zero). */
 int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const float* background, const float* means3D, const float* shs, const float* colors_precomp,
                  const float* alphas, const float* scales, float scale_modifier, const float* rotations,
@@ -212,7 +213,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const void* geom_ws, const void* binning_ws, const void* image_ws,
                  const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
                  float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
-                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int outputs_zeroed, void* stream,
+                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int accum_zeroed, void* stream,
                  int debug);
 
 /* ---- the submodels of a frame in one go ----------------------------------------------------------
@@ -266,12 +267,10 @@ typedef struct rgs_frame_layer {
 	float* dL_dsh;
 	float* dL_dscale;
 	float* dL_drot;
-	int outputs_zeroed;
-	void* grad_block;          /* with outputs_zeroed = 0: NULL, or one block of grad_block_bytes (a multiple of 4) that holds the */
-	size_t grad_block_bytes;   /* eight gradient arrays and nothing that must survive: cleared in one go instead of array by array */
-	void* stream;              /* NULL, or a second HIP stream for the backward: work that is bound by memory bandwidth (clearing
-	                              the gradient arrays, the per-Gaussian backward of the layers whose blend is done) then runs on it
-	                              beside the blend, which is bound by instruction issue; the frame's stream waits for it */
+	int accum_zeroed;          /* as in rgs_backward: grad_accum arrives cleared */
+	void* stream;              /* NULL, or a second HIP stream for the backward: work that is bound by memory bandwidth (the
+	                              per-Gaussian backward of the layers whose blend is done) then runs on it beside the blend,
+	                              which is bound by instruction issue; the frame's stream waits for it */
 } rgs_frame_layer;
 /* rgs_forward_geom for every layer (P > 0 each): every geometry stage is queued (on the layer's stream) before
  * the host waits for the first instance count; returns when all counts have arrived in counts_pinned[0..K)

@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("RGS_LIBRARY") or os.path.join(_HERE, "librgs_gfx950.s
 
 GEOM_FIELDS = ("depths", "tiles_touched", "point_offsets",
                "clamped", "block_sums", "total", "blend_record", "depth_order", "block_visible", "visible_count",
-               "visible_list", "order_scratch")
+               "order_scratch")
 BIN_FIELDS = ("keys_unsorted", "keys_sorted", "values_unsorted", "values_sorted", "sort_temp", "strip_lists")
 IMG_FIELDS = ("ranges", "n_contrib", "strip_filed", "strip_order", "strip_total", "strip_order_forward")
 ACC_FLOATS = 12
@@ -60,8 +60,8 @@ class FrameLayer(C.Structure):
                 ("dL_dpix", C.c_void_p), ("dL_dpix_depth", C.c_void_p), ("dL_dalphas", C.c_void_p),
                 ("grad_accum", C.c_void_p), ("dL_dmean2D", C.c_void_p), ("dL_dopacity", C.c_void_p),
                 ("dL_dcolor", C.c_void_p), ("dL_dmean3D", C.c_void_p), ("dL_dcov3D", C.c_void_p), ("dL_dsh", C.c_void_p),
-                ("dL_dscale", C.c_void_p), ("dL_drot", C.c_void_p), ("outputs_zeroed", C.c_int),
-                ("grad_block", C.c_void_p), ("grad_block_bytes", C.c_size_t), ("stream", C.c_void_p)]
+                ("dL_dscale", C.c_void_p), ("dL_drot", C.c_void_p), ("accum_zeroed", C.c_int),
+                ("stream", C.c_void_p)]
 
 
 class RgsError(RuntimeError):

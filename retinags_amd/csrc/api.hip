@@ -214,7 +214,6 @@ size_t geom_layout(size_t P, size_t* off)
 	off[RGS_GEOM_DEPTH_ORDER] = c.take(4 * P);
 	off[RGS_GEOM_BLOCK_VISIBLE] = c.take(4 * ((P + 255) / 256 + 1));
 	off[RGS_GEOM_VISIBLE_COUNT] = c.take(4);
-	off[RGS_GEOM_VISIBLE_LIST] = c.take(4 * P);
 	off[RGS_GEOM_ORDER_SCRATCH] = c.take(order_scratch(P).total);
 	return c.cursor;
 }
@@ -523,7 +522,6 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 		d.P = c.P;
 		d.depths = a.depths; d.tiles_touched = a.tiles_touched; d.block_visible = a.block_visible;
 		d.visible_count = at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_COUNT]);
-		d.visible_list = at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_LIST]);
 		d.keys_a = at<uint32_t>(scratch, o.keys_a); d.keys_b = at<uint32_t>(scratch, o.keys_b);
 		d.order = at<uint32_t>(ws, off[RGS_GEOM_DEPTH_ORDER]); d.vals_b = at<uint32_t>(scratch, o.vals_b);
 		d.tiles_in_order = at<uint32_t>(scratch, o.tiles_in_order);
@@ -800,9 +798,7 @@ void fill_backward_geometry(rgs::PreprocessBackwardArgs& p, int P, int D, int M,
 	p.sums = grad_accum;
 	p.dL_dmean2D = dL_dmean2D; p.dL_dopacity = dL_dopacity; p.dL_dcolor = dL_dcolor;
 	p.dL_dmeans = dL_dmean3D; p.dL_dcov3D = dL_dcov3D; p.dL_dsh = dL_dsh; p.dL_dscale = dL_dscale; p.dL_drot = dL_drot;
-	p.visible_list = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_LIST]);
 	p.sh_rows_by_16_bytes = sh_rows_by_16_bytes(shs, M, D) && (reinterpret_cast<uintptr_t>(dL_dsh) & 15) == 0;
-	p.visible_count = at<uint32_t>(geom_ws, goff[RGS_GEOM_VISIBLE_COUNT]);
 }
 
 // Events for ordering a frame's stream against its layers' own streams: a few per host thread and device, reused.
@@ -903,7 +899,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
                  const void* geom_ws, const void* binning_ws, const void* image_ws,
                  const float* dL_dpix, const float* dL_dpix_depth, const float* dL_dalphas,
                  float* grad_accum, float* dL_dmean2D, float* dL_dopacity, float* dL_dcolor, float* dL_dmean3D,
-                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int outputs_zeroed, void* stream,
+                 float* dL_dcov3D, float* dL_dsh, float* dL_dscale, float* dL_drot, int accum_zeroed, void* stream,
                  int debug)
 {
 	hipStream_t s = static_cast<hipStream_t>(stream);
@@ -914,7 +910,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	                                     range_up, cam_pos, radii, geom_ws, binning_ws, image_ws, dL_dpix, grad_accum, dL_dmean2D,
 	                                     dL_dopacity, dL_dcolor, dL_dmean3D, dL_dcov3D, dL_dsh, dL_dscale, dL_drot))
 		return rc;
-	if (!outputs_zeroed) {
+	if (!accum_zeroed) {
 		rgs::launch_fill_u32(reinterpret_cast<uint32_t*>(grad_accum), 0u, (size_t)RGS_ACC_FLOATS * (size_t)P, s);
 		RGS_STAGE("clear gradient sums");
 	}
@@ -932,7 +928,7 @@ int rgs_backward(int P, int D, int M, int R, int width, int height,
 	fill_backward_geometry(p, P, D, M, width, height, means3D, shs, scales, scale_modifier, rotations, cov3D_precomp, viewmatrix,
 	                       projmatrix, cam_pos, tan_fovx, tan_fovy, radii, geom_ws, grad_accum, dL_dmean2D, dL_dopacity,
 	                       dL_dcolor, dL_dmean3D, dL_dcov3D, dL_dsh, dL_dscale, dL_drot);
-	rgs::launch_preprocess_backward(&p, &outputs_zeroed, 1, s);
+	rgs::launch_preprocess_backward(&p, 1, s);
 	RGS_STAGE("preprocess_backward");
 	return 0;
 }
@@ -991,7 +987,7 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 	std::vector<rgs::BlendArgs> jobs;
 	std::vector<int> job_layer;
 	std::vector<rgs::PreprocessBackwardArgs> geometry((size_t)K);
-	std::vector<rgs::FillJob> sums_to_clear, blocks_to_clear;
+	std::vector<rgs::FillJob> sums_to_clear;
 	for (int k = 0; k < K; k++) {
 		const rgs_frame_layer& l = layers[k];
 		if (int rc = check_backward_pointers("rgs_frame_backward", l.P, l.R, view->width, view->height, l.background, l.means3D,
@@ -1001,8 +997,7 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		                                     l.dL_dmean2D, l.dL_dopacity, l.dL_dcolor, l.dL_dmean3D, l.dL_dcov3D, l.dL_dsh,
 		                                     l.dL_dscale, l.dL_drot))
 			return rc;
-		RGS_REQUIRE(!l.grad_block || (l.grad_block_bytes & 3) == 0, "rgs_frame_backward: grad_block_bytes must be a multiple of 4");
-		if (!l.outputs_zeroed)  // the blend adds into the rows of sums: they come first, on the frame's stream
+		if (!l.accum_zeroed)  // the blend adds into the rows of sums: they come first, on the frame's stream
 			sums_to_clear.push_back(rgs::FillJob{reinterpret_cast<uint32_t*>(l.grad_accum), (size_t)RGS_ACC_FLOATS * (size_t)l.P});
 		if (l.R > 0) {
 			rgs::BlendArgs a;
@@ -1024,9 +1019,6 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 		rgs::launch_fill_many(sums_to_clear.data(), (int)sums_to_clear.size(), 0u, s);
 		RGS_STAGE("clear gradient sums");
 	}
-	// Gradient arrays that the caller has not cleared are cleared here, on the second stream if there is one (a caller
-	// with a second stream does better to clear them there during the forward: the backward blend fills every SIMD's
-	// registers, and stores beside it were measured to slow it down by as much as they take).
 	hipError_t e = hipSuccess;
 	if (beside != s) {
 		hipEvent_t begun = frame_event(0);
@@ -1035,22 +1027,6 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 			e = hipStreamWaitEvent(beside, begun, 0);
 		if (e != hipSuccess)
 			return fail("rgs_frame_backward: ordering the streams failed: %s", hipGetErrorString(e));
-	}
-	std::vector<int> already((size_t)K, 1);  // as far as launch_preprocess_backward is concerned: cleared here, or by the caller
-	for (int k = 0; k < K; k++) {
-		const rgs_frame_layer& l = layers[k];
-		if (l.outputs_zeroed)
-			continue;
-		if (l.grad_block)
-			blocks_to_clear.push_back(rgs::FillJob{static_cast<uint32_t*>(l.grad_block), l.grad_block_bytes / 4});
-		else
-			already[(size_t)k] = 0;
-	}
-	if (!blocks_to_clear.empty()) {  // one launch for every layer's block
-		if (beside == s)
-			rgs::stage_mark("clear_gradients", s);
-		rgs::launch_fill_many(blocks_to_clear.data(), (int)blocks_to_clear.size(), 0u, beside);
-		RGS_STAGE("clear gradients");
 	}
 	// With a second stream the blend goes in two halves, so that the per-Gaussian backward of the first half's layers
 	// (memory bandwidth) runs beside the blend of the second half.  Layers without instances go with the last half.
@@ -1067,12 +1043,9 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 			RGS_STAGE("blend_backward");
 		}
 		std::vector<rgs::PreprocessBackwardArgs> part;
-		std::vector<int> part_zeroed;
 		for (int k = 0; k < K; k++)
-			if (halves == 1 || (in_first[(size_t)k] != 0) == (half == 0)) {
+			if (halves == 1 || (in_first[(size_t)k] != 0) == (half == 0))
 				part.push_back(geometry[(size_t)k]);
-				part_zeroed.push_back(already[(size_t)k]);
-			}
 		if (part.empty())
 			continue;
 		if (beside != s) {
@@ -1083,7 +1056,7 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 			if (e != hipSuccess)
 				return fail("rgs_frame_backward: ordering the streams failed: %s", hipGetErrorString(e));
 		}
-		rgs::launch_preprocess_backward(part.data(), part_zeroed.data(), (int)part.size(), beside);
+		rgs::launch_preprocess_backward(part.data(), (int)part.size(), beside);
 		RGS_STAGE("preprocess_backward");
 	}
 	if (beside != s) {

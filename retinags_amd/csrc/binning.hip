@@ -260,7 +260,6 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 	const uint32_t* __restrict__ visible_base = j.block_visible;
 	uint32_t* __restrict__ keys = j.keys_a;
 	uint32_t* __restrict__ values = j.order;
-	uint32_t* __restrict__ visible_list = j.visible_list;
 #pragma unroll
 	for (int p = 0; p < 4; p++)
 		s_hist[p][threadIdx.x] = 0u;
@@ -294,7 +293,6 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 				const uint32_t key = __float_as_uint(depth[q]);
 				keys[at] = key;
 				values[at] = (uint32_t)(idx0 + q);
-				visible_list[at] = (uint32_t)(idx0 + q);  // the sort reorders `values`; this copy stays in index order
 				at++;
 #pragma unroll
 				for (int p = 0; p < 4; p++)

@@ -418,26 +418,35 @@ __attribute__((amdgpu_waves_per_eu(RGS_PB_WAVES, RGS_PB_WAVES)))
 __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<PreprocessBackwardArgs> batch)
 {
 	__shared__ float4 s_rows[2][32 * kShRowStride];
-	__shared__ uint32_t s_index[2][64];
+	__shared__ uint8_t s_listed[2][64];
 	const PreprocessBackwardArgs& a = batch.job[blockIdx.y];
-	const uint32_t listed = *a.visible_count;
+	if (blockIdx.x * 128u >= (uint32_t)a.P)
+		return;  // the launch is sized for the job with the most Gaussians
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	const uint32_t k_first = blockIdx.x * 128 + wave * 64;
-	if (k_first >= listed)
-		return;  // the whole wavefront
-	// Spare lanes of the list's last wavefront repeat its last Gaussian (the same values go to the
-	// same places), so that the whole wavefront takes part where its lanes share the work.
-	const uint32_t k_vis = min(k_first + (uint32_t)lane, listed - 1u);
-	const size_t i = (size_t)a.visible_list[k_vis];
+	const size_t i = (size_t)blockIdx.x * 128 + threadIdx.x;
+	const bool present = i < (size_t)a.P;
+	const bool rendered = present && a.radii[i] > 0;  // backward.cu:357: the others get zeros
 	const int n_sh = a.shs ? a.M * 3 : 0;
 	float mean2d_x = 0.f, mean2d_y = 0.f, opacity_sum = 0.f, color_sum[3] = {0.f, 0.f, 0.f};
+	float3 dmean = {0.f, 0.f, 0.f};
+	float dcov[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+	float ds[3] = {0.f, 0.f, 0.f};
+	float4 dq = {0.f, 0.f, 0.f, 0.f};
 
-	{
 	const float* __restrict__ view = a.view;
 	const float* __restrict__ proj = a.proj;
-	const float3 mean = {a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
-	const float4* sums = reinterpret_cast<const float4*>(a.sums + kSumCols * i);
-	const float4 sum0 = sums[0], sum1 = sums[1], sum2v = sums[2];
+	float3 mean = {0.f, 0.f, 0.f};
+	float4 sum0 = {0.f, 0.f, 0.f, 0.f}, sum1 = sum0, sum2v = sum0;
+	uint32_t cl = 0;
+	if (rendered) {
+		mean = float3{a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
+		const float4* sums = reinterpret_cast<const float4*>(a.sums + kSumCols * i);
+		sum0 = sums[0];
+		sum1 = sums[1];
+		sum2v = sums[2];
+		if (a.shs)
+			cl = a.clamped[i];
+	}
 	const float3 dLc = {sum0.z, sum0.w, sum1.x};  // kSumConicXX, kSumConicXY, kSumConicYY
 	const float sum_color[3] = {sum1.z, sum1.w, sum2v.x};
 	mean2d_x = sum0.x;
@@ -455,65 +464,43 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 		const float3 d0 = {mean.x - cam.x, mean.y - cam.y, mean.z - cam.z};
 		const float len = sqrtf(d0.x * d0.x + d0.y * d0.y + d0.z * d0.z);
 		const float x = d0.x / len, y = d0.y / len, z = d0.z / len;
-		const uint32_t cl = a.clamped[i];
-		const float* sh = a.shs + i * n_sh;
 		float ddx = 0.f, ddy = 0.f, ddz = 0.f;
+		float g[3];
+#pragma unroll
+		for (int ch = 0; ch < 3; ch++)
+			g[ch] = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
 		if (a.sh_rows_by_16_bytes) {
-			// The usual case.  The wavefront reads the SH rows of its Gaussians together, 16 lanes
-			// to a row and 16 bytes a lane, parks them in LDS (32 rows at a time) where each lane
-			// picks up its own; the rows of dL_dsh leave the same way.
+			// The usual case.  The wavefront reads the SH rows of its rendered Gaussians together,
+			// 16 lanes to a row and 16 bytes a lane, parks them in LDS (32 rows at a time) where
+			// each lane picks up its own; the rows of dL_dsh, zeros for the others, leave the same way.
 			const int piece = lane & 15, sub = lane >> 4;
 			const int row_pieces = n_sh / 4;
 			const int needed = 3 * (a.D + 1) * (a.D + 1);
 			const int needed_pieces = (needed + 3) / 4;
 			float4* parked = s_rows[wave];
-			uint32_t* index = s_index[wave];
-			index[lane] = (uint32_t)i;
+			uint8_t* listed = s_listed[wave];
+			const uint64_t seen = __ballot(rendered);
+			const int n_seen = __popcll(seen);
+			const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(seen >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)seen, 0u));
+			const size_t wave_first = i - (size_t)lane;
+			const float4* __restrict__ rows = reinterpret_cast<const float4*>(a.shs) + wave_first * row_pieces;
+			float4* __restrict__ grads = reinterpret_cast<float4*>(a.dL_dsh) + wave_first * row_pieces;
+			if (rendered)
+				listed[rank] = (uint8_t)lane;
 			wave_lds_fence();
-			const float4* __restrict__ rows = reinterpret_cast<const float4*>(a.shs);
-			float4* __restrict__ grads = reinterpret_cast<float4*>(a.dL_dsh);
-			float g[3];
-#pragma unroll
-			for (int ch = 0; ch < 3; ch++)
-				g[ch] = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-			for (int h = 0; h < 2; h++) {
-				float4* mine = parked + (lane & 31) * kShRowStride;
+			for (int base = 0; base < n_seen; base += 32) {
 				// (what a lane computes here does not depend on the turn; made opaque so that it is
 				// computed in its turn and not kept in registers across both)
 				float xo = x, yo = y, zo = z, go[3] = {g[0], g[1], g[2]};
 				asm volatile("" : "+v"(xo), "+v"(yo), "+v"(zo), "+v"(go[0]), "+v"(go[1]), "+v"(go[2]));
-				if ((lane >> 5) == h) {
-					// the rows of dL_dsh, which do not depend on the coefficients
-					float none[kShRegs], out[kShRegs];
-#pragma unroll
-					for (int k = 0; k < kShRegs; k++) {
-						none[k] = 0.f;
-						out[k] = 0.f;
-					}
-					float t0 = 0.f, t1 = 0.f, t2 = 0.f;
-#pragma unroll
-					for (int ch = 0; ch < 3; ch++)
-						sh_backward_channel(a.D, xo, yo, zo, none + ch, go[ch], out + ch, t0, t1, t2);
-#pragma unroll
-					for (int k = 0; k < kShRegs; k += 4)
-						if (k < needed)
-							mine[k / 4] = float4{out[k], out[k + 1], out[k + 2], out[k + 3]};
-				}
-				wave_lds_fence();
-				__builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-				for (int r = 0; r < 8; r++)
-					if (piece < needed_pieces)
-						grads[(size_t)index[32 * h + 4 * r + sub] * row_pieces + piece] =
-						    parked[(4 * r + sub) * kShRowStride + piece];
-				wave_lds_fence();
 				{
 					float4 v[8];
 #pragma unroll
 					for (int r = 0; r < 8; r++) {
+						const int slot = base + 4 * r + sub;
 						v[r] = float4{0.f, 0.f, 0.f, 0.f};
-						if (piece < needed_pieces)
-							v[r] = rows[(size_t)index[32 * h + 4 * r + sub] * row_pieces + piece];
+						if (piece < needed_pieces && slot < n_seen)
+							v[r] = rows[(size_t)listed[slot] * row_pieces + piece];
 					}
 #pragma unroll
 					for (int r = 0; r < 8; r++)
@@ -522,8 +509,9 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 				}
 				wave_lds_fence();
 				__builtin_amdgcn_sched_barrier(0);
-				if ((lane >> 5) == h) {
+				if (rendered && rank >= base && rank < base + 32) {
 					// the coefficients' part in the gradient of the view direction
+					const float4* mine = parked + (rank - base) * kShRowStride;
 					float row[kShRegs], unused[kShRegs];
 #pragma unroll
 					for (int k = 0; k < kShRegs; k += 4) {
@@ -542,12 +530,53 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 				wave_lds_fence();
 				__builtin_amdgcn_sched_barrier(0);
 			}
-		} else {
+			for (int h = 0; h < 2; h++) {
+				// the rows of dL_dsh of 32 neighbouring Gaussians; they do not depend on the coefficients
+				if ((size_t)(32 * h) + wave_first >= (size_t)a.P)
+					break;
+				float xo = x, yo = y, zo = z, go[3] = {g[0], g[1], g[2]};
+				asm volatile("" : "+v"(xo), "+v"(yo), "+v"(zo), "+v"(go[0]), "+v"(go[1]), "+v"(go[2]));
+				if ((lane >> 5) == h) {
+					float4* mine = parked + (lane & 31) * kShRowStride;
+					float none[kShRegs], out[kShRegs];
 #pragma unroll
-			for (int ch = 0; ch < 3; ch++) {
-				const float g = sum_color[ch] * (((cl >> ch) & 1u) ? 0.f : 1.f);
-				sh_backward_channel(a.D, x, y, z, sh + ch, g, a.dL_dsh + i * n_sh + ch, ddx, ddy, ddz);
+					for (int k = 0; k < kShRegs; k++) {
+						none[k] = 0.f;
+						out[k] = 0.f;
+					}
+					if (rendered) {
+						float t0 = 0.f, t1 = 0.f, t2 = 0.f;
+#pragma unroll
+						for (int ch = 0; ch < 3; ch++)
+							sh_backward_channel(a.D, xo, yo, zo, none + ch, go[ch], out + ch, t0, t1, t2);
+					}
+#pragma unroll
+					for (int k = 0; k < kShRegs; k += 4)
+						if (k < n_sh)
+							mine[k / 4] = float4{out[k], out[k + 1], out[k + 2], out[k + 3]};
+				}
+				wave_lds_fence();
+				__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+				for (int r = 0; r < 8; r++) {
+					const int row = 32 * h + 4 * r + sub;
+					if (piece < row_pieces && wave_first + (size_t)row < (size_t)a.P)
+						grads[(size_t)row * row_pieces + piece] = parked[(4 * r + sub) * kShRowStride + piece];
+				}
+				wave_lds_fence();
+				__builtin_amdgcn_sched_barrier(0);
 			}
+		} else if (present) {
+			float* dst = a.dL_dsh + i * n_sh;
+			const int needed = 3 * (a.D + 1) * (a.D + 1);
+			if (rendered) {
+				const float* sh = a.shs + i * n_sh;
+#pragma unroll
+				for (int ch = 0; ch < 3; ch++)
+					sh_backward_channel(a.D, x, y, z, sh + ch, g[ch], dst + ch, ddx, ddy, ddz);
+			}
+			for (int k = rendered ? needed : 0; k < n_sh; k++)
+				dst[k] = 0.f;
 		}
 		// normalisation Jacobian (auxiliary.h:123-133)
 		const float sum2 = d0.x * d0.x + d0.y * d0.y + d0.z * d0.z;
@@ -557,6 +586,7 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 		sh_dmean.z = (-d0.x * d0.z * ddx - d0.y * d0.z * ddy + (sum2 - d0.z * d0.z) * ddz) * invsum32;
 	}
 
+	if (rendered) {
 	// -- conic -> cov2D -> cov3D and mean (backward.cu:144-274)
 	float cov6r[6];
 	if (a.cov3D_precomp) {
@@ -575,7 +605,6 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	const float denom = ca * cc - cb * cb;
 	float dL_da = 0.f, dL_db = 0.f, dL_dc = 0.f;
 	const float denom2inv = 1.0f / ((denom * denom) + 0.0000001f);
-	float dcov[6];
 #define TM(i, j) e.T.c[i][j]
 #define VM(i, j) e.Vrk.c[i][j]
 	if (denom2inv != 0.f) {
@@ -596,12 +625,6 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 		for (int k = 0; k < 6; k++)
 			dcov[k] = 0.f;
 	}
-	if (a.dL_dcov3D) {  // null when the covariance comes from scale and rotation and nobody asks for this intermediate
-#pragma unroll
-		for (int k = 0; k < 6; k++)
-			a.dL_dcov3D[6 * i + k] = dcov[k];
-	}
-
 	const float dL_dT00 = 2 * (TM(0, 0) * VM(0, 0) + TM(0, 1) * VM(0, 1) + TM(0, 2) * VM(0, 2)) * dL_da +
 	                      (TM(1, 0) * VM(0, 0) + TM(1, 1) * VM(0, 1) + TM(1, 2) * VM(0, 2)) * dL_db;
 	const float dL_dT01 = 2 * (TM(0, 0) * VM(1, 0) + TM(0, 1) * VM(1, 1) + TM(0, 2) * VM(1, 2)) * dL_da +
@@ -628,7 +651,6 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	const float dL_dty = y_grad_mul * -h_y * tz2 * dL_dJ12;
 	const float dL_dtz = -h_x * tz2 * dL_dJ00 - h_y * tz2 * dL_dJ11 + (2 * h_x * e.t.x) * tz3 * dL_dJ02 +
 	                     (2 * h_y * e.t.y) * tz3 * dL_dJ12;
-	float3 dmean;
 	dmean.x = view[0] * dL_dtx + view[1] * dL_dty + view[2] * dL_dtz;
 	dmean.y = view[4] * dL_dtx + view[5] * dL_dty + view[6] * dL_dtz;
 	dmean.z = view[8] * dL_dtx + view[9] * dL_dty + view[10] * dL_dtz;
@@ -653,9 +675,6 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 	dmean.x += sh_dmean.x;
 	dmean.y += sh_dmean.y;
 	dmean.z += sh_dmean.z;
-	a.dL_dmeans[3 * i + 0] = dmean.x;
-	a.dL_dmeans[3 * i + 1] = dmean.y;
-	a.dL_dmeans[3 * i + 2] = dmean.z;
 
 	// -- 3D covariance -> scale and raw quaternion (backward.cu:278-341)
 	if (a.scales) {
@@ -680,20 +699,15 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 		const M3 dM = m3_mul(M2, dSigma);
 		const M3 Rt = m3_transpose(R);
 		M3 dMt = m3_transpose(dM);
-		float ds[3];
 #pragma unroll
 		for (int k = 0; k < 3; k++)
 			ds[k] = Rt.c[k][0] * dMt.c[k][0] + Rt.c[k][1] * dMt.c[k][1] + Rt.c[k][2] * dMt.c[k][2];
-		a.dL_dscale[3 * i + 0] = ds[0];
-		a.dL_dscale[3 * i + 1] = ds[1];
-		a.dL_dscale[3 * i + 2] = ds[2];
 #pragma unroll
 		for (int k = 0; k < 3; k++)
 #pragma unroll
 			for (int rr = 0; rr < 3; rr++)
 				dMt.c[k][rr] *= s[k];
 #define DM(i, j) dMt.c[i][j]
-		float4 dq;
 		dq.x = 2 * z * (DM(0, 1) - DM(1, 0)) + 2 * y * (DM(2, 0) - DM(0, 2)) + 2 * x * (DM(1, 2) - DM(2, 1));
 		dq.y = 2 * y * (DM(1, 0) + DM(0, 1)) + 2 * z * (DM(2, 0) + DM(0, 2)) + 2 * r * (DM(1, 2) - DM(2, 1)) -
 		       4 * x * (DM(2, 2) + DM(1, 1));
@@ -702,13 +716,31 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 		dq.w = 2 * r * (DM(0, 1) - DM(1, 0)) + 2 * x * (DM(2, 0) + DM(0, 2)) + 2 * y * (DM(1, 2) + DM(2, 1)) -
 		       4 * z * (DM(1, 1) + DM(0, 0));
 #undef DM
-		reinterpret_cast<float4*>(a.dL_drot)[i] = dq;
 	}
 	}
 
+	// Every Gaussian's rows are written, zeros for those that were not rendered: the arrays need no clearing.
+	if (!present)
+		return;
+	a.dL_dmeans[3 * i + 0] = dmean.x;
+	a.dL_dmeans[3 * i + 1] = dmean.y;
+	a.dL_dmeans[3 * i + 2] = dmean.z;
+	if (a.dL_dcov3D) {  // null when the covariance comes from scale and rotation and nobody asks for this intermediate
+#pragma unroll
+		for (int k = 0; k < 6; k++)
+			a.dL_dcov3D[6 * i + k] = dcov[k];
+	}
+	if (a.dL_dscale) {
+		a.dL_dscale[3 * i + 0] = ds[0];
+		a.dL_dscale[3 * i + 1] = ds[1];
+		a.dL_dscale[3 * i + 2] = ds[2];
+	}
+	if (a.dL_drot)
+		reinterpret_cast<float4*>(a.dL_drot)[i] = dq;
 	// the sums that are gradients as they stand
 	a.dL_dmean2D[3 * i + 0] = mean2d_x;
 	a.dL_dmean2D[3 * i + 1] = mean2d_y;
+	a.dL_dmean2D[3 * i + 2] = 0.f;
 	a.dL_dopacity[i] = opacity_sum;
 	if (a.dL_dcolor) {  // null when the colours come from SH and nobody asks for this intermediate
 		a.dL_dcolor[3 * i + 0] = color_sum[0];
@@ -759,27 +791,8 @@ void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_
 	}
 }
 
-void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, const int* outputs_zeroed, int count, hipStream_t s)
+void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, int count, hipStream_t s)
 {
-	for (int k = 0; k < count; k++)
-		if (!outputs_zeroed[k]) {
-			const PreprocessBackwardArgs& a = jobs[k];
-			stage_mark("clear_gradients", s);
-			const size_t n = (size_t)a.P;
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmean2D), 0u, 3 * n, s);
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dopacity), 0u, n, s);
-			if (a.dL_dcolor)
-				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcolor), 0u, 3 * n, s);
-			launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dmeans), 0u, 3 * n, s);
-			if (a.dL_dcov3D)
-				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dcov3D), 0u, 6 * n, s);
-			if (a.shs)
-				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dsh), 0u, (size_t)a.M * 3 * n, s);
-			if (a.scales) {
-				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_dscale), 0u, 3 * n, s);
-				launch_fill_u32(reinterpret_cast<uint32_t*>(a.dL_drot), 0u, 4 * n, s);
-			}
-		}
 	stage_mark("preprocess_backward", s);
 	for (int at = 0; at < count; at += kMaxBatch) {
 		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;

@@ -60,10 +60,8 @@ struct PreprocessBackwardArgs {
 	const float* campos;
 	float focal_x, focal_y, tanfovx, tanfovy;
 	const float* sums;  // (P, kSumCols): what the backward blend accumulated, see SumCol
-	const uint32_t* visible_list;   // the Gaussians that touch a tile, in index order
-	const uint32_t* visible_count;  // how many (on the device)
 	bool sh_rows_by_16_bytes;       // SH rows are 16-byte aligned, a multiple of 16 bytes long and at most 48 floats
-	// outputs: rows of the listed Gaussians are written, all other rows must be zero already
+	// outputs: every row is written, zeros where radii[i] <= 0
 	float* dL_dmean2D;  // (P,3), third column 0
 	float* dL_dopacity; // (P)
 	float* dL_dcolor;   // (P,3)
@@ -280,8 +278,8 @@ void launch_mark_visible(int P, const float* means, const float* view, uint8_t* 
 void launch_covariance3d(int P, const float* scales, float scale_modifier, const float* rotations, float* cov3D, hipStream_t s);
 // `jobs` are host arrays: the submodels of a frame in one launch (kMaxBatch of them at a time).
 void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_t s);
-// Where outputs_zeroed[k] is 0 the eight output arrays of job k are cleared first.
-void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, const int* outputs_zeroed, int count, hipStream_t s);
+// Writes every row of the output arrays (zeros for Gaussians that were not rendered).
+void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, int count, hipStream_t s);
 
 // binning.hip
 constexpr int kSortItems = 16;                    // keys per thread in one sort block
@@ -305,7 +303,7 @@ void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t
 // their count per 256 Gaussians and *visible_count the total; sort_temp has been cleared
 // (sort_clear_words(P, 32) words).  On return order[0..count)
 // lists them by increasing depth, ties by index, and offsets_in_order is the inclusive scan of
-// their tile counts in that order; visible_list keeps them in index order.  The count stays on the device: every kernel is launched
+// their tile counts in that order.  The count stays on the device: every kernel is launched
 // for P elements and reads it.
 struct DepthOrderJob {
 	int P;
@@ -313,7 +311,6 @@ struct DepthOrderJob {
 	const uint32_t* tiles_touched;
 	uint32_t* block_visible;
 	uint32_t* visible_count;
-	uint32_t* visible_list;
 	uint32_t* keys_a;
 	uint32_t* keys_b;
 	uint32_t* order;

@@ -117,6 +117,20 @@ def raster_settings(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
         campos=cam.camera_center, prefiltered=False, debug=debug)
 
 
+def _screenspace_placeholder(sub: Submodel) -> torch.Tensor:
+    """The zero tensor whose gradient carries the screen-space gradient of the means
+    (gaussian_renderer/render.py:16 makes one with zeros_like per render).  Nothing
+    ever writes its values, so one block of zeros per submodel serves every frame: a frame that
+    takes gradients gets a fresh leaf over that block (its own .grad, no fill), one that does
+    not gets the block itself."""
+    zeros = getattr(sub, "_still_means2D", None)
+    if zeros is None or zeros.shape != sub.means3D.shape or zeros.device != sub.means3D.device \
+            or zeros.dtype != sub.means3D.dtype:
+        zeros = torch.zeros_like(sub.means3D, requires_grad=False)
+        sub._still_means2D = zeros
+    return zeros.detach().requires_grad_(True) if sub.means3D.requires_grad else zeros
+
+
 def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifier: float = 1.0,
                     debug: bool = False, started=None) -> dict:
     """Same call sequence and return dict as render4renderinfo
@@ -128,7 +142,7 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
         rasterizer, geometry = started
     means2D = sub.means2D
     if means2D is None:
-        means2D = torch.zeros_like(sub.means3D, requires_grad=sub.means3D.requires_grad)
+        means2D = _screenspace_placeholder(sub)
     color, radii, depth, alpha = rasterizer(
         means3D=sub.means3D, means2D=means2D, shs=sub.shs, colors_precomp=None, opacities=sub.opacity,
         scales=sub.scales, rotations=sub.rotations, cov3D_precomp=None, geometry=geometry)
@@ -231,14 +245,7 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
             sub = subs[m]
             means2D = sub.means2D
             if means2D is None:
-                if sub.means3D.requires_grad:
-                    means2D = torch.zeros_like(sub.means3D, requires_grad=True)
-                else:
-                    # nothing reads or writes the placeholder without a backward: one zero tensor serves every frame
-                    means2D = getattr(sub, "_still_means2D", None)
-                    if means2D is None or means2D.shape != sub.means3D.shape or means2D.device != sub.means3D.device:
-                        means2D = torch.zeros_like(sub.means3D)
-                        sub._still_means2D = means2D
+                means2D = _screenspace_placeholder(sub)
             rasterizers.append(GaussianRasterizer(raster_settings=raster_settings(cam, sub, submodel_bg)))
             inputs.append(dict(means3D=sub.means3D, means2D=means2D, shs=sub.shs, opacities=sub.opacity, scales=sub.scales,
                                rotations=sub.rotations))

@@ -229,40 +229,36 @@ def _rasterize_forward(*args):
     return _forward_blend(_forward_geometry(*args, wait=True))
 
 
-def _gradient_outputs(P, M, has_scales, device, make, scratch=()):
+def _gradient_outputs(P, M, device, scratch=(), sums=None):
     """The eight dense gradient tensors of K/rasterize_points.cu:165-174, carved out of one
-    allocation made with `make` (torch.empty or torch.zeros: one fill instead of eight), and the
-    backward's scratch for the per-Gaussian sums in an allocation of its own, so that a gradient
-    the caller keeps (the means2D gradient, say, for densification statistics) does not hold on to
-    the scratch.  The eight do share one block: keeping any of them keeps all (about 280 bytes
-    per Gaussian with SH degree 3).  Without scales the scale / rotation gradients are zeros in
-    either case.  `scratch` names those of the eight that the caller hands to nobody (the colour
-    gradient when the colours come from SH, the covariance gradient when it comes from scale and
-    rotation): they are not made at all (None), and the library does not write them."""
+    uninitialised allocation (the library writes every row of them: those of Gaussians that were
+    not rendered as zeros), and the backward's scratch for the per-Gaussian sums in an
+    allocation of its own (`sums`, if the caller has made and cleared it already), so that a
+    gradient the caller keeps (the means2D gradient, say, for densification statistics) does not
+    hold on to the scratch.  The eight do share one block: keeping any of them keeps all (about
+    280 bytes per Gaussian with SH degree 3).  `scratch` names those of the eight that the caller
+    hands to nobody (the colour gradient when the colours come from SH, the covariance gradient
+    when it comes from scale and rotation): they are not made at all (None), and the library
+    does not write them."""
     shapes = {"means2D": (P, 3), "opacity": (P, 1), "colors": (P, 3), "means3D": (P, 3), "cov3D": (P, 6),
               "sh": (P, M, 3), "scales": (P, 3), "rotations": (P, 4)}
     order = [k for k in shapes if k not in scratch]
     sizes = {k: (math.prod(v) + 63) // 64 * 64 for k, v in shapes.items()}  # 256-byte aligned parts
-    flat = make((sum(sizes[k] for k in order),), dtype=torch.float32, device=device)
+    flat = torch.empty((sum(sizes[k] for k in order),), dtype=torch.float32, device=device)
     out, at = {k: None for k in scratch}, 0
     for k in order:
         out[k] = flat[at:at + math.prod(shapes[k])].view(shapes[k])
         at += sizes[k]
-    out["block"] = flat  # what has to be cleared, as one tensor
-    out["sums"] = make((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
-    if not has_scales and make is not torch.zeros:
-        out["scales"].zero_()
-        out["rotations"].zero_()
+    out["sums"] = sums if sums is not None else torch.empty((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
     return out
 
 
 def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, scale_modifier, cov3Ds_precomp,
                         viewmatrix, projmatrix, projmatrix_inv, range_low, range_up, tanfovx, tanfovy, grad_color,
                         grad_depth, grad_alpha, sh, sh_degree, campos, geomBuffer, num_rendered, binningBuffer,
-                        imgBuffer, alpha, debug, cleared=None):
+                        imgBuffer, alpha, debug):
     """Counterpart of RasterizeGaussiansBackwardCUDA_hgs (K/rasterize_points.cu:127-220);
-    returns the same 8 tensors in the same order.  `cleared`, if given, is the dict of output
-    tensors that the forward made with _gradient_outputs(..., torch.zeros)."""
+    returns the same 8 tensors in the same order."""
     device = means3D.device
     P = int(means3D.shape[0])
     H, W = int(grad_color.shape[1]), int(grad_color.shape[2])
@@ -291,9 +287,7 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
     range_up = _dev_f32(range_up, device, "range_up")
     campos = _dev_f32(campos, device, "campos")
 
-    has_scales = scales.numel() != 0
-    outputs_zeroed = cleared is not None
-    out = cleared if outputs_zeroed else _gradient_outputs(P, M, has_scales, device, torch.empty)
+    out = _gradient_outputs(P, M, device)
     acc = out["sums"]  # scratch rows in which the blend accumulates its per-Gaussian sums
     dL_dmeans2D, dL_dopacity, dL_dcolors = out["means2D"], out["opacity"], out["colors"]
     dL_dmeans3D, dL_dcov3D, dL_dsh = out["means3D"], out["cov3D"], out["sh"]
@@ -307,8 +301,7 @@ def _rasterize_backward(bg, means3D, radii, colors_precomp, scales, rotations, s
             float(tanfovy), ptr(radii), ptr(geomBuffer), ptr(binningBuffer), ptr(imgBuffer), ptr(grad_color),
             ptr(grad_depth), ptr(grad_alpha), ptr(acc), ptr(dL_dmeans2D), ptr(dL_dopacity), ptr(dL_dcolors),
             ptr(dL_dmeans3D), ptr(dL_dcov3D), ptr(dL_dsh),
-            ptr(dL_dscales) if has_scales else C.c_void_p(0), ptr(dL_drotations) if has_scales else C.c_void_p(0),
-            int(outputs_zeroed), _stream_ptr(device), int(bool(debug))))
+            ptr(dL_dscales), ptr(dL_drotations), 0, _stream_ptr(device), int(bool(debug))))
 
     return dL_dmeans2D, dL_dcolors, dL_dopacity, dL_dmeans3D, dL_dcov3D, dL_dsh, dL_dscales, dL_drotations
 
@@ -375,15 +368,6 @@ class _RasterizeGaussians(torch.autograd.Function):
         ctx.set_materialize_grads(False)  # an output that took no part in the loss comes back as None, not as a tensor of zeros
         ctx.raster_settings = raster_settings
         ctx.num_rendered = num_rendered
-        # Only rendered Gaussians get non-zero gradients and the library writes just those rows;
-        # the rest of the gradient tensors is cleared here, behind the forward blend on this
-        # stream, where the clearing (pure memory traffic) overlaps other streams' blend kernels
-        # instead of lengthening the backward pass.
-        ctx.cleared = None
-        P = int(means3D.shape[0])
-        if P > 0 and any(ctx.needs_input_grad):
-            M = int(sh.shape[1]) if sh.numel() != 0 else 0
-            ctx.cleared = _gradient_outputs(P, M, scales.numel() != 0, means3D.device, torch.zeros)
         ctx.save_for_backward(colors_precomp, means3D, scales, rotations, cov3Ds_precomp, radii, sh, geomBuffer,
                               binningBuffer, imgBuffer, alpha)
         ctx.mark_non_differentiable(radii)
@@ -416,14 +400,13 @@ class _RasterizeGaussians(torch.autograd.Function):
         if raster_settings.debug:
             cpu_args = cpu_deep_copy_tuple(args)
             try:
-                outs = _rasterize_backward(*args, cleared=ctx.cleared)
+                outs = _rasterize_backward(*args)
             except Exception as ex:
                 torch.save(cpu_args, "snapshot_bw.dump")
                 print("\nAn error occured in backward. Writing snapshot_bw.dump for debugging.\n")
                 raise ex
         else:
-            outs = _rasterize_backward(*args, cleared=ctx.cleared)
-        ctx.cleared = None  # the tensors now belong to the caller
+            outs = _rasterize_backward(*args)
         (grad_means2D, grad_colors_precomp, grad_opacities, grad_means3D, grad_cov3Ds_precomp, grad_sh, grad_scales,
          grad_rotations) = outs
 
@@ -515,26 +498,22 @@ class _RasterizeFrame(torch.autograd.Function):
                 L.geom_bytes, L.image_bytes = geom_bytes, image_bytes
                 L.out_color, L.out_depth, L.out_alpha = ptr(package[0:3]), ptr(package[3:4]), ptr(package[4:5])
             if live:
-                # With a second stream and a backward to come, the gradient tensors are made now and cleared on that
-                # stream while this stream bins and blends (the backward blend leaves the clearing no room beside it).
+                # With a second stream and a backward to come, the backward's per-Gaussian sums are made now and cleared
+                # on that stream while this stream bins and blends.
                 cleared, cleared_event = None, None
                 side = next((h for h in streams if h != main), None) if streams is not None else None
                 if side is not None and any(ctx.needs_input_grad[2:]):
                     cleared = {}
                     for k in live:
-                        rec = records[k]
-                        t_k = rec["t"]
-                        cleared[k] = _gradient_outputs(rec["P"], rec["M"], t_k["scales"].numel() != 0, device, torch.empty,
-                                                       scratch=_frame_scratch(t_k["colors_precomp"], t_k["cov3Ds_precomp"]))
+                        cleared[k] = torch.empty((records[k]["P"], _capi.ACC_FLOATS), **f32)
                     begun = torch.cuda.Event()
                     begun.record(torch.cuda.current_stream(device))
                     side_stream = torch.cuda.ExternalStream(side, device=device)
                     side_stream.wait_event(begun)  # whatever used this memory before did so ahead of this point
                     with torch.cuda.stream(side_stream):
-                        for out in cleared.values():
-                            for name in ("block", "sums"):
-                                out[name].zero_()
-                                out[name].record_stream(side_stream)  # not to be handed out again before this is done
+                        for sums in cleared.values():
+                            sums.zero_()
+                            sums.record_stream(side_stream)  # not to be handed out again before this is done
                         cleared_event = torch.cuda.Event()
                         cleared_event.record(side_stream)
                 counts = _frame_counts(device, len(live))
@@ -590,12 +569,8 @@ class _RasterizeFrame(torch.autograd.Function):
                 continue
             if g_color is None:
                 g_color = torch.zeros((3, H, W), **f32)
-            has_scales = scales.numel() != 0
-            # Only rendered Gaussians get their gradient rows written; the library clears the rest (beside the blend,
-            # on the second stream, if it is given one).
-            ready = ctx.cleared.pop(k, None) if ctx.cleared else None  # made and cleared during the forward; used once
-            out = ready if ready is not None else _gradient_outputs(P, M, has_scales, device, torch.empty,
-                                                                    scratch=_frame_scratch(colors_precomp, cov3Ds))
+            ready = ctx.cleared.pop(k, None) if ctx.cleared else None  # the sums' rows, made and cleared during the forward; used once
+            out = _gradient_outputs(P, M, device, scratch=_frame_scratch(colors_precomp, cov3Ds), sums=ready)
             keep.append(out)   # its scratch rows must outlive the library call below
             t = dict(bg=_dev_f32(rs.bg, device, "bg"), low=_dev_f32(rs.range_low, device, "range_low"),
                      up=_dev_f32(rs.range_up, device, "range_up"), g_color=_dev_f32(g_color, device, "grad_color"),
@@ -622,11 +597,8 @@ class _RasterizeFrame(torch.autograd.Function):
             L.grad_accum = ptr(out["sums"])
             L.dL_dmean2D, L.dL_dopacity, L.dL_dcolor = ptr(out["means2D"]), ptr(out["opacity"]), ptr(out["colors"])
             L.dL_dmean3D, L.dL_dcov3D, L.dL_dsh = ptr(out["means3D"]), ptr(out["cov3D"]), ptr(out["sh"])
-            L.dL_dscale = ptr(out["scales"]) if has_scales else C.c_void_p(0)
-            L.dL_drot = ptr(out["rotations"]) if has_scales else C.c_void_p(0)
-            L.outputs_zeroed = 1 if ready is not None else 0
-            L.grad_block = out["block"].data_ptr()
-            L.grad_block_bytes = out["block"].numel() * 4
+            L.dL_dscale, L.dL_drot = ptr(out["scales"]), ptr(out["rotations"])
+            L.accum_zeroed = 1 if ready is not None else 0
             L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
             results.append((out["means2D"], out["colors"], out["opacity"], out["means3D"], out["cov3D"], out["sh"],
                             out["scales"], out["rotations"]))
@@ -669,8 +641,8 @@ def rasterize_frame(rasterizers, inputs, streams=None):
     camera and the image size); `inputs`: K dicts with the keyword arguments of GaussianRasterizer.forward
     (means3D, means2D, opacities, shs / colors_precomp, scales + rotations / cov3D_precomp); `streams`: None,
     or for every layer the handle of a HIP stream; the first that is not the current stream takes memory-bound work
-    beside the kernels of the current one: if a backward is to come, the gradient tensors are made and cleared on it
-    during the forward, and the backward runs the per-Gaussian part of the layers whose blend is done on it
+    beside the kernels of the current one: if a backward is to come, the rows of its per-Gaussian sums are made and
+    cleared on it during the forward, and the backward runs the per-Gaussian part of the layers whose blend is done on it
     (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
     forward calls, and differentiates like them."""
     flat = []
