@@ -85,8 +85,10 @@ def parse():
     ap.add_argument("--forward-only", action="store_true",
                     help="render and composite only (the ms/frame figure; ms_per_step is then the render time)")
     ap.add_argument("--cpu-threads", type=int, default=0)
-    ap.add_argument("--streams", type=int, default=4,
-                    help="render the submodels of a frame on this many HIP streams (0: all on the current stream)")
+    ap.add_argument("--streams", type=int, default=0,
+                    help="0: every kernel of a frame on the current stream (the default, and the fastest since the gradient "
+                         "arrays need no clearing); N > 0: offer the library N HIP streams (it runs the per-Gaussian "
+                         "backward beside the blend on the second); value_one_stream is then reported next to value")
     ap.add_argument("--instance-room", type=float, default=0.0,
                     help="if > 0: room for (Gaussian, tile) instances as a multiple of the first frame's count; the "
                          "forward then runs without a host round trip and the count is checked after each frame "
