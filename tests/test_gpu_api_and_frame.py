@@ -393,28 +393,51 @@ def test_frame_with_instance_bounds_matches_the_waiting_frame():
     torch.cuda.synchronize()
 
 
-def test_backward_clears_the_gradients_itself_when_the_caller_has_not():
-    """The first backward of a forward call uses gradient tensors cleared during the forward;
-    a second one over the retained graph has none and lets the library clear them.  Both give
-    the same gradients (up to the order of the float atomics)."""
-    from retinags_amd import GaussianRasterizer
+@pytest.mark.parametrize("through_frame", [False, True])
+def test_backward_writes_every_gradient_row_whatever_the_arrays_held(monkeypatch, through_frame):
+    """The reference's shim hands its backward zero-filled gradient tensors
+    (K/rasterize_points.cu:165-174) and the kernel writes the rendered Gaussians' rows; here the
+    tensors arrive uninitialised and the library writes every row, zeros for the Gaussians that
+    were not rendered.  With every output (and the scratch of the sums) poisoned beforehand the
+    gradients are those of an unpoisoned run (up to the order of the float atomics), free of
+    NaN, and exactly zero where nothing was rendered."""
+    from retinags_amd import GaussianRasterizer, rasterizer
     scene, cam, low, up = _small_inputs(n=5000, seed=4)
     scene = dict(scene)
     scene["xyz"] = scene["xyz"].clone()
     scene["xyz"][::3] = 2.0 * cam.camera_center - scene["xyz"][::3]  # every third one behind the camera
     r = GaussianRasterizer(_settings(oracle_settings(cam, low, up, torch.tensor([0.3, 0.2, 0.1]))))
-    leaves = {k: scene[k].to(DEV).requires_grad_(True) for k in ("xyz", "opacity", "shs", "scales", "rotations")}
-    m2d = torch.zeros_like(leaves["xyz"], requires_grad=True)
-    color, radii, depth, alpha = r(means3D=leaves["xyz"], means2D=m2d, opacities=leaves["opacity"], shs=leaves["shs"],
-                                   scales=leaves["scales"], rotations=leaves["rotations"])
-    g = torch.randn(color.shape, generator=torch.Generator().manual_seed(9)).to(DEV) * 1e-2
-    tensors = [m2d] + list(leaves.values())
-    first = torch.autograd.grad([color], tensors, [g], retain_graph=True)
-    second = torch.autograd.grad([color], tensors, [g])
-    assert (radii > 0).any() and not (radii > 0).all()
-    for a, b in zip(first, second):
+
+    def run():
+        leaves = {k: scene[k].to(DEV).requires_grad_(True) for k in ("xyz", "opacity", "shs", "scales", "rotations")}
+        m2d = torch.zeros_like(leaves["xyz"], requires_grad=True)
+        kw = dict(means3D=leaves["xyz"], means2D=m2d, opacities=leaves["opacity"], shs=leaves["shs"],
+                  scales=leaves["scales"], rotations=leaves["rotations"])
+        color, radii, depth, alpha = rasterizer.rasterize_frame([r], [kw])[0] if through_frame else r(**kw)
+        g = torch.randn(color.shape, generator=torch.Generator().manual_seed(9)).to(DEV) * 1e-2
+        return radii, torch.autograd.grad([color], [m2d] + list(leaves.values()), [g])
+
+    radii, clean = run()
+    make = rasterizer._gradient_outputs
+    poisoned = []
+
+    def poisoning(*args, **kwargs):
+        out = make(*args, **kwargs)
+        for name, t in out.items():
+            if t is not None and (name != "sums" or kwargs.get("sums") is None):
+                t.fill_(float("nan"))
+        poisoned.append(out)
+        return out
+
+    monkeypatch.setattr(rasterizer, "_gradient_outputs", poisoning)
+    radii2, dirty = run()
+    assert poisoned and torch.equal(radii, radii2)
+    seen = radii > 0
+    assert seen.any() and not seen.all()
+    for a, b in zip(clean, dirty):
+        assert not torch.isnan(b).any()
         assert rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-4
-        assert torch.equal((a == 0).all(dim=tuple(range(1, a.ndim))), (b == 0).all(dim=tuple(range(1, b.ndim))))
+        assert (b[~seen] == 0).all() and (a[~seen] == 0).all()
 
 
 def test_partial_images_and_their_gradients_come_packed_for_transport():
