@@ -411,10 +411,9 @@ __device__ __forceinline__ void sh_backward_channel(int deg, float x, float y, f
 	ddz += dRGBdz * g;
 }
 
-#ifndef RGS_PB_WAVES
-#define RGS_PB_WAVES 4
-#endif
-__attribute__((amdgpu_waves_per_eu(RGS_PB_WAVES, RGS_PB_WAVES)))
+// Built for 4 wavefronts per SIMD (left alone the compiler keeps both turns of the SH part in registers: 168
+// of them, 3 wavefronts; 3, 4 and 5 measure the same: the kernel is bound by its stores).
+__attribute__((amdgpu_waves_per_eu(4, 4)))
 __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<PreprocessBackwardArgs> batch)
 {
 	__shared__ float4 s_rows[2][32 * kShRowStride];
