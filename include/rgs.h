@@ -61,7 +61,7 @@ size_t rgs_image_bytes(int width, int height);
 /* Byte offsets of the arrays inside the workspaces, for tests and tools that want to
  * look at intermediate results.  The workspaces are otherwise opaque. */
 enum {
-	RGS_GEOM_DEPTHS = 0,        /* float[P]   view-space z */
+	RGS_GEOM_DEPTHS = 0,        /* float[P]   view-space z of the Gaussians that touch a tile (> 0.2), 0 for the others */
 	RGS_GEOM_TILES_TOUCHED,     /* uint32[P] */
 	RGS_GEOM_POINT_OFFSETS,     /* uint32[P]  inclusive prefix sum of the tile counts of the Gaussians in
 	                               RGS_GEOM_DEPTH_ORDER (as many entries as that has) */

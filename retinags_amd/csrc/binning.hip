@@ -256,7 +256,6 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 	if ((size_t)blockIdx.x * kScanGroup >= P)
 		return;
 	const float* __restrict__ depths = j.depths;
-	const uint32_t* __restrict__ tiles_touched = j.tiles_touched;
 	const uint32_t* __restrict__ visible_base = j.block_visible;
 	uint32_t* __restrict__ keys = j.keys_a;
 	uint32_t* __restrict__ values = j.order;
@@ -266,30 +265,27 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 	__syncthreads();
 	for (size_t group = blockIdx.x; group * kScanGroup < P; group += gridDim.x) {
 		const size_t idx0 = group * kScanGroup + 4 * (size_t)threadIdx.x;
-		uint32_t touched[4] = {0u, 0u, 0u, 0u};
+		// the depth of a Gaussian that touches no tile is stored as 0, that of one that does exceeds 0.2: the
+		// depths alone say which ones are listed
 		float depth[4] = {0.f, 0.f, 0.f, 0.f};
 		if (idx0 + 4 <= P) {
-			const uint4 t4 = *reinterpret_cast<const uint4*>(tiles_touched + idx0);
 			const float4 d4 = *reinterpret_cast<const float4*>(depths + idx0);
-			touched[0] = t4.x; touched[1] = t4.y; touched[2] = t4.z; touched[3] = t4.w;
 			depth[0] = d4.x; depth[1] = d4.y; depth[2] = d4.z; depth[3] = d4.w;
 		} else {
 #pragma unroll
 			for (int q = 0; q < 4; q++)
-				if (idx0 + q < P) {
-					touched[q] = tiles_touched[idx0 + q];
+				if (idx0 + q < P)
 					depth[q] = depths[idx0 + q];
-				}
 		}
 		uint32_t mine = 0;
 #pragma unroll
 		for (int q = 0; q < 4; q++)
-			mine += touched[q] != 0u ? 1u : 0u;
+			mine += __float_as_uint(depth[q]) != 0u ? 1u : 0u;
 		uint32_t total;
 		uint32_t at = visible_base[4 * group] + block256_exclusive_scan_u32(mine, lds, total);
 #pragma unroll
 		for (int q = 0; q < 4; q++)
-			if (touched[q] != 0u) {
+			if (__float_as_uint(depth[q]) != 0u) {
 				const uint32_t key = __float_as_uint(depth[q]);
 				keys[at] = key;
 				values[at] = (uint32_t)(idx0 + q);

@@ -303,10 +303,10 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<Preproces
 		if (rendered) {
 			if (!a.colors_precomp)
 				a.clamped[idx] = (uint8_t)clamp_bits;
-			a.depths[idx] = view_z;
 		}
 		a.radii[idx] = (int)my_radius;
 		a.tiles_touched[idx] = touched;
+		a.depths[idx] = view_z;  // 0 for a Gaussian that touches no tile: the depth order lists the others by this alone
 	}
 	{
 		// Everything later stages read of a rendered Gaussian goes into one 64-byte record: a
