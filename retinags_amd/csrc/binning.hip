@@ -528,8 +528,8 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 		for (int q = 0; q < kPerThread; q++) {
 			const bool have = tile_of[q] != 0xFFFFFFFFu;
 			for (int p = 0; p < passes; p++) {
-				const int shift = 8 * p;
-				const int bits = job.end_bit - shift < 8 ? job.end_bit - shift : 8;
+				const int shift = sort_digit_shift(job.end_bit, p);
+				const int bits = sort_digit_bits(job.end_bit, p);
 				const uint32_t d = (tile_of[q] >> shift) & ((1u << bits) - 1u);
 				if (bits <= 2) {
 					// a digit of one or two bits: every lane would add to one of a few words, one after the other
@@ -688,8 +688,8 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 			if (k + q * threads >= n)
 				break;
 			for (int p = 0; p < passes; p++) {
-				const int shift = 8 * p;
-				const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+				const int shift = sort_digit_shift(end_bit, p);
+				const int bits = sort_digit_bits(end_bit, p);
 				const uint32_t d = digit_of(key[q], shift, (1u << bits) - 1u);
 				if (bits <= 2) {
 					// a digit of one or two bits: every lane would add to one of a few words, one after the
@@ -964,8 +964,8 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 		if (!histograms_done)
 			hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
 		for (int p = 0; p < passes; p++) {
-			const int shift = 8 * p;
-			const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+			const int shift = sort_digit_shift(end_bit, p);
+			const int bits = sort_digit_bits(end_bit, p);
 			const uint32_t mask = (1u << bits) - 1u;
 			if (mark_stages)
 				stage_mark("sort_onesweep", s);

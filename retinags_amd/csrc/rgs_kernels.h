@@ -282,6 +282,19 @@ void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_
 void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, int count, hipStream_t s);
 
 // binning.hip
+// A sort on the lowest end_bit bits of its keys takes ceil(end_bit / 8) passes; the bits are shared out evenly
+// between them, the wider digits first (13 bits: 7 then 6, not 8 then 5: the fewer values a digit has, the longer
+// the runs of neighbouring keys a pass writes).
+__host__ __device__ inline int sort_digit_bits(int end_bit, int p)
+{
+	const int n = (end_bit + 7) / 8;
+	return end_bit / n + (p < end_bit % n ? 1 : 0);
+}
+__host__ __device__ inline int sort_digit_shift(int end_bit, int p)
+{
+	const int n = (end_bit + 7) / 8;
+	return p * (end_bit / n) + (p < end_bit % n ? p : end_bit % n);
+}
 constexpr int kSortItems = 16;                    // keys per thread in one sort block
 constexpr int kSortBlock = 256 * kSortItems;      // keys per sort block
 size_t scan_temp_words(size_t n);                 // u32 words of scratch for launch_inclusive_sum
