@@ -229,11 +229,11 @@ def _rasterize_forward(*args):
     return _forward_blend(_forward_geometry(*args, wait=True))
 
 
-def _gradient_outputs(P, M, device, scratch=(), sums=None):
+def _gradient_outputs(P, M, device, scratch=()):
     """The eight dense gradient tensors of K/rasterize_points.cu:165-174, carved out of one
     uninitialised allocation (the library writes every row of them: those of Gaussians that were
     not rendered as zeros), and the backward's scratch for the per-Gaussian sums in an
-    allocation of its own (`sums`, if the caller has made and cleared it already), so that a
+    allocation of its own (the library clears it), so that a
     gradient the caller keeps (the means2D gradient, say, for densification statistics) does not
     hold on to the scratch.  The eight do share one block: keeping any of them keeps all (about
     280 bytes per Gaussian with SH degree 3).  `scratch` names those of the eight that the caller
@@ -249,7 +249,7 @@ def _gradient_outputs(P, M, device, scratch=(), sums=None):
     for k in order:
         out[k] = flat[at:at + math.prod(shapes[k])].view(shapes[k])
         at += sizes[k]
-    out["sums"] = sums if sums is not None else torch.empty((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
+    out["sums"] = torch.empty((P, _capi.ACC_FLOATS), dtype=torch.float32, device=device)
     return out
 
 
@@ -498,24 +498,6 @@ class _RasterizeFrame(torch.autograd.Function):
                 L.geom_bytes, L.image_bytes = geom_bytes, image_bytes
                 L.out_color, L.out_depth, L.out_alpha = ptr(package[0:3]), ptr(package[3:4]), ptr(package[4:5])
             if live:
-                # With a second stream and a backward to come, the backward's per-Gaussian sums are made now and cleared
-                # on that stream while this stream bins and blends.
-                cleared, cleared_event = None, None
-                side = next((h for h in streams if h != main), None) if streams is not None else None
-                if side is not None and any(ctx.needs_input_grad[2:]):
-                    cleared = {}
-                    for k in live:
-                        cleared[k] = torch.empty((records[k]["P"], _capi.ACC_FLOATS), **f32)
-                    begun = torch.cuda.Event()
-                    begun.record(torch.cuda.current_stream(device))
-                    side_stream = torch.cuda.ExternalStream(side, device=device)
-                    side_stream.wait_event(begun)  # whatever used this memory before did so ahead of this point
-                    with torch.cuda.stream(side_stream):
-                        for sums in cleared.values():
-                            sums.zero_()
-                            sums.record_stream(side_stream)  # not to be handed out again before this is done
-                        cleared_event = torch.cuda.Event()
-                        cleared_event.record(side_stream)
                 counts = _frame_counts(device, len(live))
                 check(lib.rgs_frame_forward_geom(len(live), arr, C.byref(view), C.c_void_p(counts.data_ptr()), C.c_void_p(main), debug))
                 got = counts[:len(live)].tolist()
@@ -527,7 +509,6 @@ class _RasterizeFrame(torch.autograd.Function):
                     arr[j].R = rec["rendered"]
                     arr[j].binning_ws, arr[j].binning_bytes = ptr(rec["binning"]), binning_bytes
                 check(lib.rgs_frame_forward_raster(len(live), arr, C.byref(view), C.c_void_p(main), debug))
-        ctx.cleared, ctx.cleared_event = (cleared, cleared_event) if live else (None, None)
         ctx.set_materialize_grads(False)  # an output that took no part in the loss comes back as None, not as a tensor of zeros
         ctx.settings = settings
         ctx.streams = streams
@@ -569,8 +550,7 @@ class _RasterizeFrame(torch.autograd.Function):
                 continue
             if g_color is None:
                 g_color = torch.zeros((3, H, W), **f32)
-            ready = ctx.cleared.pop(k, None) if ctx.cleared else None  # the sums' rows, made and cleared during the forward; used once
-            out = _gradient_outputs(P, M, device, scratch=_frame_scratch(colors_precomp, cov3Ds), sums=ready)
+            out = _gradient_outputs(P, M, device, scratch=_frame_scratch(colors_precomp, cov3Ds))
             keep.append(out)   # its scratch rows must outlive the library call below
             t = dict(bg=_dev_f32(rs.bg, device, "bg"), low=_dev_f32(rs.range_low, device, "range_low"),
                      up=_dev_f32(rs.range_up, device, "range_up"), g_color=_dev_f32(g_color, device, "grad_color"),
@@ -598,14 +578,12 @@ class _RasterizeFrame(torch.autograd.Function):
             L.dL_dmean2D, L.dL_dopacity, L.dL_dcolor = ptr(out["means2D"]), ptr(out["opacity"]), ptr(out["colors"])
             L.dL_dmean3D, L.dL_dcov3D, L.dL_dsh = ptr(out["means3D"]), ptr(out["cov3D"]), ptr(out["sh"])
             L.dL_dscale, L.dL_drot = ptr(out["scales"]), ptr(out["rotations"])
-            L.accum_zeroed = 1 if ready is not None else 0
+            L.accum_zeroed = 0   # the library clears the rows of the sums (48 bytes per Gaussian) ahead of the blend
             L.stream = C.c_void_p(streams[k]) if streams is not None and streams[k] != main else C.c_void_p(0)
             results.append((out["means2D"], out["colors"], out["opacity"], out["means3D"], out["cov3D"], out["sh"],
                             out["scales"], out["rotations"]))
         if live:
             with torch.cuda.device(device):
-                if ctx.cleared_event is not None:
-                    torch.cuda.current_stream(device).wait_event(ctx.cleared_event)
                 check(lib.rgs_frame_backward(live, arr, C.byref(view), C.c_void_p(main), int(bool(rs0.debug))))
         flat = []
         for k in range(K):
@@ -641,9 +619,8 @@ def rasterize_frame(rasterizers, inputs, streams=None):
     camera and the image size); `inputs`: K dicts with the keyword arguments of GaussianRasterizer.forward
     (means3D, means2D, opacities, shs / colors_precomp, scales + rotations / cov3D_precomp); `streams`: None,
     or for every layer the handle of a HIP stream; the first that is not the current stream takes memory-bound work
-    beside the kernels of the current one: if a backward is to come, the rows of its per-Gaussian sums are made and
-    cleared on it during the forward, and the backward runs the per-Gaussian part of the layers whose blend is done on it
-    (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
+    beside the kernels of the current one: the backward runs the per-Gaussian part of the layers whose blend is done
+    on it (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
     forward calls, and differentiates like them."""
     flat = []
     for rz, kw in zip(rasterizers, inputs):
