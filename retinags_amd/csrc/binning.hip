@@ -439,7 +439,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 			const uint32_t step = (hi - lo + 63u) / 64u;
 			const uint32_t probe = lo + (uint32_t)lane * step;
 			const bool below = probe < hi && offsets[probe] <= start;
-			const uint32_t c = (uint32_t)__popcll(__ballot(below));  // the predicate is monotone: the first c probes hold
+			const uint32_t c = (uint32_t)__popcll(lanes_where(below));  // the predicate is monotone: the first c probes hold
 			if (c == 0u) {
 				hi = lo;
 			} else {
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 				if (bits <= 2) {
 					// a digit of one or two bits: every lane would add to one of a few words, one after the other
 					for (uint32_t v = 0; v < (1u << bits); v++) {
-						const uint32_t c = (uint32_t)__popcll(__ballot(have && d == v));
+						const uint32_t c = (uint32_t)__popcll(lanes_where(have && d == v));
 						if (lane == 0 && c != 0u)
 							atomicAdd(&s_digits[256 * p + v], c);
 					}
@@ -695,7 +695,7 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 					// a digit of one or two bits: every lane would add to one of a few words, one after the
 					// other; count the lanes of each value instead
 					for (uint32_t v = 0; v < (1u << bits); v++) {
-						const uint32_t c = (uint32_t)__popcll(__ballot(d == v));
+						const uint32_t c = (uint32_t)__popcll(lanes_where(d == v));
 						if ((threadIdx.x & 63) == 0 && c != 0u)
 							atomicAdd(&s_hist[p][v], c);
 					}
@@ -781,7 +781,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 #pragma unroll
 		for (int b = 0; b < 8; b++) {
 			const bool bit = (d >> b) & 1u;
-			const uint64_t vote = __ballot(bit);
+			const uint64_t vote = lanes_where(bit);
 			same &= bit ? vote : ~vote;
 		}
 		const uint32_t below = (uint32_t)__popcll(same & lanes_below);

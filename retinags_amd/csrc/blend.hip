@@ -254,7 +254,6 @@ __global__ __launch_bounds__(kFileBlock) void strip_file_place_kernel(BlendBatch
 // ---- forward (K/cuda_rasterizer_hgs/forward.cu:263-405) ---------------------------------------
 
 struct ForwardPixel {
-	bool done;
 	float T, C0, C1, C2, weight, D;
 	uint32_t last_contributor;
 	uint32_t last_filed;  // like last_contributor, but counted in entries filed for the strip
@@ -272,20 +271,23 @@ struct ForwardStage {  // one per workgroup (a single wavefront)
 
 // `first` is the number of entries filed for the strip ahead of the chunk; `slot` is the packed slot in the
 // pixel's half.
-__device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, float power, const float4 g,
+// `done` holds a bit per pixel (lane) that takes no further entries: kept as a lane mask in scalar registers,
+// so that "a candidate that is not done" is two scalar instructions and not a flag byte per lane to test and set.
+__device__ __forceinline__ void forward_visit(ForwardPixel& p, uint64_t& done, uint64_t candidates, float power, const float4 g,
                                               const float4 co, const ForwardStage& st, int half, int slot, uint32_t first,
                                               const PixelRay& ray, const BoxFrame& box)
 {
-	candidate = candidate && !p.done;
-	if (__ballot(candidate) == 0ull)
+	const uint64_t taking = candidates & ~done;
+	if (taking == 0ull)
 		return;
-	if (candidate) {
+	bool finished = false;
+	if (__builtin_amdgcn_inverse_ballot_w64(taking)) {
 		const float clip_w = g.w;  // NaN: the whole strip is inside the box
 		const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
 		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, box))) {
 			const float test_T = p.T * (1 - alpha);
 			if (test_T < 0.0001f) {
-				p.done = true;
+				finished = true;
 			} else {
 				const uint32_t entry = st.entry[half][slot];
 				const float4 cd = st.cd[entry];
@@ -303,6 +305,7 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, bool candidate, f
 			}
 		}
 	}
+	done |= lanes_where(finished);
 }
 
 // Number of set bits of a ballot below the calling lane.
@@ -339,8 +342,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
 	const BoxFrame box = load_box_frame(a);
 
-	ForwardPixel p = {!inside, 1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u, 0u};
-	uint64_t live = __ballot(!p.done);
+	ForwardPixel p = {1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u, 0u};
+	uint64_t done = lanes_where(!inside);
+	uint64_t live = ~done;
 	// the entries filed for this strip, in list order: list position, bit 31 = strip inside the box
 	const uint32_t filed = a.strip_total[strip_id];
 	// A long list is a long chain of dependent steps: its wavefront goes first where it shares a SIMD with
@@ -389,7 +393,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 				left = reaches_columns(dxa, reach);
 				right = reaches_columns(dxa - 8.f, reach);
 			}
-			const uint64_t in_left = __ballot(left), in_right = __ballot(right);
+			const uint64_t in_left = lanes_where(left), in_right = lanes_where(right);
 			const int n_left = __popcll(in_left), n_right = __popcll(in_right);
 			const int steps = max(n_left, n_right), padded = (steps + 3) & ~3;
 			if (lane < count) {
@@ -437,16 +441,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 				float2 d;
 				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
 				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
-				// written with negations so that a NaN exponent is kept, as in the exact loop
-				const bool q0 = !(w0 > 0.0f) && !(w0 < g0.z), q1 = !(w1 > 0.0f) && !(w1 < g1.z),
-				           q2 = !(w2 > 0.0f) && !(w2 < g2.z), q3 = !(w3 > 0.0f) && !(w3 < g3.z);
-				if (__ballot((q0 | q1 | q2 | q3) && !p.done) == 0ull)
+				// written with negations so that a NaN exponent is kept, as in the exact loop; each mask from single
+				// comparisons (a comparison's result is the mask; that of a combined flag is formed through a register)
+				const uint64_t q0 = lanes_where(!(w0 > 0.0f)) & lanes_where(!(w0 < g0.z)),
+				               q1 = lanes_where(!(w1 > 0.0f)) & lanes_where(!(w1 < g1.z)),
+				               q2 = lanes_where(!(w2 > 0.0f)) & lanes_where(!(w2 < g2.z)),
+				               q3 = lanes_where(!(w3 > 0.0f)) & lanes_where(!(w3 < g3.z));
+				if (((q0 | q1 | q2 | q3) & ~done) == 0ull)
 					continue;
-				forward_visit(p, q0, w0, g0, c0, st, half, k, first, ray, box);
-				forward_visit(p, q1, w1, g1, c1, st, half, k + 1, first, ray, box);
-				forward_visit(p, q2, w2, g2, c2, st, half, k + 2, first, ray, box);
-				forward_visit(p, q3, w3, g3, c3, st, half, k + 3, first, ray, box);
-				live = __ballot(!p.done);
+				forward_visit(p, done, q0, w0, g0, c0, st, half, k, first, ray, box);
+				forward_visit(p, done, q1, w1, g1, c1, st, half, k + 1, first, ray, box);
+				forward_visit(p, done, q2, w2, g2, c2, st, half, k + 2, first, ray, box);
+				forward_visit(p, done, q3, w3, g3, c3, st, half, k + 3, first, ray, box);
+				live = ~done;
 			}
 			__builtin_amdgcn_wave_barrier();
 		}
@@ -676,7 +683,7 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
                                                const float4 co, BackwardStage& st, int slot, int& rows, uint64_t& row_slots,
                                                const StripFrame& f, const PixelRay& ray, const BlendArgs& a, int lane)
 {
-	if (__ballot(candidate) == 0ull)
+	if (lanes_where(candidate) == 0ull)
 		return;
 	float u = 0.f, aT = 0.f;
 	bool valid = false;
@@ -716,7 +723,8 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 			u = G * dL_dopa;
 		}
 	}
-	if (__ballot(valid) == 0ull)
+	// (a lane that took part has a weight alpha T > 0, or a NaN; asked of the weight, the mask comes from one comparison)
+	if (lanes_where(!(aT <= 0.f)) == 0ull)
 		return;
 	st.u_at[rows * kRowStride + row_column(lane)] = float2{u, aT};
 	row_slots |= (uint64_t)slot << (8 * rows);

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<Preproces
 
 	// the rendered Gaussians of the wavefront, listed in lane order
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	const uint64_t seen = __ballot(rendered);
+	const uint64_t seen = lanes_where(rendered);
 	const int n_seen = __popcll(seen);
 	const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(seen >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)seen, 0u));
 	float4* parked = s_rows[wave];
@@ -478,7 +478,7 @@ __global__ __launch_bounds__(128) void preprocess_backward_kernel(Batch<Preproce
 			const int needed_pieces = (needed + 3) / 4;
 			float4* parked = s_rows[wave];
 			uint8_t* listed = s_listed[wave];
-			const uint64_t seen = __ballot(rendered);
+			const uint64_t seen = lanes_where(rendered);
 			const int n_seen = __popcll(seen);
 			const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(seen >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)seen, 0u));
 			const size_t wave_first = i - (size_t)lane;

@@ -135,6 +135,14 @@ __device__ __forceinline__ float dpp_shift_add(float v)
 }
 
 // Sum over the 64 lanes; the total is valid in lane 63 only.
+// The lanes for which `b` holds, as a mask.  (HIP's __ballot takes an int: a flag first becomes 0 or 1 in a vector
+// register and is then compared with 0 again, two vector instructions per ballot; a comparison's result already is
+// the mask.)
+__device__ __forceinline__ uint64_t lanes_where(bool b)
+{
+	return __builtin_amdgcn_ballot_w64(b);
+}
+
 __device__ __forceinline__ float wave_sum_to_lane63(float v)
 {
 	v = dpp_shift_add<0x111, 0xF, 0xF>(v);  // row_shr:1
