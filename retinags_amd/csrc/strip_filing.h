@@ -78,7 +78,7 @@ __device__ __forceinline__ float2 strip_rows_ndc(int tile_y, int strip, int H)
 // coordinates, p_k = A_k nx + B_k ny + C_k per world coordinate k, so its range over a strip is the
 // sum of the ranges of the two terms; the box tolerance is taken from the magnitudes of the terms, not
 // of the result, so that it also covers the rounding of this regrouped evaluation when the terms
-// cancel.  The edge minima of the quadratic form use the reciprocals of a and c.
+// cancel.  The rows an ellipse reaches are computed with the reciprocals of a and c.
 struct StripTests {
 	float gx, gy, hx, hy;
 	float a, b, c, limit;   // conic; -2 floor
@@ -128,7 +128,6 @@ __device__ __forceinline__ uint32_t strips_filed_for(const StripTests& t, float 
 	const float a = t.a, b = t.b, c = t.c;
 	const bool ellipse = (t.flags & 1u) != 0u;
 	const float dxl = t.gx - (x0 + 15.f), dxh = t.gx - x0;
-	const bool x_within = !(dxl > 0.f) && !(dxh < 0.f);
 
 	// range of the ray sample's world coordinates over the tile's columns, per coordinate
 	float xlo[3], xhi[3];
@@ -155,6 +154,31 @@ __device__ __forceinline__ uint32_t strips_filed_for(const StripTests& t, float 
 	if (tile_outside)
 		return 0u;
 
+	// The rows the ellipse q(d) = a dx^2 + 2 b dx dy + c dy^2 <= limit reaches over the tile's 16 columns, once for the four
+	// strips (d = centre - pixel, so dx runs over [dxl, dxh]).  For a given dx the ellipse holds the dy between
+	// (-b dx -+ sqrt(c limit - det dx^2)) / c; the upper end is concave in dx and the lower convex, so over an interval
+	// of dx each is extreme at the ellipse's own extreme point (dy = +-Y at dx = -+b Y / a, Y = sqrt(a limit / det)) if
+	// that lies inside the interval, at one of its ends otherwise.  The limit gets room for the rounding
+	// of q (relative to its largest terms over the tile), and the rows a margin of a hundredth of a pixel.
+	float dy_low = -INFINITY, dy_high = INFINITY;
+	if (ellipse) {
+		const float dy_first = t.gy - y0, dy_last = t.gy - (y0 + 15.f);
+		const float largest = a * fmaxf(dxl * dxl, dxh * dxh) + c * fmaxf(dy_first * dy_first, dy_last * dy_last);
+		const float limit = t.limit + (1e-3f + 1e-4f * t.limit + 1e-5f * largest);
+		const float det = a * c - b * b;
+		const float rdet = 1.f / det;
+		const float X = sqrtf(c * limit * rdet), Y = sqrtf(a * limit * rdet);
+		const float dl = fmaxf(dxl, -X), dh = fminf(dxh, X);
+		if (dl > dh)
+			return 0u;  // the columns lie beside the ellipse
+		const float sl = sqrtf(fmaxf(c * limit - det * dl * dl, 0.f)), sh = sqrtf(fmaxf(c * limit - det * dh * dh, 0.f));
+		const float at_top = -b * Y * t.ra;  // dx of the ellipse's highest dy; that of its lowest is -at_top
+		const float top = fmaxf((-b * dl + sl) * t.rc, (-b * dh + sh) * t.rc);
+		const float bottom = fminf((-b * dl - sl) * t.rc, (-b * dh - sh) * t.rc);
+		const float margin = 1e-2f + 1e-5f * Y;
+		dy_high = ((!(at_top < dl) && !(at_top > dh)) ? Y : top) + margin;
+		dy_low = ((!(-at_top < dl) && !(-at_top > dh)) ? -Y : bottom) - margin;
+	}
 	uint32_t bits = 0;
 #pragma unroll
 	for (int s = 0; s < 4; s++) {
@@ -162,28 +186,8 @@ __device__ __forceinline__ uint32_t strips_filed_for(const StripTests& t, float 
 		if ((t.gy + t.hy < ya) || (t.gy - t.hy > ya + 3.f))
 			continue;
 		const float dyl = t.gy - (ya + 3.f), dyh = t.gy - ya;
-		if (ellipse && !(x_within && !(dyl > 0.f) && !(dyh < 0.f))) {
-			// the smallest value over the strip's rectangle of q(d) = a dx^2 + 2 b dx dy + c dy^2 (d = centre - pixel):
-			// with the centre outside, the minimum of the convex q lies on one of the four edges, where it is a
-			// clamped parabola vertex; compared with the -2 floor that power = -q / 2 >= floor allows, with room
-			// for the rounding of q (relative to its largest terms)
-			float qmin = INFINITY;
-#pragma unroll
-			for (int edge = 0; edge < 2; edge++) {
-				const float dy = edge ? dyh : dyl;
-				const float dx = fminf(dxh, fmaxf(dxl, -b * dy * t.ra));
-				qmin = fminf(qmin, (a * dx + 2.f * b * dy) * dx + c * dy * dy);
-			}
-#pragma unroll
-			for (int edge = 0; edge < 2; edge++) {
-				const float dx = edge ? dxh : dxl;
-				const float dy = fminf(dyh, fmaxf(dyl, -b * dx * t.rc));
-				qmin = fminf(qmin, (c * dy + 2.f * b * dx) * dy + a * dx * dx);
-			}
-			const float largest = a * fmaxf(dxl * dxl, dxh * dxh) + c * fmaxf(dyl * dyl, dyh * dyh);
-			if (qmin > t.limit + (1e-3f + 1e-4f * t.limit + 1e-5f * largest))
-				continue;
-		}
+		if ((dyh < dy_low) || (dyl > dy_high))
+			continue;
 		bool inside = true, outside = false;
 		if (!tile_inside) {
 #pragma unroll
