@@ -74,6 +74,10 @@ class _CompositePartialImages(torch.autograd.Function):
                 ptr(g_alpha), ptr_table(d_images), ptr_table(d_depths), ptr_table(d_alphas),
                 C.c_void_p(torch.cuda.current_stream(device).cuda_stream)))
         # The reference's background is a constant (or a fresh random tensor); it gets no gradient.
+        if g_depth is None:
+            # no gradient for the composited depth: none for the layers' depths either (their planes of the blocks hold
+            # the zeros the kernel wrote); told so, the rasterizer's backward leaves out the terms it would multiply
+            return (None, None, *d_images, *([None] * K), *d_alphas)
         return (None, None, *d_images, *d_depths, *d_alphas)
 
 

@@ -614,6 +614,9 @@ __device__ __forceinline__ float dpp_exchange_add(float v)
 // row of `sums`: eight neighbouring columns in one atomic instruction, the last two in a second.
 // `row_slots` holds, one byte per row, which staged entry of the current chunk the row belongs to: the entry's centre,
 // conic and Gaussian are read from where the chunk was staged (so the rows are flushed before the next chunk is).
+// kDepth: a gradient arrived for the depth image (without one, the usual case of a loss on the colour image alone, the
+// terms it multiplies are left out: the depth column of `sums` stays zero).
+template <bool kDepth>
 __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, uint64_t row_slots, const StripFrame& f,
                                            const BlendArgs& a, int lane)
 {
@@ -642,16 +645,17 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 		cr += tt * g.x;
 		cg += tt * g.y;
 		cb += tt * g.z;
-		cdp += tt * g.w;
+		if (kDepth)
+			cdp += tt * g.w;
 	}
 	// the two halves of the strip row first (dy is theirs in common), then the four strip rows
 	float w[7] = {s0, sx, sxx, cr, cg, cb, cdp};
 #pragma unroll
-	for (int q = 0; q < 7; q++)
+	for (int q = 0; q < (kDepth ? 7 : 6); q++)
 		w[q] = dpp_exchange_add<0xB1>(w[q]);  // quad_perm:[1,0,3,2]
 	float v[10] = {w[0], w[1], dy * w[0], w[2], dy * w[1], dy * dy * w[0], w[3], w[4], w[5], w[6]};
 #pragma unroll
-	for (int q = 0; q < 10; q++) {
+	for (int q = 0; q < (kDepth ? 10 : 9); q++) {
 		v[q] = dpp_exchange_add<0x4E>(v[q]);   // quad_perm:[2,3,0,1]
 		v[q] = dpp_exchange_add<0x141>(v[q]);  // row_half_mirror: the other quad of the eight
 	}
@@ -679,6 +683,7 @@ __device__ __forceinline__ void update_behind(float& behind, float keep, float a
 }
 
 // Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
+template <bool kDepth>
 __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
                                                const float4 co, BackwardStage& st, int slot, int& rows, uint64_t& row_slots,
                                                const StripFrame& f, const PixelRay& ray, const BlendArgs& a, int lane)
@@ -711,13 +716,15 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 			dL_dopa += (cd.x - p.behind_r) * p.g_r;
 			dL_dopa += (cd.y - p.behind_g) * p.g_g;
 			dL_dopa += (cd.z - p.behind_b) * p.g_b;
-			dL_dopa += (cd.w - p.behind_depth) * p.g_depth;
+			if (kDepth)
+				dL_dopa += (cd.w - p.behind_depth) * p.g_depth;
 			dL_dopa += (1 - p.behind_alpha) * p.g_alpha;
 			dL_dopa *= p.T;
 			update_behind(p.behind_r, keep, alpha * cd.x);
 			update_behind(p.behind_g, keep, alpha * cd.y);
 			update_behind(p.behind_b, keep, alpha * cd.z);
-			update_behind(p.behind_depth, keep, alpha * cd.w);
+			if (kDepth)
+				update_behind(p.behind_depth, keep, alpha * cd.w);
 			update_behind(p.behind_alpha, keep, alpha);
 			dL_dopa += (-p.T_final * inv_one_minus_alpha) * p.bg_dot_dpixel;
 			u = G * dL_dopa;
@@ -730,7 +737,7 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	row_slots |= (uint64_t)slot << (8 * rows);
 	rows++;
 	if (rows == kRows) {
-		flush_rows(st, kRows, row_slots, f, a, lane);
+		flush_rows<kDepth>(st, kRows, row_slots, f, a, lane);
 		rows = 0;
 		row_slots = 0ull;
 	}
@@ -738,6 +745,7 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 
 // 128 registers and under 10 KB of LDS: four wavefronts per SIMD (three, as the compiler chooses by itself, were
 // measured 19 % slower; five spill)
+template <bool kDepth>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void blend_backward_kernel(BlendBatch batch)
 {
 	__shared__ BackwardStage s_stage;
@@ -835,18 +843,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 			// ballot): nearly every walked entry has some, so a test for the four together would save little, and
 			// four sets of flags kept alive across the visits are packed into a byte mask by the compiler, a dozen
 			// vector instructions per step.
-			backward_visit(p, (p0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z), w0, g0, c0, st, k, rows, row_slots, frame,
+			backward_visit<kDepth>(p, (p0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z), w0, g0, c0, st, k, rows, row_slots, frame,
 			               ray, a, lane);
-			backward_visit(p, (p1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z), w1, g1, c1, st, k + 1, rows, row_slots,
+			backward_visit<kDepth>(p, (p1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z), w1, g1, c1, st, k + 1, rows, row_slots,
 			               frame, ray, a, lane);
-			backward_visit(p, (p2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z), w2, g2, c2, st, k + 2, rows, row_slots,
+			backward_visit<kDepth>(p, (p2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z), w2, g2, c2, st, k + 2, rows, row_slots,
 			               frame, ray, a, lane);
-			backward_visit(p, (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z), w3, g3, c3, st, k + 3, rows, row_slots,
+			backward_visit<kDepth>(p, (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z), w3, g3, c3, st, k + 3, rows, row_slots,
 			               frame, ray, a, lane);
 		}
 		// the rows point into this chunk's staged entries: they go before the next chunk takes their place
 		if (rows > 0) {
-			flush_rows(st, rows, row_slots, frame, a, lane);
+			flush_rows<kDepth>(st, rows, row_slots, frame, a, lane);
 			rows = 0;
 			row_slots = 0ull;
 		}
@@ -975,7 +983,13 @@ void launch_blend_backward(const BlendArgs* jobs, int count, hipStream_t s)
 		batch.count = count - at < kMaxBlendBatch ? count - at : kMaxBlendBatch;
 		for (int k = 0; k < batch.count; k++)
 			batch.job[k] = jobs[at + k];
-		hipLaunchKernelGGL(blend_backward_kernel, dim3(strips * (unsigned)batch.count), dim3(64), 0, s, batch);
+		bool depth = false;  // does any job of the batch bring a gradient of the depth image?
+		for (int k = 0; k < batch.count; k++)
+			depth = depth || batch.job[k].dL_dpix_depth != nullptr;
+		if (depth)
+			hipLaunchKernelGGL(blend_backward_kernel<true>, dim3(strips * (unsigned)batch.count), dim3(64), 0, s, batch);
+		else
+			hipLaunchKernelGGL(blend_backward_kernel<false>, dim3(strips * (unsigned)batch.count), dim3(64), 0, s, batch);
 	}
 }
 
