@@ -106,6 +106,13 @@ def parse():
                     help="one rasterizer call per submodel, as the reference issues them (default: the submodels of a frame "
                          "go through one call that blends them in one launch per direction)")
     ap.add_argument("--no-asides", action="store_true", help="skip the stages beside the metric (sharing, loss, optimiser)")
+    ap.add_argument("--whole-iteration", action="store_true",
+                    help="also time one whole training iteration from the stored parameters (activation, sharing, render, loss, "
+                         "backward, Adam); not part of the metric")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip fwd+bwd at C0, C2 and C3 and the one-call-per-submodel figure in the default run")
+    ap.add_argument("--no-verify", action="store_true",
+                    help="skip the check of the timed path (all submodels through one call) against one call per submodel")
     return ap.parse_args()
 
 
@@ -127,26 +134,45 @@ def main():
         sys.exit(2)
     ensure_built()
     default_run = (args.config == "C1" and not args.forward_only and args.shrink == 1.0 and args.resolution_scale == 1.0)
-    line = measure(args, args.config, args.forward_only, asides=not args.no_asides, cpu=not args.no_cpu_baseline)
+    line = measure(args, args.config, args.forward_only, asides=not args.no_asides, cpu=not args.no_cpu_baseline,
+                   apart_too=default_run and not args.no_other_configs)
     if default_run and not args.no_render_metric:
         # the second half of the metric: render only (every related submodel's forward and the compositing)
         for name in ("C3", "C4"):
             try:
-                sub = measure(args, name, True, asides=False, cpu=False)
+                sub = measure(args, name, True, asides=False, cpu=not args.no_cpu_baseline)
                 line[f"render_ms_per_frame_{name.lower()}"] = {
                     "value": sub["ms_per_step"], "unit": "ms/frame", "ms_per_frame_one_stream": sub["ms_per_step_one_stream"],
+                    "verified": sub["verified"], "verification": sub["verification"],
                     "workload": sub["config"]["workload"], "instances": sub["config"]["instances"],
                     "visible": sub["config"]["visible"], "setup_s": sub["config"]["setup_s"],
                     "peak_device_memory_GB": sub["config"]["peak_device_memory_GB"], "roofline": sub["roofline"],
+                    "cpu_baseline": sub["cpu_baseline"],
                     "blend_forward": sub["stages"].get("blend_forward"), "stages_ms": {k: v["ms_per_step"] for k, v in sub["stages"].items()},
                     "blend_work": sub["blend_work"]}
             except Exception as ex:   # the first half of the metric must not be lost with the second
                 torch.cuda.synchronize()
                 line[f"render_ms_per_frame_{name.lower()}"] = {"error": f"{type(ex).__name__}: {ex}"}
+    if default_run and not args.no_other_configs:
+        # forward + backward at the other configurations the reference's table lists (same step as `value`)
+        for name in ("C0", "C2", "C3"):
+            try:
+                sub = measure(args, name, False, asides=False, cpu=False)
+                line[f"fwd_bwd_{name.lower()}"] = {
+                    "value": sub["value"], "unit": "it/s", "ms_per_step": sub["ms_per_step"], "steps": sub["steps"],
+                    "verified": sub["verified"], "verification": sub["verification"],
+                    "workload": sub["config"]["workload"], "instances": sub["config"]["instances"],
+                    "visible": sub["config"]["visible"], "sort_passes": sub["config"]["sort_passes"],
+                    "peak_device_memory_GB": sub["config"]["peak_device_memory_GB"], "roofline": sub["roofline"],
+                    "stages_ms": {k: v["ms_per_step"] for k, v in sub["stages"].items()},
+                    "gpu_kernel_ms_per_step": sub["gpu_kernel_ms_per_step"], "blend_work": sub["blend_work"]}
+            except Exception as ex:
+                torch.cuda.synchronize()
+                line[f"fwd_bwd_{name.lower()}"] = {"error": f"{type(ex).__name__}: {ex}"}
     print(json.dumps(line))
 
 
-def measure(args, config, forward_only, asides, cpu):
+def measure(args, config, forward_only, asides, cpu, apart_too=False):
     """Times `config` and returns the JSON line's dictionary."""
     from retinags_amd import _capi, rasterizer as R
     from retinags_amd.harness import scenes, partition, pipeline
@@ -194,7 +220,7 @@ def measure(args, config, forward_only, asides, cpu):
     bounds = None   # room for each submodel's instances; None: wait for every count
     together = not args.apart and args.instance_room <= 0 and not args.host_threads
 
-    def step(streams=streams, host_threads=args.host_threads):
+    def step(streams=streams, host_threads=args.host_threads, together=together):
         nonlocal bounds
         while True:
             for s in subs:
@@ -233,7 +259,8 @@ def measure(args, config, forward_only, asides, cpu):
         t2 = time.perf_counter()   # everything is queued; what is left is the device catching up
         torch.cuda.synchronize()
         t3 = time.perf_counter()
-        host_ms["one_stream" if kw.get("streams", streams) is None else "streams"] = (t2 - t1) * 1e3 / args.steps
+        host_ms["one_call_per_submodel" if kw.get("together", together) is False and together else
+                "one_stream" if kw.get("streams", streams) is None else "streams"] = (t2 - t1) * 1e3 / args.steps
         return t3 - t1
 
     elapsed = timed()
@@ -241,6 +268,12 @@ def measure(args, config, forward_only, asides, cpu):
     # the same steps with every submodel on the caller's stream, one after the other
     elapsed_one = timed(streams=None) if streams is not None else elapsed
     peak_gb = torch.cuda.max_memory_allocated(dev) / 1e9   # inputs, workspaces and gradients of the timed steps
+    # the same steps with one rasterizer call per submodel, as the reference issues them (result_aggregator.py:22-38)
+    elapsed_apart = timed(together=False) if (apart_too and together) else None
+
+    # ---- the timed path against one call per submodel, on this very workload
+    verification = (verify_timed_path(pipeline, R, _capi, cam_d, cam, subs, rel, bg, upstream, do_backward, streams)
+                    if (together and not args.no_verify) else None)
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -316,6 +349,17 @@ def measure(args, config, forward_only, asides, cpu):
         "composite_backward": (40.0 * K + 20.0) * N,
     }
     alg_flops = {"blend_forward": flops_fwd, "blend_backward": flops_bwd}
+    # Where this design's bytes differ from those of the reference's design, both are carried.  The reference's backward
+    # preprocess writes the rendered rows only, into arrays its caller has cleared (4 P + 559 P_vis, or with that clearing
+    # 304 P more); here every row of the dense outputs is written once, zeros included.  The reference sorts 12-byte pairs
+    # on (tile << 32 | depth) in ceil((32 + bits) / 8) passes after one read of the keys (R (8 + 24 p)); here the instances
+    # are emitted in depth order and sorted on the tile alone, 8-byte pairs, ceil(bits / 8) passes.
+    ref_passes = (32 + int(_capi.lib.rgs_get_higher_msb(T)) + 7) // 8
+    reference_design_bytes = {
+        "preprocess_backward": {"rendered_rows_only": 4.0 * P_tot + 559.0 * P_vis,
+                                "with_the_clearing_of_the_outputs": (4.0 + 304.0) * P_tot + 559.0 * P_vis},
+        "sort_onesweep": {f"one_sort_of_12_byte_pairs_in_{ref_passes}_passes": R_tot * (8.0 + 24.0 * ref_passes)},
+    }
 
     stages = {}
     for name, (ms, launches) in stage_ms.items():
@@ -326,6 +370,11 @@ def measure(args, config, forward_only, asides, cpu):
             entry["bound"] = "hbm"
             entry["achieved_GBps"] = round(alg_bytes[name] / (per_step * 1e-3) / 1e9, 2)
             entry["frac"] = round(entry["achieved_GBps"] / HBM_PEAK_GBS, 4)
+        if name in reference_design_bytes and per_step > 0:
+            # the same stage time priced with the bytes of the reference's design (an equivalent rate, not traffic)
+            entry["by_reference_design_bytes"] = {
+                k: {"bytes": v, "equivalent_GBps": round(v / (per_step * 1e-3) / 1e9, 2),
+                    "frac": round(v / (per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)} for k, v in reference_design_bytes[name].items()}
         if name in alg_flops and per_step > 0:
             entry["bound"] = "valu"
             entry["achieved_TFLOPs"] = round(alg_flops[name] / (per_step * 1e-3) / 1e12, 3)
@@ -389,12 +438,15 @@ def measure(args, config, forward_only, asides, cpu):
 
     # ---- everything together: one training iteration for this camera
     whole = (aside(lambda: whole_iteration(scene, part, cam_d, rel, bg, streams, dev, args.steps))
-             if (part is not None and do_backward and asides) else None)
+             if (part is not None and do_backward and asides and args.whole_iteration) else None)
 
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
     cpu_line = None
     if cpu and scene is not None:
         cpu_line = cpu_baseline(scene, members, part, cam, rel, related, upstream.cpu().numpy(), do_backward, args)
+    elif cpu and not do_backward:
+        # a scene that lives on the device only (C3, C4): the render on the CPU checker, one submodel copied to the host at a time
+        cpu_line = cpu_render_baseline(subs, cam, rel, related, args)
 
     return {
         "metric": "fwd+bwd iterations/s, 5.6M Gaussians, 1600x1036, 4 composited submodels"
@@ -405,6 +457,11 @@ def measure(args, config, forward_only, asides, cpu):
         # every submodel on one stream, rendered strictly one after the other (`value` offers the independent
         # submodels to the GPU on several HIP streams; no work differs)
         "value_one_stream": round(args.steps / elapsed_one, 4), "ms_per_step_one_stream": round(elapsed_one * 1e3 / args.steps, 3),
+        # one rasterizer call per submodel, as the reference issues them (the default batches the submodels of a frame)
+        "value_apart": round(args.steps / elapsed_apart, 4) if elapsed_apart else None,
+        "ms_per_step_apart": round(elapsed_apart * 1e3 / args.steps, 3) if elapsed_apart else None,
+        # the timed calls (all submodels through one call per stage) checked against one call per submodel on this workload
+        "verified": verification["verified"] if verification else None, "verification": verification,
         # how long the host takes to queue a step (the forward's waits for the instance counts included)
         "host_ms_per_step": {k: round(v, 3) for k, v in host_ms.items()},
         "config": {"workload": f"{config}: {cfg['n']} Gaussians, {W}x{H}, bvh_depth={depth} "
@@ -653,6 +710,106 @@ def training_stages(subs, H, W, dev, repeats):
             out[name]["achieved_GBps"] = round(alg[name] / (per * 1e-3) / 1e9, 1)
             out[name]["frac"] = round(out[name]["achieved_GBps"] / HBM_PEAK_GBS, 4)
     return out
+
+
+def verify_timed_path(pipeline, R, _capi, cam_d, cam, subs, rel, bg, upstream, do_backward, streams):
+    """One frame through the calls that were timed (every submodel of the frame in one call per stage:
+    rgs_frame_forward_geom / _raster / rgs_frame_backward) against one call per submodel (rgs_forward_geom /
+    rgs_forward_raster / rgs_backward) on the same inputs: instance counts, radii, images and n_contrib must agree bit
+    for bit, the composited image too, and every gradient to 1e-5 relative L2 (the same atomic sums in another order)."""
+    H, W = cam.image_height, cam.image_width
+    related = [m for m in range(len(subs)) if rel[m] >= 0]
+    for s in subs:
+        for p in s.parameters():
+            p.grad = None
+    fields = ("means3D", "opacity", "scales", "rotations", "shs")
+    grad_ctx = torch.enable_grad() if do_backward else torch.no_grad()
+    with grad_ctx:
+        frame = pipeline.render_frame(cam_d, subs, rel, bg, streams=streams, together=True, keep_workspaces=True)
+        if do_backward:
+            torch.autograd.backward([frame["render"]], [upstream])
+    frame_grads = {m: {f: getattr(subs[m], f).grad for f in fields} for m in related} if do_backward else None
+    for s in subs:
+        for p in s.parameters():
+            p.grad = None
+    im = _capi.image_layout(W, H)
+    e = torch.Tensor([])
+    ok, mismatches, worst = True, [], 0.0
+    with torch.no_grad():
+        for m in related:
+            s = subs[m]
+            outs = R._rasterize_forward(bg, s.means3D.detach(), e, s.opacity.detach(), s.scales.detach(), s.rotations.detach(),
+                                        1.0, e, cam_d.world_view_transform, cam_d.full_proj_transform, cam_d.projection_matrix_inv,
+                                        s.range_low, s.range_up, cam.tanfovx, cam.tanfovy, H, W, s.shs.detach(), 3,
+                                        cam_d.camera_center, False, False)
+            Rn, geom, binning, img = frame["workspaces"][m]
+            layer = frame["partial"][m]
+            n0, n1 = im["n_contrib"], im["n_contrib"] + 4 * W * H
+            same = (outs[0] == Rn and torch.equal(outs[4], layer["radii"]) and torch.equal(outs[1], layer["render"].detach())
+                    and torch.equal(outs[2], layer["depth"].detach()) and torch.equal(outs[3], layer["alpha"].detach())
+                    and torch.equal(outs[7][n0:n1], img[n0:n1]))
+            if not same:
+                ok = False
+                mismatches.append(int(m))
+            del outs
+    if do_backward:
+        with torch.enable_grad():
+            again = pipeline.render_frame(cam_d, subs, rel, bg, together=False)
+            ok = ok and torch.equal(again["render"], frame["render"])
+            torch.autograd.backward([again["render"]], [upstream])
+        for m in related:
+            for f in fields:
+                a, b = frame_grads[m][f], getattr(subs[m], f).grad
+                err = float((a - b).double().norm() / b.double().norm().clamp_min(1e-300))
+                worst = max(worst, err)
+        ok = ok and worst <= 1e-5
+        del again
+        for s in subs:
+            for p in s.parameters():
+                p.grad = None
+    return {"verified": bool(ok), "against": "one rgs_forward_geom / rgs_forward_raster" + (" / rgs_backward" if do_backward else "")
+            + " call per submodel", "bit_for_bit": "instance counts, radii, colour, depth, alpha, n_contrib of every submodel"
+            + (", composited image" if do_backward else ""), "submodels": len(related), "submodels_that_differ": mismatches,
+            "worst_gradient_rel_l2": worst if do_backward else None}
+
+
+def cpu_render_baseline(subs, cam, rel, related, args):
+    """The render (every related submodel's forward, then the compositing) on the CPU checker for a scene that lives
+    on the device: one submodel is copied to the host at a time.  Bounded to about 25 s of wall time: if the submodels do
+    not all fit, the figure is extrapolated from the share of the Gaussians that did, and says so."""
+    from oracle import rgs_oracle as orc
+    np32 = lambda t: np.ascontiguousarray(t.detach().cpu().numpy().astype(np.float32))
+    threads = args.cpu_threads or min(16, orc.max_threads(), os.cpu_count() or 1)
+    orc.set_threads(threads)
+    order = sorted(related, key=lambda m: rel[m])
+    total = sum(int(subs[m].means3D.shape[0]) for m in order)
+    spent, seen, states = 0.0, 0, []
+    try:
+        for m in order:
+            s = subs[m]
+            arrays = [np32(t) for t in (s.means3D, s.opacity, s.shs, s.scales, s.rotations)]
+            settings = orc.settings_from_camera(cam, s.range_low.cpu(), s.range_up.cpu(), torch.zeros(3))
+            t0 = time.perf_counter()
+            st = orc.forward(settings, arrays[0], arrays[1], shs=arrays[2], scales=arrays[3], rotations=arrays[4])
+            spent += time.perf_counter() - t0
+            states.append((st.color, st.depth, st.alpha))
+            seen += arrays[0].shape[0]
+            del arrays, st
+            if spent > 25.0:
+                break
+        t0 = time.perf_counter()
+        orc.composite_forward([c for c, _, _ in states], [d for _, d, _ in states], [a for _, _, a in states], np.zeros(3, np.float32))
+        spent += time.perf_counter() - t0
+    finally:
+        orc.set_threads(1)
+    whole = seen == total
+    seconds = spent if whole else spent * total / max(seen, 1)
+    return {"value": round(seconds * 1e3, 1), "unit": "ms/frame", "cores": threads, "kind": "port",
+            "extrapolated": not whole,
+            "sample": (f"the forward of {len(states)} of {len(order)} related submodels ({seen} of {total} Gaussians) and their "
+                       f"compositing, {spent:.1f} s wall, C checker with OpenMP"
+                       + ("" if whole else "; scaled by the share of the Gaussians")),
+            "host_cpus": os.cpu_count()}
 
 
 def cpu_baseline(scene, members, part, cam, rel, related, upstream, do_backward, args):

@@ -268,21 +268,25 @@ typedef struct rgs_frame_layer {
 	float* dL_dscale;
 	float* dL_drot;
 	int accum_zeroed;          /* as in rgs_backward: grad_accum arrives cleared */
-	void* stream;              /* NULL, or a second HIP stream for the backward: work that is bound by memory bandwidth (the
-	                              per-Gaussian backward of the layers whose blend is done) then runs on it beside the blend,
-	                              which is bound by instruction issue; the frame's stream waits for it */
+	void* stream;              /* NULL, or a second HIP stream for rgs_frame_backward (the forward calls ignore it): work that is
+	                              bound by memory bandwidth (the per-Gaussian backward of the layers whose blend is done) then
+	                              runs on it beside the blend, which is bound by instruction issue; the frame's stream waits for it */
 } rgs_frame_layer;
-/* rgs_forward_geom for every layer (P > 0 each): every geometry stage is queued (on the layer's stream) before
- * the host waits for the first instance count; returns when all counts have arrived in counts_pinned[0..K)
- * (pinned host memory), which is also where the layers' R for the next call is read from. */
+/* rgs_forward_geom for every layer (P > 0 each): every geometry stage of every layer is queued on `stream` (one
+ * launch per stage for all layers; rgs_frame_layer.stream is not looked at by the forward) before the host waits for
+ * the instance counts; returns when all counts have arrived in counts_pinned[0..K) (pinned host memory), which is
+ * also where the layers' R for the next call is read from. */
 int rgs_frame_forward_geom(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, uint32_t* counts_pinned,
                            void* stream, int debug);
-/* rgs_forward_raster for every layer (P > 0 each): per layer the key duplication, sort, ranges and strip
- * lists, then one blend launch for all.  `layers` and `view` are HOST structures. */
+/* rgs_forward_raster for every layer (P > 0 each): the key duplication, sort, ranges and strip lists, each one
+ * launch for all layers, then one blend launch for all, everything on `stream`.  `layers` and `view` are HOST
+ * structures. */
 int rgs_frame_forward_raster(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug);
 /* rgs_backward for every layer: the blend backward of all layers in one launch (two, one behind the other, when a
  * layer names a second stream, so that the first half's per-Gaussian backward runs beside the second half's blend),
- * then each layer's per-Gaussian backward. */
+ * then each layer's per-Gaussian backward.  Only the first stream among the layers' that differs from `stream` is
+ * used; `stream` waits for it before the call's work counts as done.  While rgs_stage_timing is on, everything runs
+ * on `stream`. */
 int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_view* view, void* stream, int debug);
 
 /* ---- measurement aids (no counterpart in the reference, which times whole iterations
@@ -292,7 +296,9 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
  * starts recording, rgs_stage_timing(0) stops.  rgs_stage_timing_read waits for the recorded
  * work, fills up to max_stages (name, total milliseconds, launches) triples, clears the record
  * and returns the number of stages (negative on error).  The names are static strings.
- * Recording is process-wide and not thread-safe; leave it off outside measurements. */
+ * Recording is process-wide and not thread-safe; leave it off outside measurements.  The time between two
+ * consecutive events is charged to the earlier one's stage, which takes a single stream: while recording is on,
+ * rgs_frame_backward does not use a second stream. */
 int rgs_stage_timing(int enable);
 int rgs_stage_timing_read(int max_stages, const char** names, float* total_ms, int* launches);
 
@@ -323,7 +329,8 @@ int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uin
                    int end_bit, void* temp, void* stream);
 
 /* Waits for `stream`, then returns non-zero (and clears the report) if a sort of an earlier call on
- * the current device gave up; see the note at the top. */
+ * the current device gave up; see the note at the top.  That includes rgs_sort_pairs_static, whose report is a word
+ * of device memory beside its scratch (read here with a 4-byte copy; nothing is allocated for it). */
 int rgs_sort_fault(void* stream);
 
 /* Test hook: the number of polls a look-back of the sorts allows before it gives up (0 restores

@@ -34,7 +34,7 @@ SOURCES = {
     "training.hip": [],
 }
 
-HEADERS = ["rgs_device.h", "rgs_kernels.h", os.path.join("..", "..", "include", "rgs.h")]
+HEADERS = ["rgs_device.h", "rgs_kernels.h", "strip_filing.h", "tile_order.h", os.path.join("..", "..", "include", "rgs.h")]
 
 
 def _hipcc() -> str:

@@ -18,6 +18,9 @@
 // for hipGetSymbolAddress; the address the kernels get is looked up once per device (static_sort_scratch).
 constexpr size_t kStaticSortWords = rgs::sort_temp_words_for(RGS_STATIC_SORT_MAX_PAIRS);
 static __device__ __align__(256) uint32_t scratch[kStaticSortWords];
+// Set (and left set until rgs_sort_fault has read it) when a sort of rgs_sort_pairs_static gave up: that entry point may
+// not allocate the pinned word the other sorts report through, so its report lives in device memory like its scratch.
+static __device__ __align__(256) uint32_t scratch_sort_gave_up[64];
 
 namespace {
 
@@ -100,6 +103,7 @@ constexpr int kMaxDevices = 64;
 std::mutex g_device_mutex;
 uint32_t* g_fault_word[kMaxDevices] = {};
 uint32_t* g_static_scratch[kMaxDevices] = {};
+uint32_t* g_static_gave_up[kMaxDevices] = {};
 
 int current_device()
 {
@@ -145,22 +149,52 @@ int take_sort_fault(const char* who)
 			return rc_;                            \
 	} while (0)
 
-// Device address of this device's copy of `scratch`, looked up once per device with that device current.
-int static_sort_scratch(uint32_t** out)
+// Device addresses of this device's copies of `scratch` and of its give-up word, looked up once per device with that
+// device current.
+int static_sort_scratch(uint32_t** out, uint32_t** gave_up)
 {
 	const int dev = current_device();
 	if (dev < 0)
 		return fail("rgs_sort_pairs_static: no current device");
 	std::lock_guard<std::mutex> lock(g_device_mutex);
-	if (!g_static_scratch[dev]) {
+	if (!g_static_scratch[dev] || !g_static_gave_up[dev]) {
 		void* p = nullptr;
-		const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-		if (e != hipSuccess || !p)
+		void* q = nullptr;
+		hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+		if (e == hipSuccess)
+			e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch_sort_gave_up));
+		if (e != hipSuccess || !p || !q)
 			return fail("rgs_sort_pairs_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
 		g_static_scratch[dev] = static_cast<uint32_t*>(p);
+		g_static_gave_up[dev] = static_cast<uint32_t*>(q);
 	}
 	*out = g_static_scratch[dev];
+	*gave_up = g_static_gave_up[dev];
 	return 0;
+}
+
+// Non-zero (with the error set) if a sort of rgs_sort_pairs_static on this device gave up; clears the report.  The
+// caller has waited for the stream that sort ran on.
+int take_static_sort_fault(const char* who)
+{
+	const int dev = current_device();
+	uint32_t* word = nullptr;
+	{
+		std::lock_guard<std::mutex> lock(g_device_mutex);
+		word = dev >= 0 ? g_static_gave_up[dev] : nullptr;
+	}
+	if (!word)
+		return 0;  // no such sort has run on this device
+	uint32_t seen = 0;
+	hipError_t e = hipMemcpy(&seen, word, sizeof(seen), hipMemcpyDeviceToHost);
+	if (e == hipSuccess && seen != 0u)
+		e = hipMemset(word, 0, sizeof(seen));
+	if (e != hipSuccess)
+		return fail("%s: reading the report of rgs_sort_pairs_static failed: %s", who, hipGetErrorString(e));
+	if (seen == 0u)
+		return 0;
+	return fail("%s: a radix sort of an earlier rgs_sort_pairs_static call on this device gave up waiting for a neighbouring "
+	            "workgroup; its output is not sorted and the call must be repeated", who);
 }
 
 constexpr size_t kAlign = 256;
@@ -983,7 +1017,9 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 	RGS_REQUIRE(K >= 1 && K <= RGS_MAX_FRAME_LAYERS && layers && view, "rgs_frame_backward: K = %d outside 1..%d, or null", K,
 	            RGS_MAX_FRAME_LAYERS);
 	const std::vector<hipStream_t> sides = side_streams(K, layers, s);
-	hipStream_t beside = sides.empty() ? s : sides[0];  // where the bandwidth-bound work goes
+	// where the bandwidth-bound work goes; the stage timing charges the time between consecutive events of one stream,
+	// so while it is on everything stays on the frame's stream
+	hipStream_t beside = (sides.empty() || g_timer.on) ? s : sides[0];
 	std::vector<rgs::BlendArgs> jobs;
 	std::vector<int> job_layer;
 	std::vector<rgs::PreprocessBackwardArgs> geometry((size_t)K);
@@ -1117,13 +1153,14 @@ size_t rgs_sort_temp_bytes(size_t n)
 	return 4 * rgs::sort_temp_words(n);
 }
 
+// fault: pinned host word (may be null); device_fault: a word of device memory (may be null).  A sort that gave up sets both.
 static int sort_pairs_u64(const char* who, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
-                          size_t n, int end_bit, uint32_t* temp, uint32_t* fault, hipStream_t s)
+                          size_t n, int end_bit, uint32_t* temp, uint32_t* fault, uint32_t* device_fault, hipStream_t s)
 {
 	const int debug = 0;
 	rgs::launch_sort_pairs(keys_in, keys_out, vals_in, vals_out, n, end_bit, temp, s);
 	RGS_STAGE("sort_pairs");
-	rgs::launch_report_sort_status(temp, fault, s);
+	rgs::launch_report_sort_status(temp, fault, device_fault, s);
 	if ((((end_bit + 7) / 8) % 2) == 0) {
 		// An even number of passes leaves the result in the input buffers; hand it over.
 		hipError_t e = hipMemcpyAsync(keys_out, keys_in, n * sizeof(uint64_t), hipMemcpyDeviceToDevice, s);
@@ -1146,7 +1183,7 @@ int rgs_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uin
 	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out && temp, "rgs_sort_pairs: null pointer");
 	RGS_REQUIRE(n < 0x40000000ull, "rgs_sort_pairs: 2^30 pairs or more");
 	return sort_pairs_u64("rgs_sort_pairs", keys_in, keys_out, vals_in, vals_out, n, end_bit, static_cast<uint32_t*>(temp),
-	                      fault_word(true), s);
+	                      fault_word(true), nullptr, s);
 }
 
 int rgs_sort_pairs_static(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
@@ -1163,10 +1200,13 @@ int rgs_sort_pairs_static(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_
 	RGS_REQUIRE(keys_in && keys_out && vals_in && vals_out, "rgs_sort_pairs_static: null pointer");
 	RGS_REQUIRE(rgs::sort_temp_words(n) <= kStaticSortWords, "rgs_sort_pairs_static: scratch layout mismatch");
 	uint32_t* temp = nullptr;
-	if (int rc = static_sort_scratch(&temp))
+	uint32_t* gave_up = nullptr;
+	if (int rc = static_sort_scratch(&temp, &gave_up))
 		return rc;
-	// the report word is only used if an earlier call has set it up: nothing is allocated here
-	return sort_pairs_u64("rgs_sort_pairs_static", keys_in, keys_out, vals_in, vals_out, n, end_bit, temp, fault_word(false), s);
+	// Nothing is allocated here: a give-up is reported in a word of device memory beside the scratch, which
+	// rgs_sort_fault reads, and also in the pinned word of the other entry points if an earlier call has set that up.
+	return sort_pairs_u64("rgs_sort_pairs_static", keys_in, keys_out, vals_in, vals_out, n, end_bit, temp, fault_word(false), gave_up,
+	                      s);
 }
 
 int rgs_set_lookback_spin_limit(int polls)
@@ -1181,7 +1221,9 @@ int rgs_sort_fault(void* stream)
 	const hipError_t e = hipStreamSynchronize(s);
 	if (e != hipSuccess)
 		return fail("rgs_sort_fault: %s", hipGetErrorString(e));
-	return take_sort_fault("rgs_sort_fault");
+	const int pinned = take_sort_fault("rgs_sort_fault");
+	const int in_device_memory = take_static_sort_fault("rgs_sort_fault");  // read (and cleared) either way
+	return pinned ? pinned : in_device_memory;
 }
 
 static int fill_composite(rgs::CompositeArgs& a, int K, int height, int width, const float* const* images,

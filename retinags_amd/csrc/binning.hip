@@ -1140,16 +1140,21 @@ __global__ __launch_bounds__(kFileBlock) void tile_ranges_kernel(Batch<TileRange
 	}
 }
 
-__global__ void report_sort_status_kernel(const uint32_t* __restrict__ status, uint32_t* __restrict__ fault)
+__global__ void report_sort_status_kernel(const uint32_t* __restrict__ status, uint32_t* __restrict__ fault,
+                                          uint32_t* __restrict__ device_fault)
 {
-	if (threadIdx.x == 0 && *status != 0u)
-		__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+	if (threadIdx.x == 0 && *status != 0u) {
+		if (fault)
+			__hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+		if (device_fault)
+			*device_fault = 1u;
+	}
 }
 
-void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_t s)
+void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, uint32_t* device_fault, hipStream_t s)
 {
-	if (fault)
-		hipLaunchKernelGGL(report_sort_status_kernel, dim3(1), dim3(64), 0, s, temp + kSortStatus, fault);
+	if (fault || device_fault)
+		hipLaunchKernelGGL(report_sort_status_kernel, dim3(1), dim3(64), 0, s, temp + kSortStatus, fault, device_fault);
 }
 
 void launch_tile_ranges(const TileRangesJob* jobs, int count, hipStream_t s)

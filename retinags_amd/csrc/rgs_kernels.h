@@ -408,8 +408,9 @@ const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a fai
 // Polls a look-back allows before it gives up (0 restores the default; negative: give up at once,
 // which is how a test exercises the give-up path with every kernel still running to its end).
 void set_lookback_spin_limit(int polls);
-// Sets *fault (host memory the device can write; null: nothing is launched) if the sort that used `temp` gave up.
-void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, hipStream_t s);
+// Sets *fault (host memory the device can write, may be null) and *device_fault (device memory, may be null) if the sort
+// that used `temp` gave up; with both null nothing is launched.
+void launch_report_sort_status(const uint32_t* temp, uint32_t* fault, uint32_t* device_fault, hipStream_t s);
 // The tile ranges from the sorted keys.  Either status word (may be null) being non-zero leaves every range empty
 // and sets *fault (host memory the device can write, may be null).  The caller has cleared `ranges`.  With a non-null
 // n_device the number of keys is min(n, *n_device) and the launch is sized for n.  file_tail (may be null)

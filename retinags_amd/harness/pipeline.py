@@ -150,6 +150,94 @@ def render_submodel(cam: Camera, sub: Submodel, bg: torch.Tensor, scaling_modifi
                          "depth": depth, "alpha": alpha, "num_rendered": -1})
 
 
+@dataclass
+class PipelineSwitches:
+    """The fields of the reference's PipelineParams that the renderer reads (arguments/__init__.py:71-79)."""
+    convert_SHs_python: bool = False
+    compute_cov3D_python: bool = False
+    debug: bool = False
+
+
+_SH_C0 = 0.5 * math.sqrt(1.0 / math.pi)
+_SH_C1 = math.sqrt(3.0 / (4.0 * math.pi))
+_SH_C2 = (0.5 * math.sqrt(15.0 / math.pi), 0.25 * math.sqrt(5.0 / math.pi), 0.25 * math.sqrt(15.0 / math.pi))
+_SH_C3 = (0.25 * math.sqrt(35.0 / (2.0 * math.pi)), 0.5 * math.sqrt(105.0 / math.pi), 0.25 * math.sqrt(21.0 / (2.0 * math.pi)),
+          0.25 * math.sqrt(7.0 / math.pi), 0.25 * math.sqrt(105.0 / math.pi))
+
+
+def sh_basis(degree: int, directions: torch.Tensor) -> torch.Tensor:
+    """(N, (degree+1)^2) values of the real spherical harmonics in the sign convention of the reference's eval_sh
+    (utils/sh_utils.py:57-115) at unit directions (N,3): column k multiplies SH coefficient k."""
+    if not 0 <= degree <= 3:
+        raise ValueError("SH degree must be 0..3")
+    x, y, z = directions.unbind(-1)
+    cols = [torch.full_like(x, _SH_C0)]
+    if degree > 0:
+        cols += [-_SH_C1 * y, _SH_C1 * z, -_SH_C1 * x]
+    if degree > 1:
+        xx, yy, zz = x * x, y * y, z * z
+        cols += [_SH_C2[0] * x * y, -_SH_C2[0] * y * z, _SH_C2[1] * (2 * zz - xx - yy), -_SH_C2[0] * x * z,
+                 _SH_C2[2] * (xx - yy)]
+    if degree > 2:
+        cols += [-_SH_C3[0] * y * (3 * xx - yy), _SH_C3[1] * x * y * z, -_SH_C3[2] * y * (4 * zz - xx - yy),
+                 _SH_C3[3] * z * (2 * zz - 3 * xx - 3 * yy), -_SH_C3[2] * x * (4 * zz - xx - yy), _SH_C3[4] * z * (xx - yy),
+                 -_SH_C3[0] * x * (xx - 3 * yy)]
+    return torch.stack(cols, dim=-1)
+
+
+def colours_from_sh(shs: torch.Tensor, degree: int, means3D: torch.Tensor, camera_center: torch.Tensor) -> torch.Tensor:
+    """The convert_SHs_python branch of render4BoundedGaussianModel (gaussian_renderer/render_half_gs.py:69-74): the
+    view-dependent colour of every Gaussian from its SH coefficients (N,16,3) as tensor operations,
+    clamp_min(SH(direction) + 0.5, 0), differentiable by autograd."""
+    direction = means3D - camera_center.view(1, 3)
+    direction = direction / direction.norm(dim=1, keepdim=True)
+    basis = sh_basis(degree, direction)                                   # (N, n)
+    rgb = torch.einsum("nk,nkc->nc", basis, shs[:, :basis.shape[1], :])
+    return torch.clamp_min(rgb + 0.5, 0.0)
+
+
+def covariance_from_scaling_rotation(scales: torch.Tensor, scaling_modifier: float, rotations: torch.Tensor) -> torch.Tensor:
+    """The compute_cov3D_python branch (render_half_gs.py:57-58 -> scene/gaussian_nn_module.py:298-302,
+    utils/general_utils.py:79-111): L = R(q / |q|) diag(modifier * s), Sigma = L L^T, returned as its six upper
+    entries (xx, xy, xz, yy, yz, zz)."""
+    q = rotations / rotations.norm(dim=1, keepdim=True)
+    r, x, y, z = q.unbind(-1)
+    R = torch.stack([1 - 2 * (y * y + z * z), 2 * (x * y - r * z), 2 * (x * z + r * y),
+                     2 * (x * y + r * z), 1 - 2 * (x * x + z * z), 2 * (y * z - r * x),
+                     2 * (x * z - r * y), 2 * (y * z + r * x), 1 - 2 * (x * x + y * y)], dim=-1).view(-1, 3, 3)
+    L = R * (scaling_modifier * scales).unsqueeze(1)                      # scales the columns: R @ diag(s)
+    sigma = L @ L.transpose(1, 2)
+    return torch.stack([sigma[:, 0, 0], sigma[:, 0, 1], sigma[:, 0, 2], sigma[:, 1, 1], sigma[:, 1, 2], sigma[:, 2, 2]], dim=-1)
+
+
+def render_bounded_model(cam: Camera, sub: Submodel, pipe: PipelineSwitches, bg: torch.Tensor, scaling_modifier: float = 1.0,
+                         override_color: Optional[torch.Tensor] = None) -> dict:
+    """render4BoundedGaussianModel (gaussian_renderer/render_half_gs.py:21-101) for a Submodel: the same switches decide
+    whether the rasterizer gets scales and rotations or a 3D covariance computed by tensor operations, and SH
+    coefficients, colours computed from them by tensor operations, or the caller's override_color; same return dict."""
+    rasterizer = GaussianRasterizer(raster_settings=raster_settings(cam, sub, bg, scaling_modifier, pipe.debug))
+    means2D = sub.means2D
+    if means2D is None:
+        means2D = _screenspace_placeholder(sub)
+    scales = rotations = cov3D_precomp = None
+    if pipe.compute_cov3D_python:
+        cov3D_precomp = covariance_from_scaling_rotation(sub.scales, scaling_modifier, sub.rotations)
+    else:
+        scales, rotations = sub.scales, sub.rotations
+    shs = colors_precomp = None
+    if override_color is None:
+        if pipe.convert_SHs_python:
+            colors_precomp = colours_from_sh(sub.shs, sub.active_sh_degree, sub.means3D, cam.camera_center)
+        else:
+            shs = sub.shs
+    else:
+        colors_precomp = override_color
+    color, radii, depth, alpha = rasterizer(means3D=sub.means3D, means2D=means2D, shs=shs, colors_precomp=colors_precomp,
+                                            opacities=sub.opacity, scales=scales, rotations=rotations, cov3D_precomp=cov3D_precomp)
+    return RenderResult({"render": color, "viewspace_points": means2D, "radii": radii, "depth": depth, "alpha": alpha,
+                         "num_rendered": -1})
+
+
 class RenderResult(dict):
     """What the reference's render() returns for a submodel (gaussian_renderer/__init__.py: "render",
     "viewspace_points", "visibility_filter", "radii", "depth", "alpha", "num_rendered").  The visibility filter
@@ -206,7 +294,8 @@ def _host_pool(n: int):
 def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, background: torch.Tensor,
                  submodel_bg: Optional[torch.Tensor] = None,
                  streams: Optional[List["torch.cuda.Stream"]] = None, host_threads: bool = False,
-                 instance_bounds: Optional[Dict[int, int]] = None, together: bool = False) -> dict:
+                 instance_bounds: Optional[Dict[int, int]] = None, together: bool = False,
+                 keep_workspaces: bool = False) -> dict:
     """Render every related submodel (black background, as the trainer does:
     trainer4tree_partition.py:397) and composite the partial images in BVH order.
 
@@ -221,9 +310,11 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     own (ctypes releases the interpreter lock inside the library); measured no faster, and less
     steady, than the two rounds: the threads contend for the interpreter between the calls.
 
-    together: the related submodels go through rasterize_frame: three library calls per frame, which blend all
-    submodels in one launch per direction (the stages that run once per submodel are queued on `streams`, if
-    given, beside each other); same results.
+    together: the related submodels go through rasterize_frame: three library calls per frame, every stage one
+    launch for all submodels.  Every forward stage runs on the current stream; `streams`, if given, only offers the
+    backward a second stream (the first that is not the current one) for its per-Gaussian half; same results.
+    keep_workspaces (with together): the frame also carries, under "workspaces", per submodel id what a single
+    forward call returns beside its images: (num_rendered, geomBuffer, binningBuffer, imgBuffer).
 
     instance_bounds (submodel id -> room for that many instances; with or without `streams`): the
     forward of each submodel is issued in one go, without waiting for its instance count.  The
@@ -249,8 +340,10 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
             rasterizers.append(GaussianRasterizer(raster_settings=raster_settings(cam, sub, submodel_bg)))
             inputs.append(dict(means3D=sub.means3D, means2D=means2D, shs=sub.shs, opacities=sub.opacity, scales=sub.scales,
                                rotations=sub.rotations))
+        taps = [] if keep_workspaces else None
         outs = rasterize_frame(rasterizers, inputs,
-                               streams=[lanes[k % len(lanes)].cuda_stream for k in range(len(related))] if streams else None)
+                               streams=[lanes[k % len(lanes)].cuda_stream for k in range(len(related))] if streams else None,
+                               workspaces=taps)
         partial = {}
         for k, m in enumerate(related):
             color, radii, depth, alpha = outs[k]
@@ -328,6 +421,8 @@ def render_frame(cam: Camera, subs: List[Submodel], relation: np.ndarray, backgr
     out = blender_render_result(partial, relation, background)
     out["partial"] = partial
     out["stages"] = stages
+    if together and keep_workspaces:
+        out["workspaces"] = {m: taps[k] for k, m in enumerate(related)}
     return out
 
 

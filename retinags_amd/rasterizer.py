@@ -432,16 +432,17 @@ class _RasterizeFrame(torch.autograd.Function):
     (every layer's geometry stage, then binning and one blend launch for all, and for the backward one
     blend launch for all and every layer's per-Gaussian backward).
 
-    apply(settings, streams, *flat): `settings` a tuple of K GaussianRasterizationSettings (same camera and
-    image size), `streams` None or a tuple of K HIP stream handles (the first that differs from the current
-    stream serves the backward as a second stream for its memory-bound work), flat = for every layer
-    (means3D, means2D, sh, colors_precomp, opacities, scales, rotations, cov3Ds_precomp).
-    Returns for every layer (color, radii, depth, alpha)."""
+    apply(settings, streams, workspaces, *flat): `settings` a tuple of K GaussianRasterizationSettings (same
+    camera and image size), `streams` None or a tuple of K HIP stream handles (the first that differs from the
+    current stream serves the backward as a second stream for its memory-bound work), `workspaces` None or a
+    list that receives, per layer, what a single call returns beside its images: (num_rendered, geomBuffer,
+    binningBuffer, imgBuffer), flat = for every layer (means3D, means2D, sh, colors_precomp, opacities, scales,
+    rotations, cov3Ds_precomp).  Returns for every layer (color, radii, depth, alpha)."""
 
     FIELDS = 8
 
     @staticmethod
-    def forward(ctx, settings, streams, *flat):
+    def forward(ctx, settings, streams, workspaces, *flat):
         K = len(settings)
         if K == 0 or len(flat) != _RasterizeFrame.FIELDS * K:
             raise RuntimeError("rasterize_frame: one group of eight tensors per layer is needed")
@@ -522,6 +523,8 @@ class _RasterizeFrame(torch.autograd.Function):
             outs += [rec["package"][0:3], rec["radii"], rec["package"][3:4], rec["package"][4:5]]
         ctx.save_for_backward(*saved)
         ctx.mark_non_differentiable(*[outs[4 * k + 1] for k in range(K)])
+        if workspaces is not None:
+            workspaces.extend((rec["rendered"], rec["geom"], rec["binning"], rec["img"]) for rec in records)
         return tuple(outs)
 
     @staticmethod
@@ -592,7 +595,7 @@ class _RasterizeFrame(torch.autograd.Function):
             flat += [g_means3D, g_means2D, g_sh if sh.numel() else None, g_colors if colors_precomp.numel() else None,
                      g_opacity, g_scales if scales.numel() else None, g_rot if rotations.numel() else None,
                      g_cov3D if cov3Ds.numel() else None]
-        return (None, None, *flat)
+        return (None, None, None, *flat)
 
 
 def _frame_scratch(colors_precomp, cov3Ds_precomp):
@@ -614,13 +617,15 @@ def _frame_counts(device: torch.device, n: int) -> torch.Tensor:
     return t
 
 
-def rasterize_frame(rasterizers, inputs, streams=None):
+def rasterize_frame(rasterizers, inputs, streams=None, workspaces=None):
     """All layers of a frame through one call.  `rasterizers`: K GaussianRasterizer (their settings share the
     camera and the image size); `inputs`: K dicts with the keyword arguments of GaussianRasterizer.forward
     (means3D, means2D, opacities, shs / colors_precomp, scales + rotations / cov3D_precomp); `streams`: None,
     or for every layer the handle of a HIP stream; the first that is not the current stream takes memory-bound work
     beside the kernels of the current one: the backward runs the per-Gaussian part of the layers whose blend is done
-    on it (the caller's stream waits for it).  Returns K tuples (color, radii, depth, alpha), the results of K
+    on it (the caller's stream waits for it); every forward stage runs on the current stream.  `workspaces`: None, or a
+    list that receives per layer (num_rendered, geomBuffer, binningBuffer, imgBuffer), the rest of the 8-tuple a single
+    forward call returns (K/rasterize_points.cu:124).  Returns K tuples (color, radii, depth, alpha), the results of K
     forward calls, and differentiates like them."""
     flat = []
     for rz, kw in zip(rasterizers, inputs):
@@ -628,7 +633,7 @@ def rasterize_frame(rasterizers, inputs, streams=None):
             kw.get("shs"), kw.get("colors_precomp"), kw.get("scales"), kw.get("rotations"), kw.get("cov3D_precomp"))
         flat += [kw["means3D"], kw["means2D"], shs, colors_precomp, kw["opacities"], scales, rotations, cov3D]
     outs = _RasterizeFrame.apply(tuple(rz.raster_settings for rz in rasterizers),
-                                 None if streams is None else tuple(streams), *flat)
+                                 None if streams is None else tuple(streams), workspaces, *flat)
     return [tuple(outs[4 * k:4 * k + 4]) for k in range(len(rasterizers))]
 
 

@@ -119,6 +119,8 @@ def render_reference(params, cam, W, H, low, up, bg, sh_degree=3, mod=1.0):
     w_clip = p_clip[:, 3]
     ndc = p_clip[:, :2] / (w_clip[:, None] + 1e-7)
     pix = torch.stack([((ndc[:, 0] + 1) * W - 1) * 0.5, ((ndc[:, 1] + 1) * H - 1) * 0.5], -1)
+    if pix.requires_grad:
+        pix.retain_grad()   # the blend is the only differentiable reader of the pixel centres: see aux["pix_node"]
     cov3d = covariance3d(scales, quats, mod)
     cov2d = ewa_cov2d(xyz, cov3d, view_t, W, H, tanx, tany)
     conic = torch.linalg.inv(cov2d)
@@ -200,7 +202,7 @@ def render_reference(params, cam, W, H, low, up, bg, sh_degree=3, mod=1.0):
             color[:, py, px] = (wgt[:, None] * rgb[idt]).sum(0) + Tend * bg
             out_depth[0, py, px] = (wgt * depth[idt]).sum()
             out_alpha[0, py, px] = wgt.sum()
-    aux = dict(radius=radius, rects=rects, visible=visible, pix=pix.detach(), conic=conic.detach(),
+    aux = dict(radius=radius, rects=rects, visible=visible, pix=pix.detach(), pix_node=pix, conic=conic.detach(),
                depth=depth.detach(), rgb=rgb.detach(), cov3d=cov3d.detach(), cov2d=cov2d.detach())
     return color, out_depth, out_alpha, aux
 

@@ -240,3 +240,37 @@ def test_entry_points_refuse_bad_arguments_before_touching_the_gpu():
             "no room for the SH gradients")
     assert lib.rgs_activate_forward(0, 15, *([null] * 10)) == 0 and lib.rgs_activate_backward(0, 15, *([null] * 13)) == 0
     assert lib.rgs_straddler_scratch_bytes(-1, 4) == 0 and lib.rgs_straddler_scratch_bytes(1025, 3) == 4 * 3 * 3
+
+
+def test_tensor_expression_branches_of_the_renderer_match_the_checker():
+    """The convert_SHs_python and compute_cov3D_python branches of render4BoundedGaussianModel
+    (gaussian_renderer/render_half_gs.py:55-77) as the harness restates them: colours and 3D covariances from tensor
+    operations against what the checker's preprocess computes in its kernel-order arithmetic, SH degrees 0 to 3,
+    a scale modifier, and quaternions that are not normalised (the tensor expression normalises them, the kernel
+    uses them as given: equal only for unit quaternions, which is what a model's get_rotation hands out)."""
+    from helpers import np32, oracle_settings, scenes
+    from retinags_amd.harness import pipeline
+    scene, cam, _ = scenes.make_config("C0", shrink=100, resolution_scale=0.25)
+    pad = 3.0 * float(scene["scales"].max()) + 1.0
+    low, up = scene["xyz"].min(0).values - pad, scene["xyz"].max(0).values + pad
+    for degree, mod in ((0, 1.0), (1, 1.0), (2, 1.0), (3, 1.0), (3, 0.7)):
+        s = oracle_settings(cam, low, up, torch.zeros(3), sh_degree=degree, scale_modifier=mod)
+        st = orc.forward(s, np32(scene["xyz"]), np32(scene["opacity"]), shs=np32(scene["shs"]), scales=np32(scene["scales"]),
+                         rotations=np32(scene["rotations"]))
+        vis = st.radii > 0
+        assert vis.sum() > 100
+        rgb = pipeline.colours_from_sh(scene["shs"], degree, scene["xyz"], cam.camera_center).numpy()
+        cov = pipeline.covariance_from_scaling_rotation(scene["scales"], mod, scene["rotations"]).numpy()
+        assert np.abs(rgb[vis] - st.rgb[vis]).max() <= 1e-6
+        assert np.abs(cov[vis] - st.cov3D[vis]).max() <= 1e-6 * np.abs(st.cov3D[vis]).max()
+        # clamped channels are zero in both
+        assert np.array_equal(rgb[vis] == 0.0, st.clamped[vis].astype(bool)) or np.abs((rgb[vis] == 0.0) ^ st.clamped[vis].astype(bool)).mean() < 1e-3
+    # the basis itself against scipy's complex harmonics, through the test-side polynomials (sign convention (-1)^m)
+    import refmath
+    d = torch.randn(64, 3, dtype=torch.float64)
+    d = d / d.norm(dim=1, keepdim=True)
+    assert torch.allclose(pipeline.sh_basis(3, d), refmath.sh_polynomials(d), atol=1e-12)
+    assert np.allclose(pipeline.sh_basis(3, d).numpy(), refmath.real_sh_basis(d.numpy(), 3), atol=1e-12)
+    scaled = pipeline.covariance_from_scaling_rotation(scene["scales"], 1.0, 3.0 * scene["rotations"])
+    plain = pipeline.covariance_from_scaling_rotation(scene["scales"], 1.0, scene["rotations"])
+    assert float((scaled - plain).abs().max()) <= 1e-6 * float(plain.abs().max())

@@ -4,7 +4,14 @@ to size-independent properties: structure of the binning output (sortedness, sta
 partition, counts), bit-for-bit determinism, the compositing identity, and exact linearity of
 the rendered loss in the SH DC coefficients (a finite-difference check of dL/dSH that needs no
 oracle).  The scenes of C3 (62.9 M Gaussians) and C4 (217.3 M) are generated and partitioned
-on the device.  Config names are those of retinags_amd.harness.scenes.CONFIGS."""
+on the device.  Config names are those of retinags_amd.harness.scenes.CONFIGS.
+
+Every configuration is rendered both ways the library offers: one call per submodel
+(rgs_forward_geom / rgs_forward_raster / rgs_backward, the reference's call pattern) and all
+submodels of the frame through rgs_frame_forward_geom / _raster / rgs_frame_backward (one launch
+per stage for the whole frame, which is what bench.py times).  The two must agree bit for bit in
+everything but the atomically summed gradients, and the comparisons with the CPU checker are
+taken from the frame path's outputs."""
 import numpy as np
 import pytest
 import torch
@@ -103,46 +110,118 @@ def _frame_setup_on_device(name):
     return cam, cfg, subs, rel, part
 
 
-def _submodel_against_checker(sub, cam, low, up, seed, with_backward):
-    """One submodel of a device-resident scene against the CPU checker (OpenMP): instance count, radii,
-    binning bit for bit, images, and with_backward every gradient."""
+FRAME_GRAD_TOL = 1e-5   # relative L2 between the two paths' gradients: same terms, another order of the atomic adds
+
+
+def _frame_against_calls_per_submodel(cam, subs, rel, bg, with_backward, seed, grads_on_layers=False):
+    """Renders the frame through rasterize_frame (pipeline.render_frame(together=True)) and again with one call per
+    submodel, and holds the former to the latter: instance counts, radii, the sorted lists, tile ranges, n_contrib and
+    the images bit for bit; with_backward every gradient to FRAME_GRAD_TOL.  The upstream gradient is put on the
+    composited image, or (grads_on_layers) directly on every layer's image.  Returns the frame path's output (with
+    its workspaces) and, with_backward, {submodel: {field: gradient}} of the frame path, and the upstream gradient."""
+    from retinags_amd import _capi
+    from retinags_amd.harness import pipeline
+    cam_d = cam.to(DEV)
+    H, W = cam.image_height, cam.image_width
+    related = [m for m in range(len(subs)) if rel[m] >= 0]
+    g = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(seed)) * 1e-2).to(DEV)
+    fields = ("means3D", "opacity", "scales", "rotations", "shs")
+
+    def take_grads():
+        out = {}
+        for m in related:
+            out[m] = {f: getattr(subs[m], f).grad for f in fields}
+            out[m]["means2D"] = subs[m].means2D.grad
+            for t in subs[m].parameters():
+                t.grad = None
+            subs[m].means2D = None
+        return out
+
+    def prepare():
+        for m in related:
+            subs[m].requires_grad_(with_backward)
+            subs[m].means2D = torch.zeros_like(subs[m].means3D, requires_grad=True) if with_backward else None
+
+    def send_back(out):
+        if grads_on_layers:
+            torch.autograd.backward([out["partial"][m]["render"] for m in related], [g for _ in related])
+        else:
+            torch.autograd.backward([out["render"]], [g])
+
+    prepare()
+    frame = pipeline.render_frame(cam_d, subs, rel, bg, together=True, keep_workspaces=True)
+    frame_grads = None
+    if with_backward:
+        send_back(frame)
+        frame_grads = take_grads()
+    prepare()
+    zero = torch.zeros(3, device=DEV)
+    im = _capi.image_layout(W, H)
+    T = ((W + 15) // 16) * ((H + 15) // 16)
+    piece = lambda buf, off, nbytes: buf[off:off + nbytes]
+    for m in related:
+        Rn, geom, binning, img = frame["workspaces"][m]
+        raw = _forward_raw(subs[m], cam_d, cam, zero)
+        assert raw[0] == Rn, m
+        layer = frame["partial"][m]
+        assert torch.equal(raw[4], layer["radii"]), m
+        for k, key in ((1, "render"), (2, "depth"), (3, "alpha")):
+            assert torch.equal(raw[k], layer[key].detach()), (m, key)          # the images, bit for bit
+        assert torch.equal(piece(raw[7], im["n_contrib"], 4 * W * H), piece(img, im["n_contrib"], 4 * W * H)), m
+        assert torch.equal(piece(raw[7], im["ranges"], 8 * T), piece(img, im["ranges"], 8 * T)), m
+        if Rn:
+            b = _capi.binning_layout(Rn, W, H)
+            for name in ("keys_sorted", "values_sorted"):
+                assert torch.equal(piece(raw[6], b[name], 4 * Rn), piece(binning, b[name], 4 * Rn)), (m, name)
+        del raw
+    if with_backward:
+        again = pipeline.render_frame(cam_d, subs, rel, bg)   # one call per submodel
+        assert torch.equal(again["render"], frame["render"]) and torch.equal(again["alpha"], frame["alpha"])
+        send_back(again)
+        call_grads = take_grads()
+        from helpers import rel_l2
+        for m in related:
+            for f, want in call_grads[m].items():
+                got = frame_grads[m][f]
+                assert (got is None) == (want is None), (m, f)
+                if want is not None:
+                    assert rel_l2(got.cpu().numpy(), want.cpu().numpy()) <= FRAME_GRAD_TOL, (m, f)
+        del again, call_grads
+    for m in related:
+        subs[m].requires_grad_(False)
+        subs[m].means2D = None
+    return frame, frame_grads, g
+
+
+def _frame_layer_against_checker(frame, frame_grads, m, sub, cam, low, up, g_layer):
+    """Submodel m of a frame rendered through rasterize_frame against the CPU checker (OpenMP): instance count,
+    radii, binning bit for bit, images, and (with frame_grads: gradients taken with g_layer on this layer's image)
+    every gradient."""
     import os
     from helpers import DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, np32, orc, rel_l2
-    from retinags_amd.harness import pipeline
     H, W = cam.image_height, cam.image_width
-    cam_d = cam.to(DEV)
-    bg = torch.zeros(3, device=DEV)
-    g = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(seed)) * 1e-2)
     xyz, opa, sc, rot, shs = (np32(t) for t in (sub.means3D, sub.opacity, sub.scales, sub.rotations, sub.shs))
     orc.set_threads(min(16, orc.max_threads(), os.cpu_count() or 1))
     try:
         s = orc.settings_from_camera(cam, low, up, torch.zeros(3))
         st = orc.forward(s, xyz, opa, shs=shs, scales=sc, rotations=rot, want_margin=True)
-        want = orc.backward(s, st, np32(g)) if with_backward else None
+        want = orc.backward(s, st, np32(g_layer)) if frame_grads is not None else None
     finally:
         orc.set_threads(1)
-    raw = _forward_raw(sub, cam_d, cam, bg)
-    assert raw[0] == st.R
-    check_binning_against(st, raw[5], raw[6], st.P, st.R, W, H)
-    del raw
-    sub.requires_grad_(with_backward)
-    layer = pipeline.render_submodel(cam_d, sub, bg)
+    Rn, geom, binning, img = frame["workspaces"][m]
+    assert Rn == st.R
+    check_binning_against(st, geom, binning, st.P, st.R, W, H)
+    layer = frame["partial"][m]
     assert np.array_equal(layer["radii"].cpu().numpy(), st.radii)
     safe = (st.margin > DECISION_MARGIN).reshape(H, W)
     assert (~safe).mean() < 1e-3
     for key, want_plane in (("render", st.color), ("alpha", st.alpha), ("depth", st.depth)):
-        # colour and alpha are of order one; the depth plane is in scene units (hundreds in the city scene),
-        # so its bound is taken relative to the largest depth
         tol = IMAGE_TOL * (max(1.0, float(np.abs(want_plane).max())) if key == "depth" else 1.0)
         assert np.abs(layer[key].detach().cpu().numpy() - want_plane)[:, safe].max() <= tol, key
-    if with_backward:
-        torch.autograd.backward([layer["render"]], [g.to(DEV)])
-        for key, t in (("means3D", sub.means3D), ("sh", sub.shs), ("opacity", sub.opacity), ("scales", sub.scales),
-                       ("rotations", sub.rotations)):
-            assert rel_l2(t.grad.cpu().numpy(), want[key]) <= GRAD_TOL, key
-        sub.requires_grad_(False)
-        for t in sub.parameters():
-            t.grad = None
+    if frame_grads is not None:
+        for key, f in (("means3D", "means3D"), ("means2D", "means2D"), ("sh", "shs"), ("opacity", "opacity"), ("scales", "scales"),
+                       ("rotations", "rotations")):
+            assert rel_l2(frame_grads[m][f].cpu().numpy(), want[key]) <= GRAD_TOL, (m, key)
     return st
 
 
@@ -234,10 +313,11 @@ def test_garden_full_size_structure_determinism_and_sh_linearity():
 
 
 def test_garden_full_size_against_checker():
-    """Config C1 at full size against the CPU checker (OpenMP makes it fast enough): every
-    submodel's binning bit for bit, its images and every gradient, the screen-space gradient
-    included, with the upstream gradients that the compositor's backward hands each layer; then
-    the composited frame."""
+    """Config C1 at full size against the CPU checker (OpenMP makes it fast enough), rendered the way bench.py times
+    it: all four submodels through rasterize_frame (rgs_frame_forward_geom / _raster / rgs_frame_backward).  Every
+    submodel's binning bit for bit, its images and every gradient, the screen-space gradient included, with the
+    upstream gradients that the compositor's backward hands each layer; then the composited frame.  The same frame
+    with one call per submodel must give the same bits (gradients: the same sums in another order)."""
     from helpers import DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, np32, orc, rel_l2
     from retinags_amd.harness import partition, pipeline
     from retinags_amd import _capi
@@ -246,14 +326,12 @@ def test_garden_full_size_against_checker():
     part = partition.partition_scene(scene["xyz"], scene["scales"], 2)
     rel = partition.relation_vector(part, cam)
     assert (rel >= 0).all()
-    subs = [s_.requires_grad_(True) for s_ in pipeline.submodels_from_partition(scene, part, DEV)]
-    for s_ in subs:
-        s_.means2D = torch.zeros_like(s_.means3D, requires_grad=True)
+    subs = pipeline.submodels_from_partition(scene, part, DEV)
     H, W = cam.image_height, cam.image_width
-    g = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(11)) * 1e-2)
     bg = torch.tensor([0.1, 0.3, 0.2])
+    frame, grads, g = _frame_against_calls_per_submodel(cam, subs, rel, bg.to(DEV), with_backward=True, seed=11)
+    g = g.cpu()
     xyz, opa, sc, rot, shs = (np32(scene[k]) for k in ("xyz", "opacity", "scales", "rotations", "shs"))
-    cam_d = cam.to(DEV)
     orc.set_threads(min(16, orc.max_threads(), os.cpu_count() or 1))
     try:
         order = sorted(range(4), key=lambda m: rel[m])
@@ -263,23 +341,21 @@ def test_garden_full_size_against_checker():
             sets[m] = orc.settings_from_camera(cam, part.box_low[m], part.box_up[m], torch.zeros(3))
             states[m] = orc.forward(sets[m], xyz[ids], opa[ids], shs=shs[ids], scales=sc[ids], rotations=rot[ids],
                                     want_margin=True)
-        for m in order:   # binning, bit for bit
+        for m in order:   # binning of the frame path, bit for bit
             st = states[m]
-            raw = _forward_raw(subs[m], cam_d, cam, torch.zeros(3, device=DEV))
-            assert raw[0] == st.R
-            check_binning_against(st, raw[5], raw[6], st.P, st.R, W, H)
-            assert np.array_equal(view_ws(raw[7], _capi.image_layout(W, H)["ranges"], 2 * len(st.ranges), np.uint32),
+            Rn, geom, binning, img = frame["workspaces"][m]
+            assert Rn == st.R
+            check_binning_against(st, geom, binning, st.P, st.R, W, H)
+            assert np.array_equal(view_ws(img, _capi.image_layout(W, H)["ranges"], 2 * len(st.ranges), np.uint32),
                                   st.ranges.ravel())
-            del raw
-        out = pipeline.render_frame(cam_d, subs, rel, bg.to(DEV))
-        torch.autograd.backward([out["render"]], [g.to(DEV)])
+        out = frame
         imgs, deps, alps = ([states[m].color for m in order], [states[m].depth for m in order],
                             [states[m].alpha for m in order])
         want_img, want_dep, want_alpha = orc.composite_forward(imgs, deps, alps, np32(bg))
         d_img, d_dep, d_alp = orc.composite_backward(imgs, deps, alps, np32(bg), np32(g))
         safe_all = np.ones((H, W), dtype=bool)
         for k, m in enumerate(order):
-            st, sub, layer = states[m], subs[m], out["partial"][m]
+            st, layer = states[m], out["partial"][m]
             want = orc.backward(sets[m], st, d_img[k], d_dep[k], d_alp[k])
             assert np.array_equal(layer["radii"].cpu().numpy(), st.radii)
             safe = (st.margin > DECISION_MARGIN).reshape(H, W)
@@ -288,9 +364,9 @@ def test_garden_full_size_against_checker():
             assert np.abs(layer["render"].detach().cpu().numpy() - st.color)[:, safe].max() <= IMAGE_TOL
             assert np.abs(layer["alpha"].detach().cpu().numpy() - st.alpha)[:, safe].max() <= IMAGE_TOL
             assert np.abs(layer["depth"].detach().cpu().numpy() - st.depth)[:, safe].max() <= IMAGE_TOL
-            for key, t in (("means3D", sub.means3D), ("means2D", sub.means2D), ("sh", sub.shs), ("opacity", sub.opacity),
-                           ("scales", sub.scales), ("rotations", sub.rotations)):
-                assert rel_l2(t.grad.cpu().numpy(), want[key]) <= GRAD_TOL, (m, key)
+            for key, f in (("means3D", "means3D"), ("means2D", "means2D"), ("sh", "shs"), ("opacity", "opacity"),
+                           ("scales", "scales"), ("rotations", "rotations")):
+                assert rel_l2(grads[m][f].cpu().numpy(), want[key]) <= GRAD_TOL, (m, key)
         assert np.abs(out["render"].detach().cpu().numpy() - want_img)[:, safe_all].max() <= IMAGE_TOL
         assert np.abs(out["alpha"].detach().cpu().numpy() - want_alpha)[:, safe_all].max() <= IMAGE_TOL
         assert np.abs(out["depth"].detach().cpu().numpy() - want_dep)[:, safe_all].max() <= IMAGE_TOL
@@ -301,8 +377,8 @@ def test_garden_full_size_against_checker():
 def test_high_resolution_full_size():
     """Config C2 at full size: the 5.6 M Gaussians of C1 at 5185x3359 (68 250 tiles: 17-bit tile keys, three
     radix passes, an odd count, so the sorted lists end in the other buffer pair than at C1), about 71 M
-    instances.  Structure and determinism of every submodel, the compositing identity, SH linearity, and the
-    submodel with the most instances against the CPU checker."""
+    instances.  Structure and determinism of every submodel, the compositing identity, SH linearity, the frame through
+    rasterize_frame against one call per submodel, and the submodel with the most instances against the CPU checker."""
     from helpers import DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, np32, orc, rel_l2
     from retinags_amd.harness import partition, pipeline
     from retinags_amd import _capi
@@ -331,31 +407,12 @@ def test_high_resolution_full_size():
                                     rel, torch.tensor([0.1, 0.2, 0.3], device=DEV))
     _sh_linearity(cam, subs, rel, which=None, seed=4)
 
+    # the whole frame through rasterize_frame against one call per submodel, forward and backward; then the submodel
+    # with the most instances, as the frame path rendered it, against the CPU checker
+    bg = torch.zeros(3, device=DEV)
+    frame, grads, g = _frame_against_calls_per_submodel(cam, subs, rel, bg, with_backward=True, seed=12, grads_on_layers=True)
     m = max(counts, key=counts.get)
-    ids = part.members[m]
-    xyz, opa, sc, rot, shs = (np32(scene[k][ids]) for k in ("xyz", "opacity", "scales", "rotations", "shs"))
-    g = (torch.randn(3, H, W, generator=torch.Generator().manual_seed(12)) * 1e-2)
-    orc.set_threads(min(16, orc.max_threads(), os.cpu_count() or 1))
-    try:
-        s = orc.settings_from_camera(cam, part.box_low[m], part.box_up[m], torch.zeros(3))
-        st = orc.forward(s, xyz, opa, shs=shs, scales=sc, rotations=rot, want_margin=True)
-        want = orc.backward(s, st, np32(g))
-    finally:
-        orc.set_threads(1)
-    sub = subs[m].requires_grad_(True)
-    raw = _forward_raw(sub, cam_d, cam, bg)
-    assert raw[0] == st.R
-    check_binning_against(st, raw[5], raw[6], st.P, st.R, W, H)
-    del raw
-    layer = pipeline.render_submodel(cam_d, sub, bg)
-    torch.autograd.backward([layer["render"]], [g.to(DEV)])
-    safe = (st.margin > DECISION_MARGIN).reshape(H, W)
-    assert (~safe).mean() < 1e-3
-    assert np.abs(layer["render"].detach().cpu().numpy() - st.color)[:, safe].max() <= IMAGE_TOL
-    assert np.abs(layer["alpha"].detach().cpu().numpy() - st.alpha)[:, safe].max() <= IMAGE_TOL
-    for key, t in (("means3D", sub.means3D), ("sh", sub.shs), ("opacity", sub.opacity), ("scales", sub.scales),
-                   ("rotations", sub.rotations)):
-        assert rel_l2(t.grad.cpu().numpy(), want[key]) <= GRAD_TOL, key
+    _frame_layer_against_checker(frame, grads, m, subs[m], cam, part.box_low[m], part.box_up[m], g)
 
 
 def test_dense_scene_full_size_sixteen_submodels():
@@ -376,9 +433,15 @@ def test_dense_scene_full_size_sixteen_submodels():
         counts[m] = outs[0]
         del outs, again
     assert sum(counts.values()) > 20_000_000
-    # the two submodels with the most instances against the CPU checker, forward and backward
+    # the whole frame (every submodel the camera sees, one launch per stage) against one call per submodel, forward
+    # and backward; then the two submodels with the most instances, as the frame path rendered them, against the
+    # CPU checker, forward and backward
+    frame, grads, g = _frame_against_calls_per_submodel(cam, subs, rel, torch.zeros(3, device=DEV), with_backward=True, seed=40,
+                                                        grads_on_layers=True)
     for m in sorted(counts, key=counts.get)[-2:]:
-        _submodel_against_checker(subs[m], cam, part.box_low[m], part.box_up[m], seed=40 + m, with_backward=True)
+        _frame_layer_against_checker(frame, grads, m, subs[m], cam, part.box_low[m], part.box_up[m], g)
+    del frame, grads
+    torch.cuda.empty_cache()
     bg = torch.tensor([0.1, 0.2, 0.3], device=DEV)
     with torch.no_grad():
         _check_compositing_identity(pipeline.render_frame(cam_d, subs, rel, bg), rel, bg)
@@ -402,8 +465,14 @@ def test_city_full_size_forward_only_thirty_two_submodels():
         assert outs[0] == again[0] and all(torch.equal(outs[k], again[k]) for k in (1, 2, 3, 4))
         counts[m] = outs[0]
         del outs, again
-    m = max(counts, key=counts.get)   # the submodel with the most instances against the CPU checker
-    _submodel_against_checker(subs[m], cam, part.box_low[m], part.box_up[m], seed=50, with_backward=False)
+    # the frame through rasterize_frame against one call per submodel, then the submodel with the most instances,
+    # as the frame path rendered it, against the CPU checker
+    with torch.no_grad():
+        frame, _, _ = _frame_against_calls_per_submodel(cam, subs, rel, bg, with_backward=False, seed=50)
+    m = max(counts, key=counts.get)
+    _frame_layer_against_checker(frame, None, m, subs[m], cam, part.box_low[m], part.box_up[m], None)
+    del frame
+    torch.cuda.empty_cache()
     with torch.no_grad():
         out = pipeline.render_frame(cam_d, subs, rel, torch.tensor([0.3, 0.2, 0.1], device=DEV))
     _check_compositing_identity(out, rel, torch.tensor([0.3, 0.2, 0.1], device=DEV))

@@ -358,13 +358,22 @@ def _oracle_vs_autograd(scene, cam, low, up, bg, seed, with_aux_outputs):
     s, st = run_oracle(scene, cam, low, up, bg)
     got = orc.backward(s, st, np32(g_color), None if g_depth is None else np32(g_depth),
                        None if g_alpha is None else np32(g_alpha))
-    p, (color, depth, alpha, _) = _reference_render(scene, cam, low, up, bg, grad=True)
+    p, (color, depth, alpha, aux) = _reference_render(scene, cam, low, up, bg, grad=True)
     loss = (color * g_color).sum()
     if with_aux_outputs:
         loss = loss + (depth * g_depth).sum() + (alpha * g_alpha).sum()
     loss.backward()
     pairs = (("means3D", "xyz"), ("opacity", "opacity"), ("scales", "scales"), ("rotations", "rotations"), ("sh", "shs"))
-    return {a: rel_l2(got[a], p[b].grad.numpy()) for a, b in pairs}, got, st
+    errs = {a: rel_l2(got[a], p[b].grad.numpy()) for a, b in pairs}
+    # The screen-space gradient the rasterizer hands back is taken with respect to the NDC position through the blend
+    # alone (K/cuda_rasterizer_hgs/backward.cu:496-497, 610-611: dL/ddelta times 0.5 W, 0.5 H); the independent
+    # renderer's pixel centre is (ndc + 1) * 0.5 * (W, H) - 0.5 and only its blend reads it, so dL/dmean2D =
+    # 0.5 (W, H) dL/dpixel-centre, and the third column stays zero.
+    H, W = cam.image_height, cam.image_width
+    d_pix = aux["pix_node"].grad.numpy()
+    want_2d = np.concatenate([d_pix * np.array([0.5 * W, 0.5 * H]), np.zeros((d_pix.shape[0], 1))], axis=1)
+    errs["means2D"] = rel_l2(got["means2D"], want_2d)
+    return errs, got, st
 
 
 def test_backward_matches_autograd_colour_only():
