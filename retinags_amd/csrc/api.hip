@@ -216,7 +216,7 @@ struct Carver {
 
 // Scratch of the depth sort of the Gaussians, inside the geometry workspace.
 struct OrderScratch {
-	size_t keys_a, keys_b, vals_b, tiles_in_order, sort_temp, scan_temp, dup_first, tile_digits, total;
+	size_t keys_a, keys_b, vals_a, vals_b, tiles_in_order, sort_temp, scan_temp, dup_first, tile_digits, total;
 };
 
 OrderScratch order_scratch(size_t P)
@@ -225,6 +225,7 @@ OrderScratch order_scratch(size_t P)
 	OrderScratch o;
 	o.keys_a = c.take(4 * P);
 	o.keys_b = c.take(4 * P);
+	o.vals_a = c.take(4 * P);
 	o.vals_b = c.take(4 * P);
 	o.tiles_in_order = c.take(4 * P);
 	o.sort_temp = c.take(4 * rgs::sort_temp_words(P));
@@ -406,7 +407,7 @@ int rgs_binning_layout(int R, int width, int height, size_t offsets[RGS_BIN_FIEL
 {
 	RGS_REQUIRE(R >= 0 && width > 0 && height > 0 && offsets, "rgs_binning_layout: bad arguments");
 	const BinningPhysical b = binning_physical((size_t)R);
-	const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
+	const bool sorted_in_a = (rgs::sort_passes(tile_key_bits(width, height), rgs::kDigitBitsU32) % 2) == 0;
 	offsets[RGS_BIN_KEYS_UNSORTED] = sorted_in_a ? b.keys_b : b.keys_a;
 	offsets[RGS_BIN_KEYS_SORTED] = sorted_in_a ? b.keys_a : b.keys_b;
 	offsets[RGS_BIN_VALUES_UNSORTED] = sorted_in_a ? b.vals_b : b.vals_a;
@@ -548,7 +549,7 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 		const OrderScratch o = order_scratch((size_t)c.P);
 		char* scratch = at<char>(ws, off[RGS_GEOM_ORDER_SCRATCH]);
 		a.clear = at<uint32_t>(scratch, o.sort_temp);
-		a.clear_words = rgs::sort_clear_words((size_t)c.P, 32);
+		a.clear_words = rgs::depth_sort_clear_words((size_t)c.P);
 
 		totals[(size_t)k] = rgs::TotalsJob{a.block_sums, a.block_visible, c.P, at<uint32_t>(ws, off[RGS_GEOM_TOTAL]),
 		                                   frame_counts + k, at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_COUNT])};
@@ -557,7 +558,8 @@ static int forward_geom(bool wait_for_count, void* count_ready_event, const char
 		d.depths = a.depths; d.tiles_touched = a.tiles_touched; d.block_visible = a.block_visible;
 		d.visible_count = at<uint32_t>(ws, off[RGS_GEOM_VISIBLE_COUNT]);
 		d.keys_a = at<uint32_t>(scratch, o.keys_a); d.keys_b = at<uint32_t>(scratch, o.keys_b);
-		d.order = at<uint32_t>(ws, off[RGS_GEOM_DEPTH_ORDER]); d.vals_b = at<uint32_t>(scratch, o.vals_b);
+		d.order = at<uint32_t>(ws, off[RGS_GEOM_DEPTH_ORDER]); d.vals_a = at<uint32_t>(scratch, o.vals_a);
+		d.vals_b = at<uint32_t>(scratch, o.vals_b);
 		d.tiles_in_order = at<uint32_t>(scratch, o.tiles_in_order);
 		d.offsets_in_order = at<uint32_t>(ws, off[RGS_GEOM_POINT_OFFSETS]);
 		d.sort_temp = at<uint32_t>(scratch, o.sort_temp); d.scan_temp = at<uint32_t>(scratch, o.scan_temp);
@@ -655,7 +657,7 @@ void fill_blend_args(rgs::BlendArgs& a, int P, int R, int width, int height, flo
 	a.capacity = (uint32_t)R;
 	if (R > 0) {
 		const BinningPhysical b = binning_physical((size_t)R);
-		const bool sorted_in_a = (((tile_key_bits(width, height) + 7) / 8) % 2) == 0;
+		const bool sorted_in_a = (rgs::sort_passes(tile_key_bits(width, height), rgs::kDigitBitsU32) % 2) == 0;
 		void* bin = const_cast<void*>(binning_ws);
 		a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
 		a.tile_keys = at<uint32_t>(binning_ws, sorted_in_a ? b.keys_a : b.keys_b);
@@ -746,14 +748,17 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 		d.filing.tanfovx = tan_fovx; d.filing.tanfovy = tan_fovy;
 		d.filing.W = width; d.filing.H = height;
 		d.keys = keys_a; d.values = vals_a; d.capacity = (uint32_t)R;
-		d.clear = temp; d.clear_words = rgs::sort_clear_words((size_t)R, end_bit);
+		d.clear = temp; d.clear_words = rgs::sort_clear_words((size_t)R, end_bit, rgs::kDigitBitsU32);
 		// it also clears the tile ranges (and the counters and totals behind them) and counts the digits of the tiles
 		// it writes, so the sort starts with its passes
 		uint32_t* tile_digits = at<uint32_t>(at<char>(c.geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).tile_digits);
 		d.tile_digits = tile_digits; d.end_bit = end_bit;
 		d.also_clear = reinterpret_cast<uint32_t*>(ranges); d.also_clear_words = clear_words;
 		dups.push_back(d);
-		sorts.push_back(rgs::SortJob<uint32_t>{keys_a, keys_b, vals_a, vals_b, (size_t)R, count, temp, nullptr, 0, tile_digits});
+		rgs::SortJob<uint32_t> sj = {};
+		sj.keys_in = keys_a; sj.keys_out = keys_b; sj.vals_in = vals_a; sj.vals_out = vals_b;
+		sj.n = (size_t)R; sj.n_device = count; sj.temp = temp; sj.digit_counts = tile_digits;
+		sorts.push_back(sj);
 		ranges_jobs.push_back(rgs::TileRangesJob{a.tile_keys, (size_t)R, count, ranges, a.sort_status, a.order_status, fault,
 		                                         at<uint4>(c.binning_ws, b.file_tail), tile_digits});
 		with_instances.push_back(k);
@@ -1161,7 +1166,7 @@ static int sort_pairs_u64(const char* who, uint64_t* keys_in, uint64_t* keys_out
 	rgs::launch_sort_pairs(keys_in, keys_out, vals_in, vals_out, n, end_bit, temp, s);
 	RGS_STAGE("sort_pairs");
 	rgs::launch_report_sort_status(temp, fault, device_fault, s);
-	if ((((end_bit + 7) / 8) % 2) == 0) {
+	if ((rgs::sort_passes(end_bit, rgs::kDigitBitsU64) % 2) == 0) {
 		// An even number of passes leaves the result in the input buffers; hand it over.
 		hipError_t e = hipMemcpyAsync(keys_out, keys_in, n * sizeof(uint64_t), hipMemcpyDeviceToDevice, s);
 		if (e == hipSuccess)

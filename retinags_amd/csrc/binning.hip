@@ -240,42 +240,74 @@ void launch_totals_from_block_sums(const TotalsJob* jobs, int count, hipStream_t
 
 // ---- depth order and key duplication (K/cuda_rasterizer_hgs/rasterizer_impl.cu:70-111) -------
 
-// (depth bits, index) pairs of the Gaussians that touch a tile, compacted in index order: the
+// Keys of the depth sort.  A rendered Gaussian's depth exceeds 0.2, so its bit pattern, which orders like the value,
+// lies above that of 0.125: the sort looks at bits - kDepthKeyBase, whose low kDepthKeyBits bits (three 9-bit digits)
+// tell every depth below 8192 apart.  Should a key have bits above those (a depth of 8192 or more), the kernel that
+// writes the keys says so in the sort's scratch and a fourth pass over the remaining bits runs; otherwise that pass
+// returns at once.  Either way the order is that of the full 32 bits.
+constexpr uint32_t kDepthKeyBase = 0x3E000000u;
+constexpr int kDepthKeyBits = 27;
+constexpr int kDepthPasses = 3;                 // of 9 bits each, plus the one on demand
+constexpr uint32_t kSortExtraPass = 2057;       // word of the sort scratch's header: non-zero = the fourth pass is needed
+
+// The values of the depth sort carry the Gaussian's tile count above its index, so that the pass that ends the sort
+// can write the counts in depth order itself (a gather of its own over the sorted indices cost as much as a pass).
+// A count that does not fit is stored as all ones and looked up by that pass.
+__host__ __device__ inline uint32_t depth_index_bits(uint32_t P)
+{
+	uint32_t bits = 1;
+	while (bits < 31u && (P - 1u) >> bits)
+		bits++;
+	return bits;
+}
+
+// (depth key, index and tile count) pairs of the Gaussians that touch a tile, compacted in index order: the
 // group of Gaussians [kScanGroup b, kScanGroup (b + 1)), four neighbouring ones per thread, is written
-// from visible_base[4 b] on (the bases are per 256 Gaussians).  Depths of rendered Gaussians are
-// positive floats (> 0.2), whose bit patterns order like the values.  A workgroup takes every
-// gridDim.x-th group and counts the four digits of the keys it writes on the way: at the end it adds
-// its counts to the digit histograms the sort of these pairs starts from (cleared beforehand), which
-// saves that sort its own pass over the keys.
+// from visible_base[4 b] on (the bases are per 256 Gaussians).  A workgroup takes every gridDim.x-th group and
+// counts the digits of the keys it writes on the way: at the end it adds its counts to the digit histograms
+// the sort of these pairs starts from (cleared beforehand), which saves that sort its own pass over the keys.
 __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
-	__shared__ uint32_t s_hist[4][256];
+	__shared__ uint32_t s_hist[kDepthPasses][512];
+	__shared__ uint32_t s_top[32];   // digit of the pass on demand; value 0 is not counted here but derived
 	const DepthOrderJob& j = batch.job[blockIdx.y];
 	const size_t P = (size_t)j.P;
 	if ((size_t)blockIdx.x * kScanGroup >= P)
 		return;
 	const float* __restrict__ depths = j.depths;
+	const uint32_t* __restrict__ tiles_touched = j.tiles_touched;
 	const uint32_t* __restrict__ visible_base = j.block_visible;
 	uint32_t* __restrict__ keys = j.keys_a;
-	uint32_t* __restrict__ values = j.order;
+	uint32_t* __restrict__ values = j.vals_a;
+	const uint32_t index_bits = depth_index_bits((uint32_t)j.P), cap = 0xFFFFFFFFu >> index_bits;
 #pragma unroll
-	for (int p = 0; p < 4; p++)
+	for (int p = 0; p < kDepthPasses; p++) {
 		s_hist[p][threadIdx.x] = 0u;
+		s_hist[p][256 + threadIdx.x] = 0u;
+	}
+	if (threadIdx.x < 32)
+		s_top[threadIdx.x] = 0u;
 	__syncthreads();
+	uint32_t written = 0;
 	for (size_t group = blockIdx.x; group * kScanGroup < P; group += gridDim.x) {
 		const size_t idx0 = group * kScanGroup + 4 * (size_t)threadIdx.x;
 		// the depth of a Gaussian that touches no tile is stored as 0, that of one that does exceeds 0.2: the
 		// depths alone say which ones are listed
 		float depth[4] = {0.f, 0.f, 0.f, 0.f};
+		uint32_t count[4] = {0u, 0u, 0u, 0u};
 		if (idx0 + 4 <= P) {
 			const float4 d4 = *reinterpret_cast<const float4*>(depths + idx0);
+			const uint4 c4 = *reinterpret_cast<const uint4*>(tiles_touched + idx0);
 			depth[0] = d4.x; depth[1] = d4.y; depth[2] = d4.z; depth[3] = d4.w;
+			count[0] = c4.x; count[1] = c4.y; count[2] = c4.z; count[3] = c4.w;
 		} else {
 #pragma unroll
 			for (int q = 0; q < 4; q++)
-				if (idx0 + q < P)
+				if (idx0 + q < P) {
 					depth[q] = depths[idx0 + q];
+					count[q] = tiles_touched[idx0 + q];
+				}
 		}
 		uint32_t mine = 0;
 #pragma unroll
@@ -283,31 +315,51 @@ __global__ __launch_bounds__(256) void depth_pairs_kernel(Batch<DepthOrderJob> b
 			mine += __float_as_uint(depth[q]) != 0u ? 1u : 0u;
 		uint32_t total;
 		uint32_t at = visible_base[4 * group] + block256_exclusive_scan_u32(mine, lds, total);
+		written += mine;
 #pragma unroll
 		for (int q = 0; q < 4; q++)
 			if (__float_as_uint(depth[q]) != 0u) {
-				const uint32_t key = __float_as_uint(depth[q]);
+				const uint32_t key = __float_as_uint(depth[q]) - kDepthKeyBase;
 				keys[at] = key;
-				values[at] = (uint32_t)(idx0 + q);
+				values[at] = (uint32_t)(idx0 + q) | (min(count[q], cap) << index_bits);
 				at++;
 #pragma unroll
-				for (int p = 0; p < 4; p++)
-					atomicAdd(&s_hist[p][(key >> (8 * p)) & 255u], 1u);
+				for (int p = 0; p < kDepthPasses; p++)
+					atomicAdd(&s_hist[p][(key >> (9 * p)) & 511u], 1u);
+				if (key >> kDepthKeyBits)
+					atomicAdd(&s_top[key >> kDepthKeyBits], 1u);
 			}
 	}
 	__syncthreads();
 #pragma unroll
-	for (int p = 0; p < 4; p++) {
-		const uint32_t c = s_hist[p][threadIdx.x];
+	for (int p = 0; p < kDepthPasses; p++)
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const uint32_t c = s_hist[p][256 * h + threadIdx.x];
+			if (c)
+				atomicAdd(&j.sort_temp[512 * p + 256 * h + threadIdx.x], c);
+		}
+	// the digit of the pass on demand: value 0 takes every key that was not counted under another value
+	uint32_t all_written;
+	(void)block256_exclusive_scan_u32(written, lds, all_written);
+	if (threadIdx.x < 32) {
+		uint32_t c = s_top[threadIdx.x];
+		if (threadIdx.x == 0) {
+			uint32_t others = 0;
+			for (int v = 1; v < 32; v++)
+				others += s_top[v];
+			c = all_written - others;
+			if (others)
+				atomicOr(&j.sort_temp[kSortExtraPass], 1u);
+		}
 		if (c)
-			atomicAdd(&j.sort_temp[p * 256 + threadIdx.x], c);
+			atomicAdd(&j.sort_temp[512 * kDepthPasses + threadIdx.x], c);
 	}
 }
 
-// out[k] = in[index[k]] for k below the count on the device, and the sum of every kScanGroup of them
-// (the first level of the scan that follows), four neighbouring k per thread.  `in` has in_size entries;
-// an index beyond it (only possible in what a sort that gave up left behind) reads the last entry instead.
-__global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> batch)
+// The sum of every kScanGroup of the tile counts in depth order (the first level of the scan that follows),
+// four neighbouring ones per thread; the count of them is on the device.
+__global__ __launch_bounds__(256) void order_totals_kernel(Batch<DepthOrderJob> batch)
 {
 	__shared__ uint32_t lds[8];
 	const DepthOrderJob& j = batch.job[blockIdx.y];
@@ -317,33 +369,22 @@ __global__ __launch_bounds__(256) void gather_u32_kernel(Batch<DepthOrderJob> ba
 	const size_t n = min((size_t)*j.visible_count, (size_t)j.P);
 	if ((size_t)blockIdx.x * kScanGroup >= n)
 		return;
-	const uint32_t* __restrict__ index = j.order;
-	const uint32_t* __restrict__ in = j.tiles_touched;
-	const uint32_t in_size = (uint32_t)j.P;
-	uint32_t* __restrict__ out = j.tiles_in_order;
-	uint32_t* __restrict__ block_totals = j.scan_temp;
+	const uint32_t* __restrict__ in = j.tiles_in_order;
 	const size_t k0 = (size_t)blockIdx.x * kScanGroup + 4 * (size_t)threadIdx.x;
-	uint32_t v[4] = {0u, 0u, 0u, 0u};
-	const bool whole = k0 + 4 <= n;
-	if (whole) {
-		const uint4 i4 = *reinterpret_cast<const uint4*>(index + k0);
-		v[0] = in[min(i4.x, in_size - 1u)];
-		v[1] = in[min(i4.y, in_size - 1u)];
-		v[2] = in[min(i4.z, in_size - 1u)];
-		v[3] = in[min(i4.w, in_size - 1u)];
-		*reinterpret_cast<uint4*>(out + k0) = uint4{v[0], v[1], v[2], v[3]};
+	uint32_t sum = 0;
+	if (k0 + 4 <= n) {
+		const uint4 v = *reinterpret_cast<const uint4*>(in + k0);
+		sum = v.x + v.y + v.z + v.w;
 	} else {
 #pragma unroll
 		for (int q = 0; q < 4; q++)
-			if (k0 + q < n) {
-				v[q] = in[min(index[k0 + q], in_size - 1u)];
-				out[k0 + q] = v[q];
-			}
+			if (k0 + q < n)
+				sum += in[k0 + q];
 	}
 	uint32_t total;
-	(void)block256_exclusive_scan_u32(v[0] + v[1] + v[2] + v[3], lds, total);
+	(void)block256_exclusive_scan_u32(sum, lds, total);
 	if (threadIdx.x == 0)
-		block_totals[blockIdx.x] = total;
+		j.scan_temp[blockIdx.x] = total;
 }
 
 // Instances of the Gaussians in depth order, tiles row by row like the reference, at the offsets
@@ -404,7 +445,7 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	const uint32_t limit = min(total, capacity);  // positions beyond the room the caller gave are dropped
 	if (blockIdx.x * (uint32_t)kDupPositions >= limit)
 		return;
-	const int passes = (job.end_bit + 7) / 8;
+	const int passes = sort_passes(job.end_bit, kDigitBitsU32);
 	for (int w = tid; w < kTileDigitWords; w += 256)
 		s_digits[w] = 0u;
 
@@ -497,8 +538,18 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 				continue;
 			const TileRect rc = tile_rect(r0[q].x, r0[q].y, __float_as_int(r3[q].z), gx, gy);
 			const uint32_t t = pos - first[q], w = max(rc.x1 - rc.x0, 1u);
-			const uint32_t row = t / w;
-			const int tx = (int)(rc.x0 + (t - row * w)), ty = (int)(rc.y0 + row);
+			// t / w through the reciprocal in single precision (both are below 2^24, so exact as floats; the quotient
+			// is off by one at most, which the remainder shows): a third of the instructions of the integer division
+			uint32_t row = (uint32_t)((float)t * __builtin_amdgcn_rcpf((float)w));
+			int col = (int)(t - row * w);
+			if (col < 0) {
+				row--;
+				col += (int)w;
+			} else if (col >= (int)w) {
+				row++;
+				col -= (int)w;
+			}
+			const int tx = (int)rc.x0 + col, ty = (int)(rc.y0 + row);
 			const uint32_t tile = (uint32_t)ty * (uint32_t)gx + (uint32_t)tx;
 			float2 nx;
 			float ny[8];
@@ -528,18 +579,18 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 		for (int q = 0; q < kPerThread; q++) {
 			const bool have = tile_of[q] != 0xFFFFFFFFu;
 			for (int p = 0; p < passes; p++) {
-				const int shift = sort_digit_shift(job.end_bit, p);
-				const int bits = sort_digit_bits(job.end_bit, p);
+				const int shift = sort_digit_shift(job.end_bit, p, kDigitBitsU32);
+				const int bits = sort_digit_bits(job.end_bit, p, kDigitBitsU32);
 				const uint32_t d = (tile_of[q] >> shift) & ((1u << bits) - 1u);
 				if (bits <= 2) {
 					// a digit of one or two bits: every lane would add to one of a few words, one after the other
 					for (uint32_t v = 0; v < (1u << bits); v++) {
 						const uint32_t c = (uint32_t)__popcll(lanes_where(have && d == v));
 						if (lane == 0 && c != 0u)
-							atomicAdd(&s_digits[256 * p + v], c);
+							atomicAdd(&s_digits[512 * p + v], c);
 					}
 				} else if (have) {
-					atomicAdd(&s_digits[256 * p + d], 1u);
+					atomicAdd(&s_digits[512 * p + d], 1u);
 				}
 			}
 		}
@@ -549,45 +600,10 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	}
 	}
 	__syncthreads();
-	for (int w = tid; w < 256 * passes; w += 256) {
+	for (int w = tid; w < 512 * passes; w += 256) {
 		const uint32_t c = s_digits[w];
 		if (c)
 			atomicAdd(&job.tile_digits[w], c);
-	}
-}
-
-void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)
-{
-	stage_mark("depth_order", s);
-	for (int at = 0; at < count; at += kMaxBatch) {
-		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
-		Batch<DepthOrderJob> b = {};
-		Batch<BlockScanJob> scan = {};
-		Batch<BlockInclusiveJob> inc = {};
-		SortJob<uint32_t> sorts[kMaxBatch];
-		int max_p = 0;
-		for (int k = 0; k < nj; k++)
-			max_p = jobs[at + k].P > max_p ? jobs[at + k].P : max_p;
-		const bool few_groups = ((size_t)max_p + kScanGroup - 1) / kScanGroup <= 4096;
-		for (int k = 0; k < nj; k++) {
-			const DepthOrderJob& j = jobs[at + k];
-			b.job[k] = j;
-			// 4 passes: the sorted pairs end up in the first buffer pair again
-			sorts[k] = SortJob<uint32_t>{j.keys_a, j.keys_b, j.order, j.vals_b, (size_t)j.P, j.visible_count, j.sort_temp, nullptr, 0};
-			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + kScanGroup - 1) / kScanGroup, j.visible_count, (uint32_t)kScanGroup, nullptr, nullptr,
-			                           nullptr, nullptr};
-			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order, j.dup_first,
-			                               (uint32_t)dup_first_words((size_t)j.P), few_groups ? 1u : 0u};
-		}
-		const dim3 grid((unsigned)((max_p + kScanGroup - 1) / kScanGroup), (unsigned)nj);
-		// few workgroups per job, each over many groups: every one ends with an atomic add per digit into its job's counts
-		const unsigned most = nj >= 8 ? 256u : 2048u / (unsigned)nj;
-		hipLaunchKernelGGL(depth_pairs_kernel, dim3(grid.x < most ? grid.x : most, (unsigned)nj), dim3(256), 0, s, b);
-		launch_sort_pairs_u32(sorts, nj, 32, true, true, nullptr, s);
-		hipLaunchKernelGGL(gather_u32_kernel, grid, dim3(256), 0, s, b);
-		if (!few_groups)
-			hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1, (unsigned)nj), dim3(1024), 0, s, scan);
-		hipLaunchKernelGGL(block_inclusive_scan_kernel<4>, grid, dim3(256), 0, s, inc);
 	}
 }
 
@@ -618,19 +634,22 @@ void launch_duplicate_with_keys(const DuplicateJob* jobs, int count, int grid_x,
 
 // ---- radix sort -------------------------------------------------------------------------------
 // Replaces cub::DeviceRadixSort::SortPairs at K/cuda_rasterizer_hgs/rasterizer_impl.cu:312-317:
-// a stable least-significant-digit sort of (u64 key, u32 value) on key bits [0, end_bit),
-// 8 bits per pass, in the one-sweep form: one kernel reads the keys once and builds the digit
-// histogram of every pass, then each pass is a single kernel whose blocks take tiles of
+// a stable least-significant-digit sort of (key, u32 value) pairs on key bits [0, end_bit), in the one-sweep form:
+// the digit histogram of every pass is built while the keys are written (or, for the stand-alone entry points, by one
+// kernel that reads them once), then each pass is a single kernel whose blocks take tiles of
 // kSortBlock pairs in arrival order, rank them in LDS, obtain their global digit offsets from
 // the blocks before them through a chained look-back over per-tile status words, and scatter.
 // Element order inside a tile is (wave, round, lane); ranking preserves it, and tiles are
-// ordered by their id, so every pass is stable.
+// ordered by their id, so every pass is stable.  A digit has up to kBits bits (template parameter): 9 for 32-bit
+// keys, which sorts 17 or 18 tile bits in two passes and 27 depth bits in three, 8 for 64-bit keys, whose tiles of
+// pairs fill the LDS.
 //
-// Scratch layout (u32 words):
-//   [0, 2048)      digit histograms of up to 8 passes (every block of a pass scans its 256 counts itself)
+// Scratch layout (u32 words), B = 2^kBits:
+//   [0, 2048)      digit histograms, B words per pass (every block of a pass scans its counts itself)
 //   [2048, 2056)   tile counter of each pass
 //   [2056]         status: non-zero if a look-back ever gave up waiting (never expected)
-//   [kSortHeader + pass * 256 * tiles + tile * 256 + digit]  look-back words
+//   [2057]         depth sort only: non-zero if its pass on demand is needed (kSortExtraPass)
+//   [kSortHeader + pass * B * tiles + tile * B + digit]  look-back words
 
 constexpr uint32_t kSortCounters = 2048;
 constexpr uint32_t kSortStatus = 2056;
@@ -656,10 +675,12 @@ __device__ __forceinline__ uint32_t digit_of(KeyT key, int shift, uint32_t mask)
 	return (uint32_t)(key >> shift) & mask;
 }
 
+// Only the stand-alone sort entry points run this (64-bit keys, digits of kDigitBitsU64 bits).
 template <typename KeyT>
 __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob<KeyT>> batch, int passes, int end_bit)
 {
-	__shared__ uint32_t s_hist[kSortMaxPasses][256];
+	constexpr int kMaxPasses = 8;
+	__shared__ uint32_t s_hist[kMaxPasses][256];
 	const SortJob<KeyT>& j = batch.job[blockIdx.y];
 	const KeyT* __restrict__ keys = j.keys_in;
 	size_t n = j.n;
@@ -672,7 +693,7 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 	if (n_device)
 		n = min(n, (size_t)*n_device);
 #pragma unroll
-	for (int p = 0; p < kSortMaxPasses; p++)
+	for (int p = 0; p < kMaxPasses; p++)
 		s_hist[p][threadIdx.x] = 0;
 	__syncthreads();
 	// four keys per thread and round, requested together: one key at a time the loop waits for
@@ -688,8 +709,8 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 			if (k + q * threads >= n)
 				break;
 			for (int p = 0; p < passes; p++) {
-				const int shift = sort_digit_shift(end_bit, p);
-				const int bits = sort_digit_bits(end_bit, p);
+				const int shift = sort_digit_shift(end_bit, p, kDigitBitsU64);
+				const int bits = sort_digit_bits(end_bit, p, kDigitBitsU64);
 				const uint32_t d = digit_of(key[q], shift, (1u << bits) - 1u);
 				if (bits <= 2) {
 					// a digit of one or two bits: every lane would add to one of a few words, one after the
@@ -713,10 +734,29 @@ __global__ __launch_bounds__(256) void sort_digit_histogram_kernel(Batch<SortJob
 	}
 }
 
-template <typename KeyT>
+// What a pass does with its output:
+//   kPassPlain        keys and values to the other buffer pair;
+//   kPassEndsUnless   depth sort, third pass: if the scratch says that a fourth pass is needed, as kPassPlain; otherwise the
+//                     sort ends here and the values are taken apart (Gaussian index to final_index, its tile count to
+//                     final_count, see SortJob);
+//   kPassOnDemand     depth sort, fourth pass: returns at once unless the scratch says it is needed; ends the sort.
+enum SortPassKind { kPassPlain = 0, kPassEndsUnless = 1, kPassOnDemand = 2 };
+
+// Per-wave digit counts fit 16 bits (a wavefront ranks kSortItems * 64 keys), and so does a digit's place inside a tile.
+template <int kBits>
+struct SortCounts {
+	uint16_t wave_hist[4][1 << kBits];  // per-wave digit counts, then exclusive prefix over waves
+	uint16_t digit_base[1 << kBits];    // exclusive prefix over digits within the tile
+	uint32_t global_base[1 << kBits];   // where this tile's run of each digit starts globally
+};
+
+template <typename KeyT, int kBits, int kKind>
 __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>> batch, int pass, int shift, uint32_t mask,
                                                              int spin_limit)
 {
+	constexpr int kBins = 1 << kBits;
+	constexpr int kOwn = kBins / 256;  // digit values a thread owns: kOwn * tid .. kOwn * tid + kOwn - 1
+	static_assert(kOwn == 1 || kOwn == 2, "256 threads own one or two digit values each");
 	const SortJob<KeyT>& j = batch.job[blockIdx.y];
 	// the passes ping-pong between the two buffer pairs, starting in -> out
 	const KeyT* __restrict__ keys_in = (pass & 1) ? j.keys_out : j.keys_in;
@@ -728,28 +768,38 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 	const size_t job_tiles = (j.n + kSortBlock - 1) / kSortBlock;
 	if (blockIdx.x >= job_tiles)
 		return;  // the launch is sized for the job with the most tiles
-	const uint32_t* __restrict__ digit_count = (j.digit_counts ? j.digit_counts : j.temp) + pass * 256;
-	uint32_t* __restrict__ lookback = j.temp + kSortHeader + (size_t)pass * 256 * job_tiles;
+	bool ends_here = false;
+	if (kKind != kPassPlain) {
+		const bool extra = j.temp[kSortExtraPass] != 0u;
+		if (kKind == kPassOnDemand && !extra)
+			return;
+		ends_here = kKind == kPassOnDemand || !extra;
+	}
+	const uint32_t* __restrict__ digit_count = (j.digit_counts ? j.digit_counts : j.temp) + pass * kBins;
+	uint32_t* __restrict__ lookback = j.temp + kSortHeader + (size_t)pass * kBins * job_tiles;
 	uint32_t* __restrict__ tile_counter = j.temp + kSortCounters + pass;
 	uint32_t* __restrict__ status = j.temp + kSortStatus;
 	__shared__ KeyT s_keys[kSortBlock];
 	__shared__ uint32_t s_vals[kSortBlock];
-	__shared__ uint32_t s_wave_hist[4][256];  // per-wave digit counts, then exclusive prefix over waves
-	__shared__ uint32_t s_digit_base[256];    // exclusive prefix over digits within the tile
-	__shared__ uint32_t s_global_base[256];   // where this tile's run of each digit starts globally
+	__shared__ SortCounts<kBits> sc;
 	__shared__ uint32_t s_scan[8];
 	__shared__ uint32_t s_tile;
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	// asked for before anything else: needed only after the look-back, by when it has long arrived
-	const uint32_t digit_total = digit_count[tid];
+	uint32_t digit_total[kOwn];
+#pragma unroll
+	for (int o = 0; o < kOwn; o++)
+		digit_total[o] = digit_count[kOwn * tid + o];
 	// Tiles are handed out in arrival order, so every tile a block waits for below belongs to
 	// a block that is already running.
 	if (tid == 0)
 		s_tile = atomicAdd(tile_counter, 1u);
 #pragma unroll
 	for (int w = 0; w < 4; w++)
-		s_wave_hist[w][tid] = 0;
+#pragma unroll
+		for (int o = 0; o < kOwn; o++)
+			sc.wave_hist[w][kOwn * tid + o] = 0;
 	__syncthreads();
 	const uint32_t tile = s_tile;
 	const size_t block_base = (size_t)tile * kSortBlock;
@@ -775,11 +825,11 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 #pragma unroll
 	for (int i = 0; i < kSortItems; i++) {
 		const size_t k = wave_base + (size_t)i * 64 + lane;
-		// Padding elements rank as digit 255 after every real element, so they never disturb one.
-		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : 255u;
+		// Padding elements rank as the last digit value after every real element, so they never disturb one.
+		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : (uint32_t)(kBins - 1);
 		uint64_t same = ~0ull;
 #pragma unroll
-		for (int b = 0; b < 8; b++) {
+		for (int b = 0; b < kBits; b++) {
 			const bool bit = (d >> b) & 1u;
 			const uint64_t vote = lanes_where(bit);
 			same &= bit ? vote : ~vote;
@@ -789,8 +839,8 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 		const int leader = __ffsll((unsigned long long)same) - 1;
 		uint32_t prior = 0;
 		if (lane == leader) {
-			prior = s_wave_hist[wave][d];
-			s_wave_hist[wave][d] = prior + count;
+			prior = sc.wave_hist[wave][d];
+			sc.wave_hist[wave][d] = (uint16_t)(prior + count);
 		}
 		prior = __shfl(prior, leader);
 		rank[i] = prior + below;
@@ -798,29 +848,53 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 	}
 	__syncthreads();
 
-	// Thread d owns digit d: prefix over the 4 waves, publish the tile's count.
+	// A thread owns kOwn neighbouring digit values: prefix over the 4 waves, publish the tile's counts.
 	const size_t remaining = n - block_base;
 	const uint32_t valid = remaining < (size_t)kSortBlock ? (uint32_t)remaining : (uint32_t)kSortBlock;
-	uint32_t* const my_word = lookback + (size_t)tile * 256 + tid;
-	uint32_t count, digit_start;
+	uint32_t* const my_word = lookback + (size_t)tile * kBins + kOwn * tid;
+	uint32_t count[kOwn], digit_start[kOwn];
 	{
-		const uint32_t c0 = s_wave_hist[0][tid], c1 = s_wave_hist[1][tid], c2 = s_wave_hist[2][tid],
-		               c3 = s_wave_hist[3][tid];
-		s_wave_hist[0][tid] = 0;
-		s_wave_hist[1][tid] = c0;
-		s_wave_hist[2][tid] = c0 + c1;
-		s_wave_hist[3][tid] = c0 + c1 + c2;
-		count = c0 + c1 + c2 + c3;
+		uint32_t mine = 0;
+#pragma unroll
+		for (int o = 0; o < kOwn; o++) {
+			const int d = kOwn * tid + o;
+			const uint32_t c0 = sc.wave_hist[0][d], c1 = sc.wave_hist[1][d], c2 = sc.wave_hist[2][d], c3 = sc.wave_hist[3][d];
+			sc.wave_hist[0][d] = 0;
+			sc.wave_hist[1][d] = (uint16_t)c0;
+			sc.wave_hist[2][d] = (uint16_t)(c0 + c1);
+			sc.wave_hist[3][d] = (uint16_t)(c0 + c1 + c2);
+			count[o] = c0 + c1 + c2 + c3;
+			mine += count[o];
+		}
 		uint32_t total;
-		const uint32_t ex = block256_exclusive_scan_u32(count, s_scan, total);
-		s_digit_base[tid] = ex;
+		uint32_t ex = block256_exclusive_scan_u32(mine, s_scan, total);
+#pragma unroll
+		for (int o = 0; o < kOwn; o++) {
+			sc.digit_base[kOwn * tid + o] = (uint16_t)ex;
+			ex += count[o];
+		}
 		if (tid == 255)
-			count -= (uint32_t)kSortBlock - valid;  // padding is not published
-		__hip_atomic_store(my_word, count | (tile == 0 ? kFlagInclusive : kFlagAggregate), __ATOMIC_RELAXED,
-		                   __HIP_MEMORY_SCOPE_AGENT);
+			count[kOwn - 1] -= (uint32_t)kSortBlock - valid;  // padding is not published
+		const uint32_t flag = tile == 0 ? kFlagInclusive : kFlagAggregate;
+		if (kOwn == 1) {
+			__hip_atomic_store(my_word, count[0] | flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		} else {
+			// both counts in one 8-byte store: a reader sees the pair published or not, never one of the two
+			__hip_atomic_store(reinterpret_cast<uint64_t*>(my_word),
+			                   (uint64_t)(count[0] | flag) | ((uint64_t)(count[kOwn - 1] | flag) << 32), __ATOMIC_RELAXED,
+			                   __HIP_MEMORY_SCOPE_AGENT);
+		}
 		// where the digit's run starts in the whole array: the exclusive scan of the digit counts
-		uint32_t all;
-		digit_start = block256_exclusive_scan_u32(digit_total, s_scan, all);
+		uint32_t all, totals = 0;
+#pragma unroll
+		for (int o = 0; o < kOwn; o++)
+			totals += digit_total[o];
+		uint32_t start = block256_exclusive_scan_u32(totals, s_scan, all);
+#pragma unroll
+		for (int o = 0; o < kOwn; o++) {
+			digit_start[o] = start;
+			start += digit_total[o];
+		}
 	}
 
 	// The tile's pairs in digit order, through LDS.  None of this needs the tiles before this one: by the time
@@ -828,8 +902,8 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 #pragma unroll
 	for (int i = 0; i < kSortItems; i++) {
 		const size_t k = wave_base + (size_t)i * 64 + lane;
-		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : 255u;
-		const uint32_t pos = s_digit_base[d] + s_wave_hist[wave][d] + rank[i];
+		const uint32_t d = (k < n) ? digit_of(key[i], shift, mask) : (uint32_t)(kBins - 1);
+		const uint32_t pos = (uint32_t)sc.digit_base[d] + (uint32_t)sc.wave_hist[wave][d] + rank[i];
 		s_keys[pos] = key[i];
 		s_vals[pos] = val[i];
 	}
@@ -845,29 +919,48 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 		out_val[i] = s_vals[q];
 	}
 
-	// Look back: the pairs of this digit in all earlier tiles.
+	// Look back: the pairs of this thread's digit values in all earlier tiles.
 	{
-		uint32_t exclusive = 0;
+		uint32_t exclusive[kOwn];
+#pragma unroll
+		for (int o = 0; o < kOwn; o++)
+			exclusive[o] = 0;
 		if (tile != 0) {
 			// Words of the tiles below t are still to be added.  Up to kLookBatch of them are requested
 			// together: walked one load at a time, the chain of tiles and not memory sets the pace of a pass.
 			uint32_t t = tile;
 			bool gave_up = spin_limit < 0, done = false;
 			while (!gave_up && !done) {
-				uint32_t v[kLookBatch];
+				uint32_t v[kLookBatch][kOwn];
 #pragma unroll
-				for (int q = 0; q < kLookBatch; q++)
-					v[q] = (uint32_t)q < t ? __hip_atomic_load(lookback + (size_t)(t - 1u - (uint32_t)q) * 256 + tid, __ATOMIC_RELAXED,
-					                                           __HIP_MEMORY_SCOPE_AGENT)
-					                       : kFlagInclusive;  // below the first tile there is nothing
+				for (int q = 0; q < kLookBatch; q++) {
+					const uint32_t* word = lookback + (size_t)(t - 1u - (uint32_t)q) * kBins + kOwn * tid;
+					if ((uint32_t)q < t) {
+						if (kOwn == 1) {
+							v[q][0] = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+						} else {
+							const uint64_t both = __hip_atomic_load(reinterpret_cast<const uint64_t*>(word), __ATOMIC_RELAXED,
+							                                        __HIP_MEMORY_SCOPE_AGENT);
+							v[q][0] = (uint32_t)both;
+							v[q][kOwn - 1] = (uint32_t)(both >> 32);
+						}
+					} else {
+#pragma unroll
+						for (int o = 0; o < kOwn; o++)
+							v[q][o] = kFlagInclusive;  // below the first tile there is nothing
+					}
+				}
 				uint32_t used = 0;
 #pragma unroll
 				for (int q = 0; q < kLookBatch; q++) {
-					// a word counts once every nearer one has been published and none of them closed the sum
-					if (!done && used == (uint32_t)q && (v[q] >> 30) != 0u) {
-						exclusive += v[q] & kValueMask;
+					// a word counts once every nearer one has been published and none of them closed the sum (a tile's
+					// words are published together and carry the same flag, so the first tells for all)
+					if (!done && used == (uint32_t)q && (v[q][0] >> 30) != 0u) {
+#pragma unroll
+						for (int o = 0; o < kOwn; o++)
+							exclusive[o] += v[q][o] & kValueMask;
 						used = (uint32_t)q + 1u;
-						done = (v[q] & kFlagInclusive) != 0u;
+						done = (v[q][0] & kFlagInclusive) != 0u;
 					}
 				}
 				t -= used < t ? used : t;
@@ -875,7 +968,7 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 					done = true;
 				if (!done && used < (uint32_t)kLookBatch) {
 					// tile t - 1 has not published yet: wait for its word, then look again from there
-					const uint32_t* word = lookback + (size_t)(t - 1u) * 256 + tid;
+					const uint32_t* word = lookback + (size_t)(t - 1u) * kBins + kOwn * tid;
 					uint32_t w = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 					for (int spins = 0; (w >> 30) == 0u; spins++) {
 						// give up after a bounded wait, or as soon as any other look-back has
@@ -894,10 +987,19 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 				atomicOr(status, 1u);
 			// On the (never expected) give-up path `exclusive` is too small, which keeps every
 			// scatter address inside the array; the status word tells the consumer to discard it.
-			__hip_atomic_store(my_word, ((exclusive + count) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
-			                   __HIP_MEMORY_SCOPE_AGENT);
+			if (kOwn == 1) {
+				__hip_atomic_store(my_word, ((exclusive[0] + count[0]) & kValueMask) | kFlagInclusive, __ATOMIC_RELAXED,
+				                   __HIP_MEMORY_SCOPE_AGENT);
+			} else {
+				__hip_atomic_store(reinterpret_cast<uint64_t*>(my_word),
+				                   (uint64_t)(((exclusive[0] + count[0]) & kValueMask) | kFlagInclusive) |
+				                       ((uint64_t)(((exclusive[kOwn - 1] + count[kOwn - 1]) & kValueMask) | kFlagInclusive) << 32),
+				                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
 		}
-		s_global_base[tid] = digit_start + exclusive;
+#pragma unroll
+		for (int o = 0; o < kOwn; o++)
+			sc.global_base[kOwn * tid + o] = digit_start[o] + exclusive[o];
 	}
 	__syncthreads();
 
@@ -906,7 +1008,24 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 	for (int i = 0; i < kSortItems; i++) {
 		const uint32_t p = (uint32_t)i * 256 + tid;
 		const uint32_t d = digit_of(out_key[i], shift, mask);
-		out_at[i] = p < valid ? (size_t)s_global_base[d] + (p - s_digit_base[d]) : n;
+		out_at[i] = p < valid ? (size_t)sc.global_base[d] + (p - (uint32_t)sc.digit_base[d]) : n;
+	}
+	if (kKind != kPassPlain && ends_here) {
+		// the sort ends here: a value's index and tile count go to arrays of their own (a count stored as all ones did
+		// not fit and is looked up; an index that a sort which gave up left behind may be anything and is clamped)
+		const uint32_t index_bits = j.index_bits, cap = 0xFFFFFFFFu >> index_bits, index_mask = (1u << index_bits) - 1u;
+#pragma unroll
+		for (int i = 0; i < kSortItems; i++) {
+			if (out_at[i] < n) {
+				const uint32_t index = out_val[i] & index_mask;
+				uint32_t c = out_val[i] >> index_bits;
+				if (c == cap)
+					c = j.count_of[min(index, j.in_size - 1u)];
+				j.final_index[out_at[i]] = index;
+				j.final_count[out_at[i]] = c;
+			}
+		}
+		return;
 	}
 #pragma unroll
 	for (int i = 0; i < kSortItems; i++) {
@@ -927,17 +1046,23 @@ const uint32_t* sort_status_word(const uint32_t* temp)
 	return temp + kSortStatus;
 }
 
-size_t sort_clear_words(size_t n, int end_bit)
+size_t sort_clear_words(size_t n, int end_bit, int max_bits)
 {
 	const size_t tiles = (n + kSortBlock - 1) / kSortBlock;
-	return kSortHeader + (size_t)((end_bit + 7) / 8) * 256 * tiles;
+	return kSortHeader + (size_t)sort_passes(end_bit, max_bits) * ((size_t)1 << max_bits) * tiles;
 }
 
-template <typename KeyT>
+size_t depth_sort_clear_words(size_t n)
+{
+	const size_t tiles = (n + kSortBlock - 1) / kSortBlock;
+	return kSortHeader + (size_t)(kDepthPasses + 1) * 512 * tiles;
+}
+
+template <typename KeyT, int kBits>
 static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done, bool mark_stages,
                        hipStream_t s)
 {
-	const int passes = (end_bit + 7) / 8;
+	const int passes = sort_passes(end_bit, kBits);
 	for (int at = 0; at < count; at += kMaxBatch) {
 		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
 		Batch<SortJob<KeyT>> b = {};
@@ -951,7 +1076,7 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 			const uint32_t tiles = (uint32_t)((j.n + kSortBlock - 1) / kSortBlock);
 			max_tiles = tiles > max_tiles ? tiles : max_tiles;
 			if (!temp_cleared)
-				launch_fill_u32(j.temp, 0u, sort_clear_words(j.n, end_bit), s);
+				launch_fill_u32(j.temp, 0u, sort_clear_words(j.n, end_bit, kBits), s);
 		}
 		if (live == 0)
 			continue;
@@ -961,16 +1086,18 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 		// job read the keys as fast as thousands would, and queue far fewer adds on the same words
 		const uint32_t most_blocks = live >= 8 ? 256u : 2048u / (uint32_t)live;
 		const uint32_t hist_blocks = max_tiles < most_blocks ? max_tiles : most_blocks;
-		if (!histograms_done)
-			hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
+		if (!histograms_done) {
+			if constexpr (kBits == kDigitBitsU64)
+				hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
+		}
 		for (int p = 0; p < passes; p++) {
-			const int shift = sort_digit_shift(end_bit, p);
-			const int bits = sort_digit_bits(end_bit, p);
+			const int shift = sort_digit_shift(end_bit, p, kBits);
+			const int bits = sort_digit_bits(end_bit, p, kBits);
 			const uint32_t mask = (1u << bits) - 1u;
 			if (mark_stages)
 				stage_mark("sort_onesweep", s);
-			hipLaunchKernelGGL(sort_onesweep_kernel<KeyT>, dim3(max_tiles, (unsigned)live), dim3(256), 0, s, b, p, shift, mask,
-			                   g_lookback_spin_limit.load());
+			hipLaunchKernelGGL((sort_onesweep_kernel<KeyT, kBits, kPassPlain>), dim3(max_tiles, (unsigned)live), dim3(256), 0, s, b, p, shift,
+			                   mask, g_lookback_spin_limit.load());
 		}
 	}
 }
@@ -978,14 +1105,61 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
                        int end_bit, uint32_t* temp, hipStream_t s)
 {
-	const SortJob<uint64_t> job = {keys_in, keys_out, vals_in, vals_out, n, nullptr, temp, nullptr, 0};
-	sort_pairs<uint64_t>(&job, 1, end_bit, false, false, true, s);
+	SortJob<uint64_t> job = {};
+	job.keys_in = keys_in; job.keys_out = keys_out; job.vals_in = vals_in; job.vals_out = vals_out;
+	job.n = n; job.temp = temp;
+	sort_pairs<uint64_t, kDigitBitsU64>(&job, 1, end_bit, false, false, true, s);
 }
 
+// The digit counts must come from the kernel that wrote the keys (histograms_done): nothing here reads 32-bit keys for them.
 void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done,
                            const char* stage, hipStream_t s)
 {
-	sort_pairs<uint32_t>(jobs, count, end_bit, temp_cleared, histograms_done, stage != nullptr, s);
+	sort_pairs<uint32_t, kDigitBitsU32>(jobs, count, end_bit, temp_cleared, histograms_done, stage != nullptr, s);
+}
+
+void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)
+{
+	stage_mark("depth_order", s);
+	for (int at = 0; at < count; at += kMaxBatch) {
+		const int nj = count - at < kMaxBatch ? count - at : kMaxBatch;
+		Batch<DepthOrderJob> b = {};
+		Batch<BlockScanJob> scan = {};
+		Batch<BlockInclusiveJob> inc = {};
+		Batch<SortJob<uint32_t>> sorts = {};
+		int max_p = 0;
+		for (int k = 0; k < nj; k++)
+			max_p = jobs[at + k].P > max_p ? jobs[at + k].P : max_p;
+		const bool few_groups = ((size_t)max_p + kScanGroup - 1) / kScanGroup <= 4096;
+		for (int k = 0; k < nj; k++) {
+			const DepthOrderJob& j = jobs[at + k];
+			b.job[k] = j;
+			SortJob<uint32_t>& sj = sorts.job[k];
+			sj.keys_in = j.keys_a; sj.keys_out = j.keys_b; sj.vals_in = j.vals_a; sj.vals_out = j.vals_b;
+			sj.n = (size_t)j.P; sj.n_device = j.visible_count; sj.temp = j.sort_temp;
+			sj.final_index = j.order; sj.final_count = j.tiles_in_order; sj.count_of = j.tiles_touched;
+			sj.index_bits = depth_index_bits((uint32_t)j.P); sj.in_size = (uint32_t)j.P;
+			scan.job[k] = BlockScanJob{j.scan_temp, ((size_t)j.P + kScanGroup - 1) / kScanGroup, j.visible_count, (uint32_t)kScanGroup, nullptr, nullptr,
+			                           nullptr, nullptr};
+			inc.job[k] = BlockInclusiveJob{j.tiles_in_order, j.scan_temp, (size_t)j.P, j.visible_count, j.offsets_in_order, j.dup_first,
+			                               (uint32_t)dup_first_words((size_t)j.P), few_groups ? 1u : 0u};
+		}
+		const dim3 grid((unsigned)((max_p + kScanGroup - 1) / kScanGroup), (unsigned)nj);
+		// few workgroups per job, each over many groups: every one ends with an atomic add per digit into its job's counts
+		const unsigned most = nj >= 8 ? 256u : 2048u / (unsigned)nj;
+		hipLaunchKernelGGL(depth_pairs_kernel, dim3(grid.x < most ? grid.x : most, (unsigned)nj), dim3(256), 0, s, b);
+		// three passes of nine bits (a -> b -> a -> the order and the tile counts in that order), and the pass on demand
+		const dim3 tiles((unsigned)((max_p + kSortBlock - 1) / kSortBlock), (unsigned)nj);
+		const int spin = g_lookback_spin_limit.load();
+		hipLaunchKernelGGL((sort_onesweep_kernel<uint32_t, 9, kPassPlain>), tiles, dim3(256), 0, s, sorts, 0, 0, 511u, spin);
+		hipLaunchKernelGGL((sort_onesweep_kernel<uint32_t, 9, kPassPlain>), tiles, dim3(256), 0, s, sorts, 1, 9, 511u, spin);
+		hipLaunchKernelGGL((sort_onesweep_kernel<uint32_t, 9, kPassEndsUnless>), tiles, dim3(256), 0, s, sorts, 2, 18, 511u, spin);
+		hipLaunchKernelGGL((sort_onesweep_kernel<uint32_t, 9, kPassOnDemand>), tiles, dim3(256), 0, s, sorts, 3, kDepthKeyBits, 31u, spin);
+		hipLaunchKernelGGL(order_totals_kernel, grid, dim3(256), 0, s, b);
+		if (!few_groups)
+			hipLaunchKernelGGL(single_block_exclusive_scan_kernel, dim3(1, (unsigned)nj), dim3(1024), 0, s, scan);
+		hipLaunchKernelGGL(block_inclusive_scan_kernel<4>, grid, dim3(256), 0, s, inc);
+	}
 }
 
 // Sets n words to v, 16 bytes per store where the address allows; a capped grid walks the array.

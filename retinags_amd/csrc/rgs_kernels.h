@@ -282,17 +282,24 @@ void launch_preprocess_forward(const PreprocessArgs* jobs, int count, hipStream_
 void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, int count, hipStream_t s);
 
 // binning.hip
-// A sort on the lowest end_bit bits of its keys takes ceil(end_bit / 8) passes; the bits are shared out evenly
-// between them, the wider digits first (13 bits: 7 then 6, not 8 then 5: the fewer values a digit has, the longer
+// A sort on the lowest end_bit bits of its keys takes ceil(end_bit / max_bits) passes, max_bits being the widest digit
+// its kernel handles (kDigitBitsU32 for 32-bit keys, kDigitBitsU64 for 64-bit ones); the bits are shared out evenly
+// between the passes, the wider digits first (13 bits: 7 then 6, not 9 then 4: the fewer values a digit has, the longer
 // the runs of neighbouring keys a pass writes).
-__host__ __device__ inline int sort_digit_bits(int end_bit, int p)
+constexpr int kDigitBitsU32 = 9;   // 512 digit values: the 17 tile bits of a 5185x3359 image in two passes, 27 depth bits in three
+constexpr int kDigitBitsU64 = 8;
+__host__ __device__ inline int sort_passes(int end_bit, int max_bits)
 {
-	const int n = (end_bit + 7) / 8;
+	return (end_bit + max_bits - 1) / max_bits;
+}
+__host__ __device__ inline int sort_digit_bits(int end_bit, int p, int max_bits)
+{
+	const int n = sort_passes(end_bit, max_bits);
 	return end_bit / n + (p < end_bit % n ? 1 : 0);
 }
-__host__ __device__ inline int sort_digit_shift(int end_bit, int p)
+__host__ __device__ inline int sort_digit_shift(int end_bit, int p, int max_bits)
 {
-	const int n = (end_bit + 7) / 8;
+	const int n = sort_passes(end_bit, max_bits);
 	return p * (end_bit / n) + (p < end_bit % n ? p : end_bit % n);
 }
 constexpr int kSortItems = 16;                    // keys per thread in one sort block
@@ -326,6 +333,7 @@ struct DepthOrderJob {
 	uint32_t* visible_count;
 	uint32_t* keys_a;
 	uint32_t* keys_b;
+	uint32_t* vals_a;
 	uint32_t* order;
 	uint32_t* vals_b;
 	uint32_t* tiles_in_order;
@@ -347,9 +355,10 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 constexpr int kDupPositions = 256;
 constexpr size_t dup_first_words(size_t P) { return P / 16 + 2; }
 // The key duplication also counts the digits of the tiles it writes, which is what the sort of its keys starts
-// from: counts[256 p + d] = keys whose tile bits [8 p, 8 p + 8) are d, in kTileDigitWords words that are zero when it
-// starts (the depth order leaves them so, and so does the tile-range kernel, the last to run after they were read).
-constexpr int kTileDigitWords = 3 * 256;  // tiles have at most 24 bits
+// from: counts[512 p + d] = keys whose digit p of the tile bits (sort_digit_shift / sort_digit_bits with kDigitBitsU32)
+// is d, in kTileDigitWords words that are zero when it starts (the depth order leaves them so, and so does the
+// tile-range kernel, the last to run after they were read).
+constexpr int kTileDigitWords = 3 * 512;  // tiles have at most 24 bits: three passes at most
 struct DuplicateJob {
 	int P;
 	const uint32_t* visible_count;
@@ -369,15 +378,19 @@ struct DuplicateJob {
 	size_t clear_words;
 };
 void launch_duplicate_with_keys(const DuplicateJob* jobs, int count, int grid_x, int grid_y, hipStream_t s);
-size_t sort_clear_words(size_t n, int end_bit);    // words of the sort scratch that must be zero before a sort
-constexpr int kSortMaxPasses = 8;                 // radix passes the scratch has room for (64-bit keys)
+// words of the sort scratch that must be zero before a sort on end_bit bits with digits of at most max_bits bits
+size_t sort_clear_words(size_t n, int end_bit, int max_bits);
+size_t depth_sort_clear_words(size_t n);          // the same for the depth sort of launch_depth_order
+// The scratch has room for 2048 digit counts and as many look-back words per tile of kSortBlock pairs: 8 passes of 256
+// digit values (64-bit keys) or 4 passes of 512 (32-bit keys).
+constexpr uint32_t kSortScratchPerTile = 2048;
 constexpr uint32_t kSortHeader = 2112;            // words ahead of the look-back words: histograms, counters, status
 constexpr size_t sort_temp_words_for(size_t n)
 {
-	return kSortHeader + (size_t)kSortMaxPasses * 256 * ((n + kSortBlock - 1) / kSortBlock > 0 ? (n + kSortBlock - 1) / kSortBlock : 1);
+	return kSortHeader + (size_t)kSortScratchPerTile * ((n + kSortBlock - 1) / kSortBlock > 0 ? (n + kSortBlock - 1) / kSortBlock : 1);
 }
 size_t sort_temp_words(size_t n);                 // u32 words of scratch for launch_sort_pairs* (= sort_temp_words_for)
-// Stable LSD radix sort on key bits [0, end_bit), ceil(end_bit/8) passes that ping-pong between
+// Stable LSD radix sort on key bits [0, end_bit), sort_passes(end_bit, kDigitBitsU64) passes that ping-pong between
 // the two buffer pairs starting in -> out: an odd pass count leaves the result in
 // keys_out/vals_out, an even one in keys_in/vals_in.
 void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out, size_t n,
@@ -397,11 +410,19 @@ struct SortJob {
 	uint32_t* also_clear;
 	size_t also_clear_words;
 	const uint32_t* digit_counts;  // null: the counts are at the start of temp
+	// Only for the passes that end the depth sort (launch_depth_order): the values are a Gaussian's index in the low
+	// index_bits bits and above them its tile count (all ones: too large to fit, look it up in count_of); the last pass
+	// writes index and count apart, to final_index and final_count, instead of keys and values.
+	uint32_t* final_index;
+	uint32_t* final_count;
+	const uint32_t* count_of;      // tile count of every Gaussian, in_size of them
+	uint32_t index_bits, in_size;
 };
-// The same for 32-bit keys, every job in one launch per kernel; with a null `stage` its kernels are not marked for
-// the timing aid.  temp_cleared: the caller has cleared sort_clear_words(n, end_bit) words of every temp already.
-// histograms_done: the kernel that wrote keys_in has also added every key's digits to the counts at the start of temp
-// (temp[256 p + d] = keys whose bits [8 p, 8 p + 8) are d), so the sort need not read the keys for that.
+// The same for 32-bit keys (sort_passes(end_bit, kDigitBitsU32) passes), every job in one launch per kernel; with a null
+// `stage` its kernels are not marked for the timing aid.  temp_cleared: the caller has cleared
+// sort_clear_words(n, end_bit, kDigitBitsU32) words of every temp already.  histograms_done: the kernel that wrote keys_in
+// has also added every key's digits to the counts (counts[512 p + d] = keys whose digit p is d), so the sort need not
+// read the keys for that.
 void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done,
                            const char* stage, hipStream_t s);
 const uint32_t* sort_status_word(const uint32_t* temp);  // non-zero after a failed sort (never expected)

@@ -96,8 +96,11 @@ __device__ __forceinline__ StripTests prepare_strip_tests(const FiledGeometry& e
 	const float floor = e.geom.z, w = e.geom.w;
 	t.a = e.conic.x; t.b = e.conic.y; t.c = e.conic.z;
 	t.limit = -2.f * floor;
-	t.ra = 1.f / t.a;
-	t.rc = 1.f / t.c;
+	// hardware reciprocals and square roots (one unit in the last place) here and below: these values only place the
+	// bounds of conservative tests, whose margins are three orders of magnitude wider, and a correctly rounded division
+	// or square root costs ten instructions where these cost one
+	t.ra = __builtin_amdgcn_rcpf(t.a);
+	t.rc = __builtin_amdgcn_rcpf(t.c);
 	const bool ellipse = (t.a > 0.f) && (t.c > 0.f) && (t.a * t.c - t.b * t.b > 0.f);
 	t.flags = (ellipse ? 1u : 0u) | ((floor > 0.f) ? 2u : 0u);  // floor > 0: even power = 0 gives alpha < 1/255
 	t.pad = 0u;
@@ -166,12 +169,13 @@ __device__ __forceinline__ uint32_t strips_filed_for(const StripTests& t, float 
 		const float largest = a * fmaxf(dxl * dxl, dxh * dxh) + c * fmaxf(dy_first * dy_first, dy_last * dy_last);
 		const float limit = t.limit + (1e-3f + 1e-4f * t.limit + 1e-5f * largest);
 		const float det = a * c - b * b;
-		const float rdet = 1.f / det;
-		const float X = sqrtf(c * limit * rdet), Y = sqrtf(a * limit * rdet);
+		const float rdet = __builtin_amdgcn_rcpf(det);
+		const float X = __builtin_amdgcn_sqrtf(c * limit * rdet), Y = __builtin_amdgcn_sqrtf(a * limit * rdet);
 		const float dl = fmaxf(dxl, -X), dh = fminf(dxh, X);
 		if (dl > dh)
 			return 0u;  // the columns lie beside the ellipse
-		const float sl = sqrtf(fmaxf(c * limit - det * dl * dl, 0.f)), sh = sqrtf(fmaxf(c * limit - det * dh * dh, 0.f));
+		const float sl = __builtin_amdgcn_sqrtf(fmaxf(c * limit - det * dl * dl, 0.f)),
+		            sh = __builtin_amdgcn_sqrtf(fmaxf(c * limit - det * dh * dh, 0.f));
 		const float at_top = -b * Y * t.ra;  // dx of the ellipse's highest dy; that of its lowest is -at_top
 		const float top = fmaxf((-b * dl + sl) * t.rc, (-b * dh + sh) * t.rc);
 		const float bottom = fminf((-b * dl - sl) * t.rc, (-b * dh - sh) * t.rc);

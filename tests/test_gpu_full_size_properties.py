@@ -110,7 +110,9 @@ def _frame_setup_on_device(name):
     return cam, cfg, subs, rel, part
 
 
-FRAME_GRAD_TOL = 1e-5   # relative L2 between the two paths' gradients: same terms, another order of the atomic adds
+# Relative L2 between the two paths' gradients: the same terms added atomically in another order (a frame rendered twice
+# the same way differs from itself as much: a few 1e-5 at most where a Gaussian's sum has thousands of terms of both signs)
+FRAME_GRAD_TOL = 1e-4
 
 
 def _frame_against_calls_per_submodel(cam, subs, rel, bg, with_backward, seed, grads_on_layers=False):
@@ -375,9 +377,8 @@ def test_garden_full_size_against_checker():
 
 
 def test_high_resolution_full_size():
-    """Config C2 at full size: the 5.6 M Gaussians of C1 at 5185x3359 (68 250 tiles: 17-bit tile keys, three
-    radix passes, an odd count, so the sorted lists end in the other buffer pair than at C1), about 71 M
-    instances.  Structure and determinism of every submodel, the compositing identity, SH linearity, the frame through
+    """Config C2 at full size: the 5.6 M Gaussians of C1 at 5185x3359 (68 250 tiles: 17-bit tile keys, sorted in two
+    passes of 9 and 8 bits where C1's 13 bits take 7 and 6), about 71 M instances.  Structure and determinism of every submodel, the compositing identity, SH linearity, the frame through
     rasterize_frame against one call per submodel, and the submodel with the most instances against the CPU checker."""
     from helpers import DECISION_MARGIN, GRAD_TOL, IMAGE_TOL, np32, orc, rel_l2
     from retinags_amd.harness import partition, pipeline

@@ -146,6 +146,28 @@ def test_cube_half_box_clips():
     assert st.counters[3] < st.counters[2]  # some samples were clipped by the box
 
 
+def test_depths_beyond_the_range_of_three_sort_passes():
+    """The depth sort looks at 27 bits of the depth's bit pattern in three passes, which tells depths below 8192
+    apart; a scene with Gaussians beyond that makes it run its fourth pass over the remaining bits.  Half of the cube
+    is pushed out along the viewing direction, scaled so that it covers the same pixels, to depths of 12 000 to 20 000
+    (among them keys that differ only above bit 27 from keys of the near half); the depth order, the lists and the images
+    must still be the checker's bit for bit / within tolerance, with the near half alone, the far half alone and both."""
+    from retinags_amd import _capi
+    scene, cam, _ = scenes.make_config("C0", shrink=30, resolution_scale=0.25)
+    n = scene["xyz"].shape[0]
+    far = torch.arange(n) % 2 == 1
+    eye = cam.camera_center.clone()
+    for which in ("both", "far", "near"):
+        moved = {k: v.clone() for k, v in scene.items()}
+        pick = far if which == "both" else torch.ones(n, dtype=torch.bool) if which == "far" else torch.zeros(n, dtype=torch.bool)
+        moved["xyz"][pick] = eye + (scene["xyz"][pick] - eye) * 4000.0
+        moved["scales"][pick] = scene["scales"][pick] * 4000.0
+        st = _check_forward_stages(_scene_sub(moved), cam, torch.tensor([0.1, 0.2, 0.3]), max_borderline=2e-3)
+        if which != "near":
+            assert float(st.depths[st.radii > 0].max()) > 8192.0
+        assert (st.radii > 0).sum() > n // 2
+
+
 def test_garden_odd_resolution():
     """Garden-like scene at a resolution that is not a multiple of the tile size."""
     scene, cam, _ = scenes.make_config("C1", shrink=200, resolution_scale=0.2)
