@@ -320,7 +320,8 @@ def measure(args, config, forward_only, asides, cpu, apart_too=False):
     K = len(related)
     T = ((W + 15) // 16) * ((H + 15) // 16)
     N = W * H
-    passes = (int(_capi.lib.rgs_get_higher_msb(T)) + 8) // 9   # of the instance sort, on the tile key: digits of up to 9 bits
+    tile_bits = int(_capi.lib.rgs_get_higher_msb(T))
+    passes = min((tile_bits + 8) // 9, (tile_bits + 7) // 8)   # of the instance sort, on the tile key: digits of up to 9 bits
     # The backward revisits, per pixel, the entries up to the last blended one: nAl of the nA visits.
     flops_fwd = 12 * nA + 3 * nB + 27 * nC + 3 * nD + 14 * nE
     flops_bwd = 12 * nAl + 3 * nBl + 27 * nCl + 80 * nE

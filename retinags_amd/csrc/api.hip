@@ -260,6 +260,13 @@ int tile_key_bits(int width, int height)
 	return (int)rgs_get_higher_msb(tiles);
 }
 
+// Passes of the instance sort on the tile bits.
+int tile_sort_passes(int width, int height)
+{
+	const int bits = tile_key_bits(width, height);
+	return rgs::sort_passes(bits, rgs::sort_max_digit_bits_u32(bits));
+}
+
 // Physical buffers: A receives the duplicated keys, B is its ping-pong partner.
 struct BinningPhysical {
 	size_t keys_a, keys_b, vals_a, vals_b, temp, strip_lists, file_tail, total;
@@ -407,7 +414,7 @@ int rgs_binning_layout(int R, int width, int height, size_t offsets[RGS_BIN_FIEL
 {
 	RGS_REQUIRE(R >= 0 && width > 0 && height > 0 && offsets, "rgs_binning_layout: bad arguments");
 	const BinningPhysical b = binning_physical((size_t)R);
-	const bool sorted_in_a = (rgs::sort_passes(tile_key_bits(width, height), rgs::kDigitBitsU32) % 2) == 0;
+	const bool sorted_in_a = (tile_sort_passes(width, height) % 2) == 0;
 	offsets[RGS_BIN_KEYS_UNSORTED] = sorted_in_a ? b.keys_b : b.keys_a;
 	offsets[RGS_BIN_KEYS_SORTED] = sorted_in_a ? b.keys_a : b.keys_b;
 	offsets[RGS_BIN_VALUES_UNSORTED] = sorted_in_a ? b.vals_b : b.vals_a;
@@ -657,7 +664,7 @@ void fill_blend_args(rgs::BlendArgs& a, int P, int R, int width, int height, flo
 	a.capacity = (uint32_t)R;
 	if (R > 0) {
 		const BinningPhysical b = binning_physical((size_t)R);
-		const bool sorted_in_a = (rgs::sort_passes(tile_key_bits(width, height), rgs::kDigitBitsU32) % 2) == 0;
+		const bool sorted_in_a = (tile_sort_passes(width, height) % 2) == 0;
 		void* bin = const_cast<void*>(binning_ws);
 		a.point_list = at<uint32_t>(binning_ws, sorted_in_a ? b.vals_a : b.vals_b);
 		a.tile_keys = at<uint32_t>(binning_ws, sorted_in_a ? b.keys_a : b.keys_b);
@@ -748,7 +755,7 @@ int forward_binning(const char* who, bool count_on_device, int K, const RasterCa
 		d.filing.tanfovx = tan_fovx; d.filing.tanfovy = tan_fovy;
 		d.filing.W = width; d.filing.H = height;
 		d.keys = keys_a; d.values = vals_a; d.capacity = (uint32_t)R;
-		d.clear = temp; d.clear_words = rgs::sort_clear_words((size_t)R, end_bit, rgs::kDigitBitsU32);
+		d.clear = temp; d.clear_words = rgs::sort_clear_words((size_t)R, end_bit, rgs::sort_max_digit_bits_u32(end_bit));
 		// it also clears the tile ranges (and the counters and totals behind them) and counts the digits of the tiles
 		// it writes, so the sort starts with its passes
 		uint32_t* tile_digits = at<uint32_t>(at<char>(c.geom_ws, goff[RGS_GEOM_ORDER_SCRATCH]), order_scratch((size_t)P).tile_digits);

@@ -445,7 +445,8 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	const uint32_t limit = min(total, capacity);  // positions beyond the room the caller gave are dropped
 	if (blockIdx.x * (uint32_t)kDupPositions >= limit)
 		return;
-	const int passes = sort_passes(job.end_bit, kDigitBitsU32);
+	const int digit_bits = sort_max_digit_bits_u32(job.end_bit);
+	const int passes = sort_passes(job.end_bit, digit_bits);
 	for (int w = tid; w < kTileDigitWords; w += 256)
 		s_digits[w] = 0u;
 
@@ -465,42 +466,65 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 	const BoxFrame box = load_box_frame(filing.projinv, filing.range_low, filing.range_up, filing.tanfovx, filing.tanfovy);
 
 	// A workgroup takes every gridDim.x-th run of kDupPositions positions: the tables above are set up once, and the
-	// digit counts of many runs leave with one atomic add per digit.
+	// digit counts of many runs leave with one atomic add per digit.  What a run needs first (the Gaussian its
+	// positions begin at, from the table the offset scan has filled, and the offsets and indices of the 256 Gaussians
+	// from there on: a run of 256 positions cannot span more, every listed Gaussian having an instance) is asked for
+	// one run ahead, so that these two dependent reads are under way while the previous run is worked on.
+	const uint32_t table_runs = (uint32_t)dup_first_words((size_t)P);
+	uint32_t ahead_end = 0, ahead_index = 0, ahead_begin = 0;
+	bool ahead = false;  // the same for every thread of the workgroup
+	auto ask_for = [&](uint32_t r) {
+		const uint32_t f = min(job.first_of_block[r], n - 1u);
+		const uint32_t g = f + (uint32_t)tid;
+		ahead_end = g < n ? offsets[g] : total;
+		ahead_index = g < n ? min(order[g], P - 1u) : 0u;
+		ahead_begin = f == 0u ? 0u : offsets[f - 1];
+		ahead = true;
+	};
+	if (blockIdx.x < table_runs)
+		ask_for(blockIdx.x);
 	for (uint32_t run = blockIdx.x; (uint64_t)run * kDupPositions < (uint64_t)limit; run += gridDim.x) {
 	const uint32_t start = run * (uint32_t)kDupPositions;
 	const uint32_t stop = min(start + (uint32_t)kDupPositions, limit);
 	__syncthreads();  // the previous run is done with s_first and the staged Gaussians; the tables are written
-	// the first Gaussian whose inclusive offset exceeds `start`: from the table, or by a 64-ary search of the first wavefront
-	if (run < (uint32_t)dup_first_words((size_t)P)) {
-		if (tid == 0)
-			s_first = min(job.first_of_block[run], n - 1u);
-	} else if (tid < 64) {
-		uint32_t lo = 0, hi = n;  // the answer lies in [lo, hi]
-		while (lo < hi) {
-			const uint32_t step = (hi - lo + 63u) / 64u;
-			const uint32_t probe = lo + (uint32_t)lane * step;
-			const bool below = probe < hi && offsets[probe] <= start;
-			const uint32_t c = (uint32_t)__popcll(lanes_where(below));  // the predicate is monotone: the first c probes hold
-			if (c == 0u) {
-				hi = lo;
-			} else {
-				const uint32_t last_true = lo + (c - 1u) * step;
-				lo = last_true + 1u;
-				hi = min(last_true + step, hi);
+	uint32_t staged_begin;
+	if (ahead) {
+		st.end[tid] = ahead_end;
+		st.index[tid] = ahead_index;
+		staged_begin = ahead_begin;
+	} else {
+		// beyond the table (more than 16 instances per Gaussian on average): the first Gaussian whose inclusive offset
+		// exceeds `start` by a 64-ary search of the first wavefront
+		if (tid < 64) {
+			uint32_t lo = 0, hi = n;  // the answer lies in [lo, hi]
+			while (lo < hi) {
+				const uint32_t step = (hi - lo + 63u) / 64u;
+				const uint32_t probe = lo + (uint32_t)lane * step;
+				const bool below = probe < hi && offsets[probe] <= start;
+				const uint32_t c = (uint32_t)__popcll(lanes_where(below));  // the predicate is monotone: the first c probes hold
+				if (c == 0u) {
+					hi = lo;
+				} else {
+					const uint32_t last_true = lo + (c - 1u) * step;
+					lo = last_true + 1u;
+					hi = min(last_true + step, hi);
+				}
 			}
+			if (lane == 0)
+				s_first = min(lo, n - 1u);
 		}
-		if (lane == 0)
-			s_first = lo;
-	}
-	__syncthreads();
-
-	for (uint32_t g0 = s_first; g0 < n; g0 += 256) {
-		// stage the offsets and indices of Gaussians g0 .. g0 + 255 (in depth order)
-		const uint32_t g = g0 + (uint32_t)tid;
+		__syncthreads();
+		const uint32_t g0 = s_first, g = g0 + (uint32_t)tid;
 		st.end[tid] = g < n ? offsets[g] : total;
 		st.index[tid] = g < n ? min(order[g], P - 1u) : 0u;
-		__syncthreads();
-		const uint32_t staged_begin = g0 == 0u ? 0u : offsets[g0 - 1];
+		staged_begin = g0 == 0u ? 0u : offsets[g0 - 1];
+	}
+	__syncthreads();
+	ahead = false;
+	if ((uint64_t)(run + gridDim.x) * kDupPositions < (uint64_t)limit && run + gridDim.x < table_runs)
+		ask_for(run + gridDim.x);
+
+	{
 		const uint32_t staged_end = st.end[255];
 		const uint32_t from = max(start, staged_begin), to = min(stop, staged_end);
 		// Up to kDupPositions / 256 positions per thread.  First all of them find their Gaussian and ask for its
@@ -579,8 +603,8 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 		for (int q = 0; q < kPerThread; q++) {
 			const bool have = tile_of[q] != 0xFFFFFFFFu;
 			for (int p = 0; p < passes; p++) {
-				const int shift = sort_digit_shift(job.end_bit, p, kDigitBitsU32);
-				const int bits = sort_digit_bits(job.end_bit, p, kDigitBitsU32);
+				const int shift = sort_digit_shift(job.end_bit, p, digit_bits);
+				const int bits = sort_digit_bits(job.end_bit, p, digit_bits);
 				const uint32_t d = (tile_of[q] >> shift) & ((1u << bits) - 1u);
 				if (bits <= 2) {
 					// a digit of one or two bits: every lane would add to one of a few words, one after the other
@@ -594,9 +618,6 @@ __global__ __launch_bounds__(256) void duplicate_with_keys_kernel(Batch<Duplicat
 				}
 			}
 		}
-		if (staged_end >= stop)
-			break;
-		__syncthreads();
 	}
 	}
 	__syncthreads();
@@ -775,7 +796,9 @@ __global__ __launch_bounds__(256) void sort_onesweep_kernel(Batch<SortJob<KeyT>>
 			return;
 		ends_here = kKind == kPassOnDemand || !extra;
 	}
-	const uint32_t* __restrict__ digit_count = (j.digit_counts ? j.digit_counts : j.temp) + pass * kBins;
+	// the digit counts of a pass: 512 words apart for 32-bit keys whatever the digit width, 256 for 64-bit keys
+	constexpr int kCountStride = sizeof(KeyT) == 4 ? 512 : 256;
+	const uint32_t* __restrict__ digit_count = (j.digit_counts ? j.digit_counts : j.temp) + pass * kCountStride;
 	uint32_t* __restrict__ lookback = j.temp + kSortHeader + (size_t)pass * kBins * job_tiles;
 	uint32_t* __restrict__ tile_counter = j.temp + kSortCounters + pass;
 	uint32_t* __restrict__ status = j.temp + kSortStatus;
@@ -1087,7 +1110,7 @@ static void sort_pairs(const SortJob<KeyT>* jobs, int count, int end_bit, bool t
 		const uint32_t most_blocks = live >= 8 ? 256u : 2048u / (uint32_t)live;
 		const uint32_t hist_blocks = max_tiles < most_blocks ? max_tiles : most_blocks;
 		if (!histograms_done) {
-			if constexpr (kBits == kDigitBitsU64)
+			if constexpr (sizeof(KeyT) == 8)
 				hipLaunchKernelGGL(sort_digit_histogram_kernel<KeyT>, dim3(hist_blocks, (unsigned)live), dim3(256), 0, s, b, passes, end_bit);
 		}
 		for (int p = 0; p < passes; p++) {
@@ -1115,7 +1138,10 @@ void launch_sort_pairs(uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in,
 void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done,
                            const char* stage, hipStream_t s)
 {
-	sort_pairs<uint32_t, kDigitBitsU32>(jobs, count, end_bit, temp_cleared, histograms_done, stage != nullptr, s);
+	if (sort_max_digit_bits_u32(end_bit) == 9)
+		sort_pairs<uint32_t, 9>(jobs, count, end_bit, temp_cleared, histograms_done, stage != nullptr, s);
+	else
+		sort_pairs<uint32_t, 8>(jobs, count, end_bit, temp_cleared, histograms_done, stage != nullptr, s);
 }
 
 void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s)

@@ -288,6 +288,12 @@ void launch_preprocess_backward(const PreprocessBackwardArgs* jobs, int count, h
 // the runs of neighbouring keys a pass writes).
 constexpr int kDigitBitsU32 = 9;   // 512 digit values: the 17 tile bits of a 5185x3359 image in two passes, 27 depth bits in three
 constexpr int kDigitBitsU64 = 8;
+// The widest digit the sort of 32-bit keys on end_bit bits uses: 9 bits where that saves a pass, 8 otherwise (a pass
+// over 512 digit values writes shorter runs and was measured 14 % slower than one over 256).
+__host__ __device__ inline int sort_max_digit_bits_u32(int end_bit)
+{
+	return (end_bit + 8) / 9 < (end_bit + 7) / 8 ? 9 : 8;
+}
 __host__ __device__ inline int sort_passes(int end_bit, int max_bits)
 {
 	return (end_bit + max_bits - 1) / max_bits;
@@ -355,8 +361,8 @@ void launch_depth_order(const DepthOrderJob* jobs, int count, hipStream_t s);
 constexpr int kDupPositions = 256;
 constexpr size_t dup_first_words(size_t P) { return P / 16 + 2; }
 // The key duplication also counts the digits of the tiles it writes, which is what the sort of its keys starts
-// from: counts[512 p + d] = keys whose digit p of the tile bits (sort_digit_shift / sort_digit_bits with kDigitBitsU32)
-// is d, in kTileDigitWords words that are zero when it starts (the depth order leaves them so, and so does the
+// from: counts[512 p + d] = keys whose digit p of the tile bits (sort_digit_shift / sort_digit_bits with
+// sort_max_digit_bits_u32(end_bit)) is d, in kTileDigitWords words that are zero when it starts (the depth order leaves them so, and so does the
 // tile-range kernel, the last to run after they were read).
 constexpr int kTileDigitWords = 3 * 512;  // tiles have at most 24 bits: three passes at most
 struct DuplicateJob {
@@ -418,9 +424,9 @@ struct SortJob {
 	const uint32_t* count_of;      // tile count of every Gaussian, in_size of them
 	uint32_t index_bits, in_size;
 };
-// The same for 32-bit keys (sort_passes(end_bit, kDigitBitsU32) passes), every job in one launch per kernel; with a null
-// `stage` its kernels are not marked for the timing aid.  temp_cleared: the caller has cleared
-// sort_clear_words(n, end_bit, kDigitBitsU32) words of every temp already.  histograms_done: the kernel that wrote keys_in
+// The same for 32-bit keys (sort_passes(end_bit, sort_max_digit_bits_u32(end_bit)) passes), every job in one launch per
+// kernel; with a null `stage` its kernels are not marked for the timing aid.  temp_cleared: the caller has cleared
+// sort_clear_words(n, end_bit, sort_max_digit_bits_u32(end_bit)) words of every temp already.  histograms_done: the kernel that wrote keys_in
 // has also added every key's digits to the counts (counts[512 p + d] = keys whose digit p is d), so the sort need not
 // read the keys for that.
 void launch_sort_pairs_u32(const SortJob<uint32_t>* jobs, int count, int end_bit, bool temp_cleared, bool histograms_done,
