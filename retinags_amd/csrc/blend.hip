@@ -580,10 +580,9 @@ __device__ __forceinline__ int row_column(int pixel) { return pixel + (pixel >> 
 __device__ __forceinline__ int upstream_column(int pixel) { return pixel + (pixel >> 3); }
 
 struct BackwardPixel {
-	float T, T_final;
-	float behind_r, behind_g, behind_b, behind_depth, behind_alpha;
+	float T;
+	float behind;  // what lies behind the entry being visited, weighted with the upstream gradient: see backward_visit
 	float g_r, g_g, g_b, g_depth, g_alpha;
-	float bg_dot_dpixel;
 };
 
 struct BackwardStage {  // wave-private
@@ -675,13 +674,6 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 	__builtin_amdgcn_wave_barrier();
 }
 
-// behind = keep * behind + add, in the register that holds `behind`: written as an expression, the compiler forms the
-// sum in the register of `add` and copies it over afterwards, one more instruction per colour channel and visit.
-__device__ __forceinline__ void update_behind(float& behind, float keep, float add)
-{
-	asm("v_fma_f32 %0, %1, %0, %2" : "+v"(behind) : "v"(keep), "v"(add));
-}
-
 // Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
 template <bool kDepth>
 __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
@@ -691,7 +683,6 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 	if (lanes_where(candidate) == 0ull)
 		return;
 	float u = 0.f, aT = 0.f;
-	bool valid = false;
 	const float clip_w = wave_uniform(g.w);  // NaN: the whole strip is inside the box
 	if (candidate) {
 		const float G = exp_of_exponent(power);
@@ -702,31 +693,23 @@ __device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate,
 			// From here on nothing feeds a decision: gradients are compared by tolerance, so the
 			// compiler may contract multiply-adds and the divisions use the hardware reciprocal.
 #pragma clang fp contract(fast)
-			valid = true;
 			const float inv_one_minus_alpha = __builtin_amdgcn_rcpf(1.f - alpha);
 			p.T = p.T * inv_one_minus_alpha;
 			aT = alpha * p.T;
 			const float4 cd = st.cd[slot];
-			// p.behind_* is what the entries behind this one (already visited) add up to, per unit of transmittance:
-			// the reference forms it at the next entry from this entry's alpha and colour (K/cuda_rasterizer_hgs/backward.cu:568-592:
-			// accum_rec = last_alpha * last_color + (1 - last_alpha) * accum_rec); formed here, right after its use,
-			// the same expression needs no copy of this entry's alpha and colour kept for the next visit.
-			const float keep = 1.f - alpha;
-			float dL_dopa = 0.0f;
-			dL_dopa += (cd.x - p.behind_r) * p.g_r;
-			dL_dopa += (cd.y - p.behind_g) * p.g_g;
-			dL_dopa += (cd.z - p.behind_b) * p.g_b;
+			// The pixel's outputs are sums over its blended entries j of w_j (colour_j, depth_j, 1) with w_j = alpha_j T_j,
+			// T_j the product of (1 - alpha_k) over the entries in front, plus T_final times the background.  Their
+			// derivative with respect to alpha_i is T_i (colour_i, depth_i, 1) minus (the sum over the entries behind i +
+			// T_final background) / (1 - alpha_i).  The reference carries that sum per channel and per unit of transmittance
+			// (K/cuda_rasterizer_hgs/backward.cu:568-599: accum_rec = last_alpha * last_color + (1 - last_alpha) * accum_rec,
+			// and the background term apart); only its product with the upstream gradient is needed, so one number per
+			// pixel does for all channels: `behind` = sum over the entries behind of w_j <g, (colour_j, depth_j, 1)> +
+			// T_final <g, background>, started with the latter.  Same quantity, a third of the arithmetic.
+			float weighted = __builtin_fmaf(cd.x, p.g_r, __builtin_fmaf(cd.y, p.g_g, __builtin_fmaf(cd.z, p.g_b, p.g_alpha)));
 			if (kDepth)
-				dL_dopa += (cd.w - p.behind_depth) * p.g_depth;
-			dL_dopa += (1 - p.behind_alpha) * p.g_alpha;
-			dL_dopa *= p.T;
-			update_behind(p.behind_r, keep, alpha * cd.x);
-			update_behind(p.behind_g, keep, alpha * cd.y);
-			update_behind(p.behind_b, keep, alpha * cd.z);
-			if (kDepth)
-				update_behind(p.behind_depth, keep, alpha * cd.w);
-			update_behind(p.behind_alpha, keep, alpha);
-			dL_dopa += (-p.T_final * inv_one_minus_alpha) * p.bg_dot_dpixel;
+				weighted = __builtin_fmaf(cd.w, p.g_depth, weighted);
+			const float dL_dopa = weighted * p.T - p.behind * inv_one_minus_alpha;
+			p.behind = __builtin_fmaf(aT, weighted, p.behind);
 			u = G * dL_dopa;
 		}
 	}
@@ -777,9 +760,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 	const uint32_t last_contributor = inside ? a.n_contrib[pix_id] : 0u;
 
 	BackwardPixel p;
-	p.T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
-	p.T = p.T_final;
-	p.behind_r = p.behind_g = p.behind_b = p.behind_depth = p.behind_alpha = 0.f;
+	const float T_final = inside ? (1 - a.out_alpha[pix_id]) : 0.f;
+	p.T = T_final;
 	p.g_r = p.g_g = p.g_b = p.g_depth = p.g_alpha = 0.f;
 	if (inside) {
 		p.g_r = a.dL_dpix[pix_id];
@@ -788,7 +770,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 		p.g_depth = a.dL_dpix_depth ? a.dL_dpix_depth[pix_id] : 0.f;  // absent: no gradient came in
 		p.g_alpha = a.dL_dalpha ? a.dL_dalpha[pix_id] : 0.f;
 	}
-	p.bg_dot_dpixel = (0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b;
+	p.behind = T_final * ((0.f + a.bg[0] * p.g_r + a.bg[1] * p.g_g) + a.bg[2] * p.g_b);
 	st.upstream[upstream_column(lane)] = float4{p.g_r, p.g_g, p.g_b, p.g_depth};
 	int rows = 0;
 	uint64_t row_slots = 0ull;
