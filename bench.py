@@ -107,6 +107,9 @@ def parse():
                     help="one rasterizer call per submodel, as the reference issues them (default: the submodels of a frame "
                          "go through one call that blends them in one launch per direction)")
     ap.add_argument("--no-asides", action="store_true", help="skip the stages beside the metric (sharing, loss, optimiser)")
+    ap.add_argument("--gaussian-order", default="given", choices=["given", "morton"],
+                    help="the order in which a submodel's Gaussians are stored: as the scene generator emitted them (the "
+                         "default), or along a Z-order curve, as a loader that sorts them would store them")
     ap.add_argument("--whole-iteration", action="store_true",
                     help="also time one whole training iteration from the stored parameters (activation, sharing, render, loss, "
                          "backward, Adam); not part of the metric")
@@ -136,19 +139,19 @@ def main():
     ensure_built()
     default_run = (args.config == "C1" and not args.forward_only and args.shrink == 1.0 and args.resolution_scale == 1.0)
     line = measure(args, args.config, args.forward_only, asides=not args.no_asides, cpu=not args.no_cpu_baseline,
-                   apart_too=default_run and not args.no_other_configs)
+                   apart_too=default_run and not args.no_other_configs, morton_too=default_run and not args.no_other_configs)
     if default_run and not args.no_render_metric:
         # the second half of the metric: render only (every related submodel's forward and the compositing)
         for name in ("C3", "C4"):
             try:
-                sub = measure(args, name, True, asides=False, cpu=not args.no_cpu_baseline)
+                sub = measure(args, name, True, asides=False, cpu=not args.no_cpu_baseline, morton_too=not args.no_other_configs)
                 line[f"render_ms_per_frame_{name.lower()}"] = {
                     "value": sub["ms_per_step"], "unit": "ms/frame", "ms_per_frame_one_stream": sub["ms_per_step_one_stream"],
                     "verified": sub["verified"], "verification": sub["verification"],
                     "workload": sub["config"]["workload"], "instances": sub["config"]["instances"],
                     "visible": sub["config"]["visible"], "setup_s": sub["config"]["setup_s"],
                     "peak_device_memory_GB": sub["config"]["peak_device_memory_GB"], "roofline": sub["roofline"],
-                    "cpu_baseline": sub["cpu_baseline"],
+                    "cpu_baseline": sub["cpu_baseline"], "morton_order": sub["morton_order"],
                     "blend_forward": sub["stages"].get("blend_forward"), "stages_ms": {k: v["ms_per_step"] for k, v in sub["stages"].items()},
                     "blend_work": sub["blend_work"]}
             except Exception as ex:   # the first half of the metric must not be lost with the second
@@ -173,7 +176,7 @@ def main():
     print(json.dumps(line))
 
 
-def measure(args, config, forward_only, asides, cpu, apart_too=False):
+def measure(args, config, forward_only, asides, cpu, apart_too=False, morton_too=False):
     """Times `config` and returns the JSON line's dictionary."""
     from retinags_amd import _capi, rasterizer as R
     from retinags_amd.harness import scenes, partition, pipeline
@@ -190,7 +193,7 @@ def measure(args, config, forward_only, asides, cpu, apart_too=False):
         split = partition.partition_scene_on_device if on_device else partition.partition_scene
         part = split(scene["xyz"], scene["scales"], depth)
         rel = partition.relation_vector(part, cam)
-        subs = pipeline.submodels_from_partition(scene, part, dev)
+        subs = pipeline.submodels_from_partition(scene, part, dev, order=args.gaussian_order)
         members = part.members
     else:
         part = None
@@ -443,6 +446,23 @@ def measure(args, config, forward_only, asides, cpu, apart_too=False):
     whole = (aside(lambda: whole_iteration(scene, part, cam_d, rel, bg, streams, dev, args.steps))
              if (part is not None and do_backward and asides and args.whole_iteration) else None)
 
+    # ---- the same frame with every submodel's Gaussians stored along a Z-order curve instead of in the order the scene
+    # generator emitted them: what a loader that sorts its Gaussians hands the rasterizer (same Gaussians, same images)
+    morton = None
+    if morton_too and args.gaussian_order == "given" and depth > 0:
+        for m in related:
+            subs[m] = pipeline.reorder_submodel(subs[m], partition.morton_order(subs[m].means3D.detach()))
+        torch.cuda.empty_cache()
+        elapsed_m = timed()
+        _capi.stage_timing(True)
+        for _ in range(prof_steps):
+            step(streams=None)
+        stage_m = _capi.stage_timing_read()
+        _capi.stage_timing(False)
+        morton = {"value": round(args.steps / elapsed_m, 4), "unit": "it/s", "ms_per_step": round(elapsed_m * 1e3 / args.steps, 3),
+                  "stages_ms": {k: round(v[0] / prof_steps, 4) for k, v in stage_m.items()},
+                  "order": "each submodel's Gaussians sorted by the Morton code of their centres (10 bits per axis)"}
+
     # ---- host-CPU baseline: the CPU checker on the same frame, same seeded inputs
     cpu_line = None
     if cpu and scene is not None:
@@ -465,6 +485,8 @@ def measure(args, config, forward_only, asides, cpu, apart_too=False):
         "ms_per_step_apart": round(elapsed_apart * 1e3 / args.steps, 3) if elapsed_apart else None,
         # the timed calls (all submodels through one call per stage) checked against one call per submodel on this workload
         "verified": verification["verified"] if verification else None, "verification": verification,
+        # not the metric's workload order: the same Gaussians stored along a Z-order curve (see measure())
+        "morton_order": morton,
         # how long the host takes to queue a step (the forward's waits for the instance counts included)
         "host_ms_per_step": {k: round(v, 3) for k, v in host_ms.items()},
         "config": {"workload": f"{config}: {cfg['n']} Gaussians, {W}x{H}, bvh_depth={depth} "
@@ -473,6 +495,7 @@ def measure(args, config, forward_only, asides, cpu, apart_too=False):
                    "gaussians_rendered_incl_shared": P_tot, "visible": P_vis, "instances": R_tot,
                    "tiles": T, "sort_passes": passes, "setup_s": round(setup_s, 1),
                    "scene_generated_on": "device" if on_device else "host",
+                   "gaussian_order": "as generated (uniformly random in memory)" if args.gaussian_order == "given" else "Morton order per submodel",
                    "streams": args.streams,
                    "submodels_of_a_frame": "one call, blended in one launch per direction" if together else "one call each",
                    "peak_device_memory_GB": round(peak_gb, 2),

@@ -155,270 +155,186 @@ __device__ __forceinline__ void wave_lds_fence()
 
 constexpr int kShRowStride = 13;  // float4 per parked row: 52 words, so 8 lanes' 16-byte reads meet no bank twice
 
-// The 256 Gaussians of a workgroup are first culled cheaply (behind the camera: one affine form; certainly beside the
-// image: a bound on the radius) and the remaining ones listed in index order; the rest of the work (covariance,
-// projection, radius, tile rectangle, SH colour, record) is then done by thread t for the t-th listed Gaussian, so
-// that only ceil(listed / 64) wavefronts of the four run it and the others skip it whole.  With two thirds of the
-// Gaussians of a call out of sight that is half the vector instructions of the kernel, which is bound by their
-// issue rate (a wavefront that holds a single visible Gaussian pays for the whole code).  The per-Gaussian outputs
-// (radius, tile count, depth) go through LDS and leave in index order, whole lines at a time.
 __global__ __launch_bounds__(256) void preprocess_forward_kernel(Batch<PreprocessArgs> batch)
 {
 	__shared__ uint32_t s_scan[8];
 	__shared__ float4 s_rows[4][32 * kShRowStride];
 	__shared__ uint8_t s_listed[4][64];
-	__shared__ uint8_t s_front[256];       // the workgroup's Gaussians that can touch a tile (place in the workgroup), in index order
-	__shared__ uint32_t s_wave_front[4];
-	__shared__ uint32_t s_touched[256];    // results by place in the workgroup
-	__shared__ int s_radius[256];
-	__shared__ float s_depth[256];
 	const PreprocessArgs& a = batch.job[blockIdx.y];  // one job per submodel of the frame
-	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-	const int first = blockIdx.x * 256;    // the workgroup's first Gaussian
+	const int idx = blockIdx.x * 256 + threadIdx.x;
 	// the scratch of the depth sort that follows is cleared here, which saves a launch
-	for (size_t w = (size_t)first + tid; w < a.clear_words; w += (size_t)gridDim.x * 256)
+	for (size_t w = (size_t)idx; w < a.clear_words; w += (size_t)gridDim.x * 256)
 		a.clear[w] = 0u;
-	if (first >= a.P)
+	if ((int)blockIdx.x * 256 >= a.P)
 		return;  // the launch is sized for the job with the most Gaussians
+	uint32_t touched = 0;
+	bool rendered = false;
+	float2 pix = {0.f, 0.f};
+	float4 conic_o = {0.f, 0.f, 0.f, 0.f};
+	float hom_w = 0.f, view_z = 0.f, my_radius = 0.f;
+	float3 p = {0.f, 0.f, 0.f};
 
-	// ---- in front of the camera (K/cuda_rasterizer_hgs/auxiliary.h:155-180: p_view.z <= 0.2 is culled) and not
-	// certainly beside the image?  The second test only drops Gaussians whose tile rectangle would come out empty
-	// (K/cuda_rasterizer_hgs/forward.cu:236-238), from an upper bound on the radius: the radius is ceil(3 sqrt(l)) with
-	// l the larger eigenvalue of the 2D covariance (gap floored at sqrt(0.1)), l <= trace + 0.32, and
-	// trace(J W S W^T J^T) + 0.6 <= |J|_F^2 |W|_F^2 l_max(S) + 0.6, where |J|_F^2 <= (fx^2 (1 + limx^2) + fy^2 (1 + limy^2)) / z^2
-	// by the guard-frustum clamp, and l_max(S) <= (modifier max scale (|q|^2 + |1 - |q|^2|))^2 (the matrix built from a
-	// quaternion q as given is |q|^2 times a rotation plus (1 - |q|^2) times the identity), or trace(S) for a given
-	// covariance.  The bound is widened by a quarter and the rectangle by two tiles; anything not finite fails the
-	// comparisons and goes on to the exact evaluation.
-	bool front = false;
-	if (first + tid < a.P) {
-		const size_t i = (size_t)(first + tid);
-		const float3 q = {a.means[3 * i], a.means[3 * i + 1], a.means[3 * i + 2]};
-		const float z = xform_point_4x3(q, a.view).z;
-		front = !(z <= 0.2f);
-		if (front) {
-			const float4 hom = xform_point_4x4(q, a.proj);
-			const float rw = __builtin_amdgcn_rcpf(hom.w + 0.0000001f);
-			const float px = 0.5f * ((hom.x * rw + 1.f) * (float)a.W - 1.f), py = 0.5f * ((hom.y * rw + 1.f) * (float)a.H - 1.f);
-			float lmax;
+	if (idx < a.P) {
+		do {
+			p = float3{a.means[3 * (size_t)idx], a.means[3 * (size_t)idx + 1], a.means[3 * (size_t)idx + 2]};
+			const float3 p_view = xform_point_4x3(p, a.view);
+			if (p_view.z <= 0.2f)
+				break;
+			const float4 p_hom = xform_point_4x4(p, a.proj);
+			const float p_w = 1.0f / (p_hom.w + 0.0000001f);
+			const float2 p_proj = {p_hom.x * p_w, p_hom.y * p_w};
+
+			float cov6[6];
 			if (a.cov3D_precomp) {
-				lmax = a.cov3D_precomp[6 * i] + a.cov3D_precomp[6 * i + 3] + a.cov3D_precomp[6 * i + 5];
+#pragma unroll
+				for (int i = 0; i < 6; i++)
+					cov6[i] = a.cov3D_precomp[6 * (size_t)idx + i];
 			} else {
-				const float smax = a.scale_modifier * fmaxf(fmaxf(a.scales[3 * i], a.scales[3 * i + 1]), a.scales[3 * i + 2]);
-				const float4 r = reinterpret_cast<const float4*>(a.rotations)[i];
-				const float n2 = r.x * r.x + r.y * r.y + r.z * r.z + r.w * r.w;
-				const float stretch = smax * (n2 + fabsf(1.f - n2));
-				lmax = stretch * stretch;
+				const float3 sc = {a.scales[3 * (size_t)idx], a.scales[3 * (size_t)idx + 1], a.scales[3 * (size_t)idx + 2]};
+				const float4 q = reinterpret_cast<const float4*>(a.rotations)[idx];
+				covariance3d(sc, a.scale_modifier, q, cov6);
 			}
-			const float limx = 1.3f * a.tanfovx, limy = 1.3f * a.tanfovy;
-			const float w00 = a.view[0], w01 = a.view[1], w02 = a.view[2], w10 = a.view[4], w11 = a.view[5], w12 = a.view[6],
-			            w20 = a.view[8], w21 = a.view[9], w22 = a.view[10];
-			const float wf2 = w00 * w00 + w01 * w01 + w02 * w02 + w10 * w10 + w11 * w11 + w12 * w12 + w20 * w20 + w21 * w21 + w22 * w22;
-			const float jf2 = (a.focal_x * a.focal_x * (1.f + limx * limx) + a.focal_y * a.focal_y * (1.f + limy * limy)) *
-			                  __builtin_amdgcn_rcpf(z * z);
-			const float l = 1.25f * (jf2 * wf2 * lmax + 0.6f) + 0.5f;
-			const float reach = 3.f * __builtin_amdgcn_sqrtf(l) + 2.f + 2.f * (float)kTile;
-			const bool beside = (px + reach < 0.f) || (px - reach > (float)a.W) || (py + reach < 0.f) || (py - reach > (float)a.H);
-			front = !beside;
-		}
+			Ewa e = ewa_project(p, a.focal_x, a.focal_y, a.tanfovx, a.tanfovy, cov6, a.view);
+			const float cx = e.cov.c[0][0] + 0.3f, cy = e.cov.c[0][1], cz = e.cov.c[1][1] + 0.3f;
+
+			const float det = (cx * cz - cy * cy);
+			if (det == 0.0f)
+				break;
+			const float det_inv = 1.f / det;
+
+			const float mid = 0.5f * (cx + cz);
+			const float lambda1 = mid + sqrtf(fmaxf(0.1f, mid * mid - det));
+			const float lambda2 = mid - sqrtf(fmaxf(0.1f, mid * mid - det));
+			const float radius = ceilf(3.f * sqrtf(fmaxf(lambda1, lambda2)));
+			const float2 at = {ndc_to_pix(p_proj.x, a.W), ndc_to_pix(p_proj.y, a.H)};
+			const TileRect rc = tile_rect(at.x, at.y, (int)radius, a.grid_x, a.grid_y);
+			const uint32_t ntiles = (rc.x1 - rc.x0) * (rc.y1 - rc.y0);
+			if (ntiles == 0)
+				break;
+			conic_o = float4{cz * det_inv, -cy * det_inv, cx * det_inv, a.opacities[idx]};
+			pix = at;
+			hom_w = p_hom.w;
+			view_z = p_view.z;
+			my_radius = radius;
+			touched = ntiles;
+			rendered = true;
+		} while (false);
 	}
-	s_touched[tid] = 0u;
-	s_radius[tid] = 0;
-	s_depth[tid] = 0.f;
-	const uint64_t in_front = lanes_where(front);
-	if (lane == 0)
-		s_wave_front[wave] = (uint32_t)__popcll(in_front);
-	__syncthreads();
-	uint32_t before = 0, n_front = 0;
-#pragma unroll
-	for (int w = 0; w < 4; w++) {
-		const uint32_t c = s_wave_front[w];
-		before += w < wave ? c : 0u;
-		n_front += c;
-	}
-	if (front)
-		s_front[before + __builtin_amdgcn_mbcnt_hi((uint32_t)(in_front >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)in_front, 0u))] = (uint8_t)tid;
-	__syncthreads();
 
-	// ---- thread t takes the t-th of them; wavefronts beyond the list have nothing to do until the outputs leave
-	if ((uint32_t)(wave * 64) < n_front) {
-		const bool active = (uint32_t)tid < n_front;
-		const int place = active ? (int)s_front[tid] : 0;
-		const int idx = first + place;
-		uint32_t touched = 0;
-		bool rendered = false;
-		float2 pix = {0.f, 0.f};
-		float4 conic_o = {0.f, 0.f, 0.f, 0.f};
-		float hom_w = 0.f, view_z = 0.f, my_radius = 0.f;
-		float3 p = {0.f, 0.f, 0.f};
+	// the rendered Gaussians of the wavefront, listed in lane order
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const uint64_t seen = lanes_where(rendered);
+	const int n_seen = __popcll(seen);
+	const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(seen >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)seen, 0u));
+	float4* parked = s_rows[wave];
+	uint8_t* listed = s_listed[wave];
+	if (rendered)
+		listed[rank] = (uint8_t)lane;
+	wave_lds_fence();
 
-		if (active) {
-			do {
-				p = float3{a.means[3 * (size_t)idx], a.means[3 * (size_t)idx + 1], a.means[3 * (size_t)idx + 2]};
-				const float3 p_view = xform_point_4x3(p, a.view);
-				if (p_view.z <= 0.2f)
-					break;
-				const float4 p_hom = xform_point_4x4(p, a.proj);
-				const float p_w = 1.0f / (p_hom.w + 0.0000001f);
-				const float2 p_proj = {p_hom.x * p_w, p_hom.y * p_w};
-
-				float cov6[6];
-				if (a.cov3D_precomp) {
-#pragma unroll
-					for (int i = 0; i < 6; i++)
-						cov6[i] = a.cov3D_precomp[6 * (size_t)idx + i];
-				} else {
-					const float3 sc = {a.scales[3 * (size_t)idx], a.scales[3 * (size_t)idx + 1], a.scales[3 * (size_t)idx + 2]};
-					const float4 q = reinterpret_cast<const float4*>(a.rotations)[idx];
-					covariance3d(sc, a.scale_modifier, q, cov6);
-				}
-				Ewa e = ewa_project(p, a.focal_x, a.focal_y, a.tanfovx, a.tanfovy, cov6, a.view);
-				const float cx = e.cov.c[0][0] + 0.3f, cy = e.cov.c[0][1], cz = e.cov.c[1][1] + 0.3f;
-
-				const float det = (cx * cz - cy * cy);
-				if (det == 0.0f)
-					break;
-				const float det_inv = 1.f / det;
-
-				const float mid = 0.5f * (cx + cz);
-				const float lambda1 = mid + sqrtf(fmaxf(0.1f, mid * mid - det));
-				const float lambda2 = mid - sqrtf(fmaxf(0.1f, mid * mid - det));
-				const float radius = ceilf(3.f * sqrtf(fmaxf(lambda1, lambda2)));
-				const float2 at = {ndc_to_pix(p_proj.x, a.W), ndc_to_pix(p_proj.y, a.H)};
-				const TileRect rc = tile_rect(at.x, at.y, (int)radius, a.grid_x, a.grid_y);
-				const uint32_t ntiles = (rc.x1 - rc.x0) * (rc.y1 - rc.y0);
-				if (ntiles == 0)
-					break;
-				conic_o = float4{cz * det_inv, -cy * det_inv, cx * det_inv, a.opacities[idx]};
-				pix = at;
-				hom_w = p_hom.w;
-				view_z = p_view.z;
-				my_radius = radius;
-				touched = ntiles;
-				rendered = true;
-			} while (false);
-		}
-
-		// the rendered Gaussians of the wavefront, listed in lane order by their place in the workgroup
-		const uint64_t seen = lanes_where(rendered);
-		const int n_seen = __popcll(seen);
-		const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(seen >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)seen, 0u));
-		float4* parked = s_rows[wave];
-		uint8_t* listed = s_listed[wave];
+	float3 col = {0.f, 0.f, 0.f};
+	uint32_t clamp_bits = 0;
+	if (a.colors_precomp) {
 		if (rendered)
-			listed[rank] = (uint8_t)place;
-		wave_lds_fence();
-
-		float3 col = {0.f, 0.f, 0.f};
-		uint32_t clamp_bits = 0;
-		if (a.colors_precomp) {
-			if (rendered)
-				col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
-				             a.colors_precomp[3 * (size_t)idx + 2]};
-		} else if (n_seen > 0) {
-			const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
-			const float3 dir = {p.x - cam.x, p.y - cam.y, p.z - cam.z};
-			const float len = sqrtf(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
-			const float dx = dir.x / len, dy = dir.y / len, dz = dir.z / len;
-			float raw[3] = {0.f, 0.f, 0.f};
-			if (a.sh_rows_by_16_bytes) {
-				const int piece = lane & 15, sub = lane >> 4;
-				const int row_pieces = a.M * 3 / 4;
-				const int needed = 3 * (a.D + 1) * (a.D + 1);
-				const float4* __restrict__ rows = reinterpret_cast<const float4*>(a.shs) + (size_t)first * row_pieces;
-				for (int base = 0; base < n_seen; base += 32) {
-					float4 v[8];
+			col = float3{a.colors_precomp[3 * (size_t)idx], a.colors_precomp[3 * (size_t)idx + 1],
+			             a.colors_precomp[3 * (size_t)idx + 2]};
+	} else {
+		const float3 cam = {a.campos[0], a.campos[1], a.campos[2]};
+		const float3 dir = {p.x - cam.x, p.y - cam.y, p.z - cam.z};
+		const float len = sqrtf(dir.x * dir.x + dir.y * dir.y + dir.z * dir.z);
+		const float dx = dir.x / len, dy = dir.y / len, dz = dir.z / len;
+		float raw[3] = {0.f, 0.f, 0.f};
+		if (a.sh_rows_by_16_bytes) {
+			const int piece = lane & 15, sub = lane >> 4;
+			const int row_pieces = a.M * 3 / 4;
+			const int needed = 3 * (a.D + 1) * (a.D + 1);
+			const float4* __restrict__ rows =
+			    reinterpret_cast<const float4*>(a.shs) + (size_t)(idx - lane) * row_pieces;
+			for (int base = 0; base < n_seen; base += 32) {
+				float4 v[8];
 #pragma unroll
-					for (int r = 0; r < 8; r++) {
-						const int slot = base + 4 * r + sub;
-						v[r] = float4{0.f, 0.f, 0.f, 0.f};
-						if (4 * piece < needed && slot < n_seen)
-							v[r] = rows[(size_t)listed[slot] * row_pieces + piece];
-					}
-#pragma unroll
-					for (int r = 0; r < 8; r++)
-						if (piece < 12)
-							parked[(4 * r + sub) * kShRowStride + piece] = v[r];
-					wave_lds_fence();
-					if (rendered && rank >= base && rank < base + 32) {
-						float row[kShRegs];
-						const float4* mine = parked + (rank - base) * kShRowStride;
-#pragma unroll
-						for (int k = 0; k < kShRegs; k += 4) {
-							float4 q = {0.f, 0.f, 0.f, 0.f};
-							if (k < needed)
-								q = mine[k / 4];
-							row[k] = q.x;
-							row[k + 1] = q.y;
-							row[k + 2] = q.z;
-							row[k + 3] = q.w;
-						}
-#pragma unroll
-						for (int ch = 0; ch < 3; ch++)
-							raw[ch] = sh_channel(a.D, dx, dy, dz, row + ch);
-					}
-					wave_lds_fence();
+				for (int r = 0; r < 8; r++) {
+					const int slot = base + 4 * r + sub;
+					v[r] = float4{0.f, 0.f, 0.f, 0.f};
+					if (4 * piece < needed && slot < n_seen)
+						v[r] = rows[(size_t)listed[slot] * row_pieces + piece];
 				}
-			} else if (rendered) {
-				const float* sh = a.shs + (size_t)idx * a.M * 3;
 #pragma unroll
-				for (int ch = 0; ch < 3; ch++)
-					raw[ch] = sh_channel(a.D, dx, dy, dz, sh + ch);
-			}
-			float rgb[3];
+				for (int r = 0; r < 8; r++)
+					if (piece < 12)
+						parked[(4 * r + sub) * kShRowStride + piece] = v[r];
+				wave_lds_fence();
+				if (rendered && rank >= base && rank < base + 32) {
+					float row[kShRegs];
+					const float4* mine = parked + (rank - base) * kShRowStride;
 #pragma unroll
-			for (int ch = 0; ch < 3; ch++) {
-				const float v = raw[ch];
-				clamp_bits |= (v < 0) ? (1u << ch) : 0u;
-				rgb[ch] = fmaxf(v, 0.0f);
+					for (int k = 0; k < kShRegs; k += 4) {
+						float4 q = {0.f, 0.f, 0.f, 0.f};
+						if (k < needed)
+							q = mine[k / 4];
+						row[k] = q.x;
+						row[k + 1] = q.y;
+						row[k + 2] = q.z;
+						row[k + 3] = q.w;
+					}
+#pragma unroll
+					for (int ch = 0; ch < 3; ch++)
+						raw[ch] = sh_channel(a.D, dx, dy, dz, row + ch);
+				}
+				wave_lds_fence();
 			}
-			col = float3{rgb[0], rgb[1], rgb[2]};
+		} else if (rendered) {
+			const float* sh = a.shs + (size_t)idx * a.M * 3;
+#pragma unroll
+			for (int ch = 0; ch < 3; ch++)
+				raw[ch] = sh_channel(a.D, dx, dy, dz, sh + ch);
 		}
+		float rgb[3];
+#pragma unroll
+		for (int ch = 0; ch < 3; ch++) {
+			const float v = raw[ch];
+			clamp_bits |= (v < 0) ? (1u << ch) : 0u;
+			rgb[ch] = fmaxf(v, 0.0f);
+		}
+		col = float3{rgb[0], rgb[1], rgb[2]};
+	}
 
+	if (idx < a.P) {
 		if (rendered) {
 			if (!a.colors_precomp)
 				a.clamped[idx] = (uint8_t)clamp_bits;
-			s_radius[place] = (int)my_radius;
-			s_touched[place] = touched;
-			s_depth[place] = view_z;  // stays 0 for a Gaussian that touches no tile: the depth order lists the others by this alone
 		}
-		if (n_seen > 0) {
-			// Everything later stages read of a rendered Gaussian goes into one 64-byte record: a
-			// gather by index then costs one cache line, and nothing is written a second time into
-			// arrays of their own, where a rendered Gaussian among unrendered ones dirties a whole
-			// line for a few bytes.  The 3D covariance is not kept: the backward computes it again.
-			// The records leave through LDS, four lanes to a record, so that a store instruction
-			// writes 16 whole records and not a quarter of 64.
-			wave_lds_fence();
-			if (rendered) {
-				const float floor = exponent_floor(conic_o.w);
-				const float2 half = alpha_ellipse_half_extent(conic_o, floor);
-				float4* rec = parked + rank * kRecordStride;
-				rec[0] = float4{pix.x, pix.y, floor, hom_w};
-				rec[1] = conic_o;
-				rec[2] = float4{col.x, col.y, col.z, view_z};
-				// the third word is the integer radius (as bits): the key duplication reads the tile rectangle's inputs from here
-				rec[3] = float4{half.x, half.y, __int_as_float((int)my_radius), 0.f};
-			}
-			wave_lds_fence();
-			float4* records = a.blend_record + 4 * (size_t)first;
-			for (int base = 0; base < n_seen; base += 16) {
-				const int slot = base + (lane >> 2);
-				if (slot < n_seen)
-					records[4 * (size_t)listed[slot] + (lane & 3)] = parked[slot * kRecordStride + (lane & 3)];
-			}
+		a.radii[idx] = (int)my_radius;
+		a.tiles_touched[idx] = touched;
+		a.depths[idx] = view_z;  // 0 for a Gaussian that touches no tile: the depth order lists the others by this alone
+	}
+	{
+		// Everything later stages read of a rendered Gaussian goes into one 64-byte record: a
+		// gather by index then costs one cache line, and nothing is written a second time into
+		// arrays of their own, where a rendered Gaussian among unrendered ones dirties a whole
+		// line for a few bytes.  The 3D covariance is not kept: the backward computes it again.
+		// The records leave through LDS, four lanes to a record, so that a store instruction
+		// writes 16 whole records and not a quarter of 64.
+		wave_lds_fence();
+		if (rendered) {
+			const float floor = exponent_floor(conic_o.w);
+			const float2 half = alpha_ellipse_half_extent(conic_o, floor);
+			float4* rec = parked + rank * kRecordStride;
+			rec[0] = float4{pix.x, pix.y, floor, hom_w};
+			rec[1] = conic_o;
+			rec[2] = float4{col.x, col.y, col.z, view_z};
+			// the third word is the integer radius (as bits): the key duplication reads the tile rectangle's inputs from here
+			rec[3] = float4{half.x, half.y, __int_as_float((int)my_radius), 0.f};
+		}
+		wave_lds_fence();
+		float4* records = a.blend_record + 4 * (size_t)(idx - lane);
+		for (int base = 0; base < n_seen; base += 16) {
+			const int slot = base + (lane >> 2);
+			if (slot < n_seen)
+				records[4 * (size_t)listed[slot] + (lane & 3)] = parked[slot * kRecordStride + (lane & 3)];
 		}
 	}
-	__syncthreads();
 
-	// ---- the per-Gaussian outputs leave in index order
-	const uint32_t touched = s_touched[tid];
-	if (first + tid < a.P) {
-		const size_t i = (size_t)(first + tid);
-		a.radii[i] = s_radius[tid];
-		a.tiles_touched[i] = touched;
-		a.depths[i] = s_depth[tid];
-	}
 	// Per-block total of tiles_touched: the first level of the offset scan.
 	uint32_t total;
 	(void)block256_exclusive_scan_u32(touched, s_scan, total);

@@ -291,3 +291,22 @@ def relation_vector(part: Partition, cam, z_near: float = 0.01, z_far: float = 1
     if (rel < 0).all():
         rel[:] = 0
     return rel
+
+
+def morton_order(xyz: torch.Tensor, bits: int = 10) -> torch.Tensor:
+    """Permutation that lists the points (N,3) along a Z-order curve over their bounding box (`bits` bits per
+    axis; ties keep index order).  The reference stores a submodel's Gaussians in the order its loader met them
+    (scene/gaussian_nn_module.py:176-192, a boolean mask over the file's order); stored along the curve instead,
+    the Gaussians a camera sees lie together in memory, and the per-Gaussian kernels, which read the rows of the
+    visible ones only, read runs of rows instead of every third row."""
+    if xyz.numel() == 0:
+        return torch.zeros(0, dtype=torch.long, device=xyz.device)
+    low = xyz.min(dim=0).values
+    extent = (xyz.max(dim=0).values - low).clamp_min(1e-12)
+    cells = ((xyz - low) / extent * (2 ** bits - 1)).round().to(torch.long).clamp_(0, 2 ** bits - 1)
+    code = torch.zeros(xyz.shape[0], dtype=torch.long, device=xyz.device)
+    for b in range(bits):
+        for axis in range(3):
+            code |= ((cells[:, axis] >> b) & 1) << (3 * b + axis)
+    return torch.argsort(code, stable=True)
+

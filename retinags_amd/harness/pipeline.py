@@ -42,15 +42,32 @@ class Submodel:
         return self
 
 
-def submodels_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device) -> List[Submodel]:
+def submodels_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device, order: str = "given") -> List[Submodel]:
+    """A submodel's Gaussians (its own and the straddlers lent to it) as renderer inputs.  order: "given" keeps the
+    order of part.members (the reference's: own Gaussians in file order, then the lent ones by lender); "morton"
+    stores them along a Z-order curve (partition.morton_order), which changes nothing but the order of the rows."""
+    from .partition import morton_order
+    if order not in ("given", "morton"):
+        raise ValueError("order must be 'given' or 'morton'")
     subs = []
     for k, ids in enumerate(part.members):
         idx = ids if torch.is_tensor(ids) else torch.from_numpy(ids)
+        if order == "morton":
+            idx = idx[morton_order(scene["xyz"][idx.to(scene["xyz"].device)]).to(idx.device)]
         pick = lambda t: t[idx.to(t.device)].to(device).contiguous()
         subs.append(Submodel(pick(scene["xyz"]), pick(scene["opacity"]), pick(scene["scales"]),
                              pick(scene["rotations"]), pick(scene["shs"]),
                              torch.from_numpy(part.box_low[k]).to(device), torch.from_numpy(part.box_up[k]).to(device)))
     return subs
+
+
+def reorder_submodel(sub: Submodel, permutation: torch.Tensor) -> Submodel:
+    """The same submodel with its Gaussians stored in another order (row k of every tensor becomes row
+    permutation[k] of the old one); a screen-space placeholder, if any, is dropped."""
+    flag = sub.means3D.requires_grad
+    take = lambda t: t.detach()[permutation.to(t.device)].contiguous().requires_grad_(flag)
+    return Submodel(take(sub.means3D), take(sub.opacity), take(sub.scales), take(sub.rotations), take(sub.shs), sub.range_low,
+                    sub.range_up, sub.active_sh_degree)
 
 
 def owned_models_from_partition(scene: Dict[str, torch.Tensor], part: Partition, device,

@@ -234,3 +234,20 @@ def test_partition_by_tensor_operations_matches_the_numpy_partition():
         assert np.array_equal(host.box_low, other.box_low) and np.array_equal(host.box_up, other.box_up)
         assert np.array_equal(host.owner, other.owner.numpy())
         assert all(np.array_equal(a, b.numpy()) for a, b in zip(host.members, other.members))
+
+
+def test_morton_order_is_a_permutation_that_keeps_neighbours_together():
+    """The Z-order storage offered for a submodel's Gaussians: every point once, ties in index order, and points that
+    are consecutive in the order lie far closer together on average than points that are consecutive as given."""
+    import torch
+    from retinags_amd.harness import partition
+    g = torch.Generator().manual_seed(3)
+    xyz = torch.rand(20_000, 3, generator=g) * torch.tensor([20.0, 20.0, 0.5])
+    order = partition.morton_order(xyz)
+    assert order.dtype == torch.long and torch.equal(torch.sort(order).values, torch.arange(20_000))
+    step_given = (xyz[1:] - xyz[:-1]).norm(dim=1).mean()
+    step_sorted = (xyz[order][1:] - xyz[order][:-1]).norm(dim=1).mean()
+    assert float(step_sorted) < 0.1 * float(step_given)
+    same = torch.zeros(7, 3)
+    assert torch.equal(partition.morton_order(same), torch.arange(7))          # stable
+    assert partition.morton_order(torch.zeros(0, 3)).numel() == 0
