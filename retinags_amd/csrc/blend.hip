@@ -52,18 +52,14 @@ __device__ __forceinline__ bool clipped_by_box(const PixelRay& ray, float w, con
 	return (wx <= b.lo.x) || (wx > b.hi.x) || (wy <= b.lo.y) || (wy > b.hi.y) || (wz <= b.lo.z) || (wz > b.hi.z);
 }
 
-// exp(x) for the exponents of the blend (x <= 0, modest magnitude): 2^(x log2 e) on the
-// hardware exp2 unit, with the rounding error of the product x * log2(e) folded back in, which
-// keeps the relative error at about one unit in the last place.  Forward and backward use
-// the same function, so they take the same per-pixel decisions.
+// exp(x) for the exponents of the blend (-6 < x <= 0 where the result is used): 2^(x log2 e) on the hardware exp2 unit.
+// The product's rounding (half a unit in the last place of a number below 8) and the unit's own leave the result within
+// four units in the last place, the class of a library expf; the decisions taken on it (alpha against 1/255, the
+// transmittance against 1e-4) agree with an exact evaluation except within a few 1e-7 of their thresholds.  Forward
+// and backward use the same function, so they take the same per-pixel decisions.
 __device__ __forceinline__ float exp_of_exponent(float x)
 {
-	const float kLog2eHi = 1.44269502e+0f, kLog2eLo = 1.92596303e-8f;
-	const float t = x * kLog2eHi;
-	float r = __builtin_fmaf(x, kLog2eHi, -t);
-	r = __builtin_fmaf(x, kLog2eLo, r);
-	const float e = __builtin_amdgcn_exp2f(t);
-	return __builtin_fmaf(e, r * 0.693147182f, e);
+	return __builtin_amdgcn_exp2f(x * 1.44269502e+0f);
 }
 
 // Launch-order classes of the backward's strips, by the number of entries they have to walk.
@@ -101,6 +97,16 @@ __device__ __forceinline__ float exponent_of(const float4 g, const float4 co, co
 {
 	d = float2{g.x - pixf.x, g.y - pixf.y};
 	return -0.5f * (co.x * d.x * d.x + co.z * d.y * d.y) - co.y * d.x * d.y;
+}
+
+// The blend kernels stage a conic as (-xx / 2, -xy, -yy / 2, opacity): scaling by a power of two and negation commute
+// with rounding, so the exponent below has the very bits of exponent_of() on the conic as stored, one multiplication less
+// per pixel and entry.
+__device__ __forceinline__ float4 staged_conic(const float4 co) { return float4{-0.5f * co.x, -co.y, -0.5f * co.z, co.w}; }
+__device__ __forceinline__ float exponent_of_staged(const float4 g, const float4 sc, const float2 pixf)
+{
+	const float dx = g.x - pixf.x, dy = g.y - pixf.y;
+	return (sc.x * dx * dx + sc.z * dy * dy) + sc.y * dx * dy;
 }
 
 // ---- filing ------------------------------------------------------------------------------------
@@ -255,18 +261,16 @@ __global__ __launch_bounds__(kFileBlock) void strip_file_place_kernel(BlendBatch
 
 struct ForwardPixel {
 	float T, C0, C1, C2, weight, D;
-	uint32_t last_contributor;
-	uint32_t last_filed;  // like last_contributor, but counted in entries filed for the strip
+	uint32_t last_filed;  // the last entry blended, counted in entries filed for the strip (1-based; 0: none)
 };
 
 struct ForwardStage {  // one per workgroup (a single wavefront)
-	// The chunk's entries once per 8-pixel-wide half of the strip they can reach, each half's packed to the front:
+	// The chunk's entries once per 8-pixel-wide half of the strip they can reach, each half's packed to the front, so
+	// that a step's reads are at addresses known when the step begins:
 	float4 geom[2][kChunk + 3];   // pixel x, pixel y, exponent floor, clip w (NaN: strip inside the box)
-	float4 conic[2][kChunk + 3];  // conic xx, xy, yy, opacity
+	float4 conic[2][kChunk + 3];  // staged_conic(): -xx / 2, -xy, -yy / 2, opacity
+	float4 cd[2][kChunk];         // r, g, b, view depth: what only a blended sample uses
 	uint8_t entry[2][kChunk + 4]; // which entry of the chunk a packed slot holds
-	// and once per entry of the chunk, what only a blended sample reads:
-	float4 cd[kChunk];            // r, g, b, view depth
-	uint32_t position[kChunk];    // 1-based position in the tile list
 };
 
 // `first` is the number of entries filed for the strip ahead of the chunk; `slot` is the packed slot in the
@@ -280,32 +284,34 @@ __device__ __forceinline__ void forward_visit(ForwardPixel& p, uint64_t& done, u
 	const uint64_t taking = candidates & ~done;
 	if (taking == 0ull)
 		return;
-	bool finished = false;
-	if (__builtin_amdgcn_inverse_ballot_w64(taking)) {
-		const float clip_w = g.w;  // NaN: the whole strip is inside the box
-		const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
-		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, box))) {
-			const float test_T = p.T * (1 - alpha);
-			if (test_T < 0.0001f) {
-				finished = true;
-			} else {
-				const uint32_t entry = st.entry[half][slot];
-				const float4 cd = st.cd[entry];
-				// The sums feed no decision (the images are compared by tolerance): one product alpha T and a fused
-				// multiply-add per channel instead of the reference's two products and an add each (forward.cu:378-385).
-				const float weight = alpha * p.T;
-				p.C0 = __builtin_fmaf(cd.x, weight, p.C0);
-				p.C1 = __builtin_fmaf(cd.y, weight, p.C1);
-				p.C2 = __builtin_fmaf(cd.z, weight, p.C2);
-				p.weight += weight;
-				p.D = __builtin_fmaf(cd.w, weight, p.D);
-				p.T = test_T;
-				p.last_contributor = st.position[entry];
-				p.last_filed = first + entry + 1u;
-			}
-		}
+	// Every lane evaluates alpha and the transmittance behind the entry (an instruction costs the wavefront the same
+	// whatever its lanes), and the decisions are kept as lane masks: no branch, and no flag in a register, per decision.
+	// (the entry's colour is asked for ahead of its use in the masked region: the wait falls behind the exp)
+	const float4 cd = st.cd[half][slot];
+	const uint32_t entry = st.entry[half][slot];
+	const float alpha = fminf(0.99f, co.w * exp_of_exponent(power));
+	const float test_T = p.T * (1 - alpha);
+	uint64_t ok = taking & lanes_where(!(alpha < 1.0f / 255.0f));
+	const float clip_w = g.w;  // the same for every lane; NaN: the whole strip is inside the box
+	if (lanes_where(clip_w == clip_w) != 0ull)
+		ok &= lanes_where(!clipped_by_box(ray, clip_w, box));
+	const uint64_t finished = ok & lanes_where(test_T < 0.0001f);
+	done |= finished;
+	const uint64_t blending = ok & ~finished;
+	if (blending == 0ull)
+		return;
+	if (__builtin_amdgcn_inverse_ballot_w64(blending)) {
+		// The sums feed no decision (the images are compared by tolerance): one product alpha T and a fused
+		// multiply-add per channel instead of the reference's two products and an add each (forward.cu:378-385).
+		const float weight = alpha * p.T;
+		p.C0 = __builtin_fmaf(cd.x, weight, p.C0);
+		p.C1 = __builtin_fmaf(cd.y, weight, p.C1);
+		p.C2 = __builtin_fmaf(cd.z, weight, p.C2);
+		p.weight += weight;
+		p.D = __builtin_fmaf(cd.w, weight, p.D);
+		p.T = test_T;
+		p.last_filed = first + entry + 1u;
 	}
-	done |= lanes_where(finished);
 }
 
 // Number of set bits of a ballot below the calling lane.
@@ -342,7 +348,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
 	const BoxFrame box = load_box_frame(a);
 
-	ForwardPixel p = {1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u, 0u};
+	ForwardPixel p = {1.0f, 0.f, 0.f, 0.f, 0.f, 0.f, 0u};
 	uint64_t done = lanes_where(!inside);
 	uint64_t live = ~done;
 	// the entries filed for this strip, in list order: list position, bit 31 = strip inside the box
@@ -400,18 +406,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 				float4 g = cur.geom;
 				if (pos_cur & 0x80000000u)
 					g.w = __int_as_float(0x7FC00000);  // the strip lies inside the box: no per-pixel test
-				st.cd[lane] = cur.cd;
-				st.position[lane] = (pos_cur & kPosition) + 1u;
 				if (left) {
 					const uint32_t r = lanes_below(in_left);
 					st.geom[0][r] = g;
-					st.conic[0][r] = cur.conic;
+					st.conic[0][r] = staged_conic(cur.conic);
+					st.cd[0][r] = cur.cd;
 					st.entry[0][r] = (uint8_t)lane;
 				}
 				if (right) {
 					const uint32_t r = lanes_below(in_right);
 					st.geom[1][r] = g;
-					st.conic[1][r] = cur.conic;
+					st.conic[1][r] = staged_conic(cur.conic);
+					st.cd[1][r] = cur.cd;
 					st.entry[1][r] = (uint8_t)lane;
 				}
 			}
@@ -438,9 +444,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 			for (int k = 0; k < steps && live != 0ull; k += 4) {
 				const float4 g0 = geom[k], g1 = geom[k + 1], g2 = geom[k + 2], g3 = geom[k + 3];
 				const float4 c0 = conic[k], c1 = conic[k + 1], c2 = conic[k + 2], c3 = conic[k + 3];
-				float2 d;
-				const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
-				            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
+				const float w0 = exponent_of_staged(g0, c0, pixf), w1 = exponent_of_staged(g1, c1, pixf),
+				            w2 = exponent_of_staged(g2, c2, pixf), w3 = exponent_of_staged(g3, c3, pixf);
 				// written with negations so that a NaN exponent is kept, as in the exact loop; each mask from single
 				// comparisons (a comparison's result is the mask; that of a combined flag is formed through a register)
 				const uint64_t q0 = lanes_where(!(w0 > 0.0f)) & lanes_where(!(w0 < g0.z)),
@@ -470,7 +475,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 	}
 	if (inside) {
 		const size_t plane = (size_t)a.H * a.W;
-		a.n_contrib[pix_id] = p.last_contributor;
+		// the reference's n_contrib: the 1-based position in the tile's list of the last entry the pixel blended
+		uint32_t last_contributor = 0u;
+		if (p.last_filed != 0u) {
+			const uint32_t* filed_list = a.strip_lists + 4 * (size_t)range.x + (size_t)wave * n;
+			last_contributor = (filed_list[p.last_filed - 1u] & 0x7FFFFFFFu) + 1u;
+		}
+		a.n_contrib[pix_id] = last_contributor;
 		a.out_color[pix_id] = p.C0 + p.T * a.bg[0];
 		a.out_color[plane + pix_id] = p.C1 + p.T * a.bg[1];
 		a.out_color[2 * plane + pix_id] = p.C2 + p.T * a.bg[2];
@@ -587,7 +598,7 @@ struct BackwardPixel {
 
 struct BackwardStage {  // wave-private
 	float4 geom[kChunk + 3];  // + padding up to a multiple of four entries
-	float4 conic[kChunk + 3];
+	float4 conic[kChunk + 3];  // staged_conic(): -xx / 2, -xy, -yy / 2, opacity
 	float4 cd[kChunk];
 	uint32_t entry[kChunk + 3];  // 0-based position in the tile list
 	uint32_t id[kChunk];
@@ -607,10 +618,15 @@ __device__ __forceinline__ float dpp_exchange_add(float v)
 	return v + __builtin_bit_cast(float, moved);
 }
 
-// Entry-parallel part for the first `rows` rows.  Lane (e = lane >> 3, h = (lane >> 1) & 3, half = lane & 1)
-// sums row e over the 8 pixels of one half of strip row h; the eight lanes of an entry then add up what
-// they hold (three exchanges inside their group of eight) and add the entry's ten sums into the Gaussian's
-// row of `sums`: eight neighbouring columns in one atomic instruction, the last two in a second.
+// Entry-parallel part for the first `rows` rows.  A 16-lane row of the wavefront serves two entries, e in its low
+// eight lanes and e + 4 in its high eight; lane (h = (lane >> 1) & 3, half = lane & 1) of the eight
+// sums the entry's row over the 8 pixels of one half of strip row h; the eight lanes of an entry then add up what
+// they hold (three exchanges inside their group of eight) and the entry's ten sums go into the Gaussian's
+// row of `sums` with one atomic instruction: the entry's own lanes add columns 0-7, two lanes of the other eight of
+// the 16-lane row add columns 8 and 9, so a first instruction serves entries 0-3 and a second one entries 4-7.
+// (Adding columns 0-7 of all eight entries first and columns 8-9 after them, which needs no exchange between the
+// groups, had every request of the second instruction hit a cache line that one of the first was still at work on:
+// measured, that second instruction cost eight times what the first did, a fifth of the kernel's time.)
 // `row_slots` holds, one byte per row, which staged entry of the current chunk the row belongs to: the entry's centre,
 // conic and Gaussian are read from where the chunk was staged (so the rows are flushed before the next chunk is).
 // kDepth: a gradient arrived for the depth image (without one, the usual case of a loss on the colour image alone, the
@@ -621,7 +637,8 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 {
 #pragma clang fp contract(fast)
 	__builtin_amdgcn_wave_barrier();
-	const int e = lane >> 3, h = (lane >> 1) & 3, half = lane & 1, j = lane & 7;
+	const int upper = (lane >> 3) & 1;  // which eight of the 16-lane row
+	const int e = (lane >> 4) + 4 * upper, h = (lane >> 1) & 3, half = lane & 1, j = lane & 7;
 	const int slot = (int)((row_slots >> (8 * e)) & 0xFFull);
 	const float4 centre = st.geom[slot];
 	const float2 xy = {centre.x, centre.y};
@@ -658,64 +675,83 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 		v[q] = dpp_exchange_add<0x4E>(v[q]);   // quad_perm:[2,3,0,1]
 		v[q] = dpp_exchange_add<0x141>(v[q]);  // row_half_mirror: the other quad of the eight
 	}
+	float first = 0.f, second = 0.f;
+	uint32_t id = 0u;
 	if (e < rows) {
 		const float4 co = st.conic[slot];
 		const float S0 = v[0], Sx = v[1], Sy = v[2], Sxx = v[3], Sxy = v[4], Syy = v[5];
-		const float m0 = -co.w * f.ddelx_dx * (co.x * Sx + co.y * Sy);
-		const float m1 = -co.w * f.ddely_dy * (co.z * Sy + co.y * Sx);
+		// (co is the staged conic: -xx / 2, -xy, -yy / 2, opacity)
+		const float m0 = co.w * f.ddelx_dx * (2.f * co.x * Sx + co.y * Sy);
+		const float m1 = co.w * f.ddely_dy * (2.f * co.z * Sy + co.y * Sx);
 		const float k0 = -0.5f * co.w * Sxx, k1 = -0.5f * co.w * Sxy, k3 = -0.5f * co.w * Syy;
-		// lane j of the eight takes column j of the row, lanes 0 and 1 also columns 8 and 9: see SumCol
-		const float first = j == 0 ? m0 : j == 1 ? m1 : j == 2 ? k0 : j == 3 ? k1 : j == 4 ? k3 : j == 5 ? S0 : j == 6 ? v[6] : v[7];
-		const float second = j == 0 ? v[8] : j == 1 ? v[9] : 0.f;
-		float* row = a.sums + (size_t)kSumCols * st.id[slot] + j;
-		if (first != 0.f) unsafeAtomicAdd(row, first);
-		if (second != 0.f) unsafeAtomicAdd(row + 8, second);
+		// lane j of the eight holds column j of the row, lanes 0 and 1 also columns 8 and 9: see SumCol
+		first = j == 0 ? m0 : j == 1 ? m1 : j == 2 ? k0 : j == 3 ? k1 : j == 4 ? k3 : j == 5 ? S0 : j == 6 ? v[6] : v[7];
+		second = j == 0 ? v[8] : j == 1 ? v[9] : 0.f;
+		id = st.id[slot];
+	}
+	// columns 8 and 9 and the Gaussian's index go to the same lanes of the other eight of the 16-lane row (row_ror:8)
+	const float second_there = __builtin_bit_cast(
+		float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, second), 0x128, 0xF, 0xF, true));
+	const uint32_t id_there = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)id, 0x128, 0xF, 0xF, true);
+	{
+		// entries 0-3: their own (lower) lanes add columns 0-7, the upper lanes columns 8 and 9 for them
+		const float value = upper ? second_there : first;
+		float* at = a.sums + (size_t)kSumCols * (upper ? id_there : id) + (upper ? 8 + j : j);
+		if (value != 0.f) unsafeAtomicAdd(at, value);
+	}
+	{
+		// entries 4-7: the other way round
+		const float value = upper ? first : second_there;
+		float* at = a.sums + (size_t)kSumCols * (upper ? id : id_there) + (upper ? j : 8 + j);
+		if (value != 0.f) unsafeAtomicAdd(at, value);
 	}
 	__builtin_amdgcn_wave_barrier();
 }
 
 // Pixel-parallel part for one entry; `rows` (wave-uniform) counts the LDS rows in use.
 template <bool kDepth>
-__device__ __forceinline__ void backward_visit(BackwardPixel& p, bool candidate, float power, const float4 g,
+__device__ __forceinline__ void backward_visit(BackwardPixel& p, uint64_t candidates, float power, const float4 g,
                                                const float4 co, BackwardStage& st, int slot, int& rows, uint64_t& row_slots,
                                                const StripFrame& f, const PixelRay& ray, const BlendArgs& a, int lane)
 {
-	if (lanes_where(candidate) == 0ull)
+	if (candidates == 0ull)
+		return;
+	// Every lane evaluates alpha (an instruction costs the wavefront the same whatever its lanes); the decisions are
+	// lane masks, and one masked region holds what only a blended sample computes.
+	const float4 cd = st.cd[slot];  // asked for ahead of its use in the masked region: the wait falls behind the exp
+	const float G = exp_of_exponent(power);
+	const float alpha = fminf(0.99f, co.w * G);
+	uint64_t blended = candidates & lanes_where(!(alpha < 1.0f / 255.0f));
+	// the box and the inverse projection are read where they are needed (few strips straddle a face of their
+	// box): kept in scalar registers for the whole walk they crowd out the candidate masks of a step
+	const float clip_w = g.w;  // the same for every lane; NaN: the whole strip is inside the box
+	if (lanes_where(clip_w == clip_w) != 0ull)
+		blended &= lanes_where(!clipped_by_box(ray, clip_w, load_box_frame(a)));
+	if (blended == 0ull)
 		return;
 	float u = 0.f, aT = 0.f;
-	const float clip_w = wave_uniform(g.w);  // NaN: the whole strip is inside the box
-	if (candidate) {
-		const float G = exp_of_exponent(power);
-		const float alpha = fminf(0.99f, co.w * G);
-		// the box and the inverse projection are read where they are needed (few strips straddle a face of their
-		// box): kept in scalar registers for the whole walk they crowd out the candidate masks of a step
-		if (!(alpha < 1.0f / 255.0f) && !((clip_w == clip_w) && clipped_by_box(ray, clip_w, load_box_frame(a)))) {
-			// From here on nothing feeds a decision: gradients are compared by tolerance, so the
-			// compiler may contract multiply-adds and the divisions use the hardware reciprocal.
+	if (__builtin_amdgcn_inverse_ballot_w64(blended)) {
+		// From here on nothing feeds a decision: gradients are compared by tolerance, so the
+		// compiler may contract multiply-adds and the divisions use the hardware reciprocal.
 #pragma clang fp contract(fast)
-			const float inv_one_minus_alpha = __builtin_amdgcn_rcpf(1.f - alpha);
-			p.T = p.T * inv_one_minus_alpha;
-			aT = alpha * p.T;
-			const float4 cd = st.cd[slot];
-			// The pixel's outputs are sums over its blended entries j of w_j (colour_j, depth_j, 1) with w_j = alpha_j T_j,
-			// T_j the product of (1 - alpha_k) over the entries in front, plus T_final times the background.  Their
-			// derivative with respect to alpha_i is T_i (colour_i, depth_i, 1) minus (the sum over the entries behind i +
-			// T_final background) / (1 - alpha_i).  The reference carries that sum per channel and per unit of transmittance
-			// (K/cuda_rasterizer_hgs/backward.cu:568-599: accum_rec = last_alpha * last_color + (1 - last_alpha) * accum_rec,
-			// and the background term apart); only its product with the upstream gradient is needed, so one number per
-			// pixel does for all channels: `behind` = sum over the entries behind of w_j <g, (colour_j, depth_j, 1)> +
-			// T_final <g, background>, started with the latter.  Same quantity, a third of the arithmetic.
-			float weighted = __builtin_fmaf(cd.x, p.g_r, __builtin_fmaf(cd.y, p.g_g, __builtin_fmaf(cd.z, p.g_b, p.g_alpha)));
-			if (kDepth)
-				weighted = __builtin_fmaf(cd.w, p.g_depth, weighted);
-			const float dL_dopa = weighted * p.T - p.behind * inv_one_minus_alpha;
-			p.behind = __builtin_fmaf(aT, weighted, p.behind);
-			u = G * dL_dopa;
-		}
+		const float inv_one_minus_alpha = __builtin_amdgcn_rcpf(1.f - alpha);
+		p.T = p.T * inv_one_minus_alpha;
+		aT = alpha * p.T;
+		// The pixel's outputs are sums over its blended entries j of w_j (colour_j, depth_j, 1) with w_j = alpha_j T_j,
+		// T_j the product of (1 - alpha_k) over the entries in front, plus T_final times the background.  Their
+		// derivative with respect to alpha_i is T_i (colour_i, depth_i, 1) minus (the sum over the entries behind i +
+		// T_final background) / (1 - alpha_i).  The reference carries that sum per channel and per unit of transmittance
+		// (K/cuda_rasterizer_hgs/backward.cu:568-599: accum_rec = last_alpha * last_color + (1 - last_alpha) * accum_rec,
+		// and the background term apart); only its product with the upstream gradient is needed, so one number per
+		// pixel does for all channels: `behind` = sum over the entries behind of w_j <g, (colour_j, depth_j, 1)> +
+		// T_final <g, background>, started with the latter.  Same quantity, a third of the arithmetic.
+		float weighted = __builtin_fmaf(cd.x, p.g_r, __builtin_fmaf(cd.y, p.g_g, __builtin_fmaf(cd.z, p.g_b, p.g_alpha)));
+		if (kDepth)
+			weighted = __builtin_fmaf(cd.w, p.g_depth, weighted);
+		const float dL_dopa = weighted * p.T - p.behind * inv_one_minus_alpha;
+		p.behind = __builtin_fmaf(aT, weighted, p.behind);
+		u = G * dL_dopa;
 	}
-	// (a lane that took part has a weight alpha T > 0, or a NaN; asked of the weight, the mask comes from one comparison)
-	if (lanes_where(!(aT <= 0.f)) == 0ull)
-		return;
 	st.u_at[rows * kRowStride + row_column(lane)] = float2{u, aT};
 	row_slots |= (uint64_t)slot << (8 * rows);
 	rows++;
@@ -795,7 +831,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 			if (pos_cur & 0x80000000u)
 				g.w = __int_as_float(0x7FC00000);  // the strip lies inside the box: no per-pixel test
 			st.geom[lane] = g;
-			st.conic[lane] = cur.conic;
+			st.conic[lane] = staged_conic(cur.conic);
 			st.cd[lane] = cur.cd;
 			st.entry[lane] = pos_cur & kPosition;
 			st.id[lane] = cur.id;
@@ -818,21 +854,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 			const float4 g0 = st.geom[k], g1 = st.geom[k + 1], g2 = st.geom[k + 2], g3 = st.geom[k + 3];
 			const float4 c0 = st.conic[k], c1 = st.conic[k + 1], c2 = st.conic[k + 2], c3 = st.conic[k + 3];
 			const uint32_t p0 = st.entry[k], p1 = st.entry[k + 1], p2 = st.entry[k + 2], p3 = st.entry[k + 3];
-			float2 d;
-			const float w0 = exponent_of(g0, c0, pixf, d), w1 = exponent_of(g1, c1, pixf, d),
-			            w2 = exponent_of(g2, c2, pixf, d), w3 = exponent_of(g3, c3, pixf, d);
-			// Each entry's candidates are formed right where its visit looks at them (the visit starts with their
-			// ballot): nearly every walked entry has some, so a test for the four together would save little, and
-			// four sets of flags kept alive across the visits are packed into a byte mask by the compiler, a dozen
-			// vector instructions per step.
-			backward_visit<kDepth>(p, (p0 < last_contributor) && !(w0 > 0.0f) && !(w0 < g0.z), w0, g0, c0, st, k, rows, row_slots, frame,
-			               ray, a, lane);
-			backward_visit<kDepth>(p, (p1 < last_contributor) && !(w1 > 0.0f) && !(w1 < g1.z), w1, g1, c1, st, k + 1, rows, row_slots,
-			               frame, ray, a, lane);
-			backward_visit<kDepth>(p, (p2 < last_contributor) && !(w2 > 0.0f) && !(w2 < g2.z), w2, g2, c2, st, k + 2, rows, row_slots,
-			               frame, ray, a, lane);
-			backward_visit<kDepth>(p, (p3 < last_contributor) && !(w3 > 0.0f) && !(w3 < g3.z), w3, g3, c3, st, k + 3, rows, row_slots,
-			               frame, ray, a, lane);
+			const float w0 = exponent_of_staged(g0, c0, pixf), w1 = exponent_of_staged(g1, c1, pixf),
+			            w2 = exponent_of_staged(g2, c2, pixf), w3 = exponent_of_staged(g3, c3, pixf);
+			// Each entry's candidates are formed right where its visit looks at them: nearly every walked entry has
+			// some, so a test for the four together would save little.  Each mask comes from single comparisons (a
+			// comparison's result is the mask; that of a combined flag is formed through a register).
+			backward_visit<kDepth>(p, lanes_where(p0 < last_contributor) & lanes_where(!(w0 > 0.0f)) & lanes_where(!(w0 < g0.z)), w0,
+			                       g0, c0, st, k, rows, row_slots, frame, ray, a, lane);
+			backward_visit<kDepth>(p, lanes_where(p1 < last_contributor) & lanes_where(!(w1 > 0.0f)) & lanes_where(!(w1 < g1.z)), w1,
+			                       g1, c1, st, k + 1, rows, row_slots, frame, ray, a, lane);
+			backward_visit<kDepth>(p, lanes_where(p2 < last_contributor) & lanes_where(!(w2 > 0.0f)) & lanes_where(!(w2 < g2.z)), w2,
+			                       g2, c2, st, k + 2, rows, row_slots, frame, ray, a, lane);
+			backward_visit<kDepth>(p, lanes_where(p3 < last_contributor) & lanes_where(!(w3 > 0.0f)) & lanes_where(!(w3 < g3.z)), w3,
+			                       g3, c3, st, k + 3, rows, row_slots, frame, ray, a, lane);
 		}
 		// the rows point into this chunk's staged entries: they go before the next chunk takes their place
 		if (rows > 0) {
