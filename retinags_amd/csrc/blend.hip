@@ -675,19 +675,21 @@ __device__ __forceinline__ void flush_rows(const BackwardStage& st, int rows, ui
 		v[q] = dpp_exchange_add<0x4E>(v[q]);   // quad_perm:[2,3,0,1]
 		v[q] = dpp_exchange_add<0x141>(v[q]);  // row_half_mirror: the other quad of the eight
 	}
-	float first = 0.f, second = 0.f;
-	uint32_t id = 0u;
-	if (e < rows) {
-		const float4 co = st.conic[slot];
-		const float S0 = v[0], Sx = v[1], Sy = v[2], Sxx = v[3], Sxy = v[4], Syy = v[5];
-		// (co is the staged conic: -xx / 2, -xy, -yy / 2, opacity)
-		const float m0 = co.w * f.ddelx_dx * (2.f * co.x * Sx + co.y * Sy);
-		const float m1 = co.w * f.ddely_dy * (2.f * co.z * Sy + co.y * Sx);
-		const float k0 = -0.5f * co.w * Sxx, k1 = -0.5f * co.w * Sxy, k3 = -0.5f * co.w * Syy;
-		// lane j of the eight holds column j of the row, lanes 0 and 1 also columns 8 and 9: see SumCol
-		first = j == 0 ? m0 : j == 1 ? m1 : j == 2 ? k0 : j == 3 ? k1 : j == 4 ? k3 : j == 5 ? S0 : j == 6 ? v[6] : v[7];
-		second = j == 0 ? v[8] : j == 1 ? v[9] : 0.f;
-		id = st.id[slot];
+	// (every lane forms all five products and then picks its own: a handful of multiplications more than the one or
+	// two a lane needs, but no branch per column and no wait for the conic inside one)
+	const float4 co = st.conic[slot];  // the staged conic: -xx / 2, -xy, -yy / 2, opacity
+	const uint32_t id = e < rows ? st.id[slot] : 0u;
+	const float S0 = v[0], Sx = v[1], Sy = v[2], Sxx = v[3], Sxy = v[4], Syy = v[5];
+	const float m0 = co.w * f.ddelx_dx * (2.f * co.x * Sx + co.y * Sy);
+	const float m1 = co.w * f.ddely_dy * (2.f * co.z * Sy + co.y * Sx);
+	const float half_w = -0.5f * co.w;
+	const float k0 = half_w * Sxx, k1 = half_w * Sxy, k3 = half_w * Syy;
+	// lane j of the eight holds column j of the row, lanes 0 and 1 also columns 8 and 9: see SumCol
+	float first = j == 0 ? m0 : j == 1 ? m1 : j == 2 ? k0 : j == 3 ? k1 : j == 4 ? k3 : j == 5 ? S0 : j == 6 ? v[6] : v[7];
+	float second = j == 0 ? v[8] : j == 1 ? v[9] : 0.f;
+	if (!(e < rows)) {
+		first = 0.f;
+		second = 0.f;
 	}
 	// columns 8 and 9 and the Gaussian's index go to the same lanes of the other eight of the 16-lane row (row_ror:8)
 	const float second_there = __builtin_bit_cast(
