@@ -343,7 +343,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
 	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
-	const uint32_t pix_id = (uint32_t)a.W * py + px;
 	const float2 pixf = {(float)px, (float)py};
 	const PixelRay ray = {pix_to_ndc(pixf.x, a.W), pix_to_ndc(pixf.y, a.H)};
 	const BoxFrame box = load_box_frame(a);
@@ -421,14 +420,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 					st.entry[1][r] = (uint8_t)lane;
 				}
 			}
-			// both halves are walked for `padded` slots: the rest get entries that never pass the floor test
+			// both halves are walked for `padded` slots: the rest get entries that never pass the floor test (an
+			// infinite floor; their conic may be any finite one, and the lane's own record is at hand: a real one or zeros)
 			if (lane >= n_left && lane < padded) {
 				st.geom[0][lane] = float4{0.f, 0.f, INFINITY, 0.f};
-				st.conic[0][lane] = float4{0.f, 0.f, 0.f, 0.f};
+				st.conic[0][lane] = cur.conic;
 			}
 			if (lane >= n_right && lane < padded) {
 				st.geom[1][lane] = float4{0.f, 0.f, INFINITY, 0.f};
-				st.conic[1][lane] = float4{0.f, 0.f, 0.f, 0.f};
+				st.conic[1][lane] = cur.conic;
 			}
 			__builtin_amdgcn_wave_barrier();
 			// the chunk is in LDS now: its registers take the next chunk's records, loaded during the walk
@@ -466,14 +466,17 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6, 6))) void
 
 	{
 		// how many of the filed entries the backward has to walk: up to the last one some pixel blended
-		uint32_t upto = inside ? p.last_filed : 0u;
-#pragma unroll
-		for (int off = 32; off > 0; off >>= 1)
-			upto = max(upto, (uint32_t)__shfl_xor((int)upto, off));
+		const uint32_t upto = filed != 0u ? wave_max_u32(p.last_filed) : 0u;  // (zero for a pixel outside the image)
 		if (lane == 0)
 			a.strip_filed[strip_id] = upto;
 	}
-	if (inside) {
+	// (the pixel's place is worked out again from the lane, made opaque: kept from the start it would hold a register
+	// through the whole walk, one more than the kernel's wavefronts per SIMD leave it)
+	int lane_again = lane;
+	asm volatile("" : "+v"(lane_again));
+	const uint32_t out_x = tx * kTile + (lane_again & 15), out_y = ty * kTile + wave * 4 + (lane_again >> 4);
+	if (out_x < (uint32_t)a.W && out_y < (uint32_t)a.H) {
+		const uint32_t pix_id = (uint32_t)a.W * out_y + out_x;
 		const size_t plane = (size_t)a.H * a.W;
 		// the reference's n_contrib: the 1-based position in the tile's list of the last entry the pixel blended
 		uint32_t last_contributor = 0u;

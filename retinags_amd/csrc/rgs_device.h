@@ -173,6 +173,19 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v)
 	return v;
 }
 
+// The largest of the 64 lanes' values, the same in every lane (and in a scalar register): four exchanges inside each
+// row of 16 lanes, then one lane of each row read out.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
+{
+	v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true));   // quad_perm:[1,0,3,2]
+	v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true));   // quad_perm:[2,3,0,1]
+	v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true));  // row_half_mirror
+	v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true));  // row_mirror
+	const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16),
+	               r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+	return max(max(r0, r1), max(r2, r3));
+}
+
 // Exclusive prefix sum of one u32 per thread over a 256-thread block.
 // `lds` needs 5 words; returns the block total in `total`.
 __device__ __forceinline__ uint32_t block256_exclusive_scan_u32(uint32_t v, uint32_t* lds, uint32_t& total)
