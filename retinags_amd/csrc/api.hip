@@ -662,6 +662,7 @@ void fill_blend_args(rgs::BlendArgs& a, int P, int R, int width, int height, flo
 	a.strip_total = at<uint32_t>(img, ioff[RGS_IMG_STRIP_TOTAL]);
 	a.strip_classes = reinterpret_cast<uint32_t*>(at<uint2>(img, ioff[RGS_IMG_RANGES])) + 2 * (size_t)gx * gy;
 	a.capacity = (uint32_t)R;
+	a.gaussians = (uint32_t)P;
 	if (R > 0) {
 		const BinningPhysical b = binning_physical((size_t)R);
 		const bool sorted_in_a = (tile_sort_passes(width, height) % 2) == 0;

@@ -79,6 +79,7 @@ struct LoadedRecord {
 __device__ __forceinline__ LoadedRecord load_record(const BlendArgs& a, uint32_t id, bool in_range)
 {
 	LoadedRecord e;
+	id = min(id, a.gaussians - 1u);  // (a list that is not this frame's must not lead outside the records)
 	e.id = id;
 	if (in_range) {
 		const float4* rec = a.record + 4 * (size_t)id;
@@ -778,9 +779,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 	// the jobs of the batch take turns; each hands out its strips with the most entries first: a long
 	// strip that starts late is what the whole launch waits for
 	const BlendArgs& a = batch.job[blockIdx.x % (uint32_t)batch.count];
-	const uint32_t strip_id = a.strip_order[blockIdx.x / (uint32_t)batch.count];
+	// What the forward left in the workspaces (the strips' order, the tiles' ranges, the lists, the walk lengths) comes
+	// back through the caller's hands: every index taken from it is held inside the arrays' bounds, so that a
+	// workspace that is not the forward's (stale, or another frame's) gives wrong gradients and no stray access.
+	const uint32_t strip_id = min(a.strip_order[blockIdx.x / (uint32_t)batch.count], 4u * (uint32_t)(a.grid_x * a.grid_y) - 1u);
 	const int tile = (int)(strip_id >> 2), wave = (int)(strip_id & 3u);  // wave: which strip of the tile
-	const uint2 range = a.ranges[tile];
+	uint2 range = a.ranges[tile];
+	range.y = min(range.y, a.capacity);
+	range.x = min(range.x, range.y);
 	const int tx = tile % a.grid_x, ty = tile / a.grid_x;
 	const uint32_t px = tx * kTile + (lane & 15), py = ty * kTile + wave * 4 + (lane >> 4);
 	const bool inside = px < (uint32_t)a.W && py < (uint32_t)a.H;
@@ -794,10 +800,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 
 	// The forward blend has written down which entries of the tile's list matter to this strip
 	// (its conservative filters, not repeated here), up to the last one that any pixel blended.
-	const uint32_t filed = a.strip_filed[strip_id];
+	const uint32_t n = range.y - range.x;
+	const uint32_t filed = min(a.strip_filed[strip_id], n);
 	if (filed == 0u)
 		return;
-	const uint32_t n = range.y - range.x;
 	const uint32_t last_contributor = inside ? a.n_contrib[pix_id] : 0u;
 
 	BackwardPixel p;
@@ -826,8 +832,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 	uint32_t pos_cur = (uint32_t)lane < filed ? filed_list[filed - 1 - lane] : kNone;
 	uint32_t pos_next = (uint32_t)(64 + lane) < filed ? filed_list[filed - 1 - (64 + lane)] : kNone;
 	uint32_t pos_after = (uint32_t)(128 + lane) < filed ? filed_list[filed - 1 - (128 + lane)] : kNone;
-	LoadedRecord cur = load_record(a, pos_cur != kNone ? list[pos_cur & kPosition] : 0u, pos_cur != kNone);
-	uint32_t id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
+	LoadedRecord cur = load_record(a, pos_cur != kNone ? list[min(pos_cur & kPosition, n - 1u)] : 0u, pos_cur != kNone);
+	uint32_t id_next = pos_next != kNone ? list[min(pos_next & kPosition, n - 1u)] : 0u;
 
 	for (uint32_t first = 0; first < filed; first += 64) {
 		const int count = (int)min(filed - first, 64u);
@@ -851,7 +857,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 		cur = load_record(a, id_next, pos_next != kNone);
 		pos_cur = pos_next;
 		pos_next = pos_after;
-		id_next = pos_next != kNone ? list[pos_next & kPosition] : 0u;
+		id_next = pos_next != kNone ? list[min(pos_next & kPosition, n - 1u)] : 0u;
 		const uint32_t e3 = first + 192 + (uint32_t)lane;
 		pos_after = e3 < filed ? filed_list[filed - 1 - e3] : kNone;
 

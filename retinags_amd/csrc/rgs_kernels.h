@@ -94,6 +94,7 @@ struct BlendArgs {
 	const uint32_t* tile_keys;    // the sorted key of every list position: tile and strip bits (key_tile, key_strips)
 	const uint32_t* count_device; // non-null: the number of instances is min(capacity, *count_device)
 	uint32_t capacity;      // instances the launch is sized for
+	uint32_t gaussians;     // P: the records there are
 	const uint4* file_tail; // per kFileGroup list positions: entries filed per strip for the tile of the last of them
 	const uint32_t* sort_status;   // status words of the two sorts (may be null): non-zero = the sort gave up
 	const uint32_t* order_status;
