@@ -7,7 +7,7 @@
 // the half-Gaussian box test, T(1-alpha) < 1e-4) is evaluated with the unfused
 // single-precision expressions of K/cuda_rasterizer_hgs/forward.cu:338-392
 // (K = rasterization_kernels/diff-gaussian-rasterization-half-gaussian), so a pixel
-// can only differ from that evaluation through the last-bit behaviour of exp().
+// can only differ from that evaluation through the last bits of exp() (exp_of_exponent below).
 //
 // Blending front to back gives a strip no parallelism beyond its 64 pixels, but deciding which
 // entries of a tile's list can matter to a strip needs no order at all.  So the work is split:

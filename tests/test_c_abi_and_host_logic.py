@@ -274,3 +274,29 @@ def test_tensor_expression_branches_of_the_renderer_match_the_checker():
     scaled = pipeline.covariance_from_scaling_rotation(scene["scales"], 1.0, 3.0 * scene["rotations"])
     plain = pipeline.covariance_from_scaling_rotation(scene["scales"], 1.0, scene["rotations"])
     assert float((scaled - plain).abs().max()) <= 1e-6 * float(plain.abs().max())
+
+
+def test_exponent_of_a_conic_staged_pre_scaled_has_the_bits_of_the_reference_expression():
+    """The blend kernels keep a conic as (-xx/2, -xy, -yy/2) and evaluate
+    (sxx dx) dx + (syy dy) dy + (sxy dx) dy, one multiplication less than the reference's
+    -0.5 (xx dx dx + yy dy dy) - xy dx dy (K/cuda_rasterizer_hgs/forward.cu:353).  Scaling by a
+    power of two and negation commute with rounding, so both must give the same float32 bits,
+    operation by operation; checked here in float32 arithmetic on random conics and offsets,
+    the exponents of the same magnitudes the kernels see included."""
+    rng = np.random.default_rng(5)
+    n = 400_000
+    f = np.float32
+    xx = rng.uniform(1e-3, 3.3, n).astype(f)
+    yy = rng.uniform(1e-3, 3.3, n).astype(f)
+    xy = (rng.uniform(-0.99, 0.99, n) * np.sqrt(xx.astype(np.float64) * yy)).astype(f)
+    dx = rng.uniform(-40, 40, n).astype(f)
+    dy = rng.uniform(-40, 40, n).astype(f)
+    # a share of exact zeros and of tiny offsets
+    dx[::17] = 0
+    dy[::13] = 0
+    dx[5::29] *= f(1e-4)
+    reference = f(-0.5) * (xx * dx * dx + yy * dy * dy) - xy * dx * dy
+    sxx, sxy, syy = f(-0.5) * xx, -xy, f(-0.5) * yy
+    staged = (sxx * dx * dx + syy * dy * dy) + sxy * dx * dy
+    assert reference.dtype == np.float32 and staged.dtype == np.float32
+    assert np.array_equal(reference.view(np.uint32), staged.view(np.uint32))
