@@ -296,7 +296,8 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
  * starts recording, rgs_stage_timing(0) stops.  rgs_stage_timing_read waits for the recorded
  * work, fills up to max_stages (name, total milliseconds, launches) triples, clears the record
  * and returns the number of stages (negative on error).  The names are static strings.
- * Recording is process-wide and not thread-safe; leave it off outside measurements.  The time between two
+ * Recording is process-wide: calls from several host threads are safe but land in one record, interleaved, so
+ * measure from one thread and leave it off otherwise.  The time between two
  * consecutive events is charged to the earlier one's stage, which takes a single stream: while recording is on,
  * rgs_frame_backward does not use a second stream. */
 int rgs_stage_timing(int enable);

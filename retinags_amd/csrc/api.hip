@@ -4,6 +4,7 @@
 #include "../../include/rgs.h"
 #include "rgs_kernels.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -63,8 +64,12 @@ int check_stage(const char* stage, hipStream_t s, int debug)
 // While enabled, every launcher records a HIP event on the caller's stream before its kernel
 // (rgs::stage_mark) and every entry point records one when it has queued its last kernel.
 // The time between two consecutive events is charged to the earlier event's stage.
+// The record is one per process.  Entry points may be called from several host threads: the switch is atomic (it is all
+// a call looks at while recording is off) and the record itself is taken under a lock, so concurrent calls cannot
+// corrupt it; what they record still interleaves, which is why measurements are made from one thread.
 struct StageTimer {
-	bool on = false;
+	std::atomic<bool> on{false};
+	std::mutex lock;
 	std::vector<hipEvent_t> pool;
 	std::vector<const char*> tags;  // tag of event i; nullptr closes an entry point
 	size_t used = 0;
@@ -74,7 +79,10 @@ constexpr size_t kMaxTimerEvents = 1 << 16;
 
 void timer_record(const char* tag, hipStream_t s)
 {
-	if (!g_timer.on || g_timer.used >= kMaxTimerEvents)
+	if (!g_timer.on.load(std::memory_order_relaxed))
+		return;
+	std::lock_guard<std::mutex> hold(g_timer.lock);
+	if (g_timer.used >= kMaxTimerEvents)
 		return;
 	if (g_timer.used == g_timer.pool.size()) {
 		hipEvent_t e;
@@ -325,7 +333,8 @@ extern "C" {
 
 int rgs_stage_timing(int enable)
 {
-	g_timer.on = enable != 0;
+	std::lock_guard<std::mutex> hold(g_timer.lock);
+	g_timer.on.store(enable != 0, std::memory_order_relaxed);
 	g_timer.used = 0;
 	return 0;
 }
@@ -334,6 +343,7 @@ int rgs_stage_timing_read(int max_stages, const char** names, float* total_ms, i
 {
 	RGS_REQUIRE(max_stages >= 0 && (max_stages == 0 || (names && total_ms && launches)), "rgs_stage_timing_read: bad arguments");
 	int n = 0;
+	std::lock_guard<std::mutex> hold(g_timer.lock);
 	if (g_timer.used > 0) {
 		hipError_t e = hipEventSynchronize(g_timer.pool[g_timer.used - 1]);
 		if (e != hipSuccess)
@@ -1032,7 +1042,7 @@ int rgs_frame_backward(int K, const rgs_frame_layer* layers, const rgs_frame_vie
 	const std::vector<hipStream_t> sides = side_streams(K, layers, s);
 	// where the bandwidth-bound work goes; the stage timing charges the time between consecutive events of one stream,
 	// so while it is on everything stays on the frame's stream
-	hipStream_t beside = (sides.empty() || g_timer.on) ? s : sides[0];
+	hipStream_t beside = (sides.empty() || g_timer.on.load(std::memory_order_relaxed)) ? s : sides[0];
 	std::vector<rgs::BlendArgs> jobs;
 	std::vector<int> job_layer;
 	std::vector<rgs::PreprocessBackwardArgs> geometry((size_t)K);
