@@ -38,19 +38,34 @@ __global__ __launch_bounds__(256) void composite_forward_kernel(CompositeArgs a)
 
 // dL/dimage_k = T_k g, dL/ddepth_k = T_k g_d, dL/dalpha_k = -T_k R_k with
 // R_{K-1} = <bg, g> - g_a and R_{k-1} = <image_k, g> + depth_k g_d + (1 - alpha_k) R_k.
-// No division, so alpha_k = 1 is handled exactly.  T_k is kept per thread for the
-// back-to-front sweep.
+// No division, so alpha_k = 1 is handled exactly.  T_k and alpha_k are kept per thread for the
+// back-to-front sweep: in registers when the number of layers is at most kLayers (the loops are unrolled over kLayers
+// and guarded by K, so the arrays are indexed by constants), otherwise (kLayers = 0) in an array indexed at run time,
+// which the compiler places in scratch memory: every value then goes out to memory and comes back.
+template <int kLayers>
 __global__ __launch_bounds__(256) void composite_backward_kernel(CompositeArgs a)
 {
 	const size_t n = (size_t)a.H * a.W;
 	const size_t p = (size_t)blockIdx.x * 256 + threadIdx.x;
 	if (p >= n)
 		return;
-	float Tk[kMaxComposite];
+	constexpr int kHeld = kLayers > 0 ? kLayers : kMaxComposite;
+	float Tk[kHeld], alpha[kHeld];
 	float T = 1.f;
-	for (int k = 0; k < a.K; k++) {
-		Tk[k] = T;
-		T = T * (1.f - a.alphas[k][p]);
+	if (kLayers > 0) {
+#pragma unroll
+		for (int k = 0; k < kLayers; k++)
+			if (k < a.K) {
+				alpha[k] = a.alphas[k][p];
+				Tk[k] = T;
+				T = T * (1.f - alpha[k]);
+			}
+	} else {
+		for (int k = 0; k < a.K; k++) {
+			alpha[k] = a.alphas[k][p];
+			Tk[k] = T;
+			T = T * (1.f - alpha[k]);
+		}
 	}
 	const float gr = a.g_image[p], gg = a.g_image[n + p], gb = a.g_image[2 * n + p];
 	const float gd = a.g_depth ? a.g_depth[p] : 0.f;
@@ -58,8 +73,7 @@ __global__ __launch_bounds__(256) void composite_backward_kernel(CompositeArgs a
 	float R = -ga;
 	if (a.bg)
 		R += a.bg[0] * gr + a.bg[1] * gg + a.bg[2] * gb;
-	for (int k = a.K - 1; k >= 0; k--) {
-		const float t = Tk[k];
+	auto layer = [&](int k, float t, float alpha_k) {
 		float* di = a.d_images[k];
 		di[p] = t * gr;
 		di[n + p] = t * gg;
@@ -67,7 +81,16 @@ __global__ __launch_bounds__(256) void composite_backward_kernel(CompositeArgs a
 		a.d_depths[k][p] = t * gd;
 		a.d_alphas[k][p] = -(t * R);
 		const float* img = a.images[k];
-		R = img[p] * gr + img[n + p] * gg + img[2 * n + p] * gb + a.depths[k][p] * gd + (1.f - a.alphas[k][p]) * R;
+		R = img[p] * gr + img[n + p] * gg + img[2 * n + p] * gb + a.depths[k][p] * gd + (1.f - alpha_k) * R;
+	};
+	if (kLayers > 0) {
+#pragma unroll
+		for (int k = kLayers - 1; k >= 0; k--)
+			if (k < a.K)
+				layer(k, Tk[k], alpha[k]);
+	} else {
+		for (int k = a.K - 1; k >= 0; k--)
+			layer(k, Tk[k], alpha[k]);
 	}
 }
 
@@ -82,7 +105,13 @@ void launch_composite_backward(const CompositeArgs& a, hipStream_t s)
 {
 	const size_t n = (size_t)a.H * a.W;
 	stage_mark("composite_backward", s);
-	hipLaunchKernelGGL(composite_backward_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a);
+	const dim3 grid((unsigned)((n + 255) / 256));
+	if (a.K <= 4)
+		hipLaunchKernelGGL(composite_backward_kernel<4>, grid, dim3(256), 0, s, a);
+	else if (a.K <= 16)
+		hipLaunchKernelGGL(composite_backward_kernel<16>, grid, dim3(256), 0, s, a);
+	else
+		hipLaunchKernelGGL(composite_backward_kernel<0>, grid, dim3(256), 0, s, a);
 }
 
 }  // namespace rgs
